@@ -1,0 +1,155 @@
+/*
+ * hstu_attn.h -- C ABI of the MI355X (gfx950) HSTU pointwise-SiLU attention
+ * forward.
+ *
+ *   S[b,h,i,j] = alpha * sum_c q[b,i,h,c] k[b,j,h,c]
+ *                (+ pos_tab[h|0][(L-1)+j-i]) (+ ts_tab[h|0][bucket(dt)])
+ *                (+ dense_bias[b|0][i][j])
+ *   P          = S * sigmoid(S) * inv_n
+ *   out[b,i,h,:] = sum_j (M[b,i,j] ? P : 0) * v[b,j,h,:]
+ *
+ * Every entry point is enqueue-only on the caller's HIP stream, allocates no
+ * device memory and never synchronises.  The caller owns every buffer.
+ *
+ * Reference interfaces this library stands in for (paths relative to the
+ * RecML checkout):
+ *   hstu_attn_fwd            recml/core/ops/hstu_ops.py:829-851
+ *                            (pointwise_splash_attention) and
+ *                            recml/layers/keras/hstu.py:356-390
+ *                            (HSTUBlock._pointwise_attention)
+ *   mask fields              recml/core/ops/hstu_ops.py:926-979 (mask type,
+ *                            sliding window, segment ids) and
+ *                            recml/layers/keras/utils.py:29-41 (length mask)
+ *   pos_tab                  recml/layers/keras/hstu.py:58-128
+ *   ts / ts_tab              recml/layers/keras/hstu.py:33-55, 131-237
+ */
+#ifndef HSTU_ATTN_H_
+#define HSTU_ATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HSTU_ATTN_ABI_VERSION 1
+
+/* Tensor layouts of q, k, v, out. */
+enum HstuLayout {
+  HSTU_LAYOUT_PADDED = 0, /* [B, L, H, d]; strides given per tensor          */
+  HSTU_LAYOUT_JAGGED = 1  /* [T, H, d] with seq_offsets[B+1]                  */
+};
+
+enum HstuDtype {
+  HSTU_DTYPE_FP32 = 0,
+  HSTU_DTYPE_BF16 = 1,
+  HSTU_DTYPE_FP8_E4M3FN = 2 /* q and k only; scales in q_scale / k_scale     */
+};
+
+/* Which positions take part, on top of causal / window / explicit mask. */
+enum HstuMaskMode {
+  HSTU_MASK_NONE = 0,    /* all L x Lkv positions                             */
+  HSTU_MASK_LENGTH = 1,  /* i < n_b and j < n_b; rows >= n_b are written as 0 */
+  HSTU_MASK_SEGMENT = 2  /* q_segment_ids[b,i] == kv_segment_ids[b,j]         */
+};
+
+/* Return codes (0 = launched). */
+enum HstuStatus {
+  HSTU_OK = 0,
+  HSTU_ERR_NULL = -1,         /* a required pointer is null                   */
+  HSTU_ERR_VERSION = -2,      /* struct_size / version mismatch               */
+  HSTU_ERR_DTYPE = -3,        /* unsupported dtype combination                */
+  HSTU_ERR_SHAPE = -4,        /* bad B/L/H/d, strides or option combination   */
+  HSTU_ERR_WORKSPACE = -5,    /* workspace missing or too small               */
+  HSTU_ERR_LAUNCH = -6        /* HIP reported an error at launch              */
+};
+
+typedef struct HstuAttnFwdArgs {
+  uint32_t struct_size;   /* sizeof(HstuAttnFwdArgs)                          */
+  uint32_t version;       /* HSTU_ATTN_ABI_VERSION                            */
+
+  int32_t layout;         /* HstuLayout                                       */
+  int32_t qk_dtype;       /* HstuDtype of q and k                             */
+  int32_t v_dtype;        /* HstuDtype of v                                   */
+  int32_t out_dtype;      /* HstuDtype of out (fp32 or bf16)                  */
+
+  int32_t B;              /* sequences                                        */
+  int32_t L;              /* max query length (padded length; bias geometry)  */
+  int32_t Lkv;            /* max key length; == L except padded cross-length  */
+  int32_t H;              /* heads                                            */
+  int32_t d_qk;           /* head dim of q and k                              */
+  int32_t d_v;            /* head dim of v and out                            */
+  int64_t total_tokens;   /* T for the jagged layout, else ignored            */
+
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  /* Strides in ELEMENTS; the innermost (d) stride is 1.  *_stride_b is only
+   * read for the padded layout. */
+  int64_t q_stride_b, q_stride_t, q_stride_h;
+  int64_t k_stride_b, k_stride_t, k_stride_h;
+  int64_t v_stride_b, v_stride_t, v_stride_h;
+  int64_t o_stride_b, o_stride_t, o_stride_h;
+
+  float alpha;            /* logit scale: 1 or 1/sqrt(d)                      */
+  float inv_n;            /* 1/N normaliser applied after SiLU                */
+
+  int32_t causal;         /* 1: keep j <= i                                   */
+  int32_t mask_mode;      /* HstuMaskMode                                     */
+  int32_t window;         /* keep |i-j| <= window; < 0 disables               */
+  int32_t reserved0;
+
+  const int32_t* seq_lens;     /* [B], LENGTH mode with the padded layout     */
+  const int32_t* seq_offsets;  /* [B+1], jagged layout                        */
+  const int32_t* q_segment_ids;  /* [B, L],   SEGMENT mode                    */
+  const int32_t* kv_segment_ids; /* [B, Lkv], SEGMENT mode                    */
+
+  const uint8_t* mask;    /* explicit keep-mask (non-zero = keep) or null     */
+  int32_t mask_batched;   /* 0: [L, Lkv] shared; 1: [B, L, Lkv]               */
+  int32_t dense_bias_batched; /* 0: [L, Lkv] shared; 1: [B, L, Lkv]           */
+  const float* dense_bias; /* additive logit bias shared by heads, or null    */
+
+  const float* pos_tab;   /* [pos_heads, 2L-1] relative-position table / null */
+  int32_t pos_heads;      /* 1 or H                                           */
+  int32_t ts_heads;       /* 1 or H                                           */
+  const float* ts_tab;    /* [ts_heads, ts_num_buckets+1] or null             */
+  const int64_t* ts;      /* timestamps; padded [B, ts_stride_b] or jagged [T]*/
+  int64_t ts_stride_b;    /* elements between sequences; 0 = jagged by
+                             seq_offsets                                      */
+  int32_t ts_num_buckets; /* clip bound; table has ts_num_buckets+1 entries   */
+  float ts_bucket_size;   /* 0.301 in the reference                           */
+
+  const float* q_scale;   /* [H] dequantisation scales (fp8 q), else null     */
+  const float* k_scale;   /* [H] dequantisation scales (fp8 k), else null     */
+
+  void* workspace;        /* device scratch of hstu_attn_fwd_workspace_bytes  */
+  size_t workspace_bytes;
+} HstuAttnFwdArgs;
+
+/* ABI version of the loaded library (HSTU_ATTN_ABI_VERSION at build time). */
+int hstu_attn_abi_version(void);
+
+/* Device scratch the call needs for these arguments (0 today for every
+ * supported combination; callers must still query it).  No reference
+ * counterpart: the reference's op is a pure function under jax.jit. */
+size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
+
+/* Validate `args` and enqueue the forward on `stream` (a hipStream_t passed
+ * as void* so that C callers need no HIP headers).  Returns an HstuStatus.
+ * Replaces recml/core/ops/hstu_ops.py:829-1046 and the dense path of
+ * recml/layers/keras/hstu.py:356-390. */
+int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
+
+/* Message for the last non-zero status on this thread ("" if none). */
+const char* hstu_attn_last_error(void);
+
+/* Name of the kernel variant hstu_attn_fwd would launch for `args`
+ * (diagnostics for profiles and benchmarks; static storage). */
+const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_ATTN_H_ */

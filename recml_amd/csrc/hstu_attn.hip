@@ -1,0 +1,768 @@
+// HSTU pointwise-SiLU attention forward for gfx950 (MI355X, CDNA4).
+//
+//   out[b,i,h,:] = sum_j M[b,i,j] * silu(alpha*q_i.k_j + bias(b,h,i,j)) * inv_n * v[b,j,h,:]
+//
+// Two kernels live here behind one C entry point (see include/hstu_attn.h):
+//
+//   hstu_fwd_mfma_bf16   the hot path.  bf16 Q/K/V, fp32 accumulation on the
+//                        32x32x16 bf16 MFMA, 128 query rows x 64 keys per
+//                        step, K/V double-buffered through LDS, relative
+//                        position and timestamp bias + SiLU + mask fused on
+//                        the accumulator registers, causal/length tile
+//                        skipping.  Computes S^T = K Q^T so that the
+//                        accumulator layout of S^T is already the B-operand
+//                        layout of O^T = V^T P^T: P never touches LDS.
+//   hstu_fwd_general     every option of the op (segment ids, explicit mask,
+//                        sliding window, dense bias, cross lengths, any head
+//                        dim <= 256, fp32 or bf16 storage) in plain fp32 FMA
+//                        arithmetic.  Correctness path for the options the
+//                        MFMA kernel does not cover and the fp32 reference
+//                        configuration.
+//
+// The math follows recml/layers/keras/hstu.py:356-390 (dense formulation),
+// recml/core/ops/hstu_ops.py:230-264 (order: scale, SiLU, 1/N, mask, PV in
+// fp32), hstu.py:91-113 (relative position bias = w[(L-1)+j-i]) and
+// hstu.py:33-55, 190-221 (timestamp buckets).
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "hstu_attn.h"
+
+namespace {
+
+typedef __bf16 bf16_t;
+typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
+typedef bf16_t bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+
+struct Params {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  int64_t q_sb, q_st, q_sh;
+  int64_t k_sb, k_st, k_sh;
+  int64_t v_sb, v_st, v_sh;
+  int64_t o_sb, o_st, o_sh;
+  const int32_t* seq_lens;
+  const int32_t* seq_offsets;
+  const int32_t* q_seg;
+  const int32_t* kv_seg;
+  const uint8_t* mask;
+  const float* dense_bias;
+  const float* pos_tab;
+  const float* ts_tab;
+  const int64_t* ts;
+  int64_t ts_sb;
+  int32_t B, L, Lkv, H, d_qk, d_v;
+  int32_t jagged, causal, mask_mode, window;
+  int32_t mask_batched, dense_bias_batched, pos_heads, ts_heads;
+  int32_t ts_nb;
+  float ts_bucket_size;
+  float ts_log2_scale;  // ln(2) / ts_bucket_size
+  float alpha, inv_n;
+  int32_t n_qtiles;
+};
+
+// Per-sequence geometry shared by both kernels.
+struct Seq {
+  int n_q;        // query rows that produce output
+  int n_kv;       // keys that may be attended
+  int rows;       // rows of the output tile space (L, or n_b when jagged)
+  int64_t tok0;   // first token of the sequence in the token axis
+  int64_t bq, bk, bv, bo;  // element offsets of (token 0, head h)
+  int64_t ts0;    // element offset of timestamp 0
+  int n_ts;       // timestamps addressable for this sequence
+};
+
+__device__ __forceinline__ Seq seq_info(const Params& p, int b, int h) {
+  Seq s;
+  if (p.jagged) {
+    int o0 = p.seq_offsets[b], o1 = p.seq_offsets[b + 1];
+    int n = o1 - o0;
+    n = n < 0 ? 0 : (n > p.L ? p.L : n);
+    s.n_q = n; s.n_kv = n; s.rows = n; s.tok0 = o0;
+    s.bq = (int64_t)o0 * p.q_st + (int64_t)h * p.q_sh;
+    s.bk = (int64_t)o0 * p.k_st + (int64_t)h * p.k_sh;
+    s.bv = (int64_t)o0 * p.v_st + (int64_t)h * p.v_sh;
+    s.bo = (int64_t)o0 * p.o_st + (int64_t)h * p.o_sh;
+  } else {
+    int nq = p.L, nk = p.Lkv;
+    if (p.mask_mode == HSTU_MASK_LENGTH) {
+      int n = p.seq_lens[b];
+      n = n < 0 ? 0 : n;
+      nq = n < p.L ? n : p.L;
+      nk = n < p.Lkv ? n : p.Lkv;
+    }
+    s.n_q = nq; s.n_kv = nk; s.rows = p.L; s.tok0 = 0;
+    s.bq = (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+    s.bk = (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+    s.bv = (int64_t)b * p.v_sb + (int64_t)h * p.v_sh;
+    s.bo = (int64_t)b * p.o_sb + (int64_t)h * p.o_sh;
+  }
+  if (p.ts_sb != 0) { s.ts0 = (int64_t)b * p.ts_sb; s.n_ts = p.L; }
+  else              { s.ts0 = s.tok0;               s.n_ts = s.n_kv; }
+  return s;
+}
+
+__device__ __forceinline__ float ldf(const float* p) { return *p; }
+__device__ __forceinline__ float ldf(const bf16_t* p) { return (float)*p; }
+__device__ __forceinline__ void stf(float* p, float x) { *p = x; }
+__device__ __forceinline__ void stf(bf16_t* p, float x) { *p = (bf16_t)x; }
+
+// ---------------------------------------------------------------------------
+// General kernel: fp32 FMA arithmetic, every option.
+// ---------------------------------------------------------------------------
+
+constexpr int GT = 32;       // query rows and keys per tile
+constexpr int GMAXX = 32;    // d_v / 8 accumulators per thread, d_v <= 256
+
+__device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
+                                              int b, int h, int i, int j) {
+  float bias = 0.f;
+  if (p.pos_tab) {
+    int hh = p.pos_heads > 1 ? h : 0;
+    bias += p.pos_tab[(int64_t)hh * (2 * p.L - 1) + (p.L - 1) + j - i];
+  }
+  if (p.ts_tab) {
+    int iq = i + 1 < s.n_ts ? i + 1 : s.n_ts - 1;
+    int jk = j < s.n_ts ? j : s.n_ts - 1;
+    int64_t dt = p.ts[s.ts0 + iq] - p.ts[s.ts0 + jk];
+    if (dt < 0) dt = -dt;
+    if (dt < 1) dt = 1;
+    if (dt > 1000000000LL) dt = 1000000000LL;
+    // fp32 log then fp32 divide then truncation, as the dense layer does it
+    float lg = logf((float)dt) / p.ts_bucket_size;
+    int bk = (int)lg;
+    bk = bk < 0 ? 0 : (bk > p.ts_nb ? p.ts_nb : bk);
+    int hh = p.ts_heads > 1 ? h : 0;
+    bias += p.ts_tab[(int64_t)hh * (p.ts_nb + 1) + bk];
+  }
+  if (p.dense_bias) {
+    int64_t o = p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0;
+    bias += p.dense_bias[o + (int64_t)i * p.Lkv + j];
+  }
+  return bias;
+}
+
+__device__ __forceinline__ bool general_keep(const Params& p, const Seq& s,
+                                             int b, int i, int j) {
+  bool keep = (i < s.n_q) && (j < s.n_kv);
+  if (p.causal) keep = keep && (j <= i);
+  if (p.window >= 0) {
+    int dd = i - j; dd = dd < 0 ? -dd : dd;
+    keep = keep && (dd <= p.window);
+  }
+  if (!keep) return false;
+  if (p.mask_mode == HSTU_MASK_SEGMENT)
+    keep = p.q_seg[(int64_t)b * p.L + i] == p.kv_seg[(int64_t)b * p.Lkv + j];
+  if (keep && p.mask) {
+    int64_t o = p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0;
+    keep = p.mask[o + (int64_t)i * p.Lkv + j] != 0;
+  }
+  return keep;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
+  extern __shared__ float gsm[];
+  const int dq = p.d_qk, dv = p.d_v;
+  const int kp = dq + 1;                   // odd pitch: column reads of K
+  float* Qs = gsm;                         // [GT][dq]
+  float* Ks = Qs + GT * dq;                // [GT][kp]
+  float* Vs = Ks + GT * kp;                // [GT][dv]
+  float* Ps = Vs + GT * dv;                // [GT][GT+1]
+
+  const int qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const Seq s = seq_info(p, b, h);
+  const int q0 = qt * GT;
+  if (q0 >= s.rows) return;
+  const int tid = threadIdx.x;
+  const T* __restrict__ qp = (const T*)p.q;
+  const T* __restrict__ kp_ = (const T*)p.k;
+  const T* __restrict__ vp = (const T*)p.v;
+  T* __restrict__ op = (T*)p.out;
+
+  const int oi = tid >> 3, ocg = tid & 7;  // output row / column group
+  const int nx = (dv + 7) >> 3;
+  float acc[GMAXX];
+#pragma unroll
+  for (int x = 0; x < GMAXX; ++x) acc[x] = 0.f;
+
+  if (q0 < s.n_q) {
+    for (int e = tid; e < GT * dq; e += 256) {
+      int r = e / dq, c = e - r * dq;
+      int i = q0 + r;
+      Qs[e] = (i < s.n_q) ? ldf(qp + s.bq + (int64_t)i * p.q_st + c) : 0.f;
+    }
+    int kv_end = s.n_kv;
+    if (p.causal && q0 + GT < kv_end) kv_end = q0 + GT;
+    if (p.window >= 0 && q0 + GT + p.window < kv_end) kv_end = q0 + GT + p.window;
+    int kv_begin = 0;
+    if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
+
+    for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
+      __syncthreads();
+      for (int e = tid; e < GT * dq; e += 256) {
+        int r = e / dq, c = e - r * dq;
+        int j = kv0 + r;
+        Ks[r * kp + c] = (j < s.n_kv) ? ldf(kp_ + s.bk + (int64_t)j * p.k_st + c) : 0.f;
+      }
+      for (int e = tid; e < GT * dv; e += 256) {
+        int r = e / dv, c = e - r * dv;
+        int j = kv0 + r;
+        Vs[e] = (j < s.n_kv) ? ldf(vp + s.bv + (int64_t)j * p.v_st + c) : 0.f;
+      }
+      __syncthreads();
+      {
+        const int tx = tid & 31, ty = tid >> 5;
+        float sacc[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* krow = Ks + tx * kp;
+        for (int c = 0; c < dq; ++c) {
+          float kvv = krow[c];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sacc[r] = fmaf(Qs[(ty + 8 * r) * dq + c], kvv, sacc[r]);
+        }
+        const int j = kv0 + tx;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = q0 + ty + 8 * r;
+          float pval = 0.f;
+          if (general_keep(p, s, b, i, j)) {
+            float x = p.alpha * sacc[r] + general_bias(p, s, b, h, i, j);
+            pval = x / (1.0f + expf(-x));
+          }
+          Ps[(ty + 8 * r) * (GT + 1) + tx] = pval;
+        }
+      }
+      __syncthreads();
+      for (int jj = 0; jj < GT; ++jj) {
+        float pv = Ps[oi * (GT + 1) + jj];
+        const float* vrow = Vs + jj * dv;
+#pragma unroll
+        for (int x = 0; x < GMAXX; ++x) {
+          if (x < nx) {
+            int c = ocg + 8 * x;
+            if (c < dv) acc[x] = fmaf(pv, vrow[c], acc[x]);
+          }
+        }
+      }
+    }
+  }
+  // rows past the sequence are written as exact zeros (padded layout)
+  const int i = q0 + oi;
+  if (i < s.rows) {
+    const bool live = i < s.n_q;
+#pragma unroll
+    for (int x = 0; x < GMAXX; ++x) {
+      if (x < nx) {
+        int c = ocg + 8 * x;
+        if (c < dv) stf(op + s.bo + (int64_t)i * p.o_st + c, live ? acc[x] * p.inv_n : 0.f);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// MFMA kernel: bf16, causal/full + length masking, fused pos / timestamp bias.
+// ---------------------------------------------------------------------------
+
+constexpr int BM = 128;   // query rows per workgroup (4 waves x 32)
+constexpr int BN = 64;    // keys per step
+constexpr int POSW = 192; // staged window of the position table per step
+
+template <int D>
+struct MfmaSmem {
+  static constexpr int KP = D + 8;    // K row pitch in bf16 (16 B pad)
+  static constexpr int VP = BN + 8;   // V^T row pitch in bf16
+  static constexpr int K_BYTES = BN * KP * 2;
+  static constexpr int V_BYTES = D * VP * 2;
+  static constexpr int STAGE = K_BYTES + V_BYTES;
+  static constexpr int POS_BYTES = 4 * POSW * 4;
+  static constexpr int TK_BYTES = BN * 8;
+  static constexpr int TAB_BYTES = 132 * 4;
+  static constexpr int total(bool pos, bool ts) {
+    return 2 * STAGE + (pos ? 2 * POS_BYTES : 0) + (ts ? 2 * TK_BYTES + TAB_BYTES : 0);
+  }
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  floatx2 f = {lo, hi};
+  bf16x2 r = __builtin_convertvector(f, bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ float fast_silu(float x) {
+  // x * sigmoid(x) = x / (1 + 2^(-x*log2(e)))
+  float e = __builtin_amdgcn_exp2f(x * -1.4426950408889634f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+template <int D, bool POS, bool TS>
+__global__ __launch_bounds__(256, 2) void hstu_fwd_mfma_bf16(const Params p) {
+  using SM = MfmaSmem<D>;
+  constexpr int KP = SM::KP, VP = SM::VP;
+  constexpr int KSTEPS = D / 16;       // MFMA k-steps over the head dim
+  constexpr int DVB = D / 32;          // 32-row blocks of O^T
+  constexpr int KCH = BN * D / 8;      // 16-byte chunks in a K tile
+  constexpr int KLD = (KCH + 255) / 256;
+  constexpr int VBLK = (BN / 4) * (D / 8);   // 4x8 transposition blocks in a V tile
+  constexpr int VLD = (VBLK + 255) / 256;
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // LDS map: [stage0: K | V^T][stage1: K | V^T][pos window x2][key ts x2][ts table]
+  auto Ks = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE); };
+  auto Vt = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE + SM::K_BYTES); };
+  constexpr int POS_OFF = 2 * SM::STAGE;
+  constexpr int TK_OFF = POS_OFF + (POS ? 2 * SM::POS_BYTES : 0);
+  auto Wc = [&](int buf) { return (float*)(smem + POS_OFF + buf * SM::POS_BYTES); };
+  auto Tk = [&](int buf) { return (int64_t*)(smem + TK_OFF + buf * SM::TK_BYTES); };
+  float* TsTab = (float*)(smem + TK_OFF + 2 * SM::TK_BYTES);
+
+  // Heaviest query tiles first; all tiles of one (b,h) share blockIdx % 8 so
+  // that they land on one XCD and reuse K/V from its L2.
+  const int BH = p.B * p.H;
+  const int bh = blockIdx.x % BH;
+  const int qt = p.n_qtiles - 1 - blockIdx.x / BH;
+  const int b = bh / p.H, h = bh - b * p.H;
+  const Seq s = seq_info(p, b, h);
+  const int q0 = qt * BM;
+  if (q0 >= s.rows) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, w = tid >> 6;
+  const int m = lane & 31, hh = lane >> 5;
+  const bf16_t* __restrict__ kg = (const bf16_t*)p.k + s.bk;
+  const bf16_t* __restrict__ vg = (const bf16_t*)p.v + s.bv;
+  bf16_t* __restrict__ og = (bf16_t*)p.out + s.bo;
+
+  if (q0 >= s.n_q) {
+    // padded rows of the padded layout: exact zeros
+    const int rows = (s.rows - q0) < BM ? (s.rows - q0) : BM;
+    const uint4 z = {0u, 0u, 0u, 0u};
+    for (int e = tid; e < rows * (D / 8); e += 256) {
+      int r = e / (D / 8), c = e - r * (D / 8);
+      *(uint4*)(og + (int64_t)(q0 + r) * p.o_st + c * 8) = z;
+    }
+    return;
+  }
+
+  const int r0 = q0 + 32 * w;          // first query row of this wave
+  const int qrow = r0 + m;             // this lane's query row
+  const bool wave_live = r0 < s.n_q;
+
+  // Q fragments (B operand of S^T = K Q^T): lane holds q[qrow][16ks+8hh .. +7]
+  bf16x8 qf[KSTEPS];
+  {
+    const bf16_t* qg = (const bf16_t*)p.q + s.bq + (int64_t)qrow * p.q_st + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      uint4 t = {0u, 0u, 0u, 0u};
+      if (qrow < s.n_q) t = *(const uint4*)(qg + 16 * ks);
+      qf[ks] = __builtin_bit_cast(bf16x8, t);
+    }
+  }
+
+  int kv_end = s.n_kv;
+  if (p.causal) {
+    int lim = q0 + BM < s.n_q ? q0 + BM : s.n_q;
+    kv_end = lim < kv_end ? lim : kv_end;
+  }
+  const int nt = (kv_end + BN - 1) / BN;
+  // keys this wave needs under causality
+  const int wave_kv_end = p.causal ? ((r0 + 32) < kv_end ? (r0 + 32) : kv_end) : kv_end;
+
+  int64_t tq = 0;
+  if (TS) {
+    int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
+    tq = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
+    const float* tab = p.ts_tab + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1);
+    for (int e = tid; e < 132; e += 256) {
+      int c = e <= p.ts_nb ? e : p.ts_nb;
+      TsTab[e] = tab[c > 128 ? 128 : c];
+    }
+  }
+  const float* postab = POS ? p.pos_tab + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) : nullptr;
+
+  floatx16 o[DVB];
+#pragma unroll
+  for (int i = 0; i < DVB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+
+  uint4 kreg[KLD];
+  uint4 vreg[VLD][4];
+
+  auto gload = [&](int kv0) {
+#pragma unroll
+    for (int r = 0; r < KLD; ++r) {
+      int c = tid + 256 * r;
+      int row = c / (D / 8), col = c - row * (D / 8);
+      uint4 t = {0u, 0u, 0u, 0u};
+      if (c < KCH && kv0 + row < s.n_kv)
+        t = *(const uint4*)(kg + (int64_t)(kv0 + row) * p.k_st + col * 8);
+      kreg[r] = t;
+    }
+#pragma unroll
+    for (int r = 0; r < VLD; ++r) {
+      int blk = tid + 256 * r;
+      int kvg = blk / (D / 8), dvg = blk - kvg * (D / 8);
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        uint4 t = {0u, 0u, 0u, 0u};
+        int row = kv0 + 4 * kvg + rr;
+        if (blk < VBLK && row < s.n_kv)
+          t = *(const uint4*)(vg + (int64_t)row * p.v_st + dvg * 8);
+        vreg[r][rr] = t;
+      }
+    }
+  };
+
+  auto lds_store = [&](int buf, int kv0) {
+#pragma unroll
+    for (int r = 0; r < KLD; ++r) {
+      int c = tid + 256 * r;
+      int row = c / (D / 8), col = c - row * (D / 8);
+      if (c < KCH) *(uint4*)(Ks(buf) + row * KP + col * 8) = kreg[r];
+    }
+#pragma unroll
+    for (int r = 0; r < VLD; ++r) {
+      int blk = tid + 256 * r;
+      int kvg = blk / (D / 8), dvg = blk - kvg * (D / 8);
+      if (blk < VBLK) {
+        // 4 keys x 8 channels -> 8 channels x 4 keys.  Within each 16-key
+        // chunk the 4-key groups are stored in the order 0,2,1,3 so that the
+        // 8 keys an MFMA lane needs are one 16-byte read.
+        int c16 = kvg >> 2, g4 = kvg & 3;
+        int pos = 16 * c16 + 8 * (g4 & 1) + 4 * (g4 >> 1);
+        const uint32_t a0[4] = {vreg[r][0].x, vreg[r][0].y, vreg[r][0].z, vreg[r][0].w};
+        const uint32_t a1[4] = {vreg[r][1].x, vreg[r][1].y, vreg[r][1].z, vreg[r][1].w};
+        const uint32_t a2[4] = {vreg[r][2].x, vreg[r][2].y, vreg[r][2].z, vreg[r][2].w};
+        const uint32_t a3[4] = {vreg[r][3].x, vreg[r][3].y, vreg[r][3].z, vreg[r][3].w};
+#pragma unroll
+        for (int jx = 0; jx < 4; ++jx) {
+          uint2 even, odd;
+          even.x = (a0[jx] & 0xffffu) | (a1[jx] << 16);
+          even.y = (a2[jx] & 0xffffu) | (a3[jx] << 16);
+          odd.x = (a0[jx] >> 16) | (a1[jx] & 0xffff0000u);
+          odd.y = (a2[jx] >> 16) | (a3[jx] & 0xffff0000u);
+          *(uint2*)(Vt(buf) + (dvg * 8 + 2 * jx) * VP + pos) = even;
+          *(uint2*)(Vt(buf) + (dvg * 8 + 2 * jx + 1) * VP + pos) = odd;
+        }
+      }
+    }
+    if (POS) {
+      // window[x] = pos_tab[(L-1) + kv0 - (q0+127) + x]; copy s is shifted by s
+      const int idx0 = (p.L - 1) + kv0 - (q0 + BM - 1);
+      for (int e = tid; e < 4 * POSW; e += 256) {
+        int sft = e / POSW, z = e - sft * POSW;
+        int idx = idx0 + z + sft;
+        Wc(buf)[e] = (idx >= 0 && idx < 2 * p.L - 1) ? postab[idx] : 0.f;
+      }
+    }
+    if (TS) {
+      if (tid < BN) {
+        int jk = kv0 + tid;
+        jk = jk < s.n_ts ? jk : s.n_ts - 1;
+        Tk(buf)[tid] = p.ts[s.ts0 + (jk < 0 ? 0 : jk)];
+      }
+    }
+  };
+
+  gload(0);
+  lds_store(0, 0);
+  __syncthreads();
+
+  for (int t = 0; t < nt; ++t) {
+    const int kv0 = t * BN;
+    const int buf = t & 1;
+    if (t + 1 < nt) gload(kv0 + BN);
+
+    if (wave_live) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+        const int kbs = kv0 + 32 * kb;
+        if (kbs < wave_kv_end) {
+          floatx16 sacc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+          const bf16_t* kr = Ks(buf) + (32 * kb + m) * KP + 8 * hh;
+#pragma unroll
+          for (int ks = 0; ks < KSTEPS; ++ks) {
+            bf16x8 a = *(const bf16x8*)(kr + 16 * ks);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], sacc, 0, 0, 0);
+          }
+          // lane holds S^T[kv = kbs + 8g + 4hh + t][q = qrow], r = 4g + t
+          float x[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) x[r] = p.alpha * sacc[r];
+          if (POS) {
+            const int xb = 32 * kb + 4 * hh + (BM - 1) - 32 * w - m;
+            const int sft = xb & 3;
+            const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              float4 bv = *(const float4*)(wrow + 8 * g);
+              x[4 * g + 0] += bv.x; x[4 * g + 1] += bv.y;
+              x[4 * g + 2] += bv.z; x[4 * g + 3] += bv.w;
+            }
+          }
+          if (TS) {
+            const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+              for (int tt = 0; tt < 4; ++tt) {
+                int64_t dt = tq - tk[8 * g + tt];
+                int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+                int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+                float f = __builtin_fabsf((float)sat);
+                f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
+                int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
+                bk = bk < 131 ? bk : 131;
+                x[4 * g + tt] += TsTab[bk];
+              }
+            }
+          }
+          float pv[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) pv[r] = fast_silu(x[r]);
+          // mask only where the block touches the diagonal or the tail
+          const bool need_mask = (p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv);
+          if (need_mask) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
+              bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
+              pv[r] = keep ? pv[r] : 0.f;
+            }
+          }
+#pragma unroll
+          for (int cc = 0; cc < 2; ++cc) {
+            uint4 pk;
+            pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
+            pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
+            pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
+            pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
+            bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
+            const int c = 2 * kb + cc;
+            const bf16_t* vr = Vt(buf) + m * VP + 16 * c + 8 * hh;
+#pragma unroll
+            for (int dvb = 0; dvb < DVB; ++dvb) {
+              bf16x8 a = *(const bf16x8*)(vr + 32 * dvb * VP);
+              o[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, o[dvb], 0, 0, 0);
+            }
+          }
+        }
+      }
+    }
+
+    if (t + 1 < nt) lds_store(buf ^ 1, kv0 + BN);
+    __syncthreads();
+  }
+
+  // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0
+  if (qrow < s.rows) {
+    const bool live = qrow < s.n_q;
+    bf16_t* orow = og + (int64_t)qrow * p.o_st + 4 * hh;
+#pragma unroll
+    for (int dvb = 0; dvb < DVB; ++dvb) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        uint2 pk = {0u, 0u};
+        if (live) {
+          pk.x = pack_bf16(o[dvb][4 * g + 0] * p.inv_n, o[dvb][4 * g + 1] * p.inv_n);
+          pk.y = pack_bf16(o[dvb][4 * g + 2] * p.inv_n, o[dvb][4 * g + 3] * p.inv_n);
+        }
+        *(uint2*)(orow + 32 * dvb + 8 * g) = pk;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side: validation, dispatch, C ABI.
+// ---------------------------------------------------------------------------
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+enum Variant { V_INVALID = 0, V_GENERAL_F32, V_GENERAL_BF16, V_MFMA_BF16 };
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+int validate(const HstuAttnFwdArgs* a) {
+  if (!a) return fail(HSTU_ERR_NULL, "args is null");
+  if (a->struct_size != sizeof(HstuAttnFwdArgs) || a->version != HSTU_ATTN_ABI_VERSION)
+    return fail(HSTU_ERR_VERSION, "args struct_size/version (%u/%u) do not match this library (%zu/%d)",
+                a->struct_size, a->version, sizeof(HstuAttnFwdArgs), HSTU_ATTN_ABI_VERSION);
+  if (!a->q || !a->k || !a->v || !a->out) return fail(HSTU_ERR_NULL, "q, k, v and out must be non-null");
+  if (a->B < 0 || a->L < 1 || a->Lkv < 1 || a->H < 1)
+    return fail(HSTU_ERR_SHAPE, "bad shape B=%d L=%d Lkv=%d H=%d", a->B, a->L, a->Lkv, a->H);
+  if (a->d_qk < 1 || a->d_qk > 256 || a->d_v < 1 || a->d_v > 256)
+    return fail(HSTU_ERR_SHAPE, "head dims must be in [1,256], got d_qk=%d d_v=%d", a->d_qk, a->d_v);
+  if (a->layout != HSTU_LAYOUT_PADDED && a->layout != HSTU_LAYOUT_JAGGED)
+    return fail(HSTU_ERR_SHAPE, "unknown layout %d", a->layout);
+  if (a->mask_mode < HSTU_MASK_NONE || a->mask_mode > HSTU_MASK_SEGMENT)
+    return fail(HSTU_ERR_SHAPE, "unknown mask_mode %d", a->mask_mode);
+  const bool f32 = a->qk_dtype == HSTU_DTYPE_FP32 && a->v_dtype == HSTU_DTYPE_FP32 && a->out_dtype == HSTU_DTYPE_FP32;
+  const bool b16 = a->qk_dtype == HSTU_DTYPE_BF16 && a->v_dtype == HSTU_DTYPE_BF16 && a->out_dtype == HSTU_DTYPE_BF16;
+  if (!f32 && !b16)
+    return fail(HSTU_ERR_DTYPE, "unsupported dtype combination qk=%d v=%d out=%d (all fp32 or all bf16)",
+                a->qk_dtype, a->v_dtype, a->out_dtype);
+  if (a->layout == HSTU_LAYOUT_JAGGED) {
+    if (!a->seq_offsets) return fail(HSTU_ERR_NULL, "jagged layout needs seq_offsets");
+    if (a->mask_mode == HSTU_MASK_SEGMENT) return fail(HSTU_ERR_SHAPE, "segment ids need the padded layout");
+    if (a->L != a->Lkv) return fail(HSTU_ERR_SHAPE, "jagged layout needs L == Lkv");
+    if (a->total_tokens < 0) return fail(HSTU_ERR_SHAPE, "total_tokens < 0");
+  } else if (a->mask_mode == HSTU_MASK_LENGTH && !a->seq_lens) {
+    return fail(HSTU_ERR_NULL, "LENGTH mask mode needs seq_lens");
+  }
+  if (a->mask_mode == HSTU_MASK_SEGMENT && (!a->q_segment_ids || !a->kv_segment_ids))
+    return fail(HSTU_ERR_NULL, "both or neither of q_segment_ids and kv_segment_ids must be provided");
+  if (a->pos_tab) {
+    if (a->L != a->Lkv) return fail(HSTU_ERR_SHAPE, "relative-position bias needs L == Lkv");
+    if (a->pos_heads != 1 && a->pos_heads != a->H) return fail(HSTU_ERR_SHAPE, "pos_heads must be 1 or H");
+  }
+  if (a->ts_tab || a->ts) {
+    if (!a->ts_tab || !a->ts) return fail(HSTU_ERR_NULL, "timestamp bias needs both ts and ts_tab");
+    if (a->L != a->Lkv) return fail(HSTU_ERR_SHAPE, "timestamp bias needs L == Lkv");
+    if (a->ts_heads != 1 && a->ts_heads != a->H) return fail(HSTU_ERR_SHAPE, "ts_heads must be 1 or H");
+    if (a->ts_num_buckets < 0 || !(a->ts_bucket_size > 0.f))
+      return fail(HSTU_ERR_SHAPE, "bad timestamp bucket parameters");
+    if (a->ts_stride_b == 0 && a->layout != HSTU_LAYOUT_JAGGED)
+      return fail(HSTU_ERR_SHAPE, "jagged timestamps need the jagged layout");
+  }
+  return HSTU_OK;
+}
+
+Variant pick_variant(const HstuAttnFwdArgs* a) {
+  if (a->qk_dtype == HSTU_DTYPE_FP32) return V_GENERAL_F32;
+  const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
+  const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->window < 0 &&
+                       a->L == a->Lkv && (!a->ts_tab || a->ts_num_buckets <= 128);
+  auto s8 = [](int64_t x) { return (x & 7) == 0; };
+  const bool align_ok = aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
+                        s8(a->q_stride_t) && s8(a->q_stride_h) && s8(a->k_stride_t) && s8(a->k_stride_h) &&
+                        s8(a->v_stride_t) && s8(a->v_stride_h) && s8(a->o_stride_t) && s8(a->o_stride_h) &&
+                        (a->layout == HSTU_LAYOUT_JAGGED ||
+                         (s8(a->q_stride_b) && s8(a->k_stride_b) && s8(a->v_stride_b) && s8(a->o_stride_b)));
+  if (d_ok && opts_ok && align_ok) return V_MFMA_BF16;
+  return V_GENERAL_BF16;
+}
+
+Params make_params(const HstuAttnFwdArgs* a) {
+  Params p;
+  memset(&p, 0, sizeof(p));
+  p.q = a->q; p.k = a->k; p.v = a->v; p.out = a->out;
+  p.q_sb = a->q_stride_b; p.q_st = a->q_stride_t; p.q_sh = a->q_stride_h;
+  p.k_sb = a->k_stride_b; p.k_st = a->k_stride_t; p.k_sh = a->k_stride_h;
+  p.v_sb = a->v_stride_b; p.v_st = a->v_stride_t; p.v_sh = a->v_stride_h;
+  p.o_sb = a->o_stride_b; p.o_st = a->o_stride_t; p.o_sh = a->o_stride_h;
+  p.seq_lens = a->seq_lens; p.seq_offsets = a->seq_offsets;
+  p.q_seg = a->q_segment_ids; p.kv_seg = a->kv_segment_ids;
+  p.mask = a->mask; p.dense_bias = a->dense_bias;
+  p.pos_tab = a->pos_tab; p.ts_tab = a->ts_tab; p.ts = a->ts; p.ts_sb = a->ts_stride_b;
+  p.B = a->B; p.L = a->L; p.Lkv = a->Lkv; p.H = a->H; p.d_qk = a->d_qk; p.d_v = a->d_v;
+  p.jagged = a->layout == HSTU_LAYOUT_JAGGED;
+  p.causal = a->causal != 0;
+  p.mask_mode = p.jagged ? HSTU_MASK_LENGTH : a->mask_mode;
+  p.window = a->window;
+  p.mask_batched = a->mask_batched; p.dense_bias_batched = a->dense_bias_batched;
+  p.pos_heads = a->pos_heads; p.ts_heads = a->ts_heads;
+  p.ts_nb = a->ts_num_buckets;
+  p.ts_bucket_size = a->ts_bucket_size;
+  p.ts_log2_scale = a->ts_tab ? (float)(0.6931471805599453 / (double)a->ts_bucket_size) : 0.f;
+  p.alpha = a->alpha; p.inv_n = a->inv_n;
+  p.n_qtiles = (a->L + BM - 1) / BM;
+  return p;
+}
+
+template <typename T>
+int launch_general(const Params& p, hipStream_t st) {
+  size_t smem = sizeof(float) * ((size_t)GT * p.d_qk + (size_t)GT * (p.d_qk + 1) + (size_t)GT * p.d_v + GT * (GT + 1));
+  hipError_t e = hipFuncSetAttribute((const void*)hstu_fwd_general<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  dim3 grid((p.L + GT - 1) / GT, p.H, p.B);
+  hipLaunchKernelGGL(hstu_fwd_general<T>, grid, dim3(256), smem, st, p);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "general kernel launch: %s", hipGetErrorString(e));
+  return HSTU_OK;
+}
+
+template <int D, bool POS, bool TS>
+int launch_mfma_inst(const Params& p, hipStream_t st) {
+  const int smem = MfmaSmem<D>::total(POS, TS);
+  hipError_t e = hipFuncSetAttribute((const void*)hstu_fwd_mfma_bf16<D, POS, TS>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  const long long blocks = (long long)p.n_qtiles * p.B * p.H;
+  if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
+  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS>), dim3((unsigned)blocks), dim3(256), smem, st, p);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "mfma kernel launch: %s", hipGetErrorString(e));
+  return HSTU_OK;
+}
+
+template <int D>
+int launch_mfma_d(const Params& p, hipStream_t st) {
+  const bool pos = p.pos_tab != nullptr, ts = p.ts_tab != nullptr;
+  if (pos && ts) return launch_mfma_inst<D, true, true>(p, st);
+  if (pos) return launch_mfma_inst<D, true, false>(p, st);
+  if (ts) return launch_mfma_inst<D, false, true>(p, st);
+  return launch_mfma_inst<D, false, false>(p, st);
+}
+
+}  // namespace
+
+extern "C" {
+
+int hstu_attn_abi_version(void) { return HSTU_ATTN_ABI_VERSION; }
+
+const char* hstu_attn_last_error(void) { return g_err; }
+
+size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args) {
+  (void)args;
+  return 0;
+}
+
+const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
+  if (validate(args) != HSTU_OK) return "invalid";
+  switch (pick_variant(args)) {
+    case V_GENERAL_F32: return "hstu_fwd_general<float>";
+    case V_GENERAL_BF16: return "hstu_fwd_general<bf16>";
+    case V_MFMA_BF16: return "hstu_fwd_mfma_bf16";
+    default: return "invalid";
+  }
+}
+
+int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
+  int rc = validate(args);
+  if (rc != HSTU_OK) return rc;
+  g_err[0] = 0;
+  if (args->B == 0 || (args->layout == HSTU_LAYOUT_JAGGED && args->total_tokens == 0)) return HSTU_OK;
+  const Params p = make_params(args);
+  hipStream_t st = (hipStream_t)stream;
+  switch (pick_variant(args)) {
+    case V_GENERAL_F32: return launch_general<float>(p, st);
+    case V_GENERAL_BF16: return launch_general<bf16_t>(p, st);
+    case V_MFMA_BF16:
+      if (p.d_qk == 128) return launch_mfma_d<128>(p, st);
+      if (p.d_qk == 64) return launch_mfma_d<64>(p, st);
+      return launch_mfma_d<32>(p, st);
+    default: return fail(HSTU_ERR_SHAPE, "no kernel for these arguments");
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,366 @@
+"""HSTU pointwise-SiLU attention forward on MI355X: host-side operator.
+
+Three entry points, each a thin argument check over one C call
+(`hstu_attn_fwd`, include/hstu_attn.h):
+
+  hstu_attention              the full op: padded or jagged Q/K/V, per-sequence
+                              lengths, relative-position and timestamp bias
+                              tables, normaliser N.
+  pointwise_splash_attention  same names, argument meaning and errors as the
+                              reference operator
+                              (recml/core/ops/hstu_ops.py:829-851).
+  pointwise_attention         the layer-side call with a dense mask and bias
+                              (recml/layers/keras/hstu.py:356-390).
+
+Tensors are torch tensors on the GPU; torch only supplies device memory and
+the current HIP stream.  There is no CPU path.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import enum
+import math
+
+import numpy as np
+import torch
+
+from recml_amd import _lib
+
+
+class MaskType(str, enum.Enum):
+  """Mask type of the operator (recml/core/ops/hstu_ops.py:41-45)."""
+
+  CAUSAL = "causal"
+  FULL = "full"
+
+
+_DTYPES = {torch.float32: _lib.DTYPE_FP32, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _ptr(t):
+  return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _check_gpu(name, t):
+  if not isinstance(t, torch.Tensor):
+    raise TypeError(f"{name} must be a torch.Tensor, got {type(t).__name__}")
+  if not t.is_cuda:
+    raise ValueError(f"{name} must live on the GPU (got device {t.device}); "
+                     "this operator has no CPU path")
+
+
+def _inner_contiguous(t):
+  return t if t.stride(-1) == 1 else t.contiguous()
+
+
+def _as_table(name, t, H, width, device):
+  """fp32 [heads, width] table with heads in {1, H}."""
+  _check_gpu(name, t)
+  if t.dim() == 1:
+    t = t.unsqueeze(0)
+  if t.dim() != 2 or t.shape[0] not in (1, H):
+    raise ValueError(f"{name} must have shape [{width}] or [1|{H}, {width}], got {tuple(t.shape)}")
+  if width is not None and t.shape[1] != width:
+    raise ValueError(f"{name} must have {width} entries per head, got {t.shape[1]}")
+  return t.to(device=device, dtype=torch.float32).contiguous()
+
+
+def _run(args, keep):
+  lib = _lib.load()
+  ws = lib.hstu_attn_fwd_workspace_bytes(C.byref(args))
+  if ws:
+    buf = torch.empty(ws, dtype=torch.uint8, device=keep[0].device)
+    keep.append(buf)
+    args.workspace = buf.data_ptr()
+    args.workspace_bytes = ws
+  stream = torch.cuda.current_stream(keep[0].device).cuda_stream
+  rc = lib.hstu_attn_fwd(C.byref(args), C.c_void_p(stream))
+  if rc != 0:
+    msg = lib.hstu_attn_last_error().decode()
+    if rc in (-3, -4, -1):
+      raise ValueError(f"hstu_attn_fwd rejected the arguments ({rc}): {msg}")
+    raise RuntimeError(f"hstu_attn_fwd failed ({rc}): {msg}")
+
+
+def kernel_variant(args) -> str:
+  return _lib.load().hstu_attn_fwd_variant(C.byref(args)).decode()
+
+
+def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
+               n=None, alpha=1.0, inv_n=None, causal=True, pos_bias=None,
+               timestamps=None, ts_bias=None, ts_bucket_size=0.301,
+               q_segment_ids=None, kv_segment_ids=None,
+               sliding_window_size=None, mask=None, bias=None):
+  """Validates the call and fills an HstuAttnFwdArgs.  Returns (args, keepalive)."""
+  for name, t in (("q", q), ("k", k), ("v", v)):
+    _check_gpu(name, t)
+  if q.dtype not in _DTYPES:
+    raise ValueError(f"unsupported dtype {q.dtype}: use float32 or bfloat16")
+  if k.dtype != q.dtype or v.dtype != q.dtype:
+    raise ValueError(f"q, k, v must share one dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+  keep = [q, k, v, out]
+  a = _lib.new_args()
+  dev = q.device
+  jagged = q.dim() == 3
+  if jagged:
+    if seq_offsets is None or max_len is None:
+      raise ValueError("jagged q/k/v ([T, H, d]) need seq_offsets and max_len")
+    T, H, d = q.shape
+    if k.shape != (T, H, d):
+      raise ValueError(f"k shape {tuple(k.shape)} does not match q {tuple(q.shape)}")
+    if v.shape[:2] != (T, H):
+      raise ValueError(f"v shape {tuple(v.shape)} does not match q {tuple(q.shape)}")
+    _check_gpu("seq_offsets", seq_offsets)
+    if seq_offsets.dim() != 1 or seq_offsets.numel() < 1:
+      raise ValueError("seq_offsets must have shape [B+1]")
+    seq_offsets = seq_offsets.to(torch.int32).contiguous()
+    keep.append(seq_offsets)
+    B, L, Lkv = seq_offsets.numel() - 1, int(max_len), int(max_len)
+    a.layout = _lib.LAYOUT_JAGGED
+    a.total_tokens = T
+    a.seq_offsets = seq_offsets.data_ptr()
+    a.mask_mode = _lib.MASK_LENGTH
+    if q_segment_ids is not None or kv_segment_ids is not None:
+      raise ValueError("segment ids need the padded layout")
+  else:
+    if q.dim() != 4:
+      raise ValueError(f"q must be [B, L, H, d] or [T, H, d], got {tuple(q.shape)}")
+    B, L, H, d = q.shape
+    if k.dim() != 4 or k.shape[0] != B or k.shape[2] != H or k.shape[3] != d:
+      raise ValueError(f"k shape {tuple(k.shape)} does not match q {tuple(q.shape)}")
+    Lkv = k.shape[1]
+    if v.dim() != 4 or v.shape[:3] != (B, Lkv, H):
+      raise ValueError(f"v shape {tuple(v.shape)} does not match k {tuple(k.shape)}")
+    if max_len is not None and int(max_len) != L:
+      raise ValueError(f"max_len={max_len} does not match the padded length {L}")
+    a.layout = _lib.LAYOUT_PADDED
+    if (q_segment_ids is None) != (kv_segment_ids is None):
+      raise ValueError("Both or neither of `q_segment_ids` and `kv_segment_ids` must be provided.")
+    if q_segment_ids is not None:
+      if seq_lens is not None:
+        raise ValueError("pass either seq_lens or segment ids, not both")
+      _check_gpu("q_segment_ids", q_segment_ids)
+      _check_gpu("kv_segment_ids", kv_segment_ids)
+      if tuple(q_segment_ids.shape) != (B, L):
+        raise ValueError(f"Invalid shape for q segment_ids: {tuple(q_segment_ids.shape)}. Expected: {(B, L)}")
+      if tuple(kv_segment_ids.shape) != (B, Lkv):
+        raise ValueError(f"Invalid shape for kv segment_ids: {tuple(kv_segment_ids.shape)}. Expected: {(B, Lkv)}")
+      qs = q_segment_ids.to(torch.int32).contiguous()
+      ks = kv_segment_ids.to(torch.int32).contiguous()
+      keep += [qs, ks]
+      a.q_segment_ids, a.kv_segment_ids = qs.data_ptr(), ks.data_ptr()
+      a.mask_mode = _lib.MASK_SEGMENT
+    elif seq_lens is not None:
+      _check_gpu("seq_lens", seq_lens)
+      if tuple(seq_lens.shape) != (B,):
+        raise ValueError(f"seq_lens must have shape [{B}], got {tuple(seq_lens.shape)}")
+      sl = seq_lens.to(torch.int32).contiguous()
+      keep.append(sl)
+      a.seq_lens = sl.data_ptr()
+      a.mask_mode = _lib.MASK_LENGTH
+    else:
+      a.mask_mode = _lib.MASK_NONE
+  d_v = v.shape[-1]
+  exp_out = (q.shape[0], H, d_v) if jagged else (B, L, H, d_v)
+  if tuple(out.shape) != exp_out or out.dtype != q.dtype or not out.is_cuda:
+    raise ValueError(f"out must be a {q.dtype} GPU tensor of shape {exp_out}")
+
+  q, k, v = (_inner_contiguous(t) for t in (q, k, v))
+  if out.stride(-1) != 1:
+    raise ValueError("out must be contiguous in its last dimension")
+  keep += [q, k, v]
+  a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
+  a.qk_dtype = a.v_dtype = a.out_dtype = _DTYPES[q.dtype]
+  for name, t in (("q", q), ("k", k), ("v", v), ("o", out)):
+    if jagged:
+      sb, st, sh = 0, t.stride(0), t.stride(1)
+    else:
+      sb, st, sh = t.stride(0), t.stride(1), t.stride(2)
+    setattr(a, f"{name}_stride_b", sb)
+    setattr(a, f"{name}_stride_t", st)
+    setattr(a, f"{name}_stride_h", sh)
+  a.B, a.L, a.Lkv, a.H, a.d_qk, a.d_v = B, L, Lkv, H, d, d_v
+
+  a.alpha = float(alpha)
+  if inv_n is None:
+    n = L if n is None else n
+    if not n > 0:
+      raise ValueError(f"normaliser n must be positive, got {n}")
+    inv_n = 1.0 / float(n)
+  a.inv_n = float(inv_n)
+  a.causal = 1 if causal else 0
+  if sliding_window_size is not None:
+    if int(sliding_window_size) < 0:
+      raise ValueError("sliding_window_size must be >= 0")
+    a.window = int(sliding_window_size)
+
+  if mask is not None:
+    if isinstance(mask, np.ndarray):
+      mask = torch.from_numpy(np.ascontiguousarray(mask)).to(dev)
+    _check_gpu("mask", mask)
+    if mask.dim() == 2:
+      if tuple(mask.shape) != (L, Lkv):
+        raise ValueError(f"Mask shape {tuple(mask.shape)} does not match query and key length ({L}, {Lkv}).")
+      a.mask_batched = 0
+    elif mask.dim() == 3 and tuple(mask.shape) == (B, L, Lkv):
+      a.mask_batched = 1
+    else:
+      raise ValueError(f"mask must be [{L}, {Lkv}] or [{B}, {L}, {Lkv}], got {tuple(mask.shape)}")
+    m8 = (mask != 0).to(torch.uint8).contiguous()
+    keep.append(m8)
+    a.mask = m8.data_ptr()
+  if bias is not None:
+    _check_gpu("bias", bias)
+    if bias.dim() == 2:
+      bias = bias.unsqueeze(0)
+    if bias.dim() != 3 or tuple(bias.shape[1:]) != (L, Lkv) or bias.shape[0] not in (1, B):
+      raise ValueError(f"bias must be [{L}, {Lkv}] or [1|{B}, {L}, {Lkv}], got {tuple(bias.shape)}")
+    bf = bias.to(torch.float32).contiguous()
+    keep.append(bf)
+    a.dense_bias = bf.data_ptr()
+    a.dense_bias_batched = 1 if bias.shape[0] == B and B > 1 else 0
+  if pos_bias is not None:
+    if L != Lkv:
+      raise ValueError("relative-position bias needs q_len == kv_len")
+    pt = _as_table("pos_bias", pos_bias, H, 2 * L - 1, dev)
+    keep.append(pt)
+    a.pos_tab, a.pos_heads = pt.data_ptr(), pt.shape[0]
+  if (timestamps is None) != (ts_bias is None):
+    raise ValueError("Both or neither of `timestamps` and `ts_bias` must be provided.")
+  if ts_bias is not None:
+    if L != Lkv:
+      raise ValueError("timestamp bias needs q_len == kv_len")
+    tt = _as_table("ts_bias", ts_bias, H, None, dev)
+    _check_gpu("timestamps", timestamps)
+    ts = timestamps.to(torch.int64).contiguous()
+    if ts.dim() == 2 and tuple(ts.shape) == (B, L):
+      a.ts_stride_b = L
+    elif ts.dim() == 1 and jagged and ts.numel() == q.shape[0]:
+      a.ts_stride_b = 0
+    else:
+      raise ValueError(f"timestamps must be [{B}, {L}]" + (f" or [{q.shape[0]}]" if jagged else "")
+                       + f", got {tuple(ts.shape)}")
+    keep += [tt, ts]
+    a.ts_tab, a.ts_heads, a.ts = tt.data_ptr(), tt.shape[0], ts.data_ptr()
+    a.ts_num_buckets = tt.shape[1] - 1
+    a.ts_bucket_size = float(ts_bucket_size)
+  return a, keep
+
+
+def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
+                   n=None, alpha=1.0, causal=True, pos_bias=None,
+                   timestamps=None, ts_bias=None, ts_bucket_size=0.301,
+                   q_segment_ids=None, kv_segment_ids=None,
+                   sliding_window_size=None, mask=None, bias=None, out=None):
+  """out = (silu(alpha * q k^T + bias) / n, masked) v.
+
+  Args:
+    q, k, v: padded [B, L, H, d] or jagged [T, H, d] (with `seq_offsets`
+      [B+1] and `max_len`); float32 or bfloat16 GPU tensors.
+    seq_lens: int [B] valid lengths of an end-padded batch.  Rows and keys at
+      or beyond the length are ignored and output rows there are exactly 0,
+      as with make_causal_mask (recml/layers/keras/utils.py:39-41).
+    n: the normaliser N; defaults to the padded length
+      (recml/layers/keras/hstu.py:377-378).
+    alpha: logit scale (1, or 1/sqrt(d) for the scaled variant, hstu.py:365-369).
+    causal: keep j <= i.
+    pos_bias: [2L-1] or [H, 2L-1] table; logit (i, j) gets
+      pos_bias[(L-1) + j - i] (hstu.py:91-113).
+    timestamps, ts_bias: int64 [B, L] (or jagged [T]) and [nb+1] or
+      [H, nb+1]; logit (i, j) gets ts_bias[bucket(ts[i+1] - ts[j])]
+      (hstu.py:190-221).  Jagged timestamps use the sequence's own last
+      timestamp for its last row.
+    q_segment_ids, kv_segment_ids: int [B, L] / [B, Lkv]; keep equal ids
+      (recml/core/ops/hstu_ops.py:972-979).  Both or neither.
+    sliding_window_size: keep |i - j| <= w (hstu_ops.py:940-945).
+    mask: explicit keep-mask [L, Lkv] or [B, L, Lkv].
+    bias: dense additive logit bias [L, Lkv] or [B, L, Lkv] shared by heads
+      (hstu.py:373-374).
+    out: optional preallocated output.
+
+  Returns:
+    Tensor shaped like q with v's head dim, same dtype as q.
+  """
+  _check_gpu("q", q)
+  _check_gpu("v", v)
+  if out is None:
+    shape = tuple(q.shape[:-1]) + (v.shape[-1],)
+    out = torch.empty(shape, dtype=q.dtype, device=q.device)
+  args, keep = build_args(
+      q, k, v, out, seq_lens=seq_lens, seq_offsets=seq_offsets,
+      max_len=max_len, n=n, alpha=alpha, causal=causal, pos_bias=pos_bias,
+      timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
+      q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids,
+      sliding_window_size=sliding_window_size, mask=mask, bias=bias)
+  with torch.cuda.device(q.device):
+    _run(args, keep)
+  return out
+
+
+def pointwise_splash_attention(
+    mask_type, q, k, v, *,
+    q_segment_ids=None, kv_segment_ids=None, sliding_window_size=None,
+    qkv_axis_names=(), segment_id_axis_names=(), scale=None,
+    block_q=None, block_kv=None, block_kv_compute=None, block_q_dkv=None,
+    block_kv_dkv=None, block_kv_dkv_compute=None, head_shards=1,
+    q_seq_shards=1, downcast_smem_data=True, interpret=False):
+  """Drop-in for recml/core/ops/hstu_ops.py:829-851 (forward).
+
+  out = (silu(scale * q k^T) / q_len, masked) v with scale defaulting to
+  1/sqrt(head_dim) (hstu_ops.py:909, 238).  `mask_type` is MaskType.CAUSAL,
+  MaskType.FULL or an explicit boolean [q_len, kv_len] array.  The tile-size,
+  sharding and interpret arguments belong to the TPU kernel and are accepted
+  and ignored.
+  """
+  del qkv_axis_names, segment_id_axis_names, block_q, block_kv
+  del block_kv_compute, block_q_dkv, block_kv_dkv, block_kv_dkv_compute
+  del head_shards, q_seq_shards, downcast_smem_data, interpret
+  _check_gpu("q", q)
+  if q.dim() != 4:
+    raise ValueError(f"q must be [batch, q_length, num_heads, head_dim], got {tuple(q.shape)}")
+  bs, q_len, num_heads, head_dim = q.shape
+  kv_len = v.shape[1] if v.dim() == 4 else -1
+  for name, t in (("k", k), ("v", v)):
+    if tuple(t.shape) != (bs, kv_len, num_heads, head_dim):
+      raise ValueError(f"{name} shape {tuple(t.shape)} does not match {(bs, kv_len, num_heads, head_dim)}")
+  explicit = None
+  if isinstance(mask_type, (np.ndarray, torch.Tensor)):
+    if tuple(mask_type.shape) != (q_len, kv_len):
+      raise ValueError(
+          f"Mask shape {tuple(mask_type.shape)} does not match query and key length ({q_len}, {kv_len}).")
+    explicit, causal = mask_type, False
+  elif mask_type == MaskType.CAUSAL:
+    causal = True
+  elif mask_type == MaskType.FULL:
+    causal = False
+  else:
+    raise ValueError(f"Unsupported mask type: '{mask_type}'.")
+  scale = scale if scale is not None else 1.0 / (head_dim**0.5)
+  return hstu_attention(
+      q, k, v, n=q_len, alpha=scale, causal=causal, mask=explicit,
+      q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids,
+      sliding_window_size=sliding_window_size)
+
+
+def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
+                        scaled_pointwise_attn=False, seq_lens=None):
+  """Layer-side call, recml/layers/keras/hstu.py:356-390 (inference).
+
+  `attention_mask` is the [B, L, L] 0/1 mask the layer builds with
+  make_causal_mask; `attention_bias` an optional [B or 1, L, L] additive bias
+  shared by heads.  scaled_pointwise_attn=True divides q by sqrt(d) and skips
+  the 1/L (hstu.py:365-378).  A caller that knows its batch is end-padded and
+  causal can pass `seq_lens` with attention_mask=None: same result without
+  ever building the [B, L, L] mask.
+  """
+  d = q.shape[-1]
+  alpha = 1.0 / math.sqrt(d) if scaled_pointwise_attn else 1.0
+  n = 1.0 if scaled_pointwise_attn else q.shape[1]
+  if attention_mask is None:
+    if seq_lens is None:
+      raise ValueError("pass attention_mask or seq_lens")
+    return hstu_attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha,
+                          causal=True, bias=attention_bias)
+  return hstu_attention(q, k, v, n=n, alpha=alpha, causal=False,
+                        mask=attention_mask, bias=attention_bias)

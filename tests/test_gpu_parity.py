@@ -1,0 +1,327 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle.
+
+Tolerances (stated once, used everywhere below):
+  fp32   max|out-ref| <= 1e-5 * max|ref|
+  bf16   max|out-ref| <= 2e-2 * max|ref|   (inputs rounded to bf16 for both)
+  masked / padded output positions are exactly 0.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import recml_amd
+from recml_amd import hstu_ops, workloads
+from oracle import hstu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def _dev(x, dtype=None, dev="cuda:0"):
+  if x is None:
+    return None
+  t = torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+  return t if dtype is None else t.to(dtype)
+
+
+def _err(out, ref):
+  ref = np.asarray(ref, dtype=np.float64)
+  out = np.asarray(out, dtype=np.float64)
+  return np.abs(out - ref).max() / max(np.abs(ref).max(), 1e-30)
+
+
+def _store(x, dtype):
+  """fp32 master -> what the kernel and the oracle both see."""
+  return O.round_bf16(x) if dtype == torch.bfloat16 else np.asarray(x, np.float32)
+
+
+def run_workload(w, dtype, **over):
+  q, k, v = (_store(t, dtype) for t in (w.q, w.k, w.v))
+  kw = dict(n=w.n, alpha=w.alpha, pos_bias=_dev(w.pos_tab),
+            ts_bias=_dev(w.ts_tab), timestamps=_dev(w.timestamps))
+  if w.layout == "jagged":
+    kw.update(seq_offsets=_dev(w.seq_offsets), max_len=w.L)
+  else:
+    kw.update(seq_lens=_dev(w.seq_lens))
+  kw.update(over)
+  out = recml_amd.hstu_attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), **kw)
+  torch.cuda.synchronize()
+  return q, k, v, out.float().cpu().numpy()
+
+
+def oracle_workload(w, q, k, v, dtype=np.float64, sequences=None):
+  if w.layout == "jagged":
+    return O.hstu_attention_jagged_ref(
+        q, k, v, w.seq_offsets, w.L, n=w.n, alpha=w.alpha, pos_tab=w.pos_tab,
+        timestamps=w.timestamps, ts_tab=w.ts_tab, dtype=dtype, sequences=sequences)
+  return O.hstu_attention_ref(
+      q, k, v, seq_lens=w.seq_lens, n=w.n, alpha=w.alpha, pos_tab=w.pos_tab,
+      timestamps=w.timestamps, ts_tab=w.ts_tab, dtype=dtype)
+
+
+# ---- configuration 1: fp32, the reference's CPU-runnable case
+
+
+def test_config1_fp32(gpu):
+  w = workloads.config1()
+  q, k, v, out = run_workload(w, torch.float32)
+  ref = oracle_workload(w, q, k, v)
+  assert _err(out, ref) <= FP32_TOL
+  # same inputs through the bf16 MFMA kernel
+  qb, kb, vb, outb = run_workload(w, torch.bfloat16)
+  assert _err(outb, oracle_workload(w, qb, kb, vb)) <= BF16_TOL
+
+
+def test_golden_config1(gpu):
+  g = np.load("tests/golden/config1_fp64.npz")
+  w = workloads.config1()
+  _, _, _, out = run_workload(w, torch.float32)
+  assert _err(out, g["out"]) <= FP32_TOL
+
+
+def test_golden_small_jagged(gpu):
+  g = np.load("tests/golden/small_jagged_fp64.npz")
+  w = workloads.small_jagged()
+  _, _, _, out = run_workload(w, torch.float32)
+  assert _err(out, g["out"]) <= FP32_TOL
+  _, _, _, outb = run_workload(w, torch.bfloat16)
+  assert _err(outb, g["out_bf16_inputs"]) <= BF16_TOL
+
+
+# ---- configuration 2: bf16 padded + per-head position bias
+
+
+def test_config2_bf16_padded_pos_bias(gpu):
+  w = workloads.config2()
+  q, k, v, out = run_workload(w, torch.bfloat16)
+  ref = oracle_workload(w, q, k, v, dtype=np.float32)
+  assert _err(out, ref) <= BF16_TOL
+  for b in range(w.B):
+    assert (out[b, w.seq_lens[b]:] == 0).all(), "padded rows must be exact zeros"
+  # padding content is ignored: poison it
+  q2, k2, v2 = (t.copy() for t in (w.q, w.k, w.v))
+  for b in range(w.B):
+    q2[b, w.seq_lens[b]:] = np.nan
+    k2[b, w.seq_lens[b]:] = np.inf
+    v2[b, w.seq_lens[b]:] = np.nan
+  w2 = workloads.Workload(**{**w.__dict__, "q": q2, "k": k2, "v": v2})
+  _, _, _, out2 = run_workload(w2, torch.bfloat16)
+  np.testing.assert_array_equal(out, out2)
+
+
+def test_config2_general_kernel_agrees(gpu):
+  # same workload in fp32 storage goes through the general kernel
+  w = workloads.config2()
+  q, k, v, out = run_workload(w, torch.float32)
+  ref = oracle_workload(w, q, k, v, dtype=np.float64)
+  assert _err(out, ref) <= FP32_TOL
+
+
+# ---- configuration 3: jagged, power-law lengths, position + timestamp bias
+
+
+def test_config3_reduced_fp32_and_bf16(gpu):
+  w = workloads.config3(B=8, L=512, H=2, d=128)
+  q, k, v, out = run_workload(w, torch.float32)
+  ref = oracle_workload(w, q, k, v)
+  assert _err(out, ref) <= FP32_TOL
+  qb, kb, vb, outb = run_workload(w, torch.bfloat16)
+  assert _err(outb, oracle_workload(w, qb, kb, vb)) <= BF16_TOL
+
+
+def test_config3_full_size_bf16(gpu):
+  w = workloads.config3()
+  q, k, v, out = run_workload(w, torch.bfloat16)
+  # oracle on the longest, the shortest and two middle sequences
+  order = np.argsort(w.seq_lens)
+  pick = [int(order[-1]), int(order[0]), int(order[len(order) // 2]), int(order[-2])]
+  ref = oracle_workload(w, q, k, v, dtype=np.float32, sequences=pick)
+  scale = np.abs(ref).max()
+  for b in pick:
+    s, e = w.seq_offsets[b], w.seq_offsets[b + 1]
+    assert np.abs(out[s:e] - ref[s:e]).max() / scale <= BF16_TOL, f"sequence {b}"
+  assert np.isfinite(out).all()
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("causal", [True, False])
+def test_mfma_head_dims_and_full_mask(gpu, d, causal):
+  rng = np.random.default_rng(100 + d)
+  B, L, H = 3, 200, 2
+  lens = np.array([200, 77, 1], dtype=np.int32)
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
+                                 seq_lens=_dev(lens), causal=causal, n=50)
+  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, causal=causal, n=50)
+  assert _err(out.float().cpu().numpy(), ref) <= BF16_TOL
+
+
+def test_ragged_and_empty(gpu):
+  rng = np.random.default_rng(5)
+  H, d, L = 2, 64, 300
+  lens = np.array([0, 1, 300, 0, 129, 64], dtype=np.int32)
+  off = np.zeros(len(lens) + 1, dtype=np.int32)
+  off[1:] = np.cumsum(lens)
+  T = int(off[-1])
+  q, k, v = (O.round_bf16(rng.standard_normal((T, H, d)).astype(np.float32) * 0.2) for _ in range(3))
+  pos = rng.standard_normal((H, 2 * L - 1)).astype(np.float32) * 0.1
+  for dt in (torch.bfloat16, torch.float32):
+    out = recml_amd.hstu_attention(_dev(q, dt), _dev(k, dt), _dev(v, dt), seq_offsets=_dev(off),
+                                   max_len=L, pos_bias=_dev(pos))
+    ref = O.hstu_attention_jagged_ref(q, k, v, off, L, pos_tab=pos)
+    assert _err(out.float().cpu().numpy(), ref) <= (BF16_TOL if dt == torch.bfloat16 else FP32_TOL)
+  # an empty batch and an all-empty batch are no-ops
+  e = torch.empty((0, H, d), dtype=torch.bfloat16, device="cuda:0")
+  o = recml_amd.hstu_attention(e, e, e, seq_offsets=_dev(np.zeros(3, np.int32)), max_len=L)
+  assert o.shape == (0, H, d)
+
+
+def test_jagged_equals_padded_on_gpu(gpu):
+  w = workloads.config3(B=6, L=384, H=2, d=64)
+  q, k, v, outj = run_workload(w, torch.bfloat16)
+  L = w.L
+  qp, kp, vp = (O.jagged_to_padded(t, w.seq_offsets, L) for t in (q, k, v))
+  tsp = O.jagged_to_padded(w.timestamps, w.seq_offsets, L)
+  for b in range(w.B):
+    tsp[b, w.seq_lens[b]:] = tsp[b, w.seq_lens[b] - 1]
+  outp = recml_amd.hstu_attention(
+      _dev(qp, torch.bfloat16), _dev(kp, torch.bfloat16), _dev(vp, torch.bfloat16),
+      seq_lens=_dev(w.seq_lens), n=w.n, pos_bias=_dev(w.pos_tab), ts_bias=_dev(w.ts_tab),
+      timestamps=_dev(tsp)).float().cpu().numpy()
+  np.testing.assert_array_equal(O.jagged_to_padded(outj, w.seq_offsets, L), outp)
+
+
+# ---- operator options (general kernel)
+
+
+def test_splash_signature_segment_ids(gpu):
+  # the reference's own test recipe (hstu_ops_test.py:29-58) at a smaller shape
+  rng = np.random.default_rng(42)
+  B, L, H, d = 8, 256, 2, 128
+  q, k, v = (rng.standard_normal((B, L, H, d)).astype(np.float32) for _ in range(3))
+  lens = (rng.random(B) * L).astype(np.int64)
+  seg = (np.arange(L)[None] < lens[:, None]).astype(np.int32)
+  out = recml_amd.pointwise_splash_attention(
+      recml_amd.MaskType.CAUSAL, _dev(q), _dev(k), _dev(v),
+      q_segment_ids=_dev(seg), kv_segment_ids=_dev(seg))
+  ref = O.pw_attn_ref(q, k, v, seg)
+  o = out.cpu().numpy()
+  # the reference accepts atol=rtol=5e-3 here (hstu_ops_test.py:80-83); we hold 1e-5
+  assert _err(o, ref) <= FP32_TOL
+  np.testing.assert_allclose(o, ref, atol=5e-3, rtol=5e-3)
+  # bf16 storage goes through the same kernel
+  qb, kb, vb = (O.round_bf16(t) for t in (q, k, v))
+  outb = recml_amd.pointwise_splash_attention(
+      "causal", _dev(qb, torch.bfloat16), _dev(kb, torch.bfloat16), _dev(vb, torch.bfloat16),
+      q_segment_ids=_dev(seg), kv_segment_ids=_dev(seg))
+  assert _err(outb.float().cpu().numpy(), O.pw_attn_ref(qb, kb, vb, seg)) <= BF16_TOL
+
+
+def test_splash_full_explicit_window_cross_length(gpu):
+  rng = np.random.default_rng(43)
+  B, Lq, Lk, H, d = 2, 70, 95, 3, 48
+  q = rng.standard_normal((B, Lq, H, d)).astype(np.float32)
+  k = rng.standard_normal((B, Lk, H, d)).astype(np.float32)
+  v = rng.standard_normal((B, Lk, H, d)).astype(np.float32)
+  alpha = 1 / math.sqrt(d)
+  out = recml_amd.pointwise_splash_attention(recml_amd.MaskType.FULL, _dev(q), _dev(k), _dev(v))
+  ref = O.hstu_attention_ref(q, k, v, causal=False, alpha=alpha, n=Lq)
+  assert _err(out.cpu().numpy(), ref) <= FP32_TOL
+  m = rng.random((Lq, Lk)) < 0.4
+  out = recml_amd.pointwise_splash_attention(m, _dev(q), _dev(k), _dev(v), scale=0.2)
+  ref = O.hstu_attention_ref(q, k, v, causal=False, mask=m, alpha=0.2, n=Lq)
+  assert _err(out.cpu().numpy(), ref) <= FP32_TOL
+  for wdw in (0, 5, 64):
+    out = recml_amd.pointwise_splash_attention("causal", _dev(q), _dev(k), _dev(v), sliding_window_size=wdw)
+    ref = O.hstu_attention_ref(q, k, v, causal=True, sliding_window_size=wdw, alpha=alpha, n=Lq)
+    assert _err(out.cpu().numpy(), ref) <= FP32_TOL
+    out = recml_amd.pointwise_splash_attention("full", _dev(q), _dev(k), _dev(v), sliding_window_size=wdw)
+    ref = O.hstu_attention_ref(q, k, v, causal=False, sliding_window_size=wdw, alpha=alpha, n=Lq)
+    assert _err(out.cpu().numpy(), ref) <= FP32_TOL
+
+
+def test_layer_call_dense_mask_and_bias(gpu):
+  # HSTUBlock._pointwise_attention (hstu.py:356-390): dense [B,L,L] mask + bias
+  rng = np.random.default_rng(44)
+  B, L, H, d = 3, 50, 2, 32
+  q, k, v = (rng.standard_normal((B, L, H, d)).astype(np.float32) for _ in range(3))
+  lens = np.array([50, 20, 1])
+  pad = (np.arange(L)[None] < lens[:, None]).astype(np.float32)
+  mask = recml_amd.make_causal_mask(_dev(pad))
+  np.testing.assert_array_equal(mask.cpu().numpy(), O.make_causal_mask(pad))
+  bias = rng.standard_normal((B, L, L)).astype(np.float32)
+  for scaled in (False, True):
+    out = recml_amd.pointwise_attention(_dev(q), _dev(k), _dev(v), mask, _dev(bias),
+                                        scaled_pointwise_attn=scaled)
+    ref = O.pointwise_attention_dense(q, k, v, O.make_causal_mask(pad), bias, scaled=scaled)
+    assert _err(out.cpu().numpy(), ref) <= FP32_TOL
+    for b in range(B):
+      assert (out[b, lens[b]:] == 0).all()
+  # same result from lengths, never building the mask
+  out2 = recml_amd.pointwise_attention(_dev(q), _dev(k), _dev(v), None, _dev(bias), seq_lens=_dev(lens))
+  ref = O.pointwise_attention_dense(q, k, v, O.make_causal_mask(pad), bias)
+  assert _err(out2.cpu().numpy(), ref) <= FP32_TOL
+
+
+def test_shared_tables_and_strided_inputs(gpu):
+  rng = np.random.default_rng(45)
+  B, L, H, d = 2, 130, 4, 64
+  lens = np.array([130, 61], dtype=np.int32)
+  qkv = O.round_bf16(rng.standard_normal((B, L, 3, H, d)).astype(np.float32) * 0.3)
+  pos = rng.standard_normal(2 * L - 1).astype(np.float32) * 0.1
+  tst = rng.standard_normal(129).astype(np.float32) * 0.1
+  ts = np.cumsum(rng.integers(1, 10**5, (B, L)), axis=1).astype(np.int64)
+  t = _dev(qkv, torch.bfloat16)
+  out = recml_amd.hstu_attention(t[:, :, 0], t[:, :, 1], t[:, :, 2], seq_lens=_dev(lens),
+                                 pos_bias=_dev(pos), ts_bias=_dev(tst), timestamps=_dev(ts))
+  ref = O.hstu_attention_ref(qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2], seq_lens=lens,
+                             pos_tab=pos, ts_tab=tst, timestamps=ts)
+  assert _err(out.float().cpu().numpy(), ref) <= BF16_TOL
+
+
+def test_timestamp_buckets_on_gpu(gpu):
+  # one key, zero q: out = silu(ts_tab[bucket]) * v / n  reveals the bucket per delta
+  th = O.bucket_thresholds()
+  deltas = np.concatenate([[0, 1, 2, 3, 10, 3600, 86400, 10**9, 2 * 10**9, 5 * 10**12],
+                           th[1:], th[1:] - 1, th[1:] + 1]).astype(np.int64)
+  far = ~O.near_bucket_boundary(deltas)
+  table = (np.arange(129) + 1).astype(np.float32) / 64.0
+  for dt_, tol in ((torch.float32, FP32_TOL), (torch.bfloat16, BF16_TOL)):
+    for sign in (1, -1):
+      B = len(deltas)
+      ts = np.zeros((B, 2), dtype=np.int64)
+      ts[:, 0] = 1_600_000_000
+      ts[:, 1] = ts[:, 0] + sign * deltas      # row 0 sees ts[1] - ts[0]
+      q = np.zeros((B, 2, 1, 32), np.float32)
+      v = np.ones((B, 2, 1, 32), np.float32)
+      out = recml_amd.hstu_attention(_dev(q, dt_), _dev(q, dt_), _dev(v, dt_), ts_bias=_dev(table),
+                                     timestamps=_dev(ts), n=1).float().cpu().numpy()[:, 0, 0, 0]
+      want = O.silu(table[np.clip(O.bucketize_law(deltas), 0, 128)].astype(np.float64))
+      lo = O.silu(table[np.clip(O.bucketize_law(deltas) - 1, 0, 128)].astype(np.float64))
+      hi = O.silu(table[np.clip(O.bucketize_law(deltas) + 1, 0, 128)].astype(np.float64))
+      rel = np.abs(out - want) / want
+      assert (rel[far] <= max(tol, 1e-5) * 1.0 + (4e-3 if dt_ == torch.bfloat16 else 0)).all()
+      near_ok = np.minimum(np.minimum(np.abs(out - want), np.abs(out - lo)), np.abs(out - hi)) / want
+      assert (near_ok <= 5e-3).all()
+
+
+def test_argument_errors(gpu):
+  z = torch.zeros((2, 8, 2, 32), device="cuda:0")
+  seg = torch.ones((2, 8), dtype=torch.int32, device="cuda:0")
+  with pytest.raises(ValueError, match="Both or neither"):
+    recml_amd.pointwise_splash_attention("causal", z, z, z, q_segment_ids=seg)
+  with pytest.raises(ValueError, match="Mask shape"):
+    recml_amd.pointwise_splash_attention(np.ones((7, 8), bool), z, z, z)
+  with pytest.raises(ValueError, match="Unsupported mask type"):
+    recml_amd.pointwise_splash_attention("banded", z, z, z)
+  with pytest.raises(ValueError):
+    recml_amd.hstu_attention(z, z[:, :, :1], z)
+  with pytest.raises(ValueError):
+    recml_amd.hstu_attention(z.cpu(), z, z)
+  with pytest.raises(ValueError):
+    recml_amd.hstu_attention(z.double(), z.double(), z.double())

@@ -608,7 +608,9 @@ int validate(const HstuAttnFwdArgs* a) {
   if (a->struct_size != sizeof(HstuAttnFwdArgs) || a->version != HSTU_ATTN_ABI_VERSION)
     return fail(HSTU_ERR_VERSION, "args struct_size/version (%u/%u) do not match this library (%zu/%d)",
                 a->struct_size, a->version, sizeof(HstuAttnFwdArgs), HSTU_ATTN_ABI_VERSION);
-  if (!a->q || !a->k || !a->v || !a->out) return fail(HSTU_ERR_NULL, "q, k, v and out must be non-null");
+  const bool empty = a->B == 0 || (a->layout == HSTU_LAYOUT_JAGGED && a->total_tokens == 0);
+  if (!empty && (!a->q || !a->k || !a->v || !a->out))
+    return fail(HSTU_ERR_NULL, "q, k, v and out must be non-null");
   if (a->B < 0 || a->L < 1 || a->Lkv < 1 || a->H < 1)
     return fail(HSTU_ERR_SHAPE, "bad shape B=%d L=%d Lkv=%d H=%d", a->B, a->L, a->Lkv, a->H);
   if (a->d_qk < 1 || a->d_qk > 256 || a->d_v < 1 || a->d_v > 256)

@@ -1,0 +1,186 @@
+"""Benchmark of the HSTU attention forward on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c3full|c2|c4|c5]
+
+A step is one pass of the attention forward over one synthetic batch whose
+inputs already sit in HBM.  The default workload is the one the headline
+metric is quoted on: B=64, max_len=2048, H=8, d=128 bf16, jagged power-law
+lengths, relative-position + timestamp bias, N=2048.  Prints ONE JSON line.
+
+FLOPs counted: sum_b H * n_b(n_b+1)/2 * (2 d_qk + 2 d_v) (unmasked causal
+pairs only; bias, SiLU and mask are not counted).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def make_workload(name):
+  from recml_amd import workloads
+  if name == "c3":
+    return workloads.config3()
+  if name == "c3full":
+    return workloads.config3(full=True)
+  if name == "c3full-nobias":
+    return workloads.config3(full=True, bias=False)
+  if name == "c3-nobias":
+    return workloads.config3(bias=False)
+  if name == "c2":
+    return workloads.config2()
+  if name == "c4":
+    return workloads.config4_attention()
+  if name == "c5":
+    return workloads.config5()
+  raise SystemExit(f"unknown workload {name}")
+
+
+def to_device(w, dev):
+  import torch
+  t = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+  q, k, v = (t(x).to(torch.bfloat16) for x in (w.q, w.k, w.v))
+  kw = dict(n=w.n, alpha=w.alpha, pos_bias=t(w.pos_tab), ts_bias=t(w.ts_tab),
+            timestamps=t(w.timestamps))
+  if w.layout == "jagged":
+    kw.update(seq_offsets=t(w.seq_offsets), max_len=w.L)
+  else:
+    kw.update(seq_lens=t(w.seq_lens))
+  return q, k, v, kw
+
+
+def cpu_baseline(w, q, k, v, out_gpu):
+  """The C restatement of the op (oracle/hstu_oracle.c, float accumulation,
+  OpenMP over sequence x head) timed on this host, and used as the checker."""
+  from oracle import c_oracle
+  threads = c_oracle.max_threads()
+  qf, kf, vf = (x.float().cpu().numpy() for x in (q, k, v))
+  kw = dict(n=w.n, alpha=w.alpha, pos_tab=w.pos_tab, timestamps=w.timestamps,
+            ts_tab=w.ts_tab, acc="f32")
+  if w.layout == "jagged":
+    kw.update(seq_offsets=w.seq_offsets, max_len=w.L)
+  else:
+    kw.update(seq_lens=w.seq_lens)
+  # bounded sample: whole batches until ~10 s or 3 repetitions
+  times = []
+  ref = None
+  t_all = time.perf_counter()
+  while len(times) < 3 and time.perf_counter() - t_all < 10.0:
+    t0 = time.perf_counter()
+    ref = c_oracle.hstu_attention_c(qf, kf, vf, **kw)
+    times.append(time.perf_counter() - t0)
+  best = min(times)
+  err = float(np.abs(out_gpu - ref).max() / max(np.abs(ref).max(), 1e-30))
+  return {
+      "value": w.flops / best / 1e12, "unit": "TFLOP/s", "cores": threads,
+      "kind": "port",
+      "sample": f"{len(times)} full batches of the same workload ({w.flops / 1e9:.1f} GFLOP each), "
+                f"best of {len(times)}, {best * 1e3:.0f} ms; C restatement with float accumulation, "
+                "masked work skipped",
+      "seqs_per_s": w.B / best,
+  }, err
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=200)
+  ap.add_argument("--warmup", type=int, default=20)
+  ap.add_argument("--workload", default="c3")
+  ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+  args = ap.parse_args()
+  if args.gpus != 1:
+    raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
+                     "(the forward shards over (sequence, head) with no exchange); run with --gpus 1")
+
+  import torch
+  import recml_amd
+  from recml_amd import hstu_ops
+
+  if not torch.cuda.is_available():
+    raise SystemExit("bench.py needs a GPU")
+  dev = torch.device("cuda:0")
+  w = make_workload(args.workload)
+  q, k, v, kw = to_device(w, dev)
+  out = torch.empty_like(q)
+  call_args, keep = hstu_ops.build_args(q, k, v, out, **kw)
+  variant = hstu_ops.kernel_variant(call_args)
+
+  def step():
+    hstu_ops._run(call_args, keep)
+
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+
+  # whole-region wall clock and per-launch HIP events on the launch stream
+  starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+  ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for i in range(args.steps):
+    starts[i].record()
+    step()
+    ends[i].record()
+  torch.cuda.synchronize()
+  wall = time.perf_counter() - t0
+  ev_ms = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+  region_ms = starts[0].elapsed_time(ends[-1])
+
+  ms_per_step = wall * 1e3 / args.steps
+  kernel_ms = float(ev_ms.mean())
+  flops = w.flops
+  tflops = flops / (ms_per_step * 1e-3) / 1e12
+  achieved = flops / (kernel_ms * 1e-3) / 1e12
+  bytes_alg = w.bytes_moved(2)
+  ai = flops / bytes_alg
+  capped_peak = min(PEAK_BF16_TFLOPS, ai * PEAK_HBM_GBS / 1e3)
+
+  rec = {
+      "metric": "HSTU attn fwd TFLOP/s (unmasked), L=%d bf16" % w.L,
+      "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+      "warmup": args.warmup, "ms_per_step": ms_per_step,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": f"{w.name}: B={w.B} max_len={w.L} H={w.H} d={w.d} {w.layout} "
+                             f"lens mean {w.seq_lens.mean():.0f} max {w.seq_lens.max()}, causal, "
+                             f"pos_bias={'yes' if w.pos_tab is not None else 'no'} "
+                             f"ts_bias={'yes' if w.ts_tab is not None else 'no'} N={w.n} alpha={w.alpha}",
+                 "kernel": variant},
+      "seqs_per_s": w.B / (ms_per_step * 1e-3),
+      "roofline": {
+          "bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
+          "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+          "kernel_ms_avg": kernel_ms, "kernel_ms_min": float(ev_ms.min()),
+          "kernel_ms_median": float(np.median(ev_ms)),
+          "region_ms_per_step": region_ms / args.steps,
+          "algorithmic_flops": flops, "algorithmic_bytes": bytes_alg,
+          "arithmetic_intensity": ai,
+          "hbm_GBps_algorithmic": bytes_alg / (kernel_ms * 1e-3) / 1e9,
+          "roofline_capped_peak": capped_peak,
+          "frac_of_capped_peak": achieved / capped_peak,
+      },
+  }
+  if not args.no_cpu:
+    base, err = cpu_baseline(w, q, k, v, out.float().cpu().numpy())
+    rec["cpu_baseline"] = base
+    rec["parity_max_abs_over_max_ref"] = err
+    if not err <= 2e-2:
+      raise SystemExit(f"parity failed in the benchmark run: {err}")
+  print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+  main()

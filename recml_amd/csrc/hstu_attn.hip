@@ -30,6 +30,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "hstu_attn.h"
 
 namespace {
@@ -270,18 +272,33 @@ __global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
 
 // ---------------------------------------------------------------------------
 // MFMA kernel: bf16, causal/full + length masking, fused pos / timestamp bias.
+//
+// One workgroup = 2 wavefronts = 128 query rows; each wavefront owns 64 rows
+// (two 32-row blocks) so that every K / V fragment read from LDS feeds two
+// MFMAs.  Keys are streamed 64 at a time through a double-buffered LDS stage.
+//
+//   S^T[kv, q] = K Q^T   A = K fragment (LDS, 16-byte reads), B = Q (registers)
+//   O^T[dv, q] = V^T P^T A = V fragment (LDS transpose reads), B = P (registers)
+//
+// The 32x32 fp32 accumulator of S^T leaves lane (q = lane%32, half = lane/32)
+// holding keys 8g + 4*half + t (g, t in 0..3).  Read as the B operand of the
+// second product, those 16 values are two 16-key chunks whose k-slot e of
+// half h is key 16c + 8(e/4) + 4h + e%4 -- exactly what two 4-key transpose
+// reads of row-major V deliver.  P therefore never leaves registers.
 // ---------------------------------------------------------------------------
 
-constexpr int BM = 128;   // query rows per workgroup (4 waves x 32)
+constexpr int BM = 128;   // query rows per workgroup (2 waves x 64)
 constexpr int BN = 64;    // keys per step
 constexpr int POSW = 192; // staged window of the position table per step
+constexpr int MFMA_THREADS = 128;
+constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D>
 struct MfmaSmem {
-  static constexpr int KP = D + 8;    // K row pitch in bf16 (16 B pad)
-  static constexpr int VP = BN + 8;   // V^T row pitch in bf16
+  static constexpr int KP = D + 8;    // K row pitch in bf16: 16-byte reads, one row per lane
+  static constexpr int VP = D + 16;   // V row pitch in bf16: transpose reads of 8 rows x 64 bytes
   static constexpr int K_BYTES = BN * KP * 2;
-  static constexpr int V_BYTES = D * VP * 2;
+  static constexpr int V_BYTES = BN * VP * 2;
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int POS_BYTES = 4 * POSW * 4;
   static constexpr int TK_BYTES = BN * 8;
@@ -297,27 +314,37 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, r);
 }
 
-__device__ __forceinline__ float fast_silu(float x) {
-  // x * sigmoid(x) = x / (1 + 2^(-x*log2(e)))
-  float e = __builtin_amdgcn_exp2f(x * -1.4426950408889634f);
-  return x * __builtin_amdgcn_rcpf(1.0f + e);
+// u = x * log2(e);  returns u * sigmoid(x) = u / (1 + 2^-u).  The caller folds
+// the missing 1/log2(e) into the output scale.
+__device__ __forceinline__ float silu_log2(float u) {
+  float e = __builtin_amdgcn_exp2f(-u);
+  return u * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4v* lds_short4_ptr;
+
+// 4 keys x 16 channels per 16-lane group, transposed on the way out of LDS:
+// lane i of a group receives channel i of 4 consecutive keys.
+__device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
+  short4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)p);
+  return __builtin_bit_cast(uint2, v);
 }
 
 template <int D, bool POS, bool TS>
-__global__ __launch_bounds__(256, 2) void hstu_fwd_mfma_bf16(const Params p) {
+__global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Params p) {
   using SM = MfmaSmem<D>;
   constexpr int KP = SM::KP, VP = SM::VP;
   constexpr int KSTEPS = D / 16;       // MFMA k-steps over the head dim
   constexpr int DVB = D / 32;          // 32-row blocks of O^T
-  constexpr int KCH = BN * D / 8;      // 16-byte chunks in a K tile
-  constexpr int KLD = (KCH + 255) / 256;
-  constexpr int VBLK = (BN / 4) * (D / 8);   // 4x8 transposition blocks in a V tile
-  constexpr int VLD = (VBLK + 255) / 256;
+  constexpr int CH = BN * D / 8;       // 16-byte chunks in a K (or V) tile
+  constexpr int LD = CH / MFMA_THREADS;  // chunks per thread
+  static_assert(CH % MFMA_THREADS == 0, "tile must split evenly over the workgroup");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // LDS map: [stage0: K | V^T][stage1: K | V^T][pos window x2][key ts x2][ts table]
+  // LDS map: [stage0: K | V][stage1: K | V][pos window x2][key ts x2][ts table]
   auto Ks = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE); };
-  auto Vt = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE + SM::K_BYTES); };
+  auto Vs = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE + SM::K_BYTES); };
   constexpr int POS_OFF = 2 * SM::STAGE;
   constexpr int TK_OFF = POS_OFF + (POS ? 2 * SM::POS_BYTES : 0);
   auto Wc = [&](int buf) { return (float*)(smem + POS_OFF + buf * SM::POS_BYTES); };
@@ -345,26 +372,27 @@ __global__ __launch_bounds__(256, 2) void hstu_fwd_mfma_bf16(const Params p) {
     // padded rows of the padded layout: exact zeros
     const int rows = (s.rows - q0) < BM ? (s.rows - q0) : BM;
     const uint4 z = {0u, 0u, 0u, 0u};
-    for (int e = tid; e < rows * (D / 8); e += 256) {
+    for (int e = tid; e < rows * (D / 8); e += MFMA_THREADS) {
       int r = e / (D / 8), c = e - r * (D / 8);
       *(uint4*)(og + (int64_t)(q0 + r) * p.o_st + c * 8) = z;
     }
     return;
   }
 
-  const int r0 = q0 + 32 * w;          // first query row of this wave
-  const int qrow = r0 + m;             // this lane's query row
+  const int r0 = q0 + 64 * w;          // first query row of this wave
   const bool wave_live = r0 < s.n_q;
 
-  // Q fragments (B operand of S^T = K Q^T): lane holds q[qrow][16ks+8hh .. +7]
-  bf16x8 qf[KSTEPS];
-  {
+  // Q fragments (B operand of S^T = K Q^T): lane holds q[row][16ks+8hh .. +7]
+  bf16x8 qf[2][KSTEPS];
+#pragma unroll
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qrow = r0 + 32 * qb + m;
     const bf16_t* qg = (const bf16_t*)p.q + s.bq + (int64_t)qrow * p.q_st + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       uint4 t = {0u, 0u, 0u, 0u};
       if (qrow < s.n_q) t = *(const uint4*)(qg + 16 * ks);
-      qf[ks] = __builtin_bit_cast(bf16x8, t);
+      qf[qb][ks] = __builtin_bit_cast(bf16x8, t);
     }
   }
 
@@ -374,95 +402,64 @@ __global__ __launch_bounds__(256, 2) void hstu_fwd_mfma_bf16(const Params p) {
     kv_end = lim < kv_end ? lim : kv_end;
   }
   const int nt = (kv_end + BN - 1) / BN;
-  // keys this wave needs under causality
-  const int wave_kv_end = p.causal ? ((r0 + 32) < kv_end ? (r0 + 32) : kv_end) : kv_end;
 
-  int64_t tq = 0;
+  const float alpha2 = p.alpha * LOG2E;
+  int64_t tq[2] = {0, 0};
   if (TS) {
-    int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
-    tq = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      int iq = r0 + 32 * qb + m + 1;
+      iq = iq < s.n_ts ? iq : s.n_ts - 1;
+      tq[qb] = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
+    }
     const float* tab = p.ts_tab + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1);
-    for (int e = tid; e < 132; e += 256) {
+    for (int e = tid; e < 132; e += MFMA_THREADS) {
       int c = e <= p.ts_nb ? e : p.ts_nb;
-      TsTab[e] = tab[c > 128 ? 128 : c];
+      TsTab[e] = tab[c > 128 ? 128 : c] * LOG2E;
     }
   }
   const float* postab = POS ? p.pos_tab + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) : nullptr;
 
-  floatx16 o[DVB];
+  floatx16 o[2][DVB];
 #pragma unroll
-  for (int i = 0; i < DVB; ++i)
+  for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+    for (int i = 0; i < DVB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[qb][i][r] = 0.f;
 
-  uint4 kreg[KLD];
-  uint4 vreg[VLD][4];
+  uint4 kreg[LD], vreg[LD];
 
   auto gload = [&](int kv0) {
 #pragma unroll
-    for (int r = 0; r < KLD; ++r) {
-      int c = tid + 256 * r;
+    for (int r = 0; r < LD; ++r) {
+      int c = tid + MFMA_THREADS * r;
       int row = c / (D / 8), col = c - row * (D / 8);
-      uint4 t = {0u, 0u, 0u, 0u};
-      if (c < KCH && kv0 + row < s.n_kv)
-        t = *(const uint4*)(kg + (int64_t)(kv0 + row) * p.k_st + col * 8);
-      kreg[r] = t;
-    }
-#pragma unroll
-    for (int r = 0; r < VLD; ++r) {
-      int blk = tid + 256 * r;
-      int kvg = blk / (D / 8), dvg = blk - kvg * (D / 8);
-#pragma unroll
-      for (int rr = 0; rr < 4; ++rr) {
-        uint4 t = {0u, 0u, 0u, 0u};
-        int row = kv0 + 4 * kvg + rr;
-        if (blk < VBLK && row < s.n_kv)
-          t = *(const uint4*)(vg + (int64_t)row * p.v_st + dvg * 8);
-        vreg[r][rr] = t;
+      uint4 tk4 = {0u, 0u, 0u, 0u}, tv4 = {0u, 0u, 0u, 0u};
+      if (kv0 + row < s.n_kv) {
+        tk4 = *(const uint4*)(kg + (int64_t)(kv0 + row) * p.k_st + col * 8);
+        tv4 = *(const uint4*)(vg + (int64_t)(kv0 + row) * p.v_st + col * 8);
       }
+      kreg[r] = tk4;
+      vreg[r] = tv4;
     }
   };
 
   auto lds_store = [&](int buf, int kv0) {
 #pragma unroll
-    for (int r = 0; r < KLD; ++r) {
-      int c = tid + 256 * r;
+    for (int r = 0; r < LD; ++r) {
+      int c = tid + MFMA_THREADS * r;
       int row = c / (D / 8), col = c - row * (D / 8);
-      if (c < KCH) *(uint4*)(Ks(buf) + row * KP + col * 8) = kreg[r];
-    }
-#pragma unroll
-    for (int r = 0; r < VLD; ++r) {
-      int blk = tid + 256 * r;
-      int kvg = blk / (D / 8), dvg = blk - kvg * (D / 8);
-      if (blk < VBLK) {
-        // 4 keys x 8 channels -> 8 channels x 4 keys.  Within each 16-key
-        // chunk the 4-key groups are stored in the order 0,2,1,3 so that the
-        // 8 keys an MFMA lane needs are one 16-byte read.
-        int c16 = kvg >> 2, g4 = kvg & 3;
-        int pos = 16 * c16 + 8 * (g4 & 1) + 4 * (g4 >> 1);
-        const uint32_t a0[4] = {vreg[r][0].x, vreg[r][0].y, vreg[r][0].z, vreg[r][0].w};
-        const uint32_t a1[4] = {vreg[r][1].x, vreg[r][1].y, vreg[r][1].z, vreg[r][1].w};
-        const uint32_t a2[4] = {vreg[r][2].x, vreg[r][2].y, vreg[r][2].z, vreg[r][2].w};
-        const uint32_t a3[4] = {vreg[r][3].x, vreg[r][3].y, vreg[r][3].z, vreg[r][3].w};
-#pragma unroll
-        for (int jx = 0; jx < 4; ++jx) {
-          uint2 even, odd;
-          even.x = (a0[jx] & 0xffffu) | (a1[jx] << 16);
-          even.y = (a2[jx] & 0xffffu) | (a3[jx] << 16);
-          odd.x = (a0[jx] >> 16) | (a1[jx] & 0xffff0000u);
-          odd.y = (a2[jx] >> 16) | (a3[jx] & 0xffff0000u);
-          *(uint2*)(Vt(buf) + (dvg * 8 + 2 * jx) * VP + pos) = even;
-          *(uint2*)(Vt(buf) + (dvg * 8 + 2 * jx + 1) * VP + pos) = odd;
-        }
-      }
+      *(uint4*)(Ks(buf) + row * KP + col * 8) = kreg[r];
+      *(uint4*)(Vs(buf) + row * VP + col * 8) = vreg[r];
     }
     if (POS) {
-      // window[x] = pos_tab[(L-1) + kv0 - (q0+127) + x]; copy s is shifted by s
+      // window[x] = log2e * pos_tab[(L-1) + kv0 - (q0+127) + x]; copy s is shifted by s
       const int idx0 = (p.L - 1) + kv0 - (q0 + BM - 1);
-      for (int e = tid; e < 4 * POSW; e += 256) {
+      for (int e = tid; e < 4 * POSW; e += MFMA_THREADS) {
         int sft = e / POSW, z = e - sft * POSW;
         int idx = idx0 + z + sft;
-        Wc(buf)[e] = (idx >= 0 && idx < 2 * p.L - 1) ? postab[idx] : 0.f;
+        Wc(buf)[e] = (idx >= 0 && idx < 2 * p.L - 1) ? postab[idx] * LOG2E : 0.f;
       }
     }
     if (TS) {
@@ -474,67 +471,74 @@ __global__ __launch_bounds__(256, 2) void hstu_fwd_mfma_bf16(const Params p) {
     }
   };
 
-  gload(0);
-  lds_store(0, 0);
-  __syncthreads();
+  // One 64-key step for this wave.  MASKED = false: every key of the step is
+  // visible to every row of the wave (no per-element predicate, no skipping).
+  auto compute = [&](int buf, int kv0, auto masked_tag) {
+    constexpr bool MASKED = decltype(masked_tag)::value;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      const int kbs = kv0 + 32 * kb;
+      if (MASKED) {
+        // keys of this block all beyond the wave's last row (causal) or the sequence
+        const int last = p.causal ? ((r0 + 63) < (s.n_kv - 1) ? (r0 + 63) : (s.n_kv - 1)) : (s.n_kv - 1);
+        if (kbs > last) continue;
+      }
+      bf16x8 kf[KSTEPS];
+      const bf16_t* kr = Ks(buf) + (32 * kb + m) * KP + 8 * hh;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + 16 * ks);
 
-  for (int t = 0; t < nt; ++t) {
-    const int kv0 = t * BN;
-    const int buf = t & 1;
-    if (t + 1 < nt) gload(kv0 + BN);
-
-    if (wave_live) {
+      bf16x8 pb[2][2];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        const int kbs = kv0 + 32 * kb;
-        if (kbs < wave_kv_end) {
-          floatx16 sacc;
+      for (int qb = 0; qb < 2; ++qb) {
+        floatx16 sacc;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-          const bf16_t* kr = Ks(buf) + (32 * kb + m) * KP + 8 * hh;
+        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
 #pragma unroll
-          for (int ks = 0; ks < KSTEPS; ++ks) {
-            bf16x8 a = *(const bf16x8*)(kr + 16 * ks);
-            sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], sacc, 0, 0, 0);
+        for (int ks = 0; ks < KSTEPS; ++ks)
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks], sacc, 0, 0, 0);
+        // lane holds S^T[kv = kbs + 8g + 4hh + t][q = r0 + 32qb + m], r = 4g + t
+        float u[16];
+        if (POS) {
+          const int xb = 32 * kb + 4 * hh + (BM - 1) - 64 * w - 32 * qb - m;
+          const int sft = xb & 3;
+          const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            float4 bv = *(const float4*)(wrow + 8 * g);
+            u[4 * g + 0] = __builtin_fmaf(sacc[4 * g + 0], alpha2, bv.x);
+            u[4 * g + 1] = __builtin_fmaf(sacc[4 * g + 1], alpha2, bv.y);
+            u[4 * g + 2] = __builtin_fmaf(sacc[4 * g + 2], alpha2, bv.z);
+            u[4 * g + 3] = __builtin_fmaf(sacc[4 * g + 3], alpha2, bv.w);
           }
-          // lane holds S^T[kv = kbs + 8g + 4hh + t][q = qrow], r = 4g + t
-          float x[16];
+        } else {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) x[r] = p.alpha * sacc[r];
-          if (POS) {
-            const int xb = 32 * kb + 4 * hh + (BM - 1) - 32 * w - m;
-            const int sft = xb & 3;
-            const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
+          for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
+        }
+        if (TS) {
+          const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              float4 bv = *(const float4*)(wrow + 8 * g);
-              x[4 * g + 0] += bv.x; x[4 * g + 1] += bv.y;
-              x[4 * g + 2] += bv.z; x[4 * g + 3] += bv.w;
+          for (int g = 0; g < 4; ++g) {
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+              int64_t dt = tq[qb] - tk[8 * g + tt];
+              int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+              int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+              float f = __builtin_fabsf((float)sat);
+              f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
+              int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
+              u[4 * g + tt] += TsTab[bk];
             }
           }
-          if (TS) {
-            const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
+        }
+        float pv[16];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-#pragma unroll
-              for (int tt = 0; tt < 4; ++tt) {
-                int64_t dt = tq - tk[8 * g + tt];
-                int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-                int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-                float f = __builtin_fabsf((float)sat);
-                f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
-                int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
-                bk = bk < 131 ? bk : 131;
-                x[4 * g + tt] += TsTab[bk];
-              }
-            }
-          }
-          float pv[16];
-#pragma unroll
-          for (int r = 0; r < 16; ++r) pv[r] = fast_silu(x[r]);
-          // mask only where the block touches the diagonal or the tail
-          const bool need_mask = (p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv);
-          if (need_mask) {
+        for (int r = 0; r < 16; ++r) pv[r] = silu_log2(u[r]);
+        if (MASKED) {
+          const int qrow = r0 + 32 * qb + m;
+          const int rb = r0 + 32 * qb;
+          // predicate only where the block touches the diagonal or the tail
+          if ((p.causal && kbs + 31 > rb) || (kbs + 32 > s.n_kv)) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
@@ -542,44 +546,74 @@ __global__ __launch_bounds__(256, 2) void hstu_fwd_mfma_bf16(const Params p) {
               pv[r] = keep ? pv[r] : 0.f;
             }
           }
+        }
 #pragma unroll
-          for (int cc = 0; cc < 2; ++cc) {
-            uint4 pk;
-            pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
-            pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
-            pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
-            pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
-            bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
-            const int c = 2 * kb + cc;
-            const bf16_t* vr = Vt(buf) + m * VP + 16 * c + 8 * hh;
+        for (int cc = 0; cc < 2; ++cc) {
+          uint4 pk;
+          pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
+          pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
+          pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
+          pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
+          pb[qb][cc] = __builtin_bit_cast(bf16x8, pk);
+        }
+      }
+      // V fragments: lane (channel = 32dvb + m, half hh) gets keys 16c + 4hh + 0..3 and 16c + 8 + 4hh + 0..3
+      const int gi = lane & 15;
+      const bf16_t* vr = Vs(buf) + (32 * kb + 4 * hh + (gi >> 2)) * VP + 16 * ((lane >> 4) & 1) + 4 * (gi & 3);
 #pragma unroll
-            for (int dvb = 0; dvb < DVB; ++dvb) {
-              bf16x8 a = *(const bf16x8*)(vr + 32 * dvb * VP);
-              o[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb, o[dvb], 0, 0, 0);
-            }
-          }
+      for (int cc = 0; cc < 2; ++cc) {
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb) {
+          uint2 lo = lds_read_tr(vr + (16 * cc) * VP + 32 * dvb);
+          uint2 hi = lds_read_tr(vr + (16 * cc + 8) * VP + 32 * dvb);
+          uint4 av = {lo.x, lo.y, hi.x, hi.y};
+          bf16x8 a = __builtin_bit_cast(bf16x8, av);
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb)
+            o[qb][dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[qb][cc], o[qb][dvb], 0, 0, 0);
         }
       }
     }
+  };
 
+  gload(0);
+  lds_store(0, 0);
+  __syncthreads();
+
+  // steps whose 64 keys are all visible to all 64 rows of this wave
+  const int full_end = p.causal ? (r0 < s.n_kv ? r0 : s.n_kv) : s.n_kv;
+  for (int t = 0; t < nt; ++t) {
+    const int kv0 = t * BN;
+    const int buf = t & 1;
+    if (t + 1 < nt) gload(kv0 + BN);
+    if (wave_live) {
+      if (kv0 + BN <= full_end) compute(buf, kv0, std::false_type{});
+      else compute(buf, kv0, std::true_type{});
+    }
     if (t + 1 < nt) lds_store(buf ^ 1, kv0 + BN);
     __syncthreads();
   }
 
-  // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0
-  if (qrow < s.rows) {
-    const bool live = qrow < s.n_q;
-    bf16_t* orow = og + (int64_t)qrow * p.o_st + 4 * hh;
+  // O^T[dv = 32 dvb + 8g + 4hh + t][q]; rows past the sequence are 0.  The
+  // 1/log2(e) left out of the SiLU is folded into the output scale.
+  const float oscale = p.inv_n * (1.0f / LOG2E);
 #pragma unroll
-    for (int dvb = 0; dvb < DVB; ++dvb) {
+  for (int qb = 0; qb < 2; ++qb) {
+    const int qrow = r0 + 32 * qb + m;
+    if (qrow < s.rows) {
+      const bool live = qrow < s.n_q;
+      bf16_t* orow = og + (int64_t)qrow * p.o_st + 4 * hh;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint2 pk = {0u, 0u};
-        if (live) {
-          pk.x = pack_bf16(o[dvb][4 * g + 0] * p.inv_n, o[dvb][4 * g + 1] * p.inv_n);
-          pk.y = pack_bf16(o[dvb][4 * g + 2] * p.inv_n, o[dvb][4 * g + 3] * p.inv_n);
+      for (int dvb = 0; dvb < DVB; ++dvb) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 pk = {0u, 0u};
+          if (live) {
+            pk.x = pack_bf16(o[qb][dvb][4 * g + 0] * oscale, o[qb][dvb][4 * g + 1] * oscale);
+            pk.y = pack_bf16(o[qb][dvb][4 * g + 2] * oscale, o[qb][dvb][4 * g + 3] * oscale);
+          }
+          *(uint2*)(orow + 32 * dvb + 8 * g) = pk;
         }
-        *(uint2*)(orow + 32 * dvb + 8 * g) = pk;
       }
     }
   }
@@ -692,11 +726,26 @@ Params make_params(const HstuAttnFwdArgs* a) {
   return p;
 }
 
+// Raises the dynamic-LDS limit of a kernel once per device (the attribute is
+// sticky; asking again on every launch would only cost host time).
+int allow_lds(const void* fn, int bytes, int* granted /* [kMaxDev] */) {
+  constexpr int kMaxDev = 64;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev >= 0 && dev < kMaxDev && __atomic_load_n(&granted[dev], __ATOMIC_ACQUIRE) >= bytes) return HSTU_OK;
+  e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
+  if (dev >= 0 && dev < kMaxDev) __atomic_store_n(&granted[dev], bytes, __ATOMIC_RELEASE);
+  return HSTU_OK;
+}
+
 template <typename T>
 int launch_general(const Params& p, hipStream_t st) {
   size_t smem = sizeof(float) * ((size_t)GT * p.d_qk + (size_t)GT * (p.d_qk + 1) + (size_t)GT * p.d_v + GT * (GT + 1));
-  hipError_t e = hipFuncSetAttribute((const void*)hstu_fwd_general<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  static int granted[64];
+  if (int rc = allow_lds((const void*)hstu_fwd_general<T>, (int)smem, granted)) return rc;
+  hipError_t e;
   dim3 grid((p.L + GT - 1) / GT, p.H, p.B);
   hipLaunchKernelGGL(hstu_fwd_general<T>, grid, dim3(256), smem, st, p);
   e = hipGetLastError();
@@ -707,11 +756,12 @@ int launch_general(const Params& p, hipStream_t st) {
 template <int D, bool POS, bool TS>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D>::total(POS, TS);
-  hipError_t e = hipFuncSetAttribute((const void*)hstu_fwd_mfma_bf16<D, POS, TS>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  static int granted[64];
+  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS>, smem, granted)) return rc;
+  hipError_t e;
   const long long blocks = (long long)p.n_qtiles * p.B * p.H;
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS>), dim3((unsigned)blocks), dim3(256), smem, st, p);
+  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "mfma kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;

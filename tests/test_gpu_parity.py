@@ -307,7 +307,8 @@ def test_timestamp_buckets_on_gpu(gpu):
       rel = np.abs(out - want) / want
       assert (rel[far] <= max(tol, 1e-5) * 1.0 + (4e-3 if dt_ == torch.bfloat16 else 0)).all()
       near_ok = np.minimum(np.minimum(np.abs(out - want), np.abs(out - lo)), np.abs(out - hi)) / want
-      assert (near_ok <= 5e-3).all()
+      # bf16 rounds P and the output (2 x 2^-9); adjacent buckets differ by >= 1.4 %
+      assert (near_ok <= (1e-2 if dt_ == torch.bfloat16 else 1e-5)).all()
 
 
 def test_argument_errors(gpu):

@@ -7,7 +7,7 @@ import os
 import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libhstu_attn.so")
+LIB_PATH = os.environ.get("RECML_AMD_LIB") or os.path.join(_HERE, "lib", "libhstu_attn.so")
 
 ABI_VERSION = 1
 

@@ -295,10 +295,14 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D>
 struct MfmaSmem {
-  static constexpr int KP = D + 8;    // K row pitch in bf16: 16-byte reads, one row per lane
-  static constexpr int VP = D + 16;   // V row pitch in bf16: transpose reads of 8 rows x 64 bytes
-  static constexpr int K_BYTES = BN * KP * 2;
-  static constexpr int V_BYTES = BN * VP * 2;
+  // K and V tiles are stored unpadded ([64 keys][D] bf16) because they arrive
+  // by direct global->LDS loads, which write 64 lanes x 16 bytes contiguously.
+  // Bank conflicts are avoided by XOR-swizzling the 16-byte chunk index of a
+  // row instead (different functions for K and V, matched to how each is read).
+  static constexpr int CPR = D / 8;                 // 16-byte chunks per row
+  static constexpr int RPB = CPR >= 16 ? 1 : 16 / CPR;  // rows per 256 bytes (one sweep of the banks)
+  static constexpr int K_BYTES = BN * D * 2;
+  static constexpr int V_BYTES = BN * D * 2;
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int POS_BYTES = 4 * POSW * 4;
   static constexpr int TK_BYTES = BN * 8;
@@ -306,7 +310,27 @@ struct MfmaSmem {
   static constexpr int total(bool pos, bool ts) {
     return 2 * STAGE + (pos ? 2 * POS_BYTES : 0) + (ts ? 2 * TK_BYTES + TAB_BYTES : 0);
   }
+  // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
+  __device__ static constexpr int swz_k(int row) { return (row / RPB) % CPR; }
+  // V is read 4 rows x 64 bytes per half-wave: the 4 rows must land in 4 different 64-byte groups
+  __device__ static constexpr int swz_v(int row) { return (4 * ((row / RPB) & 3)) % CPR; }
 };
+
+typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
+
+// 64 lanes x 16 bytes, global -> LDS without passing through registers: lane l
+// of the wave writes LDS bytes [lds_base + 16 l, +16).  Issued as inline
+// assembly on purpose: the compiler then does not know that LDS is written and
+// does not put a "wait for all outstanding loads" in front of every LDS read
+// of the tile that is being computed meanwhile.  The caller waits (vmcnt(0))
+// and barriers before anybody reads the destination.
+__device__ __forceinline__ void lds_dma16(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_byte_ptr)lds_dst_wave_uniform);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(base), "v"(byte_off), "s"(gbase_uniform)
+               : "memory", "m0");
+}
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   floatx2 f = {lo, hi};
@@ -317,8 +341,12 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // u = x * log2(e);  returns u * sigmoid(x) = u / (1 + 2^-u).  The caller folds
 // the missing 1/log2(e) into the output scale.
 __device__ __forceinline__ float silu_log2(float u) {
+#ifdef HSTU_DBG_NOACT
+  return u;
+#else
   float e = __builtin_amdgcn_exp2f(-u);
   return u * __builtin_amdgcn_rcpf(1.0f + e);
+#endif
 }
 
 typedef short short4v __attribute__((ext_vector_type(4)));
@@ -334,11 +362,11 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
 template <int D, bool POS, bool TS>
 __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Params p) {
   using SM = MfmaSmem<D>;
-  constexpr int KP = SM::KP, VP = SM::VP;
+  constexpr int CPR = SM::CPR;
   constexpr int KSTEPS = D / 16;       // MFMA k-steps over the head dim
   constexpr int DVB = D / 32;          // 32-row blocks of O^T
   constexpr int CH = BN * D / 8;       // 16-byte chunks in a K (or V) tile
-  constexpr int LD = CH / MFMA_THREADS;  // chunks per thread
+  constexpr int LD = CH / MFMA_THREADS;  // direct loads per lane per tile (each wave: LD x 1 KB)
   static_assert(CH % MFMA_THREADS == 0, "tile must split evenly over the workgroup");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -351,18 +379,25 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
   auto Tk = [&](int buf) { return (int64_t*)(smem + TK_OFF + buf * SM::TK_BYTES); };
   float* TsTab = (float*)(smem + TK_OFF + 2 * SM::TK_BYTES);
 
-  // Heaviest query tiles first; all tiles of one (b,h) share blockIdx % 8 so
-  // that they land on one XCD and reuse K/V from its L2.
+  // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with
+  // its own L2.  All query tiles of one (sequence, head) go to the same XCD and
+  // are adjacent in launch order, heaviest first, so that the tiles running
+  // together stream the same K/V rows and share them through that L2 instead
+  // of each pulling its own copy from HBM.
   const int BH = p.B * p.H;
-  const int bh = blockIdx.x % BH;
-  const int qt = p.n_qtiles - 1 - blockIdx.x / BH;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int bhk = slot / p.n_qtiles;
+  const int qt = p.n_qtiles - 1 - (slot - bhk * p.n_qtiles);
+  const int bh = bhk * 8 + xcd;
+  if (bh >= BH) return;
   const int b = bh / p.H, h = bh - b * p.H;
   const Seq s = seq_info(p, b, h);
   const int q0 = qt * BM;
   if (q0 >= s.rows) return;
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, w = tid >> 6;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept scalar
   const int m = lane & 31, hh = lane >> 5;
   const bf16_t* __restrict__ kg = (const bf16_t*)p.k + s.bk;
   const bf16_t* __restrict__ vg = (const bf16_t*)p.v + s.bv;
@@ -404,6 +439,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
   const int nt = (kv_end + BN - 1) / BN;
 
   const float alpha2 = p.alpha * LOG2E;
+  const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
   int64_t tq[2] = {0, 0};
   if (TS) {
 #pragma unroll
@@ -428,31 +464,32 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
 #pragma unroll
       for (int r = 0; r < 16; ++r) o[qb][i][r] = 0.f;
 
-  uint4 kreg[LD], vreg[LD];
-
-  auto gload = [&](int kv0) {
+  // Direct global->LDS loads of the next K/V tile: wave w fills 1 KB pieces
+  // w*LD .. w*LD+LD-1 of each tile; lane l of piece j lands at chunk 64j + l,
+  // i.e. row (64j+l)/CPR, physical chunk (64j+l)%CPR, and fetches the logical
+  // chunk that the swizzle maps there.  Rows past the sequence re-read the
+  // last valid row (finite data; their P is masked to exactly 0).
+  auto gload = [&](int buf, int kv0) {
+#ifdef HSTU_DBG_NOLOAD
+    if (kv0 > 0) return;
+#endif
+    const int last = s.n_kv - 1;
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
-      int c = tid + MFMA_THREADS * r;
-      int row = c / (D / 8), col = c - row * (D / 8);
-      uint4 tk4 = {0u, 0u, 0u, 0u}, tv4 = {0u, 0u, 0u, 0u};
-      if (kv0 + row < s.n_kv) {
-        tk4 = *(const uint4*)(kg + (int64_t)(kv0 + row) * p.k_st + col * 8);
-        tv4 = *(const uint4*)(vg + (int64_t)(kv0 + row) * p.v_st + col * 8);
-      }
-      kreg[r] = tk4;
-      vreg[r] = tv4;
+      const int j = w * LD + r;
+      const int c = 64 * j + lane;
+      const int row = c / CPR, pc = c - row * CPR;
+      int grow = kv0 + row;
+      grow = grow < last ? grow : last;
+      const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
+      const uint32_t voff = (uint32_t)grow * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
+      lds_dma16(kg, koff, Ks(buf) + j * 512);
+      lds_dma16(vg, voff, Vs(buf) + j * 512);
     }
   };
 
-  auto lds_store = [&](int buf, int kv0) {
-#pragma unroll
-    for (int r = 0; r < LD; ++r) {
-      int c = tid + MFMA_THREADS * r;
-      int row = c / (D / 8), col = c - row * (D / 8);
-      *(uint4*)(Ks(buf) + row * KP + col * 8) = kreg[r];
-      *(uint4*)(Vs(buf) + row * VP + col * 8) = vreg[r];
-    }
+  // bias operands of the next tile (small; staged through registers)
+  auto stage_bias = [&](int buf, int kv0) {
     if (POS) {
       // window[x] = log2e * pos_tab[(L-1) + kv0 - (q0+127) + x]; copy s is shifted by s
       const int idx0 = (p.L - 1) + kv0 - (q0 + BM - 1);
@@ -471,126 +508,216 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
     }
   };
 
-  // One 64-key step for this wave.  MASKED = false: every key of the step is
-  // visible to every row of the wave (no per-element predicate, no skipping).
-  auto compute = [&](int buf, int kv0, auto masked_tag) {
-    constexpr bool MASKED = decltype(masked_tag)::value;
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const int kbs = kv0 + 32 * kb;
-      if (MASKED) {
-        // keys of this block all beyond the wave's last row (causal) or the sequence
-        const int last = p.causal ? ((r0 + 63) < (s.n_kv - 1) ? (r0 + 63) : (s.n_kv - 1)) : (s.n_kv - 1);
-        if (kbs > last) continue;
-      }
-      bf16x8 kf[KSTEPS];
-      const bf16_t* kr = Ks(buf) + (32 * kb + m) * KP + 8 * hh;
-#pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + 16 * ks);
+  // One 64-key step for this wave: four 32x32 blocks (kb = key half, qb = row
+  // half), hand-interleaved so that the MFMAs of the next block's logits and of
+  // the previous block's P.V sit between the SiLU arithmetic of the current
+  // block.  The wavefront issues in order: an MFMA placed behind another one
+  // would stall everything after it for 32 cycles, so each MFMA is followed by
+  // about one element's worth of VALU work and a scheduling fence keeps that order.
+  //   phase 0: S0                      (logits kb0 x qb0)
+  //   phase 1: S1        | act(S0)
+  //   phase 2: S2, PV0   | act(S1)
+  //   phase 3: S3, PV1   | act(S2)
+  //   phase 4: PV2       | act(S3)
+  //   phase 5: PV3
+  // Blocks that touch the causal diagonal or the end of the sequence get their
+  // logits and bias zeroed where masked: silu(0) = 0 exactly, so no predicate
+  // is needed after the activation and full blocks pay nothing.
+  auto compute = [&](int buf, int kv0) {
+    // K: lane (row m, half hh) reads logical chunk 2ks+hh of rows m and 32+m (same swizzle for both)
+    const bf16_t* kr = Ks(buf) + m * D;
+    const int gk = SM::swz_k(m);
+    // V: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc + 32kb):
+    // logical chunk 4dvb + 2(G&1) + (i&3)/2, byte half (i&3)&1
+    const int gi = lane & 15;
+    const int vrow = 4 * hh + (gi >> 2);
+    const int gq = SM::swz_v(vrow) >> 2;          // swizzle acts on the chunk's upper bits only
+    const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
+    const bf16_t* vr = Vs(buf) + vrow * D + 4 * (gi & 1);
 
-      bf16x8 pb[2][2];
+    bf16x8 kf[KSTEPS];
+    uint4 vf[2][DVB];        // V fragments of one key half: [16-key chunk][channel block]
+    floatx16 sa, sb;         // two logit blocks in flight
+    uint4 pcur[2], pprev[2]; // packed P of the block being activated / waiting for P.V
+    float bias[16];
+    float e0 = 0.f;
+    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    auto load_k = [&](int kb) {
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) {
-        floatx16 sacc;
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + 32 * kb * D + (((2 * ks + hh) ^ gk) * 8));
+    };
+    auto load_v = [&](int kb) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks)
-          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks], sacc, 0, 0, 0);
-        // lane holds S^T[kv = kbs + 8g + 4hh + t][q = r0 + 32qb + m], r = 4g + t
-        float u[16];
-        if (POS) {
-          const int xb = 32 * kb + 4 * hh + (BM - 1) - 64 * w - 32 * qb - m;
-          const int sft = xb & 3;
-          const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            float4 bv = *(const float4*)(wrow + 8 * g);
-            u[4 * g + 0] = __builtin_fmaf(sacc[4 * g + 0], alpha2, bv.x);
-            u[4 * g + 1] = __builtin_fmaf(sacc[4 * g + 1], alpha2, bv.y);
-            u[4 * g + 2] = __builtin_fmaf(sacc[4 * g + 2], alpha2, bv.z);
-            u[4 * g + 3] = __builtin_fmaf(sacc[4 * g + 3], alpha2, bv.w);
-          }
-        } else {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
-        }
-        if (TS) {
-          const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-#pragma unroll
-            for (int tt = 0; tt < 4; ++tt) {
-              int64_t dt = tq[qb] - tk[8 * g + tt];
-              int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-              int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-              float f = __builtin_fabsf((float)sat);
-              f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
-              int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
-              u[4 * g + tt] += TsTab[bk];
-            }
-          }
-        }
-        float pv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) pv[r] = silu_log2(u[r]);
-        if (MASKED) {
-          const int qrow = r0 + 32 * qb + m;
-          const int rb = r0 + 32 * qb;
-          // predicate only where the block touches the diagonal or the tail
-          if ((p.causal && kbs + 31 > rb) || (kbs + 32 > s.n_kv)) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-              bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
-              pv[r] = keep ? pv[r] : 0.f;
-            }
-          }
-        }
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          uint4 pk;
-          pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
-          pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
-          pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
-          pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
-          pb[qb][cc] = __builtin_bit_cast(bf16x8, pk);
-        }
-      }
-      // V fragments: lane (channel = 32dvb + m, half hh) gets keys 16c + 4hh + 0..3 and 16c + 8 + 4hh + 0..3
-      const int gi = lane & 15;
-      const bf16_t* vr = Vs(buf) + (32 * kb + 4 * hh + (gi >> 2)) * VP + 16 * ((lane >> 4) & 1) + 4 * (gi & 3);
-#pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
+      for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
         for (int dvb = 0; dvb < DVB; ++dvb) {
-          uint2 lo = lds_read_tr(vr + (16 * cc) * VP + 32 * dvb);
-          uint2 hi = lds_read_tr(vr + (16 * cc + 8) * VP + 32 * dvb);
-          uint4 av = {lo.x, lo.y, hi.x, hi.y};
-          bf16x8 a = __builtin_bit_cast(bf16x8, av);
+          const int pch = (4 * ((dvb ^ gq) % (CPR / 4 > 0 ? CPR / 4 : 1)) + vc2) * 8;
+          uint2 lo = lds_read_tr(vr + (32 * kb + 16 * cc) * D + pch);
+          uint2 hi = lds_read_tr(vr + (32 * kb + 16 * cc + 8) * D + pch);
+          vf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
+        }
+    };
+    // bias for the 16 logits of block (kb, qb) held by this lane, times log2(e)
+    auto bias16 = [&](int kb, int qb) {
+      if (POS) {
+        const int xb = 32 * kb + 4 * hh + (BM - 1) - 64 * w - 32 * qb - m;
+        const int sft = xb & 3;
+        const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
 #pragma unroll
-          for (int qb = 0; qb < 2; ++qb)
-            o[qb][dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[qb][cc], o[qb][dvb], 0, 0, 0);
+        for (int g = 0; g < 4; ++g) {
+          float4 bv = *(const float4*)(wrow + 8 * g);
+          bias[4 * g + 0] = bv.x; bias[4 * g + 1] = bv.y; bias[4 * g + 2] = bv.z; bias[4 * g + 3] = bv.w;
+        }
+      } else if (TS) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bias[r] = 0.f;
+      }
+      if (TS) {
+        const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt) {
+            int64_t dt = tq[qb] - tk[8 * g + tt];
+            int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+            int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+            float f = __builtin_fabsf((float)sat);
+            f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
+            int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
+            bias[4 * g + tt] += TsTab[bk];
+          }
         }
       }
+    };
+    // zero the masked logits (and their bias) of block (kb, qb); nothing to do for interior blocks
+    auto mask16 = [&](floatx16& sacc, int kb, int qb) {
+      const int kbs = kv0 + 32 * kb, rb = r0 + 32 * qb;
+      if ((p.causal && kbs + 31 > rb) || (kbs + 32 > s.n_kv)) {
+        const int qrow = rb + m;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
+          const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
+          sacc[r] = keep ? sacc[r] : 0.f;
+          if (POS || TS) bias[r] = keep ? bias[r] : 0.f;
+        }
+      }
+    };
+    // element r of a logit block -> u * sigmoid(x)
+    auto act1 = [&](const floatx16& sacc, int r) -> float {
+      const float u = (POS || TS) ? __builtin_fmaf(sacc[r], alpha2, bias[r]) : sacc[r] * alpha2;
+      return silu_log2(u);
+    };
+    auto set_p = [&](int r, uint32_t v) {
+      // r = index of the odd element of the pair just packed
+      const int wd = r >> 1;  // 0..7
+      if (wd == 0) pcur[0].x = v; else if (wd == 1) pcur[0].y = v; else if (wd == 2) pcur[0].z = v; else if (wd == 3) pcur[0].w = v;
+      else if (wd == 4) pcur[1].x = v; else if (wd == 5) pcur[1].y = v; else if (wd == 6) pcur[1].z = v; else pcur[1].w = v;
+    };
+    auto act_range = [&](const floatx16& sacc, int rlo, int rhi) {
+#pragma unroll
+      for (int r = rlo; r < rhi; ++r) {
+        const float pvv = act1(sacc, r);
+        if (r & 1) set_p(r, pack_bf16(e0, pvv)); else e0 = pvv;
+      }
+    };
+    auto qk_step = [&](floatx16& sacc, int qb, int ks) {
+#ifdef HSTU_DBG_NOQK
+      if (ks > 0) return;
+#endif
+      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks], ks == 0 ? zero : sacc, 0, 0, 0);
+    };
+    // i-th of the 2*DVB MFMAs of P.V for one block
+    auto pv_step = [&](const uint4 (&pk)[2], int qb, int i) {
+      const int cc = i / DVB, dvb = i % DVB;
+#ifdef HSTU_DBG_NOPV
+      if (i > 0) return;
+#endif
+      o[qb][dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[cc][dvb]),
+                                                            __builtin_bit_cast(bf16x8, pk[cc]), o[qb][dvb], 0, 0, 0);
+    };
+    constexpr int NM = KSTEPS + 2 * DVB;   // MFMAs in a full phase (logits of one block + P.V of another)
+
+    // ---- phase 0: S0
+    load_k(0);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) qk_step(sa, 0, ks);
+    bias16(0, 0);
+    mask16(sa, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 1: S1 | act(S0)
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      qk_step(sb, 1, ks);
+      act_range(sa, (16 * ks) / KSTEPS, (16 * (ks + 1)) / KSTEPS);
+      __builtin_amdgcn_sched_barrier(0);
     }
+    pprev[0] = pcur[0]; pprev[1] = pcur[1];   // P0
+    load_v(0);
+    load_k(1);
+    bias16(0, 1);
+    mask16(sb, 0, 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 2: S2, PV0 | act(S1)
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      if (i < 2 * KSTEPS && i < 4 * DVB) { if (i % 2 == 0) qk_step(sa, 0, i / 2); else pv_step(pprev, 0, i / 2); }
+      else if (KSTEPS > 2 * DVB) qk_step(sa, 0, i - 2 * DVB);
+      else pv_step(pprev, 0, i - KSTEPS);
+      act_range(sb, (16 * i) / NM, (16 * (i + 1)) / NM);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    pprev[0] = pcur[0]; pprev[1] = pcur[1];   // P1
+    bias16(1, 0);
+    mask16(sa, 1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 3: S3, PV1 | act(S2)
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      if (i < 2 * KSTEPS && i < 4 * DVB) { if (i % 2 == 0) qk_step(sb, 1, i / 2); else pv_step(pprev, 1, i / 2); }
+      else if (KSTEPS > 2 * DVB) qk_step(sb, 1, i - 2 * DVB);
+      else pv_step(pprev, 1, i - KSTEPS);
+      act_range(sa, (16 * i) / NM, (16 * (i + 1)) / NM);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    pprev[0] = pcur[0]; pprev[1] = pcur[1];   // P2
+    load_v(1);
+    bias16(1, 1);
+    mask16(sb, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- phase 4: PV2 | act(S3)
+#pragma unroll
+    for (int i = 0; i < 2 * DVB; ++i) {
+      pv_step(pprev, 0, i);
+      act_range(sb, (16 * i) / (2 * DVB), (16 * (i + 1)) / (2 * DVB));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- phase 5: PV3
+#pragma unroll
+    for (int i = 0; i < 2 * DVB; ++i) pv_step(pcur, 1, i);
   };
 
-  gload(0);
-  lds_store(0, 0);
+  gload(0, 0);
+  stage_bias(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads have landed in LDS
   __syncthreads();
 
-  // steps whose 64 keys are all visible to all 64 rows of this wave
-  const int full_end = p.causal ? (r0 < s.n_kv ? r0 : s.n_kv) : s.n_kv;
+  // keys this wave needs at all
+  const int wave_kv_end = p.causal ? ((r0 + 64) < kv_end ? (r0 + 64) : kv_end) : kv_end;
   for (int t = 0; t < nt; ++t) {
     const int kv0 = t * BN;
     const int buf = t & 1;
-    if (t + 1 < nt) gload(kv0 + BN);
-    if (wave_live) {
-      if (kv0 + BN <= full_end) compute(buf, kv0, std::false_type{});
-      else compute(buf, kv0, std::true_type{});
+    if (t + 1 < nt) gload(buf ^ 1, kv0 + BN);
+    if (wave_live && kv0 < wave_kv_end) {
+      compute(buf, kv0);
     }
-    if (t + 1 < nt) lds_store(buf ^ 1, kv0 + BN);
+    if (t + 1 < nt) stage_bias(buf ^ 1, kv0 + BN);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
   }
 
@@ -759,7 +886,7 @@ int launch_mfma_inst(const Params& p, hipStream_t st) {
   static int granted[64];
   if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS>, smem, granted)) return rc;
   hipError_t e;
-  const long long blocks = (long long)p.n_qtiles * p.B * p.H;
+  const long long blocks = 8LL * p.n_qtiles * (((long long)p.B * p.H + 7) / 8);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
   hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();

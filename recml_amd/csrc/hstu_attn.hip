@@ -273,9 +273,11 @@ __global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
 // ---------------------------------------------------------------------------
 // MFMA kernel: bf16, causal/full + length masking, fused pos / timestamp bias.
 //
-// One workgroup = 2 wavefronts = 128 query rows; each wavefront owns 64 rows
-// (two 32-row blocks) so that every K / V fragment read from LDS feeds two
-// MFMAs.  Keys are streamed 64 at a time through a double-buffered LDS stage.
+// One workgroup = 4 wavefronts = 128 query rows (32 per wavefront); two
+// workgroups per CU, i.e. two wavefronts per SIMD, so that the matrix pipe of
+// a SIMD runs one wavefront's MFMAs while its VALU runs the other's SiLU.
+// Keys are streamed 64 at a time through a double-buffered LDS stage that is
+// filled by direct global->LDS loads (no staging registers).
 //
 //   S^T[kv, q] = K Q^T   A = K fragment (LDS, 16-byte reads), B = Q (registers)
 //   O^T[dv, q] = V^T P^T A = V fragment (LDS transpose reads), B = P (registers)
@@ -287,10 +289,10 @@ __global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
 // reads of row-major V deliver.  P therefore never leaves registers.
 // ---------------------------------------------------------------------------
 
-constexpr int BM = 128;   // query rows per workgroup (2 waves x 64)
+constexpr int BM = 128;   // query rows per workgroup (4 waves x 32)
 constexpr int BN = 64;    // keys per step
 constexpr int POSW = 192; // staged window of the position table per step
-constexpr int MFMA_THREADS = 128;
+constexpr int MFMA_THREADS = 256;
 constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D>
@@ -319,11 +321,12 @@ struct MfmaSmem {
 typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
 
 // 64 lanes x 16 bytes, global -> LDS without passing through registers: lane l
-// of the wave writes LDS bytes [lds_base + 16 l, +16).  Issued as inline
-// assembly on purpose: the compiler then does not know that LDS is written and
-// does not put a "wait for all outstanding loads" in front of every LDS read
-// of the tile that is being computed meanwhile.  The caller waits (vmcnt(0))
-// and barriers before anybody reads the destination.
+// of the wave writes LDS bytes [lds_base + 16 l, +16) with the 16 bytes at
+// gbase + byte_off(l).  Issued as inline assembly on purpose: the compiler
+// then does not know that LDS is written and does not put a "wait for all
+// outstanding loads" in front of every LDS read of the tile that is being
+// computed meanwhile.  The caller waits (vmcnt(0)) and barriers before anybody
+// reads the destination.
 __device__ __forceinline__ void lds_dma16(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
   const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_byte_ptr)lds_dst_wave_uniform);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
@@ -341,12 +344,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // u = x * log2(e);  returns u * sigmoid(x) = u / (1 + 2^-u).  The caller folds
 // the missing 1/log2(e) into the output scale.
 __device__ __forceinline__ float silu_log2(float u) {
-#ifdef HSTU_DBG_NOACT
-  return u;
-#else
   float e = __builtin_amdgcn_exp2f(-u);
   return u * __builtin_amdgcn_rcpf(1.0f + e);
-#endif
 }
 
 typedef short short4v __attribute__((ext_vector_type(4)));
@@ -360,7 +359,7 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
 }
 
 template <int D, bool POS, bool TS>
-__global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Params p) {
+__global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   using SM = MfmaSmem<D>;
   constexpr int CPR = SM::CPR;
   constexpr int KSTEPS = D / 16;       // MFMA k-steps over the head dim
@@ -414,20 +413,19 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
     return;
   }
 
-  const int r0 = q0 + 64 * w;          // first query row of this wave
+  const int r0 = q0 + 32 * w;          // first query row of this wave
+  const int qrow = r0 + m;             // this lane's query row
   const bool wave_live = r0 < s.n_q;
 
-  // Q fragments (B operand of S^T = K Q^T): lane holds q[row][16ks+8hh .. +7]
-  bf16x8 qf[2][KSTEPS];
-#pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    const int qrow = r0 + 32 * qb + m;
+  // Q fragments (B operand of S^T = K Q^T): lane holds q[qrow][16ks+8hh .. +7]
+  bf16x8 qf[KSTEPS];
+  {
     const bf16_t* qg = (const bf16_t*)p.q + s.bq + (int64_t)qrow * p.q_st + 8 * hh;
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
       uint4 t = {0u, 0u, 0u, 0u};
       if (qrow < s.n_q) t = *(const uint4*)(qg + 16 * ks);
-      qf[qb][ks] = __builtin_bit_cast(bf16x8, t);
+      qf[ks] = __builtin_bit_cast(bf16x8, t);
     }
   }
 
@@ -437,17 +435,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
     kv_end = lim < kv_end ? lim : kv_end;
   }
   const int nt = (kv_end + BN - 1) / BN;
+  // last key this wave needs
+  const int wave_last = p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1);
 
   const float alpha2 = p.alpha * LOG2E;
   const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
-  int64_t tq[2] = {0, 0};
+  int64_t tq = 0;
   if (TS) {
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      int iq = r0 + 32 * qb + m + 1;
-      iq = iq < s.n_ts ? iq : s.n_ts - 1;
-      tq[qb] = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
-    }
+    int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
+    tq = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
     const float* tab = p.ts_tab + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1);
     for (int e = tid; e < 132; e += MFMA_THREADS) {
       int c = e <= p.ts_nb ? e : p.ts_nb;
@@ -456,23 +452,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
   }
   const float* postab = POS ? p.pos_tab + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) : nullptr;
 
-  floatx16 o[2][DVB];
+  floatx16 o[DVB];
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb)
+  for (int i = 0; i < DVB; ++i)
 #pragma unroll
-    for (int i = 0; i < DVB; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[qb][i][r] = 0.f;
+    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
 
   // Direct global->LDS loads of the next K/V tile: wave w fills 1 KB pieces
   // w*LD .. w*LD+LD-1 of each tile; lane l of piece j lands at chunk 64j + l,
   // i.e. row (64j+l)/CPR, physical chunk (64j+l)%CPR, and fetches the logical
   // chunk that the swizzle maps there.  Rows past the sequence re-read the
-  // last valid row (finite data; their P is masked to exactly 0).
+  // last valid row (finite data; their logits are masked).
   auto gload = [&](int buf, int kv0) {
-#ifdef HSTU_DBG_NOLOAD
-    if (kv0 > 0) return;
-#endif
     const int last = s.n_kv - 1;
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
@@ -508,198 +499,103 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
     }
   };
 
-  // One 64-key step for this wave: four 32x32 blocks (kb = key half, qb = row
-  // half), hand-interleaved so that the MFMAs of the next block's logits and of
-  // the previous block's P.V sit between the SiLU arithmetic of the current
-  // block.  The wavefront issues in order: an MFMA placed behind another one
-  // would stall everything after it for 32 cycles, so each MFMA is followed by
-  // about one element's worth of VALU work and a scheduling fence keeps that order.
-  //   phase 0: S0                      (logits kb0 x qb0)
-  //   phase 1: S1        | act(S0)
-  //   phase 2: S2, PV0   | act(S1)
-  //   phase 3: S3, PV1   | act(S2)
-  //   phase 4: PV2       | act(S3)
-  //   phase 5: PV3
-  // Blocks that touch the causal diagonal or the end of the sequence get their
-  // logits and bias zeroed where masked: silu(0) = 0 exactly, so no predicate
-  // is needed after the activation and full blocks pay nothing.
-  auto compute = [&](int buf, int kv0) {
-    // K: lane (row m, half hh) reads logical chunk 2ks+hh of rows m and 32+m (same swizzle for both)
-    const bf16_t* kr = Ks(buf) + m * D;
-    const int gk = SM::swz_k(m);
-    // V: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc + 32kb):
-    // logical chunk 4dvb + 2(G&1) + (i&3)/2, byte half (i&3)&1
-    const int gi = lane & 15;
-    const int vrow = 4 * hh + (gi >> 2);
-    const int gq = SM::swz_v(vrow) >> 2;          // swizzle acts on the chunk's upper bits only
-    const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
-    const bf16_t* vr = Vs(buf) + vrow * D + 4 * (gi & 1);
+  // K: lane (row m, half hh) reads logical chunk 2ks+hh of rows m and 32+m (same swizzle for both)
+  const int gk = SM::swz_k(m);
+  // V: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc + 32kb):
+  // logical chunk 4dvb + 2(G&1) + (i&3)/2, byte half (i&3)&1
+  const int gi = lane & 15;
+  const int vrow = 4 * hh + (gi >> 2);
+  const int gq = SM::swz_v(vrow) >> 2;          // the swizzle acts on the chunk's upper bits only
+  const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
 
-    bf16x8 kf[KSTEPS];
-    uint4 vf[2][DVB];        // V fragments of one key half: [16-key chunk][channel block]
-    floatx16 sa, sb;         // two logit blocks in flight
-    uint4 pcur[2], pprev[2]; // packed P of the block being activated / waiting for P.V
-    float bias[16];
-    float e0 = 0.f;
-    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-
-    auto load_k = [&](int kb) {
+  // One 32-key block for this wave: logits, bias, SiLU, P.V.  Blocks that touch
+  // the causal diagonal or the end of the sequence get their logits and bias
+  // zeroed where masked: silu(0) = 0 exactly, so nothing is needed after the
+  // activation and interior blocks pay nothing.
+  auto block = [&](int buf, int kv0, int kb) {
+    const int kbs = kv0 + 32 * kb;
+    const bf16_t* kr = Ks(buf) + (32 * kb + m) * D;
+    floatx16 sacc;
+    {
+      bf16x8 kf[KSTEPS];
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + 32 * kb * D + (((2 * ks + hh) ^ gk) * 8));
-    };
-    auto load_v = [&](int kb) {
+      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + (((2 * ks + hh) ^ gk) * 8));
+      const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks)
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], ks == 0 ? zero : sacc, 0, 0, 0);
+    }
+    // V fragments, requested now so that they arrive while the SiLU runs
+    uint4 vf[2][DVB];
+    {
+      const bf16_t* vr = Vs(buf) + (32 * kb + vrow) * D + 4 * (gi & 1);
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
         for (int dvb = 0; dvb < DVB; ++dvb) {
           const int pch = (4 * ((dvb ^ gq) % (CPR / 4 > 0 ? CPR / 4 : 1)) + vc2) * 8;
-          uint2 lo = lds_read_tr(vr + (32 * kb + 16 * cc) * D + pch);
-          uint2 hi = lds_read_tr(vr + (32 * kb + 16 * cc + 8) * D + pch);
+          uint2 lo = lds_read_tr(vr + (16 * cc) * D + pch);
+          uint2 hi = lds_read_tr(vr + (16 * cc + 8) * D + pch);
           vf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
         }
-    };
-    // bias for the 16 logits of block (kb, qb) held by this lane, times log2(e)
-    auto bias16 = [&](int kb, int qb) {
-      if (POS) {
-        const int xb = 32 * kb + 4 * hh + (BM - 1) - 64 * w - 32 * qb - m;
-        const int sft = xb & 3;
-        const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
+    }
+    // lane holds S^T[kv = kbs + 8g + 4hh + t][q = qrow], r = 4g + t
+    float u[16];
+    if (POS) {
+      const int xb = 32 * kb + 4 * hh + (BM - 1) - 32 * w - m;
+      const int sft = xb & 3;
+      const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          float4 bv = *(const float4*)(wrow + 8 * g);
-          bias[4 * g + 0] = bv.x; bias[4 * g + 1] = bv.y; bias[4 * g + 2] = bv.z; bias[4 * g + 3] = bv.w;
-        }
-      } else if (TS) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) bias[r] = 0.f;
+      for (int g = 0; g < 4; ++g) {
+        float4 bv = *(const float4*)(wrow + 8 * g);
+        u[4 * g + 0] = __builtin_fmaf(sacc[4 * g + 0], alpha2, bv.x);
+        u[4 * g + 1] = __builtin_fmaf(sacc[4 * g + 1], alpha2, bv.y);
+        u[4 * g + 2] = __builtin_fmaf(sacc[4 * g + 2], alpha2, bv.z);
+        u[4 * g + 3] = __builtin_fmaf(sacc[4 * g + 3], alpha2, bv.w);
       }
-      if (TS) {
-        const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
+    } else {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
+      for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
+    }
+    if (TS) {
+      const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
 #pragma unroll
-          for (int tt = 0; tt < 4; ++tt) {
-            int64_t dt = tq[qb] - tk[8 * g + tt];
-            int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-            int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-            float f = __builtin_fabsf((float)sat);
-            f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
-            int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
-            bias[4 * g + tt] += TsTab[bk];
-          }
-        }
-      }
-    };
-    // zero the masked logits (and their bias) of block (kb, qb); nothing to do for interior blocks
-    auto mask16 = [&](floatx16& sacc, int kb, int qb) {
-      const int kbs = kv0 + 32 * kb, rb = r0 + 32 * qb;
-      if ((p.causal && kbs + 31 > rb) || (kbs + 32 > s.n_kv)) {
-        const int qrow = rb + m;
+      for (int g = 0; g < 4; ++g) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-          const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
-          sacc[r] = keep ? sacc[r] : 0.f;
-          if (POS || TS) bias[r] = keep ? bias[r] : 0.f;
+        for (int tt = 0; tt < 4; ++tt) {
+          int64_t dt = tq - tk[8 * g + tt];
+          int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+          int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+          float f = __builtin_fabsf((float)sat);
+          f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
+          int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
+          u[4 * g + tt] += TsTab[bk];
         }
       }
-    };
-    // element r of a logit block -> u * sigmoid(x)
-    auto act1 = [&](const floatx16& sacc, int r) -> float {
-      const float u = (POS || TS) ? __builtin_fmaf(sacc[r], alpha2, bias[r]) : sacc[r] * alpha2;
-      return silu_log2(u);
-    };
-    auto set_p = [&](int r, uint32_t v) {
-      // r = index of the odd element of the pair just packed
-      const int wd = r >> 1;  // 0..7
-      if (wd == 0) pcur[0].x = v; else if (wd == 1) pcur[0].y = v; else if (wd == 2) pcur[0].z = v; else if (wd == 3) pcur[0].w = v;
-      else if (wd == 4) pcur[1].x = v; else if (wd == 5) pcur[1].y = v; else if (wd == 6) pcur[1].z = v; else pcur[1].w = v;
-    };
-    auto act_range = [&](const floatx16& sacc, int rlo, int rhi) {
+    }
+    if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv)) {
 #pragma unroll
-      for (int r = rlo; r < rhi; ++r) {
-        const float pvv = act1(sacc, r);
-        if (r & 1) set_p(r, pack_bf16(e0, pvv)); else e0 = pvv;
+      for (int r = 0; r < 16; ++r) {
+        const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
+        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
+        u[r] = keep ? u[r] : 0.f;
       }
-    };
-    auto qk_step = [&](floatx16& sacc, int qb, int ks) {
-#ifdef HSTU_DBG_NOQK
-      if (ks > 0) return;
-#endif
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[qb][ks], ks == 0 ? zero : sacc, 0, 0, 0);
-    };
-    // i-th of the 2*DVB MFMAs of P.V for one block
-    auto pv_step = [&](const uint4 (&pk)[2], int qb, int i) {
-      const int cc = i / DVB, dvb = i % DVB;
-#ifdef HSTU_DBG_NOPV
-      if (i > 0) return;
-#endif
-      o[qb][dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[cc][dvb]),
-                                                            __builtin_bit_cast(bf16x8, pk[cc]), o[qb][dvb], 0, 0, 0);
-    };
-    constexpr int NM = KSTEPS + 2 * DVB;   // MFMAs in a full phase (logits of one block + P.V of another)
-
-    // ---- phase 0: S0
-    load_k(0);
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) qk_step(sa, 0, ks);
-    bias16(0, 0);
-    mask16(sa, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- phase 1: S1 | act(S0)
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      qk_step(sb, 1, ks);
-      act_range(sa, (16 * ks) / KSTEPS, (16 * (ks + 1)) / KSTEPS);
-      __builtin_amdgcn_sched_barrier(0);
     }
-    pprev[0] = pcur[0]; pprev[1] = pcur[1];   // P0
-    load_v(0);
-    load_k(1);
-    bias16(0, 1);
-    mask16(sb, 0, 1);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- phase 2: S2, PV0 | act(S1)
+    float pv[16];
 #pragma unroll
-    for (int i = 0; i < NM; ++i) {
-      if (i < 2 * KSTEPS && i < 4 * DVB) { if (i % 2 == 0) qk_step(sa, 0, i / 2); else pv_step(pprev, 0, i / 2); }
-      else if (KSTEPS > 2 * DVB) qk_step(sa, 0, i - 2 * DVB);
-      else pv_step(pprev, 0, i - KSTEPS);
-      act_range(sb, (16 * i) / NM, (16 * (i + 1)) / NM);
-      __builtin_amdgcn_sched_barrier(0);
+    for (int r = 0; r < 16; ++r) pv[r] = silu_log2(u[r]);
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      uint4 pk;
+      pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
+      pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
+      pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
+      pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
+      const bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
+#pragma unroll
+      for (int dvb = 0; dvb < DVB; ++dvb)
+        o[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[cc][dvb]), pb, o[dvb], 0, 0, 0);
     }
-    pprev[0] = pcur[0]; pprev[1] = pcur[1];   // P1
-    bias16(1, 0);
-    mask16(sa, 1, 0);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- phase 3: S3, PV1 | act(S2)
-#pragma unroll
-    for (int i = 0; i < NM; ++i) {
-      if (i < 2 * KSTEPS && i < 4 * DVB) { if (i % 2 == 0) qk_step(sb, 1, i / 2); else pv_step(pprev, 1, i / 2); }
-      else if (KSTEPS > 2 * DVB) qk_step(sb, 1, i - 2 * DVB);
-      else pv_step(pprev, 1, i - KSTEPS);
-      act_range(sa, (16 * i) / NM, (16 * (i + 1)) / NM);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    pprev[0] = pcur[0]; pprev[1] = pcur[1];   // P2
-    load_v(1);
-    bias16(1, 1);
-    mask16(sb, 1, 1);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // ---- phase 4: PV2 | act(S3)
-#pragma unroll
-    for (int i = 0; i < 2 * DVB; ++i) {
-      pv_step(pprev, 0, i);
-      act_range(sb, (16 * i) / (2 * DVB), (16 * (i + 1)) / (2 * DVB));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // ---- phase 5: PV3
-#pragma unroll
-    for (int i = 0; i < 2 * DVB; ++i) pv_step(pcur, 1, i);
   };
 
   gload(0, 0);
@@ -707,40 +603,35 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_fwd_mfma_bf16(const Para
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads have landed in LDS
   __syncthreads();
 
-  // keys this wave needs at all
-  const int wave_kv_end = p.causal ? ((r0 + 64) < kv_end ? (r0 + 64) : kv_end) : kv_end;
   for (int t = 0; t < nt; ++t) {
     const int kv0 = t * BN;
     const int buf = t & 1;
     if (t + 1 < nt) gload(buf ^ 1, kv0 + BN);
-    if (wave_live && kv0 < wave_kv_end) {
-      compute(buf, kv0);
+    if (wave_live) {
+      if (kv0 <= wave_last) block(buf, kv0, 0);
+      if (kv0 + 32 <= wave_last) block(buf, kv0, 1);
     }
     if (t + 1 < nt) stage_bias(buf ^ 1, kv0 + BN);
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
   }
 
-  // O^T[dv = 32 dvb + 8g + 4hh + t][q]; rows past the sequence are 0.  The
-  // 1/log2(e) left out of the SiLU is folded into the output scale.
+  // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0.
+  // The 1/log2(e) left out of the SiLU is folded into the output scale.
   const float oscale = p.inv_n * (1.0f / LOG2E);
+  if (qrow < s.rows) {
+    const bool live = qrow < s.n_q;
+    bf16_t* orow = og + (int64_t)qrow * p.o_st + 4 * hh;
 #pragma unroll
-  for (int qb = 0; qb < 2; ++qb) {
-    const int qrow = r0 + 32 * qb + m;
-    if (qrow < s.rows) {
-      const bool live = qrow < s.n_q;
-      bf16_t* orow = og + (int64_t)qrow * p.o_st + 4 * hh;
+    for (int dvb = 0; dvb < DVB; ++dvb) {
 #pragma unroll
-      for (int dvb = 0; dvb < DVB; ++dvb) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          uint2 pk = {0u, 0u};
-          if (live) {
-            pk.x = pack_bf16(o[qb][dvb][4 * g + 0] * oscale, o[qb][dvb][4 * g + 1] * oscale);
-            pk.y = pack_bf16(o[qb][dvb][4 * g + 2] * oscale, o[qb][dvb][4 * g + 3] * oscale);
-          }
-          *(uint2*)(orow + 32 * dvb + 8 * g) = pk;
+      for (int g = 0; g < 4; ++g) {
+        uint2 pk = {0u, 0u};
+        if (live) {
+          pk.x = pack_bf16(o[dvb][4 * g + 0] * oscale, o[dvb][4 * g + 1] * oscale);
+          pk.y = pack_bf16(o[dvb][4 * g + 2] * oscale, o[dvb][4 * g + 3] * oscale);
         }
+        *(uint2*)(orow + 32 * dvb + 8 * g) = pk;
       }
     }
   }

@@ -60,6 +60,7 @@ struct Params {
   const float* pos_tab;
   const float* ts_tab;
   const int64_t* ts;
+  const float* pos_scaled;   // workspace: log2(e) * pos_tab, zero-padded (MFMA kernel)
   int64_t ts_sb;
   int32_t B, L, Lkv, H, d_qk, d_v;
   int32_t jagged, causal, mask_mode, window;
@@ -274,10 +275,11 @@ __global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
 // MFMA kernel: bf16, causal/full + length masking, fused pos / timestamp bias.
 //
 // One workgroup = 4 wavefronts = 128 query rows (32 per wavefront); two
-// workgroups per CU, i.e. two wavefronts per SIMD, so that the matrix pipe of
-// a SIMD runs one wavefront's MFMAs while its VALU runs the other's SiLU.
-// Keys are streamed 64 at a time through a double-buffered LDS stage that is
-// filled by direct global->LDS loads (no staging registers).
+// workgroups per CU, i.e. two wavefronts per SIMD, so that one wavefront's
+// MFMAs can run while the other's SiLU arithmetic does.  Keys are streamed 32
+// at a time through a 4-stage LDS ring filled by direct global->LDS loads that
+// are issued three steps ahead (no staging registers, ~48 KB in flight per
+// workgroup).
 //
 //   S^T[kv, q] = K Q^T   A = K fragment (LDS, 16-byte reads), B = Q (registers)
 //   O^T[dv, q] = V^T P^T A = V fragment (LDS transpose reads), B = P (registers)
@@ -289,10 +291,12 @@ __global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
 // reads of row-major V deliver.  P therefore never leaves registers.
 // ---------------------------------------------------------------------------
 
-constexpr int BM = 128;   // query rows per workgroup (4 waves x 32)
-constexpr int BN = 64;    // keys per step
-constexpr int POSW = 192; // staged window of the position table per step
+constexpr int BM = 128;       // query rows per workgroup (4 waves x 32)
+constexpr int BN = 32;        // keys per step
+constexpr int NSTAGE = 4;     // LDS ring depth
 constexpr int MFMA_THREADS = 256;
+constexpr int NWAVES = MFMA_THREADS / 64;
+constexpr int POS_PAD = 256;  // zero margin on both sides of the scaled position table
 constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D>
@@ -306,11 +310,13 @@ struct MfmaSmem {
   static constexpr int K_BYTES = BN * D * 2;
   static constexpr int V_BYTES = BN * D * 2;
   static constexpr int STAGE = K_BYTES + V_BYTES;
-  static constexpr int POS_BYTES = 4 * POSW * 4;
-  static constexpr int TK_BYTES = BN * 8;
+  static constexpr int POS_LANES = (BM + BN - 1 + 3 + 3) / 4;   // 16-byte pieces of one window copy
+  static constexpr int POS_COPY = POS_LANES * 16;   // one shifted copy of the window
+  static constexpr int POS_BYTES = 4 * POS_COPY;    // 4 copies shifted by 0..3 floats
+  static constexpr int TK_BYTES = BN * 8;           // int64 key timestamps
   static constexpr int TAB_BYTES = 132 * 4;
   static constexpr int total(bool pos, bool ts) {
-    return 2 * STAGE + (pos ? 2 * POS_BYTES : 0) + (ts ? 2 * TK_BYTES + TAB_BYTES : 0);
+    return NSTAGE * STAGE + (pos ? NSTAGE * POS_BYTES : 0) + (ts ? NSTAGE * TK_BYTES + TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
   __device__ static constexpr int swz_k(int row) { return (row / RPB) % CPR; }
@@ -320,16 +326,24 @@ struct MfmaSmem {
 
 typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
 
-// 64 lanes x 16 bytes, global -> LDS without passing through registers: lane l
-// of the wave writes LDS bytes [lds_base + 16 l, +16) with the 16 bytes at
-// gbase + byte_off(l).  Issued as inline assembly on purpose: the compiler
-// then does not know that LDS is written and does not put a "wait for all
-// outstanding loads" in front of every LDS read of the tile that is being
-// computed meanwhile.  The caller waits (vmcnt(0)) and barriers before anybody
-// reads the destination.
+// Direct global -> LDS loads, 64 lanes x 16 (or 4) bytes: lane l of the wave
+// writes LDS bytes [lds_base + size*l, +size) with the bytes at gbase +
+// byte_off(l).  Issued as inline assembly on purpose: the compiler then does
+// not know that LDS is written (it would otherwise put a wait for ALL
+// outstanding loads in front of every LDS read) nor that a load is in flight
+// (so it never waits for these itself).  The kernel counts them by hand:
+// every wave issues the same number per step and waits with s_waitcnt vmcnt(n)
+// before the barrier that publishes a stage.
 __device__ __forceinline__ void lds_dma16(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
   const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_byte_ptr)lds_dst_wave_uniform);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(base), "v"(byte_off), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+__device__ __forceinline__ void lds_dma4(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_byte_ptr)lds_dst_wave_uniform);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                :
                : "s"(base), "v"(byte_off), "s"(gbase_uniform)
                : "memory", "m0");
@@ -358,6 +372,20 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
   return __builtin_bit_cast(uint2, v);
 }
 
+// vmcnt(n) with expcnt / lgkmcnt left alone (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
+#define HSTU_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 15) | ((((n) >> 4) & 3) << 14)) | 0x0F70)
+
+// Scaled, zero-padded copy of the relative-position table: [heads][POS_PAD + 2L-1 + POS_PAD],
+// values times log2(e).  The margins make every window read of the main kernel in-bounds.
+__global__ void hstu_scale_pos_table(const float* __restrict__ tab, float* __restrict__ out, int heads, int len) {
+  const int stride = len + 2 * POS_PAD;
+  const int total = heads * stride;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
+    const int hd = i / stride, j = i - hd * stride - POS_PAD;
+    out[i] = (j >= 0 && j < len) ? tab[(int64_t)hd * len + j] * LOG2E : 0.f;
+  }
+}
+
 template <int D, bool POS, bool TS>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   using SM = MfmaSmem<D>;
@@ -365,18 +393,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   constexpr int KSTEPS = D / 16;       // MFMA k-steps over the head dim
   constexpr int DVB = D / 32;          // 32-row blocks of O^T
   constexpr int CH = BN * D / 8;       // 16-byte chunks in a K (or V) tile
-  constexpr int LD = CH / MFMA_THREADS;  // direct loads per lane per tile (each wave: LD x 1 KB)
-  static_assert(CH % MFMA_THREADS == 0, "tile must split evenly over the workgroup");
+  constexpr int NPIECE = CH / 64;      // 1 KB pieces (one wave-wide direct load each) in a tile
+  constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;  // direct loads per wave per tile and tensor
+  static_assert(CH % 64 == 0, "tile must be a whole number of 1 KB pieces");
+  constexpr int NDMA = 2 * LD + (POS ? 1 : 0) + (TS ? 1 : 0);   // direct loads per wave per step
+  static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // LDS map: [stage0: K | V][stage1: K | V][pos window x2][key ts x2][ts table]
-  auto Ks = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE); };
-  auto Vs = [&](int buf) { return (bf16_t*)(smem + buf * SM::STAGE + SM::K_BYTES); };
-  constexpr int POS_OFF = 2 * SM::STAGE;
-  constexpr int TK_OFF = POS_OFF + (POS ? 2 * SM::POS_BYTES : 0);
-  auto Wc = [&](int buf) { return (float*)(smem + POS_OFF + buf * SM::POS_BYTES); };
-  auto Tk = [&](int buf) { return (int64_t*)(smem + TK_OFF + buf * SM::TK_BYTES); };
-  float* TsTab = (float*)(smem + TK_OFF + 2 * SM::TK_BYTES);
+  // LDS map: [ring: NSTAGE x (K | V)][pos windows x NSTAGE][key timestamps x NSTAGE][ts table]
+  auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
+  auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
+  constexpr int POS_OFF = NSTAGE * SM::STAGE;
+  constexpr int TK_OFF = POS_OFF + (POS ? NSTAGE * SM::POS_BYTES : 0);
+  auto Wc = [&](int st) { return (float*)(smem + POS_OFF + st * SM::POS_BYTES); };
+  auto Tk = [&](int st) { return (int64_t*)(smem + TK_OFF + st * SM::TK_BYTES); };
+  float* TsTab = (float*)(smem + TK_OFF + NSTAGE * SM::TK_BYTES);
 
   // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with
   // its own L2.  All query tiles of one (sequence, head) go to the same XCD and
@@ -417,18 +448,6 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const int qrow = r0 + m;             // this lane's query row
   const bool wave_live = r0 < s.n_q;
 
-  // Q fragments (B operand of S^T = K Q^T): lane holds q[qrow][16ks+8hh .. +7]
-  bf16x8 qf[KSTEPS];
-  {
-    const bf16_t* qg = (const bf16_t*)p.q + s.bq + (int64_t)qrow * p.q_st + 8 * hh;
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-      uint4 t = {0u, 0u, 0u, 0u};
-      if (qrow < s.n_q) t = *(const uint4*)(qg + 16 * ks);
-      qf[ks] = __builtin_bit_cast(bf16x8, t);
-    }
-  }
-
   int kv_end = s.n_kv;
   if (p.causal) {
     int lim = q0 + BM < s.n_q ? q0 + BM : s.n_q;
@@ -436,21 +455,90 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   }
   const int nt = (kv_end + BN - 1) / BN;
   // last key this wave needs
-  const int wave_last = p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1);
+  const int wave_last = !wave_live ? -1 : (p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1));
 
   const float alpha2 = p.alpha * LOG2E;
   const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
+  // start of this head's padded table; entry x of the unpadded table sits at posw[POS_PAD + x]
+  const float* posw = POS ? (const float*)p.pos_scaled + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1 + 2 * POS_PAD) : nullptr;
+  const int64_t* tsg = TS ? p.ts + s.ts0 : nullptr;
+
+  // Direct loads of step t into ring stage t % NSTAGE.  Wave w fills 1 KB
+  // pieces w*LD .. w*LD+LD-1 of K and of V; lane l of piece j lands at chunk
+  // 64j + l, i.e. row (64j+l)/CPR, physical chunk (64j+l)%CPR, and fetches the
+  // logical chunk that the swizzle maps there.  Rows past the sequence re-read
+  // the last valid row (finite data; their logits are masked).  One more load
+  // per wave brings the bias operands: a shifted copy of the position window
+  // (waves 0-3, or 4-7 when there are no timestamps) or half of the 64 key
+  // timestamps (waves 4-5; the others repeat a load so that every wave issues
+  // the same number, which the vmcnt arithmetic relies on).
+  auto dma_step = [&](int t) {
+    const int st = t % NSTAGE;
+    const int kv0 = t * BN;
+    const int last = s.n_kv - 1;
+#pragma unroll
+    for (int r = 0; r < LD; ++r) {
+      const int j = (w * LD + r) % NPIECE;   // small tiles: two waves repeat the same piece
+      const int c = 64 * j + lane;
+      const int row = c / CPR, pc = c - row * CPR;
+      int grow = kv0 + row;
+      grow = grow < last ? grow : last;
+      const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
+      const uint32_t voff = (uint32_t)grow * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
+      lds_dma16(kg, koff, Ks(st) + j * 512);
+      lds_dma16(vg, voff, Vs(st) + j * 512);
+    }
+    if (POS) {
+      // copy c (wave c) holds window[x + c], window[x] = pos[(L-1) + kv0 - (q0+127) + x];
+      // the index is >= POS_PAD - 127 > 0 and inside the padded table (the offset register is
+      // unsigned: a negative index would address 4 GB past the base)
+      if (lane < SM::POS_LANES) {
+        const int idx = POS_PAD + (p.L - 1) + kv0 - (q0 + BM - 1) + w + 4 * lane;
+        lds_dma16(posw, (uint32_t)idx * 4u, (const unsigned char*)Wc(st) + w * SM::POS_COPY);
+      }
+    }
+    if (TS) {
+      // BN int64 = 2*BN dwords, one per lane (every wave repeats this load so that all issue
+      // the same number, which the vmcnt arithmetic relies on)
+      int jk = kv0 + (lane >> 1);
+      jk = jk < s.n_ts ? jk : s.n_ts - 1;
+      jk = jk < 0 ? 0 : jk;
+      lds_dma4(tsg, (uint32_t)(jk * 8 + 4 * (lane & 1)), Tk(st));
+    }
+  };
+
+  // prologue: three steps in flight before anything else
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t)
+    if (t < nt) dma_step(t);
+
+  // Q fragments (B operand of S^T = K Q^T): lane holds q[qrow][16ks+8hh .. +7]
+  bf16x8 qf[KSTEPS];
+  {
+    const bf16_t* qg = (const bf16_t*)p.q + s.bq + (int64_t)qrow * p.q_st + 8 * hh;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      uint4 t4 = {0u, 0u, 0u, 0u};
+      if (qrow < s.n_q) t4 = *(const uint4*)(qg + 16 * ks);
+      qf[ks] = __builtin_bit_cast(bf16x8, t4);
+    }
+    // Use the fragments here so that the compiler's wait for these loads sits in the prologue.
+    // Left to the first use inside the loop it would be a vmcnt(0) on every step, which also
+    // waits for every direct load in flight and serialises the whole ring.
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[ks]));
+  }
   int64_t tq = 0;
   if (TS) {
     int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
     tq = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
+    asm volatile("" ::"v"(tq));
     const float* tab = p.ts_tab + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1);
     for (int e = tid; e < 132; e += MFMA_THREADS) {
       int c = e <= p.ts_nb ? e : p.ts_nb;
       TsTab[e] = tab[c > 128 ? 128 : c] * LOG2E;
     }
   }
-  const float* postab = POS ? p.pos_tab + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) : nullptr;
 
   floatx16 o[DVB];
 #pragma unroll
@@ -458,50 +546,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
 
-  // Direct global->LDS loads of the next K/V tile: wave w fills 1 KB pieces
-  // w*LD .. w*LD+LD-1 of each tile; lane l of piece j lands at chunk 64j + l,
-  // i.e. row (64j+l)/CPR, physical chunk (64j+l)%CPR, and fetches the logical
-  // chunk that the swizzle maps there.  Rows past the sequence re-read the
-  // last valid row (finite data; their logits are masked).
-  auto gload = [&](int buf, int kv0) {
-    const int last = s.n_kv - 1;
-#pragma unroll
-    for (int r = 0; r < LD; ++r) {
-      const int j = w * LD + r;
-      const int c = 64 * j + lane;
-      const int row = c / CPR, pc = c - row * CPR;
-      int grow = kv0 + row;
-      grow = grow < last ? grow : last;
-      const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
-      const uint32_t voff = (uint32_t)grow * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
-      lds_dma16(kg, koff, Ks(buf) + j * 512);
-      lds_dma16(vg, voff, Vs(buf) + j * 512);
-    }
-  };
-
-  // bias operands of the next tile (small; staged through registers)
-  auto stage_bias = [&](int buf, int kv0) {
-    if (POS) {
-      // window[x] = log2e * pos_tab[(L-1) + kv0 - (q0+127) + x]; copy s is shifted by s
-      const int idx0 = (p.L - 1) + kv0 - (q0 + BM - 1);
-      for (int e = tid; e < 4 * POSW; e += MFMA_THREADS) {
-        int sft = e / POSW, z = e - sft * POSW;
-        int idx = idx0 + z + sft;
-        Wc(buf)[e] = (idx >= 0 && idx < 2 * p.L - 1) ? postab[idx] * LOG2E : 0.f;
-      }
-    }
-    if (TS) {
-      if (tid < BN) {
-        int jk = kv0 + tid;
-        jk = jk < s.n_ts ? jk : s.n_ts - 1;
-        Tk(buf)[tid] = p.ts[s.ts0 + (jk < 0 ? 0 : jk)];
-      }
-    }
-  };
-
-  // K: lane (row m, half hh) reads logical chunk 2ks+hh of rows m and 32+m (same swizzle for both)
+  // K: lane (row m, half hh) reads logical chunk 2ks+hh of row m
   const int gk = SM::swz_k(m);
-  // V: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc + 32kb):
+  // V: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc):
   // logical chunk 4dvb + 2(G&1) + (i&3)/2, byte half (i&3)&1
   const int gi = lane & 15;
   const int vrow = 4 * hh + (gi >> 2);
@@ -509,15 +556,16 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
 
   // One 32-key block for this wave: logits, bias, SiLU, P.V.  Blocks that touch
-  // the causal diagonal or the end of the sequence get their logits and bias
-  // zeroed where masked: silu(0) = 0 exactly, so nothing is needed after the
-  // activation and interior blocks pay nothing.
-  auto block = [&](int buf, int kv0, int kb) {
-    const int kbs = kv0 + 32 * kb;
-    const bf16_t* kr = Ks(buf) + (32 * kb + m) * D;
+  // the causal diagonal or the end of the sequence get their logits zeroed where
+  // masked: silu(0) = 0 exactly, so nothing is needed after the activation and
+  // interior blocks pay nothing.
+  auto block = [&](int t) {
+    const int st = t % NSTAGE;
+    const int kbs = t * BN;
     floatx16 sacc;
     {
       bf16x8 kf[KSTEPS];
+      const bf16_t* kr = Ks(st) + m * D;
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + (((2 * ks + hh) ^ gk) * 8));
       const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -528,7 +576,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     // V fragments, requested now so that they arrive while the SiLU runs
     uint4 vf[2][DVB];
     {
-      const bf16_t* vr = Vs(buf) + (32 * kb + vrow) * D + 4 * (gi & 1);
+      const bf16_t* vr = Vs(st) + vrow * D + 4 * (gi & 1);
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
@@ -539,12 +587,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
           vf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
         }
     }
-    // lane holds S^T[kv = kbs + 8g + 4hh + t][q = qrow], r = 4g + t
+    // lane holds S^T[kv = kbs + 8g + 4hh + tt][q = qrow], r = 4g + tt
     float u[16];
     if (POS) {
-      const int xb = 32 * kb + 4 * hh + (BM - 1) - 32 * w - m;
+      const int xb = 4 * hh + (BM - 1) - 32 * w - m;
       const int sft = xb & 3;
-      const float* wrow = Wc(buf) + sft * POSW + (xb - sft);
+      const float* wrow = (const float*)((const unsigned char*)Wc(st) + sft * SM::POS_COPY) + (xb - sft);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         float4 bv = *(const float4*)(wrow + 8 * g);
@@ -558,7 +606,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
     if (TS) {
-      const int64_t* tk = Tk(buf) + 32 * kb + 4 * hh;
+      const int64_t* tk = Tk(st) + 4 * hh;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
 #pragma unroll
@@ -598,21 +646,25 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     }
   };
 
-  gload(0, 0);
-  stage_bias(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads have landed in LDS
+  // wait until this wave's loads of step `t` have landed, leaving younger steps in flight
+  auto wait_step = [&](int t) {
+    int younger = nt - 1 - t;                  // steps issued after t
+    younger = younger > NSTAGE - 2 ? NSTAGE - 2 : younger;
+    if (younger >= 2) HSTU_WAIT_VMCNT(2 * NDMA);
+    else if (younger == 1) HSTU_WAIT_VMCNT(NDMA);
+    else HSTU_WAIT_VMCNT(0);
+  };
+
+  wait_step(0);
   __syncthreads();
 
+  // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
+  // which now receives step t+3; the block of step t is computed; then every
+  // wave makes sure its share of step t+1 has landed before the next barrier.
   for (int t = 0; t < nt; ++t) {
-    const int kv0 = t * BN;
-    const int buf = t & 1;
-    if (t + 1 < nt) gload(buf ^ 1, kv0 + BN);
-    if (wave_live) {
-      if (kv0 <= wave_last) block(buf, kv0, 0);
-      if (kv0 + 32 <= wave_last) block(buf, kv0, 1);
-    }
-    if (t + 1 < nt) stage_bias(buf ^ 1, kv0 + BN);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+    if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
+    if (t * BN <= wave_last) block(t);
+    if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
   }
 
@@ -626,12 +678,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     for (int dvb = 0; dvb < DVB; ++dvb) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        uint2 pk = {0u, 0u};
+        uint2 pko = {0u, 0u};
         if (live) {
-          pk.x = pack_bf16(o[dvb][4 * g + 0] * oscale, o[dvb][4 * g + 1] * oscale);
-          pk.y = pack_bf16(o[dvb][4 * g + 2] * oscale, o[dvb][4 * g + 3] * oscale);
+          pko.x = pack_bf16(o[dvb][4 * g + 0] * oscale, o[dvb][4 * g + 1] * oscale);
+          pko.y = pack_bf16(o[dvb][4 * g + 2] * oscale, o[dvb][4 * g + 3] * oscale);
         }
-        *(uint2*)(orow + 32 * dvb + 8 * g) = pk;
+        *(uint2*)(orow + 32 * dvb + 8 * g) = pko;
       }
     }
   }
@@ -713,8 +765,17 @@ Variant pick_variant(const HstuAttnFwdArgs* a) {
                         s8(a->v_stride_t) && s8(a->v_stride_h) && s8(a->o_stride_t) && s8(a->o_stride_h) &&
                         (a->layout == HSTU_LAYOUT_JAGGED ||
                          (s8(a->q_stride_b) && s8(a->k_stride_b) && s8(a->v_stride_b) && s8(a->o_stride_b)));
-  if (d_ok && opts_ok && align_ok) return V_MFMA_BF16;
+  // the MFMA kernel addresses K and V rows with 32-bit byte offsets from the (sequence, head) base
+  const bool off_ok = (int64_t)a->L * a->k_stride_t * 2 < (1LL << 31) && (int64_t)a->L * a->v_stride_t * 2 < (1LL << 31) &&
+                      a->k_stride_t > 0 && a->v_stride_t > 0;
+  if (d_ok && opts_ok && align_ok && off_ok) return V_MFMA_BF16;
   return V_GENERAL_BF16;
+}
+
+// The MFMA kernel reads the relative-position table from a scaled, zero-padded copy.
+size_t workspace_needed(const HstuAttnFwdArgs* a) {
+  if (pick_variant(a) != V_MFMA_BF16 || !a->pos_tab) return 0;
+  return (size_t)a->pos_heads * (size_t)(2 * a->L - 1 + 2 * POS_PAD) * sizeof(float);
 }
 
 Params make_params(const HstuAttnFwdArgs* a) {
@@ -803,8 +864,8 @@ int hstu_attn_abi_version(void) { return HSTU_ATTN_ABI_VERSION; }
 const char* hstu_attn_last_error(void) { return g_err; }
 
 size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args) {
-  (void)args;
-  return 0;
+  if (validate(args) != HSTU_OK) return 0;
+  return workspace_needed(args);
 }
 
 const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
@@ -817,6 +878,17 @@ const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
   }
 }
 
+// Diagnostics: resident workgroups per CU of one MFMA kernel instantiation.
+int hstu_attn_debug_occupancy(int d, int pos, int ts) {
+  int n = -1;
+  hipError_t e = hipErrorInvalidValue;
+#define OCC(D_, P_, T_) if (d == D_ && !!pos == P_ && !!ts == T_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)hstu_fwd_mfma_bf16<D_, P_, T_>, MFMA_THREADS, MfmaSmem<D_>::total(P_, T_));
+  OCC(128, false, false) OCC(128, true, false) OCC(128, false, true) OCC(128, true, true)
+  OCC(64, false, false) OCC(64, true, true) OCC(32, false, false) OCC(32, true, true)
+#undef OCC
+  return e == hipSuccess ? n : -(int)e;
+}
+
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
   int rc = validate(args);
   if (rc != HSTU_OK) return rc;
@@ -827,10 +899,29 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
   switch (pick_variant(args)) {
     case V_GENERAL_F32: return launch_general<float>(p, st);
     case V_GENERAL_BF16: return launch_general<bf16_t>(p, st);
-    case V_MFMA_BF16:
+    case V_MFMA_BF16: {
+      const size_t ws = workspace_needed(args);
+      if (ws) {
+        if (!args->workspace || args->workspace_bytes < ws)
+          return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes needed (see hstu_attn_fwd_workspace_bytes), got %zu",
+                      ws, args->workspace ? args->workspace_bytes : (size_t)0);
+        if (((uintptr_t)args->workspace & 15u) != 0) return fail(HSTU_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+        Params q = p;
+        q.pos_scaled = (const float*)args->workspace;
+        const int len = 2 * p.L - 1;
+        const int total = p.pos_heads * (len + 2 * POS_PAD);
+        hipLaunchKernelGGL(hstu_scale_pos_table, dim3((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024), dim3(256), 0, st,
+                           p.pos_tab, (float*)args->workspace, p.pos_heads, len);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "table kernel launch: %s", hipGetErrorString(e));
+        if (q.d_qk == 128) return launch_mfma_d<128>(q, st);
+        if (q.d_qk == 64) return launch_mfma_d<64>(q, st);
+        return launch_mfma_d<32>(q, st);
+      }
       if (p.d_qk == 128) return launch_mfma_d<128>(p, st);
       if (p.d_qk == 64) return launch_mfma_d<64>(p, st);
       return launch_mfma_d<32>(p, st);
+    }
     default: return fail(HSTU_ERR_SHAPE, "no kernel for these arguments");
   }
 }

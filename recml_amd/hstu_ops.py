@@ -66,14 +66,18 @@ def _as_table(name, t, H, width, device):
   return t.to(device=device, dtype=torch.float32).contiguous()
 
 
-def _run(args, keep):
-  lib = _lib.load()
-  ws = lib.hstu_attn_fwd_workspace_bytes(C.byref(args))
+def _attach_workspace(args, keep):
+  """Allocates the device scratch the library asks for (once per argument set)."""
+  ws = _lib.load().hstu_attn_fwd_workspace_bytes(C.byref(args))
   if ws:
     buf = torch.empty(ws, dtype=torch.uint8, device=keep[0].device)
     keep.append(buf)
     args.workspace = buf.data_ptr()
     args.workspace_bytes = ws
+
+
+def _run(args, keep):
+  lib = _lib.load()
   stream = torch.cuda.current_stream(keep[0].device).cuda_stream
   rc = lib.hstu_attn_fwd(C.byref(args), C.c_void_p(stream))
   if rc != 0:
@@ -245,6 +249,8 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
     a.ts_tab, a.ts_heads, a.ts = tt.data_ptr(), tt.shape[0], ts.data_ptr()
     a.ts_num_buckets = tt.shape[1] - 1
     a.ts_bucket_size = float(ts_bucket_size)
+  if q.is_cuda:
+    _attach_workspace(a, keep)
   return a, keep
 
 

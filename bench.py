@@ -93,6 +93,16 @@ def cpu_baseline(w, q, k, v, out_gpu):
   }, err
 
 
+def measured_traffic(workload):
+  """HBM bytes per launch from the rocprofv3 counter runs recorded in profiles/traffic.json
+  (FETCH_SIZE + WRITE_SIZE of the attention kernel, scaled by a copy kernel of known size)."""
+  path = os.path.join(ROOT, "profiles", "traffic.json")
+  if not os.path.exists(path):
+    return None
+  rec = json.load(open(path)).get(workload)
+  return None if rec is None else rec["hbm_bytes_per_launch"]
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -100,6 +110,8 @@ def main():
   ap.add_argument("--warmup", type=int, default=20)
   ap.add_argument("--workload", default="c3")
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+  ap.add_argument("--calib-copy", action="store_true",
+                  help="also run one 512 MiB device copy (reference point for HBM byte counters)")
   args = ap.parse_args()
   if args.gpus != 1:
     raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -120,6 +132,13 @@ def main():
 
   def step():
     hstu_ops._run(call_args, keep)
+
+  if args.calib_copy:
+    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
   for _ in range(args.warmup):
     step()
@@ -162,7 +181,7 @@ def main():
       "seqs_per_s": w.B / (ms_per_step * 1e-3),
       "roofline": {
           "bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-          "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+          "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic(args.workload),
           "kernel_ms_avg": kernel_ms, "kernel_ms_min": float(ev_ms.min()),
           "kernel_ms_median": float(np.median(ev_ms)),
           "region_ms_per_step": region_ms / args.steps,

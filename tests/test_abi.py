@@ -1,0 +1,103 @@
+"""The C ABI: the library loads, exports every declared symbol, and the ctypes
+image of HstuAttnFwdArgs matches the C struct.  No GPU work is launched: every
+call here returns from argument validation."""
+
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import pytest
+
+from recml_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hstu_attn.h")
+
+
+def _declared_functions():
+  text = open(HEADER).read()
+  return sorted(set(re.findall(r"\b(hstu_attn_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+  lib = _lib.load()
+  names = _declared_functions()
+  assert set(names) == set(_lib.EXPORTS)
+  for n in names:
+    assert getattr(lib, n) is not None
+  assert lib.hstu_attn_abi_version() == _lib.ABI_VERSION
+
+
+def test_struct_layout_matches_header():
+  fields = [f[0] for f in _lib.HstuAttnFwdArgs._fields_]
+  prog = ['#include <stdio.h>', '#include <stddef.h>', '#include "hstu_attn.h"', "int main(void) {",
+          '  printf("%zu\\n", sizeof(HstuAttnFwdArgs));']
+  prog += [f'  printf("%zu\\n", offsetof(HstuAttnFwdArgs, {f}));' for f in fields]
+  prog += ["  return 0;", "}"]
+  with tempfile.TemporaryDirectory() as d:
+    src = os.path.join(d, "layout.c")
+    exe = os.path.join(d, "layout")
+    open(src, "w").write("\n".join(prog))
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), "-o", exe, src], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
+  assert int(out[0]) == C.sizeof(_lib.HstuAttnFwdArgs)
+  for f, off in zip(fields, out[1:]):
+    assert getattr(_lib.HstuAttnFwdArgs, f).offset == int(off), f
+
+
+def test_validation_errors_without_gpu():
+  lib = _lib.load()
+  assert lib.hstu_attn_fwd(None, None) == -1                 # HSTU_ERR_NULL
+  a = _lib.new_args()
+  a.version = 99
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -2           # HSTU_ERR_VERSION
+  assert b"version" in lib.hstu_attn_last_error()
+  a = _lib.new_args()
+  a.B, a.L, a.Lkv, a.H, a.d_qk, a.d_v = 1, 8, 8, 1, 32, 32
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -1           # q/k/v/out null
+  a.q = a.k = a.v = a.out = 0x1000                           # never dereferenced: validation fails first
+  a.d_qk = 512
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -4           # HSTU_ERR_SHAPE
+  a.d_qk = 32
+  a.qk_dtype, a.v_dtype, a.out_dtype = 0, 1, 1
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -3           # HSTU_ERR_DTYPE
+  a.qk_dtype = a.v_dtype = a.out_dtype = 1
+  a.mask_mode = _lib.MASK_SEGMENT
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -1           # one-sided / missing segment ids
+  assert b"segment" in lib.hstu_attn_last_error()
+  a.mask_mode = _lib.MASK_LENGTH
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -1           # LENGTH needs seq_lens
+  a.mask_mode = _lib.MASK_NONE
+  a.layout = _lib.LAYOUT_JAGGED
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -1           # jagged needs offsets
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"invalid"
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 0
+
+
+def test_variant_and_workspace_query():
+  lib = _lib.load()
+  a = _lib.new_args()
+  a.B, a.L, a.Lkv, a.H, a.d_qk, a.d_v = 2, 256, 256, 4, 128, 128
+  a.q = a.k = a.v = a.out = 0x10000
+  a.q_stride_t = a.k_stride_t = a.v_stride_t = a.o_stride_t = 4 * 128
+  a.q_stride_h = a.k_stride_h = a.v_stride_h = a.o_stride_h = 128
+  a.q_stride_b = a.k_stride_b = a.v_stride_b = a.o_stride_b = 256 * 4 * 128
+  a.alpha, a.inv_n, a.causal = 1.0, 1.0 / 256, 1
+  a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 0
+  a.pos_tab, a.pos_heads = 0x20000, 4
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 4 * (2 * 256 - 1 + 512) * 4
+  # a launch without the workspace is refused before anything is enqueued
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -5
+  a.pos_tab = None
+  a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_FP32
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<float>"
+  a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
+  a.window = 4
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"
+  a.window = -1
+  a.d_qk = a.d_v = 48
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"

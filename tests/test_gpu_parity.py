@@ -161,6 +161,36 @@ def test_mfma_head_dims_and_full_mask(gpu, d, causal):
   assert _err(out.float().cpu().numpy(), ref) <= BF16_TOL
 
 
+@pytest.mark.parametrize("layout", ["padded", "jagged"])
+def test_few_long_sequences(gpu, layout):
+  # few sequences of very different lengths, length not a multiple of any tile size,
+  # called twice on the same buffers (a call must not depend on what the previous one left)
+  rng = np.random.default_rng(77)
+  B, L, H, d = 3, 1100, 2, 64
+  lens = np.array([1100, 513, 40], dtype=np.int32)
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.2) for _ in range(3))
+  pos = rng.standard_normal((H, 2 * L - 1)).astype(np.float32) * 0.1
+  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, pos_tab=pos, dtype=np.float32)
+  for rep in range(2):
+    if layout == "padded":
+      out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
+                                     seq_lens=_dev(lens), pos_bias=_dev(pos)).float().cpu().numpy()
+      for b in range(B):
+        assert (out[b, lens[b]:] == 0).all()
+    else:
+      qj, off = O.padded_to_jagged(q, lens)
+      kj, _ = O.padded_to_jagged(k, lens)
+      vj, _ = O.padded_to_jagged(v, lens)
+      outj = recml_amd.hstu_attention(_dev(qj, torch.bfloat16), _dev(kj, torch.bfloat16), _dev(vj, torch.bfloat16),
+                                      seq_offsets=_dev(off.astype(np.int32)), max_len=L, pos_bias=_dev(pos))
+      out = O.jagged_to_padded(outj.float().cpu().numpy(), off, L)
+    assert _err(out, ref) <= BF16_TOL
+  # full (non-causal) mask through the same path
+  out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
+                                 seq_lens=_dev(lens), causal=False).float().cpu().numpy()
+  assert _err(out, O.hstu_attention_ref(q, k, v, seq_lens=lens, causal=False, dtype=np.float32)) <= BF16_TOL
+
+
 def test_ragged_and_empty(gpu):
   rng = np.random.default_rng(5)
   H, d, L = 2, 64, 300

@@ -39,6 +39,15 @@ def make_workload(name):
     return workloads.config3(full=True, bias=False)
   if name == "c3-nobias":
     return workloads.config3(bias=False)
+  if name in ("c3full-ts", "c3full-pos", "c3-ts", "c3-pos"):
+    # one bias only (profiling aid)
+    w = workloads.config3(full=name.startswith("c3full"))
+    if name.endswith("-ts"):
+      w.pos_tab = None
+    else:
+      w.ts_tab = None
+      w.timestamps = None
+    return w
   if name == "c2":
     return workloads.config2()
   if name == "c4":

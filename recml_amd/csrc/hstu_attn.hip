@@ -61,6 +61,13 @@ struct Params {
   const float* ts_tab;
   const int64_t* ts;
   const float* pos_scaled;   // workspace: log2(e) * pos_tab, zero-padded (MFMA kernel)
+  // workspace of the MFMA kernel's timestamp path: per sequence, 1 when max - min timestamp fits
+  // 31 bits; then timestamps minus the sequence minimum as int32, and their (min, max) per 32-key tile
+  const int32_t* ts_ok;
+  const int32_t* ts_rel;
+  const int32_t* ts_range;
+  const float* ts_scaled;    // workspace: log2(e) * ts_tab as [heads][TS_TAB_LEN], indices past the last bucket repeat it
+  const void* ws_base;       // start of the workspace (all of the above lie within 4 GB of it)
   int64_t ts_sb;
   int32_t B, L, Lkv, H, d_qk, d_v;
   int32_t jagged, causal, mask_mode, window;
@@ -297,6 +304,7 @@ constexpr int NSTAGE = 4;     // LDS ring depth
 constexpr int MFMA_THREADS = 256;
 constexpr int NWAVES = MFMA_THREADS / 64;
 constexpr int POS_PAD = 256;  // zero margin on both sides of the scaled position table
+constexpr int TS_TAB_LEN = 192;  // entries of the scaled bucket table (3 waves x 64 lanes of one direct load)
 constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D>
@@ -313,10 +321,12 @@ struct MfmaSmem {
   static constexpr int POS_LANES = (BM + BN - 1 + 3 + 3) / 4;   // 16-byte pieces of one window copy
   static constexpr int POS_COPY = POS_LANES * 16;   // one shifted copy of the window
   static constexpr int POS_BYTES = 4 * POS_COPY;    // 4 copies shifted by 0..3 floats
-  static constexpr int TK_BYTES = BN * 8;           // int64 key timestamps
-  static constexpr int TAB_BYTES = 132 * 4;
+  static constexpr int TK_LANES = BN / 4 + 1;       // 16-byte pieces: 32 int32 key timestamps, then (min, max, -, -)
+  static constexpr int TK_BYTES = TK_LANES * 16;
+  static constexpr int TAB_BYTES = TS_TAB_LEN * 4;
+  static constexpr int bias_stage(bool pos, bool ts) { return (pos ? POS_BYTES : 0) + (ts ? TK_BYTES : 0); }
   static constexpr int total(bool pos, bool ts) {
-    return NSTAGE * STAGE + (pos ? NSTAGE * POS_BYTES : 0) + (ts ? NSTAGE * TK_BYTES + TAB_BYTES : 0);
+    return NSTAGE * (STAGE + bias_stage(pos, ts)) + (ts ? TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
   __device__ static constexpr int swz_k(int row) { return (row / RPB) % CPR; }
@@ -375,14 +385,96 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
 // vmcnt(n) with expcnt / lgkmcnt left alone (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
 #define HSTU_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 15) | ((((n) >> 4) & 3) << 14)) | 0x0F70)
 
-// Scaled, zero-padded copy of the relative-position table: [heads][POS_PAD + 2L-1 + POS_PAD],
-// values times log2(e).  The margins make every window read of the main kernel in-bounds.
-__global__ void hstu_scale_pos_table(const float* __restrict__ tab, float* __restrict__ out, int heads, int len) {
-  const int stride = len + 2 * POS_PAD;
-  const int total = heads * stride;
-  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < total; i += gridDim.x * blockDim.x) {
-    const int hd = i / stride, j = i - hd * stride - POS_PAD;
-    out[i] = (j >= 0 && j < len) ? tab[(int64_t)hd * len + j] * LOG2E : 0.f;
+// Where sequence b starts in the int32 timestamp copy and in the per-tile range table.
+// Timestamps that follow the token axis are packed like it (tiles by an upper bound of
+// the tiles before them); timestamps with a batch stride are [B][L].
+__device__ __forceinline__ int64_t ts_rel_base(const Params& p, int b, int64_t tok0) {
+  return p.ts_sb != 0 ? (int64_t)b * p.L : tok0;
+}
+__device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_t tok0) {
+  return p.ts_sb != 0 ? (int64_t)b * ((p.L + BN - 1) / BN) : (tok0 >> 5) + b;
+}
+
+// What the main kernel reads from the workspace, rebuilt by every call:
+//  * the relative-position table scaled by log2(e) and zero-padded,
+//    [heads][POS_PAD + 2L-1 + POS_PAD]; the margins make every window read in-bounds;
+//  * the timestamp bucket table scaled by log2(e), [heads][TS_TAB_LEN];
+//  * per sequence whose timestamps span less than 2^31: the timestamps minus their minimum
+//    as int32 (differences of two of them are then exact in 32 bits), and the (min, max)
+//    of those in each 32-key tile.  One workgroup per sequence.
+__global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __restrict__ pos_out, float* __restrict__ tab_out,
+                                                    int32_t* __restrict__ ok_out, int32_t* __restrict__ rel_out,
+                                                    int32_t* __restrict__ range_out) {
+  const int tid = threadIdx.x;
+  const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
+  if (tab_out) {
+    // bucket table times log2(e); indices past the last bucket repeat it (the clip of the bucket law)
+    for (int i = gtid; i < p.ts_heads * TS_TAB_LEN; i += gsz) {
+      const int hd = i / TS_TAB_LEN, e = i - hd * TS_TAB_LEN;
+      tab_out[i] = p.ts_tab[(int64_t)hd * (p.ts_nb + 1) + (e < p.ts_nb ? e : p.ts_nb)] * LOG2E;
+    }
+  }
+  if (pos_out) {
+    const int len = 2 * p.L - 1;
+    const int stride = len + 2 * POS_PAD;
+    const int total = p.pos_heads * stride;
+    for (int i = gtid; i < total; i += gsz) {
+      const int hd = i / stride, j = i - hd * stride - POS_PAD;
+      pos_out[i] = (j >= 0 && j < len) ? p.pos_tab[(int64_t)hd * len + j] * LOG2E : 0.f;
+    }
+  }
+  if (!ok_out) return;
+  static_assert(BN == 32, "one lane per key of a tile");
+  __shared__ int64_t red_lo[4], red_hi[4];
+  const int lane = tid & 63, wv = tid >> 6, l32 = tid & 31;
+  for (int b = blockIdx.x; b < p.B; b += gridDim.x) {
+    const Seq s = seq_info(p, b, 0);
+    const int n = s.n_ts;
+    if (n <= 0) {
+      if (tid == 0) ok_out[b] = 0;
+      continue;
+    }
+    const int64_t* ts = p.ts + s.ts0;
+    int64_t lo_v = ts[0], hi_v = lo_v;
+    for (int j = tid; j < n; j += 256) {
+      const int64_t x = ts[j];
+      lo_v = x < lo_v ? x : lo_v;
+      hi_v = x > hi_v ? x : hi_v;
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+      const int64_t a = __shfl_xor(lo_v, d, 64), c = __shfl_xor(hi_v, d, 64);
+      lo_v = a < lo_v ? a : lo_v;
+      hi_v = c > hi_v ? c : hi_v;
+    }
+    __syncthreads();   // the previous sequence's readers are done with red_*
+    if (lane == 0) { red_lo[wv] = lo_v; red_hi[wv] = hi_v; }
+    __syncthreads();
+    for (int i = 0; i < 4; ++i) {
+      lo_v = red_lo[i] < lo_v ? red_lo[i] : lo_v;
+      hi_v = red_hi[i] > hi_v ? red_hi[i] : hi_v;
+    }
+    const bool ok = ((uint64_t)hi_v - (uint64_t)lo_v) < 0x7fffffffull;
+    if (tid == 0) ok_out[b] = ok ? 1 : 0;
+    if (!ok) continue;
+    int32_t* rel = rel_out + ts_rel_base(p, b, s.tok0);
+    int32_t* rng = range_out + 2 * ts_range_slot0(p, b, s.tok0);
+    const int tiles = (n + BN - 1) / BN;
+    for (int t = tid >> 5; t < tiles; t += 8) {   // one half-wave per tile
+      int j = t * BN + l32;
+      const bool live = j < n;
+      j = live ? j : n - 1;
+      const int32_t r = (int32_t)(ts[j] - lo_v);
+      if (live) rel[j] = r;
+      int32_t mn = r, mx = r;
+#pragma unroll
+      for (int d = 16; d >= 1; d >>= 1) {
+        const int32_t a = __shfl_xor(mn, d, 32), c = __shfl_xor(mx, d, 32);
+        mn = a < mn ? a : mn;
+        mx = c > mx ? c : mx;
+      }
+      if (l32 == 0) { rng[2 * t] = mn; rng[2 * t + 1] = mx; }
+    }
   }
 }
 
@@ -396,18 +488,20 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   constexpr int NPIECE = CH / 64;      // 1 KB pieces (one wave-wide direct load each) in a tile
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;  // direct loads per wave per tile and tensor
   static_assert(CH % 64 == 0, "tile must be a whole number of 1 KB pieces");
-  constexpr int NDMA = 2 * LD + (POS ? 1 : 0) + (TS ? 1 : 0);   // direct loads per wave per step
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);   // direct loads per wave per step
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  // LDS map: [ring: NSTAGE x (K | V)][pos windows x NSTAGE][key timestamps x NSTAGE][ts table]
+  // LDS map: [ring: NSTAGE x (K | V)][bias operands x NSTAGE: 4 pos windows | key timestamps][ts table].
+  // The key timestamps sit right behind the last position window so that one direct load of the
+  // last wave can fill both.
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
-  constexpr int POS_OFF = NSTAGE * SM::STAGE;
-  constexpr int TK_OFF = POS_OFF + (POS ? NSTAGE * SM::POS_BYTES : 0);
-  auto Wc = [&](int st) { return (float*)(smem + POS_OFF + st * SM::POS_BYTES); };
-  auto Tk = [&](int st) { return (int64_t*)(smem + TK_OFF + st * SM::TK_BYTES); };
-  float* TsTab = (float*)(smem + TK_OFF + NSTAGE * SM::TK_BYTES);
+  constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS);
+  auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
+  auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
+  float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
 
   // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with
   // its own L2.  All query tiles of one (sequence, head) go to the same XCD and
@@ -459,9 +553,17 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 
   const float alpha2 = p.alpha * LOG2E;
   const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
-  // start of this head's padded table; entry x of the unpadded table sits at posw[POS_PAD + x]
-  const float* posw = POS ? (const float*)p.pos_scaled + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1 + 2 * POS_PAD) : nullptr;
+  // Bias operands are fetched with 32-bit byte offsets from the start of the workspace.
+  // pos_off: this head's padded table; entry x of the unpadded table sits at float POS_PAD + x.
+  const char* wsb = (const char*)p.ws_base;
+  const uint32_t pos_off = POS ? (uint32_t)((const char*)(p.pos_scaled + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1 + 2 * POS_PAD)) - wsb) : 0u;
   const int64_t* tsg = TS ? p.ts + s.ts0 : nullptr;
+  // int32 timestamps of this sequence, valid when its time span allows them (ts_ok, same for the
+  // whole workgroup; read now, needed only when the first block is computed)
+  const int32_t* trel = TS ? p.ts_rel + ts_rel_base(p, b, s.tok0) : nullptr;
+  const int ts32 = TS ? p.ts_ok[b] : 0;
+  const uint32_t rel_off = TS ? (uint32_t)((const char*)trel - wsb) : 0u;
+  const uint32_t rng_off = TS ? (uint32_t)((const char*)(p.ts_range + 2 * ts_range_slot0(p, b, s.tok0)) - wsb) : 0u;
 
   // Direct loads of step t into ring stage t % NSTAGE.  Wave w fills 1 KB
   // pieces w*LD .. w*LD+LD-1 of K and of V; lane l of piece j lands at chunk
@@ -488,26 +590,41 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       lds_dma16(kg, koff, Ks(st) + j * 512);
       lds_dma16(vg, voff, Vs(st) + j * 512);
     }
-    if (POS) {
-      // copy c (wave c) holds window[x + c], window[x] = pos[(L-1) + kv0 - (q0+127) + x];
-      // the index is >= POS_PAD - 127 > 0 and inside the padded table (the offset register is
-      // unsigned: a negative index would address 4 GB past the base)
-      if (lane < SM::POS_LANES) {
-        const int idx = POS_PAD + (p.L - 1) + kv0 - (q0 + BM - 1) + w + 4 * lane;
-        lds_dma16(posw, (uint32_t)idx * 4u, (const unsigned char*)Wc(st) + w * SM::POS_COPY);
+    if (POS || TS) {
+      // One more load per wave brings the bias operands.  Wave c writes position-window copy c:
+      // window[x + c], window[x] = pos[(L-1) + kv0 - (q0+127) + x]; the table index is
+      // >= POS_PAD - 127 > 0 and inside the padded table (the offset register is unsigned: a
+      // negative index would address 4 GB past the base).  The lanes behind the last wave's copy
+      // (or the first lanes of every wave when there is no position bias) bring 32 int32 key
+      // timestamps, 4 per lane, and the tile's (min, max).  Keys past the sequence read whatever
+      // follows in the workspace: their logits are masked.
+      constexpr int TS_LANE0 = POS ? SM::POS_LANES : 0;
+      const bool ts_wave = TS && (!POS || w == NWAVES - 1);
+      const int tl = lane - TS_LANE0;
+      uint32_t off = 0;
+      bool on = false;
+      if (POS && lane < SM::POS_LANES) {
+        off = pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (q0 + BM - 1) + w + 4 * lane) * 4u;
+        on = true;
       }
-    }
-    if (TS) {
-      // BN int64 = 2*BN dwords, one per lane (every wave repeats this load so that all issue
-      // the same number, which the vmcnt arithmetic relies on)
-      int jk = kv0 + (lane >> 1);
-      jk = jk < s.n_ts ? jk : s.n_ts - 1;
-      jk = jk < 0 ? 0 : jk;
-      lds_dma4(tsg, (uint32_t)(jk * 8 + 4 * (lane & 1)), Tk(st));
+      if (ts_wave && tl >= 0 && tl < SM::TK_LANES) {
+        int tr = t;                                  // tiles past the last timestamp repeat the last tile's range
+        const int tr_last = (s.n_ts - 1) >> 5;
+        tr = tr < tr_last ? tr : tr_last;
+        off = tl < BN / 4 ? rel_off + (uint32_t)(kv0 + 4 * tl) * 4u : rng_off + (uint32_t)tr * 8u;
+        on = true;
+      }
+      if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
     }
   };
 
-  // prologue: three steps in flight before anything else
+  // prologue: the scaled bucket table (64 entries per wave, the last wave repeats the first), then
+  // three steps in flight before anything else
+  if (TS) {
+    const int c = w < 3 ? w : 0;
+    const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
+    lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
+  }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t < nt) dma_step(t);
@@ -529,15 +646,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[ks]));
   }
   int64_t tq = 0;
+  int32_t tq32 = 0;
   if (TS) {
     int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
-    tq = p.ts[s.ts0 + (iq < 0 ? 0 : iq)];
-    asm volatile("" ::"v"(tq));
-    const float* tab = p.ts_tab + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1);
-    for (int e = tid; e < 132; e += MFMA_THREADS) {
-      int c = e <= p.ts_nb ? e : p.ts_nb;
-      TsTab[e] = tab[c > 128 ? 128 : c] * LOG2E;
-    }
+    iq = iq < 0 ? 0 : iq;
+    tq32 = trel[iq];     // meaningless when !ts32, and then unused
+    tq = tsg[iq];
+    asm volatile("" ::"v"(tq), "v"(tq32));
   }
 
   floatx16 o[DVB];
@@ -606,18 +721,46 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
     if (TS) {
-      const int64_t* tk = Tk(st) + 4 * hh;
+      auto bucket_f = [&](float f) {
+        f = __builtin_amdgcn_fmed3f(__builtin_fabsf(f), 1.0f, 1.0e9f);
+        return (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
+      };
+      if (ts32) {
+        const int32_t* tk = Tk(st);
+        const int2 rg = *(const int2*)(tk + BN);
+        // |tq - tk| grows as tk falls: when no key of the tile is later than tq and both ends of
+        // the tile fall in the same bucket, so does everything between
+        const int d_near = tq32 - rg.y, d_far = tq32 - rg.x;
+        const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
+        const bool same = d_near >= 0 && b_near == b_far;
+        if (__builtin_amdgcn_ballot_w64(!same) == 0) {
+          const float add = TsTab[b_near];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+          for (int r = 0; r < 16; ++r) u[r] += add;
+        } else {
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          int64_t dt = tq - tk[8 * g + tt];
-          int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-          int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-          float f = __builtin_fabsf((float)sat);
-          f = __builtin_amdgcn_fmed3f(f, 1.0f, 1.0e9f);
-          int bk = (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
-          u[4 * g + tt] += TsTab[bk];
+          for (int g = 0; g < 4; ++g) {
+            const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
+            u[4 * g + 0] += TsTab[bucket_f((float)(tq32 - kk.x))];
+            u[4 * g + 1] += TsTab[bucket_f((float)(tq32 - kk.y))];
+            u[4 * g + 2] += TsTab[bucket_f((float)(tq32 - kk.z))];
+            u[4 * g + 3] += TsTab[bucket_f((float)(tq32 - kk.w))];
+          }
+        }
+      } else {
+        // time span of the sequence beyond 31 bits: 64-bit differences of timestamps read
+        // straight from memory (rare; correctness over speed)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt) {
+            int j = kbs + 8 * g + 4 * hh + tt;
+            j = j < s.n_ts ? j : s.n_ts - 1;
+            const int64_t dt = tq - tsg[j];
+            const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+            const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+            u[4 * g + tt] += TsTab[bucket_f((float)sat)];
+          }
         }
       }
     }
@@ -758,7 +901,9 @@ Variant pick_variant(const HstuAttnFwdArgs* a) {
   if (a->qk_dtype == HSTU_DTYPE_FP32) return V_GENERAL_F32;
   const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
   const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->window < 0 &&
-                       a->L == a->Lkv && (!a->ts_tab || a->ts_num_buckets <= 128);
+                       a->L == a->Lkv &&
+                       // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
+                       (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
   auto s8 = [](int64_t x) { return (x & 7) == 0; };
   const bool align_ok = aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
                         s8(a->q_stride_t) && s8(a->q_stride_h) && s8(a->k_stride_t) && s8(a->k_stride_h) &&
@@ -772,10 +917,30 @@ Variant pick_variant(const HstuAttnFwdArgs* a) {
   return V_GENERAL_BF16;
 }
 
-// The MFMA kernel reads the relative-position table from a scaled, zero-padded copy.
-size_t workspace_needed(const HstuAttnFwdArgs* a) {
-  if (pick_variant(a) != V_MFMA_BF16 || !a->pos_tab) return 0;
-  return (size_t)a->pos_heads * (size_t)(2 * a->L - 1 + 2 * POS_PAD) * sizeof(float);
+// Workspace of the MFMA kernel: [scaled, padded position table][per-sequence int32-timestamp flag]
+// [int32 timestamps][their (min, max) per key tile], each part a multiple of 256 bytes.
+struct WorkspacePlan {
+  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes;
+  size_t total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes; }
+};
+
+WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
+  WorkspacePlan w = {0, 0, 0, 0, 0};
+  if (pick_variant(a) != V_MFMA_BF16) return w;
+  auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  if (a->pos_tab) w.pos_bytes = up((size_t)a->pos_heads * (size_t)(2 * a->L - 1 + 2 * POS_PAD) * sizeof(float));
+  if (a->ts_tab) {
+    const size_t tiles_per_seq = (size_t)((a->L + BN - 1) / BN);
+    const bool by_token = a->ts_stride_b == 0;
+    const size_t n_ts = by_token ? (size_t)a->total_tokens : (size_t)a->B * (size_t)a->L;
+    const size_t tiles = by_token ? (size_t)(a->total_tokens >> 5) + (size_t)a->B + tiles_per_seq : (size_t)a->B * tiles_per_seq;
+    w.tab_bytes = up((size_t)a->ts_heads * TS_TAB_LEN * sizeof(float));
+    w.ok_bytes = up((size_t)a->B * sizeof(int32_t));
+    // the kernel fetches whole 16-byte pieces: up to 31 timestamps and one range past the end
+    w.rel_bytes = up(n_ts * sizeof(int32_t) + 128);
+    w.range_bytes = up(tiles * 2 * sizeof(int32_t) + 16);
+  }
+  return w;
 }
 
 Params make_params(const HstuAttnFwdArgs* a) {
@@ -865,7 +1030,7 @@ const char* hstu_attn_last_error(void) { return g_err; }
 
 size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args) {
   if (validate(args) != HSTU_OK) return 0;
-  return workspace_needed(args);
+  return plan_workspace(args).total();
 }
 
 const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
@@ -900,27 +1065,37 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
     case V_GENERAL_F32: return launch_general<float>(p, st);
     case V_GENERAL_BF16: return launch_general<bf16_t>(p, st);
     case V_MFMA_BF16: {
-      const size_t ws = workspace_needed(args);
-      if (ws) {
-        if (!args->workspace || args->workspace_bytes < ws)
+      const WorkspacePlan ws = plan_workspace(args);
+      Params q = p;
+      if (ws.total()) {
+        if (!args->workspace || args->workspace_bytes < ws.total())
           return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes needed (see hstu_attn_fwd_workspace_bytes), got %zu",
-                      ws, args->workspace ? args->workspace_bytes : (size_t)0);
-        if (((uintptr_t)args->workspace & 15u) != 0) return fail(HSTU_ERR_WORKSPACE, "workspace must be 16-byte aligned");
-        Params q = p;
-        q.pos_scaled = (const float*)args->workspace;
-        const int len = 2 * p.L - 1;
-        const int total = p.pos_heads * (len + 2 * POS_PAD);
-        hipLaunchKernelGGL(hstu_scale_pos_table, dim3((total + 255) / 256 < 1024 ? (total + 255) / 256 : 1024), dim3(256), 0, st,
-                           p.pos_tab, (float*)args->workspace, p.pos_heads, len);
+                      ws.total(), args->workspace ? args->workspace_bytes : (size_t)0);
+        if (((uintptr_t)args->workspace & 255u) != 0) return fail(HSTU_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+        char* base = (char*)args->workspace;
+        if (ws.total() >= (1ull << 32)) return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes is beyond what the kernel addresses", ws.total());
+        float* pos_out = ws.pos_bytes ? (float*)base : nullptr;
+        float* tab_out = ws.tab_bytes ? (float*)(base + ws.pos_bytes) : nullptr;
+        int32_t* ok_out = ws.ok_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes) : nullptr;
+        int32_t* rel_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes);
+        int32_t* range_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes);
+        q.ws_base = base;
+        q.ts_scaled = tab_out;
+        q.pos_scaled = pos_out;
+        q.ts_ok = ok_out;
+        q.ts_rel = rel_out;
+        q.ts_range = range_out;
+        const long long blocks_pos = ws.pos_bytes ? ((long long)p.pos_heads * (2 * p.L - 1 + 2 * POS_PAD) + 255) / 256 : 0;
+        const long long blocks_ts = ws.ok_bytes ? p.B : 0;
+        long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
+        blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+        hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, p, pos_out, tab_out, ok_out, rel_out, range_out);
         hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "table kernel launch: %s", hipGetErrorString(e));
-        if (q.d_qk == 128) return launch_mfma_d<128>(q, st);
-        if (q.d_qk == 64) return launch_mfma_d<64>(q, st);
-        return launch_mfma_d<32>(q, st);
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
       }
-      if (p.d_qk == 128) return launch_mfma_d<128>(p, st);
-      if (p.d_qk == 64) return launch_mfma_d<64>(p, st);
-      return launch_mfma_d<32>(p, st);
+      if (q.d_qk == 128) return launch_mfma_d<128>(q, st);
+      if (q.d_qk == 64) return launch_mfma_d<64>(q, st);
+      return launch_mfma_d<32>(q, st);
     }
     default: return fail(HSTU_ERR_SHAPE, "no kernel for these arguments");
   }

@@ -341,6 +341,37 @@ def test_timestamp_buckets_on_gpu(gpu):
       assert (near_ok <= (1e-2 if dt_ == torch.bfloat16 else 1e-5)).all()
 
 
+def test_timestamp_spans_sorted_unsorted_and_huge(gpu):
+  # sequences whose time span fits 31 bits (sorted and shuffled) next to ones whose span does not:
+  # each goes down a different timestamp path of the bf16 kernel, all must match the oracle
+  rng = np.random.default_rng(41)
+  B, L, H, d = 6, 300, 2, 64
+  lens = np.array([300, 257, 96, 300, 33, 180], dtype=np.int32)
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.2) for _ in range(3))
+  ts = 1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, (B, L))), axis=1).astype(np.int64)
+  ts[1] = rng.permutation(ts[1])                       # unsorted: keys later than the query exist
+  ts[2] = -5_000_000_000 + ts[2] * 40                  # span of 96 * 3600 * 40 < 2^31, negative origin
+  ts[3, 150:] += 3_000_000_000                         # span > 2^31
+  ts[4] = rng.integers(-2**40, 2**40, L)               # huge, unsorted
+  ts[5] = ts[5, 0]                                     # all equal
+  tab = (rng.standard_normal((H, 129)) * 0.5).astype(np.float32)
+  pos = (rng.standard_normal((2 * L - 1,)) * 0.1).astype(np.float32)
+  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, pos_tab=pos, timestamps=ts, ts_tab=tab, dtype=np.float32)
+  out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
+                                 seq_lens=_dev(lens), pos_bias=_dev(pos), timestamps=_dev(ts), ts_bias=_dev(tab))
+  assert _err(out.float().cpu().numpy(), ref) <= BF16_TOL
+  qj, off = O.padded_to_jagged(q, lens)
+  kj, _ = O.padded_to_jagged(k, lens)
+  vj, _ = O.padded_to_jagged(v, lens)
+  tsj = np.concatenate([ts[b, :lens[b]] for b in range(B)])
+  # jagged timestamps end at the sequence: the last row's "next" timestamp is its own
+  refj = O.hstu_attention_jagged_ref(qj, kj, vj, off, L, pos_tab=pos, timestamps=tsj, ts_tab=tab, dtype=np.float32)
+  outj = recml_amd.hstu_attention(_dev(qj, torch.bfloat16), _dev(kj, torch.bfloat16), _dev(vj, torch.bfloat16),
+                                  seq_offsets=_dev(off.astype(np.int32)), max_len=L, pos_bias=_dev(pos),
+                                  timestamps=_dev(tsj), ts_bias=_dev(tab))
+  assert _err(outj.float().cpu().numpy(), refj) <= BF16_TOL
+
+
 def test_argument_errors(gpu):
   z = torch.zeros((2, 8, 2, 32), device="cuda:0")
   seg = torch.ones((2, 8), dtype=torch.int32, device="cuda:0")

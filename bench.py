@@ -26,6 +26,7 @@ if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 
@@ -54,15 +55,27 @@ def make_workload(name):
     return workloads.config4_attention()
   if name == "c5":
     return workloads.config5()
+  if name == "c5-bf16":
+    return workloads.config5(fp8=False)
   raise SystemExit(f"unknown workload {name}")
 
 
 def to_device(w, dev):
   import torch
   t = lambda x: None if x is None else torch.from_numpy(np.ascontiguousarray(x)).to(dev)
-  q, k, v = (t(x).to(torch.bfloat16) for x in (w.q, w.k, w.v))
+  q, k, v = (t(x) for x in (w.q, w.k, w.v))
   kw = dict(n=w.n, alpha=w.alpha, pos_bias=t(w.pos_tab), ts_bias=t(w.ts_tab),
             timestamps=t(w.timestamps))
+  if w.dtype == "fp8":
+    # per-head symmetric quantisation of q and k: scale = amax / 448
+    def quant(x):
+      scale = x.abs().amax(dim=tuple(i for i in range(x.dim()) if i != x.dim() - 2)).clamp_min(1e-30) / 448.0
+      return (x / scale[:, None]).to(torch.float8_e4m3fn), scale
+    (q, qs), (k, ks) = quant(q), quant(k)
+    kw.update(q_scale=qs, k_scale=ks)
+    v = v.to(torch.bfloat16)
+  else:
+    q, k, v = (x.to(torch.bfloat16) for x in (q, k, v))
   if w.layout == "jagged":
     kw.update(seq_offsets=t(w.seq_offsets), max_len=w.L)
   else:
@@ -70,12 +83,15 @@ def to_device(w, dev):
   return q, k, v, kw
 
 
-def cpu_baseline(w, q, k, v, out_gpu):
+def cpu_baseline(w, q, k, v, out_gpu, dev_kw):
   """The C restatement of the op (oracle/hstu_oracle.c, float accumulation,
   OpenMP over sequence x head) timed on this host, and used as the checker."""
   from oracle import c_oracle
   threads = c_oracle.max_threads()
   qf, kf, vf = (x.float().cpu().numpy() for x in (q, k, v))
+  if w.dtype == "fp8":   # the checker works on the dequantised inputs the kernel sees
+    qf = qf * dev_kw["q_scale"].cpu().numpy()[:, None]
+    kf = kf * dev_kw["k_scale"].cpu().numpy()[:, None]
   kw = dict(n=w.n, alpha=w.alpha, pos_tab=w.pos_tab, timestamps=w.timestamps,
             ts_tab=w.ts_tab, acc="f32")
   if w.layout == "jagged":
@@ -135,7 +151,7 @@ def main():
   dev = torch.device("cuda:0")
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
-  out = torch.empty_like(q)
+  out = torch.empty_like(v)
   call_args, keep = hstu_ops.build_args(q, k, v, out, **kw)
   variant = hstu_ops.kernel_variant(call_args)
 
@@ -172,16 +188,18 @@ def main():
   flops = w.flops
   tflops = flops / (ms_per_step * 1e-3) / 1e12
   achieved = flops / (kernel_ms * 1e-3) / 1e12
-  bytes_alg = w.bytes_moved(2)
+  bytes_alg = w.bytes_moved(2, 1 if w.dtype == "fp8" else None)
   ai = flops / bytes_alg
-  capped_peak = min(PEAK_BF16_TFLOPS, ai * PEAK_HBM_GBS / 1e3)
+  # fp8 q/k: half of the flops (q k^T) run at the fp8 rate, half (P V) at the bf16 rate
+  peak = PEAK_BF16_TFLOPS if w.dtype != "fp8" else 1.0 / (0.5 / PEAK_FP8_TFLOPS + 0.5 / PEAK_BF16_TFLOPS)
+  capped_peak = min(peak, ai * PEAK_HBM_GBS / 1e3)
 
   rec = {
       "metric": "HSTU attn fwd TFLOP/s (unmasked), L=%d bf16" % w.L,
       "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
       "warmup": args.warmup, "ms_per_step": ms_per_step,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-      "dtype": "bf16", "data": "synthetic",
+      "dtype": "fp8 q/k, bf16 v/out" if w.dtype == "fp8" else "bf16", "data": "synthetic",
       "config": {"workload": f"{w.name}: B={w.B} max_len={w.L} H={w.H} d={w.d} {w.layout} "
                              f"lens mean {w.seq_lens.mean():.0f} max {w.seq_lens.max()}, causal, "
                              f"pos_bias={'yes' if w.pos_tab is not None else 'no'} "
@@ -189,8 +207,8 @@ def main():
                  "kernel": variant},
       "seqs_per_s": w.B / (ms_per_step * 1e-3),
       "roofline": {
-          "bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
-          "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": measured_traffic(args.workload),
+          "bound": "mfma", "achieved": achieved, "peak": peak,
+          "unit": "TFLOP/s", "frac": achieved / peak, "traffic": measured_traffic(args.workload),
           "kernel_ms_avg": kernel_ms, "kernel_ms_min": float(ev_ms.min()),
           "kernel_ms_median": float(np.median(ev_ms)),
           "region_ms_per_step": region_ms / args.steps,
@@ -202,7 +220,7 @@ def main():
       },
   }
   if not args.no_cpu:
-    base, err = cpu_baseline(w, q, k, v, out.float().cpu().numpy())
+    base, err = cpu_baseline(w, q, k, v, out.float().cpu().numpy(), kw)
     rec["cpu_baseline"] = base
     rec["parity_max_abs_over_max_ref"] = err
     if not err <= 2e-2:

@@ -32,6 +32,9 @@ How each function is pinned (tests/test_oracle.py):
                                 single-key closed form, the zero-Q Toeplitz
                                 case, SiLU special values, causality and
                                 padding invariants, linearity in 1/N.
+  round_e4m3fn / encode_e4m3fn  torch's CPU float8_e4m3fn cast on every code
+                                point, every midpoint and random values (fp8
+                                is not in the reference at all).
   splash_mask with sliding_window_size  parity unpinned: the window rule
                                 (|i-j| <= w) comes from jax's splash-attention
                                 LocalMask, which is not vendored in the
@@ -405,6 +408,55 @@ def round_bf16(x):
   u = a.view(np.uint32).astype(np.uint64)
   r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
   return r.astype(np.uint32).view(np.float32).reshape(a.shape)
+
+
+E4M3FN_MAX = 448.0
+
+
+def round_e4m3fn(x):
+  """Round to the nearest float8 e4m3fn value (ties to even, saturating at
+  +-448) and return it as fp32.
+
+  The format (OCP 8-bit floating point, "fn" = finite + NaN, no infinities):
+  1 sign, 4 exponent bits with bias 7, 3 mantissa bits; normal values
+  2^e * (1 + m/8) for e in -6..8 (e = 8 only up to m = 6, i.e. 448),
+  subnormals m * 2^-9.  Not part of the reference (its README lists fp8 as
+  roadmap only); pinned against torch's CPU float8_e4m3fn cast.
+  """
+  a = np.asarray(x, dtype=np.float64)
+  mag = np.minimum(np.abs(a), E4M3FN_MAX)
+  # exponent of the value, clamped to the subnormal range
+  e = np.floor(np.log2(np.maximum(mag, 2.0 ** -20)))
+  e = np.clip(e, -6, 8)
+  step = 2.0 ** (e - 3)                       # spacing of representable values in [2^e, 2^(e+1))
+  r = np.round(mag / step) * step             # np.round is ties-to-even
+  r = np.minimum(r, E4M3FN_MAX)
+  return (np.sign(a) * r).astype(np.float32)
+
+
+def encode_e4m3fn(x):
+  """uint8 bit patterns of values that are already exactly representable."""
+  a = np.asarray(x, dtype=np.float64)
+  sign = (np.signbit(a)).astype(np.uint8) << 7
+  mag = np.abs(a)
+  e = np.floor(np.log2(np.maximum(mag, 2.0 ** -20)))
+  normal = mag >= 2.0 ** -6
+  e = np.clip(e, -6, 8)
+  m_norm = np.round((mag / 2.0 ** e - 1.0) * 8).astype(np.int64)
+  m_sub = np.round(mag / 2.0 ** -9).astype(np.int64)
+  code = np.where(normal, ((e + 7).astype(np.int64) << 3) | m_norm, m_sub)
+  return (sign | code.astype(np.uint8)).astype(np.uint8)
+
+
+def quantize_e4m3fn_per_head(x):
+  """Per-head symmetric quantisation of [..., H, d]: scale[h] = amax_h / 448,
+  returns (x / scale rounded to e4m3fn, as fp32; scale [H] fp32)."""
+  a = np.asarray(x, dtype=np.float32)
+  H = a.shape[-2]
+  amax = np.abs(a).reshape(-1, H, a.shape[-1]).max(axis=(0, 2))
+  scale = (np.maximum(amax, 1e-30) / E4M3FN_MAX).astype(np.float32)
+  q = round_e4m3fn(a / scale[:, None])
+  return q, scale
 
 
 def padded_to_jagged(x, seq_lens):

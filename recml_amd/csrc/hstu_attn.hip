@@ -68,6 +68,8 @@ struct Params {
   const int32_t* ts_range;
   const float* ts_scaled;    // workspace: log2(e) * ts_tab as [heads][TS_TAB_LEN], indices past the last bucket repeat it
   const void* ws_base;       // start of the workspace (all of the above lie within 4 GB of it)
+  const float* q_scale;      // [H] or null: dequantisation scales of fp8 q / k
+  const float* k_scale;
   int64_t ts_sb;
   int32_t B, L, Lkv, H, d_qk, d_v;
   int32_t jagged, causal, mask_mode, window;
@@ -307,15 +309,17 @@ constexpr int POS_PAD = 256;  // zero margin on both sides of the scaled positio
 constexpr int TS_TAB_LEN = 192;  // entries of the scaled bucket table (3 waves x 64 lanes of one direct load)
 constexpr float LOG2E = 1.4426950408889634f;
 
-template <int D>
+template <int D, int KB>   // KB: bytes per q / k element (2 = bf16, 1 = fp8)
 struct MfmaSmem {
-  // K and V tiles are stored unpadded ([64 keys][D] bf16) because they arrive
-  // by direct global->LDS loads, which write 64 lanes x 16 bytes contiguously.
-  // Bank conflicts are avoided by XOR-swizzling the 16-byte chunk index of a
-  // row instead (different functions for K and V, matched to how each is read).
-  static constexpr int CPR = D / 8;                 // 16-byte chunks per row
-  static constexpr int RPB = CPR >= 16 ? 1 : 16 / CPR;  // rows per 256 bytes (one sweep of the banks)
-  static constexpr int K_BYTES = BN * D * 2;
+  // K and V tiles are stored unpadded ([32 keys][D]) because they arrive by direct
+  // global->LDS loads, which write 64 lanes x 16 bytes contiguously.  Bank conflicts
+  // are avoided by XOR-swizzling the 16-byte chunk index of a row instead (different
+  // functions for K and V, matched to how each is read).
+  static constexpr int CPR = D / 8;                       // 16-byte chunks per V row
+  static constexpr int RPB = CPR >= 16 ? 1 : 16 / CPR;    // V rows per 256 bytes (one sweep of the banks)
+  static constexpr int KCPR = D * KB / 16;                // the same for K
+  static constexpr int KRPB = KCPR >= 16 ? 1 : 16 / KCPR;
+  static constexpr int K_BYTES = BN * D * KB;
   static constexpr int V_BYTES = BN * D * 2;
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int POS_LANES = (BM + BN - 1 + 3 + 3) / 4;   // 16-byte pieces of one window copy
@@ -329,7 +333,7 @@ struct MfmaSmem {
     return NSTAGE * (STAGE + bias_stage(pos, ts)) + (ts ? TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
-  __device__ static constexpr int swz_k(int row) { return (row / RPB) % CPR; }
+  __device__ static constexpr int swz_k(int row) { return (row / KRPB) % KCPR; }
   // V is read 4 rows x 64 bytes per half-wave: the 4 rows must land in 4 different 64-byte groups
   __device__ static constexpr int swz_v(int row) { return (4 * ((row / RPB) & 3)) % CPR; }
 };
@@ -478,17 +482,21 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
   }
 }
 
-template <int D, bool POS, bool TS>
+template <int D, bool POS, bool TS, bool F8>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
-  using SM = MfmaSmem<D>;
+  constexpr int KB = F8 ? 1 : 2;       // bytes per q / k element
+  using SM = MfmaSmem<D, KB>;
   constexpr int CPR = SM::CPR;
+  constexpr int KCPR = SM::KCPR;
   constexpr int KSTEPS = D / 16;       // MFMA k-steps over the head dim
+  constexpr int QCH = D * KB / 32;     // 16-byte chunks of a q (or k) row per lane: chunk 2j + hh, j < QCH
   constexpr int DVB = D / 32;          // 32-row blocks of O^T
-  constexpr int CH = BN * D / 8;       // 16-byte chunks in a K (or V) tile
-  constexpr int NPIECE = CH / 64;      // 1 KB pieces (one wave-wide direct load each) in a tile
-  constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;  // direct loads per wave per tile and tensor
-  static_assert(CH % 64 == 0, "tile must be a whole number of 1 KB pieces");
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);   // direct loads per wave per step
+  // 1 KB pieces (one wave-wide direct load each) in a K and in a V tile, and direct loads per wave per tile
+  constexpr int NPIECE_K = SM::K_BYTES / 1024, NPIECE = SM::V_BYTES / 1024;
+  constexpr int LDK = NPIECE_K >= NWAVES ? NPIECE_K / NWAVES : 1;
+  constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
+  static_assert(SM::K_BYTES % 1024 == 0 && SM::V_BYTES % 1024 == 0, "tile must be a whole number of 1 KB pieces");
+  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0);   // direct loads per wave per step
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -523,7 +531,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept scalar
   const int m = lane & 31, hh = lane >> 5;
-  const bf16_t* __restrict__ kg = (const bf16_t*)p.k + s.bk;
+  const char* __restrict__ kg = (const char*)p.k + s.bk * KB;
   const bf16_t* __restrict__ vg = (const bf16_t*)p.v + s.bv;
   bf16_t* __restrict__ og = (bf16_t*)p.out + s.bo;
 
@@ -551,8 +559,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // last key this wave needs
   const int wave_last = !wave_live ? -1 : (p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1));
 
-  const float alpha2 = p.alpha * LOG2E;
-  const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
+  // fp8 q and k carry per-head dequantisation scales: they multiply the logits
+  const float alpha2 = p.alpha * LOG2E * (F8 && p.q_scale ? p.q_scale[h] : 1.0f) * (F8 && p.k_scale ? p.k_scale[h] : 1.0f);
+  const uint32_t kst_bytes = (uint32_t)p.k_st * (uint32_t)KB, vst_bytes = (uint32_t)p.v_st * 2u;
   // Bias operands are fetched with 32-bit byte offsets from the start of the workspace.
   // pos_off: this head's padded table; entry x of the unpadded table sits at float POS_PAD + x.
   const char* wsb = (const char*)p.ws_base;
@@ -579,15 +588,23 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     const int kv0 = t * BN;
     const int last = s.n_kv - 1;
 #pragma unroll
+    for (int r = 0; r < LDK; ++r) {
+      const int j = (w * LDK + r) % NPIECE_K;   // small tiles: several waves repeat the same piece
+      const int c = 64 * j + lane;
+      const int row = c / KCPR, pc = c - row * KCPR;
+      int grow = kv0 + row;
+      grow = grow < last ? grow : last;
+      const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
+      lds_dma16(kg, koff, (const unsigned char*)Ks(st) + j * 1024);
+    }
+#pragma unroll
     for (int r = 0; r < LD; ++r) {
-      const int j = (w * LD + r) % NPIECE;   // small tiles: two waves repeat the same piece
+      const int j = (w * LD + r) % NPIECE;
       const int c = 64 * j + lane;
       const int row = c / CPR, pc = c - row * CPR;
       int grow = kv0 + row;
       grow = grow < last ? grow : last;
-      const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
       const uint32_t voff = (uint32_t)grow * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
-      lds_dma16(kg, koff, Ks(st) + j * 512);
       lds_dma16(vg, voff, Vs(st) + j * 512);
     }
     if (POS || TS) {
@@ -629,21 +646,24 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t < nt) dma_step(t);
 
-  // Q fragments (B operand of S^T = K Q^T): lane holds q[qrow][16ks+8hh .. +7]
-  bf16x8 qf[KSTEPS];
+  // Q fragments (B operand of S^T = K Q^T).  bf16: k-step ks of lane (row, hh) holds
+  // q[qrow][16ks+8hh .. +7], i.e. 16-byte chunk 2ks+hh of the row.  fp8: the lane holds chunks
+  // 2j+hh of the row, each feeding two k-steps (its low and its high 8 bytes); K is read the
+  // same way, and the order of the terms of a dot product is free.
+  uint4 qf[QCH];
   {
-    const bf16_t* qg = (const bf16_t*)p.q + s.bq + (int64_t)qrow * p.q_st + 8 * hh;
+    const char* qg = (const char*)p.q + (s.bq + (int64_t)qrow * p.q_st) * KB + 16 * hh;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
+    for (int ks = 0; ks < QCH; ++ks) {
       uint4 t4 = {0u, 0u, 0u, 0u};
-      if (qrow < s.n_q) t4 = *(const uint4*)(qg + 16 * ks);
-      qf[ks] = __builtin_bit_cast(bf16x8, t4);
+      if (qrow < s.n_q) t4 = *(const uint4*)(qg + 32 * ks);
+      qf[ks] = t4;
     }
     // Use the fragments here so that the compiler's wait for these loads sits in the prologue.
     // Left to the first use inside the loop it would be a vmcnt(0) on every step, which also
     // waits for every direct load in flight and serialises the whole ring.
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) asm volatile("" ::"v"(qf[ks]));
+    for (int ks = 0; ks < QCH; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].y), "v"(qf[ks].z), "v"(qf[ks].w));
   }
   int64_t tq = 0;
   int32_t tq32 = 0;
@@ -679,14 +699,25 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     const int kbs = t * BN;
     floatx16 sacc;
     {
-      bf16x8 kf[KSTEPS];
-      const bf16_t* kr = Ks(st) + m * D;
+      uint4 kf[QCH];
+      const unsigned char* kr = (const unsigned char*)Ks(st) + m * (D * KB);
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks) kf[ks] = *(const bf16x8*)(kr + (((2 * ks + hh) ^ gk) * 8));
+      for (int ks = 0; ks < QCH; ++ks) kf[ks] = *(const uint4*)(kr + (((2 * ks + hh) ^ gk) * 16));
       const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (F8) {
 #pragma unroll
-      for (int ks = 0; ks < KSTEPS; ++ks)
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], ks == 0 ? zero : sacc, 0, 0, 0);
+        for (int ks = 0; ks < QCH; ++ks) {
+          const long ka = (long)(((uint64_t)kf[ks].y << 32) | kf[ks].x), kb = (long)(((uint64_t)kf[ks].w << 32) | kf[ks].z);
+          const long qa = (long)(((uint64_t)qf[ks].y << 32) | qf[ks].x), qb = (long)(((uint64_t)qf[ks].w << 32) | qf[ks].z);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(ka, qa, ks == 0 ? zero : sacc, 0, 0, 0);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(kb, qb, sacc, 0, 0, 0);
+        }
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < QCH; ++ks)
+          sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]), __builtin_bit_cast(bf16x8, qf[ks]),
+                                                         ks == 0 ? zero : sacc, 0, 0, 0);
+      }
     }
     // V fragments, requested now so that they arrive while the SiLU runs
     uint4 vf[2][DVB];
@@ -846,9 +877,30 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-enum Variant { V_INVALID = 0, V_GENERAL_F32, V_GENERAL_BF16, V_MFMA_BF16 };
+enum Variant { V_INVALID = 0, V_GENERAL_F32, V_GENERAL_BF16, V_MFMA_BF16, V_MFMA_FP8 };
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// Whether the matrix-core kernel covers these arguments (dtype aside: bf16, or fp8 q/k).
+bool mfma_eligible(const HstuAttnFwdArgs* a) {
+  const int kb = a->qk_dtype == HSTU_DTYPE_FP8_E4M3FN ? 1 : 2;   // bytes per q / k element
+  const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
+  const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->window < 0 &&
+                       a->L == a->Lkv &&
+                       // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
+                       (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
+  auto s8 = [](int64_t x) { return (x & 7) == 0; };
+  auto sq = [kb](int64_t x) { return (x * kb & 15) == 0; };
+  const bool align_ok = aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
+                        sq(a->q_stride_t) && sq(a->q_stride_h) && sq(a->k_stride_t) && sq(a->k_stride_h) &&
+                        s8(a->v_stride_t) && s8(a->v_stride_h) && s8(a->o_stride_t) && s8(a->o_stride_h) &&
+                        (a->layout == HSTU_LAYOUT_JAGGED ||
+                         (sq(a->q_stride_b) && sq(a->k_stride_b) && s8(a->v_stride_b) && s8(a->o_stride_b)));
+  // the kernel addresses K and V rows with 32-bit byte offsets from the (sequence, head) base
+  const bool off_ok = (int64_t)a->L * a->k_stride_t * kb < (1LL << 31) && (int64_t)a->L * a->v_stride_t * 2 < (1LL << 31) &&
+                      a->k_stride_t > 0 && a->v_stride_t > 0;
+  return d_ok && opts_ok && align_ok && off_ok;
+}
 
 int validate(const HstuAttnFwdArgs* a) {
   if (!a) return fail(HSTU_ERR_NULL, "args is null");
@@ -868,8 +920,9 @@ int validate(const HstuAttnFwdArgs* a) {
     return fail(HSTU_ERR_SHAPE, "unknown mask_mode %d", a->mask_mode);
   const bool f32 = a->qk_dtype == HSTU_DTYPE_FP32 && a->v_dtype == HSTU_DTYPE_FP32 && a->out_dtype == HSTU_DTYPE_FP32;
   const bool b16 = a->qk_dtype == HSTU_DTYPE_BF16 && a->v_dtype == HSTU_DTYPE_BF16 && a->out_dtype == HSTU_DTYPE_BF16;
-  if (!f32 && !b16)
-    return fail(HSTU_ERR_DTYPE, "unsupported dtype combination qk=%d v=%d out=%d (all fp32 or all bf16)",
+  const bool f8 = a->qk_dtype == HSTU_DTYPE_FP8_E4M3FN && a->v_dtype == HSTU_DTYPE_BF16 && a->out_dtype == HSTU_DTYPE_BF16;
+  if (!f32 && !b16 && !f8)
+    return fail(HSTU_ERR_DTYPE, "unsupported dtype combination qk=%d v=%d out=%d (all fp32, all bf16, or fp8 q/k with bf16 v/out)",
                 a->qk_dtype, a->v_dtype, a->out_dtype);
   if (a->layout == HSTU_LAYOUT_JAGGED) {
     if (!a->seq_offsets) return fail(HSTU_ERR_NULL, "jagged layout needs seq_offsets");
@@ -894,26 +947,15 @@ int validate(const HstuAttnFwdArgs* a) {
     if (a->ts_stride_b == 0 && a->layout != HSTU_LAYOUT_JAGGED)
       return fail(HSTU_ERR_SHAPE, "jagged timestamps need the jagged layout");
   }
+  if (f8 && !mfma_eligible(a))
+    return fail(HSTU_ERR_DTYPE, "fp8 q/k runs on the matrix-core kernel only: d_qk == d_v in {32, 64, 128}, q_len == kv_len, "
+                "16-byte aligned pointers and row strides, no segment ids, explicit mask, dense bias or window");
   return HSTU_OK;
 }
 
 Variant pick_variant(const HstuAttnFwdArgs* a) {
   if (a->qk_dtype == HSTU_DTYPE_FP32) return V_GENERAL_F32;
-  const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
-  const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->window < 0 &&
-                       a->L == a->Lkv &&
-                       // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
-                       (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
-  auto s8 = [](int64_t x) { return (x & 7) == 0; };
-  const bool align_ok = aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
-                        s8(a->q_stride_t) && s8(a->q_stride_h) && s8(a->k_stride_t) && s8(a->k_stride_h) &&
-                        s8(a->v_stride_t) && s8(a->v_stride_h) && s8(a->o_stride_t) && s8(a->o_stride_h) &&
-                        (a->layout == HSTU_LAYOUT_JAGGED ||
-                         (s8(a->q_stride_b) && s8(a->k_stride_b) && s8(a->v_stride_b) && s8(a->o_stride_b)));
-  // the MFMA kernel addresses K and V rows with 32-bit byte offsets from the (sequence, head) base
-  const bool off_ok = (int64_t)a->L * a->k_stride_t * 2 < (1LL << 31) && (int64_t)a->L * a->v_stride_t * 2 < (1LL << 31) &&
-                      a->k_stride_t > 0 && a->v_stride_t > 0;
-  if (d_ok && opts_ok && align_ok && off_ok) return V_MFMA_BF16;
+  if (mfma_eligible(a)) return a->qk_dtype == HSTU_DTYPE_FP8_E4M3FN ? V_MFMA_FP8 : V_MFMA_BF16;
   return V_GENERAL_BF16;
 }
 
@@ -926,7 +968,8 @@ struct WorkspacePlan {
 
 WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
   WorkspacePlan w = {0, 0, 0, 0, 0};
-  if (pick_variant(a) != V_MFMA_BF16) return w;
+  const Variant var = pick_variant(a);
+  if (var != V_MFMA_BF16 && var != V_MFMA_FP8) return w;
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
   if (a->pos_tab) w.pos_bytes = up((size_t)a->pos_heads * (size_t)(2 * a->L - 1 + 2 * POS_PAD) * sizeof(float));
   if (a->ts_tab) {
@@ -966,6 +1009,7 @@ Params make_params(const HstuAttnFwdArgs* a) {
   p.ts_bucket_size = a->ts_bucket_size;
   p.ts_log2_scale = a->ts_tab ? (float)(0.6931471805599453 / (double)a->ts_bucket_size) : 0.f;
   p.alpha = a->alpha; p.inv_n = a->inv_n;
+  p.q_scale = a->q_scale; p.k_scale = a->k_scale;
   p.n_qtiles = (a->L + BM - 1) / BM;
   return p;
 }
@@ -997,27 +1041,34 @@ int launch_general(const Params& p, hipStream_t st) {
   return HSTU_OK;
 }
 
-template <int D, bool POS, bool TS>
+template <int D, bool POS, bool TS, bool F8>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D>::total(POS, TS);
+  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS);
   static int granted[64];
-  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS>, smem, granted)) return rc;
+  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8>, smem, granted)) return rc;
   hipError_t e;
   const long long blocks = 8LL * p.n_qtiles * (((long long)p.B * p.H + 7) / 8);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "mfma kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
 }
 
-template <int D>
+template <int D, bool F8>
 int launch_mfma_d(const Params& p, hipStream_t st) {
   const bool pos = p.pos_tab != nullptr, ts = p.ts_tab != nullptr;
-  if (pos && ts) return launch_mfma_inst<D, true, true>(p, st);
-  if (pos) return launch_mfma_inst<D, true, false>(p, st);
-  if (ts) return launch_mfma_inst<D, false, true>(p, st);
-  return launch_mfma_inst<D, false, false>(p, st);
+  if (pos && ts) return launch_mfma_inst<D, true, true, F8>(p, st);
+  if (pos) return launch_mfma_inst<D, true, false, F8>(p, st);
+  if (ts) return launch_mfma_inst<D, false, true, F8>(p, st);
+  return launch_mfma_inst<D, false, false, F8>(p, st);
+}
+
+template <bool F8>
+int launch_mfma(const Params& p, hipStream_t st) {
+  if (p.d_qk == 128) return launch_mfma_d<128, F8>(p, st);
+  if (p.d_qk == 64) return launch_mfma_d<64, F8>(p, st);
+  return launch_mfma_d<32, F8>(p, st);
 }
 
 }  // namespace
@@ -1039,6 +1090,7 @@ const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
     case V_GENERAL_F32: return "hstu_fwd_general<float>";
     case V_GENERAL_BF16: return "hstu_fwd_general<bf16>";
     case V_MFMA_BF16: return "hstu_fwd_mfma_bf16";
+    case V_MFMA_FP8: return "hstu_fwd_mfma_fp8";
     default: return "invalid";
   }
 }
@@ -1047,7 +1099,7 @@ const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
 int hstu_attn_debug_occupancy(int d, int pos, int ts) {
   int n = -1;
   hipError_t e = hipErrorInvalidValue;
-#define OCC(D_, P_, T_) if (d == D_ && !!pos == P_ && !!ts == T_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)hstu_fwd_mfma_bf16<D_, P_, T_>, MFMA_THREADS, MfmaSmem<D_>::total(P_, T_));
+#define OCC(D_, P_, T_) if (d == D_ && !!pos == P_ && !!ts == T_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)hstu_fwd_mfma_bf16<D_, P_, T_, false>, MFMA_THREADS, MfmaSmem<D_, 2>::total(P_, T_));
   OCC(128, false, false) OCC(128, true, false) OCC(128, false, true) OCC(128, true, true)
   OCC(64, false, false) OCC(64, true, true) OCC(32, false, false) OCC(32, true, true)
 #undef OCC
@@ -1064,7 +1116,9 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
   switch (pick_variant(args)) {
     case V_GENERAL_F32: return launch_general<float>(p, st);
     case V_GENERAL_BF16: return launch_general<bf16_t>(p, st);
-    case V_MFMA_BF16: {
+    case V_MFMA_BF16:
+    case V_MFMA_FP8: {
+      const bool f8 = args->qk_dtype == HSTU_DTYPE_FP8_E4M3FN;
       const WorkspacePlan ws = plan_workspace(args);
       Params q = p;
       if (ws.total()) {
@@ -1093,9 +1147,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
       }
-      if (q.d_qk == 128) return launch_mfma_d<128>(q, st);
-      if (q.d_qk == 64) return launch_mfma_d<64>(q, st);
-      return launch_mfma_d<32>(q, st);
+      return f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st);
     }
     default: return fail(HSTU_ERR_SHAPE, "no kernel for these arguments");
   }

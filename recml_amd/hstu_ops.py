@@ -35,7 +35,8 @@ class MaskType(str, enum.Enum):
   FULL = "full"
 
 
-_DTYPES = {torch.float32: _lib.DTYPE_FP32, torch.bfloat16: _lib.DTYPE_BF16}
+_DTYPES = {torch.float32: _lib.DTYPE_FP32, torch.bfloat16: _lib.DTYPE_BF16,
+           torch.float8_e4m3fn: _lib.DTYPE_FP8_E4M3FN}
 
 
 def _ptr(t):
@@ -95,14 +96,21 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
                n=None, alpha=1.0, inv_n=None, causal=True, pos_bias=None,
                timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                q_segment_ids=None, kv_segment_ids=None,
-               sliding_window_size=None, mask=None, bias=None):
+               sliding_window_size=None, mask=None, bias=None,
+               q_scale=None, k_scale=None):
   """Validates the call and fills an HstuAttnFwdArgs.  Returns (args, keepalive)."""
   for name, t in (("q", q), ("k", k), ("v", v)):
     _check_gpu(name, t)
   if q.dtype not in _DTYPES:
-    raise ValueError(f"unsupported dtype {q.dtype}: use float32 or bfloat16")
-  if k.dtype != q.dtype or v.dtype != q.dtype:
+    raise ValueError(f"unsupported dtype {q.dtype}: use float32, bfloat16 or float8_e4m3fn (q and k)")
+  fp8 = q.dtype == torch.float8_e4m3fn
+  if fp8:
+    if k.dtype != q.dtype or v.dtype != torch.bfloat16:
+      raise ValueError(f"float8_e4m3fn q needs float8_e4m3fn k and bfloat16 v, got {k.dtype}, {v.dtype}")
+  elif k.dtype != q.dtype or v.dtype != q.dtype:
     raise ValueError(f"q, k, v must share one dtype, got {q.dtype}, {k.dtype}, {v.dtype}")
+  if not fp8 and (q_scale is not None or k_scale is not None):
+    raise ValueError("q_scale / k_scale belong to float8_e4m3fn q and k")
   keep = [q, k, v, out]
   a = _lib.new_args()
   dev = q.device
@@ -167,15 +175,24 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
       a.mask_mode = _lib.MASK_NONE
   d_v = v.shape[-1]
   exp_out = (q.shape[0], H, d_v) if jagged else (B, L, H, d_v)
-  if tuple(out.shape) != exp_out or out.dtype != q.dtype or not out.is_cuda:
-    raise ValueError(f"out must be a {q.dtype} GPU tensor of shape {exp_out}")
+  if tuple(out.shape) != exp_out or out.dtype != v.dtype or not out.is_cuda:
+    raise ValueError(f"out must be a {v.dtype} GPU tensor of shape {exp_out}")
 
   q, k, v = (_inner_contiguous(t) for t in (q, k, v))
   if out.stride(-1) != 1:
     raise ValueError("out must be contiguous in its last dimension")
   keep += [q, k, v]
   a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
-  a.qk_dtype = a.v_dtype = a.out_dtype = _DTYPES[q.dtype]
+  a.qk_dtype = _DTYPES[q.dtype]
+  a.v_dtype = a.out_dtype = _DTYPES[v.dtype]
+  for name, sc in (("q_scale", q_scale), ("k_scale", k_scale)):
+    if sc is not None:
+      _check_gpu(name, sc)
+      if sc.numel() not in (1, H):
+        raise ValueError(f"{name} must have 1 or {H} entries, got {tuple(sc.shape)}")
+      sc = sc.to(torch.float32).reshape(-1).expand(H).contiguous()
+      keep.append(sc)
+      setattr(a, name, sc.data_ptr())
   for name, t in (("q", q), ("k", k), ("v", v), ("o", out)):
     if jagged:
       sb, st, sh = 0, t.stride(0), t.stride(1)
@@ -258,12 +275,16 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
                    n=None, alpha=1.0, causal=True, pos_bias=None,
                    timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                    q_segment_ids=None, kv_segment_ids=None,
-                   sliding_window_size=None, mask=None, bias=None, out=None):
+                   sliding_window_size=None, mask=None, bias=None, out=None,
+                   q_scale=None, k_scale=None):
   """out = (silu(alpha * q k^T + bias) / n, masked) v.
 
   Args:
     q, k, v: padded [B, L, H, d] or jagged [T, H, d] (with `seq_offsets`
-      [B+1] and `max_len`); float32 or bfloat16 GPU tensors.
+      [B+1] and `max_len`); float32 or bfloat16 GPU tensors, or
+      float8_e4m3fn q and k with bfloat16 v.
+    q_scale, k_scale: per-head (or scalar) dequantisation scales of
+      float8_e4m3fn q and k: the logits are alpha * q_scale * k_scale * q8.k8.
     seq_lens: int [B] valid lengths of an end-padded batch.  Rows and keys at
       or beyond the length are ignored and output rows there are exactly 0,
       as with make_causal_mask (recml/layers/keras/utils.py:39-41).
@@ -286,19 +307,20 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
     out: optional preallocated output.
 
   Returns:
-    Tensor shaped like q with v's head dim, same dtype as q.
+    Tensor shaped like q with v's head dim and v's dtype.
   """
   _check_gpu("q", q)
   _check_gpu("v", v)
   if out is None:
     shape = tuple(q.shape[:-1]) + (v.shape[-1],)
-    out = torch.empty(shape, dtype=q.dtype, device=q.device)
+    out = torch.empty(shape, dtype=v.dtype, device=q.device)
   args, keep = build_args(
       q, k, v, out, seq_lens=seq_lens, seq_offsets=seq_offsets,
       max_len=max_len, n=n, alpha=alpha, causal=causal, pos_bias=pos_bias,
       timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
       q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids,
-      sliding_window_size=sliding_window_size, mask=mask, bias=bias)
+      sliding_window_size=sliding_window_size, mask=mask, bias=bias,
+      q_scale=q_scale, k_scale=k_scale)
   with torch.cuda.device(q.device):
     _run(args, keep)
   return out

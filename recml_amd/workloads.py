@@ -23,7 +23,7 @@ class Workload:
   L: int
   H: int
   d: int
-  dtype: str                     # "fp32" | "bf16"
+  dtype: str                     # "fp32" | "bf16" | "fp8" (q and k float8_e4m3fn with per-head scales, v bf16)
   layout: str                    # "padded" | "jagged"
   seq_lens: np.ndarray           # int32 [B]
   q: np.ndarray                  # padded [B,L,H,d] or jagged [T,H,d], fp32
@@ -41,12 +41,13 @@ class Workload:
     nn = self.seq_lens.astype(np.int64)
     return int((self.H * (nn * (nn + 1) // 2) * 4 * self.d).sum())
 
-  def bytes_moved(self, elem_bytes: int) -> int:
+  def bytes_moved(self, elem_bytes: int, qk_bytes: int | None = None) -> int:
     """Q, K, V read once and O written once over the valid tokens."""
     tokens = int(self.seq_lens.astype(np.int64).sum())
     if self.layout == "padded":
       tokens = self.B * self.L
-    return tokens * self.H * 4 * self.d * elem_bytes
+    qk = elem_bytes if qk_bytes is None else qk_bytes
+    return tokens * self.H * self.d * (2 * qk + 2 * elem_bytes)
 
 
 def power_law_lengths(rng, B, lo, hi, exponent):
@@ -137,14 +138,16 @@ def config4_attention(seed=4, B=128, L=1024, H=8, d=64):
                   pos_tab=pos, seq_offsets=_offsets(lens))
 
 
-def config5(seed=5, B=32, L=4096, H=8, d=128):
-  """Low-precision shape: lens U{1024..4096}, pos bias, N=4096 (bf16 masters)."""
+def config5(seed=5, B=32, L=4096, H=8, d=128, fp8=True):
+  """Low-precision shape: lens U{1024..4096}, pos bias, N=4096.  With fp8 the
+  caller quantises q and k per head (scale = amax / 448) to float8_e4m3fn and
+  keeps v in bf16; the masters here are fp32."""
   rng = np.random.Generator(np.random.PCG64(seed))
   lens = rng.integers(1024, L + 1, B).astype(np.int32)
   T = int(lens.sum())
   q, k, v = (_normal(rng, (T, H, d), 0.1) for _ in range(3))
   pos = _normal(rng, (H, 2 * L - 1), 0.02)
-  return Workload("C5", B, L, H, d, "bf16", "jagged", lens, q, k, v, n=L,
+  return Workload("C5", B, L, H, d, "fp8" if fp8 else "bf16", "jagged", lens, q, k, v, n=L,
                   pos_tab=pos, seq_offsets=_offsets(lens))
 
 

@@ -372,6 +372,59 @@ def test_timestamp_spans_sorted_unsorted_and_huge(gpu):
   assert _err(outj.float().cpu().numpy(), refj) <= BF16_TOL
 
 
+def _quant(x):
+  """Per-head float8_e4m3fn quantisation on the host: (fp8 tensor on the GPU, scales, dequantised fp32)."""
+  xq, scale = O.quantize_e4m3fn_per_head(x)
+  dev8 = torch.from_numpy(xq).to("cuda:0").to(torch.float8_e4m3fn)   # exact: xq is representable
+  return dev8, _dev(scale), xq * scale[:, None]
+
+
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_fp8_qk_against_dequantised_oracle(gpu, d):
+  rng = np.random.default_rng(50 + d)
+  B, L, H = 3, 200, 2
+  lens = np.array([200, 77, 129], dtype=np.int32)
+  q, k = (rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3 for _ in range(2))
+  v = O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3)
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.1).astype(np.float32)
+  ts = 1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, (B, L))), axis=1).astype(np.int64)
+  tab = (rng.standard_normal((H, 129)) * 0.2).astype(np.float32)
+  q8, qs, qd = _quant(q)
+  k8, ks, kd = _quant(k)
+  # the kernel's error alone: oracle on exactly the values the kernel multiplies
+  ref = O.hstu_attention_ref(qd, kd, v, seq_lens=lens, pos_tab=pos, timestamps=ts, ts_tab=tab, dtype=np.float32)
+  out = recml_amd.hstu_attention(q8, k8, _dev(v, torch.bfloat16), q_scale=qs, k_scale=ks, seq_lens=_dev(lens),
+                                 pos_bias=_dev(pos), timestamps=_dev(ts), ts_bias=_dev(tab))
+  assert out.dtype == torch.bfloat16
+  out = out.float().cpu().numpy()
+  assert _err(out, ref) <= BF16_TOL
+  for b in range(B):
+    assert (out[b, lens[b]:] == 0).all()
+  # against the unquantised inputs: the quantisation error itself (reported, loosely bounded)
+  full = O.hstu_attention_ref(q, k, v, seq_lens=lens, pos_tab=pos, timestamps=ts, ts_tab=tab, dtype=np.float32)
+  assert _err(out, full) <= 0.15
+  # jagged, no bias, non-causal
+  qj8 = torch.cat([q8[b, :lens[b]] for b in range(B)])
+  kj8 = torch.cat([k8[b, :lens[b]] for b in range(B)])
+  vj, off = O.padded_to_jagged(v, lens)
+  outj = recml_amd.hstu_attention(qj8, kj8, _dev(vj, torch.bfloat16), q_scale=qs, k_scale=ks,
+                                  seq_offsets=_dev(off.astype(np.int32)), max_len=L, causal=False)
+  refj = O.hstu_attention_ref(qd, kd, v, seq_lens=lens, causal=False, dtype=np.float32)
+  assert _err(O.jagged_to_padded(outj.float().cpu().numpy(), off, L), refj) <= BF16_TOL
+
+
+def test_fp8_argument_errors(gpu):
+  z8 = torch.zeros((2, 8, 2, 32), device="cuda:0").to(torch.float8_e4m3fn)
+  zb = torch.zeros((2, 8, 2, 32), device="cuda:0", dtype=torch.bfloat16)
+  with pytest.raises(ValueError, match="bfloat16 v"):
+    recml_amd.hstu_attention(z8, z8, z8)
+  with pytest.raises(ValueError, match="matrix-core"):
+    recml_amd.hstu_attention(z8, z8, zb, sliding_window_size=2)
+  with pytest.raises(ValueError, match="q_scale"):
+    recml_amd.hstu_attention(zb, zb, zb, q_scale=torch.ones(2, device="cuda:0"))
+  assert recml_amd.hstu_attention(z8, z8, zb).abs().max().item() == 0.0
+
+
 def test_argument_errors(gpu):
   z = torch.zeros((2, 8, 2, 32), device="cuda:0")
   seg = torch.ones((2, 8), dtype=torch.int32, device="cuda:0")

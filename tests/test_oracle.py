@@ -295,3 +295,28 @@ def test_round_bf16():
   import torch
   t = torch.from_numpy(np.random.default_rng(0).standard_normal(1000).astype(np.float32))
   np.testing.assert_array_equal(O.round_bf16(t.numpy()), t.bfloat16().float().numpy())
+
+
+def test_e4m3fn_rounding_against_torch_cast():
+  import torch
+  codes = np.arange(256, dtype=np.uint8)
+  vals = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()
+  finite = np.isfinite(vals)
+  assert finite.sum() == 254 and np.abs(vals[finite]).max() == 448.0
+  v = vals[finite]
+  # every representable value is a fixed point and encodes to its own bit pattern
+  assert (O.round_e4m3fn(v) == v).all()
+  assert (O.encode_e4m3fn(v) == codes[finite]).all()
+  # midpoints between neighbours (ties to even) and points either side of them
+  pos = np.sort(np.unique(v[v >= 0]))
+  mids = (pos[:-1] + pos[1:]) / 2
+  probe = np.concatenate([mids, mids * (1 + 1e-6), mids * (1 - 1e-6)]).astype(np.float32)
+  probe = np.concatenate([probe, -probe])
+  rng = np.random.default_rng(0)
+  probe = np.concatenate([probe, rng.uniform(-448, 448, 20000).astype(np.float32),
+                          (rng.standard_normal(20000) * 0.05).astype(np.float32)])
+  want = torch.from_numpy(probe).to(torch.float8_e4m3fn).float().numpy()
+  got = O.round_e4m3fn(probe)
+  assert (got == want).all()
+  q, scale = O.quantize_e4m3fn_per_head(rng.standard_normal((5, 7, 3, 16)).astype(np.float32))
+  assert scale.shape == (3,) and np.abs(q).max() == 448.0 and (O.round_e4m3fn(q) == q).all()

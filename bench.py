@@ -195,7 +195,7 @@ def main():
   capped_peak = min(peak, ai * PEAK_HBM_GBS / 1e3)
 
   rec = {
-      "metric": "HSTU attn fwd TFLOP/s (unmasked), L=%d bf16" % w.L,
+      "metric": "HSTU attn fwd TFLOP/s (unmasked), L=%d %s" % (w.L, "fp8" if w.dtype == "fp8" else "bf16"),
       "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
       "warmup": args.warmup, "ms_per_step": ms_per_step,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

@@ -1,8 +1,9 @@
 """MI355X-native HSTU pointwise-SiLU attention (forward).
 
 Public surface mirrors the reference operator
-(recml/core/ops/hstu_ops.py:829-851) and the layer-side call
-(recml/layers/keras/hstu.py:356-390).
+(recml/core/ops/hstu_ops.py:829-851), the layer-side call
+(recml/layers/keras/hstu.py:356-390) and, as a harness around the kernel, the
+HSTU block and model forward (recml/layers/keras/hstu.py:240-621).
 """
 
 from recml_amd.hstu_ops import (  # noqa: F401
@@ -12,3 +13,4 @@ from recml_amd.hstu_ops import (  # noqa: F401
     pointwise_splash_attention,
 )
 from recml_amd.masks import make_attention_mask, make_causal_mask  # noqa: F401
+from recml_amd.hstu_layer import HSTU, HSTUBlock  # noqa: F401

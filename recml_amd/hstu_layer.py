@@ -1,0 +1,171 @@
+"""HSTU block and model forward around the MI355X attention kernel.
+
+The harness for the end-to-end (config-4) shape: everything except the
+attention is plain torch on the GPU (embedding gather, layer norms, the
+projections as rocBLAS / hipBLASLt GEMMs); the attention is
+`recml_amd.hstu_attention`, i.e. the HIP kernel behind the C ABI.  Inference
+forward only (no dropout, no autograd through the kernel).
+
+Mirrors, name for name:
+  HSTUBlock   recml/layers/keras/hstu.py:240-474 (weights :281-354, call :422-474)
+  HSTU        recml/layers/keras/hstu.py:492-621 (call :585-621)
+
+Differences from the reference layer, on purpose:
+  * the [B, L, L] attention mask and bias tensors are never built: the block
+    takes `seq_lens` (end-padded batches, as the reference's data pipeline
+    produces) and the bias *tables* (`pos_bias`, `timestamps` + `ts_bias`);
+  * U, Q, K, V come from one fused [D, 4D] GEMM; the four kernels are stored
+    separately under the reference's names and concatenated at call time;
+  * softmax attention (hstu.py:392-420) is not implemented here.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+from recml_amd import hstu_ops
+from recml_amd import masks
+
+
+def _glorot_uniform(shape, fan_in, fan_out, generator, dtype, device):
+  limit = math.sqrt(6.0 / (fan_in + fan_out))
+  w = torch.empty(shape, dtype=torch.float32)
+  w.uniform_(-limit, limit, generator=generator)
+  return w.to(device=device, dtype=dtype)
+
+
+class HSTUBlock(torch.nn.Module):
+  """One HSTU block: LN -> U,Q,K,V = act(x W) -> pointwise attention -> LN over
+  (heads, head_dim) -> U * normed -> output projection -> + inputs
+  (recml/layers/keras/hstu.py:444-474)."""
+
+  def __init__(self, hidden_dim: int, num_heads: int, use_bias: bool = False,
+               layer_norm_epsilon: float = 1e-6, scaled_pointwise_attn: bool = False,
+               softmax_attention: bool = False, dropout: float = 0.0,
+               dtype=torch.float32, device=None, generator=None):
+    super().__init__()
+    if softmax_attention:
+      raise NotImplementedError("softmax attention is outside this build; only the pointwise path is accelerated")
+    if hidden_dim % num_heads:
+      raise ValueError(f"hidden_dim {hidden_dim} is not a multiple of num_heads {num_heads}")
+    del dropout  # inference only
+    self.num_heads = num_heads
+    self.head_dim = hidden_dim // num_heads
+    self.hidden_dim = hidden_dim
+    self.eps = layer_norm_epsilon
+    self.scaled_pointwise_attn = scaled_pointwise_attn
+    H, hd, D = num_heads, self.head_dim, hidden_dim
+    P = torch.nn.Parameter
+    # EinsumDense "btd,dnh->btnh": kernel [D, H, hd], Glorot-uniform with the fans Keras
+    # computes for a rank-3 shape (see _fans)
+    fi, fo = self._fans((D, H, hd))
+    for name in ("u", "q", "k", "v"):
+      self.register_parameter(f"{name}_kernel", P(_glorot_uniform((D, H, hd), fi, fo, generator, dtype, device), requires_grad=False))
+      if use_bias:
+        self.register_parameter(f"{name}_bias", P(torch.zeros((H, hd), dtype=dtype, device=device), requires_grad=False))
+    fi, fo = self._fans((H, hd, D))
+    self.output_kernel = P(_glorot_uniform((H, hd, D), fi, fo, generator, dtype, device), requires_grad=False)
+    self.output_bias = P(torch.zeros((D,), dtype=dtype, device=device), requires_grad=False) if use_bias else None
+    self.use_bias = use_bias
+    self.input_ln_gamma = P(torch.ones((D,), dtype=dtype, device=device), requires_grad=False)
+    self.input_ln_beta = P(torch.zeros((D,), dtype=dtype, device=device), requires_grad=False)
+    self.attn_ln_gamma = P(torch.ones((H, hd), dtype=dtype, device=device), requires_grad=False)
+    self.attn_ln_beta = P(torch.zeros((H, hd), dtype=dtype, device=device), requires_grad=False)
+
+  @staticmethod
+  def _fans(shape):
+    """Keras' fan computation for a rank-3 kernel: the leading axes are the
+    receptive field (keras/src/initializers/random_initializers.py,
+    compute_fans): fan_in = shape[-2] * prod(shape[:-2]), fan_out = shape[-1] * prod(shape[:-2])."""
+    rf = 1
+    for s in shape[:-2]:
+      rf *= s
+    return shape[-2] * rf, shape[-1] * rf
+
+  def forward(self, inputs, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None,
+              attention_mask=None, attention_bias=None):
+    """inputs [B, L, D] -> [B, L, D].
+
+    Give `seq_lens` [B] (keys and rows at or past the length are masked, as
+    make_causal_mask does for an end-padded batch) with optional bias tables;
+    or, for the reference's calling convention, a dense `attention_mask`
+    [B, L, L] and optional `attention_bias` [B, L, L]
+    (recml/layers/keras/hstu.py:422-440).
+    """
+    B, L, D = inputs.shape
+    H, hd = self.num_heads, self.head_dim
+    x = F.layer_norm(inputs, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
+    w = torch.cat([self.u_kernel, self.q_kernel, self.k_kernel, self.v_kernel], dim=1).reshape(D, 4 * H * hd)
+    uqkv = x.reshape(B * L, D) @ w
+    if self.use_bias:
+      uqkv = uqkv + torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1)
+    uqkv = F.silu(uqkv).reshape(B, L, 4, H, hd)
+    u, q, k, v = uqkv.unbind(dim=2)
+    if attention_mask is not None:
+      attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
+                                          scaled_pointwise_attn=self.scaled_pointwise_attn)
+    else:
+      alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
+      attn = hstu_ops.hstu_attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
+                                     timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias)
+    normed = F.layer_norm(attn.reshape(B, L, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
+                          self.attn_ln_beta.reshape(-1), self.eps)
+    gated = u.reshape(B, L, H * hd) * normed
+    out = gated.reshape(B * L, H * hd) @ self.output_kernel.reshape(H * hd, D)
+    if self.use_bias:
+      out = out + self.output_bias
+    return out.reshape(B, L, D) + inputs
+
+
+class HSTU(torch.nn.Module):
+  """The HSTU model forward (recml/layers/keras/hstu.py:585-621): item
+  embedding (x sqrt(D)) + position embedding -> final_norm -> blocks ->
+  final_norm (the same layer both times) -> optional untied output head."""
+
+  def __init__(self, *, vocab_size: int, max_positions: int | None = None, model_dim: int,
+               num_heads: int, num_layers: int, dropout: float = 0.0, norm_eps: float = 1e-6,
+               scale_by_sqrt_dim: bool = False, add_head: bool = True,
+               dtype=torch.float32, device=None, seed: int = 0):
+    super().__init__()
+    g = torch.Generator().manual_seed(seed)
+    P = torch.nn.Parameter
+    normal = lambda shape: (torch.randn(shape, generator=g) * 0.02).to(device=device, dtype=dtype)
+    self.item_embedding = P(normal((vocab_size, model_dim)), requires_grad=False)
+    self.position_embedding = P(normal((max_positions, model_dim)), requires_grad=False) if max_positions else None
+    self.decoder_blocks = torch.nn.ModuleList(
+        HSTUBlock(model_dim, num_heads, layer_norm_epsilon=norm_eps, dropout=dropout, dtype=dtype, device=device, generator=g)
+        for _ in range(num_layers))
+    self.final_norm_gamma = P(torch.ones((model_dim,), dtype=dtype, device=device), requires_grad=False)
+    self.final_norm_beta = P(torch.zeros((model_dim,), dtype=dtype, device=device), requires_grad=False)
+    self.reverse_embedding = P(normal((model_dim, vocab_size)), requires_grad=False) if add_head else None
+    self.model_dim = model_dim
+    self.eps = norm_eps
+    self.scale_by_sqrt_dim = scale_by_sqrt_dim
+
+  def count_params(self) -> int:
+    return sum(p.numel() for p in self.parameters())
+
+  def _final_norm(self, x):
+    return F.layer_norm(x, (self.model_dim,), self.final_norm_gamma, self.final_norm_beta, self.eps)
+
+  def forward(self, inputs, padding_mask=None, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None):
+    """inputs: item ids [B, L]; `padding_mask` [B, L] (1 = real item, end-padded) or `seq_lens` [B]."""
+    if seq_lens is None:
+      if padding_mask is None:
+        raise ValueError("Either `padding_mask` or `seq_lens` must be set.")
+      seq_lens = masks.lengths_from_padding_mask(padding_mask)
+    x = self.item_embedding[inputs]
+    if self.scale_by_sqrt_dim:
+      x = x * (self.model_dim ** 0.5)
+    if self.position_embedding is not None:
+      x = x + self.position_embedding[: x.shape[1]]
+    x = self._final_norm(x)
+    for block in self.decoder_blocks:
+      x = block(x, seq_lens=seq_lens, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
+    x = self._final_norm(x)
+    if self.reverse_embedding is None:
+      return x
+    return x @ self.reverse_embedding

@@ -1,0 +1,151 @@
+"""HSTU block / model harness: the oracle's pieces pinned on the CPU, the torch
+harness (with the HIP attention inside) against the oracle on the GPU."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hstu_block_oracle as BO
+from oracle import hstu_oracle as O
+
+
+def test_layer_norm_definition_and_torch():
+  # hand case: x = [1, 2, 3, 4]: mean 2.5, biased var 1.25
+  x = np.array([[1.0, 2.0, 3.0, 4.0]])
+  got = BO.layer_norm(x, np.ones(4), np.zeros(4), 0.0)
+  assert np.allclose(got, (x - 2.5) / np.sqrt(1.25), rtol=0, atol=1e-15)
+  got = BO.layer_norm(x, np.array([2.0, 2, 2, 2]), np.array([1.0, 1, 1, 1]), 1e-6)
+  assert np.allclose(got, 2 * (x - 2.5) / np.sqrt(1.25 + 1e-6) + 1, atol=1e-15)
+  # joint normalisation over two axes == normalisation of the flattened vector
+  rng = np.random.default_rng(0)
+  y = rng.standard_normal((3, 5, 4, 8))
+  g, b = rng.standard_normal((4, 8)), rng.standard_normal((4, 8))
+  two = BO.layer_norm(y, g, b, 1e-6, axes=(-2, -1))
+  flat = BO.layer_norm(y.reshape(3, 5, 32), g.reshape(32), b.reshape(32), 1e-6).reshape(y.shape)
+  assert np.allclose(two, flat, atol=1e-14)
+  # an independent implementation
+  t = torch.nn.functional.layer_norm(torch.from_numpy(y.reshape(3, 5, 32)), (32,), torch.from_numpy(g.reshape(32)),
+                                     torch.from_numpy(b.reshape(32)), 1e-6).numpy().reshape(y.shape)
+  assert np.allclose(two, t, atol=1e-12)
+
+
+def test_param_count_matches_reference_literal():
+  # recml/layers/keras/hstu_test.py:38-48 with vocab 500, positions 20, dim 32, 3 layers
+  want = (500 * 32) + (20 * 32) + 3 * ((32 * 32 * 4 + 32 * 32) + (2 * 32) * 2) + (2 * 32) + (500 * 32)
+  assert BO.hstu_param_count(500, 20, 32, 3) == want
+  from recml_amd.hstu_layer import HSTU
+  m = HSTU(vocab_size=500, max_positions=20, model_dim=32, num_heads=4, num_layers=3, dropout=0.1)
+  assert m.count_params() == want
+  with pytest.raises(ValueError, match="padding_mask"):
+    m(torch.zeros((2, 3), dtype=torch.long))
+  with pytest.raises(NotImplementedError):
+    from recml_amd.hstu_layer import HSTUBlock
+    HSTUBlock(32, 4, softmax_attention=True)
+
+
+def test_block_oracle_padded_rows_and_independence():
+  # padded rows: attention output 0 -> LN gives beta -> out = W(u * beta) + x; sequences independent
+  rng = np.random.default_rng(1)
+  B, L, D, H = 2, 6, 16, 2
+  w = _rand_block(rng, D, H)
+  x = rng.standard_normal((B, L, D))
+  lens = np.array([6, 3])
+  out = BO.hstu_block(x, w, num_heads=H, seq_lens=lens)
+  normed = BO.layer_norm(x, w["input_ln_gamma"], w["input_ln_beta"], 1e-6)
+  u = O.silu(np.einsum("btd,dnh->btnh", normed, w["u_kernel"]))
+  pad = np.einsum("btnh,nhd->btd", u * w["attn_ln_beta"], w["output_kernel"]) + x
+  assert np.allclose(out[1, 3:], pad[1, 3:], atol=1e-12)
+  x2 = x.copy()
+  x2[0] += 1.0
+  out2 = BO.hstu_block(x2, w, num_heads=H, seq_lens=lens)
+  assert np.array_equal(out2[1], out[1])
+  # causality: changing a later token leaves earlier rows alone
+  x3 = x.copy()
+  x3[0, 4] += 1.0
+  out3 = BO.hstu_block(x3, w, num_heads=H, seq_lens=lens)
+  assert np.allclose(out3[0, :4], out[0, :4], atol=1e-13) and not np.allclose(out3[0, 4:], out[0, 4:])
+
+
+def _rand_block(rng, D, H, bias=False):
+  hd = D // H
+  w = {f"{n}_kernel": rng.standard_normal((D, H, hd)) / np.sqrt(D) for n in "uqkv"}
+  w["output_kernel"] = rng.standard_normal((H, hd, D)) / np.sqrt(D)
+  w["input_ln_gamma"] = 1 + 0.1 * rng.standard_normal(D)
+  w["input_ln_beta"] = 0.1 * rng.standard_normal(D)
+  w["attn_ln_gamma"] = 1 + 0.1 * rng.standard_normal((H, hd))
+  w["attn_ln_beta"] = 0.1 * rng.standard_normal((H, hd))
+  if bias:
+    for n in "uqkv":
+      w[f"{n}_bias"] = 0.1 * rng.standard_normal((H, hd))
+    w["output_bias"] = 0.1 * rng.standard_normal(D)
+  return w
+
+
+def _load_block(block, w, dtype):
+  name_map = {"output_kernel": "output_kernel", "output_bias": "output_bias"}
+  for k, val in w.items():
+    getattr(block, name_map.get(k, k)).data = torch.from_numpy(np.asarray(val)).to(device="cuda:0", dtype=dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_block_on_gpu_against_oracle(gpu, dtype, tol):
+  from recml_amd.hstu_layer import HSTUBlock
+  rng = np.random.default_rng(2)
+  B, L, D, H = 3, 70, 128, 2
+  lens = np.array([70, 33, 1], dtype=np.int32)
+  for use_bias, scaled in ((False, False), (True, True)):
+    w = _rand_block(rng, D, H, bias=use_bias)
+    x = rng.standard_normal((B, L, D))
+    pos = 0.1 * rng.standard_normal(2 * L - 1)
+    blk = HSTUBlock(D, H, use_bias=use_bias, scaled_pointwise_attn=scaled, dtype=dtype, device="cuda:0")
+    _load_block(blk, w, dtype)
+    rd = lambda a: torch.from_numpy(np.asarray(a)).to(device="cuda:0", dtype=dtype).double().cpu().numpy()
+    wq = {k: rd(v) for k, v in w.items()}          # the oracle sees the weights as stored
+    xq = rd(x)
+    ref = BO.hstu_block(xq, wq, num_heads=H, seq_lens=lens, scaled_pointwise_attn=scaled, pos_tab=pos)
+    out = blk(torch.from_numpy(xq).to(device="cuda:0", dtype=dtype), seq_lens=torch.from_numpy(lens).cuda(),
+              pos_bias=torch.from_numpy(pos).float().cuda()).double().cpu().numpy()
+    assert np.abs(out - ref).max() / np.abs(ref).max() <= tol
+    # the reference's calling convention: dense mask + dense bias
+    mask = O.make_causal_mask((np.arange(L)[None] < lens[:, None]).astype(np.float32))
+    out2 = blk(torch.from_numpy(xq).to(device="cuda:0", dtype=dtype), attention_mask=torch.from_numpy(mask).cuda(),
+               attention_bias=torch.from_numpy(O.rel_pos_bias(pos, L)).float().cuda()).double().cpu().numpy()
+    assert np.abs(out2 - ref).max() / np.abs(ref).max() <= tol
+
+
+@pytest.mark.gpu
+def test_model_on_gpu_against_oracle(gpu):
+  from recml_amd.hstu_layer import HSTU
+  m = HSTU(vocab_size=500, max_positions=20, model_dim=32, num_heads=4, num_layers=3, device="cuda:0", seed=3)
+  ids = torch.tensor([[1, 2, 3], [4, 5, 0]], device="cuda:0")
+  pm = torch.tensor([[1, 1, 1], [1, 1, 0]], device="cuda:0")
+  out = m(ids, pm)
+  assert tuple(out.shape) == (2, 3, 500) and out.dtype == torch.float32   # hstu_test.py:52-60
+  g = lambda p: p.detach().double().cpu().numpy()
+  w = {"item_embedding": g(m.item_embedding), "position_embedding": g(m.position_embedding),
+       "final_norm_gamma": g(m.final_norm_gamma), "final_norm_beta": g(m.final_norm_beta),
+       "reverse_embedding": g(m.reverse_embedding),
+       "blocks": [{n: g(p) for n, p in b.named_parameters()} for b in m.decoder_blocks]}
+  ref = BO.hstu_model(ids.cpu().numpy(), w, num_heads=4, seq_lens=np.array([3, 2]))
+  assert np.abs(out.double().cpu().numpy() - ref).max() / np.abs(ref).max() <= 2e-5
+
+
+@pytest.mark.gpu
+def test_block_config4_shape_bf16(gpu):
+  # B=128, L=1024, D=512, H=8 (hd=64), lens U{128..1024}, pos bias: one layer at full size,
+  # checked on three sequences (the block treats sequences independently)
+  from recml_amd.hstu_layer import HSTUBlock
+  rng = np.random.default_rng(4)
+  B, L, D, H = 128, 1024, 512, 8
+  lens = rng.integers(128, L + 1, B).astype(np.int32)
+  lens[:3] = [1024, 128, 517]
+  blk = HSTUBlock(D, H, dtype=torch.bfloat16, device="cuda:0", generator=torch.Generator().manual_seed(4))
+  x = (torch.randn((B, L, D), generator=torch.Generator().manual_seed(5)) * 1.0).to(device="cuda:0", dtype=torch.bfloat16)
+  pos = (torch.randn((2 * L - 1,), generator=torch.Generator().manual_seed(6)) * 0.02).cuda()
+  out = blk(x, seq_lens=torch.from_numpy(lens).cuda(), pos_bias=pos)
+  assert tuple(out.shape) == (B, L, D) and torch.isfinite(out.float()).all()
+  w = {n: p.detach().double().cpu().numpy() for n, p in blk.named_parameters()}
+  ref = BO.hstu_block(x[:3].double().cpu().numpy(), w, num_heads=H, seq_lens=lens[:3], pos_tab=pos.double().cpu().numpy())
+  got = out[:3].double().cpu().numpy()
+  assert np.abs(got - ref).max() / np.abs(ref).max() <= 3e-2

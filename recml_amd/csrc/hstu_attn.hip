@@ -41,6 +41,7 @@ typedef bf16_t bf16x8 __attribute__((ext_vector_type(8)));
 typedef bf16_t bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 struct Params {
   const void* q;
@@ -79,6 +80,20 @@ struct Params {
   float ts_log2_scale;  // ln(2) / ts_bucket_size
   float alpha, inv_n;
   int32_t n_qtiles;
+  // Key-range splitting (MFMA kernel; off when split_steps == 0): a query tile with more than
+  // split_steps 32-key steps is shared by up to MAX_CHUNKS workgroups, each covering a contiguous
+  // part of the keys and leaving its fp32 partial O^T in `partial`; hstu_combine sums them.
+  int32_t split_steps;
+  int32_t qt_split;          // first query tile that can be split
+  int32_t entries_per_bh;    // workgroups per (sequence, head): sum over query tiles of chunks_max
+  float* partial;            // [tile slot][head][chunk][BM x d_v floats in register order]
+  // Work list built on the device by hstu_prepare (MFMA kernel; null = workgroups enumerate every
+  // possible (sequence, tile, chunk) and most exit): sched[0] = number of items, then from
+  // sched[4] on one int4 per (sequence, query tile, chunk) that has work:
+  // {b, qt | chunk << 16, first token, stored length}.
+  const int32_t* sched;
+  int64_t items_max;         // capacity of the list (sizes the grid)
+  int64_t split_max;         // capacity of the list of split tiles behind it: sched[1] int4s at sched + 4 + 4 items_max
 };
 
 // Per-sequence geometry shared by both kernels.
@@ -92,11 +107,12 @@ struct Seq {
   int n_ts;       // timestamps addressable for this sequence
 };
 
-__device__ __forceinline__ Seq seq_info(const Params& p, int b, int h) {
+// o0: first token (jagged layout); nraw: the sequence's length as stored (offset difference or
+// seq_lens entry; ignored for the padded layout without a length mask).
+__device__ __forceinline__ Seq seq_from(const Params& p, int b, int h, int o0, int nraw) {
   Seq s;
   if (p.jagged) {
-    int o0 = p.seq_offsets[b], o1 = p.seq_offsets[b + 1];
-    int n = o1 - o0;
+    int n = nraw;
     n = n < 0 ? 0 : (n > p.L ? p.L : n);
     s.n_q = n; s.n_kv = n; s.rows = n; s.tok0 = o0;
     s.bq = (int64_t)o0 * p.q_st + (int64_t)h * p.q_sh;
@@ -106,7 +122,7 @@ __device__ __forceinline__ Seq seq_info(const Params& p, int b, int h) {
   } else {
     int nq = p.L, nk = p.Lkv;
     if (p.mask_mode == HSTU_MASK_LENGTH) {
-      int n = p.seq_lens[b];
+      int n = nraw;
       n = n < 0 ? 0 : n;
       nq = n < p.L ? n : p.L;
       nk = n < p.Lkv ? n : p.Lkv;
@@ -120,6 +136,23 @@ __device__ __forceinline__ Seq seq_info(const Params& p, int b, int h) {
   if (p.ts_sb != 0) { s.ts0 = (int64_t)b * p.ts_sb; s.n_ts = p.L; }
   else              { s.ts0 = s.tok0;               s.n_ts = s.n_kv; }
   return s;
+}
+
+__device__ __forceinline__ void seq_raw(const Params& p, int b, int& o0, int& nraw) {
+  o0 = 0;
+  nraw = p.L;
+  if (p.jagged) {
+    o0 = p.seq_offsets[b];
+    nraw = p.seq_offsets[b + 1] - o0;
+  } else if (p.mask_mode == HSTU_MASK_LENGTH) {
+    nraw = p.seq_lens[b];
+  }
+}
+
+__device__ __forceinline__ Seq seq_info(const Params& p, int b, int h) {
+  int o0, nraw;
+  seq_raw(p, b, o0, nraw);
+  return seq_from(p, b, h, o0, nraw);
 }
 
 __device__ __forceinline__ float ldf(const float* p) { return *p; }
@@ -389,6 +422,75 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
 // vmcnt(n) with expcnt / lgkmcnt left alone (gfx9 encoding: vmcnt = bits 3:0 and 15:14)
 #define HSTU_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 15) | ((((n) >> 4) & 3) << 14)) | 0x0F70)
 
+constexpr int MAX_CHUNKS = 4;
+
+// Most workgroups a query tile can be shared by (from its position alone), and how many share
+// it given its actual number of steps.
+__host__ __device__ __forceinline__ int chunks_max(int split_steps, int causal, int L, int qt) {
+  if (split_steps <= 0) return 1;
+  const int all = (L + BN - 1) / BN;
+  int nt = causal ? (qt + 1) * (BM / BN) : all;
+  nt = nt < all ? nt : all;
+  const int c = (nt + split_steps - 1) / split_steps;
+  return c < MAX_CHUNKS ? c : MAX_CHUNKS;
+}
+__device__ __forceinline__ int chunks_of(const Params& p, int nt) {
+  if (p.split_steps <= 0) return 1;
+  static_assert(MAX_CHUNKS == 4, "min(MAX_CHUNKS, ceil(nt / split_steps)) without a division");
+  const int s = p.split_steps;
+  return 1 + (nt > s ? 1 : 0) + (nt > 2 * s ? 1 : 0) + (nt > 3 * s ? 1 : 0);
+}
+// Slot of a split tile in the partial buffer: jagged sequences are packed by an upper bound of
+// the tiles before them.
+__device__ __forceinline__ int64_t partial_slot(const Params& p, int b, int64_t tok0, int qt) {
+  return (p.jagged ? (tok0 >> 7) + b : (int64_t)b * (p.n_qtiles - p.qt_split)) + (qt - p.qt_split);
+}
+// Steps of a tile: keys [0, kv_end) in 32-key steps
+__device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0) {
+  int kv_end = s.n_kv;
+  if (p.causal) {
+    int lim = q0 + BM < s.n_q ? q0 + BM : s.n_q;
+    kv_end = lim < kv_end ? lim : kv_end;
+  }
+  return (kv_end + BN - 1) / BN;
+}
+
+// Which (sequence, head, query tile, chunk) a workgroup of the main (or combine) kernel has.
+// Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with its own L2: every
+// tile of one (sequence, head) goes to the same XCD, and tiles of a sequence are adjacent in
+// launch order, the one with most keys first, so that the tiles running together stream the
+// same K/V rows and share them through that L2.  Returns false when there is nothing to do.
+struct Work { int b, h, qt, chunk; Seq s; };
+template <bool SPLIT_LIST = false>
+__device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, Work& wk) {
+  const int xcd = block & 7, j = block >> 3;
+  if (p.sched) {
+    // from the work list: with H >= 8 head h runs on XCD h % 8, else 8 / H items share a round
+    int it, h;
+    if (p.H >= 8) { const int hx = p.H >> 3; it = j / hx; h = (j - it * hx) * 8 + xcd; }
+    else          { const int r = 8 / p.H;   it = j * r + xcd / p.H; h = xcd % p.H; }
+    if (it >= p.sched[SPLIT_LIST ? 1 : 0]) return false;
+    const int4 item = ((const int4*)(p.sched + 4))[(SPLIT_LIST ? p.items_max : 0) + it];
+    wk.b = item.x; wk.h = h; wk.qt = item.y & 0xffff; wk.chunk = item.y >> 16;
+    wk.s = seq_from(p, wk.b, h, item.z, item.w);
+    return true;
+  }
+  // without a list: entry -> (query tile, chunk of its key range), tiles from the last one down
+  const int bhk = j / p.entries_per_bh;
+  int qt = p.n_qtiles - 1, chunk = j - bhk * p.entries_per_bh;
+  for (;;) {
+    const int c = chunks_max(p.split_steps, p.causal, p.L, qt);
+    if (chunk < c) break;
+    chunk -= c;
+    --qt;
+  }
+  const int bh = bhk * 8 + xcd;
+  if (bh >= p.B * p.H) return false;
+  wk.b = bh / p.H; wk.h = bh - wk.b * p.H; wk.qt = qt; wk.chunk = chunk;
+  wk.s = seq_info(p, wk.b, wk.h);
+  return true;
+}
+
 // Where sequence b starts in the int32 timestamp copy and in the per-tile range table.
 // Timestamps that follow the token axis are packed like it (tiles by an upper bound of
 // the tiles before them); timestamps with a batch stride are [B][L].
@@ -408,9 +510,94 @@ __device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_
 //    of those in each 32-key tile.  One workgroup per sequence.
 __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __restrict__ pos_out, float* __restrict__ tab_out,
                                                     int32_t* __restrict__ ok_out, int32_t* __restrict__ rel_out,
-                                                    int32_t* __restrict__ range_out) {
+                                                    int32_t* __restrict__ range_out, int32_t* __restrict__ sched_out) {
   const int tid = threadIdx.x;
   const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
+  if (sched_out && blockIdx.x == gridDim.x - 1) {
+    // The work lists, by the last workgroup (the host launches one more than the rest needs).
+    // Sequences are taken longest first (batches of up to SORT_MAX sequences; larger ones in
+    // batch order): the tiles with most keys start first and short ones fill in behind them.
+    // Thread t owns a run of sequences in that order, counts their items, finds where they start
+    // from the counts of the threads before it, and writes them out, last query tile (most keys)
+    // first within a sequence.  Items with chunk 1 also go to the list of split tiles.
+    constexpr int SORT_MAX = 1024;
+    __shared__ int counts[4], counts_split[4];
+    __shared__ int keys[SORT_MAX], firsts[SORT_MAX], order[SORT_MAX];
+    const bool sorted = p.B <= SORT_MAX;
+    if (sorted) {
+      for (int b = tid; b < p.B; b += 256) {
+        int o0, nraw;
+        seq_raw(p, b, o0, nraw);
+        keys[b] = nraw;
+        firsts[b] = o0;
+      }
+      __syncthreads();
+      for (int b = tid; b < p.B; b += 256) {
+        const int kb = keys[b];
+        int rank = 0;
+#pragma unroll 8
+        for (int c = 0; c < p.B; ++c) rank += (keys[c] > kb || (keys[c] == kb && c < b)) ? 1 : 0;
+        order[rank] = b;
+      }
+      __syncthreads();
+    }
+    const int per = (p.B + 255) / 256;
+    const int r_lo = tid * per < p.B ? tid * per : p.B, r_hi = r_lo + per < p.B ? r_lo + per : p.B;
+    int4* items = (int4*)(sched_out + 4);
+    int4* split_items = items + p.items_max;
+    auto walk = [&](int b, int base, int base_split, bool write, int& n_split) {
+      int o0, nraw;
+      if (sorted) { o0 = firsts[b]; nraw = keys[b]; }
+      else seq_raw(p, b, o0, nraw);
+      const Seq sq = seq_from(p, b, 0, o0, nraw);
+      int n = 0;
+      n_split = 0;
+      for (int qt = (sq.rows + BM - 1) / BM - 1; qt >= 0; --qt) {
+        const int c = qt * BM >= sq.n_q ? 1 : chunks_of(p, tile_steps(p, sq, qt * BM));
+        for (int k = 0; k < c; ++k, ++n) {
+          const int4 it = int4{b, qt | (k << 16), o0, nraw};
+          if (write && base + n < p.items_max) items[base + n] = it;
+          if (k == 1) {
+            if (write && base_split + n_split < p.split_max) split_items[base_split + n_split] = it;
+            ++n_split;
+          }
+        }
+      }
+      return n;
+    };
+    int cnt = 0, cnt_split = 0;
+    for (int r = r_lo; r < r_hi; ++r) {
+      int ns;
+      cnt += walk(sorted ? order[r] : r, 0, 0, false, ns);
+      cnt_split += ns;
+    }
+    // exclusive prefix sums over the 256 threads: within the wave by shuffles, across the 4 waves by LDS
+    int inc = cnt, inc_split = cnt_split;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int a = __shfl_up(inc, d, 64), c = __shfl_up(inc_split, d, 64);
+      if ((tid & 63) >= d) { inc += a; inc_split += c; }
+    }
+    if ((tid & 63) == 63) { counts[tid >> 6] = inc; counts_split[tid >> 6] = inc_split; }
+    __syncthreads();
+    int base = inc - cnt, total = 0, base_split = inc_split - cnt_split, total_split = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      base += i < (tid >> 6) ? counts[i] : 0;
+      total += counts[i];
+      base_split += i < (tid >> 6) ? counts_split[i] : 0;
+      total_split += counts_split[i];
+    }
+    for (int r = r_lo; r < r_hi; ++r) {
+      int ns;
+      base += walk(sorted ? order[r] : r, base, base_split, true, ns);
+      base_split += ns;
+    }
+    if (tid == 0) {
+      sched_out[0] = total < p.items_max ? total : (int)p.items_max;
+      sched_out[1] = total_split < p.split_max ? total_split : (int)p.split_max;
+    }
+  }
   if (tab_out) {
     // bucket table times log2(e); indices past the last bucket repeat it (the clip of the bucket law)
     for (int i = gtid; i < p.ts_heads * TS_TAB_LEN; i += gsz) {
@@ -511,21 +698,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
 
-  // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with
-  // its own L2.  All query tiles of one (sequence, head) go to the same XCD and
-  // are adjacent in launch order, heaviest first, so that the tiles running
-  // together stream the same K/V rows and share them through that L2 instead
-  // of each pulling its own copy from HBM.
-  const int BH = p.B * p.H;
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int bhk = slot / p.n_qtiles;
-  const int qt = p.n_qtiles - 1 - (slot - bhk * p.n_qtiles);
-  const int bh = bhk * 8 + xcd;
-  if (bh >= BH) return;
-  const int b = bh / p.H, h = bh - b * p.H;
-  const Seq s = seq_info(p, b, h);
+  Work wk;
+  if (!work_of_block(p, blockIdx.x, wk)) return;
+  const int b = wk.b, h = wk.h, qt = wk.qt, chunk = wk.chunk;
+  const Seq& s = wk.s;
   const int q0 = qt * BM;
   if (q0 >= s.rows) return;
+  if (chunk > 0 && q0 >= s.n_q) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -550,12 +729,17 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const int qrow = r0 + m;             // this lane's query row
   const bool wave_live = r0 < s.n_q;
 
-  int kv_end = s.n_kv;
-  if (p.causal) {
-    int lim = q0 + BM < s.n_q ? q0 + BM : s.n_q;
-    kv_end = lim < kv_end ? lim : kv_end;
+  // this workgroup's steps [t_lo, nt) of the tile's
+  int nt = tile_steps(p, s, q0);
+  const int n_chunks = chunks_of(p, nt);
+  if (chunk >= n_chunks) return;
+  int t_lo = 0;
+  if (n_chunks > 1) {
+    const int per = (nt + n_chunks - 1) / n_chunks;
+    t_lo = chunk * per;
+    nt = t_lo + per < nt ? t_lo + per : nt;
+    if (t_lo >= nt) return;    // cannot happen for n_chunks = ceil(nt / split_steps) <= nt, kept as a guard
   }
-  const int nt = (kv_end + BN - 1) / BN;
   // last key this wave needs
   const int wave_last = !wave_live ? -1 : (p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1));
 
@@ -644,7 +828,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
-    if (t < nt) dma_step(t);
+    if (t_lo + t < nt) dma_step(t_lo + t);
 
   // Q fragments (B operand of S^T = K Q^T).  bf16: k-step ks of lane (row, hh) holds
   // q[qrow][16ks+8hh .. +7], i.e. 16-byte chunk 2ks+hh of the row.  fp8: the lane holds chunks
@@ -829,13 +1013,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     else HSTU_WAIT_VMCNT(0);
   };
 
-  wait_step(0);
+  wait_step(t_lo);
   __syncthreads();
 
   // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
   // which now receives step t+3; the block of step t is computed; then every
   // wave makes sure its share of step t+1 has landed before the next barrier.
-  for (int t = 0; t < nt; ++t) {
+  for (int t = t_lo; t < nt; ++t) {
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
     if (t * BN <= wave_last) block(t);
     if (t + 1 < nt) wait_step(t + 1);
@@ -844,6 +1028,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 
   // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0.
   // The 1/log2(e) left out of the SiLU is folded into the output scale.
+  if (n_chunks > 1) {
+    // fp32 partial in register order: float4 number (16 w + i) * 64 + lane of this (tile, head, chunk)
+    floatx4* dst = (floatx4*)(p.partial + ((partial_slot(p, b, s.tok0, qt) * p.H + h) * MAX_CHUNKS + chunk) * (int64_t)(BM * D)) +
+                   (w * (DVB * 4)) * 64 + lane;
+#pragma unroll
+    for (int i = 0; i < DVB * 4; ++i)
+      dst[i * 64] = floatx4{o[i >> 2][4 * (i & 3) + 0], o[i >> 2][4 * (i & 3) + 1], o[i >> 2][4 * (i & 3) + 2], o[i >> 2][4 * (i & 3) + 3]};
+    return;
+  }
   const float oscale = p.inv_n * (1.0f / LOG2E);
   if (qrow < s.rows) {
     const bool live = qrow < s.n_q;
@@ -859,6 +1052,62 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         }
         *(uint2*)(orow + 32 * dvb + 8 * g) = pko;
       }
+    }
+  }
+}
+
+// Sums the fp32 partials of the query tiles whose key range was split and writes their
+// output rows.  One workgroup per (sequence, head, splittable tile) with the lane roles of the
+// main kernel, so that each lane reads back exactly what lanes in its place wrote.
+template <int D>
+__global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
+  constexpr int DVB = D / 32;
+  // with a work list: one workgroup per entry of the list of split tiles; without: launched over
+  // the main kernel's grid, and the workgroup that has chunk 1 of a tile sums it
+  Work wk;
+  if (!work_of_block<true>(p, blockIdx.x, wk)) return;
+  if (wk.chunk != 1) return;
+  const int b = wk.b, h = wk.h, qt = wk.qt;
+  const Seq& s = wk.s;
+  const int q0 = qt * BM;
+  if (q0 >= s.n_q) return;
+  const int n_chunks = chunks_of(p, tile_steps(p, s, q0));
+  if (n_chunks <= 1) return;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int m = lane & 31, hh = lane >> 5;
+  const int qrow = q0 + 32 * w + m;
+  const floatx4* src = (const floatx4*)(p.partial + ((partial_slot(p, b, s.tok0, qt) * p.H + h) * MAX_CHUNKS) * (int64_t)(BM * D)) +
+                       (w * (DVB * 4)) * 64 + lane;
+  const float oscale = p.inv_n * (1.0f / LOG2E);
+  if (qrow >= s.rows) return;
+  const bool live = qrow < s.n_q;
+  bf16_t* orow = (bf16_t*)p.out + s.bo + (int64_t)qrow * p.o_st + 4 * hh;
+  // Every chunk slot is read, absent ones as a repeat of chunk 0 with weight 0, so that all the
+  // loads of a group are independent and in flight together.
+  constexpr int NP = DVB * 4, GRP = NP < 8 ? NP : 8;
+  const int c2 = n_chunks > 2 ? 2 : 0, c3 = n_chunks > 3 ? 3 : 0;
+  const float w2 = n_chunks > 2 ? 1.f : 0.f, w3 = n_chunks > 3 ? 1.f : 0.f;
+  constexpr int CS = BM * D / 4;   // float4s per chunk
+#pragma unroll
+  for (int g0 = 0; g0 < NP; g0 += GRP) {
+    floatx4 v0[GRP], v1[GRP], v2[GRP], v3[GRP];
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) {
+      v0[i] = src[(g0 + i) * 64];
+      v1[i] = src[(g0 + i) * 64 + CS];
+      v2[i] = src[(g0 + i) * 64 + c2 * CS];
+      v3[i] = src[(g0 + i) * 64 + c3 * CS];
+    }
+#pragma unroll
+    for (int i = 0; i < GRP; ++i) {
+      const floatx4 a = v0[i] + v1[i] + v2[i] * w2 + v3[i] * w3;
+      uint2 pko = {0u, 0u};
+      if (live) {
+        pko.x = pack_bf16(a.x * oscale, a.y * oscale);
+        pko.y = pack_bf16(a.z * oscale, a.w * oscale);
+      }
+      const int ii = g0 + i;
+      *(uint2*)(orow + 32 * (ii >> 2) + 8 * (ii & 3)) = pko;
     }
   }
 }
@@ -962,15 +1211,50 @@ Variant pick_variant(const HstuAttnFwdArgs* a) {
 // Workspace of the MFMA kernel: [scaled, padded position table][per-sequence int32-timestamp flag]
 // [int32 timestamps][their (min, max) per key tile], each part a multiple of 256 bytes.
 struct WorkspacePlan {
-  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes;
-  size_t total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes; }
+  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes, sched_bytes, partial_bytes;
+  int split_steps, qt_split, entries_per_bh;
+  long long items_max, split_max;   // capacities of the work list and of the list of split tiles (0 = no list)
+  size_t bias_total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes; }
+  size_t total() const { return bias_total() + sched_bytes + partial_bytes; }
 };
 
 WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
-  WorkspacePlan w = {0, 0, 0, 0, 0};
+  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const Variant var = pick_variant(a);
   if (var != V_MFMA_BF16 && var != V_MFMA_FP8) return w;
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
+  // Key-range splitting pays when there are fewer query tiles than the GPU runs at once (512
+  // workgroups) or little more: then the tile with most keys sets the run time.  With more tiles,
+  // taking the longest sequences first keeps the GPU busy behind it and the extra pass that sums
+  // the partials costs more than it saves.  The lengths are on the device, so the decision rests
+  // on what the shapes allow.
+  const int n_qtiles = (a->L + BM - 1) / BM;
+  const int steps_max = (a->L + BN - 1) / BN;
+  const bool jag = a->layout == HSTU_LAYOUT_JAGGED;
+  const long long tiles_est = (long long)a->H * (jag ? (a->total_tokens / BM + a->B) : (long long)a->B * n_qtiles);
+  w.entries_per_bh = n_qtiles;
+  if (tiles_est < 1024 && steps_max > 16) {
+    w.split_steps = (steps_max + MAX_CHUNKS - 1) / MAX_CHUNKS;
+    w.split_steps = w.split_steps < 16 ? 16 : w.split_steps;
+    // first tile with more steps than that (a causal tile qt has up to 4 (qt + 1) steps)
+    w.qt_split = a->causal ? w.split_steps / (BM / BN) : 0;
+    w.entries_per_bh = 0;
+    for (int qt = 0; qt < n_qtiles; ++qt) w.entries_per_bh += chunks_max(w.split_steps, a->causal != 0, a->L, qt);
+    const size_t slots = jag ? (size_t)(a->total_tokens / BM) + (size_t)a->B + 1 : (size_t)a->B * (size_t)(n_qtiles - w.qt_split);
+    w.partial_bytes = up(slots * (size_t)a->H * MAX_CHUNKS * (size_t)BM * (size_t)a->d_v * sizeof(float));
+  }
+  // A work list built on the device spares the launch of workgroups that would find nothing to do
+  // (a jagged batch with a long maximum length and mostly short sequences is mostly such).  Its
+  // head mapping needs H to divide 8 or 8 to divide H; its builder is one workgroup.
+  if ((a->H % 8 == 0 || 8 % a->H == 0) && a->B <= 8192) {
+    const long long t128 = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
+    // every tile one item, plus up to MAX_CHUNKS - 1 more for each tile that can be split
+    const long long extra = w.split_steps ? (MAX_CHUNKS - 1) * (jag ? a->total_tokens / BM + 1 + (w.qt_split ? 0 : a->B)
+                                                                          : (long long)a->B * (n_qtiles - w.qt_split)) : 0;
+    w.items_max = t128 + extra;
+    w.split_max = extra / (MAX_CHUNKS - 1);
+    w.sched_bytes = up((size_t)(4 + 4 * (w.items_max + w.split_max)) * sizeof(int32_t));
+  }
   if (a->pos_tab) w.pos_bytes = up((size_t)a->pos_heads * (size_t)(2 * a->L - 1 + 2 * POS_PAD) * sizeof(float));
   if (a->ts_tab) {
     const size_t tiles_per_seq = (size_t)((a->L + BN - 1) / BN);
@@ -1041,13 +1325,23 @@ int launch_general(const Params& p, hipStream_t st) {
   return HSTU_OK;
 }
 
+// Workgroups of the main kernel (and of the combine kernel, which shares its mapping).
+long long mfma_grid(const Params& p, bool split_list = false) {
+  if (p.sched) {
+    const long long n = split_list ? p.split_max : p.items_max;
+    const long long rounds = p.H >= 8 ? n * (p.H / 8) : (n + 8 / p.H - 1) / (8 / p.H);
+    return 8LL * rounds;
+  }
+  return 8LL * p.entries_per_bh * (((long long)p.B * p.H + 7) / 8);
+}
+
 template <int D, bool POS, bool TS, bool F8>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS);
   static int granted[64];
   if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8>, smem, granted)) return rc;
   hipError_t e;
-  const long long blocks = 8LL * p.n_qtiles * (((long long)p.B * p.H + 7) / 8);
+  const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
   hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();
@@ -1121,19 +1415,27 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
       const bool f8 = args->qk_dtype == HSTU_DTYPE_FP8_E4M3FN;
       const WorkspacePlan ws = plan_workspace(args);
       Params q = p;
+      q.split_steps = ws.split_steps;
+      q.qt_split = ws.qt_split;
+      q.entries_per_bh = ws.entries_per_bh;
       if (ws.total()) {
         if (!args->workspace || args->workspace_bytes < ws.total())
           return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes needed (see hstu_attn_fwd_workspace_bytes), got %zu",
                       ws.total(), args->workspace ? args->workspace_bytes : (size_t)0);
         if (((uintptr_t)args->workspace & 255u) != 0) return fail(HSTU_ERR_WORKSPACE, "workspace must be 256-byte aligned");
         char* base = (char*)args->workspace;
-        if (ws.total() >= (1ull << 32)) return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes is beyond what the kernel addresses", ws.total());
+        if (ws.bias_total() >= (1ull << 32)) return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes is beyond what the kernel addresses", ws.bias_total());
         float* pos_out = ws.pos_bytes ? (float*)base : nullptr;
         float* tab_out = ws.tab_bytes ? (float*)(base + ws.pos_bytes) : nullptr;
         int32_t* ok_out = ws.ok_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes) : nullptr;
         int32_t* rel_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes);
         int32_t* range_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes);
         q.ws_base = base;
+        int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
+        q.sched = sched_out;
+        q.items_max = ws.items_max;
+        q.split_max = ws.split_max;
+        q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
         q.ts_scaled = tab_out;
         q.pos_scaled = pos_out;
         q.ts_ok = ok_out;
@@ -1143,11 +1445,23 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
         const long long blocks_ts = ws.ok_bytes ? p.B : 0;
         long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
         blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
-        hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, p, pos_out, tab_out, ok_out, rel_out, range_out);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
+        if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
+        if (ws.bias_total() || ws.sched_bytes) {
+          hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out);
+          hipError_t e = hipGetLastError();
+          if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
+        }
       }
-      return f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st);
+      if (int rc2 = f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st)) return rc2;
+      const long long cb = q.split_steps > 0 ? mfma_grid(q, true) : 0;
+      if (cb > 0) {
+        if (q.d_v == 128) hipLaunchKernelGGL(hstu_combine<128>, dim3((unsigned)cb), dim3(MFMA_THREADS), 0, st, q);
+        else if (q.d_v == 64) hipLaunchKernelGGL(hstu_combine<64>, dim3((unsigned)cb), dim3(MFMA_THREADS), 0, st, q);
+        else hipLaunchKernelGGL(hstu_combine<32>, dim3((unsigned)cb), dim3(MFMA_THREADS), 0, st, q);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "combine kernel launch: %s", hipGetErrorString(e));
+      }
+      return HSTU_OK;
     }
     default: return fail(HSTU_ERR_SHAPE, "no kernel for these arguments");
   }

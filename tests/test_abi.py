@@ -87,14 +87,21 @@ def test_variant_and_workspace_query():
   a.alpha, a.inv_n, a.causal = 1.0, 1.0 / 256, 1
   a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
-  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 0
+  # the matrix-core kernel always wants a workspace: a work list of one int4 per query tile
+  # (2 sequences x 2 tiles here) behind a 16-byte header ...
+  up = lambda x: (x + 255) // 256 * 256
+  sched = up(16 + 16 * 2 * 2)
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == sched
+  # ... plus, with a position table, its scaled and padded copy
   a.pos_tab, a.pos_heads = 0x20000, 4
-  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == (4 * (2 * 256 - 1 + 512) * 4 + 255) // 256 * 256
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == up(4 * (2 * 256 - 1 + 512) * 4) + sched
+  # general-kernel calls need none
   # a launch without the workspace is refused before anything is enqueued
   assert lib.hstu_attn_fwd(C.byref(a), None) == -5
   a.pos_tab = None
   a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_FP32
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<float>"
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 0
   a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
   a.window = 4
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"

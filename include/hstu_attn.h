@@ -44,7 +44,9 @@ enum HstuLayout {
 enum HstuDtype {
   HSTU_DTYPE_FP32 = 0,
   HSTU_DTYPE_BF16 = 1,
-  HSTU_DTYPE_FP8_E4M3FN = 2 /* q and k only; scales in q_scale / k_scale     */
+  HSTU_DTYPE_FP8_E4M3FN = 2 /* q and k only (v, out bf16); per-head scales in
+                               q_scale / k_scale multiply the logits; not in
+                               the reference (its README lists fp8 as roadmap) */
 };
 
 /* Which positions take part, on top of causal / window / explicit mask. */
@@ -121,8 +123,8 @@ typedef struct HstuAttnFwdArgs {
   int32_t ts_num_buckets; /* clip bound; table has ts_num_buckets+1 entries   */
   float ts_bucket_size;   /* 0.301 in the reference                           */
 
-  const float* q_scale;   /* [H] dequantisation scales (fp8 q), else null     */
-  const float* k_scale;   /* [H] dequantisation scales (fp8 k), else null     */
+  const float* q_scale;   /* [H] dequantisation scales (fp8 q); null = 1      */
+  const float* k_scale;   /* [H] dequantisation scales (fp8 k); null = 1      */
 
   void* workspace;        /* device scratch of hstu_attn_fwd_workspace_bytes  */
   size_t workspace_bytes;
@@ -131,9 +133,17 @@ typedef struct HstuAttnFwdArgs {
 /* ABI version of the loaded library (HSTU_ATTN_ABI_VERSION at build time). */
 int hstu_attn_abi_version(void);
 
-/* Device scratch the call needs for these arguments (0 today for every
- * supported combination; callers must still query it).  No reference
- * counterpart: the reference's op is a pure function under jax.jit. */
+/* Bytes of device scratch the call needs for these arguments; pass a buffer of
+ * at least that size, 256-byte aligned, in args->workspace.  0 for calls the
+ * general kernel serves.  For the matrix-core kernel it holds what a small
+ * preparation kernel rebuilds on every call: the work list of (sequence,
+ * query tile) items, the scaled position and bucket tables, int32 timestamps
+ * with their per-tile ranges and, when few long sequences underfill the GPU,
+ * fp32 partial outputs of query tiles whose key range is split.  The size
+ * depends on shapes, options and total_tokens only, never on device data.
+ * The contents mean nothing between calls; two calls that overlap on one GPU
+ * need two buffers.  No reference counterpart: the reference's op is a pure
+ * function under jax.jit. */
 size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
 
 /* Validate `args` and enqueue the forward on `stream` (a hipStream_t passed

@@ -2,16 +2,22 @@
 //
 //   out[b,i,h,:] = sum_j M[b,i,j] * silu(alpha*q_i.k_j + bias(b,h,i,j)) * inv_n * v[b,j,h,:]
 //
-// Two kernels live here behind one C entry point (see include/hstu_attn.h):
+// Kernels behind the one C entry point (see include/hstu_attn.h):
 //
-//   hstu_fwd_mfma_bf16   the hot path.  bf16 Q/K/V, fp32 accumulation on the
-//                        32x32x16 bf16 MFMA, 128 query rows x 64 keys per
-//                        step, K/V double-buffered through LDS, relative
-//                        position and timestamp bias + SiLU + mask fused on
-//                        the accumulator registers, causal/length tile
-//                        skipping.  Computes S^T = K Q^T so that the
+//   hstu_fwd_mfma_bf16   the hot path.  bf16 (or fp8 e4m3fn) Q/K, bf16 V, fp32
+//                        accumulation on the 32x32x16 MFMA; 128 query rows per
+//                        workgroup, keys streamed 32 at a time through a
+//                        4-stage LDS ring filled by direct global->LDS loads;
+//                        relative-position and timestamp bias + SiLU + mask
+//                        fused on the accumulator registers; causal / length
+//                        tile skipping.  Computes S^T = K Q^T so that the
 //                        accumulator layout of S^T is already the B-operand
 //                        layout of O^T = V^T P^T: P never touches LDS.
+//   hstu_prepare         runs before it: work list of (sequence, tile) items,
+//                        longest sequences first; scaled bias tables; int32
+//                        timestamps and their per-tile ranges.
+//   hstu_combine         runs after it when query tiles were split over
+//                        several workgroups by key range: sums the partials.
 //   hstu_fwd_general     every option of the op (segment ids, explicit mask,
 //                        sliding window, dense bias, cross lengths, any head
 //                        dim <= 256, fp32 or bf16 storage) in plain fp32 FMA
@@ -762,11 +768,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // pieces w*LD .. w*LD+LD-1 of K and of V; lane l of piece j lands at chunk
   // 64j + l, i.e. row (64j+l)/CPR, physical chunk (64j+l)%CPR, and fetches the
   // logical chunk that the swizzle maps there.  Rows past the sequence re-read
-  // the last valid row (finite data; their logits are masked).  One more load
-  // per wave brings the bias operands: a shifted copy of the position window
-  // (waves 0-3, or 4-7 when there are no timestamps) or half of the 64 key
-  // timestamps (waves 4-5; the others repeat a load so that every wave issues
-  // the same number, which the vmcnt arithmetic relies on).
+  // the last valid row (finite data; their logits are masked).  Every wave
+  // issues the same number of loads per step: the vmcnt arithmetic relies on it.
   auto dma_step = [&](int t) {
     const int st = t % NSTAGE;
     const int kv0 = t * BN;
@@ -1387,17 +1390,6 @@ const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
     case V_MFMA_FP8: return "hstu_fwd_mfma_fp8";
     default: return "invalid";
   }
-}
-
-// Diagnostics: resident workgroups per CU of one MFMA kernel instantiation.
-int hstu_attn_debug_occupancy(int d, int pos, int ts) {
-  int n = -1;
-  hipError_t e = hipErrorInvalidValue;
-#define OCC(D_, P_, T_) if (d == D_ && !!pos == P_ && !!ts == T_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)hstu_fwd_mfma_bf16<D_, P_, T_, false>, MFMA_THREADS, MfmaSmem<D_, 2>::total(P_, T_));
-  OCC(128, false, false) OCC(128, true, false) OCC(128, false, true) OCC(128, true, true)
-  OCC(64, false, false) OCC(64, true, true) OCC(32, false, false) OCC(32, true, true)
-#undef OCC
-  return e == hipSuccess ? n : -(int)e;
 }
 
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {

@@ -56,6 +56,15 @@ enum HstuMaskMode {
   HSTU_MASK_SEGMENT = 2  /* q_segment_ids[b,i] == kv_segment_ids[b,j]         */
 };
 
+/* Bits of HstuAttnFwdArgs.flags. */
+enum HstuFwdFlags {
+  /* The workspace still holds what an earlier call prepared from the same
+   * shapes, lengths / offsets, timestamps and bias tables (for example the
+   * same call repeated, or a benchmark timing the main kernel alone): skip
+   * the preparation kernel.  Undefined results if that does not hold. */
+  HSTU_FWD_WORKSPACE_PREPARED = 1
+};
+
 /* Return codes (0 = launched). */
 enum HstuStatus {
   HSTU_OK = 0,
@@ -101,7 +110,7 @@ typedef struct HstuAttnFwdArgs {
   int32_t causal;         /* 1: keep j <= i                                   */
   int32_t mask_mode;      /* HstuMaskMode                                     */
   int32_t window;         /* keep |i-j| <= window; < 0 disables               */
-  int32_t reserved0;
+  int32_t flags;          /* HstuFwdFlags, 0 by default                       */
 
   const int32_t* seq_lens;     /* [B], LENGTH mode with the padded layout     */
   const int32_t* seq_offsets;  /* [B+1], jagged layout                        */

@@ -13,6 +13,7 @@ ABI_VERSION = 1
 
 LAYOUT_PADDED, LAYOUT_JAGGED = 0, 1
 DTYPE_FP32, DTYPE_BF16, DTYPE_FP8_E4M3FN = 0, 1, 2
+FWD_WORKSPACE_PREPARED = 1
 MASK_NONE, MASK_LENGTH, MASK_SEGMENT = 0, 1, 2
 
 EXPORTS = (
@@ -42,7 +43,7 @@ class HstuAttnFwdArgs(C.Structure):
       ("o_stride_b", C.c_int64), ("o_stride_t", C.c_int64), ("o_stride_h", C.c_int64),
       ("alpha", C.c_float), ("inv_n", C.c_float),
       ("causal", C.c_int32), ("mask_mode", C.c_int32),
-      ("window", C.c_int32), ("reserved0", C.c_int32),
+      ("window", C.c_int32), ("flags", C.c_int32),
       ("seq_lens", C.c_void_p), ("seq_offsets", C.c_void_p),
       ("q_segment_ids", C.c_void_p), ("kv_segment_ids", C.c_void_p),
       ("mask", C.c_void_p),

@@ -1438,7 +1438,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
         long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
         blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
         if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
-        if (ws.bias_total() || ws.sched_bytes) {
+        if ((ws.bias_total() || ws.sched_bytes) && !(args->flags & HSTU_FWD_WORKSPACE_PREPARED)) {
           hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out);
           hipError_t e = hipGetLastError();
           if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));

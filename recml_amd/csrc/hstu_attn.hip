@@ -1040,10 +1040,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       dst[i * 64] = floatx4{o[i >> 2][4 * (i & 3) + 0], o[i >> 2][4 * (i & 3) + 1], o[i >> 2][4 * (i & 3) + 2], o[i >> 2][4 * (i & 3) + 3]};
     return;
   }
+  // Each wave turns its O^T fragment into whole output rows through LDS (the ring is free now: the
+  // loop ended on a barrier and no load is in flight), so that global memory sees 16-byte stores that
+  // cover full rows instead of 8-byte pieces: lane (row m, half hh) writes 8 bytes of row m at a
+  // time, 16-byte chunks XOR-swizzled by row against bank conflicts, then reads 16 bytes per lane,
+  // 64 / (D/8) rows per instruction.  Only lanes of the same wave exchange data here and LDS
+  // executes a wave's operations in order: no barrier is needed.
   const float oscale = p.inv_n * (1.0f / LOG2E);
-  if (qrow < s.rows) {
+  unsigned char* ot = smem + w * (32 * D * 2);
+  auto oswz = [](int row) { return (row / SM::RPB) % CPR; };
+  {
     const bool live = qrow < s.n_q;
-    bf16_t* orow = og + (int64_t)qrow * p.o_st + 4 * hh;
+    unsigned char* orow = ot + m * (D * 2) + 8 * hh;
 #pragma unroll
     for (int dvb = 0; dvb < DVB; ++dvb) {
 #pragma unroll
@@ -1053,9 +1061,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
           pko.x = pack_bf16(o[dvb][4 * g + 0] * oscale, o[dvb][4 * g + 1] * oscale);
           pko.y = pack_bf16(o[dvb][4 * g + 2] * oscale, o[dvb][4 * g + 3] * oscale);
         }
-        *(uint2*)(orow + 32 * dvb + 8 * g) = pko;
+        *(uint2*)(orow + (((4 * dvb + g) ^ oswz(m)) * 16)) = pko;
       }
     }
+  }
+  constexpr int ROWS_PER_STORE = 64 / CPR;
+  const int rr = lane / CPR, cc = lane - rr * CPR;
+#pragma unroll
+  for (int r0s = 0; r0s < 32; r0s += ROWS_PER_STORE) {
+    const int row = r0s + rr;
+    const uint4 val = *(const uint4*)(ot + row * (D * 2) + ((cc ^ oswz(row)) * 16));
+    const int grow = r0 + row;
+    if (grow < s.rows) *(uint4*)(og + (int64_t)grow * p.o_st + cc * 8) = val;
   }
 }
 

@@ -124,6 +124,26 @@ def near_bucket_boundary(delta, bucket_size: float = 0.301, ulps: float = 8.0):
   return (dist <= tol) & (np.rint(y) >= 1)
 
 
+def rows_near_bucket_boundary(timestamps, seq_offsets, causal: bool = True, bucket_size: float = 0.301):
+  """Jagged timestamps [T] -> bool [T]: rows whose time delta to one of their (causal) keys is
+  a boundary case of the bucket law (near_bucket_boundary).  On such a row an fp32 evaluation
+  of the law may land in the neighbouring bucket (parity unpinned there), so checkers compare
+  those rows with a looser bound."""
+  ts = np.asarray(timestamps).astype(np.int64)
+  off = np.asarray(seq_offsets).astype(np.int64)
+  flag = np.zeros(ts.shape[0], dtype=bool)
+  for b in range(len(off) - 1):
+    t = ts[off[b]:off[b + 1]]
+    if t.size == 0:
+      continue
+    d = time_delta(t[None])[0]
+    near = near_bucket_boundary(d, bucket_size)
+    if causal:
+      near &= np.tril(np.ones_like(near, dtype=bool))
+    flag[off[b]:off[b + 1]] = near.any(axis=1)
+  return flag
+
+
 def rel_pos_bias_recipe(w, n: int):
   """The pad/tile/reshape/slice recipe of recml/layers/keras/hstu.py:105-113.
 

@@ -320,3 +320,13 @@ def test_e4m3fn_rounding_against_torch_cast():
   assert (got == want).all()
   q, scale = O.quantize_e4m3fn_per_head(rng.standard_normal((5, 7, 3, 16)).astype(np.float32))
   assert scale.shape == (3,) and np.abs(q).max() == 448.0 and (O.round_e4m3fn(q) == q).all()
+
+
+def test_rows_near_bucket_boundary():
+  # ln(15245) / 0.301 = 32.0000004: a boundary case of the law in fp32; 15000 is not
+  assert O.near_bucket_boundary(np.array([15245]))[0] and not O.near_bucket_boundary(np.array([15000]))[0]
+  # sequence 0: row 0's next timestamp is 15245 after key 0; sequence 1: nowhere near a boundary
+  ts = np.array([1000, 1000 + 15245, 1000 + 15245 + 7, 5000, 5003, 5010], dtype=np.int64)
+  off = np.array([0, 3, 6])
+  flag = O.rows_near_bucket_boundary(ts, off)
+  assert flag.tolist()[0] is True and not flag[3:].any()

@@ -170,11 +170,14 @@ def test_few_long_sequences(gpu, layout):
   lens = np.array([1100, 513, 40], dtype=np.int32)
   q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.2) for _ in range(3))
   pos = rng.standard_normal((H, 2 * L - 1)).astype(np.float32) * 0.1
-  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, pos_tab=pos, dtype=np.float32)
+  ts = 1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, (B, L))), axis=1).astype(np.int64)
+  tab = (rng.standard_normal((H, 129)) * 0.1).astype(np.float32)
+  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, pos_tab=pos, timestamps=ts, ts_tab=tab, dtype=np.float32)
   for rep in range(2):
     if layout == "padded":
       out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
-                                     seq_lens=_dev(lens), pos_bias=_dev(pos)).float().cpu().numpy()
+                                     seq_lens=_dev(lens), pos_bias=_dev(pos), timestamps=_dev(ts),
+                                     ts_bias=_dev(tab)).float().cpu().numpy()
       for b in range(B):
         assert (out[b, lens[b]:] == 0).all()
     else:
@@ -182,13 +185,48 @@ def test_few_long_sequences(gpu, layout):
       kj, _ = O.padded_to_jagged(k, lens)
       vj, _ = O.padded_to_jagged(v, lens)
       outj = recml_amd.hstu_attention(_dev(qj, torch.bfloat16), _dev(kj, torch.bfloat16), _dev(vj, torch.bfloat16),
-                                      seq_offsets=_dev(off.astype(np.int32)), max_len=L, pos_bias=_dev(pos))
+                                      seq_offsets=_dev(off.astype(np.int32)), max_len=L, pos_bias=_dev(pos),
+                                      timestamps=_dev(ts), ts_bias=_dev(tab))
       out = O.jagged_to_padded(outj.float().cpu().numpy(), off, L)
     assert _err(out, ref) <= BF16_TOL
   # full (non-causal) mask through the same path
   out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
                                  seq_lens=_dev(lens), causal=False).float().cpu().numpy()
   assert _err(out, O.hstu_attention_ref(q, k, v, seq_lens=lens, causal=False, dtype=np.float32)) <= BF16_TOL
+
+
+@pytest.mark.parametrize("B,L,H,d,layout", [
+    (5, 200, 1, 64, "jagged"),      # one head: eight work items share a round of XCDs
+    (2, 700, 3, 64, "padded"),      # 3 heads: no work list (static enumeration), key ranges split
+    (2, 700, 3, 64, "jagged"),
+    (3, 300, 12, 32, "jagged"),     # 12 heads: static enumeration, no split
+    (4, 260, 16, 32, "padded"),     # 16 heads: two rounds of XCDs per item
+    (1100, 40, 2, 32, "jagged"),    # more sequences than the list builder sorts
+    (8200, 33, 1, 32, "padded"),    # more sequences than the list builder takes: static enumeration
+])
+def test_block_mappings(gpu, B, L, H, d, layout):
+  rng = np.random.default_rng(B * 7 + H)
+  lens = rng.integers(1, L + 1, B).astype(np.int32)
+  lens[0] = L
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.1).astype(np.float32)
+  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, pos_tab=pos, dtype=np.float32)
+  if layout == "padded":
+    out = recml_amd.hstu_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
+                                   seq_lens=_dev(lens), pos_bias=_dev(pos)).float().cpu().numpy()
+  else:
+    qj, off = O.padded_to_jagged(q, lens)
+    kj, _ = O.padded_to_jagged(k, lens)
+    vj, _ = O.padded_to_jagged(v, lens)
+    a, keep = hstu_ops.build_args(_dev(qj, torch.bfloat16), _dev(kj, torch.bfloat16), _dev(vj, torch.bfloat16),
+                                  torch.empty((qj.shape[0], H, d), dtype=torch.bfloat16, device="cuda:0"),
+                                  seq_offsets=_dev(off.astype(np.int32)), max_len=L, pos_bias=_dev(pos))
+    assert hstu_ops.kernel_variant(a) == "hstu_fwd_mfma_bf16"
+    hstu_ops._run(a, keep)
+    out = O.jagged_to_padded(keep[3].float().cpu().numpy(), off, L)
+  assert _err(out, ref) <= BF16_TOL
+  for b in range(min(B, 50)):
+    assert (out[b, lens[b]:] == 0).all()
 
 
 def test_ragged_and_empty(gpu):

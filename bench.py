@@ -135,6 +135,73 @@ def measured_traffic(workload):
   return None if rec is None else rec["hbm_bytes_per_launch"]
 
 
+PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32
+
+
+def bench_backward(args, w, q, k, v, kw, dev):
+  """The backward pass (general fp32-arithmetic kernels) on the same workload: one JSON line.
+
+  FLOPs counted: four products per unmasked pair (dV, dP, dQ, dK) = 2x the forward's; the
+  recomputation of S in both kernels is not counted."""
+  import torch
+  import recml_amd
+  from oracle import hstu_oracle as O
+  dout = torch.randn(v.shape, generator=torch.Generator().manual_seed(1)).to(dev).to(v.dtype)
+  run = lambda: recml_amd.hstu_attention_bwd(q, k, v, dout, **kw)
+  steps, warm = max(1, args.steps // 10), max(1, args.warmup // 10)
+  for _ in range(warm):
+    got = run()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(steps):
+    got = run()
+  torch.cuda.synchronize()
+  ms = (time.perf_counter() - t0) * 1e3 / steps
+  flops = 2 * w.flops
+  rec = {
+      "metric": "HSTU attn bwd TFLOP/s (unmasked), L=%d bf16" % w.L, "value": flops / (ms * 1e-3) / 1e12,
+      "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, fp32 arithmetic",
+      "data": "synthetic", "config": {"workload": w.name + " backward", "kernel": "hstu_bwd_dq + hstu_bwd_dkv"},
+      "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                   "frac": flops / (ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, "traffic": None,
+                   "note": "fp32 FMA kernels (no matrix cores yet); time covers both kernels, the table memsets and the host call"},
+  }
+  if not args.no_cpu and w.layout == "jagged":
+    # bounded sample: the numpy oracle on the shortest sequences that add up to ~5 % of the pairs
+    off = w.seq_offsets
+    order = np.argsort(w.seq_lens)
+    take, pairs = [], 0
+    total_pairs = int((w.seq_lens.astype(np.int64) ** 2).sum())
+    for b in order:
+      take.append(int(b))
+      pairs += int(w.seq_lens[b]) ** 2
+      if pairs > 0.05 * total_pairs:
+        break
+    qf, kf, vf, df = (x.float().cpu().numpy() for x in (q, k, v, dout))
+    t0 = time.perf_counter()
+    worst = 0.0
+    fl = 0
+    for b in take:
+      sl = slice(int(off[b]), int(off[b + 1]))
+      n = sl.stop - sl.start
+      tsb = None if w.timestamps is None else w.timestamps[sl][None]
+      ref = O.hstu_attention_bwd_ref(qf[sl][None], kf[sl][None], vf[sl][None], df[sl][None], n=w.n, alpha=w.alpha,
+                                     pos_tab=None if w.pos_tab is None else w.pos_tab[:, w.L - n: w.L + n - 1],
+                                     timestamps=tsb, ts_tab=w.ts_tab, dtype=np.float32)
+      fl += 2 * w.H * (n * (n + 1) // 2) * 4 * w.d
+      for g, r in zip(got[:3], ref[:3]):
+        worst = max(worst, float(np.abs(g[sl].float().cpu().numpy() - r[0]).max() / max(np.abs(r).max(), 1e-30)))
+    dt = time.perf_counter() - t0
+    rec["cpu_baseline"] = {"value": fl / dt / 1e12, "unit": "TFLOP/s", "cores": os.cpu_count(), "kind": "port",
+                           "sample": f"numpy fp32 dense backward on the {len(take)} shortest sequences "
+                                     f"({fl / 1e9:.2f} GFLOP of unmasked work), {dt:.1f} s"}
+    rec["parity_max_abs_over_max_ref"] = worst
+    if not worst <= 2e-2:
+      raise SystemExit(f"backward parity failed in the benchmark run: {worst}")
+  print(json.dumps(rec))
+
+
 def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--gpus", type=int, default=1)
@@ -144,6 +211,7 @@ def main():
   ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
   ap.add_argument("--no-cold", dest="cold", action="store_false",
                   help="skip the cold-cache variant (a 1 GiB fill between launches)")
+  ap.add_argument("--backward", action="store_true", help="measure the backward pass instead of the forward")
   ap.add_argument("--calib-copy", action="store_true",
                   help="also run one 512 MiB device copy (reference point for HBM byte counters)")
   args = ap.parse_args()
@@ -160,6 +228,10 @@ def main():
   dev = torch.device("cuda:0")
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
+  if args.backward:
+    if w.dtype == "fp8":
+      raise SystemExit("the backward takes fp32 or bf16 storage")
+    return bench_backward(args, w, q, k, v, kw, dev)
   out = torch.empty_like(v)
   call_args, keep = hstu_ops.build_args(q, k, v, out, **kw)
   variant = hstu_ops.kernel_variant(call_args)

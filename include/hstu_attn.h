@@ -161,6 +161,32 @@ size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
  * recml/layers/keras/hstu.py:356-390. */
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
 
+/* Backward of the same op: gradients of sum(out * dout) with respect to q, k, v
+ * and the two bias tables.  `fwd` describes the forward call (its `out` and
+ * `workspace` are not used).  dout has the layout, dtype and strides of out;
+ * dq, dk, dv those of q, k, v and are fully written (rows past a sequence's
+ * length as zeros).  dpos_tab / dts_tab are fp32 tables shaped like pos_tab /
+ * ts_tab that are ACCUMULATED into by atomic adds: the caller zero-fills them
+ * (or passes null when the table gradient is not wanted).  fp32 or bf16
+ * storage, every option of the forward, fp32 arithmetic; fp8 q/k is not
+ * supported.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which
+ * the reference reaches through jax.custom_vjp (hstu_ops.py:551-826), extended
+ * by the table gradients that jax derives for recml/layers/keras/hstu.py:91-113,
+ * 190-221. */
+typedef struct HstuAttnBwdArgs {
+  uint32_t struct_size;   /* sizeof(HstuAttnBwdArgs)                          */
+  uint32_t version;       /* HSTU_ATTN_ABI_VERSION                            */
+  HstuAttnFwdArgs fwd;
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  float* dpos_tab;
+  float* dts_tab;
+} HstuAttnBwdArgs;
+
+int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream);
+
 /* Message for the last non-zero status on this thread ("" if none). */
 const char* hstu_attn_last_error(void);
 

@@ -18,6 +18,7 @@ reference checkout):
   pw_attn_ref                   recml/core/ops/hstu_ops_test.py:44-58
   splash_mask                   recml/core/ops/hstu_ops.py:926-945, 107-194
   hstu_attention_ref            the union of the above behind one signature
+  hstu_attention_bwd_ref        its gradients; math of recml/core/ops/hstu_ops.py:461-517
 
 How each function is pinned (tests/test_oracle.py):
 
@@ -32,6 +33,9 @@ How each function is pinned (tests/test_oracle.py):
                                 single-key closed form, the zero-Q Toeplitz
                                 case, SiLU special values, causality and
                                 padding invariants, linearity in 1/N.
+  hstu_attention_bwd_ref        central finite differences of the pinned forward
+                                in fp64 (every input and both tables), on tiny
+                                inputs with every option.
   round_e4m3fn / encode_e4m3fn  torch's CPU float8_e4m3fn cast on every code
                                 point, every midpoint and random values (fp8
                                 is not in the reference at all).
@@ -361,6 +365,75 @@ def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
   p = np.where(m[:, None], p, np.zeros_like(p))
   # Keys beyond the sequence never contribute, whatever the padding holds.
   return np.einsum("bhts,bshd->bthd", p, v)
+
+
+def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
+                           causal=True, pos_tab=None, timestamps=None,
+                           ts_tab=None, ts_bucket_size=0.301, bucket_law=False,
+                           q_segment_ids=None, kv_segment_ids=None,
+                           sliding_window_size=None, mask=None, bias=None,
+                           dtype=np.float64):
+  """Gradients of sum(out * dout) for hstu_attention_ref, dense, on padded inputs.
+
+  The math of the reference's backward kernel (recml/core/ops/hstu_ops.py:461-517):
+    dV = P^T dO;  dP = dO V^T;  dS = dP * sigma(S) (1 + S (1 - sigma(S))) / n  (masked);
+    dQ = alpha dS K;  dK = alpha dS^T Q
+  extended by the bias terms of the forward: every (i, j) adds dS to the table entry it
+  read (position entry (L-1)+j-i, timestamp entry bucket(i, j)), summed over heads when
+  the table has one row for all heads.  Returns dq, dk, dv, dpos_tab (or None),
+  dts_tab (or None) with the shapes of the inputs.
+  """
+  q = np.asarray(q, dtype=dtype)
+  k = np.asarray(k, dtype=dtype)
+  v = np.asarray(v, dtype=dtype)
+  dout = np.asarray(dout, dtype=dtype)
+  B, L, H, _ = q.shape
+  Lkv = k.shape[1]
+  n = L if n is None else n
+  s = alpha * np.einsum("bthd,bshd->bhts", q, k)
+  tb = _bias_term(L, Lkv, H, pos_tab, timestamps, ts_tab, ts_bucket_size, bucket_law)
+  if tb is not None:
+    s = s + tb.astype(dtype)
+  if bias is not None:
+    s = s + np.asarray(bias, dtype=dtype)[:, None]
+  m = splash_mask(L, Lkv, causal=causal,
+                  explicit=None if (mask is None or np.ndim(mask) == 3) else mask,
+                  sliding_window_size=sliding_window_size,
+                  q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids)
+  if mask is not None and np.ndim(mask) == 3:
+    m = m & np.asarray(mask).astype(bool)
+  if seq_lens is not None:
+    lens = np.asarray(seq_lens)
+    vq = np.arange(L)[None, :] < lens[:, None]
+    vk = np.arange(Lkv)[None, :] < lens[:, None]
+    m = m & (vq[:, :, None] & vk[:, None, :])
+  m = np.broadcast_to(m, (B, L, Lkv))[:, None]
+  sg = 1.0 / (1.0 + np.exp(-s))
+  p = np.where(m, s * sg / n, 0.0)
+  dv = np.einsum("bhts,bthd->bshd", p, dout)
+  dp = np.einsum("bthd,bshd->bhts", dout, v)
+  ds = np.where(m, dp * sg * (1.0 + s * (1.0 - sg)) / n, 0.0)
+  dq = alpha * np.einsum("bhts,bshd->bthd", ds, k)
+  dk = alpha * np.einsum("bhts,bthd->bshd", ds, q)
+  dpos = dts = None
+  if pos_tab is not None:
+    pt = np.atleast_2d(np.asarray(pos_tab))
+    dpos = np.zeros(pt.shape, dtype=dtype)
+    idx = (L - 1) + np.arange(Lkv)[None, :] - np.arange(L)[:, None]          # [L, Lkv]
+    per_head = ds.sum(axis=0)                                                  # [H, L, Lkv]
+    for h in range(H):
+      np.add.at(dpos[h if pt.shape[0] > 1 else 0], idx, per_head[h])
+    dpos = dpos.reshape(np.asarray(pos_tab).shape)
+  if ts_tab is not None:
+    tt = np.atleast_2d(np.asarray(ts_tab))
+    nb = tt.shape[1] - 1
+    dts = np.zeros(tt.shape, dtype=dtype)
+    fn = bucketize_law if bucket_law else default_bucketization
+    bucket = np.clip(fn(time_delta(timestamps), ts_bucket_size), 0, nb)
+    for h in range(H):
+      np.add.at(dts[h if tt.shape[0] > 1 else 0], bucket, ds[:, h])
+    dts = dts.reshape(np.asarray(ts_tab).shape)
+  return dq, dk, dv, dpos, dts
 
 
 def hstu_attention_bruteforce(q, k, v, *, seq_lens=None, n=None, alpha=1.0,

@@ -9,6 +9,8 @@ HSTU block and model forward (recml/layers/keras/hstu.py:240-621).
 from recml_amd.hstu_ops import (  # noqa: F401
     MaskType,
     hstu_attention,
+    hstu_attention_autograd,
+    hstu_attention_bwd,
     pointwise_attention,
     pointwise_splash_attention,
 )

@@ -22,6 +22,7 @@ EXPORTS = (
     "hstu_attn_fwd",
     "hstu_attn_last_error",
     "hstu_attn_fwd_variant",
+    "hstu_attn_bwd",
 )
 
 
@@ -59,6 +60,17 @@ class HstuAttnFwdArgs(C.Structure):
   ]
 
 
+class HstuAttnBwdArgs(C.Structure):
+  """Field-for-field image of `struct HstuAttnBwdArgs`."""
+
+  _fields_ = [
+      ("struct_size", C.c_uint32), ("version", C.c_uint32),
+      ("fwd", HstuAttnFwdArgs),
+      ("dout", C.c_void_p), ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
+      ("dpos_tab", C.c_void_p), ("dts_tab", C.c_void_p),
+  ]
+
+
 _lock = threading.Lock()
 _lib = None
 
@@ -89,6 +101,8 @@ def load():
     lib.hstu_attn_last_error.argtypes = []
     lib.hstu_attn_fwd_variant.restype = C.c_char_p
     lib.hstu_attn_fwd_variant.argtypes = [C.POINTER(HstuAttnFwdArgs)]
+    lib.hstu_attn_bwd.restype = C.c_int
+    lib.hstu_attn_bwd.argtypes = [C.POINTER(HstuAttnBwdArgs), C.c_void_p]
     ver = lib.hstu_attn_abi_version()
     if ver != ABI_VERSION:
       raise RuntimeError(f"libhstu_attn.so has ABI {ver}, expected {ABI_VERSION}")

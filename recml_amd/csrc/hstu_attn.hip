@@ -98,6 +98,14 @@ struct Params {
   // sched[4] on one int4 per (sequence, query tile, chunk) that has work:
   // {b, qt | chunk << 16, first token, stored length}.
   const int32_t* sched;
+  // backward pass: gradient of out in, gradients of q, k, v out (layouts of out, q, k, v), and
+  // fp32 table gradients that are accumulated into (null = not wanted)
+  const void* dout;
+  void* dq;
+  void* dk;
+  void* dv;
+  float* dpos;
+  float* dts;
   int64_t items_max;         // capacity of the list (sizes the grid)
   int64_t split_max;         // capacity of the list of split tiles behind it: sched[1] int4s at sched + 4 + 4 items_max
 };
@@ -174,7 +182,7 @@ constexpr int GT = 32;       // query rows and keys per tile
 constexpr int GMAXX = 32;    // d_v / 8 accumulators per thread, d_v <= 256
 
 __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
-                                              int b, int h, int i, int j) {
+                                              int b, int h, int i, int j, int* bucket = nullptr) {
   float bias = 0.f;
   if (p.pos_tab) {
     int hh = p.pos_heads > 1 ? h : 0;
@@ -191,6 +199,7 @@ __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
     float lg = logf((float)dt) / p.ts_bucket_size;
     int bk = (int)lg;
     bk = bk < 0 ? 0 : (bk > p.ts_nb ? p.ts_nb : bk);
+    if (bucket) *bucket = bk;
     int hh = p.ts_heads > 1 ? h : 0;
     bias += p.ts_tab[(int64_t)hh * (p.ts_nb + 1) + bk];
   }
@@ -315,6 +324,270 @@ __global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
         int c = ocg + 8 * x;
         if (c < dv) stf(op + s.bo + (int64_t)i * p.o_st + c, live ? acc[x] * p.inv_n : 0.f);
       }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Backward, general form (fp32 FMA arithmetic, every option of the forward):
+//   P = silu(S)/N masked, dV = P^T dO, dP = dO V^T,
+//   dS = dP sigma(S) (1 + S (1 - sigma(S))) / N masked, dQ = alpha dS K, dK = alpha dS^T Q,
+// and every (i, j) adds dS to the table entries its logit read
+// (recml/core/ops/hstu_ops.py:461-517 for q, k, v).  S is recomputed in both kernels.
+// ---------------------------------------------------------------------------
+
+// logit x, keep flag and timestamp bucket of pair (i, j); returns dS given dP, and P through *pout
+__device__ __forceinline__ float bwd_pair(const Params& p, const Seq& s, int b, int h, int i, int j,
+                                          float qk, float dp, float* pout, int* bucket) {
+  *pout = 0.f;
+  if (!general_keep(p, s, b, i, j)) return 0.f;
+  const float x = p.alpha * qk + general_bias(p, s, b, h, i, j, bucket);
+  const float sg = 1.0f / (1.0f + expf(-x));
+  *pout = x * sg * p.inv_n;
+  return dp * sg * (1.0f + x * (1.0f - sg)) * p.inv_n;
+}
+
+// dQ and the table gradients: one workgroup per 32 query rows of one (sequence, head), keys streamed
+template <typename T>
+__global__ __launch_bounds__(256) void hstu_bwd_dq(const Params p) {
+  extern __shared__ float gsm[];
+  const int dq = p.d_qk, dv = p.d_v;
+  const int kp = dq + 1, vp_ = dv + 1;     // odd pitches: one row per lane reads
+  float* Qs = gsm;                         // [GT][dq]
+  float* Os = Qs + GT * dq;                // [GT][dv]   dO rows
+  float* Ks = Os + GT * dv;                // [GT][kp]
+  float* Vs = Ks + GT * kp;                // [GT][vp_]
+  float* Ds = Vs + GT * vp_;               // [GT][GT+1] dS
+  float* Hist = Ds + GT * (GT + 1);        // [ts_nb + 1] timestamp-bucket sums of this tile
+  int* Bk = (int*)(Hist + 132);            // [GT][GT] bucket of each pair
+
+  const int qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const Seq s = seq_info(p, b, h);
+  const int q0 = qt * GT;
+  if (q0 >= s.rows) return;
+  const int tid = threadIdx.x;
+  const T* __restrict__ qp = (const T*)p.q;
+  const T* __restrict__ kp_ = (const T*)p.k;
+  const T* __restrict__ vp = (const T*)p.v;
+  const T* __restrict__ dop = (const T*)p.dout;
+  T* __restrict__ dqp = (T*)p.dq;
+  const bool want_ts = p.dts != nullptr && p.ts_tab != nullptr;
+  const bool want_pos = p.dpos != nullptr && p.pos_tab != nullptr;
+
+  const int oi = tid >> 3, ocg = tid & 7;
+  const int nx = (dq + 7) >> 3;
+  float acc[GMAXX];
+#pragma unroll
+  for (int x = 0; x < GMAXX; ++x) acc[x] = 0.f;
+
+  if (q0 < s.n_q) {
+    for (int e = tid; e < GT * dq; e += 256) {
+      int r = e / dq, c = e - r * dq, i = q0 + r;
+      Qs[e] = (i < s.n_q) ? ldf(qp + s.bq + (int64_t)i * p.q_st + c) : 0.f;
+    }
+    for (int e = tid; e < GT * dv; e += 256) {
+      int r = e / dv, c = e - r * dv, i = q0 + r;
+      Os[e] = (i < s.n_q) ? ldf(dop + s.bo + (int64_t)i * p.o_st + c) : 0.f;
+    }
+    if (want_ts) for (int e = tid; e <= p.ts_nb; e += 256) Hist[e] = 0.f;
+    int kv_end = s.n_kv;
+    if (p.causal && q0 + GT < kv_end) kv_end = q0 + GT;
+    if (p.window >= 0 && q0 + GT + p.window < kv_end) kv_end = q0 + GT + p.window;
+    int kv_begin = 0;
+    if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
+
+    for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
+      __syncthreads();
+      for (int e = tid; e < GT * dq; e += 256) {
+        int r = e / dq, c = e - r * dq, j = kv0 + r;
+        Ks[r * kp + c] = (j < s.n_kv) ? ldf(kp_ + s.bk + (int64_t)j * p.k_st + c) : 0.f;
+      }
+      for (int e = tid; e < GT * dv; e += 256) {
+        int r = e / dv, c = e - r * dv, j = kv0 + r;
+        Vs[r * vp_ + c] = (j < s.n_kv) ? ldf(vp + s.bv + (int64_t)j * p.v_st + c) : 0.f;
+      }
+      __syncthreads();
+      {
+        const int tx = tid & 31, ty = tid >> 5;
+        float sacc[4] = {0.f, 0.f, 0.f, 0.f}, pacc[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* krow = Ks + tx * kp;
+        for (int c = 0; c < dq; ++c) {
+          const float kvv = krow[c];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sacc[r] = fmaf(Qs[(ty + 8 * r) * dq + c], kvv, sacc[r]);
+        }
+        const float* vrow = Vs + tx * vp_;
+        for (int c = 0; c < dv; ++c) {
+          const float vv = vrow[c];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) pacc[r] = fmaf(Os[(ty + 8 * r) * dv + c], vv, pacc[r]);
+        }
+        const int j = kv0 + tx;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = q0 + ty + 8 * r;
+          float pval;
+          int bk = 0;
+          const float ds = bwd_pair(p, s, b, h, i, j, sacc[r], pacc[r], &pval, &bk);
+          Ds[(ty + 8 * r) * (GT + 1) + tx] = ds;
+          if (want_ts) Bk[(ty + 8 * r) * GT + tx] = bk;
+        }
+      }
+      __syncthreads();
+      // table gradients of this tile: one sum per diagonal (position), one LDS histogram (time)
+      if (want_pos && tid < 2 * GT - 1) {
+        const int dd = tid - (GT - 1);           // j - i inside the tile
+        float sum = 0.f;
+        for (int r = 0; r < GT; ++r) {
+          const int c = r + dd;
+          if (c >= 0 && c < GT) sum += Ds[r * (GT + 1) + c];
+        }
+        const int idx = (p.L - 1) + (kv0 - q0) + dd;
+        if (sum != 0.f && idx >= 0 && idx < 2 * p.L - 1)
+          atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, sum);
+      }
+      if (want_ts) {
+        for (int e = tid; e < GT * GT; e += 256) {
+          const float ds = Ds[(e >> 5) * (GT + 1) + (e & 31)];
+          if (ds != 0.f) atomicAdd(Hist + Bk[e], ds);
+        }
+      }
+      for (int jj = 0; jj < GT; ++jj) {
+        const float ds = Ds[oi * (GT + 1) + jj];
+        const float* krow = Ks + jj * kp;
+#pragma unroll
+        for (int x = 0; x < GMAXX; ++x) {
+          if (x < nx) {
+            const int c = ocg + 8 * x;
+            if (c < dq) acc[x] = fmaf(ds, krow[c], acc[x]);
+          }
+        }
+      }
+    }
+    if (want_ts) {
+      __syncthreads();
+      for (int e = tid; e <= p.ts_nb; e += 256)
+        if (Hist[e] != 0.f) atomicAdd(p.dts + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1) + e, Hist[e]);
+    }
+  }
+  const int i = q0 + oi;
+  if (i < s.rows) {
+    const bool live = i < s.n_q;
+#pragma unroll
+    for (int x = 0; x < GMAXX; ++x) {
+      if (x < nx) {
+        const int c = ocg + 8 * x;
+        if (c < dq) stf(dqp + s.bq + (int64_t)i * p.q_st + c, live ? acc[x] * p.alpha : 0.f);
+      }
+    }
+  }
+}
+
+// dK and dV: one workgroup per 32 keys of one (sequence, head), query rows streamed
+template <typename T>
+__global__ __launch_bounds__(256) void hstu_bwd_dkv(const Params p) {
+  extern __shared__ float gsm[];
+  const int dq = p.d_qk, dv = p.d_v;
+  const int kp = dq + 1, vp_ = dv + 1;
+  float* Ks = gsm;                         // [GT][kp]
+  float* Vs = Ks + GT * kp;                // [GT][vp_]
+  float* Qs = Vs + GT * vp_;               // [GT][dq]
+  float* Os = Qs + GT * dq;                // [GT][dv]
+  float* Ds = Os + GT * dv;                // [GT][GT+1] dS   [row][key]
+  float* Ps = Ds + GT * (GT + 1);          // [GT][GT+1] P
+
+  const int kt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const Seq s = seq_info(p, b, h);
+  const int kv0 = kt * GT;
+  const int krows = p.jagged ? s.n_kv : p.Lkv;      // rows of dk / dv that exist
+  if (kv0 >= krows) return;
+  const int tid = threadIdx.x;
+  const T* __restrict__ qp = (const T*)p.q;
+  const T* __restrict__ kp_ = (const T*)p.k;
+  const T* __restrict__ vp = (const T*)p.v;
+  const T* __restrict__ dop = (const T*)p.dout;
+  T* __restrict__ dkp = (T*)p.dk;
+  T* __restrict__ dvp = (T*)p.dv;
+
+  const int oj = tid >> 3, ocg = tid & 7;
+  const int nxk = (dq + 7) >> 3, nxv = (dv + 7) >> 3;
+  float acck[GMAXX], accv[GMAXX];
+#pragma unroll
+  for (int x = 0; x < GMAXX; ++x) { acck[x] = 0.f; accv[x] = 0.f; }
+
+  if (kv0 < s.n_kv) {
+    for (int e = tid; e < GT * dq; e += 256) {
+      int r = e / dq, c = e - r * dq, j = kv0 + r;
+      Ks[r * kp + c] = (j < s.n_kv) ? ldf(kp_ + s.bk + (int64_t)j * p.k_st + c) : 0.f;
+    }
+    for (int e = tid; e < GT * dv; e += 256) {
+      int r = e / dv, c = e - r * dv, j = kv0 + r;
+      Vs[r * vp_ + c] = (j < s.n_kv) ? ldf(vp + s.bv + (int64_t)j * p.v_st + c) : 0.f;
+    }
+    // query rows that can see these keys
+    int q_begin = 0, q_end = s.n_q;
+    if (p.causal) q_begin = kv0;
+    if (p.window >= 0 && kv0 - p.window > q_begin) q_begin = kv0 - p.window;
+    if (p.window >= 0 && kv0 + GT + p.window < q_end) q_end = kv0 + GT + p.window;
+    q_begin = (q_begin / GT) * GT;
+    for (int q0 = q_begin; q0 < q_end; q0 += GT) {
+      __syncthreads();
+      for (int e = tid; e < GT * dq; e += 256) {
+        int r = e / dq, c = e - r * dq, i = q0 + r;
+        Qs[e] = (i < s.n_q) ? ldf(qp + s.bq + (int64_t)i * p.q_st + c) : 0.f;
+      }
+      for (int e = tid; e < GT * dv; e += 256) {
+        int r = e / dv, c = e - r * dv, i = q0 + r;
+        Os[e] = (i < s.n_q) ? ldf(dop + s.bo + (int64_t)i * p.o_st + c) : 0.f;
+      }
+      __syncthreads();
+      {
+        const int tx = tid & 31, ty = tid >> 5;
+        float sacc[4] = {0.f, 0.f, 0.f, 0.f}, pacc[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* krow = Ks + tx * kp;
+        for (int c = 0; c < dq; ++c) {
+          const float kvv = krow[c];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sacc[r] = fmaf(Qs[(ty + 8 * r) * dq + c], kvv, sacc[r]);
+        }
+        const float* vrow = Vs + tx * vp_;
+        for (int c = 0; c < dv; ++c) {
+          const float vv = vrow[c];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) pacc[r] = fmaf(Os[(ty + 8 * r) * dv + c], vv, pacc[r]);
+        }
+        const int j = kv0 + tx;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = q0 + ty + 8 * r;
+          float pval;
+          const float ds = bwd_pair(p, s, b, h, i, j, sacc[r], pacc[r], &pval, nullptr);
+          Ds[(ty + 8 * r) * (GT + 1) + tx] = ds;
+          Ps[(ty + 8 * r) * (GT + 1) + tx] = pval;
+        }
+      }
+      __syncthreads();
+      for (int ii = 0; ii < GT; ++ii) {
+        const float ds = Ds[ii * (GT + 1) + oj], pv = Ps[ii * (GT + 1) + oj];
+        const float* qrow = Qs + ii * dq;
+        const float* orow = Os + ii * dv;
+#pragma unroll
+        for (int x = 0; x < GMAXX; ++x) {
+          const int c = ocg + 8 * x;
+          if (x < nxk && c < dq) acck[x] = fmaf(ds, qrow[c], acck[x]);
+          if (x < nxv && c < dv) accv[x] = fmaf(pv, orow[c], accv[x]);
+        }
+      }
+    }
+  }
+  const int j = kv0 + oj;
+  if (j < krows) {
+    const bool live = j < s.n_kv;
+#pragma unroll
+    for (int x = 0; x < GMAXX; ++x) {
+      const int c = ocg + 8 * x;
+      if (x < nxk && c < dq) stf(dkp + s.bk + (int64_t)j * p.k_st + c, live ? acck[x] * p.alpha : 0.f);
+      if (x < nxv && c < dv) stf(dvp + s.bv + (int64_t)j * p.v_st + c, live ? accv[x] : 0.f);
     }
   }
 }
@@ -1355,6 +1628,23 @@ long long mfma_grid(const Params& p, bool split_list = false) {
   return 8LL * p.entries_per_bh * (((long long)p.B * p.H + 7) / 8);
 }
 
+template <typename T>
+int launch_bwd(const Params& p, hipStream_t st) {
+  const size_t tile = (size_t)GT * p.d_qk + (size_t)GT * p.d_v + (size_t)GT * (p.d_qk + 1) + (size_t)GT * (p.d_v + 1);
+  const size_t smem_q = sizeof(float) * (tile + GT * (GT + 1) + 132 + GT * GT);
+  const size_t smem_kv = sizeof(float) * (tile + 2 * GT * (GT + 1));
+  static int granted_q[64], granted_kv[64];
+  if (int rc = allow_lds((const void*)hstu_bwd_dq<T>, (int)smem_q, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv<T>, (int)smem_kv, granted_kv)) return rc;
+  hipLaunchKernelGGL(hstu_bwd_dq<T>, dim3((p.L + GT - 1) / GT, p.H, p.B), dim3(256), smem_q, st, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL(hstu_bwd_dkv<T>, dim3((p.Lkv + GT - 1) / GT, p.H, p.B), dim3(256), smem_kv, st, p);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
+  return HSTU_OK;
+}
+
 template <int D, bool POS, bool TS, bool F8>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS);
@@ -1407,6 +1697,28 @@ const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
     case V_MFMA_FP8: return "hstu_fwd_mfma_fp8";
     default: return "invalid";
   }
+}
+
+int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {
+  if (!args) return fail(HSTU_ERR_NULL, "args is null");
+  if (args->struct_size != sizeof(HstuAttnBwdArgs) || args->version != HSTU_ATTN_ABI_VERSION)
+    return fail(HSTU_ERR_VERSION, "backward args struct_size/version (%u/%u) do not match this library (%zu/%d)",
+                args->struct_size, args->version, sizeof(HstuAttnBwdArgs), HSTU_ATTN_ABI_VERSION);
+  const HstuAttnFwdArgs* f = &args->fwd;
+  // the forward's own checks apply, except that its `out` is not needed
+  HstuAttnFwdArgs probe = *f;
+  if (!probe.out) probe.out = (void*)args->dout;
+  int rc = validate(&probe);
+  if (rc != HSTU_OK) return rc;
+  g_err[0] = 0;
+  if (f->qk_dtype == HSTU_DTYPE_FP8_E4M3FN) return fail(HSTU_ERR_DTYPE, "the backward takes fp32 or bf16 storage, not fp8 q/k");
+  if (f->B == 0 || (f->layout == HSTU_LAYOUT_JAGGED && f->total_tokens == 0)) return HSTU_OK;
+  if (!args->dout || !args->dq || !args->dk || !args->dv) return fail(HSTU_ERR_NULL, "dout, dq, dk and dv must be non-null");
+  Params p = make_params(f);
+  p.dout = args->dout; p.dq = args->dq; p.dk = args->dk; p.dv = args->dv;
+  p.dpos = args->dpos_tab; p.dts = args->dts_tab;
+  hipStream_t st = (hipStream_t)stream;
+  return f->qk_dtype == HSTU_DTYPE_FP32 ? launch_bwd<float>(p, st) : launch_bwd<bf16_t>(p, st);
 }
 
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {

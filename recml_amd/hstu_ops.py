@@ -77,6 +77,11 @@ def _attach_workspace(args, keep):
     args.workspace_bytes = ws
 
 
+def _passed_inputs(keep):
+  """The q, k, v tensors whose pointers build_args put into the struct (after any copy)."""
+  return keep[0], keep[1], keep[2]
+
+
 def _run(args, keep):
   lib = _lib.load()
   stream = torch.cuda.current_stream(keep[0].device).cuda_stream
@@ -181,7 +186,7 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
   q, k, v = (_inner_contiguous(t) for t in (q, k, v))
   if out.stride(-1) != 1:
     raise ValueError("out must be contiguous in its last dimension")
-  keep += [q, k, v]
+  keep[0:3] = [q, k, v]     # the tensors whose pointers go into the struct
   a.q, a.k, a.v, a.out = q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr()
   a.qk_dtype = _DTYPES[q.dtype]
   a.v_dtype = a.out_dtype = _DTYPES[v.dtype]
@@ -324,6 +329,93 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
   with torch.cuda.device(q.device):
     _run(args, keep)
   return out
+
+
+def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_len=None,
+                       n=None, alpha=1.0, causal=True, pos_bias=None,
+                       timestamps=None, ts_bias=None, ts_bucket_size=0.301,
+                       q_segment_ids=None, kv_segment_ids=None,
+                       sliding_window_size=None, mask=None, bias=None):
+  """Gradients of sum(hstu_attention(q, k, v, ...) * dout).
+
+  Same arguments as hstu_attention (fp32 or bf16; not fp8).  Returns
+  (dq, dk, dv, dpos_bias, dts_bias): dq, dk, dv shaped and typed like q, k, v;
+  the table gradients fp32 and shaped like the tables (None for a table that
+  was not given).  Math of the reference's backward kernel
+  (recml/core/ops/hstu_ops.py:417-548).
+  """
+  for name, t in (("q", q), ("k", k), ("v", v), ("dout", dout)):
+    _check_gpu(name, t)
+  if q.dtype not in (torch.float32, torch.bfloat16):
+    raise ValueError(f"the backward takes float32 or bfloat16, got {q.dtype}")
+  exp = tuple(q.shape[:-1]) + (v.shape[-1],)
+  if tuple(dout.shape) != exp or dout.dtype != q.dtype:
+    raise ValueError(f"dout must be a {q.dtype} tensor of shape {exp}")
+  out_like = torch.empty_strided(dout.shape, dout.stride(), dtype=dout.dtype, device=dout.device) \
+      if dout.stride(-1) == 1 else torch.empty_like(dout.contiguous())
+  dout = dout if dout.stride() == out_like.stride() else dout.contiguous()
+  fa, keep = build_args(
+      q, k, v, out_like, seq_lens=seq_lens, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
+      causal=causal, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
+      q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids, sliding_window_size=sliding_window_size,
+      mask=mask, bias=bias)
+  # build_args may have made q, k, v contiguous in d: the gradients take the layout it passed on
+  qi, ki, vi = _passed_inputs(keep)
+  dq, dk, dv = torch.empty_like(qi), torch.empty_like(ki), torch.empty_like(vi)
+  ba = _lib.HstuAttnBwdArgs()
+  ba.struct_size = C.sizeof(_lib.HstuAttnBwdArgs)
+  ba.version = _lib.ABI_VERSION
+  ba.fwd = fa
+  ba.dout, ba.dq, ba.dk, ba.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+  dpos = dts = None
+  if pos_bias is not None:
+    dpos = torch.zeros((fa.pos_heads, 2 * fa.L - 1), dtype=torch.float32, device=q.device)
+    ba.dpos_tab = dpos.data_ptr()
+  if ts_bias is not None:
+    dts = torch.zeros((fa.ts_heads, fa.ts_num_buckets + 1), dtype=torch.float32, device=q.device)
+    ba.dts_tab = dts.data_ptr()
+  lib = _lib.load()
+  with torch.cuda.device(q.device):
+    stream = torch.cuda.current_stream(q.device).cuda_stream
+    rc = lib.hstu_attn_bwd(C.byref(ba), C.c_void_p(stream))
+  if rc != 0:
+    msg = lib.hstu_attn_last_error().decode()
+    if rc in (-3, -4, -1):
+      raise ValueError(f"hstu_attn_bwd rejected the arguments ({rc}): {msg}")
+    raise RuntimeError(f"hstu_attn_bwd failed ({rc}): {msg}")
+  del keep
+  if dpos is not None:
+    dpos = dpos.reshape(pos_bias.shape)
+  if dts is not None:
+    dts = dts.reshape(ts_bias.shape)
+  return dq, dk, dv, dpos, dts
+
+
+class _HstuAttentionFn(torch.autograd.Function):
+  """hstu_attention with gradients for q, k, v and the two bias tables."""
+
+  @staticmethod
+  def forward(ctx, q, k, v, pos_bias, ts_bias, kwargs):
+    ctx.kwargs = kwargs
+    ctx.save_for_backward(q, k, v, *(t for t in (pos_bias, ts_bias) if t is not None))
+    ctx.has = (pos_bias is not None, ts_bias is not None)
+    return hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kwargs)
+
+  @staticmethod
+  def backward(ctx, dout):
+    saved = list(ctx.saved_tensors)
+    q, k, v = saved[:3]
+    rest = saved[3:]
+    pos = rest.pop(0) if ctx.has[0] else None
+    ts = rest.pop(0) if ctx.has[1] else None
+    dq, dk, dv, dpos, dts = hstu_attention_bwd(q, k, v, dout.contiguous(), pos_bias=pos, ts_bias=ts, **ctx.kwargs)
+    cast = lambda g, t: None if g is None else g.to(t.dtype)
+    return dq, dk, dv, cast(dpos, pos) if pos is not None else None, cast(dts, ts) if ts is not None else None, None
+
+
+def hstu_attention_autograd(q, k, v, *, pos_bias=None, ts_bias=None, **kwargs):
+  """hstu_attention as a differentiable torch op (gradients for q, k, v, pos_bias, ts_bias)."""
+  return _HstuAttentionFn.apply(q, k, v, pos_bias, ts_bias, kwargs)
 
 
 def pointwise_splash_attention(

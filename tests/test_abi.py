@@ -30,11 +30,13 @@ def test_library_exports_every_declared_symbol():
   assert lib.hstu_attn_abi_version() == _lib.ABI_VERSION
 
 
-def test_struct_layout_matches_header():
-  fields = [f[0] for f in _lib.HstuAttnFwdArgs._fields_]
+@pytest.mark.parametrize("name", ["HstuAttnFwdArgs", "HstuAttnBwdArgs"])
+def test_struct_layout_matches_header(name):
+  struct = getattr(_lib, name)
+  fields = [f[0] for f in struct._fields_]
   prog = ['#include <stdio.h>', '#include <stddef.h>', '#include "hstu_attn.h"', "int main(void) {",
-          '  printf("%zu\\n", sizeof(HstuAttnFwdArgs));']
-  prog += [f'  printf("%zu\\n", offsetof(HstuAttnFwdArgs, {f}));' for f in fields]
+          f'  printf("%zu\\n", sizeof({name}));']
+  prog += [f'  printf("%zu\\n", offsetof({name}, {f}));' for f in fields]
   prog += ["  return 0;", "}"]
   with tempfile.TemporaryDirectory() as d:
     src = os.path.join(d, "layout.c")
@@ -42,9 +44,27 @@ def test_struct_layout_matches_header():
     open(src, "w").write("\n".join(prog))
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), "-o", exe, src], check=True)
     out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
-  assert int(out[0]) == C.sizeof(_lib.HstuAttnFwdArgs)
+  assert int(out[0]) == C.sizeof(struct)
   for f, off in zip(fields, out[1:]):
-    assert getattr(_lib.HstuAttnFwdArgs, f).offset == int(off), f
+    assert getattr(struct, f).offset == int(off), f
+
+
+def test_backward_validation_errors_without_gpu():
+  lib = _lib.load()
+  assert lib.hstu_attn_bwd(None, None) == -1
+  b = _lib.HstuAttnBwdArgs()
+  assert lib.hstu_attn_bwd(C.byref(b), None) == -2            # struct_size / version not filled in
+  b.struct_size, b.version = C.sizeof(_lib.HstuAttnBwdArgs), _lib.ABI_VERSION
+  b.fwd = _lib.new_args()
+  f = b.fwd
+  f.B, f.L, f.Lkv, f.H, f.d_qk, f.d_v = 1, 8, 8, 1, 32, 32
+  f.q = f.k = f.v = 0x1000
+  f.qk_dtype, f.v_dtype, f.out_dtype = _lib.DTYPE_FP8_E4M3FN, _lib.DTYPE_BF16, _lib.DTYPE_BF16
+  b.dout = 0x1000
+  assert lib.hstu_attn_bwd(C.byref(b), None) == -3            # no fp8 backward
+  f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_BF16
+  assert lib.hstu_attn_bwd(C.byref(b), None) == -1            # dq, dk, dv missing
+  assert b"dq" in lib.hstu_attn_last_error()
 
 
 def test_validation_errors_without_gpu():

@@ -1,0 +1,97 @@
+"""Backward of the attention op on the GPU against the numpy oracle (itself pinned by finite differences)."""
+
+import numpy as np
+import pytest
+import torch
+
+import recml_amd
+from oracle import hstu_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(x, dtype=None):
+  t = torch.from_numpy(np.ascontiguousarray(x)).to("cuda:0")
+  return t if dtype is None else t.to(dtype)
+
+
+def _rel(a, b):
+  return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_backward_lengths_and_tables(gpu, dtype, tol):
+  rng = np.random.default_rng(21)
+  B, L, H, d = 3, 70, 2, 32
+  lens = np.array([70, 33, 1], dtype=np.int32)
+  rd = O.round_bf16 if dtype == torch.bfloat16 else (lambda x: x)
+  q, k, v, dout = (rd(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+  tab = (rng.standard_normal((129,)) * 0.3).astype(np.float32)
+  ts = 1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, (B, L))), axis=1).astype(np.int64)
+  kw = dict(seq_lens=lens, pos_tab=pos, timestamps=ts, ts_tab=tab)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  got = recml_amd.hstu_attention_bwd(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), _dev(dout, dtype),
+                                     seq_lens=_dev(lens), pos_bias=_dev(pos), timestamps=_dev(ts), ts_bias=_dev(tab))
+  for name, g, w in zip(("dq", "dk", "dv", "dpos", "dts"), got, want):
+    assert tuple(g.shape) == w.shape, name
+    assert _rel(g.float().cpu().numpy(), w) <= tol, name
+  dq, dk, dv = (g.float().cpu().numpy() for g in got[:3])
+  for b in range(B):
+    assert (dq[b, lens[b]:] == 0).all() and (dk[b, lens[b]:] == 0).all() and (dv[b, lens[b]:] == 0).all()
+
+
+def test_backward_jagged_equals_padded(gpu):
+  rng = np.random.default_rng(22)
+  B, L, H, d = 4, 90, 2, 64
+  lens = np.array([90, 17, 64, 33], dtype=np.int32)
+  q, k, v, dout = (rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.4 for _ in range(4))
+  pos = (rng.standard_normal((2 * L - 1,)) * 0.3).astype(np.float32)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, seq_lens=lens, pos_tab=pos)
+  pack = lambda x: O.padded_to_jagged(x, lens)
+  (qj, off), (kj, _), (vj, _), (dj, _) = pack(q), pack(k), pack(v), pack(dout)
+  got = recml_amd.hstu_attention_bwd(_dev(qj), _dev(kj), _dev(vj), _dev(dj), seq_offsets=_dev(off.astype(np.int32)),
+                                     max_len=L, pos_bias=_dev(pos))
+  for name, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(O.jagged_to_padded(g.cpu().numpy(), off, L), w) <= 2e-5, name
+  assert _rel(got[3].cpu().numpy(), want[3]) <= 2e-5 and got[4] is None
+
+
+def test_backward_options(gpu):
+  # segment ids + window (the reference's test recipe, hstu_ops_test.py:36-83), then full mask + dense bias + cross length
+  rng = np.random.default_rng(23)
+  B, L, H, d = 2, 40, 2, 16
+  q, k, v, dout = (rng.standard_normal((B, L, H, d)).astype(np.float32) for _ in range(4))
+  seg = np.ones((B, L), np.int32)
+  seg[0, 25:] = 0
+  seg[1, 10:30] = 2
+  kw = dict(alpha=1 / np.sqrt(d), q_segment_ids=seg, kv_segment_ids=seg, sliding_window_size=7)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  got = recml_amd.hstu_attention_bwd(_dev(q), _dev(k), _dev(v), _dev(dout), alpha=kw["alpha"], q_segment_ids=_dev(seg),
+                                     kv_segment_ids=_dev(seg), sliding_window_size=7)
+  for name, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(g.cpu().numpy(), w) <= 2e-5, name     # the reference accepts 5e-3 here
+  Lk = 55
+  k2, v2 = (rng.standard_normal((B, Lk, H, d)).astype(np.float32) for _ in range(2))
+  m = rng.random((B, L, Lk)) > 0.3
+  bias = rng.standard_normal((B, L, Lk)).astype(np.float32)
+  want = O.hstu_attention_bwd_ref(q, k2, v2, dout, causal=False, mask=m, bias=bias, n=7.0)
+  got = recml_amd.hstu_attention_bwd(_dev(q), _dev(k2), _dev(v2), _dev(dout), causal=False, mask=_dev(m), bias=_dev(bias), n=7.0)
+  for name, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(g.cpu().numpy(), w) <= 2e-5, name
+
+
+def test_autograd_function(gpu):
+  rng = np.random.default_rng(24)
+  B, L, H, d = 2, 64, 2, 64
+  lens = np.array([64, 20], dtype=np.int32)
+  mk = lambda *s: torch.from_numpy(rng.standard_normal(s).astype(np.float32) * 0.4).to("cuda:0").requires_grad_(True)
+  q, k, v = mk(B, L, H, d), mk(B, L, H, d), mk(B, L, H, d)
+  pos = mk(H, 2 * L - 1)
+  dout = torch.from_numpy(rng.standard_normal((B, L, H, d)).astype(np.float32)).to("cuda:0")
+  out = recml_amd.hstu_attention_autograd(q, k, v, pos_bias=pos, seq_lens=_dev(lens))
+  (out * dout).sum().backward()
+  n = lambda t: t.detach().cpu().numpy()
+  want = O.hstu_attention_bwd_ref(n(q), n(k), n(v), n(dout), seq_lens=lens, pos_tab=n(pos))
+  for name, g, w in zip(("dq", "dk", "dv", "dpos"), (q.grad, k.grad, v.grad, pos.grad), want):
+    assert _rel(n(g), w) <= 2e-5, name

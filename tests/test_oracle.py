@@ -330,3 +330,55 @@ def test_rows_near_bucket_boundary():
   off = np.array([0, 3, 6])
   flag = O.rows_near_bucket_boundary(ts, off)
   assert flag.tolist()[0] is True and not flag[3:].any()
+
+
+def _fd_grad(f, x, eps=1e-6):
+  """Central finite differences of the scalar f with respect to every entry of x (fp64)."""
+  g = np.zeros_like(x, dtype=np.float64)
+  it = np.nditer(x, flags=["multi_index"])
+  for _ in it:
+    idx = it.multi_index
+    old = x[idx]
+    x[idx] = old + eps
+    fp = f()
+    x[idx] = old - eps
+    fm = f()
+    x[idx] = old
+    g[idx] = (fp - fm) / (2 * eps)
+  return g
+
+
+@pytest.mark.parametrize("case", ["lengths_bias", "segments_window", "full_mask_dense_bias"])
+def test_backward_oracle_against_finite_differences(case):
+  rng = np.random.default_rng(11)
+  B, L, H, d, dv = 2, 6, 2, 4, 3
+  q, k = rng.standard_normal((B, L, H, d)), rng.standard_normal((B, L, H, d))
+  v, dout = rng.standard_normal((B, L, H, dv)), rng.standard_normal((B, L, H, dv))
+  kw = dict(alpha=0.7, n=5.0)
+  pos = ts_tab = None
+  if case == "lengths_bias":
+    pos = rng.standard_normal((H, 2 * L - 1))
+    ts_tab = rng.standard_normal((1, 130))             # one row shared by the heads
+    ts = 1000 + np.cumsum(rng.integers(1, 5000, (B, L)), axis=1)
+    kw.update(seq_lens=np.array([6, 4]), pos_tab=pos, timestamps=ts, ts_tab=ts_tab)
+  elif case == "segments_window":
+    seg = np.array([[1, 1, 1, 2, 2, 0], [1, 1, 1, 1, 1, 1]])
+    pos = rng.standard_normal((2 * L - 1,))            # one row shared by the heads
+    kw.update(q_segment_ids=seg, kv_segment_ids=seg, sliding_window_size=2, pos_tab=pos)
+  else:
+    m = rng.random((B, L, L)) > 0.3
+    kw.update(causal=False, mask=m, bias=rng.standard_normal((B, L, L)))
+  loss = lambda: float((O.hstu_attention_ref(q, k, v, **kw) * dout).sum())
+  dq, dk, dvv, dpos, dts = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  for name, x, g in (("q", q, dq), ("k", k, dk), ("v", v, dvv)):
+    fd = _fd_grad(loss, x)
+    assert np.abs(fd - g).max() <= 1e-7 * max(1.0, np.abs(fd).max()), name
+  if pos is not None:
+    fd = _fd_grad(loss, pos)
+    assert dpos.shape == pos.shape and np.abs(fd - dpos).max() <= 1e-7 * max(1.0, np.abs(fd).max())
+  else:
+    assert dpos is None
+  if ts_tab is not None:
+    fd = _fd_grad(loss, ts_tab)
+    assert dts.shape == ts_tab.shape and np.abs(fd - dts).max() <= 1e-7 * max(1.0, np.abs(fd).max())
+    assert np.abs(dts).max() > 0

@@ -16,3 +16,8 @@ from recml_amd.hstu_ops import (  # noqa: F401
 )
 from recml_amd.masks import make_attention_mask, make_causal_mask  # noqa: F401
 from recml_amd.hstu_layer import HSTU, HSTUBlock  # noqa: F401
+from recml_amd.hstu_bias import (  # noqa: F401
+    RelativeBucketedTimeAndPositionBasedBias,
+    RelativePositionalBias,
+    default_bucketization,
+)

@@ -1,6 +1,6 @@
 """Benchmark of the HSTU attention forward on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c3full|c2|c4|c5]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c3full|c2|c4|c5|c4-model] [--backward]
 
 A step is one pass of the attention forward over one synthetic batch whose
 inputs already sit in HBM.  The default workload is the one the headline
@@ -138,6 +138,67 @@ def measured_traffic(workload):
 PEAK_FP32_TFLOPS = 157.3    # MI355X dense fp32
 
 
+def bench_model(args, dev):
+  """Config 4 end to end: embedding gather (10 M x 512 bf16 table, Zipf ids) -> 4 HSTU blocks
+  (D=512, H=8, head dim 64, position bias) -> final norm, padded [128, 1024] batch with
+  lengths U{128..1024}.  torch for everything but the attention.  One JSON line."""
+  import torch
+  import recml_amd
+  rng = np.random.Generator(np.random.PCG64(4))
+  B, L, D, H, layers, vocab = 128, 1024, 512, 8, 4, 10_000_000
+  lens = rng.integers(128, L + 1, B).astype(np.int32)
+  ids = np.minimum(rng.zipf(1.05, (B, L)), vocab - 1).astype(np.int64)
+  ids[np.arange(L)[None, :] >= lens[:, None]] = 0
+  model = recml_amd.HSTU(vocab_size=8, max_positions=L, model_dim=D, num_heads=H, num_layers=layers, add_head=False,
+                         dtype=torch.bfloat16, device=dev, seed=4)
+  table = torch.empty((vocab, D), dtype=torch.bfloat16, device=dev)
+  table.normal_(0.0, 0.01, generator=torch.Generator(device=dev).manual_seed(4))
+  model.item_embedding = torch.nn.Parameter(table, requires_grad=False)
+  ids_d = torch.from_numpy(ids).to(dev)
+  lens_d = torch.from_numpy(lens).to(dev)
+  pos = (torch.randn((2 * L - 1,), generator=torch.Generator().manual_seed(5)) * 0.02).to(dev)
+  steps, warm = max(1, args.steps // 10), max(2, args.warmup // 10)
+  with torch.no_grad():
+    def timed(fn):
+      for _ in range(warm):
+        o = fn()
+      torch.cuda.synchronize()
+      t0 = time.perf_counter()
+      for _ in range(steps):
+        o = fn()
+      torch.cuda.synchronize()
+      return (time.perf_counter() - t0) * 1e3 / steps, o
+    ms, out = timed(lambda: model(ids_d, seq_lens=lens_d, pos_bias=pos))
+    ms_jagged, outj = timed(lambda: model(ids_d, seq_lens=lens_d, pos_bias=pos, jagged=True))
+    keep = (torch.arange(L, device=dev)[None, :] < lens_d[:, None])[:, :, None]
+    jag_err = float(((outj.float() - out.float()) * keep).abs().max() / out.float().abs().max())
+    # the attention alone on the same shapes (padded layout with lengths, as the block calls it)
+    q = torch.randn((B, L, 4, H, D // H), device=dev, dtype=torch.bfloat16)
+    att = lambda: recml_amd.hstu_attention(q[:, :, 1], q[:, :, 2], q[:, :, 3], seq_lens=lens_d, pos_bias=pos)
+    for _ in range(warm):
+      att()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+      att()
+    torch.cuda.synchronize()
+    att_ms = (time.perf_counter() - t0) * 1e3 / steps
+  assert tuple(out.shape) == (B, L, D) and bool(torch.isfinite(out.float()).all())
+  nn = lens.astype(np.int64)
+  attn_flops = int((H * (nn * (nn + 1) // 2) * 4 * (D // H)).sum()) * layers
+  proj_flops = B * L * (2 * D * 4 * D + 2 * D * D) * layers
+  print(json.dumps({
+      "metric": "HSTU 4-layer forward (config 4), sequences/s", "value": B / (ms * 1e-3), "unit": "seqs/s", "n_gpus": 1,
+      "steps": steps, "warmup": warm, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": f"C4 model: B={B} L={L} D={D} H={H} layers={layers} vocab={vocab} lens U{{128..1024}}, padded, pos bias, no head"},
+      "ms_per_step_packed_tokens": ms_jagged, "seqs_per_s_packed_tokens": B / (ms_jagged * 1e-3),
+      "packed_vs_padded_max_abs_over_max": jag_err,
+      "attention_ms_per_layer": att_ms, "attention_share": layers * att_ms / ms,
+      "attention_gflop_unmasked": attn_flops / 1e9, "projection_gflop_padded": proj_flops / 1e9,
+      "model_tflops": (attn_flops + proj_flops) / (ms * 1e-3) / 1e12}))
+
+
 def bench_backward(args, w, q, k, v, kw, dev):
   """The backward pass (general fp32-arithmetic kernels) on the same workload: one JSON line.
 
@@ -226,6 +287,8 @@ def main():
   if not torch.cuda.is_available():
     raise SystemExit("bench.py needs a GPU")
   dev = torch.device("cuda:0")
+  if args.workload == "c4-model":
+    return bench_model(args, dev)
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
   if args.backward:

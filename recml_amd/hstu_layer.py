@@ -120,6 +120,29 @@ class HSTUBlock(torch.nn.Module):
     return out.reshape(B, L, D) + inputs
 
 
+  def forward_jagged(self, tokens, seq_offsets, max_len, *, pos_bias=None, timestamps=None, ts_bias=None):
+    """The block on packed tokens [T, D] (sequence b = rows seq_offsets[b]..seq_offsets[b+1]):
+    no work at all for padding, in the projections either.  `timestamps` is jagged [T]."""
+    T, D = tokens.shape
+    H, hd = self.num_heads, self.head_dim
+    x = F.layer_norm(tokens, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
+    w = torch.cat([self.u_kernel, self.q_kernel, self.k_kernel, self.v_kernel], dim=1).reshape(D, 4 * H * hd)
+    uqkv = x @ w
+    if self.use_bias:
+      uqkv = uqkv + torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1)
+    uqkv = F.silu(uqkv).reshape(T, 4, H, hd)
+    u, q, k, v = uqkv.unbind(dim=1)
+    alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
+    attn = hstu_ops.hstu_attention(q, k, v, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
+                                   pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
+    normed = F.layer_norm(attn.reshape(T, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
+                          self.attn_ln_beta.reshape(-1), self.eps)
+    out = (u.reshape(T, H * hd) * normed) @ self.output_kernel.reshape(H * hd, D)
+    if self.use_bias:
+      out = out + self.output_bias
+    return out + tokens
+
+
 class HSTU(torch.nn.Module):
   """The HSTU model forward (recml/layers/keras/hstu.py:585-621): item
   embedding (x sqrt(D)) + position embedding -> final_norm -> blocks ->
@@ -151,12 +174,20 @@ class HSTU(torch.nn.Module):
   def _final_norm(self, x):
     return F.layer_norm(x, (self.model_dim,), self.final_norm_gamma, self.final_norm_beta, self.eps)
 
-  def forward(self, inputs, padding_mask=None, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None):
-    """inputs: item ids [B, L]; `padding_mask` [B, L] (1 = real item, end-padded) or `seq_lens` [B]."""
+  def forward(self, inputs, padding_mask=None, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None,
+              jagged=False):
+    """inputs: item ids [B, L]; `padding_mask` [B, L] (1 = real item, end-padded) or `seq_lens` [B].
+
+    jagged=True packs the valid tokens once and runs every block on [T, D]: nothing is computed
+    for padding.  Rows past a sequence's length are then returned as zeros, whereas the padded
+    form (like the reference) carries the padded positions' own embeddings through the blocks.
+    """
     if seq_lens is None:
       if padding_mask is None:
         raise ValueError("Either `padding_mask` or `seq_lens` must be set.")
       seq_lens = masks.lengths_from_padding_mask(padding_mask)
+    if jagged:
+      return self._forward_jagged(inputs, seq_lens, pos_bias, timestamps, ts_bias)
     x = self.item_embedding[inputs]
     if self.scale_by_sqrt_dim:
       x = x * (self.model_dim ** 0.5)
@@ -169,3 +200,27 @@ class HSTU(torch.nn.Module):
     if self.reverse_embedding is None:
       return x
     return x @ self.reverse_embedding
+
+  def _forward_jagged(self, inputs, seq_lens, pos_bias, timestamps, ts_bias):
+    B, L = inputs.shape
+    lens = seq_lens.to(torch.int64).clamp(0, L)
+    valid = torch.arange(L, device=inputs.device)[None, :] < lens[:, None]          # [B, L]
+    offsets = torch.zeros(B + 1, dtype=torch.int32, device=inputs.device)
+    offsets[1:] = torch.cumsum(lens, 0)
+    ids = inputs[valid]                                                              # [T], sequence-major
+    x = self.item_embedding[ids]
+    if self.scale_by_sqrt_dim:
+      x = x * (self.model_dim ** 0.5)
+    if self.position_embedding is not None:
+      pos_idx = torch.arange(L, device=inputs.device)[None, :].expand(B, L)[valid]
+      x = x + self.position_embedding[pos_idx]
+    x = self._final_norm(x)
+    ts = None if timestamps is None else timestamps[valid]
+    for block in self.decoder_blocks:
+      x = block.forward_jagged(x, offsets, L, pos_bias=pos_bias, timestamps=ts, ts_bias=ts_bias)
+    x = self._final_norm(x)
+    if self.reverse_embedding is not None:
+      x = x @ self.reverse_embedding
+    out = torch.zeros((B, L, x.shape[-1]), dtype=x.dtype, device=x.device)
+    out[valid] = x
+    return out

@@ -129,6 +129,10 @@ def test_model_on_gpu_against_oracle(gpu):
        "blocks": [{n: g(p) for n, p in b.named_parameters()} for b in m.decoder_blocks]}
   ref = BO.hstu_model(ids.cpu().numpy(), w, num_heads=4, seq_lens=np.array([3, 2]))
   assert np.abs(out.double().cpu().numpy() - ref).max() / np.abs(ref).max() <= 2e-5
+  # packed tokens: the same values on the valid positions, zeros elsewhere
+  outj = m(ids, pm, jagged=True).double().cpu().numpy()
+  assert np.abs(outj[0] - ref[0]).max() / np.abs(ref).max() <= 2e-5
+  assert np.abs(outj[1, :2] - ref[1, :2]).max() / np.abs(ref).max() <= 2e-5 and (outj[1, 2] == 0).all()
 
 
 @pytest.mark.gpu

@@ -74,6 +74,7 @@ struct Params {
   const int32_t* ts_rel;
   const int32_t* ts_range;
   const float* ts_scaled;    // workspace: log2(e) * ts_tab as [heads][TS_TAB_LEN], indices past the last bucket repeat it
+  const int32_t* ts_thr;     // workspace: [TS_TAB_LEN] smallest |dt| that the kernel's bucket function puts in bucket >= b
   const void* ws_base;       // start of the workspace (all of the above lie within 4 GB of it)
   const float* q_scale;      // [H] or null: dequantisation scales of fp8 q / k
   const float* k_scale;
@@ -639,7 +640,7 @@ struct MfmaSmem {
   static constexpr int POS_BYTES = 4 * POS_COPY;    // 4 copies shifted by 0..3 floats
   static constexpr int TK_LANES = BN / 4 + 1;       // 16-byte pieces: 32 int32 key timestamps, then (min, max, -, -)
   static constexpr int TK_BYTES = TK_LANES * 16;
-  static constexpr int TAB_BYTES = TS_TAB_LEN * 4;
+  static constexpr int TAB_BYTES = 2 * TS_TAB_LEN * 4;   // scaled bucket table, then the bucket thresholds
   static constexpr int bias_stage(bool pos, bool ts) { return (pos ? POS_BYTES : 0) + (ts ? TK_BYTES : 0); }
   static constexpr int total(bool pos, bool ts) {
     return NSTAGE * (STAGE + bias_stage(pos, ts)) + (ts ? TAB_BYTES : 0);
@@ -770,6 +771,13 @@ __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, W
   return true;
 }
 
+// Timestamp bucket of a time difference already converted to float, as the MFMA kernel computes it:
+// trunc(log2(clamp(|f|, 1, 1e9)) * ln2 / bucket_size) by v_log_f32.
+__device__ __forceinline__ int ts_bucket_hw(float f, float log2_scale) {
+  f = __builtin_amdgcn_fmed3f(__builtin_fabsf(f), 1.0f, 1.0e9f);
+  return (int)(__builtin_amdgcn_logf(f) * log2_scale);
+}
+
 // Where sequence b starts in the int32 timestamp copy and in the per-tile range table.
 // Timestamps that follow the token axis are packed like it (tiles by an upper bound of
 // the tiles before them); timestamps with a batch stride are [B][L].
@@ -883,6 +891,18 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       const int hd = i / TS_TAB_LEN, e = i - hd * TS_TAB_LEN;
       tab_out[i] = p.ts_tab[(int64_t)hd * (p.ts_nb + 1) + (e < p.ts_nb ? e : p.ts_nb)] * LOG2E;
     }
+    // thr[b] = smallest |dt| >= 0 whose bucket, by the very instructions the main kernel uses, is >= b
+    // (INT_MAX when no 31-bit value reaches b): a bisection that relies on that function being monotone
+    int32_t* thr = (int32_t*)(tab_out + p.ts_heads * TS_TAB_LEN);
+    for (int bkt = gtid; bkt < TS_TAB_LEN; bkt += gsz) {
+      unsigned lo = 0, hi = 0x7fffffffu;          // invariant: bucket(hi) >= bkt or hi is the cap
+      if (ts_bucket_hw((float)(int)hi, p.ts_log2_scale) < bkt) { thr[bkt] = 0x7fffffff; continue; }
+      while (lo < hi) {
+        const unsigned mid = lo + (hi - lo) / 2;
+        if (ts_bucket_hw((float)(int)mid, p.ts_log2_scale) >= bkt) hi = mid; else lo = mid + 1;
+      }
+      thr[bkt] = (int32_t)lo;
+    }
   }
   if (pos_out) {
     const int len = 2 * p.L - 1;
@@ -976,6 +996,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
+  const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -1101,6 +1122,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     const int c = w < 3 ? w : 0;
     const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
     lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
+    lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
   }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
@@ -1212,10 +1234,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
     if (TS) {
-      auto bucket_f = [&](float f) {
-        f = __builtin_amdgcn_fmed3f(__builtin_fabsf(f), 1.0f, 1.0e9f);
-        return (int)(__builtin_amdgcn_logf(f) * p.ts_log2_scale);
-      };
+      auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
       if (ts32) {
         const int32_t* tk = Tk(st);
         const int2 rg = *(const int2*)(tk + BN);
@@ -1224,10 +1243,24 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         const int d_near = tq32 - rg.y, d_far = tq32 - rg.x;
         const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
         const bool same = d_near >= 0 && b_near == b_far;
+        const bool two = d_near >= 0 && b_far - b_near <= 1;
         if (__builtin_amdgcn_ballot_w64(!same) == 0) {
           const float add = TsTab[b_near];
 #pragma unroll
           for (int r = 0; r < 16; ++r) u[r] += add;
+        } else if (__builtin_amdgcn_ballot_w64(!two) == 0) {
+          // at most one bucket boundary inside the tile for every lane: a key is in the farther
+          // bucket exactly when tq - tk >= thr[b_near + 1], i.e. tk <= tq - thr
+          const float add_near = TsTab[b_near], add_far = TsTab[b_near + 1];
+          const int cut = tq32 - TsThr[b_near + 1];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
+            u[4 * g + 0] += kk.x <= cut ? add_far : add_near;
+            u[4 * g + 1] += kk.y <= cut ? add_far : add_near;
+            u[4 * g + 2] += kk.z <= cut ? add_far : add_near;
+            u[4 * g + 3] += kk.w <= cut ? add_far : add_near;
+          }
         } else {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
@@ -1554,7 +1587,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
     const bool by_token = a->ts_stride_b == 0;
     const size_t n_ts = by_token ? (size_t)a->total_tokens : (size_t)a->B * (size_t)a->L;
     const size_t tiles = by_token ? (size_t)(a->total_tokens >> 5) + (size_t)a->B + tiles_per_seq : (size_t)a->B * tiles_per_seq;
-    w.tab_bytes = up((size_t)a->ts_heads * TS_TAB_LEN * sizeof(float));
+    w.tab_bytes = up(((size_t)a->ts_heads + 1) * TS_TAB_LEN * sizeof(float));   // scaled tables, then the thresholds
     w.ok_bytes = up((size_t)a->B * sizeof(int32_t));
     // the kernel fetches whole 16-byte pieces: up to 31 timestamps and one range past the end
     w.rel_bytes = up(n_ts * sizeof(int32_t) + 128);
@@ -1758,6 +1791,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
         q.split_max = ws.split_max;
         q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
         q.ts_scaled = tab_out;
+        q.ts_thr = tab_out ? (const int32_t*)(tab_out + (size_t)p.ts_heads * TS_TAB_LEN) : nullptr;
         q.pos_scaled = pos_out;
         q.ts_ok = ok_out;
         q.ts_rel = rel_out;

@@ -162,14 +162,19 @@ size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
 
 /* Backward of the same op: gradients of sum(out * dout) with respect to q, k, v
- * and the two bias tables.  `fwd` describes the forward call (its `out` and
- * `workspace` are not used).  dout has the layout, dtype and strides of out;
+ * and the two bias tables.  `fwd` describes the forward call (its `out` is
+ * not used; its `workspace`, sized by hstu_attn_fwd_workspace_bytes, is
+ * overwritten when the matrix-core kernels run, see below).  dout has the
+ * layout, dtype and strides of out;
  * dq, dk, dv those of q, k, v and are fully written (rows past a sequence's
  * length as zeros).  dpos_tab / dts_tab are fp32 tables shaped like pos_tab /
  * ts_tab that are ACCUMULATED into by atomic adds: the caller zero-fills them
  * (or passes null when the table gradient is not wanted).  fp32 or bf16
  * storage, every option of the forward, fp32 arithmetic; fp8 q/k is not
- * supported.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which
+ * supported.  bf16 calls with d_qk = d_v = 128 that meet the conditions of the
+ * matrix-core forward, ask for no table gradient, pass 16-byte aligned
+ * gradient buffers and bring the workspace run on the matrix cores instead
+ * (bf16 products, fp32 accumulation); hstu_attn_bwd_variant tells which.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which
  * the reference reaches through jax.custom_vjp (hstu_ops.py:551-826), extended
  * by the table gradients that jax derives for recml/layers/keras/hstu.py:91-113,
  * 190-221. */
@@ -186,6 +191,10 @@ typedef struct HstuAttnBwdArgs {
 } HstuAttnBwdArgs;
 
 int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream);
+
+/* Name of the kernel pair hstu_attn_bwd would launch for `args` (diagnostics;
+ * static storage): "hstu_bwd_mfma_bf16", "hstu_bwd_general<...>" or "invalid". */
+const char* hstu_attn_bwd_variant(const HstuAttnBwdArgs* args);
 
 /* Message for the last non-zero status on this thread ("" if none). */
 const char* hstu_attn_last_error(void);

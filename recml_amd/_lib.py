@@ -23,6 +23,7 @@ EXPORTS = (
     "hstu_attn_last_error",
     "hstu_attn_fwd_variant",
     "hstu_attn_bwd",
+    "hstu_attn_bwd_variant",
 )
 
 
@@ -103,6 +104,8 @@ def load():
     lib.hstu_attn_fwd_variant.argtypes = [C.POINTER(HstuAttnFwdArgs)]
     lib.hstu_attn_bwd.restype = C.c_int
     lib.hstu_attn_bwd.argtypes = [C.POINTER(HstuAttnBwdArgs), C.c_void_p]
+    lib.hstu_attn_bwd_variant.restype = C.c_char_p
+    lib.hstu_attn_bwd_variant.argtypes = [C.POINTER(HstuAttnBwdArgs)]
     ver = lib.hstu_attn_abi_version()
     if ver != ABI_VERSION:
       raise RuntimeError(f"libhstu_attn.so has ABI {ver}, expected {ABI_VERSION}")

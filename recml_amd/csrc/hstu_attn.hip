@@ -1439,6 +1439,669 @@ __global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
 }
 
 // ---------------------------------------------------------------------------
+// Backward on the matrix cores: bf16, d = 128, the options of the MFMA forward.
+//
+// Two kernels, each recomputing the logits (recml/core/ops/hstu_ops.py:461-517):
+//
+//   hstu_bwd_dq_mfma   one workgroup per 128 query rows, keys streamed as in the forward:
+//     S^T = K Q^T, dP^T = V dO^T, dS^T = dP^T f'(S^T), dQ^T += K^T dS^T
+//   hstu_bwd_dkv_mfma  one workgroup per 128 keys, query rows streamed 32 at a time:
+//     S = Q K^T, dP = dO V^T, dV^T += dO^T P, dK^T += Q^T dS
+//
+// with f'(x) = sigma(x) (1 + x (1 - sigma(x))); the factors alpha and 1/N are applied to the
+// accumulators at the end.  In both, the operand that stays (Q and dO rows of the wave; K and V
+// rows of the wave) is held in registers as the B operand, the streamed tiles are the A operand:
+// read by rows for the first two products and through transpose reads for the last.  A streamed
+// tile is therefore read both ways, and one swizzle serves both: 16-byte chunk c of row r sits at
+// chunk c ^ swz_rt(r), which sends 16 consecutive rows to 16 different chunks (row reads) and 4
+// consecutive rows to 4 different 64-byte groups (transpose reads).  P and dS are rounded to bf16
+// for the last products like P in the forward.  Neither kernel splits its streamed range and
+// neither computes table gradients: calls that want those run the general kernels.
+// ---------------------------------------------------------------------------
+
+constexpr float LN2 = 0.6931471805599453f;
+
+__device__ __forceinline__ constexpr int swz_rt(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+// sigma and f' from u = x log2(e): returns sigma(x), stores f'(x)
+__device__ __forceinline__ float silu_grad_log2(float u, float* fprime) {
+  const float e = __builtin_amdgcn_exp2f(-u);
+  const float sg = __builtin_amdgcn_rcpf(1.0f + e);
+  *fprime = sg * __builtin_fmaf(u * LN2, 1.0f - sg, 1.0f);
+  return sg;
+}
+
+// Turns a wave's 32 x 128 accumulator (lane (col m, half hh) holds channels 32 dvb + 8g + 4hh + t of
+// row m) into whole bf16 rows through the wave's own 8 KB of LDS and stores rows [row0, row0 + 32)
+// that are below `rows`, rows at or past `n_live` as zeros.
+__device__ __forceinline__ void store_rows_128(const floatx16 (&acc)[4], float scale, unsigned char* ot, bf16_t* __restrict__ dst,
+                                               int64_t row_stride, int row0, int n_live, int rows, int lane) {
+  constexpr int D = 128, CPR = 16;
+  const int m = lane & 31, hh = lane >> 5;
+  const bool live = row0 + m < n_live;
+  unsigned char* orow = ot + m * (D * 2) + 8 * hh;
+#pragma unroll
+  for (int dvb = 0; dvb < 4; ++dvb) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint2 pko = {0u, 0u};
+      if (live) {
+        pko.x = pack_bf16(acc[dvb][4 * g + 0] * scale, acc[dvb][4 * g + 1] * scale);
+        pko.y = pack_bf16(acc[dvb][4 * g + 2] * scale, acc[dvb][4 * g + 3] * scale);
+      }
+      *(uint2*)(orow + (((4 * dvb + g) ^ (m % CPR)) * 16)) = pko;
+    }
+  }
+  const int rr = lane / CPR, cc = lane - rr * CPR;
+#pragma unroll
+  for (int r0s = 0; r0s < 32; r0s += 4) {
+    const int row = r0s + rr;
+    const uint4 val = *(const uint4*)(ot + row * (D * 2) + ((cc ^ (row % CPR)) * 16));
+    const int grow = row0 + row;
+    if (grow < rows) *(uint4*)(dst + (int64_t)grow * row_stride + cc * 8) = val;
+  }
+}
+
+template <bool POS, bool TS>
+__global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
+  constexpr int D = 128;
+  using SM = MfmaSmem<D, 2>;
+  constexpr int CPR = SM::CPR;
+  constexpr int QCH = D / 16;
+  constexpr int DVB = D / 32;
+  constexpr int NPIECE = SM::V_BYTES / 1024;
+  constexpr int LD = NPIECE / NWAVES;
+  static_assert(NPIECE % NWAVES == 0, "whole pieces per wave");
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
+  static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
+  auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
+  constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS);
+  auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
+  auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
+  float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
+
+  Work wk;
+  if (!work_of_block(p, blockIdx.x, wk)) return;
+  const int b = wk.b, h = wk.h, qt = wk.qt;
+  const Seq& s = wk.s;
+  const int q0 = qt * BM;
+  if (q0 >= s.rows || wk.chunk > 0) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m = lane & 31, hh = lane >> 5;
+  const char* __restrict__ kg = (const char*)p.k + s.bk * 2;
+  const char* __restrict__ vg = (const char*)p.v + s.bv * 2;
+  bf16_t* __restrict__ dqg = (bf16_t*)p.dq + s.bq;
+
+  if (q0 >= s.n_q) {
+    const int rows = (s.rows - q0) < BM ? (s.rows - q0) : BM;
+    const uint4 z = {0u, 0u, 0u, 0u};
+    for (int e = tid; e < rows * (D / 8); e += MFMA_THREADS) {
+      int r = e / (D / 8), c = e - r * (D / 8);
+      *(uint4*)(dqg + (int64_t)(q0 + r) * p.q_st + c * 8) = z;
+    }
+    return;
+  }
+
+  const int r0 = q0 + 32 * w;
+  const int qrow = r0 + m;
+  const bool wave_live = r0 < s.n_q;
+  const int nt = tile_steps(p, s, q0);
+  const int wave_last = !wave_live ? -1 : (p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1));
+
+  const float alpha2 = p.alpha * LOG2E;
+  const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
+  const char* wsb = (const char*)p.ws_base;
+  const uint32_t pos_off = POS ? (uint32_t)((const char*)(p.pos_scaled + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1 + 2 * POS_PAD)) - wsb) : 0u;
+  const int64_t* tsg = TS ? p.ts + s.ts0 : nullptr;
+  const int32_t* trel = TS ? p.ts_rel + ts_rel_base(p, b, s.tok0) : nullptr;
+  const int ts32 = TS ? p.ts_ok[b] : 0;
+  const uint32_t rel_off = TS ? (uint32_t)((const char*)trel - wsb) : 0u;
+  const uint32_t rng_off = TS ? (uint32_t)((const char*)(p.ts_range + 2 * ts_range_slot0(p, b, s.tok0)) - wsb) : 0u;
+
+  // direct loads of step t, as in the forward, both tiles with the two-way swizzle
+  auto dma_step = [&](int t) {
+    const int st = t % NSTAGE;
+    const int kv0 = t * BN;
+    const int last = s.n_kv - 1;
+#pragma unroll
+    for (int r = 0; r < LD; ++r) {
+      const int j = w * LD + r;
+      const int c = 64 * j + lane;
+      const int row = c / CPR, pc = c - row * CPR;
+      int grow = kv0 + row;
+      grow = grow < last ? grow : last;
+      const uint32_t sw = (uint32_t)((pc ^ swz_rt(row)) * 16);
+      lds_dma16(kg, (uint32_t)grow * kst_bytes + sw, (const unsigned char*)Ks(st) + j * 1024);
+      lds_dma16(vg, (uint32_t)grow * vst_bytes + sw, (const unsigned char*)Vs(st) + j * 1024);
+    }
+    if (POS || TS) {
+      constexpr int TS_LANE0 = POS ? SM::POS_LANES : 0;
+      const bool ts_wave = TS && (!POS || w == NWAVES - 1);
+      const int tl = lane - TS_LANE0;
+      uint32_t off = 0;
+      bool on = false;
+      if (POS && lane < SM::POS_LANES) {
+        off = pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (q0 + BM - 1) + w + 4 * lane) * 4u;
+        on = true;
+      }
+      if (ts_wave && tl >= 0 && tl < SM::TK_LANES) {
+        int tr = t;
+        const int tr_last = (s.n_ts - 1) >> 5;
+        tr = tr < tr_last ? tr : tr_last;
+        off = tl < BN / 4 ? rel_off + (uint32_t)(kv0 + 4 * tl) * 4u : rng_off + (uint32_t)tr * 8u;
+        on = true;
+      }
+      if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
+    }
+  };
+
+  if (TS) {
+    const int c = w < 3 ? w : 0;
+    const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
+    lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
+  }
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t)
+    if (t < nt) dma_step(t);
+
+  // Q and dO fragments of this lane's row (B operands): 16-byte chunk 2ks + hh of the row
+  uint4 qf[QCH], dof[QCH];
+  {
+    const char* qg = (const char*)p.q + (s.bq + (int64_t)qrow * p.q_st) * 2 + 16 * hh;
+    const char* dg = (const char*)p.dout + (s.bo + (int64_t)qrow * p.o_st) * 2 + 16 * hh;
+#pragma unroll
+    for (int ks = 0; ks < QCH; ++ks) {
+      uint4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
+      if (qrow < s.n_q) { a = *(const uint4*)(qg + 32 * ks); c = *(const uint4*)(dg + 32 * ks); }
+      qf[ks] = a;
+      dof[ks] = c;
+    }
+    // consumed here so that the wait for these loads stays out of the loop (it would be a wait for
+    // every direct load in flight as well)
+#pragma unroll
+    for (int ks = 0; ks < QCH; ++ks) {
+      asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].y), "v"(qf[ks].z), "v"(qf[ks].w));
+      asm volatile("" ::"v"(dof[ks].x), "v"(dof[ks].y), "v"(dof[ks].z), "v"(dof[ks].w));
+    }
+  }
+  int64_t tq = 0;
+  int32_t tq32 = 0;
+  if (TS) {
+    int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
+    iq = iq < 0 ? 0 : iq;
+    tq32 = trel[iq];
+    tq = tsg[iq];
+    asm volatile("" ::"v"(tq), "v"(tq32));
+  }
+
+  floatx16 acc[DVB];
+#pragma unroll
+  for (int i = 0; i < DVB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+
+  const int gk = swz_rt(m);
+  // transpose reads of K: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc),
+  // logical chunk 4 dvb + 2 (G & 1) + (i & 3) / 2.  For those rows swz_rt = 4 (i/4) + ((hh + 2x) & 3).
+  const int gi = lane & 15;
+  const int vrow = 4 * hh + (gi >> 2);
+  const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
+  const int c_lo = vc2 ^ hh, c_hi = vc2 ^ (hh + 2);
+
+  auto block = [&](int t) {
+    const int st = t % NSTAGE;
+    const int kbs = t * BN;
+    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    floatx16 sacc, dpacc;
+    {
+      uint4 kf[QCH];
+      const unsigned char* kr = (const unsigned char*)Ks(st) + m * (D * 2);
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks) kf[ks] = *(const uint4*)(kr + (((2 * ks + hh) ^ gk) * 16));
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks)
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[ks]), __builtin_bit_cast(bf16x8, qf[ks]),
+                                                       ks == 0 ? zero : sacc, 0, 0, 0);
+    }
+    {
+      uint4 vf[QCH];
+      const unsigned char* vr = (const unsigned char*)Vs(st) + m * (D * 2);
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks) vf[ks] = *(const uint4*)(vr + (((2 * ks + hh) ^ gk) * 16));
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks)
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[ks]), __builtin_bit_cast(bf16x8, dof[ks]),
+                                                        ks == 0 ? zero : dpacc, 0, 0, 0);
+    }
+    // K^T fragments for the last product
+    uint4 ktf[2][DVB];
+    {
+      const bf16_t* kr = Ks(st) + vrow * D + 4 * (gi & 1);
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb) {
+          const int cb = 4 * (dvb ^ (gi >> 2));
+          uint2 lo = lds_read_tr(kr + (16 * cc) * D + (cb + c_lo) * 8);
+          uint2 hi = lds_read_tr(kr + (16 * cc + 8) * D + (cb + c_hi) * 8);
+          ktf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
+        }
+    }
+    // lane holds S^T[kv = kbs + 8g + 4hh + tt][q = qrow], r = 4g + tt
+    float u[16];
+    if (POS) {
+      const int xb = 4 * hh + (BM - 1) - 32 * w - m;
+      const int sft = xb & 3;
+      const float* wrow = (const float*)((const unsigned char*)Wc(st) + sft * SM::POS_COPY) + (xb - sft);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float4 bv = *(const float4*)(wrow + 8 * g);
+        u[4 * g + 0] = __builtin_fmaf(sacc[4 * g + 0], alpha2, bv.x);
+        u[4 * g + 1] = __builtin_fmaf(sacc[4 * g + 1], alpha2, bv.y);
+        u[4 * g + 2] = __builtin_fmaf(sacc[4 * g + 2], alpha2, bv.z);
+        u[4 * g + 3] = __builtin_fmaf(sacc[4 * g + 3], alpha2, bv.w);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
+    }
+    if (TS) {
+      auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
+      if (ts32) {
+        const int32_t* tk = Tk(st);
+        const int2 rg = *(const int2*)(tk + BN);
+        const int d_near = tq32 - rg.y, d_far = tq32 - rg.x;
+        const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
+        const bool same = d_near >= 0 && b_near == b_far;
+        if (__builtin_amdgcn_ballot_w64(!same) == 0) {
+          const float add = TsTab[b_near];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) u[r] += add;
+        } else {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
+            u[4 * g + 0] += TsTab[bucket_f((float)(tq32 - kk.x))];
+            u[4 * g + 1] += TsTab[bucket_f((float)(tq32 - kk.y))];
+            u[4 * g + 2] += TsTab[bucket_f((float)(tq32 - kk.z))];
+            u[4 * g + 3] += TsTab[bucket_f((float)(tq32 - kk.w))];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt) {
+            int j = kbs + 8 * g + 4 * hh + tt;
+            j = j < s.n_ts ? j : s.n_ts - 1;
+            const int64_t dt = tq - tsg[j];
+            const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+            const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+            u[4 * g + tt] += TsTab[bucket_f((float)sat)];
+          }
+        }
+      }
+    }
+    float ds[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float fp;
+      silu_grad_log2(u[r], &fp);
+      ds[r] = dpacc[r] * fp;
+    }
+    // f'(0) is not 0: masked pairs are cleared after the activation's derivative
+    if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
+        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
+        ds[r] = keep ? ds[r] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      uint4 pk;
+      pk.x = pack_bf16(ds[8 * cc + 0], ds[8 * cc + 1]);
+      pk.y = pack_bf16(ds[8 * cc + 2], ds[8 * cc + 3]);
+      pk.z = pack_bf16(ds[8 * cc + 4], ds[8 * cc + 5]);
+      pk.w = pack_bf16(ds[8 * cc + 6], ds[8 * cc + 7]);
+      const bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
+#pragma unroll
+      for (int dvb = 0; dvb < DVB; ++dvb)
+        acc[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ktf[cc][dvb]), pb, acc[dvb], 0, 0, 0);
+    }
+  };
+
+  auto wait_step = [&](int t) {
+    int younger = nt - 1 - t;
+    younger = younger > NSTAGE - 2 ? NSTAGE - 2 : younger;
+    if (younger >= 2) HSTU_WAIT_VMCNT(2 * NDMA);
+    else if (younger == 1) HSTU_WAIT_VMCNT(NDMA);
+    else HSTU_WAIT_VMCNT(0);
+  };
+
+  wait_step(0);
+  __syncthreads();
+  for (int t = 0; t < nt; ++t) {
+    if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
+    if (t * BN <= wave_last) block(t);
+    if (t + 1 < nt) wait_step(t + 1);
+    __syncthreads();
+  }
+
+  // dQ^T[d][q] -> rows of dq (the ring is free: the loop ended on a barrier, no load is in flight)
+  store_rows_128(acc, p.alpha * p.inv_n, smem + w * (32 * D * 2), dqg, p.q_st, r0, s.n_q, s.rows, lane);
+}
+
+template <bool POS, bool TS>
+__global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Params p) {
+  constexpr int D = 128;
+  using SM = MfmaSmem<D, 2>;
+  constexpr int CPR = SM::CPR;
+  constexpr int QCH = D / 16;
+  constexpr int DVB = D / 32;
+  constexpr int NPIECE = SM::V_BYTES / 1024;
+  constexpr int LD = NPIECE / NWAVES;
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
+  static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
+  constexpr int TQ_LANES = BN / 4 + 1;     // 36 int32 query-side timestamps: rows qbs .. qbs + 35
+  static_assert(TQ_LANES * 16 <= SM::TK_BYTES, "fits the forward's timestamp slot");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // ring stage: [Q tile | dO tile], 32 rows each
+  auto Qs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
+  auto Os = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
+  constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS);
+  auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
+  auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
+  float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
+
+  Work wk;
+  if (!work_of_block(p, blockIdx.x, wk)) return;
+  const int b = wk.b, h = wk.h;
+  const Seq& s = wk.s;
+  if (wk.chunk > 0) return;
+  // The list names query tiles, the one with most keys first; here the key tile with most query
+  // rows behind it goes first: under the causal mask that is the reverse order.
+  const int n_live = (s.n_kv + BM - 1) / BM;
+  const int kt = (p.causal && wk.qt < n_live) ? n_live - 1 - wk.qt : wk.qt;
+  const int kv0 = kt * BM;
+  if (kv0 >= s.rows) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m = lane & 31, hh = lane >> 5;
+  const char* __restrict__ qg = (const char*)p.q + s.bq * 2;
+  const char* __restrict__ dog = (const char*)p.dout + s.bo * 2;
+  bf16_t* __restrict__ dkg = (bf16_t*)p.dk + s.bk;
+  bf16_t* __restrict__ dvg = (bf16_t*)p.dv + s.bv;
+
+  if (kv0 >= s.n_kv) {
+    const int rows = (s.rows - kv0) < BM ? (s.rows - kv0) : BM;
+    const uint4 z = {0u, 0u, 0u, 0u};
+    for (int e = tid; e < rows * (D / 8); e += MFMA_THREADS) {
+      int r = e / (D / 8), c = e - r * (D / 8);
+      *(uint4*)(dkg + (int64_t)(kv0 + r) * p.k_st + c * 8) = z;
+      *(uint4*)(dvg + (int64_t)(kv0 + r) * p.v_st + c * 8) = z;
+    }
+    return;
+  }
+
+  const int r0 = kv0 + 32 * w;          // first key of this wave
+  const int kcol = r0 + m;              // this lane's key
+  const bool wave_live = r0 < s.n_kv;
+  // steps: 32 query rows each; under the causal mask only rows from the tile's first key on
+  const int nt = (s.n_q + BN - 1) / BN;
+  const int t_lo = p.causal ? kv0 / BN : 0;
+  const int t_wave = p.causal ? r0 / BN : 0;   // first step with a row that sees a key of this wave
+
+  const float alpha2 = p.alpha * LOG2E;
+  const uint32_t qst_bytes = (uint32_t)p.q_st * 2u, ost_bytes = (uint32_t)p.o_st * 2u;
+  const char* wsb = (const char*)p.ws_base;
+  const uint32_t pos_off = POS ? (uint32_t)((const char*)(p.pos_scaled + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1 + 2 * POS_PAD)) - wsb) : 0u;
+  const int64_t* tsg = TS ? p.ts + s.ts0 : nullptr;
+  const int32_t* trel = TS ? p.ts_rel + ts_rel_base(p, b, s.tok0) : nullptr;
+  const int ts32 = TS ? p.ts_ok[b] : 0;
+  const uint32_t rel_off = TS ? (uint32_t)((const char*)trel - wsb) : 0u;
+
+  auto dma_step = [&](int t) {
+    const int st = t % NSTAGE;
+    const int qbs = t * BN;
+    const int last = s.n_q - 1;
+#pragma unroll
+    for (int r = 0; r < LD; ++r) {
+      const int j = w * LD + r;
+      const int c = 64 * j + lane;
+      const int row = c / CPR, pc = c - row * CPR;
+      int grow = qbs + row;
+      grow = grow < last ? grow : last;
+      const uint32_t sw = (uint32_t)((pc ^ swz_rt(row)) * 16);
+      lds_dma16(qg, (uint32_t)grow * qst_bytes + sw, (const unsigned char*)Qs(st) + j * 1024);
+      lds_dma16(dog, (uint32_t)grow * ost_bytes + sw, (const unsigned char*)Os(st) + j * 1024);
+    }
+    if (POS || TS) {
+      // wave c writes position-window copy c: window[x + c], window[x] = pos[(L-1) + kv0 - (qbs+31) + x]
+      // (table index >= POS_PAD - 31 > 0); behind the last wave's copy, 36 int32 timestamps from row qbs on
+      constexpr int TS_LANE0 = POS ? SM::POS_LANES : 0;
+      const bool ts_wave = TS && (!POS || w == NWAVES - 1);
+      const int tl = lane - TS_LANE0;
+      uint32_t off = 0;
+      bool on = false;
+      if (POS && lane < SM::POS_LANES) {
+        off = pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (qbs + BN - 1) + w + 4 * lane) * 4u;
+        on = true;
+      }
+      if (ts_wave && tl >= 0 && tl < TQ_LANES) {
+        off = rel_off + (uint32_t)(qbs + 4 * tl) * 4u;
+        on = true;
+      }
+      if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
+    }
+  };
+
+  if (TS) {
+    const int c = w < 3 ? w : 0;
+    const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
+    lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
+  }
+#pragma unroll
+  for (int t = 0; t < NSTAGE - 1; ++t)
+    if (t_lo + t < nt) dma_step(t_lo + t);
+
+  // K and V fragments of this lane's key (B operands)
+  uint4 kfr[QCH], vfr[QCH];
+  {
+    const char* kp = (const char*)p.k + (s.bk + (int64_t)kcol * p.k_st) * 2 + 16 * hh;
+    const char* vp = (const char*)p.v + (s.bv + (int64_t)kcol * p.v_st) * 2 + 16 * hh;
+#pragma unroll
+    for (int ks = 0; ks < QCH; ++ks) {
+      uint4 a = {0u, 0u, 0u, 0u}, c = {0u, 0u, 0u, 0u};
+      if (kcol < s.n_kv) { a = *(const uint4*)(kp + 32 * ks); c = *(const uint4*)(vp + 32 * ks); }
+      kfr[ks] = a;
+      vfr[ks] = c;
+    }
+#pragma unroll
+    for (int ks = 0; ks < QCH; ++ks) {
+      asm volatile("" ::"v"(kfr[ks].x), "v"(kfr[ks].y), "v"(kfr[ks].z), "v"(kfr[ks].w));
+      asm volatile("" ::"v"(vfr[ks].x), "v"(vfr[ks].y), "v"(vfr[ks].z), "v"(vfr[ks].w));
+    }
+  }
+  int64_t tk = 0;
+  int32_t tk32 = 0;
+  if (TS) {
+    int ik = kcol < s.n_ts ? kcol : s.n_ts - 1;
+    ik = ik < 0 ? 0 : ik;
+    tk32 = trel[ik];     // meaningless when !ts32, and then unused
+    tk = tsg[ik];
+    asm volatile("" ::"v"(tk), "v"(tk32));
+  }
+
+  floatx16 dka[DVB], dva[DVB];
+#pragma unroll
+  for (int i = 0; i < DVB; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dka[i][r] = 0.f; dva[i][r] = 0.f; }
+
+  const int gk = swz_rt(m);
+  const int gi = lane & 15;
+  const int vrow = 4 * hh + (gi >> 2);
+  const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
+  const int c_lo = vc2 ^ hh, c_hi = vc2 ^ (hh + 2);
+
+  // One block: 32 query rows against this wave's 32 keys.  Lane (key m, half hh) holds
+  // S[q = qbs + 8g + 4hh + tt][kcol], r = 4g + tt.
+  auto block = [&](int t) {
+    const int st = t % NSTAGE;
+    const int qbs = t * BN;
+    const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    floatx16 sacc, dpacc;
+    {
+      uint4 af[QCH];
+      const unsigned char* ar = (const unsigned char*)Qs(st) + m * (D * 2);
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks)
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, kfr[ks]),
+                                                       ks == 0 ? zero : sacc, 0, 0, 0);
+    }
+    {
+      uint4 af[QCH];
+      const unsigned char* ar = (const unsigned char*)Os(st) + m * (D * 2);
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
+#pragma unroll
+      for (int ks = 0; ks < QCH; ++ks)
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, vfr[ks]),
+                                                        ks == 0 ? zero : dpacc, 0, 0, 0);
+    }
+    float u[16];
+    if (POS) {
+      // pair (q = qbs + 8g + 4hh + tt, key): window index 32w + m + 31 - 8g - 4hh - tt; the four tt of a
+      // group are four consecutive entries, read as one float4 from the copy that aligns them
+      const int a0 = 32 * w + m + 28 - 4 * hh;
+      const int sft = a0 & 3;
+      const float* wrow = (const float*)((const unsigned char*)Wc(st) + sft * SM::POS_COPY) + (a0 - sft);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float4 bv = *(const float4*)(wrow - 8 * g);
+        u[4 * g + 0] = __builtin_fmaf(sacc[4 * g + 0], alpha2, bv.w);
+        u[4 * g + 1] = __builtin_fmaf(sacc[4 * g + 1], alpha2, bv.z);
+        u[4 * g + 2] = __builtin_fmaf(sacc[4 * g + 2], alpha2, bv.y);
+        u[4 * g + 3] = __builtin_fmaf(sacc[4 * g + 3], alpha2, bv.x);
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
+    }
+    if (TS) {
+      auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
+      const int32_t* tqs = Tq(st);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        // row i's logit takes the timestamp of row min(i + 1, last)
+        int iq = qbs + 8 * (r >> 2) + 4 * hh + (r & 3) + 1;
+        iq = iq < s.n_ts - 1 ? iq : s.n_ts - 1;
+        iq = iq < qbs ? qbs : iq;                 // only for rows past the sequence (masked below)
+        int32_t sat;
+        if (ts32) {
+          sat = tqs[iq - qbs] - tk32;
+        } else {
+          const int64_t dt = tsg[iq] - tk;
+          const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+          sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+        }
+        u[r] += TsTab[bucket_f((float)sat)];
+      }
+    }
+    // transposed fragments of dO (for dV) and of Q (for dK)
+    uint4 otf[2][DVB], qtf[2][DVB];
+    {
+      const bf16_t* orr = Os(st) + vrow * D + 4 * (gi & 1);
+      const bf16_t* qrr = Qs(st) + vrow * D + 4 * (gi & 1);
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb) {
+          const int cb = 4 * (dvb ^ (gi >> 2));
+          uint2 lo = lds_read_tr(orr + (16 * cc) * D + (cb + c_lo) * 8);
+          uint2 hi = lds_read_tr(orr + (16 * cc + 8) * D + (cb + c_hi) * 8);
+          otf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
+          lo = lds_read_tr(qrr + (16 * cc) * D + (cb + c_lo) * 8);
+          hi = lds_read_tr(qrr + (16 * cc + 8) * D + (cb + c_hi) * 8);
+          qtf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
+        }
+    }
+    float pv[16], ds[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float fp;
+      const float sg = silu_grad_log2(u[r], &fp);
+      pv[r] = u[r] * sg;
+      ds[r] = dpacc[r] * fp;
+    }
+    // rows past the sequence hold a repeat of the last row: they are masked like the rest
+    if ((p.causal && qbs < r0 + 31) || (qbs + 32 > s.n_q) || (r0 + 32 > s.n_kv)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int qi = qbs + 8 * (r >> 2) + 4 * hh + (r & 3);
+        const bool keep = (qi < s.n_q) && (kcol < s.n_kv) && (!p.causal || kcol <= qi);
+        pv[r] = keep ? pv[r] : 0.f;
+        ds[r] = keep ? ds[r] : 0.f;
+      }
+    }
+#pragma unroll
+    for (int cc = 0; cc < 2; ++cc) {
+      uint4 pk, dk4;
+      pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
+      pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
+      pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
+      pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
+      dk4.x = pack_bf16(ds[8 * cc + 0], ds[8 * cc + 1]);
+      dk4.y = pack_bf16(ds[8 * cc + 2], ds[8 * cc + 3]);
+      dk4.z = pack_bf16(ds[8 * cc + 4], ds[8 * cc + 5]);
+      dk4.w = pack_bf16(ds[8 * cc + 6], ds[8 * cc + 7]);
+      const bf16x8 pb = __builtin_bit_cast(bf16x8, pk), db = __builtin_bit_cast(bf16x8, dk4);
+#pragma unroll
+      for (int dvb = 0; dvb < DVB; ++dvb) {
+        dva[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, otf[cc][dvb]), pb, dva[dvb], 0, 0, 0);
+        dka[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qtf[cc][dvb]), db, dka[dvb], 0, 0, 0);
+      }
+    }
+  };
+
+  auto wait_step = [&](int t) {
+    int younger = nt - 1 - t;
+    younger = younger > NSTAGE - 2 ? NSTAGE - 2 : younger;
+    if (younger >= 2) HSTU_WAIT_VMCNT(2 * NDMA);
+    else if (younger == 1) HSTU_WAIT_VMCNT(NDMA);
+    else HSTU_WAIT_VMCNT(0);
+  };
+
+  wait_step(t_lo);
+  __syncthreads();
+  for (int t = t_lo; t < nt; ++t) {
+    if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
+    if (wave_live && t >= t_wave) block(t);
+    if (t + 1 < nt) wait_step(t + 1);
+    __syncthreads();
+  }
+
+  unsigned char* ot = smem + w * (32 * D * 2);
+  store_rows_128(dka, p.alpha * p.inv_n, ot, dkg, p.k_st, r0, s.n_kv, s.rows, lane);
+  store_rows_128(dva, p.inv_n * (1.0f / LOG2E), ot, dvg, p.v_st, r0, s.n_kv, s.rows, lane);
+}
+
+// ---------------------------------------------------------------------------
 // Host side: validation, dispatch, C ABI.
 // ---------------------------------------------------------------------------
 
@@ -1544,7 +2207,7 @@ struct WorkspacePlan {
   size_t total() const { return bias_total() + sched_bytes + partial_bytes; }
 };
 
-WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
+WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) {
   WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const Variant var = pick_variant(a);
   if (var != V_MFMA_BF16 && var != V_MFMA_FP8) return w;
@@ -1559,7 +2222,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
   const bool jag = a->layout == HSTU_LAYOUT_JAGGED;
   const long long tiles_est = (long long)a->H * (jag ? (a->total_tokens / BM + a->B) : (long long)a->B * n_qtiles);
   w.entries_per_bh = n_qtiles;
-  if (tiles_est < 1024 && steps_max > 16) {
+  if (allow_split && tiles_est < 1024 && steps_max > 16) {
     w.split_steps = (steps_max + MAX_CHUNKS - 1) / MAX_CHUNKS;
     w.split_steps = w.split_steps < 16 ? 16 : w.split_steps;
     // first tile with more steps than that (a causal tile qt has up to 4 (qt + 1) steps)
@@ -1589,8 +2252,8 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a) {
     const size_t tiles = by_token ? (size_t)(a->total_tokens >> 5) + (size_t)a->B + tiles_per_seq : (size_t)a->B * tiles_per_seq;
     w.tab_bytes = up(((size_t)a->ts_heads + 1) * TS_TAB_LEN * sizeof(float));   // scaled tables, then the thresholds
     w.ok_bytes = up((size_t)a->B * sizeof(int32_t));
-    // the kernel fetches whole 16-byte pieces: up to 31 timestamps and one range past the end
-    w.rel_bytes = up(n_ts * sizeof(int32_t) + 128);
+    // the kernels fetch whole 16-byte pieces: up to 35 timestamps and one range past the end
+    w.rel_bytes = up(n_ts * sizeof(int32_t) + 160);
     w.range_bytes = up(tiles * 2 * sizeof(int32_t) + 16);
   }
   return w;
@@ -1708,6 +2371,96 @@ int launch_mfma(const Params& p, hipStream_t st) {
   return launch_mfma_d<32, F8>(p, st);
 }
 
+
+// Points the workspace fields of `q` into the caller's buffer as `ws` lays it out and enqueues the
+// kernel that fills it (unless the caller says it is filled already).
+int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params& q, hipStream_t st) {
+  q.split_steps = ws.split_steps;
+  q.qt_split = ws.qt_split;
+  q.entries_per_bh = ws.entries_per_bh;
+  if (!ws.total()) return HSTU_OK;
+  if (!args->workspace || args->workspace_bytes < ws.total())
+    return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes needed (see hstu_attn_fwd_workspace_bytes), got %zu",
+                ws.total(), args->workspace ? args->workspace_bytes : (size_t)0);
+  if (((uintptr_t)args->workspace & 255u) != 0) return fail(HSTU_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  char* base = (char*)args->workspace;
+  if (ws.bias_total() >= (1ull << 32)) return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes is beyond what the kernel addresses", ws.bias_total());
+  float* pos_out = ws.pos_bytes ? (float*)base : nullptr;
+  float* tab_out = ws.tab_bytes ? (float*)(base + ws.pos_bytes) : nullptr;
+  int32_t* ok_out = ws.ok_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes) : nullptr;
+  int32_t* rel_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes);
+  int32_t* range_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes);
+  q.ws_base = base;
+  int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
+  q.sched = sched_out;
+  q.items_max = ws.items_max;
+  q.split_max = ws.split_max;
+  q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
+  q.ts_scaled = tab_out;
+  q.ts_thr = tab_out ? (const int32_t*)(tab_out + (size_t)q.ts_heads * TS_TAB_LEN) : nullptr;
+  q.pos_scaled = pos_out;
+  q.ts_ok = ok_out;
+  q.ts_rel = rel_out;
+  q.ts_range = range_out;
+  const long long blocks_pos = ws.pos_bytes ? ((long long)q.pos_heads * (2 * q.L - 1 + 2 * POS_PAD) + 255) / 256 : 0;
+  const long long blocks_ts = ws.ok_bytes ? q.B : 0;
+  long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
+  blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
+  if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
+  if ((ws.bias_total() || ws.sched_bytes) && !(args->flags & HSTU_FWD_WORKSPACE_PREPARED)) {
+    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
+  }
+  return HSTU_OK;
+}
+
+// The matrix-core backward: bf16 with d = 128 under the conditions of the matrix-core forward, no
+// table gradients, 16-byte aligned gradient buffers, and the forward's workspace at hand.
+bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
+  HstuAttnFwdArgs f = b->fwd;
+  f.out = (void*)b->dout;
+  if (f.qk_dtype != HSTU_DTYPE_BF16 || f.d_qk != 128 || !mfma_eligible(&f)) return false;
+  if (b->dpos_tab || b->dts_tab) return false;
+  if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
+  // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
+  if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
+      f.q_stride_t <= 0 || f.o_stride_t <= 0) return false;
+  const WorkspacePlan ws = plan_workspace(&f, false);
+  return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
+}
+
+template <bool POS, bool TS>
+int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
+  const int smem = MfmaSmem<128, 2>::total(POS, TS);
+  static int granted_q[64], granted_kv[64];
+  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<POS, TS>, smem, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<POS, TS>, smem, granted_kv)) return rc;
+  const long long blocks = mfma_grid(p);
+  if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
+  hipLaunchKernelGGL((hstu_bwd_dq_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
+  return HSTU_OK;
+}
+
+int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
+  HstuAttnFwdArgs f = b->fwd;
+  f.out = (void*)b->dout;
+  f.flags &= ~HSTU_FWD_WORKSPACE_PREPARED;   // the backward lays the work list out without key-range splits
+  const WorkspacePlan ws = plan_workspace(&f, false);
+  Params q = p;
+  if (int rc = setup_workspace(&f, ws, q, st)) return rc;
+  const bool pos = q.pos_tab != nullptr, ts = q.ts_tab != nullptr;
+  if (pos && ts) return launch_bwd_mfma_inst<true, true>(q, st);
+  if (pos) return launch_bwd_mfma_inst<true, false>(q, st);
+  if (ts) return launch_bwd_mfma_inst<false, true>(q, st);
+  return launch_bwd_mfma_inst<false, false>(q, st);
+}
+
 }  // namespace
 
 extern "C" {
@@ -1732,6 +2485,15 @@ const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {
   }
 }
 
+const char* hstu_attn_bwd_variant(const HstuAttnBwdArgs* args) {
+  if (!args || args->struct_size != sizeof(HstuAttnBwdArgs) || args->version != HSTU_ATTN_ABI_VERSION) return "invalid";
+  HstuAttnFwdArgs probe = args->fwd;
+  if (!probe.out) probe.out = (void*)args->dout;
+  if (validate(&probe) != HSTU_OK || probe.qk_dtype == HSTU_DTYPE_FP8_E4M3FN) return "invalid";
+  if (bwd_mfma_eligible(args)) return "hstu_bwd_mfma_bf16";
+  return probe.qk_dtype == HSTU_DTYPE_FP32 ? "hstu_bwd_general<float>" : "hstu_bwd_general<bf16>";
+}
+
 int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {
   if (!args) return fail(HSTU_ERR_NULL, "args is null");
   if (args->struct_size != sizeof(HstuAttnBwdArgs) || args->version != HSTU_ATTN_ABI_VERSION)
@@ -1751,6 +2513,7 @@ int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {
   p.dout = args->dout; p.dq = args->dq; p.dk = args->dk; p.dv = args->dv;
   p.dpos = args->dpos_tab; p.dts = args->dts_tab;
   hipStream_t st = (hipStream_t)stream;
+  if (bwd_mfma_eligible(args)) return launch_bwd_mfma(args, p, st);
   return f->qk_dtype == HSTU_DTYPE_FP32 ? launch_bwd<float>(p, st) : launch_bwd<bf16_t>(p, st);
 }
 
@@ -1769,44 +2532,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
       const bool f8 = args->qk_dtype == HSTU_DTYPE_FP8_E4M3FN;
       const WorkspacePlan ws = plan_workspace(args);
       Params q = p;
-      q.split_steps = ws.split_steps;
-      q.qt_split = ws.qt_split;
-      q.entries_per_bh = ws.entries_per_bh;
-      if (ws.total()) {
-        if (!args->workspace || args->workspace_bytes < ws.total())
-          return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes needed (see hstu_attn_fwd_workspace_bytes), got %zu",
-                      ws.total(), args->workspace ? args->workspace_bytes : (size_t)0);
-        if (((uintptr_t)args->workspace & 255u) != 0) return fail(HSTU_ERR_WORKSPACE, "workspace must be 256-byte aligned");
-        char* base = (char*)args->workspace;
-        if (ws.bias_total() >= (1ull << 32)) return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes is beyond what the kernel addresses", ws.bias_total());
-        float* pos_out = ws.pos_bytes ? (float*)base : nullptr;
-        float* tab_out = ws.tab_bytes ? (float*)(base + ws.pos_bytes) : nullptr;
-        int32_t* ok_out = ws.ok_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes) : nullptr;
-        int32_t* rel_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes);
-        int32_t* range_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes);
-        q.ws_base = base;
-        int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
-        q.sched = sched_out;
-        q.items_max = ws.items_max;
-        q.split_max = ws.split_max;
-        q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
-        q.ts_scaled = tab_out;
-        q.ts_thr = tab_out ? (const int32_t*)(tab_out + (size_t)p.ts_heads * TS_TAB_LEN) : nullptr;
-        q.pos_scaled = pos_out;
-        q.ts_ok = ok_out;
-        q.ts_rel = rel_out;
-        q.ts_range = range_out;
-        const long long blocks_pos = ws.pos_bytes ? ((long long)p.pos_heads * (2 * p.L - 1 + 2 * POS_PAD) + 255) / 256 : 0;
-        const long long blocks_ts = ws.ok_bytes ? p.B : 0;
-        long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
-        blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
-        if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
-        if ((ws.bias_total() || ws.sched_bytes) && !(args->flags & HSTU_FWD_WORKSPACE_PREPARED)) {
-          hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out);
-          hipError_t e = hipGetLastError();
-          if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
-        }
-      }
+      if (int rc2 = setup_workspace(args, ws, q, st)) return rc2;
       if (int rc2 = f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st)) return rc2;
       const long long cb = q.split_steps > 0 ? mfma_grid(q, true) : 0;
       if (cb > 0) {

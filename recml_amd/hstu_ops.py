@@ -335,14 +335,15 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
                        n=None, alpha=1.0, causal=True, pos_bias=None,
                        timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                        q_segment_ids=None, kv_segment_ids=None,
-                       sliding_window_size=None, mask=None, bias=None):
+                       sliding_window_size=None, mask=None, bias=None,
+                       table_grads=True, _variant_out=None):
   """Gradients of sum(hstu_attention(q, k, v, ...) * dout).
 
   Same arguments as hstu_attention (fp32 or bf16; not fp8).  Returns
   (dq, dk, dv, dpos_bias, dts_bias): dq, dk, dv shaped and typed like q, k, v;
   the table gradients fp32 and shaped like the tables (None for a table that
-  was not given).  Math of the reference's backward kernel
-  (recml/core/ops/hstu_ops.py:417-548).
+  was not given, and for both with table_grads=False).  Math of the reference's
+  backward kernel (recml/core/ops/hstu_ops.py:417-548).
   """
   for name, t in (("q", q), ("k", k), ("v", v), ("dout", dout)):
     _check_gpu(name, t)
@@ -368,13 +369,15 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   ba.fwd = fa
   ba.dout, ba.dq, ba.dk, ba.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
   dpos = dts = None
-  if pos_bias is not None:
+  if pos_bias is not None and table_grads:
     dpos = torch.zeros((fa.pos_heads, 2 * fa.L - 1), dtype=torch.float32, device=q.device)
     ba.dpos_tab = dpos.data_ptr()
-  if ts_bias is not None:
+  if ts_bias is not None and table_grads:
     dts = torch.zeros((fa.ts_heads, fa.ts_num_buckets + 1), dtype=torch.float32, device=q.device)
     ba.dts_tab = dts.data_ptr()
   lib = _lib.load()
+  if _variant_out is not None:
+    _variant_out.append(lib.hstu_attn_bwd_variant(C.byref(ba)).decode())
   with torch.cuda.device(q.device):
     stream = torch.cuda.current_stream(q.device).cuda_stream
     rc = lib.hstu_attn_bwd(C.byref(ba), C.c_void_p(stream))
@@ -408,7 +411,10 @@ class _HstuAttentionFn(torch.autograd.Function):
     rest = saved[3:]
     pos = rest.pop(0) if ctx.has[0] else None
     ts = rest.pop(0) if ctx.has[1] else None
-    dq, dk, dv, dpos, dts = hstu_attention_bwd(q, k, v, dout.contiguous(), pos_bias=pos, ts_bias=ts, **ctx.kwargs)
+    # needs_input_grad follows forward's arguments: q, k, v, pos_bias, ts_bias, kwargs
+    want_tables = (pos is not None and ctx.needs_input_grad[3]) or (ts is not None and ctx.needs_input_grad[4])
+    dq, dk, dv, dpos, dts = hstu_attention_bwd(q, k, v, dout.contiguous(), pos_bias=pos, ts_bias=ts,
+                                               table_grads=want_tables, **ctx.kwargs)
     cast = lambda g, t: None if g is None else g.to(t.dtype)
     return dq, dk, dv, cast(dpos, pos) if pos is not None else None, cast(dts, ts) if ts is not None else None, None
 

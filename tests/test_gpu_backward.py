@@ -95,3 +95,75 @@ def test_autograd_function(gpu):
   want = O.hstu_attention_bwd_ref(n(q), n(k), n(v), n(dout), seq_lens=lens, pos_tab=n(pos))
   for name, g, w in zip(("dq", "dk", "dv", "dpos"), (q.grad, k.grad, v.grad, pos.grad), want):
     assert _rel(n(g), w) <= 2e-5, name
+
+
+def _boundary_flags(ts, lens, causal):
+  """Query rows / key columns that have a pair whose time delta is a boundary case of the bucket
+  law: there the kernel's fp32 evaluation may take the neighbouring table entry."""
+  B, L = ts.shape
+  rows, cols = np.zeros((B, L), bool), np.zeros((B, L), bool)
+  for b in range(B):
+    n = int(lens[b])
+    near = O.near_bucket_boundary(O.time_delta(ts[b:b + 1, :n])[0], 0.301)
+    if causal:
+      near &= np.tril(np.ones_like(near, dtype=bool))
+    rows[b, :n], cols[b, :n] = near.any(1), near.any(0)
+  return rows, cols
+
+
+@pytest.mark.parametrize("name,B,L,H,lens,pos,ts,causal,jagged", [
+    ("full-length", 2, 256, 2, None, False, False, True, False),
+    ("lengths", 3, 300, 2, [300, 129, 1], False, False, True, False),
+    ("non-causal", 2, 200, 1, [200, 77], False, False, False, False),
+    ("pos", 3, 300, 2, [300, 129, 33], True, False, True, False),
+    ("ts", 3, 300, 2, [300, 129, 33], False, True, True, False),
+    ("pos+ts jagged", 4, 420, 2, [420, 129, 33, 256], True, True, True, True),
+    ("pos+ts non-causal", 2, 200, 2, [200, 100], True, True, False, False),
+])
+def test_backward_matrix_core_kernels(gpu, name, B, L, H, lens, pos, ts, causal, jagged):
+  """bf16, d = 128, no table gradients: the matrix-core pair of kernels, checked against the oracle."""
+  rng = np.random.default_rng(31)
+  d = 128
+  bf = torch.bfloat16
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  full = np.full((B,), L, np.int32)
+  ln = full if lens is None else np.array(lens, np.int32)
+  kw, gk = {}, dict(causal=causal, table_grads=False)
+  if lens is not None:
+    kw["seq_lens"] = ln
+  if pos:
+    kw["pos_tab"] = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  if ts:
+    kw["ts_tab"] = (rng.standard_normal((129,)) * 0.3).astype(np.float32)
+    t = 1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, (B, L))), axis=1).astype(np.int64)
+    for b in range(B):
+      t[b, ln[b]:] = t[b, ln[b] - 1]     # what the jagged layout's clamp to the last row sees
+    kw["timestamps"] = t
+    gk["ts_bias"] = _dev(kw["ts_tab"])
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, causal=causal, **kw)
+  variant = []
+  gk["_variant_out"] = variant
+  if jagged:
+    pack = lambda x: O.padded_to_jagged(x, ln)
+    (qj, off), (kj, _), (vj, _), (dj, _) = pack(q), pack(k), pack(v), pack(dout)
+    if ts:
+      gk["timestamps"] = _dev(np.concatenate([kw["timestamps"][b, :ln[b]] for b in range(B)]))
+    got = recml_amd.hstu_attention_bwd(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), _dev(dj, bf),
+                                       seq_offsets=_dev(off.astype(np.int32)), max_len=L, **gk)
+    got = [O.jagged_to_padded(g.float().cpu().numpy(), off, L) for g in got[:3]]
+  else:
+    if ts:
+      gk["timestamps"] = _dev(kw["timestamps"])
+    if lens is not None:
+      gk["seq_lens"] = _dev(ln)
+    got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), **gk)
+    got = [g.float().cpu().numpy() for g in got[:3]]
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  rows, cols = _boundary_flags(kw["timestamps"], ln, causal) if ts else (np.zeros((B, L), bool),) * 2
+  for nm, g, w, edge in zip(("dq", "dk", "dv"), got, want[:3], (rows, cols, cols)):
+    err = np.abs(g - w).max(axis=(2, 3)) / np.abs(w).max()
+    assert err[~edge].max() <= 2e-2, (nm, err[~edge].max())
+    assert not edge.any() or err[edge].max() <= 1e-1, (nm, err[edge].max())
+    for b in range(B):
+      assert (g[b, ln[b]:] == 0).all(), nm

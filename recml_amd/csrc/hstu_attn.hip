@@ -1455,8 +1455,8 @@ __global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
 // tile is therefore read both ways, and one swizzle serves both: 16-byte chunk c of row r sits at
 // chunk c ^ swz_rt(r), which sends 16 consecutive rows to 16 different chunks (row reads) and 4
 // consecutive rows to 4 different 64-byte groups (transpose reads).  P and dS are rounded to bf16
-// for the last products like P in the forward.  Neither kernel splits its streamed range and
-// neither computes table gradients: calls that want those run the general kernels.
+// for the last products like P in the forward.  Neither kernel splits its streamed range.  The
+// table gradients, when wanted, come from the dQ kernel, which sees every pair once.
 // ---------------------------------------------------------------------------
 
 constexpr float LN2 = 0.6931471805599453f;
@@ -1502,7 +1502,16 @@ __device__ __forceinline__ void store_rows_128(const floatx16 (&acc)[4], float s
   }
 }
 
-template <bool POS, bool TS>
+// Extra LDS of the dQ kernel when it also sums table gradients: 256 diagonal sums, then one sum per bucket
+constexpr int BWD_TG_BYTES = (256 + TS_TAB_LEN) * 4;
+
+// TG: also accumulate the table gradients.  Every pair adds its dS to the entry of each table its
+// logit read.  Position table: pair (q, key) of the tile belongs to diagonal x = key - q + (q0 + 127)
+// >= 0; the workgroup sums diagonals in a 256-entry LDS ring (LDS atomics), and since step t only
+// touches x in [32 t, 32 t + 160), the 32 diagonals below 32 (t + 1) are final after step t: one
+// wave then adds them to the table in memory and clears them.  Bucket table: one LDS sum per bucket,
+// added to memory at the end.
+template <bool POS, bool TS, bool TG>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
   constexpr int D = 128;
   using SM = MfmaSmem<D, 2>;
@@ -1523,6 +1532,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
+  float* Dg = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
+  float* TsG = Dg + 256;
+  const bool want_dpos = TG && POS && p.dpos != nullptr, want_dts = TG && TS && p.dts != nullptr;
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -1610,6 +1622,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t < nt) dma_step(t);
+  if (TG) {
+    for (int i = tid; i < 256 + TS_TAB_LEN; i += MFMA_THREADS) Dg[i] = 0.f;
+  }
 
   // Q and dO fragments of this lane's row (B operands): 16-byte chunk 2ks + hh of the row
   uint4 qf[QCH], dof[QCH];
@@ -1696,6 +1711,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     }
     // lane holds S^T[kv = kbs + 8g + 4hh + tt][q = qrow], r = 4g + tt
     float u[16];
+    // table gradients: the buckets of this lane's 16 pairs, one byte each (bucket < TS_TAB_LEN <= 255), or
+    // one bucket for all of them (bk_one >= 0; then the same holds in every lane of the wave)
+    uint32_t bkp[4] = {0u, 0u, 0u, 0u};
+    int bk_one = -1;
     if (POS) {
       const int xb = 4 * hh + (BM - 1) - 32 * w - m;
       const int sft = xb & 3;
@@ -1724,14 +1743,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
           const float add = TsTab[b_near];
 #pragma unroll
           for (int r = 0; r < 16; ++r) u[r] += add;
+          bk_one = b_near;
         } else {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
-            u[4 * g + 0] += TsTab[bucket_f((float)(tq32 - kk.x))];
-            u[4 * g + 1] += TsTab[bucket_f((float)(tq32 - kk.y))];
-            u[4 * g + 2] += TsTab[bucket_f((float)(tq32 - kk.z))];
-            u[4 * g + 3] += TsTab[bucket_f((float)(tq32 - kk.w))];
+            const int b0 = bucket_f((float)(tq32 - kk.x)), b1 = bucket_f((float)(tq32 - kk.y));
+            const int b2 = bucket_f((float)(tq32 - kk.z)), b3 = bucket_f((float)(tq32 - kk.w));
+            u[4 * g + 0] += TsTab[b0];
+            u[4 * g + 1] += TsTab[b1];
+            u[4 * g + 2] += TsTab[b2];
+            u[4 * g + 3] += TsTab[b3];
+            if (TG) bkp[g] = (uint32_t)b0 | ((uint32_t)b1 << 8) | ((uint32_t)b2 << 16) | ((uint32_t)b3 << 24);
           }
         }
       } else {
@@ -1744,7 +1767,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
             const int64_t dt = tq - tsg[j];
             const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
             const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-            u[4 * g + tt] += TsTab[bucket_f((float)sat)];
+            const int bb = bucket_f((float)sat);
+            u[4 * g + tt] += TsTab[bb];
+            if (TG) bkp[g] = tt == 0 ? (uint32_t)bb : bkp[g] | ((uint32_t)bb << (8 * tt));
           }
         }
       }
@@ -1763,6 +1788,22 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
         const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
         ds[r] = keep ? ds[r] : 0.f;
+      }
+    }
+    if (want_dpos) {
+      const int xb = kbs + 4 * hh + (BM - 1) - 32 * w - m;    // diagonal of the pair with g = tt = 0
+#pragma unroll
+      for (int r = 0; r < 16; ++r) atomicAdd(&Dg[(xb + 8 * (r >> 2) + (r & 3)) & 255], ds[r]);
+    }
+    if (want_dts) {
+      if (bk_one >= 0) {
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sum += ds[r];
+        atomicAdd(&TsG[bk_one], sum);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) atomicAdd(&TsG[(bkp[r >> 2] >> (8 * (r & 3))) & 255u], ds[r]);
       }
     }
 #pragma unroll
@@ -1787,15 +1828,40 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     else HSTU_WAIT_VMCNT(0);
   };
 
+  // adds diagonals [x0, x0 + 32) to the table in memory and clears them (one wave)
+  auto flush_diag = [&](int x0) {
+    if (lane < 32) {
+      const int x = x0 + lane;
+      float* slot = &Dg[x & 255];
+      const float val = *slot;
+      *slot = 0.f;
+      const int idx = (p.L - 1) + x - (q0 + BM - 1);
+      if (val != 0.f && idx >= 0 && idx < 2 * p.L - 1)
+        atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, val * p.inv_n);
+    }
+  };
+
   wait_step(0);
   __syncthreads();
   for (int t = 0; t < nt; ++t) {
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
+    if (want_dpos && t > 0 && w == ((t - 1) & (NWAVES - 1))) flush_diag(32 * (t - 1));
     if (t * BN <= wave_last) block(t);
     if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
   }
 
+  if (want_dpos) {
+    // what is left after the last barrier: step nt - 1's 32 diagonals and the 128 above them
+    flush_diag(32 * (nt - 1 + w));
+    if (w == 0) flush_diag(32 * (nt - 1 + NWAVES));
+  }
+  if (want_dts) {
+    for (int e = tid; e < TS_TAB_LEN; e += MFMA_THREADS) {
+      const float val = TsG[e];
+      if (val != 0.f) atomicAdd(p.dts + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1) + (e < p.ts_nb ? e : p.ts_nb), val * p.inv_n);
+    }
+  }
   // dQ^T[d][q] -> rows of dq (the ring is free: the loop ended on a barrier, no load is in flight)
   store_rows_128(acc, p.alpha * p.inv_n, smem + w * (32 * D * 2), dqg, p.q_st, r0, s.n_q, s.rows, lane);
 }
@@ -2415,13 +2481,12 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   return HSTU_OK;
 }
 
-// The matrix-core backward: bf16 with d = 128 under the conditions of the matrix-core forward, no
-// table gradients, 16-byte aligned gradient buffers, and the forward's workspace at hand.
+// The matrix-core backward: bf16 with d = 128 under the conditions of the matrix-core forward,
+// 16-byte aligned gradient buffers, and the forward's workspace at hand.
 bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
   if (f.qk_dtype != HSTU_DTYPE_BF16 || f.d_qk != 128 || !mfma_eligible(&f)) return false;
-  if (b->dpos_tab || b->dts_tab) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
@@ -2430,15 +2495,16 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
 }
 
-template <bool POS, bool TS>
+template <bool POS, bool TS, bool TG>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<128, 2>::total(POS, TS);
+  const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
   static int granted_q[64], granted_kv[64];
-  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<POS, TS>, smem, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<POS, TS, TG>, smem_q, granted_q)) return rc;
   if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<POS, TS>, smem, granted_kv)) return rc;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_bwd_dq_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dq_mfma<POS, TS, TG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
   hipLaunchKernelGGL((hstu_bwd_dkv_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
@@ -2455,10 +2521,11 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
   Params q = p;
   if (int rc = setup_workspace(&f, ws, q, st)) return rc;
   const bool pos = q.pos_tab != nullptr, ts = q.ts_tab != nullptr;
-  if (pos && ts) return launch_bwd_mfma_inst<true, true>(q, st);
-  if (pos) return launch_bwd_mfma_inst<true, false>(q, st);
-  if (ts) return launch_bwd_mfma_inst<false, true>(q, st);
-  return launch_bwd_mfma_inst<false, false>(q, st);
+  const bool tg = (pos && q.dpos) || (ts && q.dts);
+  if (pos && ts) return tg ? launch_bwd_mfma_inst<true, true, true>(q, st) : launch_bwd_mfma_inst<true, true, false>(q, st);
+  if (pos) return tg ? launch_bwd_mfma_inst<true, false, true>(q, st) : launch_bwd_mfma_inst<true, false, false>(q, st);
+  if (ts) return tg ? launch_bwd_mfma_inst<false, true, true>(q, st) : launch_bwd_mfma_inst<false, true, false>(q, st);
+  return launch_bwd_mfma_inst<false, false, false>(q, st);
 }
 
 }  // namespace

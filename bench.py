@@ -200,15 +200,16 @@ def bench_model(args, dev):
 
 
 def bench_backward(args, w, q, k, v, kw, dev):
-  """The backward pass (general fp32-arithmetic kernels) on the same workload: one JSON line.
+  """The backward pass on the same workload, table gradients included: one JSON line.
 
   FLOPs counted: four products per unmasked pair (dV, dP, dQ, dK) = 2x the forward's; the
-  recomputation of S in both kernels is not counted."""
+  recomputation of S (and of dP in the second kernel) is not counted."""
   import torch
   import recml_amd
   from oracle import hstu_oracle as O
   dout = torch.randn(v.shape, generator=torch.Generator().manual_seed(1)).to(dev).to(v.dtype)
-  run = lambda: recml_amd.hstu_attention_bwd(q, k, v, dout, **kw)
+  variant = []
+  run = lambda: recml_amd.hstu_attention_bwd(q, k, v, dout, _variant_out=variant, **kw)
   steps, warm = max(1, args.steps // 10), max(1, args.warmup // 10)
   for _ in range(warm):
     got = run()
@@ -219,14 +220,20 @@ def bench_backward(args, w, q, k, v, kw, dev):
   torch.cuda.synchronize()
   ms = (time.perf_counter() - t0) * 1e3 / steps
   flops = 2 * w.flops
+  mfma = variant[-1] == "hstu_bwd_mfma_bf16"
+  peak = PEAK_BF16_TFLOPS if mfma else PEAK_FP32_TFLOPS
   rec = {
       "metric": "HSTU attn bwd TFLOP/s (unmasked), L=%d bf16" % w.L, "value": flops / (ms * 1e-3) / 1e12,
       "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
-      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, fp32 arithmetic",
-      "data": "synthetic", "config": {"workload": w.name + " backward", "kernel": "hstu_bwd_dq + hstu_bwd_dkv"},
-      "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                   "frac": flops / (ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, "traffic": None,
-                   "note": "fp32 FMA kernels (no matrix cores yet); time covers both kernels, the table memsets and the host call"},
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "bf16" if mfma else "bf16 storage, fp32 arithmetic",
+      "data": "synthetic",
+      "config": {"workload": w.name + " backward",
+                 "kernel": "hstu_bwd_dq_mfma + hstu_bwd_dkv_mfma" if mfma else "hstu_bwd_dq + hstu_bwd_dkv"},
+      "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                   "frac": flops / (ms * 1e-3) / 1e12 / peak, "traffic": None,
+                   "note": ("matrix-core kernels" if mfma else "fp32 FMA kernels") +
+                           "; time covers both kernels, the preparation kernel, the table memsets and the host call"},
   }
   if not args.no_cpu and w.layout == "jagged":
     # bounded sample: the numpy oracle on the shortest sequences that add up to ~5 % of the pairs

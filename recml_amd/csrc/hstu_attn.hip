@@ -1502,15 +1502,38 @@ __device__ __forceinline__ void store_rows_128(const floatx16 (&acc)[4], float s
   }
 }
 
-// Extra LDS of the dQ kernel when it also sums table gradients: 256 diagonal sums, then one sum per bucket
-constexpr int BWD_TG_BYTES = (256 + TS_TAB_LEN) * 4;
+// Extra LDS of the dQ kernel when it also sums table gradients: per wave, a ring of 256 diagonal
+// sums and one sum per bucket
+constexpr int BWD_TG_BYTES = NWAVES * (256 + TS_TAB_LEN) * 4;
+
+// v of the lane `CTRL` names (data-parallel-primitive controls of the vector ALU: 0x110 + n = n lanes
+// down within a row of 16, 0x142 / 0x143 = lane 15 of the previous row / lane 31 to the rows that
+// ROW_MASK selects); 0 where there is no such lane or row
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
+// sum of v over the 64 lanes, the same value in every lane (all lanes must be active)
+__device__ __forceinline__ float wave_sum(float v) {
+  v += dpp_f<0x111>(v);
+  v += dpp_f<0x112>(v);
+  v += dpp_f<0x114>(v);
+  v += dpp_f<0x118>(v);
+  v += dpp_f<0x142, 0xa>(v);
+  v += dpp_f<0x143, 0xc>(v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
 
 // TG: also accumulate the table gradients.  Every pair adds its dS to the entry of each table its
-// logit read.  Position table: pair (q, key) of the tile belongs to diagonal x = key - q + (q0 + 127)
-// >= 0; the workgroup sums diagonals in a 256-entry LDS ring (LDS atomics), and since step t only
-// touches x in [32 t, 32 t + 160), the 32 diagonals below 32 (t + 1) are final after step t: one
-// wave then adds them to the table in memory and clears them.  Bucket table: one LDS sum per bucket,
-// added to memory at the end.
+// logit read; LDS float atomics turned out to cost about 4 cycles per lane, so the sums are formed
+// in registers first and each wave keeps its own LDS accumulators, updated without atomics.
+// Position table: pair (q, key) of a wave lies on diagonal X = key - q + (r0 + 31) >= 0.  A block's
+// 32 x 32 pairs are brought onto their 63 diagonals by lane permutes (see the block), one value per
+// lane, and added to a ring of 256 sums.  Block t only touches X in [32 t, 32 t + 63), so
+// everything below 32 (t + 1) is final after it: every fourth block the wave adds 128 finished
+// diagonals to the table in memory and clears them.
+// Bucket table: where each lane has one bucket for the whole block (or two neighbours), lanes with
+// the same bucket are summed across the wave; only blocks with more buckets per lane use atomics.
 template <bool POS, bool TS, bool TG>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
   constexpr int D = 128;
@@ -1532,8 +1555,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
-  float* Dg = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
-  float* TsG = Dg + 256;
+  const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
+  float* TgBase = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
   const bool want_dpos = TG && POS && p.dpos != nullptr, want_dts = TG && TS && p.dts != nullptr;
 
   Work wk;
@@ -1618,12 +1641,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     const int c = w < 3 ? w : 0;
     const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
     lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
+    lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
   }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t < nt) dma_step(t);
   if (TG) {
-    for (int i = tid; i < 256 + TS_TAB_LEN; i += MFMA_THREADS) Dg[i] = 0.f;
+    for (int i = tid; i < NWAVES * (256 + TS_TAB_LEN); i += MFMA_THREADS) TgBase[i] = 0.f;
   }
 
   // Q and dO fragments of this lane's row (B operands): 16-byte chunk 2ks + hh of the row
@@ -1695,26 +1719,14 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[ks]), __builtin_bit_cast(bf16x8, dof[ks]),
                                                         ks == 0 ? zero : dpacc, 0, 0, 0);
     }
-    // K^T fragments for the last product
-    uint4 ktf[2][DVB];
-    {
-      const bf16_t* kr = Ks(st) + vrow * D + 4 * (gi & 1);
-#pragma unroll
-      for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-        for (int dvb = 0; dvb < DVB; ++dvb) {
-          const int cb = 4 * (dvb ^ (gi >> 2));
-          uint2 lo = lds_read_tr(kr + (16 * cc) * D + (cb + c_lo) * 8);
-          uint2 hi = lds_read_tr(kr + (16 * cc + 8) * D + (cb + c_hi) * 8);
-          ktf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
-        }
-    }
     // lane holds S^T[kv = kbs + 8g + 4hh + tt][q = qrow], r = 4g + tt
     float u[16];
-    // table gradients: the buckets of this lane's 16 pairs, one byte each (bucket < TS_TAB_LEN <= 255), or
-    // one bucket for all of them (bk_one >= 0; then the same holds in every lane of the wave)
+    // for the table gradients: either this lane's 16 pairs are in bucket bk_lane >= 0, those with a bit
+    // in far_bits in the next one (then every lane of the wave has such a pair of buckets), or bkp holds
+    // the 16 buckets, one byte each (bucket < TS_TAB_LEN <= 255)
     uint32_t bkp[4] = {0u, 0u, 0u, 0u};
-    int bk_one = -1;
+    uint32_t far_bits = 0u;
+    int bk_lane = -1;
     if (POS) {
       const int xb = 4 * hh + (BM - 1) - 32 * w - m;
       const int sft = xb & 3;
@@ -1739,11 +1751,28 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         const int d_near = tq32 - rg.y, d_far = tq32 - rg.x;
         const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
         const bool same = d_near >= 0 && b_near == b_far;
+        const bool two = d_near >= 0 && b_far - b_near <= 1;
         if (__builtin_amdgcn_ballot_w64(!same) == 0) {
           const float add = TsTab[b_near];
 #pragma unroll
           for (int r = 0; r < 16; ++r) u[r] += add;
-          bk_one = b_near;
+          bk_lane = b_near;
+        } else if (__builtin_amdgcn_ballot_w64(!two) == 0) {
+          // at most one bucket boundary inside the tile for every lane: a key is in the farther
+          // bucket exactly when tq - tk >= thr[b_near + 1], i.e. tk <= tq - thr
+          const float add_near = TsTab[b_near], add_far = TsTab[b_near + 1];
+          const int cut = tq32 - TsThr[b_near + 1];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
+            const bool f0 = kk.x <= cut, f1 = kk.y <= cut, f2 = kk.z <= cut, f3 = kk.w <= cut;
+            u[4 * g + 0] += f0 ? add_far : add_near;
+            u[4 * g + 1] += f1 ? add_far : add_near;
+            u[4 * g + 2] += f2 ? add_far : add_near;
+            u[4 * g + 3] += f3 ? add_far : add_near;
+            if (TG) far_bits |= ((uint32_t)f0 | ((uint32_t)f1 << 1) | ((uint32_t)f2 << 2) | ((uint32_t)f3 << 3)) << (4 * g);
+          }
+          bk_lane = b_near;
         } else {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
@@ -1791,20 +1820,72 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       }
     }
     if (want_dpos) {
-      const int xb = kbs + 4 * hh + (BM - 1) - 32 * w - m;    // diagonal of the pair with g = tt = 0
+      // Pair (row m, key offset c = 8g + 4hh + tt) lies on diagonal c - m.  Lane j takes, for each of
+      // its 16 offsets, the value of row (j + c) mod 32 of its half: all 16 are then on diagonal -j or,
+      // where j + c wrapped, 32 - j.  The two sums are completed with the other half's and added to
+      // the wave's ring: lanes of the lower half own -j, lanes of the upper half 32 - j.
+      const int jj = m + 4 * hh;
+      const int half4 = (lane & 32) << 2;
+      float s_all = 0.f, s_low = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) atomicAdd(&Dg[(xb + 8 * (r >> 2) + (r & 3)) & 255], ds[r]);
+      for (int r = 0; r < 16; ++r) {
+        const int c0 = 8 * (r >> 2) + (r & 3);
+        const int addr = (((jj + c0) & 31) << 2) | half4;
+        const float rv = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(addr, __builtin_bit_cast(int, ds[r])));
+        s_all += rv;
+        s_low += (jj + c0 < 32) ? rv : 0.f;
+      }
+      const float s_high = s_all - s_low;
+      const float mine = hh ? s_high : s_low, theirs = hh ? s_low : s_high;
+      const float got = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, theirs)));
+      float* slot = TgBase + w * 256 + ((kbs + 31 - m + 32 * hh) & 255);
+      *slot += mine + got;
     }
     if (want_dts) {
-      if (bk_one >= 0) {
-        float sum = 0.f;
+      float* hist = TgBase + NWAVES * 256 + w * TS_TAB_LEN;
+      if (bk_lane >= 0) {
+        float s_near = 0.f, s_far = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sum += ds[r];
-        atomicAdd(&TsG[bk_one], sum);
+        for (int r = 0; r < 16; ++r) {
+          const bool far = (far_bits >> r) & 1u;
+          s_near += far ? 0.f : ds[r];
+          s_far += far ? ds[r] : 0.f;
+        }
+        // lanes with the same bucket are summed together, one bucket value per round
+        const bool any_far = __builtin_amdgcn_ballot_w64(far_bits != 0u) != 0;
+        bool done = false;
+        for (;;) {
+          const uint64_t act = __builtin_amdgcn_ballot_w64(!done);
+          if (act == 0) break;
+          const int leader = __builtin_ctzll(act);
+          const int b0 = __builtin_amdgcn_readlane(bk_lane, leader);
+          const bool mine = !done && bk_lane == b0;
+          const float a = wave_sum(mine ? s_near : 0.f);
+          const float c = any_far ? wave_sum(mine ? s_far : 0.f) : 0.f;
+          if (lane == 0) {
+            hist[b0] += a;
+            if (any_far) hist[b0 + 1] += c;
+          }
+          done = done || mine;
+        }
       } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) atomicAdd(&TsG[(bkp[r >> 2] >> (8 * (r & 3))) & 255u], ds[r]);
+        for (int r = 0; r < 16; ++r) atomicAdd(&hist[(bkp[r >> 2] >> (8 * (r & 3))) & 255u], ds[r]);
       }
+    }
+    // K^T fragments for the last product
+    uint4 ktf[2][DVB];
+    {
+      const bf16_t* kr = Ks(st) + vrow * D + 4 * (gi & 1);
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+        for (int dvb = 0; dvb < DVB; ++dvb) {
+          const int cb = 4 * (dvb ^ (gi >> 2));
+          uint2 lo = lds_read_tr(kr + (16 * cc) * D + (cb + c_lo) * 8);
+          uint2 hi = lds_read_tr(kr + (16 * cc + 8) * D + (cb + c_hi) * 8);
+          ktf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
+        }
     }
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
@@ -1828,37 +1909,41 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     else HSTU_WAIT_VMCNT(0);
   };
 
-  // adds diagonals [x0, x0 + 32) to the table in memory and clears them (one wave)
+  // adds diagonals [x0, x0 + 64) of this wave's ring to the table in memory and clears them
   auto flush_diag = [&](int x0) {
-    if (lane < 32) {
-      const int x = x0 + lane;
-      float* slot = &Dg[x & 255];
-      const float val = *slot;
-      *slot = 0.f;
-      const int idx = (p.L - 1) + x - (q0 + BM - 1);
-      if (val != 0.f && idx >= 0 && idx < 2 * p.L - 1)
-        atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, val * p.inv_n);
-    }
+    float* slot = TgBase + w * 256 + ((x0 + lane) & 255);
+    const float val = *slot;
+    *slot = 0.f;
+    const int idx = (p.L - 1) + (x0 + lane) - 31 - r0;
+    if (val != 0.f && idx >= 0 && idx < 2 * p.L - 1)
+      atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, val * p.inv_n);
   };
 
   wait_step(0);
   __syncthreads();
   for (int t = 0; t < nt; ++t) {
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
-    if (want_dpos && t > 0 && w == ((t - 1) & (NWAVES - 1))) flush_diag(32 * (t - 1));
-    if (t * BN <= wave_last) block(t);
+    if (t * BN <= wave_last) {
+      block(t);
+      if (want_dpos && (t & 3) == 3) {
+        flush_diag(32 * (t - 3));
+        flush_diag(32 * (t - 3) + 64);
+      }
+    }
     if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
   }
 
-  if (want_dpos) {
-    // what is left after the last barrier: step nt - 1's 32 diagonals and the 128 above them
-    flush_diag(32 * (nt - 1 + w));
-    if (w == 0) flush_diag(32 * (nt - 1 + NWAVES));
+  if (want_dpos && wave_last >= 0) {
+    // what the wave has not written out: the diagonals of its last (up to 3) blocks, then 31 more
+    const int t_done = wave_last / BN + 1;
+    flush_diag(32 * (t_done & ~3));
+    flush_diag(32 * (t_done & ~3) + 64);
   }
   if (want_dts) {
-    for (int e = tid; e < TS_TAB_LEN; e += MFMA_THREADS) {
-      const float val = TsG[e];
+    const float* hist = TgBase + NWAVES * 256 + w * TS_TAB_LEN;
+    for (int e = lane; e < TS_TAB_LEN; e += 64) {
+      const float val = hist[e];
       if (val != 0.f) atomicAdd(p.dts + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1) + (e < p.ts_nb ? e : p.ts_nb), val * p.inv_n);
     }
   }
@@ -1877,18 +1962,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
   constexpr int LD = NPIECE / NWAVES;
   constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
-  constexpr int TQ_LANES = BN / 4 + 1;     // 36 int32 query-side timestamps: rows qbs .. qbs + 35
-  static_assert(TQ_LANES * 16 <= SM::TK_BYTES, "fits the forward's timestamp slot");
+  // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
+  // (min, max) of timestamp tiles t and t + 1
+  constexpr int TQ_LANES = BN / 4 + 2;
+  constexpr int TQ_BYTES = TQ_LANES * 16;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   // ring stage: [Q tile | dO tile], 32 rows each
   auto Qs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Os = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS);
+  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0);
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
+  const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -1938,6 +2026,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
   const int32_t* trel = TS ? p.ts_rel + ts_rel_base(p, b, s.tok0) : nullptr;
   const int ts32 = TS ? p.ts_ok[b] : 0;
   const uint32_t rel_off = TS ? (uint32_t)((const char*)trel - wsb) : 0u;
+  const uint32_t rng_off = TS ? (uint32_t)((const char*)(p.ts_range + 2 * ts_range_slot0(p, b, s.tok0)) - wsb) : 0u;
 
   auto dma_step = [&](int t) {
     const int st = t % NSTAGE;
@@ -1967,7 +2056,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
         on = true;
       }
       if (ts_wave && tl >= 0 && tl < TQ_LANES) {
-        off = rel_off + (uint32_t)(qbs + 4 * tl) * 4u;
+        // the ranges of tiles (tr, tr + 1) cover rows qbs + 1 .. qbs + 32; at the end of the sequence
+        // the pair before does (what lies past the last tile only widens the range)
+        int tr = t;
+        const int tr_last = (s.n_ts - 1) >> 5;
+        tr = tr < tr_last ? tr : (tr_last > 0 ? tr_last - 1 : 0);
+        off = tl < TQ_LANES - 1 ? rel_off + (uint32_t)(qbs + 4 * tl) * 4u : rng_off + (uint32_t)tr * 8u;
         on = true;
       }
       if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
@@ -1978,6 +2072,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
     const int c = w < 3 ? w : 0;
     const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
     lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
+    lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
   }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
@@ -2072,21 +2167,43 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
     if (TS) {
       auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
       const int32_t* tqs = Tq(st);
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        // row i's logit takes the timestamp of row min(i + 1, last)
+      // row i's logit takes the timestamp of row min(i + 1, last); index into this step's 36
+      auto tq_at = [&](int r) {
         int iq = qbs + 8 * (r >> 2) + 4 * hh + (r & 3) + 1;
         iq = iq < s.n_ts - 1 ? iq : s.n_ts - 1;
-        iq = iq < qbs ? qbs : iq;                 // only for rows past the sequence (masked below)
-        int32_t sat;
-        if (ts32) {
-          sat = tqs[iq - qbs] - tk32;
+        return iq < qbs ? qbs : iq;                 // only for rows past the sequence (masked below)
+      };
+      if (ts32) {
+        // the time differences of this lane's key to the step's rows lie between those to the
+        // smallest and to the largest timestamp of the two tiles the rows come from
+        const int4 rg = *(const int4*)(tqs + 4 * (TQ_LANES - 1));
+        const int t_min = rg.x < rg.z ? rg.x : rg.z, t_max = rg.y > rg.w ? rg.y : rg.w;
+        const int d_near = t_min - tk32, d_far = t_max - tk32;
+        const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
+        const bool same = d_near >= 0 && b_near == b_far;
+        const bool two = d_near >= 0 && b_far - b_near <= 1;
+        if (__builtin_amdgcn_ballot_w64(!same) == 0) {
+          const float add = TsTab[b_near];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) u[r] += add;
+        } else if (__builtin_amdgcn_ballot_w64(!two) == 0) {
+          // one bucket boundary at most: the farther bucket exactly when tq - tk >= thr[b_near + 1]
+          const float add_near = TsTab[b_near], add_far = TsTab[b_near + 1];
+          const int thr = TsThr[b_near + 1];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) u[r] += tqs[tq_at(r) - qbs] - tk32 >= thr ? add_far : add_near;
         } else {
-          const int64_t dt = tsg[iq] - tk;
-          const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-          sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) u[r] += TsTab[bucket_f((float)(tqs[tq_at(r) - qbs] - tk32))];
         }
-        u[r] += TsTab[bucket_f((float)sat)];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int64_t dt = tsg[tq_at(r)] - tk;
+          const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
+          const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
+          u[r] += TsTab[bucket_f((float)sat)];
+        }
       }
     }
     // transposed fragments of dO (for dV) and of Q (for dK)
@@ -2501,13 +2618,14 @@ int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
   static int granted_q[64], granted_kv[64];
   if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<POS, TS, TG>, smem_q, granted_q)) return rc;
-  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<POS, TS>, smem, granted_kv)) return rc;
+  const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<POS, TS>, smem_kv, granted_kv)) return rc;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
   hipLaunchKernelGGL((hstu_bwd_dq_mfma<POS, TS, TG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;

@@ -1869,8 +1869,19 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
           done = done || mine;
         }
       } else {
+        // LDS atomics cost by the lane: neighbouring keys mostly share a bucket, so each run of equal
+        // buckets is summed first, and runs that add nothing (masked pairs) are skipped
+        float carry = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) atomicAdd(&hist[(bkp[r >> 2] >> (8 * (r & 3))) & 255u], ds[r]);
+        for (int r = 0; r < 16; ++r) {
+          const uint32_t bcur = (bkp[r >> 2] >> (8 * (r & 3))) & 255u;
+          const uint32_t bnext = r < 15 ? (bkp[(r + 1) >> 2] >> (8 * ((r + 1) & 3))) & 255u : 256u;
+          carry += ds[r];
+          if (bcur != bnext) {
+            if (carry != 0.f) atomicAdd(&hist[bcur], carry);
+            carry = 0.f;
+          }
+        }
       }
     }
     // K^T fragments for the last product

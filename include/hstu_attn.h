@@ -171,7 +171,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
  * ts_tab that are ACCUMULATED into by atomic adds: the caller zero-fills them
  * (or passes null when the table gradient is not wanted).  fp32 or bf16
  * storage, every option of the forward, fp32 arithmetic; fp8 q/k is not
- * supported.  bf16 calls with d_qk = d_v = 128 that meet the conditions of the
+ * supported.  bf16 calls that meet the conditions of the
  * matrix-core forward, ask for no table gradient, pass 16-byte aligned
  * gradient buffers and bring the workspace run on the matrix cores instead
  * (bf16 products, fp32 accumulation); hstu_attn_bwd_variant tells which.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which

@@ -1439,7 +1439,7 @@ __global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
 }
 
 // ---------------------------------------------------------------------------
-// Backward on the matrix cores: bf16, d = 128, the options of the MFMA forward.
+// Backward on the matrix cores: bf16, d in {32, 64, 128}, the options of the MFMA forward.
 //
 // Two kernels, each recomputing the logits (recml/core/ops/hstu_ops.py:461-517):
 //
@@ -1453,15 +1453,24 @@ __global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
 // rows of the wave) is held in registers as the B operand, the streamed tiles are the A operand:
 // read by rows for the first two products and through transpose reads for the last.  A streamed
 // tile is therefore read both ways, and one swizzle serves both: 16-byte chunk c of row r sits at
-// chunk c ^ swz_rt(r), which sends 16 consecutive rows to 16 different chunks (row reads) and 4
-// consecutive rows to 4 different 64-byte groups (transpose reads).  P and dS are rounded to bf16
+// chunk c ^ swz_rt<D>(r), which spreads 16 consecutive rows over the 16 chunk slots of a 256-byte
+// sweep of the banks (row reads) and 4 consecutive rows over 4 different 64-byte groups (transpose
+// reads).  P and dS are rounded to bf16
 // for the last products like P in the forward.  Neither kernel splits its streamed range.  The
 // table gradients, when wanted, come from the dQ kernel, which sees every pair once.
 // ---------------------------------------------------------------------------
 
 constexpr float LN2 = 0.6931471805599453f;
 
-__device__ __forceinline__ constexpr int swz_rt(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+template <int D>
+__device__ __forceinline__ constexpr int swz_rt(int row) {
+  // rows of 256 / 128 / 64 bytes: 16 / 8 / 4 chunks, 1 / 2 / 4 rows per sweep of the banks
+  return D == 128 ? (((row & 3) << 2) | ((row >> 2) & 3)) : D == 64 ? ((((row >> 1) & 1) << 2) | ((row >> 2) & 3)) : ((row >> 2) & 3);
+}
+// The upper part of swz_rt for the rows a lane addresses in transpose reads (row = 4hh + gi/4 + 8x + 16cc,
+// gi = lane % 16), in units of 4 chunks; its lower part is (hh + 2x) & 3 for every D.
+template <int D>
+__device__ __forceinline__ constexpr int swz_rt_group(int gi) { return D == 128 ? (gi >> 2) : D == 64 ? ((gi >> 3) & 1) : 0; }
 
 // sigma and f' from u = x log2(e): returns sigma(x), stores f'(x)
 __device__ __forceinline__ float silu_grad_log2(float u, float* fprime) {
@@ -1471,17 +1480,19 @@ __device__ __forceinline__ float silu_grad_log2(float u, float* fprime) {
   return sg;
 }
 
-// Turns a wave's 32 x 128 accumulator (lane (col m, half hh) holds channels 32 dvb + 8g + 4hh + t of
-// row m) into whole bf16 rows through the wave's own 8 KB of LDS and stores rows [row0, row0 + 32)
-// that are below `rows`, rows at or past `n_live` as zeros.
-__device__ __forceinline__ void store_rows_128(const floatx16 (&acc)[4], float scale, unsigned char* ot, bf16_t* __restrict__ dst,
-                                               int64_t row_stride, int row0, int n_live, int rows, int lane) {
-  constexpr int D = 128, CPR = 16;
+// Turns a wave's 32 x D accumulator (lane (col m, half hh) holds channels 32 dvb + 8g + 4hh + t of
+// row m) into whole bf16 rows through the wave's own 32 x D x 2 bytes of LDS and stores rows
+// [row0, row0 + 32) that are below `rows`, rows at or past `n_live` as zeros.
+template <int D>
+__device__ __forceinline__ void store_rows(const floatx16 (&acc)[D / 32], float scale, unsigned char* ot, bf16_t* __restrict__ dst,
+                                           int64_t row_stride, int row0, int n_live, int rows, int lane) {
+  constexpr int CPR = D / 8, RPB = CPR >= 16 ? 1 : 16 / CPR;
+  auto oswz = [](int row) { return (row / RPB) % CPR; };
   const int m = lane & 31, hh = lane >> 5;
   const bool live = row0 + m < n_live;
   unsigned char* orow = ot + m * (D * 2) + 8 * hh;
 #pragma unroll
-  for (int dvb = 0; dvb < 4; ++dvb) {
+  for (int dvb = 0; dvb < D / 32; ++dvb) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       uint2 pko = {0u, 0u};
@@ -1489,14 +1500,15 @@ __device__ __forceinline__ void store_rows_128(const floatx16 (&acc)[4], float s
         pko.x = pack_bf16(acc[dvb][4 * g + 0] * scale, acc[dvb][4 * g + 1] * scale);
         pko.y = pack_bf16(acc[dvb][4 * g + 2] * scale, acc[dvb][4 * g + 3] * scale);
       }
-      *(uint2*)(orow + (((4 * dvb + g) ^ (m % CPR)) * 16)) = pko;
+      *(uint2*)(orow + (((4 * dvb + g) ^ oswz(m)) * 16)) = pko;
     }
   }
+  constexpr int ROWS_PER_STORE = 64 / CPR;
   const int rr = lane / CPR, cc = lane - rr * CPR;
 #pragma unroll
-  for (int r0s = 0; r0s < 32; r0s += 4) {
+  for (int r0s = 0; r0s < 32; r0s += ROWS_PER_STORE) {
     const int row = r0s + rr;
-    const uint4 val = *(const uint4*)(ot + row * (D * 2) + ((cc ^ (row % CPR)) * 16));
+    const uint4 val = *(const uint4*)(ot + row * (D * 2) + ((cc ^ oswz(row)) * 16));
     const int grow = row0 + row;
     if (grow < rows) *(uint4*)(dst + (int64_t)grow * row_stride + cc * 8) = val;
   }
@@ -1534,16 +1546,14 @@ __device__ __forceinline__ float wave_sum(float v) {
 // diagonals to the table in memory and clears them.
 // Bucket table: where each lane has one bucket for the whole block (or two neighbours), lanes with
 // the same bucket are summed across the wave; only blocks with more buckets per lane use atomics.
-template <bool POS, bool TS, bool TG>
+template <int D, bool POS, bool TS, bool TG>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
-  constexpr int D = 128;
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
   constexpr int QCH = D / 16;
   constexpr int DVB = D / 32;
-  constexpr int NPIECE = SM::V_BYTES / 1024;
-  constexpr int LD = NPIECE / NWAVES;
-  static_assert(NPIECE % NWAVES == 0, "whole pieces per wave");
+  constexpr int NPIECE = SM::V_BYTES / 1024;            // 1 KB pieces of a tile; small tiles: several waves repeat a piece
+  constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
   constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
@@ -1607,12 +1617,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     const int last = s.n_kv - 1;
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
-      const int j = w * LD + r;
+      const int j = (w * LD + r) % NPIECE;
       const int c = 64 * j + lane;
       const int row = c / CPR, pc = c - row * CPR;
       int grow = kv0 + row;
       grow = grow < last ? grow : last;
-      const uint32_t sw = (uint32_t)((pc ^ swz_rt(row)) * 16);
+      const uint32_t sw = (uint32_t)((pc ^ swz_rt<D>(row)) * 16);
       lds_dma16(kg, (uint32_t)grow * kst_bytes + sw, (const unsigned char*)Ks(st) + j * 1024);
       lds_dma16(vg, (uint32_t)grow * vst_bytes + sw, (const unsigned char*)Vs(st) + j * 1024);
     }
@@ -1686,7 +1696,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
 
-  const int gk = swz_rt(m);
+  const int gk = swz_rt<D>(m);
   // transpose reads of K: lane i of 16-lane group G addresses 8 bytes of row 4hh + i/4 (+ 8x + 16cc),
   // logical chunk 4 dvb + 2 (G & 1) + (i & 3) / 2.  For those rows swz_rt = 4 (i/4) + ((hh + 2x) & 3).
   const int gi = lane & 15;
@@ -1892,7 +1902,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
         for (int dvb = 0; dvb < DVB; ++dvb) {
-          const int cb = 4 * (dvb ^ (gi >> 2));
+          const int cb = 4 * (dvb ^ swz_rt_group<D>(gi));
           uint2 lo = lds_read_tr(kr + (16 * cc) * D + (cb + c_lo) * 8);
           uint2 hi = lds_read_tr(kr + (16 * cc + 8) * D + (cb + c_hi) * 8);
           ktf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
@@ -1959,18 +1969,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     }
   }
   // dQ^T[d][q] -> rows of dq (the ring is free: the loop ended on a barrier, no load is in flight)
-  store_rows_128(acc, p.alpha * p.inv_n, smem + w * (32 * D * 2), dqg, p.q_st, r0, s.n_q, s.rows, lane);
+  store_rows<D>(acc, p.alpha * p.inv_n, smem + w * (32 * D * 2), dqg, p.q_st, r0, s.n_q, s.rows, lane);
 }
 
-template <bool POS, bool TS>
-__global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Params p) {
-  constexpr int D = 128;
+// d = 128 needs more than 256 registers (two 32 x 128 accumulators, K and V fragments): 1 workgroup per CU there
+template <int D, bool POS, bool TS>
+__global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
   constexpr int QCH = D / 16;
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;
-  constexpr int LD = NPIECE / NWAVES;
+  constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
   constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
   // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
@@ -2045,12 +2055,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
     const int last = s.n_q - 1;
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
-      const int j = w * LD + r;
+      const int j = (w * LD + r) % NPIECE;
       const int c = 64 * j + lane;
       const int row = c / CPR, pc = c - row * CPR;
       int grow = qbs + row;
       grow = grow < last ? grow : last;
-      const uint32_t sw = (uint32_t)((pc ^ swz_rt(row)) * 16);
+      const uint32_t sw = (uint32_t)((pc ^ swz_rt<D>(row)) * 16);
       lds_dma16(qg, (uint32_t)grow * qst_bytes + sw, (const unsigned char*)Qs(st) + j * 1024);
       lds_dma16(dog, (uint32_t)grow * ost_bytes + sw, (const unsigned char*)Os(st) + j * 1024);
     }
@@ -2123,7 +2133,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dka[i][r] = 0.f; dva[i][r] = 0.f; }
 
-  const int gk = swz_rt(m);
+  const int gk = swz_rt<D>(m);
   const int gi = lane & 15;
   const int vrow = 4 * hh + (gi >> 2);
   const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
@@ -2226,7 +2236,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
       for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
         for (int dvb = 0; dvb < DVB; ++dvb) {
-          const int cb = 4 * (dvb ^ (gi >> 2));
+          const int cb = 4 * (dvb ^ swz_rt_group<D>(gi));
           uint2 lo = lds_read_tr(orr + (16 * cc) * D + (cb + c_lo) * 8);
           uint2 hi = lds_read_tr(orr + (16 * cc + 8) * D + (cb + c_hi) * 8);
           otf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
@@ -2291,8 +2301,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 1) void hstu_bwd_dkv_mfma(const Param
   }
 
   unsigned char* ot = smem + w * (32 * D * 2);
-  store_rows_128(dka, p.alpha * p.inv_n, ot, dkg, p.k_st, r0, s.n_kv, s.rows, lane);
-  store_rows_128(dva, p.inv_n * (1.0f / LOG2E), ot, dvg, p.v_st, r0, s.n_kv, s.rows, lane);
+  store_rows<D>(dka, p.alpha * p.inv_n, ot, dkg, p.k_st, r0, s.n_kv, s.rows, lane);
+  store_rows<D>(dva, p.inv_n * (1.0f / LOG2E), ot, dvg, p.v_st, r0, s.n_kv, s.rows, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -2609,12 +2619,12 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   return HSTU_OK;
 }
 
-// The matrix-core backward: bf16 with d = 128 under the conditions of the matrix-core forward,
-// 16-byte aligned gradient buffers, and the forward's workspace at hand.
+// The matrix-core backward: bf16 under the conditions of the matrix-core forward, 16-byte aligned
+// gradient buffers, and the forward's workspace at hand.
 bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
-  if (f.qk_dtype != HSTU_DTYPE_BF16 || f.d_qk != 128 || !mfma_eligible(&f)) return false;
+  if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
@@ -2623,23 +2633,33 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
 }
 
-template <bool POS, bool TS, bool TG>
+template <int D, bool POS, bool TS, bool TG>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<128, 2>::total(POS, TS);
+  const int smem = MfmaSmem<D, 2>::total(POS, TS);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
-  static int granted_q[64], granted_kv[64];
-  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<POS, TS, TG>, smem_q, granted_q)) return rc;
   const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
-  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<POS, TS>, smem_kv, granted_kv)) return rc;
+  static int granted_q[64], granted_kv[64];
+  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG>, smem_q, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS>, smem_kv, granted_kv)) return rc;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_bwd_dq_mfma<POS, TS, TG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_kv, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
+}
+
+template <int D>
+int launch_bwd_mfma_d(const Params& q, hipStream_t st) {
+  const bool pos = q.pos_tab != nullptr, ts = q.ts_tab != nullptr;
+  const bool tg = (pos && q.dpos) || (ts && q.dts);
+  if (pos && ts) return tg ? launch_bwd_mfma_inst<D, true, true, true>(q, st) : launch_bwd_mfma_inst<D, true, true, false>(q, st);
+  if (pos) return tg ? launch_bwd_mfma_inst<D, true, false, true>(q, st) : launch_bwd_mfma_inst<D, true, false, false>(q, st);
+  if (ts) return tg ? launch_bwd_mfma_inst<D, false, true, true>(q, st) : launch_bwd_mfma_inst<D, false, true, false>(q, st);
+  return launch_bwd_mfma_inst<D, false, false, false>(q, st);
 }
 
 int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
@@ -2649,12 +2669,9 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
   const WorkspacePlan ws = plan_workspace(&f, false);
   Params q = p;
   if (int rc = setup_workspace(&f, ws, q, st)) return rc;
-  const bool pos = q.pos_tab != nullptr, ts = q.ts_tab != nullptr;
-  const bool tg = (pos && q.dpos) || (ts && q.dts);
-  if (pos && ts) return tg ? launch_bwd_mfma_inst<true, true, true>(q, st) : launch_bwd_mfma_inst<true, true, false>(q, st);
-  if (pos) return tg ? launch_bwd_mfma_inst<true, false, true>(q, st) : launch_bwd_mfma_inst<true, false, false>(q, st);
-  if (ts) return tg ? launch_bwd_mfma_inst<false, true, true>(q, st) : launch_bwd_mfma_inst<false, true, false>(q, st);
-  return launch_bwd_mfma_inst<false, false, false>(q, st);
+  if (q.d_qk == 128) return launch_bwd_mfma_d<128>(q, st);
+  if (q.d_qk == 64) return launch_bwd_mfma_d<64>(q, st);
+  return launch_bwd_mfma_d<32>(q, st);
 }
 
 }  // namespace

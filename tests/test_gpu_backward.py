@@ -111,19 +111,24 @@ def _boundary_flags(ts, lens, causal):
   return rows, cols
 
 
-@pytest.mark.parametrize("name,B,L,H,lens,pos,ts,causal,jagged", [
-    ("full-length", 2, 256, 2, None, False, False, True, False),
-    ("lengths", 3, 300, 2, [300, 129, 1], False, False, True, False),
-    ("non-causal", 2, 200, 1, [200, 77], False, False, False, False),
-    ("pos", 3, 300, 2, [300, 129, 33], True, False, True, False),
-    ("ts", 3, 300, 2, [300, 129, 33], False, True, True, False),
-    ("pos+ts jagged", 4, 420, 2, [420, 129, 33, 256], True, True, True, True),
-    ("pos+ts non-causal", 2, 200, 2, [200, 100], True, True, False, False),
+@pytest.mark.parametrize("name,d,B,L,H,lens,pos,ts,causal,jagged", [
+    ("full-length", 128, 2, 256, 2, None, False, False, True, False),
+    ("lengths", 128, 3, 300, 2, [300, 129, 1], False, False, True, False),
+    ("non-causal", 128, 2, 200, 1, [200, 77], False, False, False, False),
+    ("pos", 128, 3, 300, 2, [300, 129, 33], True, False, True, False),
+    ("ts", 128, 3, 300, 2, [300, 129, 33], False, True, True, False),
+    ("pos+ts jagged", 128, 4, 420, 2, [420, 129, 33, 256], True, True, True, True),
+    ("pos+ts non-causal", 128, 2, 200, 2, [200, 100], True, True, False, False),
+    ("d64 lengths", 64, 3, 300, 2, [300, 129, 1], False, False, True, False),
+    ("d64 pos+ts jagged", 64, 4, 420, 2, [420, 129, 33, 256], True, True, True, True),
+    ("d64 pos non-causal", 64, 2, 200, 4, [200, 100], True, False, False, False),
+    ("d32 lengths", 32, 3, 300, 2, [300, 129, 1], False, False, True, False),
+    ("d32 pos+ts jagged", 32, 4, 420, 2, [420, 129, 33, 256], True, True, True, True),
+    ("d32 ts non-causal", 32, 2, 200, 1, [200, 100], False, True, False, False),
 ])
-def test_backward_matrix_core_kernels(gpu, name, B, L, H, lens, pos, ts, causal, jagged):
-  """bf16, d = 128: the matrix-core pair of kernels, checked against the oracle (table gradients too)."""
+def test_backward_matrix_core_kernels(gpu, name, d, B, L, H, lens, pos, ts, causal, jagged):
+  """bf16, d in {32, 64, 128}: the matrix-core pair of kernels, checked against the oracle (table gradients too)."""
   rng = np.random.default_rng(31)
-  d = 128
   bf = torch.bfloat16
   q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
   full = np.full((B,), L, np.int32)

@@ -1514,9 +1514,11 @@ __device__ __forceinline__ void store_rows(const floatx16 (&acc)[D / 32], float 
   }
 }
 
-// Extra LDS of the dQ kernel when it also sums table gradients: per wave, a ring of 256 diagonal
-// sums and one sum per bucket
-constexpr int BWD_TG_BYTES = NWAVES * (256 + TS_TAB_LEN) * 4;
+// Extra LDS of the dQ kernel when it also sums table gradients: a ring of TG_RING diagonal sums per
+// wave, then one sum per bucket for the workgroup.  Kept this small on purpose: with both biases at
+// d = 128 the kernel's LDS is 78 KB, and two workgroups must still fit a CU's 160 KB.
+constexpr int TG_RING = 128;
+constexpr int BWD_TG_BYTES = (NWAVES * TG_RING + TS_TAB_LEN) * 4;
 
 // v of the lane `CTRL` names (data-parallel-primitive controls of the vector ALU: 0x110 + n = n lanes
 // down within a row of 16, 0x142 / 0x143 = lane 15 of the previous row / lane 31 to the rows that
@@ -1541,11 +1543,13 @@ __device__ __forceinline__ float wave_sum(float v) {
 // in registers first and each wave keeps its own LDS accumulators, updated without atomics.
 // Position table: pair (q, key) of a wave lies on diagonal X = key - q + (r0 + 31) >= 0.  A block's
 // 32 x 32 pairs are brought onto their 63 diagonals by lane permutes (see the block), one value per
-// lane, and added to a ring of 256 sums.  Block t only touches X in [32 t, 32 t + 63), so
-// everything below 32 (t + 1) is final after it: every fourth block the wave adds 128 finished
+// lane, and added to the wave's ring of sums.  Block t only touches X in [32 t, 32 t + 63), so
+// everything below 32 (t + 1) is final after it: every second block the wave adds 64 finished
 // diagonals to the table in memory and clears them.
 // Bucket table: where each lane has one bucket for the whole block (or two neighbours), lanes with
-// the same bucket are summed across the wave; only blocks with more buckets per lane use atomics.
+// the same bucket are summed across the wave and one lane adds the sum to the workgroup's
+// histogram (an LDS atomic, but of one lane); only blocks with more buckets per lane use one
+// atomic per lane and run of equal buckets.
 template <int D, bool POS, bool TS, bool TG>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
   using SM = MfmaSmem<D, 2>;
@@ -1657,7 +1661,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t < nt) dma_step(t);
   if (TG) {
-    for (int i = tid; i < NWAVES * (256 + TS_TAB_LEN); i += MFMA_THREADS) TgBase[i] = 0.f;
+    for (int i = tid; i < NWAVES * TG_RING + TS_TAB_LEN; i += MFMA_THREADS) TgBase[i] = 0.f;
   }
 
   // Q and dO fragments of this lane's row (B operands): 16-byte chunk 2ks + hh of the row
@@ -1848,11 +1852,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       const float s_high = s_all - s_low;
       const float mine = hh ? s_high : s_low, theirs = hh ? s_low : s_high;
       const float got = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, theirs)));
-      float* slot = TgBase + w * 256 + ((kbs + 31 - m + 32 * hh) & 255);
+      float* slot = TgBase + w * TG_RING + ((kbs + 31 - m + 32 * hh) & (TG_RING - 1));
       *slot += mine + got;
     }
     if (want_dts) {
-      float* hist = TgBase + NWAVES * 256 + w * TS_TAB_LEN;
+      float* hist = TgBase + NWAVES * TG_RING;
       if (bk_lane >= 0) {
         float s_near = 0.f, s_far = 0.f;
 #pragma unroll
@@ -1873,8 +1877,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
           const float a = wave_sum(mine ? s_near : 0.f);
           const float c = any_far ? wave_sum(mine ? s_far : 0.f) : 0.f;
           if (lane == 0) {
-            hist[b0] += a;
-            if (any_far) hist[b0 + 1] += c;
+            atomicAdd(&hist[b0], a);
+            if (any_far) atomicAdd(&hist[b0 + 1], c);
           }
           done = done || mine;
         }
@@ -1932,7 +1936,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
 
   // adds diagonals [x0, x0 + 64) of this wave's ring to the table in memory and clears them
   auto flush_diag = [&](int x0) {
-    float* slot = TgBase + w * 256 + ((x0 + lane) & 255);
+    float* slot = TgBase + w * TG_RING + ((x0 + lane) & (TG_RING - 1));
     const float val = *slot;
     *slot = 0.f;
     const int idx = (p.L - 1) + (x0 + lane) - 31 - r0;
@@ -1946,24 +1950,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
     if (t * BN <= wave_last) {
       block(t);
-      if (want_dpos && (t & 3) == 3) {
-        flush_diag(32 * (t - 3));
-        flush_diag(32 * (t - 3) + 64);
-      }
+      if (want_dpos && (t & 1) == 1) flush_diag(32 * (t - 1));
     }
     if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
   }
 
   if (want_dpos && wave_last >= 0) {
-    // what the wave has not written out: the diagonals of its last (up to 3) blocks, then 31 more
+    // what the wave has not written out: the diagonals of its last block if their number is odd, then 31 more
     const int t_done = wave_last / BN + 1;
-    flush_diag(32 * (t_done & ~3));
-    flush_diag(32 * (t_done & ~3) + 64);
+    flush_diag(32 * (t_done & ~1));
   }
   if (want_dts) {
-    const float* hist = TgBase + NWAVES * 256 + w * TS_TAB_LEN;
-    for (int e = lane; e < TS_TAB_LEN; e += 64) {
+    // every wave is past the loop's last barrier: the histogram is complete
+    const float* hist = TgBase + NWAVES * TG_RING;
+    for (int e = tid; e < TS_TAB_LEN; e += MFMA_THREADS) {
       const float val = hist[e];
       if (val != 0.f) atomicAdd(p.dts + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1) + (e < p.ts_nb ? e : p.ts_nb), val * p.inv_n);
     }

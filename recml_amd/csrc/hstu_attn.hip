@@ -1973,15 +1973,29 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   store_rows<D>(acc, p.alpha * p.inv_n, smem + w * (32 * D * 2), dqg, p.q_st, r0, s.n_q, s.rows, lane);
 }
 
-// d = 128 needs more than 256 registers (two 32 x 128 accumulators, K and V fragments): 1 workgroup per CU there
+// At d = 128 two 32 x 128 accumulators plus the K and V fragments are 192 registers before any
+// temporary, and a wave that spills into the accumulation registers spends its time moving values
+// between the two files.  There the work of 32 keys is shared by two waves (8 per workgroup, one
+// workgroup per CU): both compute S and dP, each accumulates dK and dV for one half of the channels.
+template <int D>
+struct DkvShape {
+  static constexpr int DSPLIT = D == 128 ? 2 : 1;        // waves per 32 keys
+  static constexpr int NW = NWAVES * DSPLIT;             // waves per workgroup
+  static constexpr int THREADS = 64 * NW;
+  static constexpr int DW = D / DSPLIT;                  // channels of dK / dV per wave
+};
+
 template <int D, bool POS, bool TS>
-__global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
+__global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
+  using SH = DkvShape<D>;
+  constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
+  constexpr int DVBW = DW / 32;          // 32-channel blocks of dK / dV per wave
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
   constexpr int QCH = D / 16;
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;
-  constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
+  constexpr int LD = NPIECE >= NW ? NPIECE / NW : 1;
   constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
   // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
@@ -2014,7 +2028,9 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = w8 % NWAVES;            // which 32 keys of the tile
+  const int dh = w8 / NWAVES;           // which part of the channels
   const int m = lane & 31, hh = lane >> 5;
   const char* __restrict__ qg = (const char*)p.q + s.bq * 2;
   const char* __restrict__ dog = (const char*)p.dout + s.bo * 2;
@@ -2024,7 +2040,7 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
   if (kv0 >= s.n_kv) {
     const int rows = (s.rows - kv0) < BM ? (s.rows - kv0) : BM;
     const uint4 z = {0u, 0u, 0u, 0u};
-    for (int e = tid; e < rows * (D / 8); e += MFMA_THREADS) {
+    for (int e = tid; e < rows * (D / 8); e += THREADS) {
       int r = e / (D / 8), c = e - r * (D / 8);
       *(uint4*)(dkg + (int64_t)(kv0 + r) * p.k_st + c * 8) = z;
       *(uint4*)(dvg + (int64_t)(kv0 + r) * p.v_st + c * 8) = z;
@@ -2056,7 +2072,7 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
     const int last = s.n_q - 1;
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
-      const int j = (w * LD + r) % NPIECE;
+      const int j = (w8 * LD + r) % NPIECE;
       const int c = 64 * j + lane;
       const int row = c / CPR, pc = c - row * CPR;
       int grow = qbs + row;
@@ -2128,9 +2144,9 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
     asm volatile("" ::"v"(tk), "v"(tk32));
   }
 
-  floatx16 dka[DVB], dva[DVB];
+  floatx16 dka[DVBW], dva[DVBW];
 #pragma unroll
-  for (int i = 0; i < DVB; ++i)
+  for (int i = 0; i < DVBW; ++i)
 #pragma unroll
     for (int r = 0; r < 16; ++r) { dka[i][r] = 0.f; dva[i][r] = 0.f; }
 
@@ -2229,15 +2245,15 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
       }
     }
     // transposed fragments of dO (for dV) and of Q (for dK)
-    uint4 otf[2][DVB], qtf[2][DVB];
+    uint4 otf[2][DVBW], qtf[2][DVBW];
     {
       const bf16_t* orr = Os(st) + vrow * D + 4 * (gi & 1);
       const bf16_t* qrr = Qs(st) + vrow * D + 4 * (gi & 1);
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-        for (int dvb = 0; dvb < DVB; ++dvb) {
-          const int cb = 4 * (dvb ^ swz_rt_group<D>(gi));
+        for (int dvb = 0; dvb < DVBW; ++dvb) {
+          const int cb = 4 * ((dh * DVBW + dvb) ^ swz_rt_group<D>(gi));
           uint2 lo = lds_read_tr(orr + (16 * cc) * D + (cb + c_lo) * 8);
           uint2 hi = lds_read_tr(orr + (16 * cc + 8) * D + (cb + c_hi) * 8);
           otf[cc][dvb] = uint4{lo.x, lo.y, hi.x, hi.y};
@@ -2277,7 +2293,7 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
       dk4.w = pack_bf16(ds[8 * cc + 6], ds[8 * cc + 7]);
       const bf16x8 pb = __builtin_bit_cast(bf16x8, pk), db = __builtin_bit_cast(bf16x8, dk4);
 #pragma unroll
-      for (int dvb = 0; dvb < DVB; ++dvb) {
+      for (int dvb = 0; dvb < DVBW; ++dvb) {
         dva[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, otf[cc][dvb]), pb, dva[dvb], 0, 0, 0);
         dka[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qtf[cc][dvb]), db, dka[dvb], 0, 0, 0);
       }
@@ -2301,9 +2317,9 @@ __global__ __launch_bounds__(MFMA_THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_m
     __syncthreads();
   }
 
-  unsigned char* ot = smem + w * (32 * D * 2);
-  store_rows<D>(dka, p.alpha * p.inv_n, ot, dkg, p.k_st, r0, s.n_kv, s.rows, lane);
-  store_rows<D>(dva, p.inv_n * (1.0f / LOG2E), ot, dvg, p.v_st, r0, s.n_kv, s.rows, lane);
+  unsigned char* ot = smem + w8 * (32 * DW * 2);
+  store_rows<DW>(dka, p.alpha * p.inv_n, ot, dkg + dh * DW, p.k_st, r0, s.n_kv, s.rows, lane);
+  store_rows<DW>(dva, p.inv_n * (1.0f / LOG2E), ot, dvg + dh * DW, p.v_st, r0, s.n_kv, s.rows, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -2647,7 +2663,7 @@ int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
   hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_kv, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;

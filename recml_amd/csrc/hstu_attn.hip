@@ -1974,12 +1974,35 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
 }
 
 // At d = 128 two 32 x 128 accumulators plus the K and V fragments are 192 registers before any
-// temporary, and a wave that spills into the accumulation registers spends its time moving values
-// between the two files.  There the work of 32 keys is shared by two waves (8 per workgroup, one
-// workgroup per CU): both compute S and dP, each accumulates dK and dV for one half of the channels.
+// temporary: one workgroup per CU, the accumulators in the accumulation registers, and a compiler
+// that then moves values between the two register files on every block (2.6x the vector
+// instructions of the dQ kernel).  Two remedies are built in.  KV_LDS: the wave's K and V rows
+// stay in LDS (64 KB more per workgroup, which one workgroup per CU can afford) and are read as B
+// operands on every block, so that the ordinary registers hold temporaries only.  DSPLIT = 2: the
+// work of 32 keys is shared by two waves, each accumulating dK and dV for half of the channels
+// (measured: no gain, both waves repeat S, dP and the pointwise math).
+// acc = 0 and acc += A B with the accumulator named as accumulation registers (ACC_ASM).  Left to the
+// compiler, the loop-carried accumulators of the d = 128 kernel live in ordinary registers and all
+// 128 are copied to the accumulation file and back around the products of every block.  Written
+// this way every definition of them is an accumulation register, so they stay there.  They are
+// only ever read as the C operand of the same instruction (chained by the hardware without wait
+// states) and by the final stores, which wait out the last product first.
+__device__ __forceinline__ void mfma_acc_zero(floatx16& acc) {
+  const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=a"(acc) : "v"(z));
+}
+__device__ __forceinline__ void mfma_acc(floatx16& acc, bf16x8 a, bf16x8 b) {
+  // The wait states cover an operand written by the vector ALU just before: the compiler pads such a
+  // pair to two wait states for its own matrix instructions but does not look into this statement
+  // (without them results were wrong); four leave a margin.
+  asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+
 template <int D>
 struct DkvShape {
-  static constexpr int DSPLIT = D == 128 ? 2 : 1;        // waves per 32 keys
+  static constexpr bool KV_LDS = false;
+  static constexpr bool ACC_ASM = D == 128;
+  static constexpr int DSPLIT = 1;                       // waves per 32 keys
   static constexpr int NW = NWAVES * DSPLIT;             // waves per workgroup
   static constexpr int THREADS = 64 * NW;
   static constexpr int DW = D / DSPLIT;                  // channels of dK / dV per wave
@@ -1989,6 +2012,7 @@ template <int D, bool POS, bool TS>
 __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
   using SH = DkvShape<D>;
   constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
+  constexpr bool KV_LDS = SH::KV_LDS, ACC_ASM = SH::ACC_ASM;
   constexpr int DVBW = DW / 32;          // 32-channel blocks of dK / dV per wave
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
@@ -2013,6 +2037,10 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
   const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
+  // KV_LDS: [K rows of the tile][V rows of the tile], 128 x D bf16 each, two-way swizzle by row within a wave's 32
+  constexpr int KV_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
+  unsigned char* Kst = smem + KV_OFF;
+  unsigned char* Vst = Kst + BM * D * 2;
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -2112,13 +2140,29 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
     lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
     lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
   }
+  if (KV_LDS) {
+    // this wave's 32 K rows and 32 V rows, 1 KB per load; rows past the sequence repeat the last one (masked later)
+    const int last = s.n_kv - 1;
+    const char* kgl = (const char*)p.k + s.bk * 2;
+    const char* vgl = (const char*)p.v + s.bv * 2;
+#pragma unroll
+    for (int j = 0; j < 32 * D * 2 / 1024; ++j) {
+      const int c = 64 * j + lane;
+      const int row = c / CPR, pc = c - row * CPR;
+      int grow = r0 + row;
+      grow = grow < last ? grow : last;
+      const uint32_t sw = (uint32_t)((pc ^ swz_rt<D>(row)) * 16);
+      lds_dma16(kgl, (uint32_t)grow * ((uint32_t)p.k_st * 2u) + sw, Kst + w * (32 * D * 2) + j * 1024);
+      lds_dma16(vgl, (uint32_t)grow * ((uint32_t)p.v_st * 2u) + sw, Vst + w * (32 * D * 2) + j * 1024);
+    }
+  }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t_lo + t < nt) dma_step(t_lo + t);
 
   // K and V fragments of this lane's key (B operands)
   uint4 kfr[QCH], vfr[QCH];
-  {
+  if (!KV_LDS) {
     const char* kp = (const char*)p.k + (s.bk + (int64_t)kcol * p.k_st) * 2 + 16 * hh;
     const char* vp = (const char*)p.v + (s.bv + (int64_t)kcol * p.v_st) * 2 + 16 * hh;
 #pragma unroll
@@ -2146,9 +2190,15 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
 
   floatx16 dka[DVBW], dva[DVBW];
 #pragma unroll
-  for (int i = 0; i < DVBW; ++i)
+  for (int i = 0; i < DVBW; ++i) {
+    if (ACC_ASM) {
+      mfma_acc_zero(dka[i]);
+      mfma_acc_zero(dva[i]);
+    } else {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { dka[i][r] = 0.f; dva[i][r] = 0.f; }
+      for (int r = 0; r < 16; ++r) { dka[i][r] = 0.f; dva[i][r] = 0.f; }
+    }
+  }
 
   const int gk = swz_rt<D>(m);
   const int gi = lane & 15;
@@ -2169,9 +2219,11 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
 #pragma unroll
       for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
 #pragma unroll
-      for (int ks = 0; ks < QCH; ++ks)
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, kfr[ks]),
+      for (int ks = 0; ks < QCH; ++ks) {
+        const uint4 bk = KV_LDS ? *(const uint4*)(Kst + (32 * w + m) * (D * 2) + (((2 * ks + hh) ^ gk) * 16)) : kfr[ks];
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, bk),
                                                        ks == 0 ? zero : sacc, 0, 0, 0);
+      }
     }
     {
       uint4 af[QCH];
@@ -2179,9 +2231,11 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
 #pragma unroll
       for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
 #pragma unroll
-      for (int ks = 0; ks < QCH; ++ks)
-        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, vfr[ks]),
+      for (int ks = 0; ks < QCH; ++ks) {
+        const uint4 bv = KV_LDS ? *(const uint4*)(Vst + (32 * w + m) * (D * 2) + (((2 * ks + hh) ^ gk) * 16)) : vfr[ks];
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, bv),
                                                         ks == 0 ? zero : dpacc, 0, 0, 0);
+      }
     }
     float u[16];
     if (POS) {
@@ -2294,8 +2348,13 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
       const bf16x8 pb = __builtin_bit_cast(bf16x8, pk), db = __builtin_bit_cast(bf16x8, dk4);
 #pragma unroll
       for (int dvb = 0; dvb < DVBW; ++dvb) {
-        dva[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, otf[cc][dvb]), pb, dva[dvb], 0, 0, 0);
-        dka[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qtf[cc][dvb]), db, dka[dvb], 0, 0, 0);
+        if (ACC_ASM) {
+          mfma_acc(dva[dvb], __builtin_bit_cast(bf16x8, otf[cc][dvb]), pb);
+          mfma_acc(dka[dvb], __builtin_bit_cast(bf16x8, qtf[cc][dvb]), db);
+        } else {
+          dva[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, otf[cc][dvb]), pb, dva[dvb], 0, 0, 0);
+          dka[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qtf[cc][dvb]), db, dka[dvb], 0, 0, 0);
+        }
       }
     }
   };
@@ -2317,6 +2376,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
     __syncthreads();
   }
 
+  if (ACC_ASM) asm volatile("s_nop 15\n\ts_nop 15");   // the last product has left the pipeline before its result is read
   unsigned char* ot = smem + w8 * (32 * DW * 2);
   store_rows<DW>(dka, p.alpha * p.inv_n, ot, dkg + dh * DW, p.k_st, r0, s.n_kv, s.rows, lane);
   store_rows<DW>(dva, p.inv_n * (1.0f / LOG2E), ot, dvg + dh * DW, p.v_st, r0, s.n_kv, s.rows, lane);
@@ -2654,7 +2714,8 @@ template <int D, bool POS, bool TS, bool TG>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D, 2>::total(POS, TS);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
-  const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
+  // one more 16-byte piece of timestamp operands per stage; the tile's K and V rows where they stay in LDS
+  const int smem_kv = smem + (TS ? NSTAGE * 16 : 0) + (DkvShape<D>::KV_LDS ? 2 * BM * D * 2 : 0);
   static int granted_q[64], granted_kv[64];
   if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG>, smem_q, granted_q)) return rc;
   if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS>, smem_kv, granted_kv)) return rc;

@@ -3,8 +3,10 @@
 The harness for the end-to-end (config-4) shape: everything except the
 attention is plain torch on the GPU (embedding gather, layer norms, the
 projections as rocBLAS / hipBLASLt GEMMs); the attention is
-`recml_amd.hstu_attention`, i.e. the HIP kernel behind the C ABI.  Inference
-forward only (no dropout, no autograd through the kernel).
+`recml_amd.hstu_attention`, i.e. the HIP kernel behind the C ABI.  No dropout.
+Parameters are created frozen; after `requires_grad_(True)` the attention goes
+through `recml_amd.hstu_attention_autograd` (the HIP backward kernels) and the
+rest through torch autograd.
 
 Mirrors, name for name:
   HSTUBlock   recml/layers/keras/hstu.py:240-474 (weights :281-354, call :422-474)
@@ -28,6 +30,14 @@ import torch.nn.functional as F
 
 from recml_amd import hstu_ops
 from recml_amd import masks
+
+
+def _attention(q, k, v, *, pos_bias=None, ts_bias=None, **kw):
+  """The attention op, differentiable when anything it reads wants a gradient."""
+  wants = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (q, k, v, pos_bias, ts_bias))
+  if wants:
+    return hstu_ops.hstu_attention_autograd(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
+  return hstu_ops.hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
 
 
 def _glorot_uniform(shape, fan_in, fan_out, generator, dtype, device):
@@ -109,8 +119,8 @@ class HSTUBlock(torch.nn.Module):
                                           scaled_pointwise_attn=self.scaled_pointwise_attn)
     else:
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
-      attn = hstu_ops.hstu_attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
-                                     timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias)
+      attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
+                        timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias)
     normed = F.layer_norm(attn.reshape(B, L, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
                           self.attn_ln_beta.reshape(-1), self.eps)
     gated = u.reshape(B, L, H * hd) * normed
@@ -133,8 +143,8 @@ class HSTUBlock(torch.nn.Module):
     uqkv = F.silu(uqkv).reshape(T, 4, H, hd)
     u, q, k, v = uqkv.unbind(dim=1)
     alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
-    attn = hstu_ops.hstu_attention(q, k, v, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
-                                   pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
+    attn = _attention(q, k, v, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
+                      pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
     normed = F.layer_norm(attn.reshape(T, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
                           self.attn_ln_beta.reshape(-1), self.eps)
     out = (u.reshape(T, H * hd) * normed) @ self.output_kernel.reshape(H * hd, D)

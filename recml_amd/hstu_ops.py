@@ -362,7 +362,10 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
       mask=mask, bias=bias)
   # build_args may have made q, k, v contiguous in d: the gradients take the layout it passed on
   qi, ki, vi = _passed_inputs(keep)
-  dq, dk, dv = torch.empty_like(qi), torch.empty_like(ki), torch.empty_like(vi)
+  # the kernels write dq, dk, dv with the strides of q, k, v: mirror them exactly (empty_like would
+  # compact a view with gaps, e.g. one slice of a fused projection)
+  like = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device=t.device)
+  dq, dk, dv = like(qi), like(ki), like(vi)
   ba = _lib.HstuAttnBwdArgs()
   ba.struct_size = C.sizeof(_lib.HstuAttnBwdArgs)
   ba.version = _lib.ABI_VERSION

@@ -153,3 +153,54 @@ def test_block_config4_shape_bf16(gpu):
   ref = BO.hstu_block(x[:3].double().cpu().numpy(), w, num_heads=H, seq_lens=lens[:3], pos_tab=pos.double().cpu().numpy())
   got = out[:3].double().cpu().numpy()
   assert np.abs(got - ref).max() / np.abs(ref).max() <= 3e-2
+
+
+def _dense_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None, n=None, alpha=1.0, pos_bias=None, **_):
+  """Differentiable dense torch form of the op (padded layout, causal, lengths, position table)."""
+  B, L, H, d = q.shape
+  s = alpha * torch.einsum("bihd,bjhd->bhij", q.float(), k.float())
+  i = torch.arange(L, device=q.device)
+  if pos_bias is not None:
+    s = s + pos_bias.float()[:, (L - 1) + i[None, :] - i[:, None]][None]
+  keep = (i[None, :] <= i[:, None])[None] & (i[None, None, :] < seq_lens[:, None, None]) & (i[None, :, None] < seq_lens[:, None, None])
+  p = torch.nn.functional.silu(s) / n * keep[:, None]
+  return torch.einsum("bhij,bjhd->bihd", p, v.float()).to(q.dtype)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,hd,tol", [(torch.float32, 16, 2e-4), (torch.bfloat16, 64, 6e-2)])
+def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
+  """A trainable block: gradients with the HIP attention (forward and backward kernels, q / k / v being
+  strided slices of the fused projection) against the same block with a dense torch attention."""
+  from recml_amd import hstu_layer
+  from recml_amd.hstu_layer import HSTUBlock
+  dev = torch.device("cuda:0")
+  B, L, H = 3, 160, 2
+  D = H * hd
+  gen = torch.Generator().manual_seed(5)
+  blk = HSTUBlock(D, H, dtype=dtype, device=dev, generator=gen)
+  blk.requires_grad_(True)
+  x = (torch.randn((B, L, D), generator=gen) * 0.5).to(dev).to(dtype).requires_grad_(True)
+  lens = torch.tensor([160, 77, 1], dtype=torch.int32, device=dev)
+  pos = (torch.randn((H, 2 * L - 1), generator=gen) * 0.3).to(dev).requires_grad_(True)
+  dout = torch.randn((B, L, D), generator=gen).to(dev).to(dtype)
+
+  def grads(attention):
+    saved = hstu_layer._attention
+    hstu_layer._attention = attention
+    try:
+      for t in [x, pos, *blk.parameters()]:
+        t.grad = None
+      out = blk(x, seq_lens=lens, pos_bias=pos)
+      (out.float() * dout.float()).sum().backward()
+      return {"x": x.grad.float().clone(), "pos": pos.grad.float().clone(),
+              **{n: p.grad.float().clone() for n, p in blk.named_parameters() if p.grad is not None}}
+    finally:
+      hstu_layer._attention = saved
+
+  got = grads(hstu_layer._attention)
+  want = grads(_dense_attention)
+  assert set(got) == set(want) and "q_kernel" in got and "output_kernel" in got
+  for name in want:
+    err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
+    assert err <= tol, (name, err)

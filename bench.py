@@ -184,6 +184,28 @@ def bench_model(args, dev):
     torch.cuda.synchronize()
     att_ms = (time.perf_counter() - t0) * 1e3 / steps
   assert tuple(out.shape) == (B, L, D) and bool(torch.isfinite(out.float()).all())
+  # one training step's forward + backward on packed tokens: the blocks and the position table
+  # take gradients (attention through the HIP backward kernels), the embedding table stays frozen
+  for blk in model.decoder_blocks:
+    blk.requires_grad_(True)
+  pos_t = pos.clone().requires_grad_(True)
+  dout = torch.randn((B, L, D), generator=torch.Generator().manual_seed(6)).to(dev).to(torch.bfloat16)
+  def train_step():
+    for prm in model.parameters():
+      prm.grad = None
+    pos_t.grad = None
+    o = model(ids_d, seq_lens=lens_d, pos_bias=pos_t, jagged=True)
+    (o * dout).sum().backward()
+    return o
+  for _ in range(warm):
+    train_step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(steps):
+    train_step()
+  torch.cuda.synchronize()
+  train_ms = (time.perf_counter() - t0) * 1e3 / steps
+  assert bool(torch.isfinite(pos_t.grad).all()) and float(pos_t.grad.abs().max()) > 0
   nn = lens.astype(np.int64)
   attn_flops = int((H * (nn * (nn + 1) // 2) * 4 * (D // H)).sum()) * layers
   proj_flops = B * L * (2 * D * 4 * D + 2 * D * D) * layers
@@ -194,6 +216,7 @@ def bench_model(args, dev):
       "config": {"workload": f"C4 model: B={B} L={L} D={D} H={H} layers={layers} vocab={vocab} lens U{{128..1024}}, padded, pos bias, no head"},
       "ms_per_step_packed_tokens": ms_jagged, "seqs_per_s_packed_tokens": B / (ms_jagged * 1e-3),
       "packed_vs_padded_max_abs_over_max": jag_err,
+      "train_fwd_bwd_ms_packed_tokens": train_ms,
       "attention_ms_per_layer": att_ms, "attention_share": layers * att_ms / ms,
       "attention_gflop_unmasked": attn_flops / 1e9, "projection_gflop_padded": proj_flops / 1e9,
       "model_tflops": (attn_flops + proj_flops) / (ms * 1e-3) / 1e12}))

@@ -67,6 +67,38 @@ def test_backward_validation_errors_without_gpu():
   assert b"dq" in lib.hstu_attn_last_error()
 
 
+def test_backward_variant_query():
+  lib = _lib.load()
+  b = _lib.HstuAttnBwdArgs()
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"invalid"          # struct_size / version not filled in
+  b.struct_size, b.version = C.sizeof(_lib.HstuAttnBwdArgs), _lib.ABI_VERSION
+  b.fwd = _lib.new_args()
+  f = b.fwd
+  f.B, f.L, f.Lkv, f.H, f.d_qk, f.d_v = 2, 256, 256, 4, 64, 64
+  f.q = f.k = f.v = 0x10000
+  f.q_stride_t = f.k_stride_t = f.v_stride_t = f.o_stride_t = 4 * 64
+  f.q_stride_h = f.k_stride_h = f.v_stride_h = f.o_stride_h = 64
+  f.q_stride_b = f.k_stride_b = f.v_stride_b = f.o_stride_b = 256 * 4 * 64
+  f.alpha, f.inv_n, f.causal = 1.0, 1.0 / 256, 1
+  f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_BF16
+  b.dout = b.dq = b.dk = b.dv = 0x20000
+  # bf16 at a matrix-core head dim, but no workspace: the general pair
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  f.out = 0x30000                                                     # the size query validates a forward call
+  f.workspace, f.workspace_bytes = 0x40000, lib.hstu_attn_fwd_workspace_bytes(C.byref(f))
+  f.out = None                                                        # the backward does not need it
+  assert f.workspace_bytes > 0
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
+  b.dq = 0x20004                                                      # gradient buffers must be 16-byte aligned for it
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  b.dq = 0x20000
+  f.window = 8                                                        # an option the matrix-core kernels do not take
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  f.window = -1
+  f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_FP32
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<float>"
+
+
 def test_validation_errors_without_gpu():
   lib = _lib.load()
   assert lib.hstu_attn_fwd(None, None) == -1                 # HSTU_ERR_NULL

@@ -749,8 +749,10 @@ __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, W
     int it, h;
     if (p.H >= 8) { const int hx = p.H >> 3; it = j / hx; h = (j - it * hx) * 8 + xcd; }
     else          { const int r = 8 / p.H;   it = j * r + xcd / p.H; h = xcd % p.H; }
-    if (it >= p.sched[SPLIT_LIST ? 1 : 0]) return false;
+    // the item is read before the count is checked (the grid never reaches past the list's capacity):
+    // both loads miss the cache, and one after the other they cost a workgroup twice the latency
     const int4 item = ((const int4*)(p.sched + 4))[(SPLIT_LIST ? p.items_max : 0) + it];
+    if (it >= p.sched[SPLIT_LIST ? 1 : 0]) return false;
     wk.b = item.x; wk.h = h; wk.qt = item.y & 0xffff; wk.chunk = item.y >> 16;
     wk.s = seq_from(p, wk.b, h, item.z, item.w);
     return true;
@@ -1117,16 +1119,17 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   };
 
   // prologue: the scaled bucket table (64 entries per wave, the last wave repeats the first), then
-  // three steps in flight before anything else
+  // three steps in flight before the first block
   if (TS) {
     const int c = w < 3 ? w : 0;
     const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
     lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
     lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
   }
-#pragma unroll
-  for (int t = 0; t < NSTAGE - 1; ++t)
-    if (t_lo + t < nt) dma_step(t_lo + t);
+  // The first step's tiles go out alone; the other two of the prologue follow behind the Q
+  // fragments, whose wait below covers every load issued before it: behind all three steps it
+  // held up the first block until the whole prologue had landed.
+  if (t_lo < nt) dma_step(t_lo);
 
   // Q fragments (B operand of S^T = K Q^T).  bf16: k-step ks of lane (row, hh) holds
   // q[qrow][16ks+8hh .. +7], i.e. 16-byte chunk 2ks+hh of the row.  fp8: the lane holds chunks
@@ -1156,6 +1159,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     tq = tsg[iq];
     asm volatile("" ::"v"(tq), "v"(tq32));
   }
+
+#pragma unroll
+  for (int t = 1; t < NSTAGE - 1; ++t)
+    if (t_lo + t < nt) dma_step(t_lo + t);
 
   floatx16 o[DVB];
 #pragma unroll

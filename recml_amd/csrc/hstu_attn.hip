@@ -728,10 +728,9 @@ __device__ __forceinline__ int64_t partial_slot(const Params& p, int b, int64_t 
 // Steps of a tile: keys [0, kv_end) in 32-key steps
 __device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0) {
   int kv_end = s.n_kv;
-  if (p.causal) {
-    int lim = q0 + BM < s.n_q ? q0 + BM : s.n_q;
-    kv_end = lim < kv_end ? lim : kv_end;
-  }
+  const int row_end = q0 + BM < s.n_q ? q0 + BM : s.n_q;
+  if (p.causal) kv_end = row_end < kv_end ? row_end : kv_end;
+  if (p.window >= 0 && row_end - 1 + p.window + 1 < kv_end) kv_end = row_end + p.window;   // |i - j| <= window
   return (kv_end + BN - 1) / BN;
 }
 
@@ -1042,8 +1041,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     nt = t_lo + per < nt ? t_lo + per : nt;
     if (t_lo >= nt) return;    // cannot happen for n_chunks = ceil(nt / split_steps) <= nt, kept as a guard
   }
-  // last key this wave needs
-  const int wave_last = !wave_live ? -1 : (p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1));
+  // a sliding window (never combined with key-range splitting) also drops the steps before the tile's first key
+  const int win = p.window;
+  if (win >= 0 && q0 - win > 0) t_lo = (q0 - win) / BN;
+  // last key this wave needs (under a window without the causal mask: the last key its last row sees)
+  int wave_last = p.causal ? r0 + 31 : (win >= 0 ? r0 + 31 + win : s.n_kv - 1);
+  wave_last = wave_last < s.n_kv - 1 ? wave_last : s.n_kv - 1;
+  if (!wave_live) wave_last = -1;
 
   // fp8 q and k carry per-head dequantisation scales: they multiply the logits
   const float alpha2 = p.alpha * LOG2E * (F8 && p.q_scale ? p.q_scale[h] : 1.0f) * (F8 && p.k_scale ? p.k_scale[h] : 1.0f);
@@ -1295,11 +1299,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         }
       }
     }
-    if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv)) {
+    if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv) || (win >= 0 && (r0 + 31 - kbs > win || kbs + 31 - r0 > win))) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
+        const int dist = kv > qrow ? kv - qrow : qrow - kv;
+        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow) && (win < 0 || dist <= win);
         u[r] = keep ? u[r] : 0.f;
       }
     }
@@ -1337,7 +1342,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // wave makes sure its share of step t+1 has landed before the next barrier.
   for (int t = t_lo; t < nt; ++t) {
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
-    if (t * BN <= wave_last) block(t);
+    if (t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0)) block(t);
     if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
   }
@@ -2411,8 +2416,7 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 bool mfma_eligible(const HstuAttnFwdArgs* a) {
   const int kb = a->qk_dtype == HSTU_DTYPE_FP8_E4M3FN ? 1 : 2;   // bytes per q / k element
   const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
-  const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->window < 0 &&
-                       a->L == a->Lkv &&
+  const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->L == a->Lkv &&
                        // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
                        (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
   auto s8 = [](int64_t x) { return (x & 7) == 0; };
@@ -2475,7 +2479,7 @@ int validate(const HstuAttnFwdArgs* a) {
   }
   if (f8 && !mfma_eligible(a))
     return fail(HSTU_ERR_DTYPE, "fp8 q/k runs on the matrix-core kernel only: d_qk == d_v in {32, 64, 128}, q_len == kv_len, "
-                "16-byte aligned pointers and row strides, no segment ids, explicit mask, dense bias or window");
+                "16-byte aligned pointers and row strides, no segment ids, explicit mask or dense bias");
   return HSTU_OK;
 }
 
@@ -2510,7 +2514,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) 
   const bool jag = a->layout == HSTU_LAYOUT_JAGGED;
   const long long tiles_est = (long long)a->H * (jag ? (a->total_tokens / BM + a->B) : (long long)a->B * n_qtiles);
   w.entries_per_bh = n_qtiles;
-  if (allow_split && tiles_est < 1024 && steps_max > 16) {
+  if (allow_split && a->window < 0 && tiles_est < 1024 && steps_max > 16) {
     w.split_steps = (steps_max + MAX_CHUNKS - 1) / MAX_CHUNKS;
     w.split_steps = w.split_steps < 16 ? 16 : w.split_steps;
     // first tile with more steps than that (a causal tile qt has up to 4 (qt + 1) steps)
@@ -2708,7 +2712,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
 bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
-  if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
+  if (f.qk_dtype != HSTU_DTYPE_BF16 || f.window >= 0 || !mfma_eligible(&f)) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||

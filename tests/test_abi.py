@@ -155,8 +155,11 @@ def test_variant_and_workspace_query():
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<float>"
   assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 0
   a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
-  a.window = 4
-  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"
+  a.window = 4                                         # a sliding window stays on the matrix cores
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
   a.window = -1
+  a.dense_bias = 0x30000                               # a dense bias does not
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"
+  a.dense_bias = None
   a.d_qk = a.d_v = 48
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"

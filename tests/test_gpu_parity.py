@@ -457,10 +457,11 @@ def test_fp8_argument_errors(gpu):
   with pytest.raises(ValueError, match="bfloat16 v"):
     recml_amd.hstu_attention(z8, z8, z8)
   with pytest.raises(ValueError, match="matrix-core"):
-    recml_amd.hstu_attention(z8, z8, zb, sliding_window_size=2)
+    recml_amd.hstu_attention(z8, z8, zb, bias=torch.zeros((2, 8, 8), device="cuda:0"))
   with pytest.raises(ValueError, match="q_scale"):
     recml_amd.hstu_attention(zb, zb, zb, q_scale=torch.ones(2, device="cuda:0"))
   assert recml_amd.hstu_attention(z8, z8, zb).abs().max().item() == 0.0
+  assert recml_amd.hstu_attention(z8, z8, zb, sliding_window_size=2).abs().max().item() == 0.0
 
 
 def test_argument_errors(gpu):
@@ -478,3 +479,38 @@ def test_argument_errors(gpu):
     recml_amd.hstu_attention(z.cpu(), z, z)
   with pytest.raises(ValueError):
     recml_amd.hstu_attention(z.double(), z.double(), z.double())
+
+
+@pytest.mark.parametrize("d,L,window,causal,pos", [
+    (128, 400, 0, True, False),       # the diagonal only
+    (128, 400, 37, True, True),
+    (128, 400, 150, False, True),     # the band reaches over several tiles on both sides
+    (64, 300, 31, False, False),
+    (32, 520, 260, True, True),
+])
+def test_sliding_window_on_the_matrix_core_kernel(gpu, d, L, window, causal, pos):
+  """|i - j| <= window under the bf16 matrix-core kernel: steps outside the band are skipped,
+  blocks on its edges masked (the window rule itself is the oracle's reading of jax's LocalMask)."""
+  rng = np.random.default_rng(100 + window)
+  B, H = 3, 2
+  lens = np.array([L, L // 2 + 3, 1], dtype=np.int32)
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  kw, gk = {}, {}
+  if pos:
+    kw["pos_tab"] = (rng.standard_normal((H, 2 * L - 1)) * 0.1).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  ref = O.hstu_attention_ref(q, k, v, seq_lens=lens, causal=causal, sliding_window_size=window, dtype=np.float32, **kw)
+  bf = torch.bfloat16
+  a, keep = hstu_ops.build_args(_dev(q, bf), _dev(k, bf), _dev(v, bf), torch.empty((B, L, H, d), dtype=bf, device="cuda:0"),
+                                seq_lens=_dev(lens), causal=causal, sliding_window_size=window, **gk)
+  assert hstu_ops.kernel_variant(a) == "hstu_fwd_mfma_bf16"
+  hstu_ops._run(a, keep)
+  out = keep[3].float().cpu().numpy()
+  assert _err(out, ref) <= BF16_TOL
+  for b in range(B):
+    assert (out[b, lens[b]:] == 0).all()
+  # jagged layout, same values
+  (qj, off), (kj, _), (vj, _) = (O.padded_to_jagged(x, lens) for x in (q, k, v))
+  outj = recml_amd.hstu_attention(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), seq_offsets=_dev(off.astype(np.int32)), max_len=L,
+                                  causal=causal, sliding_window_size=window, **gk)
+  assert _err(O.jagged_to_padded(outj.float().cpu().numpy(), off, L), ref) <= BF16_TOL

@@ -1614,7 +1614,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   const int qrow = r0 + m;
   const bool wave_live = r0 < s.n_q;
   const int nt = tile_steps(p, s, q0);
-  const int wave_last = !wave_live ? -1 : (p.causal ? ((r0 + 31) < (s.n_kv - 1) ? (r0 + 31) : (s.n_kv - 1)) : (s.n_kv - 1));
+  // a sliding window drops the steps before the tile's first key, and for each wave the blocks outside its band
+  const int win = p.window;
+  const int t_lo = (win >= 0 && q0 - win > 0) ? (q0 - win) / BN : 0;
+  int wave_last = p.causal ? r0 + 31 : (win >= 0 ? r0 + 31 + win : s.n_kv - 1);
+  wave_last = wave_last < s.n_kv - 1 ? wave_last : s.n_kv - 1;
+  if (!wave_live) wave_last = -1;
 
   const float alpha2 = p.alpha * LOG2E;
   const uint32_t kst_bytes = (uint32_t)p.k_st * 2u, vst_bytes = (uint32_t)p.v_st * 2u;
@@ -1671,7 +1676,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
-    if (t < nt) dma_step(t);
+    if (t_lo + t < nt) dma_step(t_lo + t);
   if (TG) {
     for (int i = tid; i < NWAVES * TG_RING + TS_TAB_LEN; i += MFMA_THREADS) TgBase[i] = 0.f;
   }
@@ -1837,11 +1842,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       ds[r] = dpacc[r] * fp;
     }
     // f'(0) is not 0: masked pairs are cleared after the activation's derivative
-    if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv)) {
+    if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv) || (win >= 0 && (r0 + 31 - kbs > win || kbs + 31 - r0 > win))) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow);
+        const int dist = kv > qrow ? kv - qrow : qrow - kv;
+        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow) && (win < 0 || dist <= win);
         ds[r] = keep ? ds[r] : 0.f;
       }
     }
@@ -1956,11 +1962,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, val * p.inv_n);
   };
 
-  wait_step(0);
+  wait_step(t_lo);
   __syncthreads();
-  for (int t = 0; t < nt; ++t) {
+  for (int t = t_lo; t < nt; ++t) {
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
-    if (t * BN <= wave_last) {
+    if (t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0)) {
       block(t);
       if (want_dpos && (t & 1) == 1) flush_diag(32 * (t - 1));
     }
@@ -2092,9 +2098,13 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   const int kcol = r0 + m;              // this lane's key
   const bool wave_live = r0 < s.n_kv;
   // steps: 32 query rows each; under the causal mask only rows from the tile's first key on
-  const int nt = (s.n_q + BN - 1) / BN;
-  const int t_lo = p.causal ? kv0 / BN : 0;
-  const int t_wave = p.causal ? r0 / BN : 0;   // first step with a row that sees a key of this wave
+  // and, under a sliding window, only rows up to the window past the tile's (the wave's) last key
+  const int win = p.window;
+  int nt = (s.n_q + BN - 1) / BN;
+  if (win >= 0 && (kv0 + BM - 1 + win) / BN + 1 < nt) nt = (kv0 + BM - 1 + win) / BN + 1;
+  const int t_lo = p.causal ? kv0 / BN : ((win >= 0 && kv0 - win > 0) ? (kv0 - win) / BN : 0);
+  const int t_wave = p.causal ? r0 / BN : ((win >= 0 && r0 - win > 0) ? (r0 - win) / BN : 0);   // first step with a row that sees a key of this wave
+  const int t_wave_end = win >= 0 ? (r0 + 31 + win) / BN : 0x7fffffff / BN;                     // last such step
 
   const float alpha2 = p.alpha * LOG2E;
   const uint32_t qst_bytes = (uint32_t)p.q_st * 2u, ost_bytes = (uint32_t)p.o_st * 2u;
@@ -2337,11 +2347,13 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
       ds[r] = dpacc[r] * fp;
     }
     // rows past the sequence hold a repeat of the last row: they are masked like the rest
-    if ((p.causal && qbs < r0 + 31) || (qbs + 32 > s.n_q) || (r0 + 32 > s.n_kv)) {
+    if ((p.causal && qbs < r0 + 31) || (qbs + 32 > s.n_q) || (r0 + 32 > s.n_kv) ||
+        (win >= 0 && (qbs + 31 - r0 > win || r0 + 31 - qbs > win))) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int qi = qbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const bool keep = (qi < s.n_q) && (kcol < s.n_kv) && (!p.causal || kcol <= qi);
+        const int dist = qi > kcol ? qi - kcol : kcol - qi;
+        const bool keep = (qi < s.n_q) && (kcol < s.n_kv) && (!p.causal || kcol <= qi) && (win < 0 || dist <= win);
         pv[r] = keep ? pv[r] : 0.f;
         ds[r] = keep ? ds[r] : 0.f;
       }
@@ -2383,7 +2395,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   __syncthreads();
   for (int t = t_lo; t < nt; ++t) {
     if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
-    if (wave_live && t >= t_wave) block(t);
+    if (wave_live && t >= t_wave && t <= t_wave_end) block(t);
     if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
   }
@@ -2712,7 +2724,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
 bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
-  if (f.qk_dtype != HSTU_DTYPE_BF16 || f.window >= 0 || !mfma_eligible(&f)) return false;
+  if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||

@@ -181,3 +181,33 @@ def test_backward_matrix_core_kernels(gpu, name, d, B, L, H, lens, pos, ts, caus
     assert not edge.any() or err[edge].max() <= 1e-1, (nm, err[edge].max())
     for b in range(B):
       assert (g[b, ln[b]:] == 0).all(), nm
+
+
+@pytest.mark.parametrize("d,L,window,causal,pos", [
+    (128, 400, 37, True, True),
+    (128, 400, 150, False, True),
+    (64, 300, 0, True, False),
+    (32, 520, 260, False, True),
+])
+def test_backward_sliding_window_on_the_matrix_cores(gpu, d, L, window, causal, pos):
+  rng = np.random.default_rng(200 + window)
+  B, H = 3, 2
+  bf = torch.bfloat16
+  lens = np.array([L, L // 2 + 3, 1], dtype=np.int32)
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  kw, gk = dict(seq_lens=lens), dict(seq_lens=_dev(lens))
+  if pos:
+    kw["pos_tab"] = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, causal=causal, sliding_window_size=window, **kw)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), causal=causal,
+                                     sliding_window_size=window, _variant_out=variant, **gk)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv", "dpos"), got[:4], want[:4]):
+    assert (g is None) == (w is None), nm
+    if g is not None:
+      assert _rel(g.float().cpu().numpy().reshape(w.shape), w) <= 2e-2, nm
+  for b in range(B):
+    for g in got[:3]:
+      assert (g[b, lens[b]:] == 0).all()

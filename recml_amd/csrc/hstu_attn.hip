@@ -641,9 +641,12 @@ struct MfmaSmem {
   static constexpr int TK_LANES = BN / 4 + 1;       // 16-byte pieces: 32 int32 key timestamps, then (min, max, -, -)
   static constexpr int TK_BYTES = TK_LANES * 16;
   static constexpr int TAB_BYTES = 2 * TS_TAB_LEN * 4;   // scaled bucket table, then the bucket thresholds
-  static constexpr int bias_stage(bool pos, bool ts) { return (pos ? POS_BYTES : 0) + (ts ? TK_BYTES : 0); }
-  static constexpr int total(bool pos, bool ts) {
-    return NSTAGE * (STAGE + bias_stage(pos, ts)) + (ts ? TAB_BYTES : 0);
+  static constexpr int SEG_BYTES = BN * 4;           // the step's 32 int32 key segment ids
+  static constexpr int bias_stage(bool pos, bool ts, bool seg = false) {
+    return (pos ? POS_BYTES : 0) + (ts ? TK_BYTES : 0) + (seg ? SEG_BYTES : 0);
+  }
+  static constexpr int total(bool pos, bool ts, bool seg = false) {
+    return NSTAGE * (STAGE + bias_stage(pos, ts, seg)) + (ts ? TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
   __device__ static constexpr int swz_k(int row) { return (row / KRPB) % KCPR; }
@@ -969,7 +972,10 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
   }
 }
 
-template <int D, bool POS, bool TS, bool F8>
+// SEG: segment ids (padded layout, L a multiple of 4): a pair is kept when its row's and its key's
+// ids are equal.  The step's 32 key ids arrive by one more direct load per wave and every block
+// compares them with the lane's row id.
+template <int D, bool POS, bool TS, bool F8, bool SEG = false>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   constexpr int KB = F8 ? 1 : 2;       // bytes per q / k element
   using SM = MfmaSmem<D, KB>;
@@ -983,7 +989,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   constexpr int LDK = NPIECE_K >= NWAVES ? NPIECE_K / NWAVES : 1;
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
   static_assert(SM::K_BYTES % 1024 == 0 && SM::V_BYTES % 1024 == 0, "tile must be a whole number of 1 KB pieces");
-  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0);   // direct loads per wave per step
+  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);   // direct loads per wave per step
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -993,9 +999,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS);
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG);
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
+  auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
   const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
 
@@ -1120,6 +1127,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
       if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
     }
+    if (SEG) {
+      // every wave brings the same 32 ids (each wave must issue the same number of loads); groups of 4
+      // past the row repeat the last group (L is a multiple of 4; those keys are masked by their index)
+      if (lane < BN / 4) {
+        int g4 = kv0 + 4 * lane;
+        g4 = g4 < p.Lkv - 4 ? g4 : p.Lkv - 4;
+        lds_dma16(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, Sg(st));
+      }
+    }
   };
 
   // prologue: the scaled bucket table (64 entries per wave, the last wave repeats the first), then
@@ -1153,6 +1169,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     // waits for every direct load in flight and serialises the whole ring.
 #pragma unroll
     for (int ks = 0; ks < QCH; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].y), "v"(qf[ks].z), "v"(qf[ks].w));
+  }
+  int32_t qseg = 0;
+  if (SEG) {
+    qseg = p.q_seg[(int64_t)b * p.L + (qrow < p.L ? qrow : p.L - 1)];
+    asm volatile("" ::"v"(qseg));
   }
   int64_t tq = 0;
   int32_t tq32 = 0;
@@ -1306,6 +1327,17 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         const int dist = kv > qrow ? kv - qrow : qrow - kv;
         const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow) && (win < 0 || dist <= win);
         u[r] = keep ? u[r] : 0.f;
+      }
+    }
+    if (SEG) {
+      const int32_t* sg = Sg(st);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int4 ks4 = *(const int4*)(sg + 8 * g + 4 * hh);
+        u[4 * g + 0] = ks4.x == qseg ? u[4 * g + 0] : 0.f;
+        u[4 * g + 1] = ks4.y == qseg ? u[4 * g + 1] : 0.f;
+        u[4 * g + 2] = ks4.z == qseg ? u[4 * g + 2] : 0.f;
+        u[4 * g + 3] = ks4.w == qseg ? u[4 * g + 3] : 0.f;
       }
     }
     float pv[16];
@@ -2428,7 +2460,10 @@ bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 bool mfma_eligible(const HstuAttnFwdArgs* a) {
   const int kb = a->qk_dtype == HSTU_DTYPE_FP8_E4M3FN ? 1 : 2;   // bytes per q / k element
   const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
-  const bool opts_ok = a->mask_mode != HSTU_MASK_SEGMENT && !a->mask && !a->dense_bias && a->L == a->Lkv &&
+  // segment ids: bf16 only, rows of a multiple of 4 ids (the kernel fetches them four at a time)
+  const bool seg_ok = a->mask_mode != HSTU_MASK_SEGMENT ||
+                      (kb == 2 && a->L % 4 == 0 && aligned16(a->q_segment_ids) && aligned16(a->kv_segment_ids));
+  const bool opts_ok = seg_ok && !a->mask && !a->dense_bias && a->L == a->Lkv &&
                        // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
                        (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
   auto s8 = [](int64_t x) { return (x & 7) == 0; };
@@ -2645,15 +2680,15 @@ int launch_bwd(const Params& p, hipStream_t st) {
   return HSTU_OK;
 }
 
-template <int D, bool POS, bool TS, bool F8>
+template <int D, bool POS, bool TS, bool F8, bool SEG = false>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS);
+  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG);
   static int granted[64];
-  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8>, smem, granted)) return rc;
+  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG>, smem, granted)) return rc;
   hipError_t e;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "mfma kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
@@ -2662,6 +2697,12 @@ int launch_mfma_inst(const Params& p, hipStream_t st) {
 template <int D, bool F8>
 int launch_mfma_d(const Params& p, hipStream_t st) {
   const bool pos = p.pos_tab != nullptr, ts = p.ts_tab != nullptr;
+  if (!F8 && p.mask_mode == HSTU_MASK_SEGMENT) {
+    if (pos && ts) return launch_mfma_inst<D, true, true, false, true>(p, st);
+    if (pos) return launch_mfma_inst<D, true, false, false, true>(p, st);
+    if (ts) return launch_mfma_inst<D, false, true, false, true>(p, st);
+    return launch_mfma_inst<D, false, false, false, true>(p, st);
+  }
   if (pos && ts) return launch_mfma_inst<D, true, true, F8>(p, st);
   if (pos) return launch_mfma_inst<D, true, false, F8>(p, st);
   if (ts) return launch_mfma_inst<D, false, true, F8>(p, st);
@@ -2724,7 +2765,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
 bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
-  if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
+  if (f.qk_dtype != HSTU_DTYPE_BF16 || f.mask_mode == HSTU_MASK_SEGMENT || !mfma_eligible(&f)) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||

@@ -514,3 +514,35 @@ def test_sliding_window_on_the_matrix_core_kernel(gpu, d, L, window, causal, pos
   outj = recml_amd.hstu_attention(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), seq_offsets=_dev(off.astype(np.int32)), max_len=L,
                                   causal=causal, sliding_window_size=window, **gk)
   assert _err(O.jagged_to_padded(outj.float().cpu().numpy(), off, L), ref) <= BF16_TOL
+
+
+@pytest.mark.parametrize("d,L,causal,window,pos", [
+    (128, 400, True, None, False),
+    (128, 400, True, 50, True),
+    (64, 260, False, None, True),
+    (32, 132, True, None, False),
+])
+def test_segment_ids_on_the_matrix_core_kernel(gpu, d, L, causal, window, pos):
+  """Packed rows: several segments per row plus a padding segment (the reference's test recipe,
+  hstu_ops_test.py:36-41, has two), bf16 on the matrix-core kernel."""
+  rng = np.random.default_rng(300 + L)
+  B, H = 3, 2
+  bf = torch.bfloat16
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  seg = np.zeros((B, L), np.int32)
+  seg[0, :L // 3], seg[0, L // 3: L - 7] = 1, 2            # two sequences and a short padding tail
+  seg[1, :] = 5                                             # one sequence over the whole row
+  cuts = np.sort(rng.choice(np.arange(1, L), 9, replace=False))
+  seg[2] = np.searchsorted(cuts, np.arange(L), side="right") + 1   # ten short ones
+  kw, gk = {}, {}
+  if pos:
+    kw["pos_tab"] = (rng.standard_normal((H, 2 * L - 1)) * 0.1).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  ref = O.hstu_attention_ref(q, k, v, causal=causal, q_segment_ids=seg, kv_segment_ids=seg,
+                             sliding_window_size=window, dtype=np.float32, **kw)
+  a, keep = hstu_ops.build_args(_dev(q, bf), _dev(k, bf), _dev(v, bf), torch.empty((B, L, H, d), dtype=bf, device="cuda:0"),
+                                causal=causal, q_segment_ids=_dev(seg), kv_segment_ids=_dev(seg),
+                                sliding_window_size=window, **gk)
+  assert hstu_ops.kernel_variant(a) == "hstu_fwd_mfma_bf16"
+  hstu_ops._run(a, keep)
+  assert _err(keep[3].float().cpu().numpy(), ref) <= BF16_TOL

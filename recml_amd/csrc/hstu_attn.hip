@@ -665,14 +665,27 @@ typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
 // every wave issues the same number per step and waits with s_waitcnt vmcnt(n)
 // before the barrier that publishes a stage.
 __device__ __forceinline__ void lds_dma16(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
-  const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_byte_ptr)lds_dst_wave_uniform);
+  // the low half of a flat pointer into LDS is the LDS address (no address-space cast: its null check
+  // trips the compiler in some instantiations)
+  const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_dst_wave_uniform);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(base), "v"(byte_off), "s"(gbase_uniform)
+               : "memory", "m0");
+}
+// The same with the destination given as an LDS byte address: the dynamic LDS array of a kernel
+// starts where its static LDS ends (these kernels have none of the latter).
+__device__ __forceinline__ void lds_dma16_at(const void* gbase_uniform, uint32_t byte_off, uint32_t lds_addr_wave_uniform) {
+  const uint32_t base = __builtin_amdgcn_readfirstlane(lds_addr_wave_uniform);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(base), "v"(byte_off), "s"(gbase_uniform)
                : "memory", "m0");
 }
 __device__ __forceinline__ void lds_dma4(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
-  const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_byte_ptr)lds_dst_wave_uniform);
+  // the low half of a flat pointer into LDS is the LDS address (no address-space cast: its null check
+  // trips the compiler in some instantiations)
+  const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_dst_wave_uniform);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                :
                : "s"(base), "v"(byte_off), "s"(gbase_uniform)
@@ -993,6 +1006,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
   // LDS map: [ring: NSTAGE x (K | V)][bias operands x NSTAGE: 4 pos windows | key timestamps][ts table].
   // The key timestamps sit right behind the last position window so that one direct load of the
   // last wave can fill both.
@@ -1133,7 +1147,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       if (lane < BN / 4) {
         int g4 = kv0 + 4 * lane;
         g4 = g4 < p.Lkv - 4 ? g4 : p.Lkv - 4;
-        lds_dma16(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, Sg(st));
+        lds_dma16_at(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
       }
     }
   };
@@ -1582,6 +1596,13 @@ __device__ __forceinline__ float wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// float atomic add on an LDS location given by an ordinary pointer (named as LDS for the compiler: on
+// a pointer of unknown address space it builds a run-time dispatch that some instantiations miscompile)
+typedef __attribute__((address_space(3))) float* lds_float_ptr;
+__device__ __forceinline__ void lds_atomic_add(float* lds_location, float v) {
+  __hip_atomic_fetch_add((lds_float_ptr)lds_location, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 // TG: also accumulate the table gradients.  Every pair adds its dS to the entry of each table its
 // logit read; LDS float atomics turned out to cost about 4 cycles per lane, so the sums are formed
 // in registers first and each wave keeps its own LDS accumulators, updated without atomics.
@@ -1594,7 +1615,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // the same bucket are summed across the wave and one lane adds the sum to the workgroup's
 // histogram (an LDS atomic, but of one lane); only blocks with more buckets per lane use one
 // atomic per lane and run of equal buckets.
-template <int D, bool POS, bool TS, bool TG>
+template <int D, bool POS, bool TS, bool TG, bool SEG = false>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
@@ -1602,16 +1623,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;            // 1 KB pieces of a tile; small tiles: several waves repeat a piece
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS);
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG);
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
+  auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
   const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
   float* TgBase = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
@@ -1698,6 +1721,14 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       }
       if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
     }
+    if (SEG) {
+      // the step's 32 key segment ids, as in the forward
+      if (lane < BN / 4) {
+        int g4 = kv0 + 4 * lane;
+        g4 = g4 < p.Lkv - 4 ? g4 : p.Lkv - 4;
+        lds_dma16_at(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
+      }
+    }
   };
 
   if (TS) {
@@ -1732,6 +1763,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].y), "v"(qf[ks].z), "v"(qf[ks].w));
       asm volatile("" ::"v"(dof[ks].x), "v"(dof[ks].y), "v"(dof[ks].z), "v"(dof[ks].w));
     }
+  }
+  int32_t qseg = 0;
+  if (SEG) {
+    qseg = p.q_seg[(int64_t)b * p.L + (qrow < p.L ? qrow : p.L - 1)];
+    asm volatile("" ::"v"(qseg));
   }
   int64_t tq = 0;
   int32_t tq32 = 0;
@@ -1883,6 +1919,17 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         ds[r] = keep ? ds[r] : 0.f;
       }
     }
+    if (SEG) {
+      const int32_t* sg = Sg(st);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int4 ks4 = *(const int4*)(sg + 8 * g + 4 * hh);
+        ds[4 * g + 0] = ks4.x == qseg ? ds[4 * g + 0] : 0.f;
+        ds[4 * g + 1] = ks4.y == qseg ? ds[4 * g + 1] : 0.f;
+        ds[4 * g + 2] = ks4.z == qseg ? ds[4 * g + 2] : 0.f;
+        ds[4 * g + 3] = ks4.w == qseg ? ds[4 * g + 3] : 0.f;
+      }
+    }
     if (want_dpos) {
       // Pair (row m, key offset c = 8g + 4hh + tt) lies on diagonal c - m.  Lane j takes, for each of
       // its 16 offsets, the value of row (j + c) mod 32 of its half: all 16 are then on diagonal -j or,
@@ -1927,8 +1974,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
           const float a = wave_sum(mine ? s_near : 0.f);
           const float c = any_far ? wave_sum(mine ? s_far : 0.f) : 0.f;
           if (lane == 0) {
-            atomicAdd(&hist[b0], a);
-            if (any_far) atomicAdd(&hist[b0 + 1], c);
+            lds_atomic_add(&hist[b0], a);
+            if (any_far) lds_atomic_add(&hist[b0 + 1], c);
           }
           done = done || mine;
         }
@@ -1942,7 +1989,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
           const uint32_t bnext = r < 15 ? (bkp[(r + 1) >> 2] >> (8 * ((r + 1) & 3))) & 255u : 256u;
           carry += ds[r];
           if (bcur != bnext) {
-            if (carry != 0.f) atomicAdd(&hist[bcur], carry);
+            if (carry != 0.f) lds_atomic_add(&hist[bcur], carry);
             carry = 0.f;
           }
         }
@@ -2058,7 +2105,7 @@ struct DkvShape {
   static constexpr int DW = D / DSPLIT;                  // channels of dK / dV per wave
 };
 
-template <int D, bool POS, bool TS>
+template <int D, bool POS, bool TS, bool SEG = false>
 __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
   using SH = DkvShape<D>;
   constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
@@ -2070,7 +2117,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;
   constexpr int LD = NPIECE >= NW ? NPIECE / NW : 1;
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0);
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
   // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
   // (min, max) of timestamp tiles t and t + 1
@@ -2078,11 +2125,13 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   constexpr int TQ_BYTES = TQ_LANES * 16;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
   // ring stage: [Q tile | dO tile], 32 rows each
   auto Qs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Os = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0);
+  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0) + (SEG ? SM::SEG_BYTES : 0);
+  auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0)); };
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
@@ -2186,6 +2235,14 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
       }
       if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
     }
+    if (SEG) {
+      // the step's 32 row segment ids (every wave the same load; groups of 4 past the row repeat the last)
+      if (lane < BN / 4) {
+        int g4 = qbs + 4 * lane;
+        g4 = g4 < p.L - 4 ? g4 : p.L - 4;
+        lds_dma16_at(p.q_seg + (int64_t)b * p.L, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
+      }
+    }
   };
 
   if (TS) {
@@ -2231,6 +2288,11 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
       asm volatile("" ::"v"(kfr[ks].x), "v"(kfr[ks].y), "v"(kfr[ks].z), "v"(kfr[ks].w));
       asm volatile("" ::"v"(vfr[ks].x), "v"(vfr[ks].y), "v"(vfr[ks].z), "v"(vfr[ks].w));
     }
+  }
+  int32_t kseg = 0;
+  if (SEG) {
+    kseg = p.kv_seg[(int64_t)b * p.Lkv + (kcol < p.Lkv ? kcol : p.Lkv - 1)];
+    asm volatile("" ::"v"(kseg));
   }
   int64_t tk = 0;
   int32_t tk32 = 0;
@@ -2388,6 +2450,18 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
         const bool keep = (qi < s.n_q) && (kcol < s.n_kv) && (!p.causal || kcol <= qi) && (win < 0 || dist <= win);
         pv[r] = keep ? pv[r] : 0.f;
         ds[r] = keep ? ds[r] : 0.f;
+      }
+    }
+    if (SEG) {
+      const int32_t* sg = Sg(st);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int4 qs4 = *(const int4*)(sg + 8 * g + 4 * hh);
+        const bool k0 = qs4.x == kseg, k1 = qs4.y == kseg, k2 = qs4.z == kseg, k3 = qs4.w == kseg;
+        pv[4 * g + 0] = k0 ? pv[4 * g + 0] : 0.f;  ds[4 * g + 0] = k0 ? ds[4 * g + 0] : 0.f;
+        pv[4 * g + 1] = k1 ? pv[4 * g + 1] : 0.f;  ds[4 * g + 1] = k1 ? ds[4 * g + 1] : 0.f;
+        pv[4 * g + 2] = k2 ? pv[4 * g + 2] : 0.f;  ds[4 * g + 2] = k2 ? ds[4 * g + 2] : 0.f;
+        pv[4 * g + 3] = k3 ? pv[4 * g + 3] : 0.f;  ds[4 * g + 3] = k3 ? ds[4 * g + 3] : 0.f;
       }
     }
 #pragma unroll
@@ -2765,7 +2839,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
 bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
-  if (f.qk_dtype != HSTU_DTYPE_BF16 || f.mask_mode == HSTU_MASK_SEGMENT || !mfma_eligible(&f)) return false;
+  if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
@@ -2774,34 +2848,39 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
 }
 
-template <int D, bool POS, bool TS, bool TG>
+template <int D, bool POS, bool TS, bool TG, bool SEG = false>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, 2>::total(POS, TS);
+  const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
   // one more 16-byte piece of timestamp operands per stage; the tile's K and V rows where they stay in LDS
   const int smem_kv = smem + (TS ? NSTAGE * 16 : 0) + (DkvShape<D>::KV_LDS ? 2 * BM * D * 2 : 0);
   static int granted_q[64], granted_kv[64];
-  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG>, smem_q, granted_q)) return rc;
-  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS>, smem_kv, granted_kv)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG>, smem_q, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG>, smem_kv, granted_kv)) return rc;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG, SEG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS, SEG>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
 }
 
-template <int D>
-int launch_bwd_mfma_d(const Params& q, hipStream_t st) {
+template <int D, bool SEG>
+int launch_bwd_mfma_ds(const Params& q, hipStream_t st) {
   const bool pos = q.pos_tab != nullptr, ts = q.ts_tab != nullptr;
   const bool tg = (pos && q.dpos) || (ts && q.dts);
-  if (pos && ts) return tg ? launch_bwd_mfma_inst<D, true, true, true>(q, st) : launch_bwd_mfma_inst<D, true, true, false>(q, st);
-  if (pos) return tg ? launch_bwd_mfma_inst<D, true, false, true>(q, st) : launch_bwd_mfma_inst<D, true, false, false>(q, st);
-  if (ts) return tg ? launch_bwd_mfma_inst<D, false, true, true>(q, st) : launch_bwd_mfma_inst<D, false, true, false>(q, st);
-  return launch_bwd_mfma_inst<D, false, false, false>(q, st);
+  if (pos && ts) return tg ? launch_bwd_mfma_inst<D, true, true, true, SEG>(q, st) : launch_bwd_mfma_inst<D, true, true, false, SEG>(q, st);
+  if (pos) return tg ? launch_bwd_mfma_inst<D, true, false, true, SEG>(q, st) : launch_bwd_mfma_inst<D, true, false, false, SEG>(q, st);
+  if (ts) return tg ? launch_bwd_mfma_inst<D, false, true, true, SEG>(q, st) : launch_bwd_mfma_inst<D, false, true, false, SEG>(q, st);
+  return launch_bwd_mfma_inst<D, false, false, false, SEG>(q, st);
+}
+
+template <int D>
+int launch_bwd_mfma_d(const Params& q, hipStream_t st) {
+  return q.mask_mode == HSTU_MASK_SEGMENT ? launch_bwd_mfma_ds<D, true>(q, st) : launch_bwd_mfma_ds<D, false>(q, st);
 }
 
 int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {

@@ -92,9 +92,12 @@ def test_backward_variant_query():
   b.dq = 0x20004                                                      # gradient buffers must be 16-byte aligned for it
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
   b.dq = 0x20000
-  f.window = 8                                                        # an option the matrix-core kernels do not take
-  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  f.window = 8                                                        # a sliding window stays on the matrix cores
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
   f.window = -1
+  f.mask = 0x50000                                                    # an explicit mask does not
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  f.mask = None
   f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_FP32
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<float>"
 

@@ -211,3 +211,36 @@ def test_backward_sliding_window_on_the_matrix_cores(gpu, d, L, window, causal, 
   for b in range(B):
     for g in got[:3]:
       assert (g[b, lens[b]:] == 0).all()
+
+
+@pytest.mark.parametrize("d,L,causal,window,pos", [
+    (128, 400, True, None, True),
+    (64, 260, False, 40, False),
+    (32, 132, True, None, False),
+])
+def test_backward_segment_ids_on_the_matrix_cores(gpu, d, L, causal, window, pos):
+  """Packed rows (several segments per row and a padding segment) through the matrix-core backward."""
+  rng = np.random.default_rng(400 + L)
+  B, H = 3, 2
+  bf = torch.bfloat16
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  seg = np.zeros((B, L), np.int32)
+  seg[0, :L // 3], seg[0, L // 3: L - 7] = 1, 2
+  seg[1, :] = 5
+  cuts = np.sort(rng.choice(np.arange(1, L), 9, replace=False))
+  seg[2] = np.searchsorted(cuts, np.arange(L), side="right") + 1
+  kw, gk = {}, {}
+  if pos:
+    kw["pos_tab"] = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, causal=causal, q_segment_ids=seg, kv_segment_ids=seg,
+                                  sliding_window_size=window, **kw)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), causal=causal,
+                                     q_segment_ids=_dev(seg), kv_segment_ids=_dev(seg), sliding_window_size=window,
+                                     _variant_out=variant, **gk)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv", "dpos"), got[:4], want[:4]):
+    assert (g is None) == (w is None), nm
+    if g is not None:
+      assert _rel(g.float().cpu().numpy().reshape(w.shape), w) <= 2e-2, nm

@@ -1,16 +1,17 @@
-// HSTU pointwise-SiLU attention forward for gfx950 (MI355X, CDNA4).
+// HSTU pointwise-SiLU attention, forward and backward, for gfx950 (MI355X, CDNA4).
 //
 //   out[b,i,h,:] = sum_j M[b,i,j] * silu(alpha*q_i.k_j + bias(b,h,i,j)) * inv_n * v[b,j,h,:]
 //
-// Kernels behind the one C entry point (see include/hstu_attn.h):
+// Kernels behind the C entry points (see include/hstu_attn.h).  Forward:
 //
 //   hstu_fwd_mfma_bf16   the hot path.  bf16 (or fp8 e4m3fn) Q/K, bf16 V, fp32
 //                        accumulation on the 32x32x16 MFMA; 128 query rows per
 //                        workgroup, keys streamed 32 at a time through a
 //                        4-stage LDS ring filled by direct global->LDS loads;
 //                        relative-position and timestamp bias + SiLU + mask
-//                        fused on the accumulator registers; causal / length
-//                        tile skipping.  Computes S^T = K Q^T so that the
+//                        fused on the accumulator registers; causal / length /
+//                        sliding-window tile skipping, segment ids.  Computes
+//                        S^T = K Q^T so that the
 //                        accumulator layout of S^T is already the B-operand
 //                        layout of O^T = V^T P^T: P never touches LDS.
 //   hstu_prepare         runs before it: work list of (sequence, tile) items,
@@ -24,6 +25,16 @@
 //                        arithmetic.  Correctness path for the options the
 //                        MFMA kernel does not cover and the fp32 reference
 //                        configuration.
+//
+// Backward (dq, dk, dv and the gradients of the two bias tables):
+//
+//   hstu_bwd_dq_mfma     bf16 on the matrix cores under the conditions of the
+//   hstu_bwd_dkv_mfma    MFMA forward: one kernel per 128 query rows streaming
+//                        K and V, one per 128 keys streaming Q and dO; both
+//                        recompute the logits; the first also sums the table
+//                        gradients.
+//   hstu_bwd_dq,         every option, fp32 FMA arithmetic.
+//   hstu_bwd_dkv
 //
 // The math follows recml/layers/keras/hstu.py:356-390 (dense formulation),
 // recml/core/ops/hstu_ops.py:230-264 (order: scale, SiLU, 1/N, mask, PV in

@@ -2082,13 +2082,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
 }
 
 // At d = 128 two 32 x 128 accumulators plus the K and V fragments are 192 registers before any
-// temporary: one workgroup per CU, the accumulators in the accumulation registers, and a compiler
-// that then moves values between the two register files on every block (2.6x the vector
-// instructions of the dQ kernel).  Two remedies are built in.  KV_LDS: the wave's K and V rows
-// stay in LDS (64 KB more per workgroup, which one workgroup per CU can afford) and are read as B
-// operands on every block, so that the ordinary registers hold temporaries only.  DSPLIT = 2: the
-// work of 32 keys is shared by two waves, each accumulating dK and dV for half of the channels
-// (measured: no gain, both waves repeat S, dP and the pointwise math).
+// temporary: one workgroup per CU, the accumulators in the accumulation registers (ACC_ASM below).
+// DSPLIT = 2 would share the work of 32 keys between two waves, each accumulating dK and dV for
+// half of the channels (8 waves per workgroup): measured, no gain -- both waves repeat S, dP and
+// the pointwise math -- and left at 1.
 // acc = 0 and acc += A B with the accumulator named as accumulation registers (ACC_ASM).  Left to the
 // compiler, the loop-carried accumulators of the d = 128 kernel live in ordinary registers and all
 // 128 are copied to the accumulation file and back around the products of every block.  Written
@@ -2108,7 +2105,6 @@ __device__ __forceinline__ void mfma_acc(floatx16& acc, bf16x8 a, bf16x8 b) {
 
 template <int D>
 struct DkvShape {
-  static constexpr bool KV_LDS = false;
   static constexpr bool ACC_ASM = D == 128;
   static constexpr int DSPLIT = 1;                       // waves per 32 keys
   static constexpr int NW = NWAVES * DSPLIT;             // waves per workgroup
@@ -2120,7 +2116,7 @@ template <int D, bool POS, bool TS, bool SEG = false>
 __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
   using SH = DkvShape<D>;
   constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
-  constexpr bool KV_LDS = SH::KV_LDS, ACC_ASM = SH::ACC_ASM;
+  constexpr bool ACC_ASM = SH::ACC_ASM;
   constexpr int DVBW = DW / 32;          // 32-channel blocks of dK / dV per wave
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
@@ -2147,10 +2143,6 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
   const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
-  // KV_LDS: [K rows of the tile][V rows of the tile], 128 x D bf16 each, two-way swizzle by row within a wave's 32
-  constexpr int KV_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
-  unsigned char* Kst = smem + KV_OFF;
-  unsigned char* Vst = Kst + BM * D * 2;
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -2262,29 +2254,13 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
     lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
     lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
   }
-  if (KV_LDS) {
-    // this wave's 32 K rows and 32 V rows, 1 KB per load; rows past the sequence repeat the last one (masked later)
-    const int last = s.n_kv - 1;
-    const char* kgl = (const char*)p.k + s.bk * 2;
-    const char* vgl = (const char*)p.v + s.bv * 2;
-#pragma unroll
-    for (int j = 0; j < 32 * D * 2 / 1024; ++j) {
-      const int c = 64 * j + lane;
-      const int row = c / CPR, pc = c - row * CPR;
-      int grow = r0 + row;
-      grow = grow < last ? grow : last;
-      const uint32_t sw = (uint32_t)((pc ^ swz_rt<D>(row)) * 16);
-      lds_dma16(kgl, (uint32_t)grow * ((uint32_t)p.k_st * 2u) + sw, Kst + w * (32 * D * 2) + j * 1024);
-      lds_dma16(vgl, (uint32_t)grow * ((uint32_t)p.v_st * 2u) + sw, Vst + w * (32 * D * 2) + j * 1024);
-    }
-  }
 #pragma unroll
   for (int t = 0; t < NSTAGE - 1; ++t)
     if (t_lo + t < nt) dma_step(t_lo + t);
 
   // K and V fragments of this lane's key (B operands)
   uint4 kfr[QCH], vfr[QCH];
-  if (!KV_LDS) {
+  {
     const char* kp = (const char*)p.k + (s.bk + (int64_t)kcol * p.k_st) * 2 + 16 * hh;
     const char* vp = (const char*)p.v + (s.bv + (int64_t)kcol * p.v_st) * 2 + 16 * hh;
 #pragma unroll
@@ -2346,11 +2322,9 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
 #pragma unroll
       for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
 #pragma unroll
-      for (int ks = 0; ks < QCH; ++ks) {
-        const uint4 bk = KV_LDS ? *(const uint4*)(Kst + (32 * w + m) * (D * 2) + (((2 * ks + hh) ^ gk) * 16)) : kfr[ks];
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, bk),
+      for (int ks = 0; ks < QCH; ++ks)
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, kfr[ks]),
                                                        ks == 0 ? zero : sacc, 0, 0, 0);
-      }
     }
     {
       uint4 af[QCH];
@@ -2358,11 +2332,9 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
 #pragma unroll
       for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
 #pragma unroll
-      for (int ks = 0; ks < QCH; ++ks) {
-        const uint4 bv = KV_LDS ? *(const uint4*)(Vst + (32 * w + m) * (D * 2) + (((2 * ks + hh) ^ gk) * 16)) : vfr[ks];
-        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, bv),
+      for (int ks = 0; ks < QCH; ++ks)
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, vfr[ks]),
                                                         ks == 0 ? zero : dpacc, 0, 0, 0);
-      }
     }
     float u[16];
     if (POS) {
@@ -2863,8 +2835,7 @@ template <int D, bool POS, bool TS, bool TG, bool SEG = false>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
-  // one more 16-byte piece of timestamp operands per stage; the tile's K and V rows where they stay in LDS
-  const int smem_kv = smem + (TS ? NSTAGE * 16 : 0) + (DkvShape<D>::KV_LDS ? 2 * BM * D * 2 : 0);
+  const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
   static int granted_q[64], granted_kv[64];
   if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG>, smem_q, granted_q)) return rc;
   if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG>, smem_kv, granted_kv)) return rc;

@@ -1946,7 +1946,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       // its 16 offsets, the value of row (j + c) mod 32 of its half: all 16 are then on diagonal -j or,
       // where j + c wrapped, 32 - j.  The two sums are completed with the other half's and added to
       // the wave's ring: lanes of the lower half own -j, lanes of the upper half 32 - j.
-      const int jj = m + 4 * hh;
+      // (the lane's index enters through a register the compiler cannot see through: it would otherwise
+      // keep the 16 permute addresses of the loop below in registers across the whole key loop, which
+      // this kernel does not have)
+      int jj = m + 4 * hh;
+      asm volatile("" : "+v"(jj));
       const int half4 = (lane & 32) << 2;
       float s_all = 0.f, s_low = 0.f;
 #pragma unroll

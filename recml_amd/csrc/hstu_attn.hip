@@ -1524,9 +1524,9 @@ __global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
 // tile is therefore read both ways, and one swizzle serves both: 16-byte chunk c of row r sits at
 // chunk c ^ swz_rt<D>(r), which spreads 16 consecutive rows over the 16 chunk slots of a 256-byte
 // sweep of the banks (row reads) and 4 consecutive rows over 4 different 64-byte groups (transpose
-// reads).  P and dS are rounded to bf16
-// for the last products like P in the forward.  Neither kernel splits its streamed range.  The
-// table gradients, when wanted, come from the dQ kernel, which sees every pair once.
+// reads).  P and dS are rounded to bf16 for the last products like P in the forward.  Neither
+// kernel splits its streamed range.  The table gradients, when wanted, come from the dQ kernel,
+// which sees every pair once.  Sliding window and segment ids as in the forward.
 // ---------------------------------------------------------------------------
 
 constexpr float LN2 = 0.6931471805599453f;

@@ -1,6 +1,6 @@
 """Benchmark of the HSTU attention forward on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c3full|c2|c4|c5|c4-model] [--backward]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c3full|c2|c4|c5|c4-model|c4-block-steps] [--backward]
 
 A step is one pass of the attention forward over one synthetic batch whose
 inputs already sit in HBM.  The default workload is the one the headline
@@ -222,6 +222,78 @@ def bench_model(args, dev):
       "model_tflops": (attn_flops + proj_flops) / (ms * 1e-3) / 1e12}))
 
 
+def bench_block_steps(args, dev):
+  """The two fused block steps at the config-4 size (T = 73 728 packed tokens, D = 512): one JSON line.
+
+  value / roofline: the norm + gate step, which is bound by HBM (3 x T x D x 2 bytes: the attention
+  output and the U slice read once, the result written once); the projection product with the SiLU
+  epilogue is reported beside it in TFLOP/s."""
+  import torch
+  import recml_amd
+  from oracle import hstu_block_oracle as BO
+  T, D = 73728, 512
+  bf = torch.bfloat16
+  gen = torch.Generator(device=dev).manual_seed(7)
+  fused = torch.randn((T, 4, D), device=dev, dtype=bf, generator=gen)
+  u = fused[:, 0]
+  attn = (torch.randn((T, D), device=dev, generator=gen) * 1e-3).to(bf)
+  gamma = (1 + 0.1 * torch.randn(D, device=dev, generator=gen)).to(bf)
+  beta = (0.1 * torch.randn(D, device=dev, generator=gen)).to(bf)
+  x = (torch.randn((T, D), device=dev, generator=gen) * 0.5).to(bf)
+  w = (torch.randn((D, 4 * D), device=dev, generator=gen) * 0.05).to(bf)
+
+  def timed(fn):
+    for _ in range(args.warmup):
+      fn()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for a, b in ev:
+      a.record()
+      fn()
+      b.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / args.steps
+    return wall, float(np.mean([a.elapsed_time(b) for a, b in ev]))
+
+  ng = lambda: recml_amd.norm_gate(attn, u, gamma, beta, 1e-6)
+  wall_ng, ker_ng = timed(ng)
+  wall_t, _ = timed(lambda: u * torch.nn.functional.layer_norm(attn, (D,), gamma, beta, 1e-6))
+  wall_g, ker_g = timed(lambda: recml_amd.gemm_silu(x, w, None, True))
+  wall_gt, _ = timed(lambda: torch.nn.functional.silu(x @ w))
+  nbytes = 3 * T * D * 2
+  gflop = 2.0 * T * D * 4 * D / 1e9
+  out = ng().float().cpu().numpy()
+  rec = {
+      "metric": "HSTU block norm + gate step, GB/s (config-4 size)", "value": nbytes / (wall_ng * 1e-3) / 1e9, "unit": "GB/s",
+      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall_ng, "higher_is_better": True,
+      "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, fp32 arithmetic", "data": "synthetic",
+      "config": {"workload": f"C4 block steps: T={T} packed tokens, D={D}", "kernel": "hstu_norm_gate<1>"},
+      "roofline": {"bound": "hbm", "achieved": nbytes / (ker_ng * 1e-3) / 1e9, "peak": 8000.0, "unit": "GB/s",
+                   "frac": nbytes / (ker_ng * 1e-3) / 1e9 / 8000.0, "traffic": None, "kernel_ms_avg": ker_ng,
+                   "algorithmic_bytes": nbytes},
+      "torch_layer_norm_then_mul_ms": wall_t,
+      "gemm_silu": {"ms_per_call": wall_g, "event_ms": ker_g, "tflops": gflop / ker_g, "torch_mm_then_silu_ms": wall_gt,
+                    "shape": [T, D, 4 * D]},
+  }
+  if not args.no_cpu:
+    rows = 4096
+    a_np, u_np = attn[:rows].float().cpu().numpy(), u[:rows].float().cpu().numpy()
+    g_np, b_np = gamma.float().cpu().numpy(), beta.float().cpu().numpy()
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 10.0:
+      ref = u_np * BO.layer_norm(a_np, g_np, b_np, 1e-6)
+      reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    rec["cpu_baseline"] = {"value": 3 * rows * D * 2 / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                           "sample": f"numpy restatement on the first {rows} rows, {reps} repetitions in 10 s"}
+    rec["parity_max_abs_over_max_ref"] = float(np.abs(out[:rows] - ref).max() / np.abs(ref).max())
+    if not rec["parity_max_abs_over_max_ref"] <= 8e-3:
+      raise SystemExit(f"norm + gate parity failed in the benchmark run: {rec['parity_max_abs_over_max_ref']}")
+  print(json.dumps(rec))
+
+
 def bench_backward(args, w, q, k, v, kw, dev):
   """The backward pass on the same workload, table gradients included: one JSON line.
 
@@ -319,6 +391,8 @@ def main():
   dev = torch.device("cuda:0")
   if args.workload == "c4-model":
     return bench_model(args, dev)
+  if args.workload == "c4-block-steps":
+    return bench_block_steps(args, dev)
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
   if args.backward:

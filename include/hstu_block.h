@@ -1,0 +1,95 @@
+/* C ABI of libhstu_block.so: the two fused steps of the HSTU block that sit on
+ * either side of the attention kernel (recml/layers/keras/hstu.py:444-474),
+ * for gfx950.  bf16 tensors, row-major, on the current device; fp32 arithmetic
+ * inside.  Plain pointers and sizes: no framework types.
+ *
+ *   hstu_gemm_silu_fwd    out = silu(x W + bias): the U, Q, K, V projections of
+ *                         the normalised input with their activation
+ *                         (hstu.py:444-449, the EinsumDense layers of :281-330
+ *                         with activation="silu"), as ONE matrix product with
+ *                         the activation applied by the product's epilogue
+ *                         (hipBLASLt) instead of a pass of its own.
+ *   hstu_norm_gate_fwd    out = u * layer_norm(attn): the layer norm over
+ *                         (heads, head_dim) of the attention output and the U
+ *                         gate (hstu.py:471-472) in one pass over memory.
+ *
+ * Every function returns 0 or a negative HstuBlockStatus; the message of the
+ * last failure on the calling thread is at hstu_block_last_error().
+ */
+#ifndef HSTU_BLOCK_H_
+#define HSTU_BLOCK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HSTU_BLOCK_ABI_VERSION 1
+
+typedef enum HstuBlockStatus {
+  HSTU_BLOCK_OK = 0,
+  HSTU_BLOCK_ERR_NULL = -1,
+  HSTU_BLOCK_ERR_VERSION = -2,
+  HSTU_BLOCK_ERR_SHAPE = -4,
+  HSTU_BLOCK_ERR_WORKSPACE = -5,
+  HSTU_BLOCK_ERR_LAUNCH = -6,
+  HSTU_BLOCK_ERR_BLAS = -7      /* hipBLASLt has no kernel for the request, or failed */
+} HstuBlockStatus;
+
+/* out[t, :] = u[t, :] * (gamma * (a[t, :] - mean_t) * rstd_t + beta), mean and
+ * (biased) variance of a[t, :] over its `width` entries, rstd = 1/sqrt(var + eps)
+ * (keras LayerNormalization over the last two axes of [.., H, hd] flattened,
+ * hstu.py:340-346 and :471-472).  a, u, out: bf16 [rows, width] with the given
+ * row strides in elements (u is usually a slice of the fused projection);
+ * gamma, beta: bf16 [width].  width a multiple of 8 up to 8192; pointers and
+ * row strides multiples of 8 elements (16 bytes). */
+typedef struct HstuNormGateArgs {
+  uint32_t struct_size;   /* sizeof(HstuNormGateArgs)  */
+  uint32_t version;       /* HSTU_BLOCK_ABI_VERSION    */
+  int64_t rows;
+  int32_t width;
+  float eps;
+  const void* a;
+  const void* u;
+  void* out;
+  int64_t a_stride, u_stride, out_stride;
+  const void* gamma;
+  const void* beta;
+} HstuNormGateArgs;
+
+int hstu_norm_gate_fwd(const HstuNormGateArgs* args, void* stream);
+
+/* out[m, n] = silu(sum_k x[m, k] w[k, n] + bias[n]); x: bf16 [M, K] (row stride
+ * x_stride), w: bf16 [K, N] contiguous, bias: bf16 [N] or null, out: bf16
+ * [M, N] contiguous.  fp32 accumulation.  `workspace` (device memory, may be
+ * null) is handed to hipBLASLt; hstu_gemm_silu_workspace_bytes() says how much
+ * it would like.  The descriptor and the chosen algorithm of a shape are kept
+ * by the library after the first call with it. */
+typedef struct HstuGemmSiluArgs {
+  uint32_t struct_size;   /* sizeof(HstuGemmSiluArgs)  */
+  uint32_t version;       /* HSTU_BLOCK_ABI_VERSION    */
+  int64_t M;
+  int32_t N, K;
+  int32_t activation;     /* 1: silu (the projections); 0: none */
+  int32_t reserved0;
+  const void* x;
+  int64_t x_stride;
+  const void* w;
+  const void* bias;
+  void* out;
+  void* workspace;
+  size_t workspace_bytes;
+} HstuGemmSiluArgs;
+
+size_t hstu_gemm_silu_workspace_bytes(void);
+int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* args, void* stream);
+
+int hstu_block_abi_version(void);
+const char* hstu_block_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_BLOCK_H_ */

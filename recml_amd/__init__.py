@@ -1,4 +1,4 @@
-"""MI355X-native HSTU pointwise-SiLU attention (forward).
+"""MI355X-native HSTU pointwise-SiLU attention (forward and backward).
 
 Public surface mirrors the reference operator
 (recml/core/ops/hstu_ops.py:829-851), the layer-side call
@@ -14,6 +14,7 @@ from recml_amd.hstu_ops import (  # noqa: F401
     pointwise_attention,
     pointwise_splash_attention,
 )
+from recml_amd.hstu_block_ops import gemm_silu, norm_gate  # noqa: F401
 from recml_amd.masks import make_attention_mask, make_causal_mask  # noqa: F401
 from recml_amd.hstu_layer import HSTU, HSTUBlock  # noqa: F401
 from recml_amd.hstu_bias import (  # noqa: F401

@@ -11,6 +11,10 @@ ROOT = os.path.dirname(_HERE)
 LIB_DIR = os.path.join(_HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libhstu_attn.so")
 SOURCES = [os.path.join(_HERE, "csrc", "hstu_attn.hip")]
+# the block-side steps live in a library of their own: they bring hipBLASLt along, the attention does not
+BLOCK_LIB_PATH = os.path.join(LIB_DIR, "libhstu_block.so")
+BLOCK_SOURCES = [os.path.join(_HERE, "csrc", "hstu_block.hip")]
+BLOCK_LINK = ["-lhipblaslt"]
 INCLUDE = os.path.join(ROOT, "include")
 
 # -packed-fp32-ops is switched off for the device pass: packed fp32
@@ -29,19 +33,29 @@ def hipcc() -> str:
   return exe
 
 
-def build_library(verbose: bool = False) -> str:
-  """Compiles every HIP source into recml_amd/lib/libhstu_attn.so."""
+def _compile(sources, out, link=(), verbose=False) -> str:
   os.makedirs(LIB_DIR, exist_ok=True)
-  tmp = LIB_PATH + ".tmp"
-  cmd = [hipcc(), *HIPCC_FLAGS, "-I", INCLUDE, "-o", tmp, *SOURCES]
+  tmp = out + ".tmp"
+  cmd = [hipcc(), *HIPCC_FLAGS, "-I", INCLUDE, "-o", tmp, *sources, *link]
   res = subprocess.run(cmd, capture_output=True, text=True)
   if res.returncode != 0:
     raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
   if verbose:
     print(res.stderr)
-  os.replace(tmp, LIB_PATH)
-  return LIB_PATH
+  os.replace(tmp, out)
+  return out
+
+
+def build_library(verbose: bool = False) -> str:
+  """Compiles the attention kernels into recml_amd/lib/libhstu_attn.so."""
+  return _compile(SOURCES, LIB_PATH, verbose=verbose)
+
+
+def build_block_library(verbose: bool = False) -> str:
+  """Compiles the block-side steps into recml_amd/lib/libhstu_block.so."""
+  return _compile(BLOCK_SOURCES, BLOCK_LIB_PATH, BLOCK_LINK, verbose=verbose)
 
 
 if __name__ == "__main__":
   print(build_library(verbose=True))
+  print(build_block_library(verbose=True))

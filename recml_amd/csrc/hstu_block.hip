@@ -1,0 +1,301 @@
+// The two fused steps of the HSTU block around the attention kernel, for gfx950
+// (MI355X): see include/hstu_block.h.
+//
+//   hstu_norm_gate   out = u * layer_norm(attn)   (recml/layers/keras/hstu.py:471-472)
+//                    one wavefront per token row, 16 bytes per lane and trip: the row is read once,
+//                    kept in registers for the two reductions (mean, then centred sum of squares) and
+//                    written once: 3 x width x 2 bytes of HBM traffic per row, which is the bound.
+//   gemm + silu      out = silu(x W + bias)       (hstu.py:444-449)
+//                    hipBLASLt matrix product with the activation in its epilogue.
+
+#include <hip/hip_runtime.h>
+#include <hipblaslt/hipblaslt.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
+
+#include "hstu_block.h"
+
+namespace {
+
+typedef __bf16 bf16_t;
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+    f[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+  }
+}
+
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  floatx2 f = {lo, hi};
+  bf16x2 r = __builtin_convertvector(f, bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+  return v;
+}
+
+struct NormGateParams {
+  const bf16_t* a;
+  const bf16_t* u;
+  bf16_t* out;
+  const bf16_t* gamma;
+  const bf16_t* beta;
+  int64_t rows, a_stride, u_stride, out_stride;
+  int32_t width;
+  float eps;
+};
+
+// One wavefront per row; lane l owns the 8-element pieces l, l + 64, ... of the row (CH of them at most).
+template <int CH>
+__global__ __launch_bounds__(256) void hstu_norm_gate(const NormGateParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= p.rows) return;
+  const bf16_t* ar = p.a + row * p.a_stride;
+  const bf16_t* ur = p.u + row * p.u_stride;
+  bf16_t* orow = p.out + row * p.out_stride;
+  float x[CH][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = (c * 64 + lane) * 8;
+    if (e < p.width) {
+      unpack8(*(const uint4*)(ar + e), x[c]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sum += x[c][i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[c][i] = 0.f;
+    }
+  }
+  const float mean = wave_sum(sum) / (float)p.width;
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = (c * 64 + lane) * 8;
+    if (e < p.width) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float d = x[c][i] - mean;
+        ss += d * d;
+      }
+    }
+  }
+  const float rstd = __builtin_amdgcn_rsqf(wave_sum(ss) / (float)p.width + p.eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = (c * 64 + lane) * 8;
+    if (e < p.width) {
+      float g[8], b[8], uu[8];
+      unpack8(*(const uint4*)(p.gamma + e), g);
+      unpack8(*(const uint4*)(p.beta + e), b);
+      unpack8(*(const uint4*)(ur + e), uu);
+      float y[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = uu[i] * __builtin_fmaf((x[c][i] - mean) * rstd, g[i], b[i]);
+      uint4 o;
+      o.x = pack2(y[0], y[1]);
+      o.y = pack2(y[2], y[3]);
+      o.z = pack2(y[4], y[5]);
+      o.w = pack2(y[6], y[7]);
+      *(uint4*)(orow + e) = o;
+    }
+  }
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+
+// ---- hipBLASLt side -------------------------------------------------------
+
+constexpr size_t kBlasWorkspace = 32u << 20;
+
+struct GemmPlan {
+  hipblasLtMatmulDesc_t desc = nullptr;
+  hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
+  hipblasLtMatmulAlgo_t algo;
+  size_t workspace = 0;
+};
+
+struct BlasState {
+  std::mutex mu;
+  hipblasLtHandle_t handle[64] = {};
+  // (device, M, N, K, x_stride, bias?, activation, workspace offered) -> plan
+  std::map<std::tuple<int, int64_t, int, int, int64_t, int, int, size_t>, GemmPlan> plans;
+};
+
+BlasState& blas() {
+  static BlasState s;
+  return s;
+}
+
+const char* blas_str(hipblasStatus_t st) {
+  switch (st) {
+    case HIPBLAS_STATUS_SUCCESS: return "success";
+    case HIPBLAS_STATUS_NOT_INITIALIZED: return "not initialized";
+    case HIPBLAS_STATUS_ALLOC_FAILED: return "allocation failed";
+    case HIPBLAS_STATUS_INVALID_VALUE: return "invalid value";
+    case HIPBLAS_STATUS_NOT_SUPPORTED: return "not supported";
+    case HIPBLAS_STATUS_EXECUTION_FAILED: return "execution failed";
+    default: return "error";
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int hstu_block_abi_version(void) { return HSTU_BLOCK_ABI_VERSION; }
+
+const char* hstu_block_last_error(void) { return g_err; }
+
+int hstu_norm_gate_fwd(const HstuNormGateArgs* a, void* stream) {
+  if (!a) return fail(HSTU_BLOCK_ERR_NULL, "args is null");
+  if (a->struct_size != sizeof(HstuNormGateArgs) || a->version != HSTU_BLOCK_ABI_VERSION)
+    return fail(HSTU_BLOCK_ERR_VERSION, "norm-gate args struct_size/version (%u/%u) do not match this library (%zu/%d)",
+                a->struct_size, a->version, sizeof(HstuNormGateArgs), HSTU_BLOCK_ABI_VERSION);
+  if (a->rows < 0 || a->width < 8 || a->width > 8192 || (a->width & 7))
+    return fail(HSTU_BLOCK_ERR_SHAPE, "rows >= 0 and width a multiple of 8 in [8, 8192] expected, got rows=%lld width=%d",
+                (long long)a->rows, a->width);
+  g_err[0] = 0;
+  if (a->rows == 0) return HSTU_BLOCK_OK;
+  if (!a->a || !a->u || !a->out || !a->gamma || !a->beta) return fail(HSTU_BLOCK_ERR_NULL, "a, u, out, gamma and beta must be non-null");
+  if (!aligned16(a->a) || !aligned16(a->u) || !aligned16(a->out) || !aligned16(a->gamma) || !aligned16(a->beta) ||
+      (a->a_stride & 7) || (a->u_stride & 7) || (a->out_stride & 7) ||
+      a->a_stride < a->width || a->u_stride < a->width || a->out_stride < a->width)
+    return fail(HSTU_BLOCK_ERR_SHAPE, "pointers must be 16-byte aligned, row strides multiples of 8 elements and >= width");
+  if ((a->rows + 3) / 4 > 0x7fffffffLL) return fail(HSTU_BLOCK_ERR_SHAPE, "too many rows");
+  NormGateParams p;
+  p.a = (const bf16_t*)a->a; p.u = (const bf16_t*)a->u; p.out = (bf16_t*)a->out;
+  p.gamma = (const bf16_t*)a->gamma; p.beta = (const bf16_t*)a->beta;
+  p.rows = a->rows; p.a_stride = a->a_stride; p.u_stride = a->u_stride; p.out_stride = a->out_stride;
+  p.width = a->width; p.eps = a->eps;
+  const dim3 grid((unsigned)((a->rows + 3) / 4)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int ch = (a->width + 511) / 512;
+  if (ch <= 1) hipLaunchKernelGGL(hstu_norm_gate<1>, grid, block, 0, st, p);
+  else if (ch <= 2) hipLaunchKernelGGL(hstu_norm_gate<2>, grid, block, 0, st, p);
+  else if (ch <= 4) hipLaunchKernelGGL(hstu_norm_gate<4>, grid, block, 0, st, p);
+  else hipLaunchKernelGGL(hstu_norm_gate<16>, grid, block, 0, st, p);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "norm-gate kernel launch: %s", hipGetErrorString(e));
+  return HSTU_BLOCK_OK;
+}
+
+size_t hstu_gemm_silu_workspace_bytes(void) { return kBlasWorkspace; }
+
+int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
+  if (!a) return fail(HSTU_BLOCK_ERR_NULL, "args is null");
+  if (a->struct_size != sizeof(HstuGemmSiluArgs) || a->version != HSTU_BLOCK_ABI_VERSION)
+    return fail(HSTU_BLOCK_ERR_VERSION, "gemm args struct_size/version (%u/%u) do not match this library (%zu/%d)",
+                a->struct_size, a->version, sizeof(HstuGemmSiluArgs), HSTU_BLOCK_ABI_VERSION);
+  if (a->M < 0 || a->N < 1 || a->K < 1 || a->M > 0x7fffffffLL || a->x_stride < a->K)
+    return fail(HSTU_BLOCK_ERR_SHAPE, "bad shape M=%lld N=%d K=%d x_stride=%lld", (long long)a->M, a->N, a->K, (long long)a->x_stride);
+  if (a->activation != 0 && a->activation != 1) return fail(HSTU_BLOCK_ERR_SHAPE, "activation must be 0 (none) or 1 (silu)");
+  g_err[0] = 0;
+  if (a->M == 0) return HSTU_BLOCK_OK;
+  if (!a->x || !a->w || !a->out) return fail(HSTU_BLOCK_ERR_NULL, "x, w and out must be non-null");
+  if (a->workspace_bytes && !a->workspace) return fail(HSTU_BLOCK_ERR_WORKSPACE, "workspace_bytes without a workspace");
+  int dev = 0;
+  hipError_t he = hipGetDevice(&dev);
+  if (he != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(he));
+  if (dev < 0 || dev >= 64) return fail(HSTU_BLOCK_ERR_LAUNCH, "device index %d out of range", dev);
+
+  BlasState& bs = blas();
+  GemmPlan plan;
+  hipblasLtHandle_t handle;
+  {
+    std::lock_guard<std::mutex> lock(bs.mu);
+    if (!bs.handle[dev]) {
+      const hipblasStatus_t st = hipblasLtCreate(&bs.handle[dev]);
+      if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtCreate: %s", blas_str(st));
+    }
+    handle = bs.handle[dev];
+    const auto key = std::make_tuple(dev, a->M, a->N, a->K, a->x_stride, a->bias ? 1 : 0, a->activation, a->workspace_bytes);
+    auto it = bs.plans.find(key);
+    if (it == bs.plans.end()) {
+      // row-major out[M, N] = x[M, K] w[K, N] is, in the column-major terms of the library,
+      // out^T [N x M] = w^T [N x K] x^T [K x M] with leading dimensions N, x_stride and N
+      GemmPlan np;
+      hipblasStatus_t st = hipblasLtMatmulDescCreate(&np.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F);
+      if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulDescCreate: %s", blas_str(st));
+      const hipblasOperation_t op_n = HIPBLAS_OP_N;
+      hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_n, sizeof(op_n));
+      hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n));
+      hipblasLtEpilogue_t epi = HIPBLASLT_EPILOGUE_DEFAULT;
+      if (a->activation == 1) epi = a->bias ? HIPBLASLT_EPILOGUE_SWISH_BIAS_EXT : HIPBLASLT_EPILOGUE_SWISH_EXT;
+      else if (a->bias) epi = HIPBLASLT_EPILOGUE_BIAS;
+      hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi));
+      if (a->bias) {
+        const hipDataType bt = HIP_R_16BF;
+        hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt));
+      }
+      st = hipblasLtMatrixLayoutCreate(&np.la, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->K, (int64_t)a->N);
+      if (st == HIPBLAS_STATUS_SUCCESS) st = hipblasLtMatrixLayoutCreate(&np.lb, HIP_R_16BF, (uint64_t)a->K, (uint64_t)a->M, a->x_stride);
+      if (st == HIPBLAS_STATUS_SUCCESS) st = hipblasLtMatrixLayoutCreate(&np.lc, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->M, (int64_t)a->N);
+      if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatrixLayoutCreate: %s", blas_str(st));
+      hipblasLtMatmulPreference_t pref;
+      st = hipblasLtMatmulPreferenceCreate(&pref);
+      if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulPreferenceCreate: %s", blas_str(st));
+      const uint64_t ws = a->workspace_bytes;
+      hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
+      if (a->bias) {
+        // the heuristic looks at the pointer's presence; the real one is set on every call below
+        hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
+      }
+      hipblasLtMatmulHeuristicResult_t res[1];
+      int found = 0;
+      st = hipblasLtMatmulAlgoGetHeuristic(handle, np.desc, np.la, np.lb, np.lc, np.lc, pref, 1, res, &found);
+      hipblasLtMatmulPreferenceDestroy(pref);
+      if (st != HIPBLAS_STATUS_SUCCESS || found < 1)
+        return fail(HSTU_BLOCK_ERR_BLAS, "hipBLASLt has no kernel for M=%lld N=%d K=%d with this epilogue (%s)",
+                    (long long)a->M, a->N, a->K, blas_str(st));
+      np.algo = res[0].algo;
+      np.workspace = res[0].workspaceSize;
+      if (bs.plans.size() >= 256) {
+        for (auto& kv : bs.plans) {
+          hipblasLtMatrixLayoutDestroy(kv.second.la);
+          hipblasLtMatrixLayoutDestroy(kv.second.lb);
+          hipblasLtMatrixLayoutDestroy(kv.second.lc);
+          hipblasLtMatmulDescDestroy(kv.second.desc);
+        }
+        bs.plans.clear();
+      }
+      it = bs.plans.emplace(key, np).first;
+    }
+    plan = it->second;
+    // the descriptor is shared by every call of this shape: the bias pointer is set under the lock
+    // and the product is enqueued before it is released
+    if (a->bias) hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
+    const float alpha = 1.0f, beta = 0.0f;
+    const hipblasStatus_t st = hipblasLtMatmul(handle, plan.desc, &alpha, a->w, plan.la, a->x, plan.lb, &beta, a->out, plan.lc,
+                                               a->out, plan.lc, &plan.algo, a->workspace, a->workspace_bytes, (hipStream_t)stream);
+    if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmul: %s", blas_str(st));
+  }
+  return HSTU_BLOCK_OK;
+}
+
+}  // extern "C"

@@ -1,9 +1,11 @@
 """HSTU block and model forward around the MI355X attention kernel.
 
-The harness for the end-to-end (config-4) shape: everything except the
-attention is plain torch on the GPU (embedding gather, layer norms, the
-projections as rocBLAS / hipBLASLt GEMMs); the attention is
-`recml_amd.hstu_attention`, i.e. the HIP kernel behind the C ABI.  No dropout.
+The harness for the end-to-end (config-4) shape: the attention is
+`recml_amd.hstu_attention`, i.e. the HIP kernel behind the C ABI; in bf16
+inference the projections' activation and the attention norm + U gate are the
+fused steps of `recml_amd.hstu_block_ops`; the rest is plain torch on the GPU
+(embedding gather, input layer norm, the output product with the residual as
+its C operand).  No dropout.
 Parameters are created frozen; after `requires_grad_(True)` the attention goes
 through `recml_amd.hstu_attention_autograd` (the HIP backward kernels) and the
 rest through torch autograd.
@@ -28,6 +30,7 @@ import math
 import torch
 import torch.nn.functional as F
 
+from recml_amd import hstu_block_ops
 from recml_amd import hstu_ops
 from recml_amd import masks
 
@@ -107,12 +110,16 @@ class HSTUBlock(torch.nn.Module):
     """
     B, L, D = inputs.shape
     H, hd = self.num_heads, self.head_dim
+    fused = self._fused_inference(inputs)
     x = F.layer_norm(inputs, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
-    w = torch.cat([self.u_kernel, self.q_kernel, self.k_kernel, self.v_kernel], dim=1).reshape(D, 4 * H * hd)
-    uqkv = x.reshape(B * L, D) @ w
-    if self.use_bias:
-      uqkv = uqkv + torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1)
-    uqkv = F.silu(uqkv).reshape(B, L, 4, H, hd)
+    w, b = self._uqkv_weights()
+    if fused:
+      uqkv = hstu_block_ops.gemm_silu(x.reshape(B * L, D), w, b, True).reshape(B, L, 4, H, hd)
+    else:
+      uqkv = x.reshape(B * L, D) @ w
+      if b is not None:
+        uqkv = uqkv + b
+      uqkv = F.silu(uqkv).reshape(B, L, 4, H, hd)
     u, q, k, v = uqkv.unbind(dim=2)
     if attention_mask is not None:
       attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
@@ -121,6 +128,12 @@ class HSTUBlock(torch.nn.Module):
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
                         timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias)
+    if fused:
+      gated = hstu_block_ops.norm_gate(attn.reshape(B * L, H * hd), u.reshape(B * L, H * hd), self.attn_ln_gamma.reshape(-1),
+                                       self.attn_ln_beta.reshape(-1), self.eps)
+      res = inputs.reshape(B * L, D)
+      res = res if self.output_bias is None else res + self.output_bias
+      return torch.addmm(res, gated, self.output_kernel.reshape(H * hd, D)).reshape(B, L, D)
     normed = F.layer_norm(attn.reshape(B, L, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
                           self.attn_ln_beta.reshape(-1), self.eps)
     gated = u.reshape(B, L, H * hd) * normed
@@ -130,21 +143,44 @@ class HSTUBlock(torch.nn.Module):
     return out.reshape(B, L, D) + inputs
 
 
+  def _fused_inference(self, t) -> bool:
+    """Whether the fused block steps apply: bf16 on a GPU, nothing asking for gradients."""
+    wants_grad = torch.is_grad_enabled() and (t.requires_grad or any(p.requires_grad for p in self.parameters()))
+    return t.is_cuda and t.dtype == torch.bfloat16 and not wants_grad
+
+  def _uqkv_weights(self):
+    w = torch.cat([self.u_kernel, self.q_kernel, self.k_kernel, self.v_kernel], dim=1).reshape(self.hidden_dim, -1)
+    b = torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1) if self.use_bias else None
+    return w, b
+
   def forward_jagged(self, tokens, seq_offsets, max_len, *, pos_bias=None, timestamps=None, ts_bias=None):
     """The block on packed tokens [T, D] (sequence b = rows seq_offsets[b]..seq_offsets[b+1]):
-    no work at all for padding, in the projections either.  `timestamps` is jagged [T]."""
+    no work at all for padding, in the projections either.  `timestamps` is jagged [T].
+
+    Inference in bf16 takes the fused steps: the projections' SiLU in the epilogue of their one
+    matrix product, the attention norm and the U gate in one pass (recml_amd.hstu_block_ops), the
+    residual as the C operand of the output product."""
     T, D = tokens.shape
     H, hd = self.num_heads, self.head_dim
+    fused = self._fused_inference(tokens)
     x = F.layer_norm(tokens, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
-    w = torch.cat([self.u_kernel, self.q_kernel, self.k_kernel, self.v_kernel], dim=1).reshape(D, 4 * H * hd)
-    uqkv = x @ w
-    if self.use_bias:
-      uqkv = uqkv + torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1)
-    uqkv = F.silu(uqkv).reshape(T, 4, H, hd)
+    w, b = self._uqkv_weights()
+    if fused:
+      uqkv = hstu_block_ops.gemm_silu(x, w, b, True).reshape(T, 4, H, hd)
+    else:
+      uqkv = x @ w
+      if b is not None:
+        uqkv = uqkv + b
+      uqkv = F.silu(uqkv).reshape(T, 4, H, hd)
     u, q, k, v = uqkv.unbind(dim=1)
     alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
     attn = _attention(q, k, v, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
                       pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
+    if fused:
+      gated = hstu_block_ops.norm_gate(attn.reshape(T, H * hd), u.reshape(T, H * hd), self.attn_ln_gamma.reshape(-1),
+                                       self.attn_ln_beta.reshape(-1), self.eps)
+      res = tokens if self.output_bias is None else tokens + self.output_bias
+      return torch.addmm(res, gated, self.output_kernel.reshape(H * hd, D))
     normed = F.layer_norm(attn.reshape(T, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
                           self.attn_ln_beta.reshape(-1), self.eps)
     out = (u.reshape(T, H * hd) * normed) @ self.output_kernel.reshape(H * hd, D)

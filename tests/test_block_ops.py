@@ -1,0 +1,136 @@
+"""The fused block steps (libhstu_block.so): ABI checks on the CPU, parity on the GPU."""
+
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+import torch
+
+from recml_amd import _lib_block
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "hstu_block.h")
+
+
+def test_library_exports_every_declared_symbol():
+  lib = _lib_block.load()
+  text = open(HEADER).read()
+  text = text[text.index("#ifdef __cplusplus"):]          # skip the prose at the top
+  names = sorted(set(re.findall(r"\b(hstu_\w+)\s*\(", text)))
+  assert set(names) == set(_lib_block.EXPORTS)
+  for n in names:
+    assert getattr(lib, n) is not None
+  assert lib.hstu_block_abi_version() == _lib_block.ABI_VERSION
+
+
+@pytest.mark.parametrize("name", ["HstuNormGateArgs", "HstuGemmSiluArgs"])
+def test_struct_layout_matches_header(name):
+  struct = getattr(_lib_block, name)
+  fields = [f[0] for f in struct._fields_]
+  prog = ['#include <stdio.h>', '#include <stddef.h>', '#include "hstu_block.h"', "int main(void) {",
+          f'  printf("%zu\\n", sizeof({name}));']
+  prog += [f'  printf("%zu\\n", offsetof({name}, {f}));' for f in fields]
+  prog += ["  return 0;", "}"]
+  with tempfile.TemporaryDirectory() as d:
+    src, exe = os.path.join(d, "layout.c"), os.path.join(d, "layout")
+    open(src, "w").write("\n".join(prog))
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), "-o", exe, src], check=True)
+    out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
+  assert int(out[0]) == C.sizeof(struct)
+  for f, off in zip(fields, out[1:]):
+    assert getattr(struct, f).offset == int(off), f
+
+
+def test_validation_errors_without_gpu():
+  lib = _lib_block.load()
+  assert lib.hstu_norm_gate_fwd(None, None) == -1
+  a = _lib_block.HstuNormGateArgs()
+  assert lib.hstu_norm_gate_fwd(C.byref(a), None) == -2
+  a.struct_size, a.version = C.sizeof(a), _lib_block.ABI_VERSION
+  a.rows, a.width = 4, 12
+  assert lib.hstu_norm_gate_fwd(C.byref(a), None) == -4          # width not a multiple of 8
+  a.width = 64
+  assert lib.hstu_norm_gate_fwd(C.byref(a), None) == -1          # null tensors
+  a.a = a.u = a.out = a.gamma = a.beta = 0x1000
+  a.a_stride, a.u_stride, a.out_stride = 64, 60, 64
+  assert lib.hstu_norm_gate_fwd(C.byref(a), None) == -4          # row stride below the width
+  assert b"stride" in lib.hstu_block_last_error()
+  a.rows = 0
+  assert lib.hstu_norm_gate_fwd(C.byref(a), None) == 0           # nothing to do
+  g = _lib_block.HstuGemmSiluArgs()
+  assert lib.hstu_gemm_silu_fwd(C.byref(g), None) == -2
+  g.struct_size, g.version = C.sizeof(g), _lib_block.ABI_VERSION
+  g.M, g.N, g.K, g.x_stride = 8, 16, 32, 16
+  assert lib.hstu_gemm_silu_fwd(C.byref(g), None) == -4          # row stride below K
+  g.x_stride, g.activation = 32, 7
+  assert lib.hstu_gemm_silu_fwd(C.byref(g), None) == -4
+  g.activation = 1
+  assert lib.hstu_gemm_silu_fwd(C.byref(g), None) == -1          # null tensors
+  assert lib.hstu_gemm_silu_workspace_bytes() > 0
+
+
+def _rel(a, b):
+  return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,width", [(1, 8), (37, 64), (513, 512), (64, 1000), (9, 4096), (3, 8192)])
+def test_norm_gate_parity(gpu, rows, width):
+  """Against fp64 arithmetic on the same bf16 inputs: the fused step rounds once, at the end."""
+  from recml_amd import hstu_block_ops as B
+  gen = torch.Generator().manual_seed(rows * 7 + width)
+  dev, bf = "cuda:0", torch.bfloat16
+  fused = (torch.randn((rows, 4, width), generator=gen) * 0.7).to(dev).to(bf)
+  u = fused[:, 1]                                              # a strided slice, as in the block
+  attn = (torch.randn((rows, width), generator=gen) * 3e-3 + 1e-3).to(dev).to(bf)
+  gamma = (1 + 0.2 * torch.randn(width, generator=gen)).to(dev).to(bf)
+  beta = (0.1 * torch.randn(width, generator=gen)).to(dev).to(bf)
+  out = B.norm_gate(attn, u, gamma, beta, 1e-6)
+  a64 = attn.double()
+  mean = a64.mean(-1, keepdim=True)
+  var = ((a64 - mean) ** 2).mean(-1, keepdim=True)
+  ref = u.double() * ((a64 - mean) / torch.sqrt(var + 1e-6) * gamma.double() + beta.double())
+  assert out.shape == attn.shape and out.dtype == bf
+  assert _rel(out.double(), ref) <= 8e-3                       # bf16 rounding of the result: 2^-8
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,N,bias,act", [(1, 64, 64, False, True), (300, 512, 2048, True, True),
+                                            (4097, 512, 2048, False, True), (129, 256, 1024, True, False)])
+def test_gemm_silu_parity(gpu, M, K, N, bias, act):
+  from recml_amd import hstu_block_ops as B
+  gen = torch.Generator().manual_seed(M + N)
+  dev, bf = "cuda:0", torch.bfloat16
+  x = (torch.randn((M, K), generator=gen) * 0.5).to(dev).to(bf)
+  w = (torch.randn((K, N), generator=gen) * 0.05).to(dev).to(bf)
+  b = (torch.randn(N, generator=gen) * 0.1).to(dev).to(bf) if bias else None
+  out = B.gemm_silu(x, w, b, act)
+  ref = x.double() @ w.double()
+  if bias:
+    ref = ref + b.double()
+  if act:
+    ref = ref * torch.sigmoid(ref)
+  assert out.shape == (M, N) and out.dtype == bf
+  assert _rel(out.double(), ref) <= 8e-3
+  # a strided x (row stride 2K) gives the same values
+  wide = torch.zeros((M, 2 * K), device=dev, dtype=bf)
+  wide[:, :K] = x
+  assert torch.equal(B.gemm_silu(wide[:, :K], w, b, act), out)
+
+
+@pytest.mark.gpu
+def test_block_ops_argument_errors(gpu):
+  from recml_amd import hstu_block_ops as B
+  z = torch.zeros((4, 64), device="cuda:0", dtype=torch.bfloat16)
+  with pytest.raises(ValueError, match="bfloat16"):
+    B.norm_gate(z.float(), z, z[0], z[0])
+  with pytest.raises(ValueError, match="differ in shape"):
+    B.norm_gate(z, z[:2], z[0], z[0])
+  with pytest.raises(ValueError, match="x \\[M, K\\]"):
+    B.gemm_silu(z, z)
+  with pytest.raises(ValueError, match="GPU tensor"):
+    B.gemm_silu(z.cpu(), z.cpu().t())

@@ -261,6 +261,17 @@ def bench_block_steps(args, dev):
   wall_t, _ = timed(lambda: u * torch.nn.functional.layer_norm(attn, (D,), gamma, beta, 1e-6))
   wall_g, ker_g = timed(lambda: recml_amd.gemm_silu(x, w, None, True))
   wall_gt, _ = timed(lambda: torch.nn.functional.silu(x @ w))
+  # the front end: 10 M x 512 table, Zipf(1.05) ids as in the model workload, position table of 1024 rows
+  vocab = 10_000_000
+  table = torch.empty((vocab, D), dtype=bf, device=dev)
+  table.normal_(0.0, 0.01, generator=gen)
+  rng = np.random.Generator(np.random.PCG64(4))
+  ids = torch.from_numpy(np.minimum(rng.zipf(1.05, T), vocab - 1).astype(np.int64)).to(dev)
+  pos_table = (torch.randn((1024, D), device=dev, generator=gen) * 0.01).to(bf)
+  positions = torch.from_numpy(rng.integers(0, 1024, T).astype(np.int64)).to(dev)
+  wall_e, ker_e = timed(lambda: recml_amd.embed_norm(ids, table, gamma, beta, 1e-6, positions=positions, pos_table=pos_table))
+  wall_et, _ = timed(lambda: torch.nn.functional.layer_norm(table[ids] + pos_table[positions], (D,), gamma, beta, 1e-6))
+  uniq = int(torch.unique(ids).numel())
   nbytes = 3 * T * D * 2
   gflop = 2.0 * T * D * 4 * D / 1e9
   out = ng().float().cpu().numpy()
@@ -273,6 +284,8 @@ def bench_block_steps(args, dev):
                    "frac": nbytes / (ker_ng * 1e-3) / 1e9 / 8000.0, "traffic": None, "kernel_ms_avg": ker_ng,
                    "algorithmic_bytes": nbytes},
       "torch_layer_norm_then_mul_ms": wall_t,
+      "embed_norm": {"ms_per_call": wall_e, "event_ms": ker_e, "torch_gather_add_layer_norm_ms": wall_et,
+                     "unique_ids": uniq, "gb_per_s_rows_read_and_written": 2 * T * D * 2 / (ker_e * 1e-3) / 1e9},
       "gemm_silu": {"ms_per_call": wall_g, "event_ms": ker_g, "tflops": gflop / ker_g, "torch_mm_then_silu_ms": wall_gt,
                     "shape": [T, D, 4 * D]},
   }

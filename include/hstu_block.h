@@ -1,6 +1,6 @@
-/* C ABI of libhstu_block.so: the two fused steps of the HSTU block that sit on
- * either side of the attention kernel (recml/layers/keras/hstu.py:444-474),
- * for gfx950.  bf16 tensors, row-major, on the current device; fp32 arithmetic
+/* C ABI of libhstu_block.so: the fused steps of the HSTU block that sit on
+ * either side of the attention kernel (recml/layers/keras/hstu.py:444-474) and
+ * of the model's front end (hstu.py:593-601), for gfx950.  bf16 tensors, row-major, on the current device; fp32 arithmetic
  * inside.  Plain pointers and sizes: no framework types.
  *
  *   hstu_gemm_silu_fwd    out = silu(x W + bias): the U, Q, K, V projections of
@@ -12,6 +12,10 @@
  *   hstu_norm_gate_fwd    out = u * layer_norm(attn): the layer norm over
  *                         (heads, head_dim) of the attention output and the U
  *                         gate (hstu.py:471-472) in one pass over memory.
+ *   hstu_embed_norm_fwd   out = layer_norm(scale * table[ids] + pos_table[positions]):
+ *                         the model's front end (hstu.py:593-601: item
+ *                         embedding, optional sqrt(D) scale, position
+ *                         embedding, final_norm) as one gather pass.
  *
  * Every function returns 0 or a negative HstuBlockStatus; the message of the
  * last failure on the calling thread is at hstu_block_last_error().
@@ -85,6 +89,35 @@ typedef struct HstuGemmSiluArgs {
 
 size_t hstu_gemm_silu_workspace_bytes(void);
 int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* args, void* stream);
+
+/* out[t, :] = gamma * (x_t - mean) * rstd + beta with x_t = scale * table[ids[t], :]
+ * (+ pos_table[positions[t], :] when pos_table is given), statistics over the
+ * `width` entries of x_t as in hstu_norm_gate_fwd.  table: bf16 [vocab, width]
+ * (row stride table_stride), pos_table: bf16 [n_positions, width] contiguous or
+ * null, ids / positions: int64 [rows] (positions null with pos_table null),
+ * out: bf16 [rows, width] contiguous.  Indices outside their table are clamped
+ * into it (the reference's gather on an accelerator does the same).  width a
+ * multiple of 8 up to 8192; pointers and table_stride multiples of 8 elements. */
+typedef struct HstuEmbedNormArgs {
+  uint32_t struct_size;   /* sizeof(HstuEmbedNormArgs) */
+  uint32_t version;       /* HSTU_BLOCK_ABI_VERSION    */
+  int64_t rows;
+  int32_t width;
+  float eps;
+  float scale;            /* 1, or sqrt(model_dim) (scale_by_sqrt_dim) */
+  int32_t reserved0;
+  const int64_t* ids;
+  const void* table;
+  int64_t vocab, table_stride;
+  const int64_t* positions;
+  const void* pos_table;
+  int64_t n_positions;
+  const void* gamma;
+  const void* beta;
+  void* out;
+} HstuEmbedNormArgs;
+
+int hstu_embed_norm_fwd(const HstuEmbedNormArgs* args, void* stream);
 
 int hstu_block_abi_version(void);
 const char* hstu_block_last_error(void);

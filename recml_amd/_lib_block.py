@@ -17,6 +17,7 @@ EXPORTS = (
     "hstu_norm_gate_fwd",
     "hstu_gemm_silu_fwd",
     "hstu_gemm_silu_workspace_bytes",
+    "hstu_embed_norm_fwd",
 )
 
 
@@ -42,6 +43,20 @@ class HstuGemmSiluArgs(C.Structure):
       ("x", C.c_void_p), ("x_stride", C.c_int64),
       ("w", C.c_void_p), ("bias", C.c_void_p), ("out", C.c_void_p),
       ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+  ]
+
+
+class HstuEmbedNormArgs(C.Structure):
+  """Field-for-field image of `struct HstuEmbedNormArgs`."""
+
+  _fields_ = [
+      ("struct_size", C.c_uint32), ("version", C.c_uint32),
+      ("rows", C.c_int64), ("width", C.c_int32), ("eps", C.c_float),
+      ("scale", C.c_float), ("reserved0", C.c_int32),
+      ("ids", C.c_void_p), ("table", C.c_void_p),
+      ("vocab", C.c_int64), ("table_stride", C.c_int64),
+      ("positions", C.c_void_p), ("pos_table", C.c_void_p), ("n_positions", C.c_int64),
+      ("gamma", C.c_void_p), ("beta", C.c_void_p), ("out", C.c_void_p),
   ]
 
 
@@ -71,6 +86,8 @@ def load():
     lib.hstu_gemm_silu_fwd.argtypes = [C.POINTER(HstuGemmSiluArgs), C.c_void_p]
     lib.hstu_gemm_silu_workspace_bytes.restype = C.c_size_t
     lib.hstu_gemm_silu_workspace_bytes.argtypes = []
+    lib.hstu_embed_norm_fwd.restype = C.c_int
+    lib.hstu_embed_norm_fwd.argtypes = [C.POINTER(HstuEmbedNormArgs), C.c_void_p]
     ver = lib.hstu_block_abi_version()
     if ver != ABI_VERSION:
       raise RuntimeError(f"libhstu_block.so has ABI {ver}, expected {ABI_VERSION}")

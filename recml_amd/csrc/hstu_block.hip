@@ -1,5 +1,5 @@
-// The two fused steps of the HSTU block around the attention kernel, for gfx950
-// (MI355X): see include/hstu_block.h.
+// Fused steps of the HSTU block around the attention kernel and of the model's front end, for
+// gfx950 (MI355X): see include/hstu_block.h.
 //
 //   hstu_norm_gate   out = u * layer_norm(attn)   (recml/layers/keras/hstu.py:471-472)
 //                    one wavefront per token row, 16 bytes per lane and trip: the row is read once,
@@ -7,6 +7,9 @@
 //                    written once: 3 x width x 2 bytes of HBM traffic per row, which is the bound.
 //   gemm + silu      out = silu(x W + bias)       (hstu.py:444-449)
 //                    hipBLASLt matrix product with the activation in its epilogue.
+//   hstu_embed_norm  out = layer_norm(scale * table[ids] + pos_table[positions])   (hstu.py:593-601)
+//                    the same one-wave-per-row scheme with a gathered row: one read of the table row
+//                    (and of the small position table, which stays in cache), one write.
 
 #include <hip/hip_runtime.h>
 #include <hipblaslt/hipblaslt.h>
@@ -127,6 +130,92 @@ __global__ __launch_bounds__(256) void hstu_norm_gate(const NormGateParams p) {
   }
 }
 
+struct EmbedNormParams {
+  const int64_t* ids;
+  const int64_t* positions;
+  const bf16_t* table;
+  const bf16_t* pos_table;
+  const bf16_t* gamma;
+  const bf16_t* beta;
+  bf16_t* out;
+  int64_t rows, vocab, table_stride, n_positions;
+  int32_t width;
+  float eps, scale;
+};
+
+// One wavefront per token: its table row (and position row) is gathered into registers, normalised
+// there and written once.
+template <int CH>
+__global__ __launch_bounds__(256) void hstu_embed_norm(const EmbedNormParams p) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= p.rows) return;
+  int64_t id = p.ids[row];
+  id = id < 0 ? 0 : (id >= p.vocab ? p.vocab - 1 : id);
+  const bf16_t* er = p.table + id * p.table_stride;
+  const bf16_t* pr = nullptr;
+  if (p.pos_table) {
+    int64_t ps = p.positions[row];
+    ps = ps < 0 ? 0 : (ps >= p.n_positions ? p.n_positions - 1 : ps);
+    pr = p.pos_table + ps * (int64_t)p.width;
+  }
+  float x[CH][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = (c * 64 + lane) * 8;
+    if (e < p.width) {
+      unpack8(*(const uint4*)(er + e), x[c]);
+      if (pr) {
+        float pe[8];
+        unpack8(*(const uint4*)(pr + e), pe);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[c][i] = __builtin_fmaf(x[c][i], p.scale, pe[i]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[c][i] *= p.scale;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sum += x[c][i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[c][i] = 0.f;
+    }
+  }
+  const float mean = wave_sum(sum) / (float)p.width;
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = (c * 64 + lane) * 8;
+    if (e < p.width) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float d = x[c][i] - mean;
+        ss += d * d;
+      }
+    }
+  }
+  const float rstd = __builtin_amdgcn_rsqf(wave_sum(ss) / (float)p.width + p.eps);
+  bf16_t* orow = p.out + row * (int64_t)p.width;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int e = (c * 64 + lane) * 8;
+    if (e < p.width) {
+      float g[8], b[8], y[8];
+      unpack8(*(const uint4*)(p.gamma + e), g);
+      unpack8(*(const uint4*)(p.beta + e), b);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = __builtin_fmaf((x[c][i] - mean) * rstd, g[i], b[i]);
+      uint4 o;
+      o.x = pack2(y[0], y[1]);
+      o.y = pack2(y[2], y[3]);
+      o.z = pack2(y[4], y[5]);
+      o.w = pack2(y[6], y[7]);
+      *(uint4*)(orow + e) = o;
+    }
+  }
+}
+
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // ---- hipBLASLt side -------------------------------------------------------
@@ -202,6 +291,41 @@ int hstu_norm_gate_fwd(const HstuNormGateArgs* a, void* stream) {
   else hipLaunchKernelGGL(hstu_norm_gate<16>, grid, block, 0, st, p);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "norm-gate kernel launch: %s", hipGetErrorString(e));
+  return HSTU_BLOCK_OK;
+}
+
+int hstu_embed_norm_fwd(const HstuEmbedNormArgs* a, void* stream) {
+  if (!a) return fail(HSTU_BLOCK_ERR_NULL, "args is null");
+  if (a->struct_size != sizeof(HstuEmbedNormArgs) || a->version != HSTU_BLOCK_ABI_VERSION)
+    return fail(HSTU_BLOCK_ERR_VERSION, "embed-norm args struct_size/version (%u/%u) do not match this library (%zu/%d)",
+                a->struct_size, a->version, sizeof(HstuEmbedNormArgs), HSTU_BLOCK_ABI_VERSION);
+  if (a->rows < 0 || a->width < 8 || a->width > 8192 || (a->width & 7) || a->vocab < 1)
+    return fail(HSTU_BLOCK_ERR_SHAPE, "rows >= 0, vocab >= 1 and width a multiple of 8 in [8, 8192] expected, got rows=%lld vocab=%lld width=%d",
+                (long long)a->rows, (long long)a->vocab, a->width);
+  g_err[0] = 0;
+  if (a->rows == 0) return HSTU_BLOCK_OK;
+  if (!a->ids || !a->table || !a->out || !a->gamma || !a->beta) return fail(HSTU_BLOCK_ERR_NULL, "ids, table, out, gamma and beta must be non-null");
+  if ((a->pos_table != nullptr) != (a->positions != nullptr) || (a->pos_table && a->n_positions < 1))
+    return fail(HSTU_BLOCK_ERR_NULL, "pos_table and positions go together (with n_positions >= 1)");
+  if (!aligned16(a->table) || !aligned16(a->pos_table) || !aligned16(a->out) || !aligned16(a->gamma) || !aligned16(a->beta) ||
+      (a->table_stride & 7) || a->table_stride < a->width)
+    return fail(HSTU_BLOCK_ERR_SHAPE, "pointers must be 16-byte aligned, table_stride a multiple of 8 elements and >= width");
+  if ((a->rows + 3) / 4 > 0x7fffffffLL) return fail(HSTU_BLOCK_ERR_SHAPE, "too many rows");
+  EmbedNormParams p;
+  p.ids = a->ids; p.positions = a->positions;
+  p.table = (const bf16_t*)a->table; p.pos_table = (const bf16_t*)a->pos_table;
+  p.gamma = (const bf16_t*)a->gamma; p.beta = (const bf16_t*)a->beta; p.out = (bf16_t*)a->out;
+  p.rows = a->rows; p.vocab = a->vocab; p.table_stride = a->table_stride; p.n_positions = a->n_positions;
+  p.width = a->width; p.eps = a->eps; p.scale = a->scale;
+  const dim3 grid((unsigned)((a->rows + 3) / 4)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int ch = (a->width + 511) / 512;
+  if (ch <= 1) hipLaunchKernelGGL(hstu_embed_norm<1>, grid, block, 0, st, p);
+  else if (ch <= 2) hipLaunchKernelGGL(hstu_embed_norm<2>, grid, block, 0, st, p);
+  else if (ch <= 4) hipLaunchKernelGGL(hstu_embed_norm<4>, grid, block, 0, st, p);
+  else hipLaunchKernelGGL(hstu_embed_norm<16>, grid, block, 0, st, p);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "embed-norm kernel launch: %s", hipGetErrorString(e));
   return HSTU_BLOCK_OK;
 }
 

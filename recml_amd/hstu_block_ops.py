@@ -2,6 +2,7 @@
 
   norm_gate(attn, u, gamma, beta, eps)     u * layer_norm(attn)       recml/layers/keras/hstu.py:471-472
   gemm_silu(x, w, bias, activation)        silu(x @ w + bias)          recml/layers/keras/hstu.py:444-449
+  embed_norm(ids, table, ...)              layer_norm(scale * table[ids] + pos_table[positions])   hstu.py:593-601
 
 bf16 on a GPU only; there is no other implementation behind these names.
 """
@@ -107,3 +108,43 @@ def gemm_silu(x, w, bias=None, activation: bool = True):
   if rc != 0:
     _raise(lib, rc, "hstu_gemm_silu_fwd")
   return out
+
+
+def embed_norm(ids, table, gamma, beta, eps: float = 1e-6, *, scale: float = 1.0, positions=None, pos_table=None):
+  """layer_norm(scale * table[ids] + pos_table[positions]) over the last axis: ids [...] int64 -> [..., W] bf16.
+  table [V, W] bf16 (row stride free), pos_table [P, W] bf16 with positions shaped like ids, or neither."""
+  _check("table", table)
+  _check("gamma", gamma)
+  _check("beta", beta)
+  _check("ids", ids, torch.int64)
+  if table.dim() != 2 or table.stride(1) != 1:
+    raise ValueError("table must be [V, W] with a contiguous last axis")
+  if (positions is None) != (pos_table is None):
+    raise ValueError("positions and pos_table go together")
+  V, W = table.shape
+  flat = ids.reshape(-1).contiguous()
+  out = torch.empty((flat.numel(), W), dtype=table.dtype, device=table.device)
+  a = _lib_block.HstuEmbedNormArgs()
+  a.struct_size, a.version = C.sizeof(_lib_block.HstuEmbedNormArgs), _lib_block.ABI_VERSION
+  a.rows, a.width, a.eps, a.scale = flat.numel(), W, float(eps), float(scale)
+  a.ids, a.table, a.vocab, a.table_stride = flat.data_ptr(), table.data_ptr(), V, table.stride(0)
+  keep = [flat]
+  if pos_table is not None:
+    _check("pos_table", pos_table)
+    _check("positions", positions, torch.int64)
+    if positions.shape != ids.shape or pos_table.dim() != 2 or pos_table.shape[1] != W:
+      raise ValueError("positions must be shaped like ids and pos_table [P, W]")
+    pt, pf = pos_table.contiguous(), positions.reshape(-1).contiguous()
+    keep += [pt, pf]
+    a.positions, a.pos_table, a.n_positions = pf.data_ptr(), pt.data_ptr(), pt.shape[0]
+  g, b = gamma.reshape(-1).contiguous(), beta.reshape(-1).contiguous()
+  if g.numel() != W or b.numel() != W:
+    raise ValueError(f"gamma and beta must have {W} entries")
+  a.gamma, a.beta, a.out = g.data_ptr(), b.data_ptr(), out.data_ptr()
+  lib = _lib_block.load()
+  with torch.cuda.device(table.device):
+    rc = lib.hstu_embed_norm_fwd(C.byref(a), C.c_void_p(torch.cuda.current_stream(table.device).cuda_stream))
+  if rc != 0:
+    _raise(lib, rc, "hstu_embed_norm_fwd")
+  del keep
+  return out.reshape(*ids.shape, W)

@@ -220,6 +220,20 @@ class HSTU(torch.nn.Module):
   def _final_norm(self, x):
     return F.layer_norm(x, (self.model_dim,), self.final_norm_gamma, self.final_norm_beta, self.eps)
 
+  def _fused_front_end(self) -> bool:
+    """bf16 inference on a GPU: gather, scale, position embedding and final_norm as one pass."""
+    t = self.item_embedding
+    wants_grad = torch.is_grad_enabled() and any(
+        p is not None and p.requires_grad
+        for p in (self.item_embedding, self.position_embedding, self.final_norm_gamma, self.final_norm_beta))
+    return t.is_cuda and t.dtype == torch.bfloat16 and not wants_grad
+
+  def _embed_norm(self, ids, positions):
+    scale = self.model_dim ** 0.5 if self.scale_by_sqrt_dim else 1.0
+    return hstu_block_ops.embed_norm(ids.to(torch.int64), self.item_embedding, self.final_norm_gamma, self.final_norm_beta,
+                                     self.eps, scale=scale, positions=None if positions is None else positions.to(torch.int64),
+                                     pos_table=self.position_embedding)
+
   def forward(self, inputs, padding_mask=None, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None,
               jagged=False):
     """inputs: item ids [B, L]; `padding_mask` [B, L] (1 = real item, end-padded) or `seq_lens` [B].
@@ -234,12 +248,18 @@ class HSTU(torch.nn.Module):
       seq_lens = masks.lengths_from_padding_mask(padding_mask)
     if jagged:
       return self._forward_jagged(inputs, seq_lens, pos_bias, timestamps, ts_bias)
-    x = self.item_embedding[inputs]
-    if self.scale_by_sqrt_dim:
-      x = x * (self.model_dim ** 0.5)
-    if self.position_embedding is not None:
-      x = x + self.position_embedding[: x.shape[1]]
-    x = self._final_norm(x)
+    if self._fused_front_end():
+      pos = None
+      if self.position_embedding is not None:
+        pos = torch.arange(inputs.shape[1], device=inputs.device)[None, :].expand(inputs.shape).contiguous()
+      x = self._embed_norm(inputs, pos)
+    else:
+      x = self.item_embedding[inputs]
+      if self.scale_by_sqrt_dim:
+        x = x * (self.model_dim ** 0.5)
+      if self.position_embedding is not None:
+        x = x + self.position_embedding[: x.shape[1]]
+      x = self._final_norm(x)
     for block in self.decoder_blocks:
       x = block(x, seq_lens=seq_lens, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
     x = self._final_norm(x)
@@ -254,13 +274,18 @@ class HSTU(torch.nn.Module):
     offsets = torch.zeros(B + 1, dtype=torch.int32, device=inputs.device)
     offsets[1:] = torch.cumsum(lens, 0)
     ids = inputs[valid]                                                              # [T], sequence-major
-    x = self.item_embedding[ids]
-    if self.scale_by_sqrt_dim:
-      x = x * (self.model_dim ** 0.5)
+    pos_idx = None
     if self.position_embedding is not None:
       pos_idx = torch.arange(L, device=inputs.device)[None, :].expand(B, L)[valid]
-      x = x + self.position_embedding[pos_idx]
-    x = self._final_norm(x)
+    if self._fused_front_end():
+      x = self._embed_norm(ids, pos_idx)
+    else:
+      x = self.item_embedding[ids]
+      if self.scale_by_sqrt_dim:
+        x = x * (self.model_dim ** 0.5)
+      if pos_idx is not None:
+        x = x + self.position_embedding[pos_idx]
+      x = self._final_norm(x)
     ts = None if timestamps is None else timestamps[valid]
     for block in self.decoder_blocks:
       x = block.forward_jagged(x, offsets, L, pos_bias=pos_bias, timestamps=ts, ts_bias=ts_bias)

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
   assert lib.hstu_block_abi_version() == _lib_block.ABI_VERSION
 
 
-@pytest.mark.parametrize("name", ["HstuNormGateArgs", "HstuGemmSiluArgs"])
+@pytest.mark.parametrize("name", ["HstuNormGateArgs", "HstuGemmSiluArgs", "HstuEmbedNormArgs"])
 def test_struct_layout_matches_header(name):
   struct = getattr(_lib_block, name)
   fields = [f[0] for f in struct._fields_]
@@ -120,6 +120,39 @@ def test_gemm_silu_parity(gpu, M, K, N, bias, act):
   wide = torch.zeros((M, 2 * K), device=dev, dtype=bf)
   wide[:, :K] = x
   assert torch.equal(B.gemm_silu(wide[:, :K], w, b, act), out)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,width,vocab,with_pos,scale", [((5,), 8, 3, False, 1.0), ((4, 33), 512, 1000, True, 512 ** 0.5),
+                                                               ((700,), 1000, 50, True, 1.0), ((3, 2), 4096, 9, False, 2.0)])
+def test_embed_norm_parity(gpu, shape, width, vocab, with_pos, scale):
+  from recml_amd import hstu_block_ops as B
+  gen = torch.Generator().manual_seed(width + vocab)
+  dev, bf = "cuda:0", torch.bfloat16
+  wide = (torch.randn((vocab, width + 8), generator=gen) * 0.02).to(dev).to(bf)
+  table = wide[:, :width]                                      # a table with a row stride of its own
+  ids = torch.randint(0, vocab, shape, generator=gen).to(dev)
+  gamma = (1 + 0.2 * torch.randn(width, generator=gen)).to(dev).to(bf)
+  beta = (0.1 * torch.randn(width, generator=gen)).to(dev).to(bf)
+  pos_table = positions = None
+  if with_pos:
+    pos_table = (torch.randn((40, width), generator=gen) * 0.02).to(dev).to(bf)
+    positions = torch.randint(0, 40, shape, generator=gen).to(dev)
+  out = B.embed_norm(ids, table, gamma, beta, 1e-6, scale=scale, positions=positions, pos_table=pos_table)
+  x = table.double()[ids] * scale
+  if with_pos:
+    x = x + pos_table.double()[positions]
+  mean = x.mean(-1, keepdim=True)
+  var = ((x - mean) ** 2).mean(-1, keepdim=True)
+  ref = (x - mean) / torch.sqrt(var + 1e-6) * gamma.double() + beta.double()
+  assert out.shape == (*shape, width) and out.dtype == bf
+  assert _rel(out.double(), ref) <= 8e-3
+  # indices outside the table are clamped into it
+  far = B.embed_norm(torch.full(shape, vocab + 5, device=dev), table, gamma, beta, 1e-6, scale=scale,
+                     positions=positions, pos_table=pos_table)
+  last = B.embed_norm(torch.full(shape, vocab - 1, device=dev), table, gamma, beta, 1e-6, scale=scale,
+                      positions=positions, pos_table=pos_table)
+  assert torch.equal(far, last)
 
 
 @pytest.mark.gpu

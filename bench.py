@@ -296,7 +296,7 @@ def bench_block_steps(args, dev):
     t0 = time.perf_counter()
     reps = 0
     while time.perf_counter() - t0 < 10.0:
-      ref = u_np * BO.layer_norm(a_np, g_np, b_np, 1e-6)
+      ref = BO.norm_gate(a_np, u_np, g_np, b_np, 1e-6)
       reps += 1
     dt = (time.perf_counter() - t0) / reps
     rec["cpu_baseline"] = {"value": 3 * rows * D * 2 / dt / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",

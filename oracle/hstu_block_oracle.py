@@ -15,6 +15,13 @@ Restates, in plain numpy:
   hstu_model           recml/layers/keras/hstu.py:585-621 (final_norm applied
                        before the blocks and again after them).
   hstu_param_count     the count asserted at recml/layers/keras/hstu_test.py:38-48.
+  norm_gate            u * layer_norm(attn), hstu.py:471-472.
+  gemm_silu            silu(x w + bias), the projections of hstu.py:444-449
+                       (EinsumDense with activation="silu", :281-330) as one product.
+  embed_norm           final_norm(scale * item_embedding[ids] + position_embedding[positions]),
+                       hstu.py:593-601.
+                       These three are compositions of layer_norm and hstu_oracle.silu,
+                       both pinned, with a product / a row lookup.
 
 Pinning (tests/test_hstu_layer.py): layer_norm against the textbook definition
 on hand-sized inputs and against torch's CPU layer_norm; the dense layers are
@@ -100,3 +107,24 @@ def hstu_param_count(vocab_size, max_positions, model_dim, num_layers, add_head=
   if add_head:
     n += vocab_size * d
   return n
+
+
+def norm_gate(attn, u, gamma, beta, eps=1e-6):
+  """u * layer_norm(attn) over the last axis (recml/layers/keras/hstu.py:471-472)."""
+  return np.asarray(u, np.float64) * layer_norm(attn, gamma, beta, eps)
+
+
+def gemm_silu(x, w, bias=None, activation=True):
+  """silu(x w + bias): the block's projections with their activation (hstu.py:444-449)."""
+  y = np.asarray(x, np.float64) @ np.asarray(w, np.float64)
+  if bias is not None:
+    y = y + np.asarray(bias, np.float64)
+  return O.silu(y) if activation else y
+
+
+def embed_norm(ids, table, gamma, beta, eps=1e-6, scale=1.0, positions=None, pos_table=None):
+  """The model's front end (hstu.py:593-601): item row, optional scale, position row, final_norm."""
+  x = np.asarray(table, np.float64)[np.asarray(ids)] * scale
+  if pos_table is not None:
+    x = x + np.asarray(pos_table, np.float64)[np.asarray(positions)]
+  return layer_norm(x, gamma, beta, eps)

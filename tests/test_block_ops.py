@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 import torch
 
+from oracle import hstu_block_oracle as BO
 from recml_amd import _lib_block
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -73,6 +74,22 @@ def test_validation_errors_without_gpu():
   assert lib.hstu_gemm_silu_workspace_bytes() > 0
 
 
+def test_oracle_compositions_on_a_hand_case():
+  # one row [1, 2, 3, 4]: mean 2.5, biased variance 1.25; gate u = [2, 0, -1, 1]
+  a = np.array([[1.0, 2.0, 3.0, 4.0]])
+  u = np.array([[2.0, 0.0, -1.0, 1.0]])
+  z = (a - 2.5) / np.sqrt(1.25)
+  assert np.allclose(BO.norm_gate(a, u, np.ones(4), np.zeros(4), 0.0), u * z, atol=1e-15)
+  x, w = np.array([[1.0, -2.0]]), np.array([[0.5, 1.0], [0.25, -1.0]])
+  y = np.array([[0.0, 3.0]]) + np.array([0.5, -1.0])              # x w + bias = [0.5, 2.0]
+  assert np.allclose(BO.gemm_silu(x, w, np.array([0.5, -1.0]), False), y, atol=1e-15)
+  assert np.allclose(BO.gemm_silu(x, w, np.array([0.5, -1.0])), y / (1 + np.exp(-y)), atol=1e-15)
+  table = np.array([[0.0, 0.0, 0.0, 0.0], [1.0, 2.0, 3.0, 4.0]])
+  pos = np.array([[0.0, 0.0, 0.0, 0.0], [1.0, 1.0, 1.0, 1.0]])    # a constant row shifts the mean only
+  got = BO.embed_norm(np.array([1, 1]), table, np.ones(4), np.zeros(4), 0.0, 2.0, np.array([0, 1]), pos)
+  assert np.allclose(got, np.stack([z[0], z[0]]), atol=1e-15)      # scale 2 and the shift both cancel in the norm
+
+
 def _rel(a, b):
   return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
 
@@ -80,7 +97,7 @@ def _rel(a, b):
 @pytest.mark.gpu
 @pytest.mark.parametrize("rows,width", [(1, 8), (37, 64), (513, 512), (64, 1000), (9, 4096), (3, 8192)])
 def test_norm_gate_parity(gpu, rows, width):
-  """Against fp64 arithmetic on the same bf16 inputs: the fused step rounds once, at the end."""
+  """Against the fp64 oracle on the same bf16 inputs: the fused step rounds once, at the end."""
   from recml_amd import hstu_block_ops as B
   gen = torch.Generator().manual_seed(rows * 7 + width)
   dev, bf = "cuda:0", torch.bfloat16
@@ -90,12 +107,10 @@ def test_norm_gate_parity(gpu, rows, width):
   gamma = (1 + 0.2 * torch.randn(width, generator=gen)).to(dev).to(bf)
   beta = (0.1 * torch.randn(width, generator=gen)).to(dev).to(bf)
   out = B.norm_gate(attn, u, gamma, beta, 1e-6)
-  a64 = attn.double()
-  mean = a64.mean(-1, keepdim=True)
-  var = ((a64 - mean) ** 2).mean(-1, keepdim=True)
-  ref = u.double() * ((a64 - mean) / torch.sqrt(var + 1e-6) * gamma.double() + beta.double())
+  n = lambda t: t.float().cpu().numpy()
+  ref = torch.from_numpy(BO.norm_gate(n(attn), n(u), n(gamma), n(beta), 1e-6))
   assert out.shape == attn.shape and out.dtype == bf
-  assert _rel(out.double(), ref) <= 8e-3                       # bf16 rounding of the result: 2^-8
+  assert _rel(out.double().cpu(), ref) <= 8e-3                 # bf16 rounding of the result: 2^-8
 
 
 @pytest.mark.gpu
@@ -109,13 +124,10 @@ def test_gemm_silu_parity(gpu, M, K, N, bias, act):
   w = (torch.randn((K, N), generator=gen) * 0.05).to(dev).to(bf)
   b = (torch.randn(N, generator=gen) * 0.1).to(dev).to(bf) if bias else None
   out = B.gemm_silu(x, w, b, act)
-  ref = x.double() @ w.double()
-  if bias:
-    ref = ref + b.double()
-  if act:
-    ref = ref * torch.sigmoid(ref)
+  n = lambda t: t.float().cpu().numpy()
+  ref = torch.from_numpy(BO.gemm_silu(n(x), n(w), n(b) if bias else None, act))
   assert out.shape == (M, N) and out.dtype == bf
-  assert _rel(out.double(), ref) <= 8e-3
+  assert _rel(out.double().cpu(), ref) <= 8e-3
   # a strided x (row stride 2K) gives the same values
   wide = torch.zeros((M, 2 * K), device=dev, dtype=bf)
   wide[:, :K] = x
@@ -139,14 +151,11 @@ def test_embed_norm_parity(gpu, shape, width, vocab, with_pos, scale):
     pos_table = (torch.randn((40, width), generator=gen) * 0.02).to(dev).to(bf)
     positions = torch.randint(0, 40, shape, generator=gen).to(dev)
   out = B.embed_norm(ids, table, gamma, beta, 1e-6, scale=scale, positions=positions, pos_table=pos_table)
-  x = table.double()[ids] * scale
-  if with_pos:
-    x = x + pos_table.double()[positions]
-  mean = x.mean(-1, keepdim=True)
-  var = ((x - mean) ** 2).mean(-1, keepdim=True)
-  ref = (x - mean) / torch.sqrt(var + 1e-6) * gamma.double() + beta.double()
+  n = lambda t: t.float().cpu().numpy()
+  ref = torch.from_numpy(BO.embed_norm(ids.cpu().numpy(), n(table), n(gamma), n(beta), 1e-6, scale,
+                                       positions.cpu().numpy() if with_pos else None, n(pos_table) if with_pos else None))
   assert out.shape == (*shape, width) and out.dtype == bf
-  assert _rel(out.double(), ref) <= 8e-3
+  assert _rel(out.double().cpu(), ref) <= 8e-3
   # indices outside the table are clamped into it
   far = B.embed_norm(torch.full(shape, vocab + 5, device=dev), table, gamma, beta, 1e-6, scale=scale,
                      positions=positions, pos_table=pos_table)

@@ -125,6 +125,10 @@ def _boundary_flags(ts, lens, causal):
     ("d32 lengths", 32, 3, 300, 2, [300, 129, 1], False, False, True, False),
     ("d32 pos+ts jagged", 32, 4, 420, 2, [420, 129, 33, 256], True, True, True, True),
     ("d32 ts non-causal", 32, 2, 200, 1, [200, 100], False, True, False, False),
+    # work-list mappings: H < 8, H = 16, and the two cases without a list (H = 3; more sequences than the builder takes)
+    ("H=4", 64, 5, 200, 4, [200, 1, 77, 129, 128], True, False, True, True),
+    ("H=16", 32, 2, 150, 16, [150, 31], True, False, True, False),
+    ("H=3 static grid", 64, 3, 140, 3, [140, 5, 129], True, False, True, True),
 ])
 def test_backward_matrix_core_kernels(gpu, name, d, B, L, H, lens, pos, ts, causal, jagged):
   """bf16, d in {32, 64, 128}: the matrix-core pair of kernels, checked against the oracle (table gradients too)."""
@@ -244,3 +248,18 @@ def test_backward_segment_ids_on_the_matrix_cores(gpu, d, L, causal, window, pos
     assert (g is None) == (w is None), nm
     if g is not None:
       assert _rel(g.float().cpu().numpy().reshape(w.shape), w) <= 2e-2, nm
+
+
+def test_backward_many_short_sequences_static_grid(gpu):
+  """More sequences than the work-list builder takes (8192): the kernels enumerate (sequence, head, tile) themselves."""
+  rng = np.random.default_rng(33)
+  B, L, H, d = 8200, 33, 1, 32
+  bf = torch.bfloat16
+  lens = rng.integers(1, L + 1, B).astype(np.int32)
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, seq_lens=lens)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), seq_lens=_dev(lens), _variant_out=variant)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(g.float().cpu().numpy(), w) <= 2e-2, nm

@@ -263,3 +263,73 @@ def test_backward_many_short_sequences_static_grid(gpu):
   assert variant == ["hstu_bwd_mfma_bf16"]
   for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
     assert _rel(g.float().cpu().numpy(), w) <= 2e-2, nm
+
+
+@pytest.mark.parametrize("seed", list(range(2000, 2014)))
+def test_matrix_core_backward_on_random_option_mixes(gpu, seed):
+  """bf16 backward against the oracle over random mixes of head dim, heads, layout, causal / full,
+  window, segment ids and the two biases with their table gradients (fixed seeds)."""
+  rng = np.random.default_rng(seed)
+  d = int(rng.choice([32, 64, 128]))
+  H = int(rng.choice([1, 2, 4, 8]))
+  L = int(rng.choice([36, 100, 128, 132, 260]))
+  B = int(rng.integers(1, 4))
+  causal = bool(rng.integers(0, 2))
+  window = None if rng.random() < 0.6 else int(rng.integers(0, L))
+  seg = L % 4 == 0 and rng.random() < 0.3
+  jagged = (not seg) and rng.random() < 0.5
+  bf = torch.bfloat16
+  lens = rng.integers(1, L + 1, B).astype(np.int32)
+  lens[rng.integers(0, B)] = L
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  kw, gk = dict(causal=causal), dict(causal=causal)
+  if window is not None:
+    kw["sliding_window_size"] = gk["sliding_window_size"] = window
+  if rng.random() < 0.5:
+    kw["pos_tab"] = (rng.standard_normal((H if rng.random() < 0.5 else 1, 2 * L - 1)) * 0.3).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  t = None
+  if rng.random() < 0.5:
+    kw["ts_tab"] = (rng.standard_normal((H if rng.random() < 0.5 else 1, 65)) * 0.3).astype(np.float32)
+    t = 1_700_000_000 + np.cumsum(np.ceil(rng.exponential(5000.0, (B, L))), axis=1).astype(np.int64)
+    for b in range(B):
+      t[b, lens[b]:] = t[b, lens[b] - 1]
+    kw["timestamps"] = t
+    gk["ts_bias"] = _dev(kw["ts_tab"])
+  if seg:
+    cuts = np.sort(rng.choice(np.arange(1, L), 3, replace=False))
+    sid = np.tile(np.searchsorted(cuts, np.arange(L), side="right").astype(np.int32), (B, 1))
+    kw["q_segment_ids"] = kw["kv_segment_ids"] = sid
+    gk["q_segment_ids"] = gk["kv_segment_ids"] = _dev(sid)
+    lens = np.full((B,), L, np.int32)
+  else:
+    kw["seq_lens"] = lens
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  variant = []
+  gk["_variant_out"] = variant
+  if jagged:
+    pack = lambda x: O.padded_to_jagged(x, lens)
+    (qj, off), (kj, _), (vj, _), (dj, _) = pack(q), pack(k), pack(v), pack(dout)
+    if t is not None:
+      gk["timestamps"] = _dev(np.concatenate([t[b, :lens[b]] for b in range(B)]))
+    got = recml_amd.hstu_attention_bwd(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), _dev(dj, bf),
+                                       seq_offsets=_dev(off.astype(np.int32)), max_len=L, **gk)
+    grads = [O.jagged_to_padded(g.float().cpu().numpy(), off, L) for g in got[:3]]
+  else:
+    if t is not None:
+      gk["timestamps"] = _dev(t)
+    if not seg:
+      gk["seq_lens"] = _dev(lens)
+    got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), **gk)
+    grads = [g.float().cpu().numpy() for g in got[:3]]
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  rows, cols = _boundary_flags(t, lens, causal) if t is not None else (np.zeros((B, L), bool),) * 2
+  for nm, g, w, edge in zip(("dq", "dk", "dv"), grads, want[:3], (rows, cols, cols)):
+    err = np.abs(g - w).max(axis=(2, 3)) / max(np.abs(w).max(), 1e-30)
+    assert err[~edge].max() <= 2e-2, (nm, seed, err[~edge].max())
+    assert not edge.any() or err[edge].max() <= 1e-1, (nm, seed)
+  has_edge = t is not None and rows.any()
+  for nm, g, w, tol in (("dpos", got[3], want[3], 2e-2), ("dts", got[4], want[4], 1e-1 if has_edge else 2e-2)):
+    assert (g is None) == (w is None), nm
+    if g is not None:
+      assert _rel(g.cpu().numpy().reshape(w.shape), w) <= tol, (nm, seed)

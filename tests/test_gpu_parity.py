@@ -546,3 +546,84 @@ def test_segment_ids_on_the_matrix_core_kernel(gpu, d, L, causal, window, pos):
   assert hstu_ops.kernel_variant(a) == "hstu_fwd_mfma_bf16"
   hstu_ops._run(a, keep)
   assert _err(keep[3].float().cpu().numpy(), ref) <= BF16_TOL
+
+
+def _random_case(seed):
+  rng = np.random.default_rng(seed)
+  d = int(rng.choice([32, 64, 128]))
+  H = int(rng.choice([1, 2, 4, 8, 16]))
+  L = int(rng.choice([36, 100, 128, 132, 260, 300]))
+  B = int(rng.integers(1, 5))
+  causal = bool(rng.integers(0, 2))
+  window = None if rng.random() < 0.6 else int(rng.integers(0, L))
+  seg = L % 4 == 0 and rng.random() < 0.3
+  jagged = (not seg) and rng.random() < 0.5
+  pos = rng.random() < 0.5
+  ts = rng.random() < 0.5
+  lens = rng.integers(1, L + 1, B).astype(np.int32)
+  lens[rng.integers(0, B)] = L
+  return dict(d=d, H=H, L=L, B=B, causal=causal, window=window, seg=seg, jagged=jagged, pos=pos, ts=ts, lens=lens, rng=rng)
+
+
+@pytest.mark.parametrize("seed", list(range(1000, 1024)))
+def test_matrix_core_forward_on_random_option_mixes(gpu, seed):
+  """bf16 forward against the oracle over random mixes of head dim, heads, layout, causal / full,
+  window, segment ids and the two biases (fixed seeds; every mix stays on the matrix-core kernel)."""
+  c = _random_case(seed)
+  rng, B, L, H, d, lens = c["rng"], c["B"], c["L"], c["H"], c["d"], c["lens"]
+  bf = torch.bfloat16
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  kw, gk = dict(causal=c["causal"]), dict(causal=c["causal"])
+  if c["window"] is not None:
+    kw["sliding_window_size"] = gk["sliding_window_size"] = c["window"]
+  if c["pos"]:
+    heads = H if rng.random() < 0.5 else 1
+    kw["pos_tab"] = (rng.standard_normal((heads, 2 * L - 1)) * 0.2).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  t = None
+  if c["ts"]:
+    heads = H if rng.random() < 0.5 else 1
+    kw["ts_tab"] = (rng.standard_normal((heads, 65)) * 0.2).astype(np.float32)
+    t = 1_700_000_000 + np.cumsum(np.ceil(rng.exponential(5000.0, (B, L))), axis=1).astype(np.int64)
+    for b in range(B):
+      t[b, lens[b]:] = t[b, lens[b] - 1]
+    kw["timestamps"] = t
+    gk["ts_bias"] = _dev(kw["ts_tab"])
+  if c["seg"]:
+    cuts = np.sort(rng.choice(np.arange(1, L), 3, replace=False))
+    seg = np.tile(np.searchsorted(cuts, np.arange(L), side="right").astype(np.int32), (B, 1))
+    kw["q_segment_ids"] = kw["kv_segment_ids"] = seg
+    gk["q_segment_ids"] = gk["kv_segment_ids"] = _dev(seg)
+    lens = np.full((B,), L, np.int32)
+  else:
+    kw["seq_lens"] = lens
+  ref = O.hstu_attention_ref(q, k, v, dtype=np.float32, **kw)
+  if c["jagged"]:
+    (qj, off), (kj, _), (vj, _) = (O.padded_to_jagged(x, lens) for x in (q, k, v))
+    if t is not None:
+      gk["timestamps"] = _dev(np.concatenate([t[b, :lens[b]] for b in range(B)]))
+    a, keep = hstu_ops.build_args(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), torch.empty((qj.shape[0], H, d), dtype=bf, device="cuda:0"),
+                                  seq_offsets=_dev(off.astype(np.int32)), max_len=L, **gk)
+  else:
+    if t is not None:
+      gk["timestamps"] = _dev(t)
+    if not c["seg"]:
+      gk["seq_lens"] = _dev(lens)
+    a, keep = hstu_ops.build_args(_dev(q, bf), _dev(k, bf), _dev(v, bf), torch.empty((B, L, H, d), dtype=bf, device="cuda:0"), **gk)
+  assert hstu_ops.kernel_variant(a) == "hstu_fwd_mfma_bf16", c
+  hstu_ops._run(a, keep)
+  out = keep[3].float().cpu().numpy()
+  if c["jagged"]:
+    out = O.jagged_to_padded(out, off, L)
+  err = np.abs(out - ref).max(axis=(2, 3)) / max(np.abs(ref).max(), 1e-30)
+  edge = np.zeros((B, L), bool)
+  if t is not None:
+    for b in range(B):
+      near = O.near_bucket_boundary(O.time_delta(t[b:b + 1, :lens[b]])[0], 0.301)
+      if c["causal"]:
+        near &= np.tril(np.ones_like(near, dtype=bool))
+      edge[b, :lens[b]] = near.any(1)
+  assert err[~edge].max() <= BF16_TOL, (c, err[~edge].max())
+  assert not edge.any() or err[edge].max() <= 1e-1, (c, err[edge].max())
+  for b in range(B):
+    assert (out[b, lens[b]:] == 0).all()

@@ -388,6 +388,8 @@ def main():
   ap.add_argument("--no-cold", dest="cold", action="store_false",
                   help="skip the cold-cache variant (a 1 GiB fill between launches)")
   ap.add_argument("--backward", action="store_true", help="measure the backward pass instead of the forward")
+  ap.add_argument("--no-graph", dest="graph", action="store_false",
+                  help="skip the variant that replays the timed calls as one HIP graph")
   ap.add_argument("--calib-copy", action="store_true",
                   help="also run one 512 MiB device copy (reference point for HBM byte counters)")
   args = ap.parse_args()
@@ -430,19 +432,40 @@ def main():
     step()
   torch.cuda.synchronize()
 
-  # whole-region wall clock and per-launch HIP events on the launch stream
-  starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-  ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+  # the timed region: exactly `steps` calls between two synchronisations, nothing else on the stream
   torch.cuda.synchronize()
   t0 = time.perf_counter()
+  for i in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  wall = time.perf_counter() - t0
+
+  # the same calls again with a pair of HIP events around each one, on the launch stream
+  starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+  ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
   for i in range(args.steps):
     starts[i].record()
     step()
     ends[i].record()
   torch.cuda.synchronize()
-  wall = time.perf_counter() - t0
   ev_ms = np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
   region_ms = starts[0].elapsed_time(ends[-1])
+
+  # and recorded once into a HIP graph of `steps` calls (the entry point only enqueues and allocates
+  # nothing): what a caller that replays its step as a graph sees per call
+  graph_ms = None
+  if args.graph:
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      for i in range(args.steps):
+        step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    graph.replay()
+    torch.cuda.synchronize()
+    graph_ms = (time.perf_counter() - t1) * 1e3 / args.steps
+    del graph
 
   # The dominant kernel alone (the roofline figure): the same launches with the preparation kernel
   # skipped -- the workspace still holds what the steps above prepared from the same inputs.
@@ -502,6 +525,7 @@ def main():
           "kernel_ms_median": float(np.median(main_ms)),
           "step_ms_avg": step_ms, "step_ms_cold_avg": cold_ms,
           "region_ms_per_step": region_ms / args.steps,
+          "graph_replay_ms_per_step": graph_ms,
           "algorithmic_flops": flops, "algorithmic_bytes": bytes_alg,
           "arithmetic_intensity": ai,
           "hbm_GBps_algorithmic": bytes_alg / (kernel_ms * 1e-3) / 1e9,

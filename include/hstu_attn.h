@@ -117,6 +117,10 @@ typedef struct HstuAttnFwdArgs {
   const int32_t* q_segment_ids;  /* [B, L],   SEGMENT mode                    */
   const int32_t* kv_segment_ids; /* [B, Lkv], SEGMENT mode                    */
 
+  /* Dense operands (the layer-side call of recml/layers/keras/hstu.py:356-390).  bf16 calls take
+   * them on the matrix cores when Lkv is a multiple of 16 (mask) / 4 (bias), the arrays are
+   * 16-byte aligned and no table bias or segment ids come with them; any other call on the
+   * general kernel. */
   const uint8_t* mask;    /* explicit keep-mask (non-zero = keep) or null     */
   int32_t mask_batched;   /* 0: [L, Lkv] shared; 1: [B, L, Lkv]               */
   int32_t dense_bias_batched; /* 0: [L, Lkv] shared; 1: [B, L, Lkv]           */

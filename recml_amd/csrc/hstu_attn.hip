@@ -10,7 +10,9 @@
 //                        4-stage LDS ring filled by direct global->LDS loads;
 //                        relative-position and timestamp bias + SiLU + mask
 //                        fused on the accumulator registers; causal / length /
-//                        sliding-window tile skipping, segment ids.  Computes
+//                        sliding-window tile skipping, segment ids; or, in
+//                        their place, tiles of a dense [L, Lkv] keep-mask and
+//                        fp32 bias streamed through the same ring.  Computes
 //                        S^T = K Q^T so that the
 //                        accumulator layout of S^T is already the B-operand
 //                        layout of O^T = V^T P^T: P never touches LDS.
@@ -656,8 +658,12 @@ struct MfmaSmem {
   static constexpr int bias_stage(bool pos, bool ts, bool seg = false) {
     return (pos ? POS_BYTES : 0) + (ts ? TK_BYTES : 0) + (seg ? SEG_BYTES : 0);
   }
-  static constexpr int total(bool pos, bool ts, bool seg = false) {
-    return NSTAGE * (STAGE + bias_stage(pos, ts, seg)) + (ts ? TAB_BYTES : 0);
+  // dense operands of a step: the fp32 bias tile (128 rows x 32 keys) and the keep-mask tile (bytes)
+  static constexpr int DB_BYTES = BM * BN * 4;
+  static constexpr int DM_BYTES = BM * BN;
+  static constexpr int dense_stage(int dense) { return ((dense & 1) ? DB_BYTES : 0) + ((dense & 2) ? DM_BYTES : 0); }
+  static constexpr int total(bool pos, bool ts, bool seg = false, int dense = 0) {
+    return NSTAGE * (STAGE + bias_stage(pos, ts, seg) + dense_stage(dense)) + (ts ? TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
   __device__ static constexpr int swz_k(int row) { return (row / KRPB) % KCPR; }
@@ -999,7 +1005,13 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 // SEG: segment ids (padded layout, L a multiple of 4): a pair is kept when its row's and its key's
 // ids are equal.  The step's 32 key ids arrive by one more direct load per wave and every block
 // compares them with the lane's row id.
-template <int D, bool POS, bool TS, bool F8, bool SEG = false>
+//
+// DENSE (bit 0: additive bias, bit 1: keep-mask; the layer-side call of
+// recml/layers/keras/hstu.py:356-390): the step's 128 x 32 tile of the [L, Lkv] fp32 bias and / or
+// of the byte mask comes through the ring like K and V (four more direct loads per wave for the
+// bias, one for the mask).  16 KB + 4 KB a stage: one workgroup per CU.  A block whose mask tile is
+// all zero is skipped.
+template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   constexpr int KB = F8 ? 1 : 2;       // bytes per q / k element
   using SM = MfmaSmem<D, KB>;
@@ -1013,12 +1025,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   constexpr int LDK = NPIECE_K >= NWAVES ? NPIECE_K / NWAVES : 1;
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
   static_assert(SM::K_BYTES % 1024 == 0 && SM::V_BYTES % 1024 == 0, "tile must be a whole number of 1 KB pieces");
-  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);   // direct loads per wave per step
+  static_assert(BM * BN * 4 / 1024 == 4 * NWAVES && BM * BN / 1024 == NWAVES, "dense tiles: 4 + 1 pieces per wave");
+  // direct loads per wave per step
+  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + ((DENSE & 1) ? 4 : 0) + ((DENSE & 2) ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
-  // LDS map: [ring: NSTAGE x (K | V)][bias operands x NSTAGE: 4 pos windows | key timestamps][ts table].
+  // LDS map: [ring: NSTAGE x (K | V)][bias operands x NSTAGE: 4 pos windows | key timestamps][ts table]
+  // [dense operands x NSTAGE: bias tile | mask tile].
   // The key timestamps sit right behind the last position window so that one direct load of the
   // last wave can fill both.
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
@@ -1030,6 +1045,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
   float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
   const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
+  constexpr int DENSE_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
+  constexpr int DENSE_STAGE = SM::dense_stage(DENSE);
+  auto Db = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE; };
+  auto Dm = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE + ((DENSE & 1) ? SM::DB_BYTES : 0); };
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -1161,6 +1180,34 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         lds_dma16_at(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
       }
     }
+    if (DENSE & 1) {
+      // Bias tile: row r of the tile at LDS byte 128 r, its 16-byte chunks XOR-swizzled by r & 7
+      // (the block reads one chunk per lane from 16 consecutive rows).  Wave w brings 1 KB pieces
+      // 4w .. 4w+3 (8 rows each); lane l of a piece lands at row l / 8, physical chunk l % 8.  Rows
+      // past L and keys past Lkv re-read the last row / the last four keys: finite data for
+      // logits that are masked by their index.
+      const float* dbg = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int j = 4 * w + r;
+        const int row = 8 * j + (lane >> 3), pc = lane & 7;
+        int gr = q0 + row;
+        gr = gr < p.L - 1 ? gr : p.L - 1;
+        int col = kv0 + 4 * (pc ^ (row & 7));
+        col = col < p.Lkv - 4 ? col : p.Lkv - 4;
+        lds_dma16(dbg, ((uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col) * 4u, Db(st) + j * 1024);
+      }
+    }
+    if (DENSE & 2) {
+      // Mask tile: row r at LDS byte 32 r; wave w brings its own 32 rows, two lanes per row.
+      const uint8_t* mg = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      const int row = 32 * w + (lane >> 1);
+      int gr = q0 + row;
+      gr = gr < p.L - 1 ? gr : p.L - 1;
+      int col = kv0 + 16 * (lane & 1);
+      col = col < p.Lkv - 16 ? col : p.Lkv - 16;
+      lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Dm(st) + w * 1024);
+    }
   };
 
   // prologue: the scaled bucket table (64 entries per wave, the last wave repeats the first), then
@@ -1236,6 +1283,14 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto block = [&](int t) {
     const int st = t % NSTAGE;
     const int kbs = t * BN;
+    uint32_t mbits[4] = {0u, 0u, 0u, 0u};
+    if (DENSE & 2) {
+      // the lane's 16 mask bytes: keys 8g + 4hh .. +3 of its row; nothing to do when the wave's whole tile is 0
+      const unsigned char* mrow = Dm(st) + (32 * w + m) * 32 + 4 * hh;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) mbits[g] = *(const uint32_t*)(mrow + 8 * g);
+      if (__builtin_amdgcn_ballot_w64((mbits[0] | mbits[1] | mbits[2] | mbits[3]) != 0u) == 0) return;
+    }
     floatx16 sacc;
     {
       uint4 kf[QCH];
@@ -1345,6 +1400,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         }
       }
     }
+    if (DENSE & 1) {
+      const int row = 32 * w + m;
+      const unsigned char* brow = Db(st) + row * 128;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float4 bv = *(const float4*)(brow + (((2 * g + hh) ^ (row & 7)) * 16));
+        u[4 * g + 0] = __builtin_fmaf(bv.x, LOG2E, u[4 * g + 0]);
+        u[4 * g + 1] = __builtin_fmaf(bv.y, LOG2E, u[4 * g + 1]);
+        u[4 * g + 2] = __builtin_fmaf(bv.z, LOG2E, u[4 * g + 2]);
+        u[4 * g + 3] = __builtin_fmaf(bv.w, LOG2E, u[4 * g + 3]);
+      }
+    }
     if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv) || (win >= 0 && (r0 + 31 - kbs > win || kbs + 31 - r0 > win))) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -1364,6 +1431,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         u[4 * g + 2] = ks4.z == qseg ? u[4 * g + 2] : 0.f;
         u[4 * g + 3] = ks4.w == qseg ? u[4 * g + 3] : 0.f;
       }
+    }
+    if (DENSE & 2) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) u[r] = ((mbits[r >> 2] >> (8 * (r & 3))) & 0xffu) ? u[r] : 0.f;
     }
     float pv[16];
 #pragma unroll
@@ -2524,7 +2595,15 @@ bool mfma_eligible(const HstuAttnFwdArgs* a) {
   // segment ids: bf16 only, rows of a multiple of 4 ids (the kernel fetches them four at a time)
   const bool seg_ok = a->mask_mode != HSTU_MASK_SEGMENT ||
                       (kb == 2 && a->L % 4 == 0 && aligned16(a->q_segment_ids) && aligned16(a->kv_segment_ids));
-  const bool opts_ok = seg_ok && !a->mask && !a->dense_bias && a->L == a->Lkv &&
+  // a dense bias or mask: bf16, in place of the table biases and the segment ids; whole 16-byte pieces of
+  // a row (4 floats, 16 mask bytes) must not straddle its end, and a [L, Lkv] matrix is addressed with 32 bits
+  const bool dense = a->mask || a->dense_bias;
+  const bool dense_ok = !dense ||
+      (kb == 2 && !a->pos_tab && !a->ts_tab && a->mask_mode != HSTU_MASK_SEGMENT &&
+       (!a->dense_bias || (a->Lkv % 4 == 0 && aligned16(a->dense_bias))) &&
+       (!a->mask || (a->Lkv % 16 == 0 && aligned16(a->mask))) &&
+       (int64_t)a->L * a->Lkv * 4 < (1LL << 32));
+  const bool opts_ok = seg_ok && dense_ok && a->L == a->Lkv &&
                        // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
                        (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
   auto s8 = [](int64_t x) { return (x & 7) == 0; };
@@ -2741,15 +2820,15 @@ int launch_bwd(const Params& p, hipStream_t st) {
   return HSTU_OK;
 }
 
-template <int D, bool POS, bool TS, bool F8, bool SEG = false>
+template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG);
+  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE);
   static int granted[64];
-  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG>, smem, granted)) return rc;
+  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE>, smem, granted)) return rc;
   hipError_t e;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "mfma kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
@@ -2758,6 +2837,11 @@ int launch_mfma_inst(const Params& p, hipStream_t st) {
 template <int D, bool F8>
 int launch_mfma_d(const Params& p, hipStream_t st) {
   const bool pos = p.pos_tab != nullptr, ts = p.ts_tab != nullptr;
+  if (!F8 && (p.mask || p.dense_bias)) {
+    if (p.mask && p.dense_bias) return launch_mfma_inst<D, false, false, false, false, 3>(p, st);
+    if (p.mask) return launch_mfma_inst<D, false, false, false, false, 2>(p, st);
+    return launch_mfma_inst<D, false, false, false, false, 1>(p, st);
+  }
   if (!F8 && p.mask_mode == HSTU_MASK_SEGMENT) {
     if (pos && ts) return launch_mfma_inst<D, true, true, false, true>(p, st);
     if (pos) return launch_mfma_inst<D, true, false, false, true>(p, st);
@@ -2827,6 +2911,7 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
   if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
+  if (f.mask || f.dense_bias) return false;   // dense operands: the general pair
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||

@@ -95,7 +95,7 @@ def test_backward_variant_query():
   f.window = 8                                                        # a sliding window stays on the matrix cores
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
   f.window = -1
-  f.mask = 0x50000                                                    # an explicit mask does not
+  f.mask = 0x50000                                                    # an explicit mask does not (the forward would)
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
   f.mask = None
   f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_FP32
@@ -161,8 +161,22 @@ def test_variant_and_workspace_query():
   a.window = 4                                         # a sliding window stays on the matrix cores
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
   a.window = -1
-  a.dense_bias = 0x30000                               # a dense bias does not
+  a.dense_bias = 0x30000                               # so do a dense bias and an explicit mask ...
+  a.mask = 0x50000
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
+  a.dense_bias = 0x30004                               # ... unless their rows cannot be fetched 16 bytes at a time,
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"
-  a.dense_bias = None
+  a.dense_bias = 0x30000
+  a.pos_tab, a.pos_heads = 0x20000, 4                  # or a table bias comes on top
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"
+  a.pos_tab, a.pos_heads = None, 0
+  a.dense_bias = a.mask = None
+  a.L = a.Lkv = 248                                    # 248 = 8 x 31: whole pieces of 4 floats, not of 16 mask bytes
+  a.dense_bias = 0x30000
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
+  a.mask = 0x50000
+  assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"
+  a.dense_bias = a.mask = None
+  a.L = a.Lkv = 256
   a.d_qk = a.d_v = 48
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_general<bf16>"

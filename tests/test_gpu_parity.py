@@ -336,6 +336,60 @@ def test_layer_call_dense_mask_and_bias(gpu):
   assert _err(out2.cpu().numpy(), ref) <= FP32_TOL
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("what", ["mask+bias", "mask", "bias", "shared"])
+def test_layer_call_dense_on_matrix_cores(gpu, d, what):
+  # the same dense call in bf16: the matrix-core kernel takes the [B, L, L] mask and bias tiles through its ring.
+  # L = 176: whole 16-byte mask pieces, a partial last key tile and a partial last query tile.
+  rng = np.random.default_rng(440 + d)
+  B, L, H = 3, 176, 2
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  lens = np.array([176, 77, 1])
+  pad = (np.arange(L)[None] < lens[:, None]).astype(np.float32)
+  causal = O.make_causal_mask(pad)
+  mask = bias = None
+  if what in ("mask+bias", "mask"):
+    mask = causal
+  if what == "shared":
+    mask = (rng.random((L, L)) < 0.5)          # one [L, L] mask and bias for the whole batch
+    bias = rng.standard_normal((L, L)).astype(np.float32) * 0.5
+  elif what in ("mask+bias", "bias"):
+    bias = rng.standard_normal((B, L, L)).astype(np.float32) * 0.5
+  qd, kd, vd = (_dev(t, torch.bfloat16) for t in (q, k, v))
+  out = torch.full_like(vd, float("nan"))
+  args, keep = hstu_ops.build_args(qd, kd, vd, out, n=L, alpha=1.0, causal=False,
+                                   mask=None if mask is None else _dev(np.asarray(mask, np.uint8)),
+                                   bias=_dev(bias))
+  assert hstu_ops.kernel_variant(args) == "hstu_fwd_mfma_bf16"
+  hstu_ops._run(args, keep)
+  torch.cuda.synchronize()
+  got = out.float().cpu().numpy()
+  ref_mask = np.ones((B, L, L)) if mask is None else np.broadcast_to(np.asarray(mask, np.float64), (B, L, L))
+  ref_bias = None if bias is None else (bias[None] if bias.ndim == 2 else bias)
+  ref = O.pointwise_attention_dense(q, k, v, ref_mask, ref_bias)
+  assert _err(got, ref) <= BF16_TOL
+  if what in ("mask+bias", "mask"):
+    for b in range(B):
+      assert (got[b, lens[b]:] == 0).all()     # fully masked rows: exact zeros
+
+
+def test_dense_bias_large_on_matrix_cores(gpu):
+  # a longer case (several query tiles, the key range split over workgroups): against the general kernel,
+  # which the fp32 call takes, on the same bf16-rounded inputs
+  rng = np.random.default_rng(450)
+  B, L, H, d = 2, 1040, 2, 64
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  lens = np.array([1040, 333])
+  pad = (np.arange(L)[None] < lens[:, None]).astype(np.float32)
+  mask = _dev(O.make_causal_mask(pad).astype(np.uint8))
+  bias = _dev(rng.standard_normal((B, L, L)).astype(np.float32) * 0.5)
+  got = recml_amd.pointwise_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16), mask, bias)
+  ref = recml_amd.pointwise_attention(_dev(q), _dev(k), _dev(v), mask, bias)
+  torch.cuda.synchronize()
+  assert _err(got.float().cpu().numpy(), ref.cpu().numpy()) <= BF16_TOL
+  assert (got[1, 333:] == 0).all()
+
+
 def test_shared_tables_and_strided_inputs(gpu):
   rng = np.random.default_rng(45)
   B, L, H, d = 2, 130, 4, 64

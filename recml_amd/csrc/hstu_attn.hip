@@ -739,9 +739,9 @@ constexpr int MAX_CHUNKS = 4;
 
 // Most workgroups a query tile can be shared by (from its position alone), and how many share
 // it given its actual number of steps.
-__host__ __device__ __forceinline__ int chunks_max(int split_steps, int causal, int L, int qt) {
+__host__ __device__ __forceinline__ int chunks_max(int split_steps, int causal, int Lkv, int qt) {
   if (split_steps <= 0) return 1;
-  const int all = (L + BN - 1) / BN;
+  const int all = (Lkv + BN - 1) / BN;
   int nt = causal ? (qt + 1) * (BM / BN) : all;
   nt = nt < all ? nt : all;
   const int c = (nt + split_steps - 1) / split_steps;
@@ -793,7 +793,7 @@ __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, W
   const int bhk = j / p.entries_per_bh;
   int qt = p.n_qtiles - 1, chunk = j - bhk * p.entries_per_bh;
   for (;;) {
-    const int c = chunks_max(p.split_steps, p.causal, p.L, qt);
+    const int c = chunks_max(p.split_steps, p.causal, p.Lkv, qt);
     if (chunk < c) break;
     chunk -= c;
     --qt;
@@ -2594,7 +2594,7 @@ bool mfma_eligible(const HstuAttnFwdArgs* a) {
   const bool d_ok = a->d_qk == a->d_v && (a->d_qk == 32 || a->d_qk == 64 || a->d_qk == 128);
   // segment ids: bf16 only, rows of a multiple of 4 ids (the kernel fetches them four at a time)
   const bool seg_ok = a->mask_mode != HSTU_MASK_SEGMENT ||
-                      (kb == 2 && a->L % 4 == 0 && aligned16(a->q_segment_ids) && aligned16(a->kv_segment_ids));
+                      (kb == 2 && a->L % 4 == 0 && a->Lkv % 4 == 0 && aligned16(a->q_segment_ids) && aligned16(a->kv_segment_ids));
   // a dense bias or mask: bf16, in place of the table biases and the segment ids; whole 16-byte pieces of
   // a row (4 floats, 16 mask bytes) must not straddle its end, and a [L, Lkv] matrix is addressed with 32 bits
   const bool dense = a->mask || a->dense_bias;
@@ -2603,7 +2603,9 @@ bool mfma_eligible(const HstuAttnFwdArgs* a) {
        (!a->dense_bias || (a->Lkv % 4 == 0 && aligned16(a->dense_bias))) &&
        (!a->mask || (a->Lkv % 16 == 0 && aligned16(a->mask))) &&
        (int64_t)a->L * a->Lkv * 4 < (1LL << 32));
-  const bool opts_ok = seg_ok && dense_ok && a->L == a->Lkv &&
+  // keys and queries of different lengths: the padded layout without the table biases (whose geometry needs one length)
+  const bool len_ok = a->L == a->Lkv || (a->layout == HSTU_LAYOUT_PADDED && !a->pos_tab && !a->ts_tab);
+  const bool opts_ok = seg_ok && dense_ok && len_ok &&
                        // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
                        (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
   auto s8 = [](int64_t x) { return (x & 7) == 0; };
@@ -2614,7 +2616,7 @@ bool mfma_eligible(const HstuAttnFwdArgs* a) {
                         (a->layout == HSTU_LAYOUT_JAGGED ||
                          (sq(a->q_stride_b) && sq(a->k_stride_b) && s8(a->v_stride_b) && s8(a->o_stride_b)));
   // the kernel addresses K and V rows with 32-bit byte offsets from the (sequence, head) base
-  const bool off_ok = (int64_t)a->L * a->k_stride_t * kb < (1LL << 31) && (int64_t)a->L * a->v_stride_t * 2 < (1LL << 31) &&
+  const bool off_ok = (int64_t)a->Lkv * a->k_stride_t * kb < (1LL << 31) && (int64_t)a->Lkv * a->v_stride_t * 2 < (1LL << 31) &&
                       a->k_stride_t > 0 && a->v_stride_t > 0;
   return d_ok && opts_ok && align_ok && off_ok;
 }
@@ -2697,7 +2699,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) 
   // the partials costs more than it saves.  The lengths are on the device, so the decision rests
   // on what the shapes allow.
   const int n_qtiles = (a->L + BM - 1) / BM;
-  const int steps_max = (a->L + BN - 1) / BN;
+  const int steps_max = (a->Lkv + BN - 1) / BN;
   const bool jag = a->layout == HSTU_LAYOUT_JAGGED;
   const long long tiles_est = (long long)a->H * (jag ? (a->total_tokens / BM + a->B) : (long long)a->B * n_qtiles);
   w.entries_per_bh = n_qtiles;
@@ -2706,10 +2708,16 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) 
     w.split_steps = w.split_steps < 16 ? 16 : w.split_steps;
     // first tile with more steps than that (a causal tile qt has up to 4 (qt + 1) steps)
     w.qt_split = a->causal ? w.split_steps / (BM / BN) : 0;
-    w.entries_per_bh = 0;
-    for (int qt = 0; qt < n_qtiles; ++qt) w.entries_per_bh += chunks_max(w.split_steps, a->causal != 0, a->L, qt);
-    const size_t slots = jag ? (size_t)(a->total_tokens / BM) + (size_t)a->B + 1 : (size_t)a->B * (size_t)(n_qtiles - w.qt_split);
-    w.partial_bytes = up(slots * (size_t)a->H * MAX_CHUNKS * (size_t)BM * (size_t)a->d_v * sizeof(float));
+    if (w.qt_split >= n_qtiles) {
+      // causal with fewer query rows than keys: no tile reaches that many steps
+      w.split_steps = 0;
+      w.qt_split = 0;
+    } else {
+      w.entries_per_bh = 0;
+      for (int qt = 0; qt < n_qtiles; ++qt) w.entries_per_bh += chunks_max(w.split_steps, a->causal != 0, a->Lkv, qt);
+      const size_t slots = jag ? (size_t)(a->total_tokens / BM) + (size_t)a->B + 1 : (size_t)a->B * (size_t)(n_qtiles - w.qt_split);
+      w.partial_bytes = up(slots * (size_t)a->H * MAX_CHUNKS * (size_t)BM * (size_t)a->d_v * sizeof(float));
+    }
   }
   // A work list built on the device spares the launch of workgroups that would find nothing to do
   // (a jagged batch with a long maximum length and mostly short sequences is mostly such).  Its
@@ -2911,7 +2919,7 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
   if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
-  if (f.mask || f.dense_bias) return false;   // dense operands: the general pair
+  if (f.mask || f.dense_bias || f.L != f.Lkv) return false;   // dense operands, keys and queries of different lengths: the general pair
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||

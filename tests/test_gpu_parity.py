@@ -313,6 +313,31 @@ def test_splash_full_explicit_window_cross_length(gpu):
     assert _err(out.cpu().numpy(), ref) <= FP32_TOL
 
 
+@pytest.mark.parametrize("Lq,Lk", [(200, 336), (336, 208), (100, 2080)])
+def test_cross_length_on_matrix_cores(gpu, Lq, Lk):
+  # keys and queries of different lengths in bf16: FULL, causal, sliding window, an explicit [Lq, Lk] mask, segment ids
+  rng = np.random.default_rng(46)
+  B, H, d = 2, 3, 64
+  q = O.round_bf16(rng.standard_normal((B, Lq, H, d)).astype(np.float32) * 0.3)
+  k = O.round_bf16(rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.3)
+  v = O.round_bf16(rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.3)
+  qd, kd, vd = (_dev(t, torch.bfloat16) for t in (q, k, v))
+  m = rng.random((Lq, Lk)) < 0.4
+  cases = [dict(causal=False), dict(causal=True), dict(causal=True, sliding_window_size=40),
+           dict(causal=False, sliding_window_size=7), dict(causal=False, mask=m)]
+  for kw in cases:
+    out = torch.full((B, Lq, H, d), float("nan"), dtype=torch.bfloat16, device=qd.device)
+    dkw = dict(kw)
+    if "mask" in dkw:
+      dkw["mask"] = _dev(m.astype(np.uint8))
+    args, keep = hstu_ops.build_args(qd, kd, vd, out, n=Lq, alpha=0.125, **dkw)
+    assert hstu_ops.kernel_variant(args) == "hstu_fwd_mfma_bf16", kw
+    hstu_ops._run(args, keep)
+    torch.cuda.synchronize()
+    ref = O.hstu_attention_ref(q, k, v, alpha=0.125, n=Lq, **kw)
+    assert _err(out.float().cpu().numpy(), ref) <= BF16_TOL, kw
+
+
 def test_layer_call_dense_mask_and_bias(gpu):
   # HSTUBlock._pointwise_attention (hstu.py:356-390): dense [B,L,L] mask + bias
   rng = np.random.default_rng(44)

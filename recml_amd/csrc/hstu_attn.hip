@@ -771,7 +771,8 @@ __device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0)
 // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with its own L2: every
 // tile of one (sequence, head) goes to the same XCD, and tiles of a sequence are adjacent in
 // launch order, the one with most keys first, so that the tiles running together stream the
-// same K/V rows and share them through that L2.  Returns false when there is nothing to do.
+// same K/V rows and share them through that L2.  (Calls with a dense mask or bias are dealt
+// differently, see below.)  Returns false when there is nothing to do.
 struct Work { int b, h, qt, chunk; Seq s; };
 template <bool SPLIT_LIST = false>
 __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, Work& wk) {
@@ -779,11 +780,23 @@ __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, W
   if (p.sched) {
     // from the work list: with H >= 8 head h runs on XCD h % 8, else 8 / H items share a round
     int it, h;
-    if (p.H >= 8) { const int hx = p.H >> 3; it = j / hx; h = (j - it * hx) * 8 + xcd; }
+    if (!SPLIT_LIST && (p.mask || p.dense_bias)) {
+      // Dense operands are shared by the heads, not by the query tiles: the H workgroups of an item
+      // are neighbours on one XCD (they start together and fetch the same mask / bias tiles, so all
+      // but the first find them in that L2), and runs of n_qtiles items -- the tiles of one full
+      // sequence, which share K and V -- stay on one XCD too, dealt round-robin over the eight.
+      const int li = j / p.H, nq = p.n_qtiles;
+      h = j - li * p.H;
+      const int grp = li / nq;
+      it = (grp * 8 + xcd) * nq + (li - grp * nq);
+    }
+    else if (p.H >= 8) { const int hx = p.H >> 3; it = j / hx; h = (j - it * hx) * 8 + xcd; }
     else          { const int r = 8 / p.H;   it = j * r + xcd / p.H; h = xcd % p.H; }
     // the item is read before the count is checked (the grid never reaches past the list's capacity):
     // both loads miss the cache, and one after the other they cost a workgroup twice the latency
-    const int4 item = ((const int4*)(p.sched + 4))[(SPLIT_LIST ? p.items_max : 0) + it];
+    // (the dense mapping rounds its grid up to whole rounds of eight runs: indices past the capacity read item 0)
+    const int it_ld = (SPLIT_LIST || it < p.items_max) ? it : 0;
+    const int4 item = ((const int4*)(p.sched + 4))[(SPLIT_LIST ? p.items_max : 0) + it_ld];
     if (it >= p.sched[SPLIT_LIST ? 1 : 0]) return false;
     wk.b = item.x; wk.h = h; wk.qt = item.y & 0xffff; wk.chunk = item.y >> 16;
     wk.s = seq_from(p, wk.b, h, item.z, item.w);
@@ -2805,6 +2818,10 @@ int launch_general(const Params& p, hipStream_t st) {
 long long mfma_grid(const Params& p, bool split_list = false) {
   if (p.sched) {
     const long long n = split_list ? p.split_max : p.items_max;
+    if (!split_list && (p.mask || p.dense_bias)) {
+      const long long groups = (n + p.n_qtiles - 1) / p.n_qtiles;     // runs of n_qtiles items, eight runs a round
+      return 8LL * ((groups + 7) / 8) * p.n_qtiles * p.H;
+    }
     const long long rounds = p.H >= 8 ? n * (p.H / 8) : (n + 8 / p.H - 1) / (8 / p.H);
     return 8LL * rounds;
   }

@@ -307,6 +307,82 @@ def bench_block_steps(args, dev):
   print(json.dumps(rec))
 
 
+def calib_copy(dev):
+  """One 512 MiB device-to-device copy: a dispatch of known size to scale the HBM byte counters by."""
+  import torch
+  src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+  dst = torch.empty_like(src)
+  dst.copy_(src)
+  torch.cuda.synchronize()
+  del src, dst
+
+
+def bench_dense(args, dev):
+  """The layer-side call (dense [B, L, L] causal mask + additive bias shared by heads) in bf16: one JSON line.
+
+  B=16, L=2048, H=8, d=128.  FLOPs: the pairs the mask keeps.  Algorithmic bytes: Q, K, V, O once and the
+  mask and the bias once (they are shared by the heads; the kernel re-reads them per head)."""
+  import torch
+  from recml_amd import hstu_ops
+  from oracle import hstu_oracle as O
+  B, L, H, d = 16, 2048, 8, 128
+  gen = torch.Generator(device=dev).manual_seed(11)
+  q, k, v = (torch.randn((B, L, H, d), device=dev, generator=gen).mul_(0.3).to(torch.bfloat16) for _ in range(3))
+  mask = torch.tril(torch.ones((L, L), device=dev, dtype=torch.uint8))[None].expand(B, L, L).contiguous()
+  bias = torch.randn((B, L, L), device=dev, generator=gen).mul_(0.3)
+  out = torch.empty_like(v)
+  call_args, keep = hstu_ops.build_args(q, k, v, out, n=L, alpha=1.0, causal=False, mask=mask, bias=bias)
+  variant = hstu_ops.kernel_variant(call_args)
+  step = lambda: hstu_ops._run(call_args, keep)
+  if args.calib_copy:
+    calib_copy(dev)
+  for _ in range(args.warmup):
+    step()
+  torch.cuda.synchronize()
+  t0 = time.perf_counter()
+  for _ in range(args.steps):
+    step()
+  torch.cuda.synchronize()
+  ms = (time.perf_counter() - t0) * 1e3 / args.steps
+  ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+  for a, b in ev:
+    a.record()
+    step()
+    b.record()
+  torch.cuda.synchronize()
+  ker = float(np.mean([a.elapsed_time(b) for a, b in ev]))
+  flops = 4.0 * d * H * B * L * (L + 1) / 2
+  nbytes = 4 * B * L * H * d * 2 + B * L * L * 5
+  rec = {
+      "metric": "HSTU attn fwd TFLOP/s (kept pairs), dense mask + bias, L=%d bf16" % L, "value": flops / (ms * 1e-3) / 1e12,
+      "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+      "config": {"workload": f"A1-dense: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",
+                 "kernel": variant},
+      "roofline": {"bound": "hbm", "achieved": nbytes / (ker * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                   "frac": nbytes / (ker * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "kernel_ms_avg": ker,
+                   "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
+                   "dense_operand_bytes_as_read_per_head": H * B * L * L * 5,
+                   "mfma_frac": flops / (ker * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
+  }
+  if not args.no_cpu:
+    # the numpy restatement on the first sequence's first 256 rows and keys (the causal mask keeps earlier keys only)
+    n = 256
+    f = lambda t: t[:1, :n].float().cpu().numpy()
+    t0 = time.perf_counter()
+    ref = O.pointwise_attention_dense(f(q), f(k), f(v), mask[:1, :n, :n].cpu().numpy(), bias[:1, :n, :n].cpu().numpy())
+    dt = time.perf_counter() - t0
+    ref = ref * (n / L)     # the restatement divides by its own length
+    got = out[:1, :n].float().cpu().numpy()
+    err = float(np.abs(got - ref).max() / np.abs(ref).max())
+    rec["cpu_baseline"] = {"value": 4.0 * d * H * n * (n + 1) / 2 / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                           "sample": f"numpy restatement, first sequence, first {n} rows and keys, one evaluation"}
+    rec["parity_max_abs_over_max_ref"] = err
+    if not err <= 2e-2:
+      raise SystemExit(f"parity failed in the benchmark run: {err}")
+  print(json.dumps(rec))
+
+
 def bench_backward(args, w, q, k, v, kw, dev):
   """The backward pass on the same workload, table gradients included: one JSON line.
 
@@ -408,6 +484,8 @@ def main():
     return bench_model(args, dev)
   if args.workload == "c4-block-steps":
     return bench_block_steps(args, dev)
+  if args.workload == "a1-dense":
+    return bench_dense(args, dev)
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
   if args.backward:
@@ -422,11 +500,7 @@ def main():
     hstu_ops._run(call_args, keep)
 
   if args.calib_copy:
-    src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
-    dst = torch.empty_like(src)
-    dst.copy_(src)
-    torch.cuda.synchronize()
-    del src, dst
+    calib_copy(dev)
 
   for _ in range(args.warmup):
     step()

@@ -398,6 +398,37 @@ def test_layer_call_dense_on_matrix_cores(gpu, d, what):
       assert (got[b, lens[b]:] == 0).all()     # fully masked rows: exact zeros
 
 
+def test_dense_bias_with_lengths_on_matrix_cores(gpu):
+  # the dense bias on top of the causal flag and a length mask (padded), and in the jagged layout
+  rng = np.random.default_rng(447)
+  B, L, H, d = 3, 208, 2, 64
+  lens = np.array([208, 97, 33], dtype=np.int32)
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  bias = rng.standard_normal((B, L, L)).astype(np.float32) * 0.5
+  pad = (np.arange(L)[None] < lens[:, None]).astype(np.float32)
+  ref = O.pointwise_attention_dense(q, k, v, O.make_causal_mask(pad), bias)
+  qd, kd, vd = (_dev(t, torch.bfloat16) for t in (q, k, v))
+  out = torch.full_like(vd, float("nan"))
+  args, keep = hstu_ops.build_args(qd, kd, vd, out, n=L, alpha=1.0, causal=True, seq_lens=_dev(lens), bias=_dev(bias))
+  assert hstu_ops.kernel_variant(args) == "hstu_fwd_mfma_bf16"
+  hstu_ops._run(args, keep)
+  torch.cuda.synchronize()
+  got = out.float().cpu().numpy()
+  assert _err(got, ref) <= BF16_TOL
+  for b in range(B):
+    assert (got[b, lens[b]:] == 0).all()
+  # jagged: the same sequences packed; bias rows and columns are the positions within a sequence
+  off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+  pack = lambda t: np.concatenate([t[b, :lens[b]] for b in range(B)])
+  qj, kj, vj = (_dev(pack(t), torch.bfloat16) for t in (q, k, v))
+  outj = torch.full_like(vj, float("nan"))
+  args, keep = hstu_ops.build_args(qj, kj, vj, outj, n=L, alpha=1.0, causal=True, seq_offsets=_dev(off), max_len=L, bias=_dev(bias))
+  assert hstu_ops.kernel_variant(args) == "hstu_fwd_mfma_bf16"
+  hstu_ops._run(args, keep)
+  torch.cuda.synchronize()
+  assert _err(outj.float().cpu().numpy(), pack(ref)) <= BF16_TOL
+
+
 def test_dense_bias_large_on_matrix_cores(gpu):
   # a longer case (several query tiles, the key range split over workgroups): against the general kernel,
   # which the fp32 call takes, on the same bf16-rounded inputs

@@ -7,7 +7,7 @@
 //   hstu_fwd_mfma_bf16   the hot path.  bf16 (or fp8 e4m3fn) Q/K, bf16 V, fp32
 //                        accumulation on the 32x32x16 MFMA; 128 query rows per
 //                        workgroup, keys streamed 32 at a time through a
-//                        4-stage LDS ring filled by direct global->LDS loads;
+//                        4-stage (d <= 64: 3-stage) LDS ring filled by direct global->LDS loads;
 //                        relative-position and timestamp bias + SiLU + mask
 //                        fused on the accumulator registers; causal / length /
 //                        sliding-window tile skipping, segment ids; or, in
@@ -662,8 +662,8 @@ struct MfmaSmem {
   static constexpr int DB_BYTES = BM * BN * 4;
   static constexpr int DM_BYTES = BM * BN;
   static constexpr int dense_stage(int dense) { return ((dense & 1) ? DB_BYTES : 0) + ((dense & 2) ? DM_BYTES : 0); }
-  static constexpr int total(bool pos, bool ts, bool seg = false, int dense = 0) {
-    return NSTAGE * (STAGE + bias_stage(pos, ts, seg) + dense_stage(dense)) + (ts ? TAB_BYTES : 0);
+  static constexpr int total(bool pos, bool ts, bool seg = false, int dense = 0, int nst = NSTAGE) {
+    return nst * (STAGE + bias_stage(pos, ts, seg) + dense_stage(dense)) + (ts ? TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
   __device__ static constexpr int swz_k(int row) { return (row / KRPB) % KCPR; }
@@ -1024,6 +1024,13 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 // of the byte mask comes through the ring like K and V (four more direct loads per wave for the
 // bias, one for the mask).  16 KB + 4 KB a stage: one workgroup per CU.  A block whose mask tile is
 // all zero is skipped.
+// Ring depth of the forward kernel.  Up to d = 64 a wave needs at most 128 registers, so four
+// workgroups fit a CU once their LDS does: three stages (two steps in flight behind the one being
+// computed) instead of four take the d = 64 kernel with a position table from 43 KB to 32 KB, three
+// workgroups per CU to four (measured: 148 -> 139 us on the d = 64 benchmark shape).  At d = 128
+// registers allow two workgroups whatever the ring, and the depth makes no measurable difference.
+constexpr int fwd_stages(int d, int dense) { return (d <= 64 && dense == 0) ? 3 : 4; }
+
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   constexpr int KB = F8 ? 1 : 2;       // bytes per q / k element
@@ -1038,6 +1045,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   constexpr int LDK = NPIECE_K >= NWAVES ? NPIECE_K / NWAVES : 1;
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
   static_assert(SM::K_BYTES % 1024 == 0 && SM::V_BYTES % 1024 == 0, "tile must be a whole number of 1 KB pieces");
+  constexpr int NSTAGE = fwd_stages(D, DENSE);   // the ring depth of this kernel (shadows the backward kernels' constant)
   static_assert(BM * BN * 4 / 1024 == 4 * NWAVES && BM * BN / 1024 == NWAVES, "dense tiles: 4 + 1 pieces per wave");
   // direct loads per wave per step
   constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + ((DENSE & 1) ? 4 : 0) + ((DENSE & 2) ? 1 : 0);
@@ -2847,7 +2855,7 @@ int launch_bwd(const Params& p, hipStream_t st) {
 
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE);
+  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE, fwd_stages(D, DENSE));
   static int granted[64];
   if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE>, smem, granted)) return rc;
   hipError_t e;

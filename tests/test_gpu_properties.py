@@ -157,12 +157,12 @@ def test_backward_identities_at_full_size(c3):
   torch.cuda.synchronize()
   assert variant == ["hstu_bwd_mfma_bf16"]
   dot = lambda a, b: (a.double() * b.double()).sum().item()
+  # both sides are sums of 16.8 M products that mostly cancel: the tolerance is on the sums themselves
+  # (observed: 3e-5 and 2e-4 of them), which a gradient off by a constant factor or one missing tile would break
   qdq, kdk = dot(c3.q, dq), dot(c3.k, dk)
-  scale = (c3.q.double().abs() * dq.double().abs()).sum().item()
-  assert abs(qdq - kdk) <= 2e-3 * scale, (qdq, kdk, scale)
+  assert abs(qdq) > 1e-3 and abs(qdq - kdk) <= 5e-3 * abs(qdq), (qdq, kdk)
   vdv, odo = dot(c3.v, dv), dot(out, dout)
-  scale = (out.double().abs() * dout.double().abs()).sum().item()
-  assert abs(vdv - odo) <= 2e-3 * scale, (vdv, odo, scale)
+  assert abs(odo) > 1e-3 and abs(vdv - odo) <= 5e-3 * abs(odo), (vdv, odo)
   # linear in dout: twice the upstream gradient, twice every gradient (a power of two: exact in bf16, and the
   # table gradients differ only by the order of their atomic sums)
   dq2, dk2, dv2, dpos2, dts2 = recml_amd.hstu_attention_bwd(c3.q, c3.k, c3.v, (2 * dout.float()).to(torch.bfloat16),

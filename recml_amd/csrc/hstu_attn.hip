@@ -44,6 +44,7 @@
 // hstu.py:33-55, 190-221 (timestamp buckets).
 
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -1142,8 +1143,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // logical chunk that the swizzle maps there.  Rows past the sequence re-read
   // the last valid row (finite data; their logits are masked).  Every wave
   // issues the same number of loads per step: the vmcnt arithmetic relies on it.
-  auto dma_step = [&](int t) {
-    const int st = t % NSTAGE;
+  // The ring stage is a compile-time constant everywhere (the step loop is unrolled over the ring):
+  // LDS addresses are then a per-lane register plus an immediate, with no address arithmetic per step.
+  // Stage of step t: (t - t_lo) % NSTAGE.
+  auto dma_step = [&](int t, auto st_) {
+    constexpr int st = decltype(st_)::value;
     const int kv0 = t * BN;
     const int last = s.n_kv - 1;
 #pragma unroll
@@ -1242,7 +1246,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // The first step's tiles go out alone; the other two of the prologue follow behind the Q
   // fragments, whose wait below covers every load issued before it: behind all three steps it
   // held up the first block until the whole prologue had landed.
-  if (t_lo < nt) dma_step(t_lo);
+  if (t_lo < nt) dma_step(t_lo, std::integral_constant<int, 0>{});
 
   // Q fragments (B operand of S^T = K Q^T).  bf16: k-step ks of lane (row, hh) holds
   // q[qrow][16ks+8hh .. +7], i.e. 16-byte chunk 2ks+hh of the row.  fp8: the lane holds chunks
@@ -1278,9 +1282,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     asm volatile("" ::"v"(tq), "v"(tq32));
   }
 
-#pragma unroll
-  for (int t = 1; t < NSTAGE - 1; ++t)
-    if (t_lo + t < nt) dma_step(t_lo + t);
+  if (t_lo + 1 < nt) dma_step(t_lo + 1, std::integral_constant<int, 1>{});
+  if constexpr (NSTAGE > 3) {
+    if (t_lo + 2 < nt) dma_step(t_lo + 2, std::integral_constant<int, 2>{});
+  }
 
   floatx16 o[DVB];
 #pragma unroll
@@ -1301,8 +1306,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // the causal diagonal or the end of the sequence get their logits zeroed where
   // masked: silu(0) = 0 exactly, so nothing is needed after the activation and
   // interior blocks pay nothing.
-  auto block = [&](int t) {
-    const int st = t % NSTAGE;
+  auto block = [&](int t, auto st_) {
+    constexpr int st = decltype(st_)::value;
     const int kbs = t * BN;
     uint32_t mbits[4] = {0u, 0u, 0u, 0u};
     if (DENSE & 2) {
@@ -1489,11 +1494,23 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
   // which now receives step t+3; the block of step t is computed; then every
   // wave makes sure its share of step t+1 has landed before the next barrier.
-  for (int t = t_lo; t < nt; ++t) {
-    if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1);
-    if (t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0)) block(t);
+  auto step = [&](int t, auto st_) {
+    constexpr int st = decltype(st_)::value;
+    if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1, std::integral_constant<int, (st + NSTAGE - 1) % NSTAGE>{});
+    if (t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0)) block(t, st_);
     if (t + 1 < nt) wait_step(t + 1);
     __syncthreads();
+  };
+  for (int t = t_lo; t < nt; t += NSTAGE) {
+    step(t, std::integral_constant<int, 0>{});
+    if (t + 1 >= nt) break;
+    step(t + 1, std::integral_constant<int, 1>{});
+    if (t + 2 >= nt) break;
+    step(t + 2, std::integral_constant<int, 2>{});
+    if constexpr (NSTAGE > 3) {
+      if (t + 3 >= nt) break;
+      step(t + 3, std::integral_constant<int, 3>{});
+    }
   }
 
   // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0.

@@ -1439,12 +1439,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
     }
     if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv) || (win >= 0 && (r0 + 31 - kbs > win || kbs + 31 - r0 > win))) {
+      // keys the lane's row keeps: lo <= kv <= hi; register r holds key kbs + 4hh + c(r), c(r) = 8 (r / 4) + r % 4,
+      // so one comparison of a constant with a per-lane bound decides each logit
+      int hi = p.causal ? qrow : (win >= 0 ? qrow + win : s.n_kv - 1);
+      hi = hi < s.n_kv - 1 ? hi : s.n_kv - 1;
+      const int hi_rel = hi - kbs - 4 * hh;
+      if (win < 0) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const int dist = kv > qrow ? kv - qrow : qrow - kv;
-        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow) && (win < 0 || dist <= win);
-        u[r] = keep ? u[r] : 0.f;
+        for (int r = 0; r < 16; ++r) u[r] = (8 * (r >> 2) + (r & 3)) <= hi_rel ? u[r] : 0.f;
+      } else {
+        const int lo_rel = qrow - win - kbs - 4 * hh;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c = 8 * (r >> 2) + (r & 3);
+          u[r] = (c <= hi_rel && c >= lo_rel) ? u[r] : 0.f;
+        }
       }
     }
     if (SEG) {

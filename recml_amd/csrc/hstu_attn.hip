@@ -2046,12 +2046,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     }
     // f'(0) is not 0: masked pairs are cleared after the activation's derivative
     if ((p.causal && kbs + 31 > r0) || (kbs + 32 > s.n_kv) || (win >= 0 && (r0 + 31 - kbs > win || kbs + 31 - r0 > win))) {
+      // lo <= kv <= hi for the lane's row; register r holds key kbs + 4hh + c(r), c(r) = 8 (r / 4) + r % 4
+      int hi = p.causal ? qrow : (win >= 0 ? qrow + win : s.n_kv - 1);
+      hi = hi < s.n_kv - 1 ? hi : s.n_kv - 1;
+      const int hi_rel = hi - kbs - 4 * hh;
+      const int lo_rel = win >= 0 ? qrow - win - kbs - 4 * hh : -1;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int kv = kbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const int dist = kv > qrow ? kv - qrow : qrow - kv;
-        const bool keep = (kv < s.n_kv) && (!p.causal || kv <= qrow) && (win < 0 || dist <= win);
-        ds[r] = keep ? ds[r] : 0.f;
+        const int c = 8 * (r >> 2) + (r & 3);
+        ds[r] = (c <= hi_rel && c >= lo_rel) ? ds[r] : 0.f;
       }
     }
     if (SEG) {
@@ -2554,11 +2557,16 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
     // rows past the sequence hold a repeat of the last row: they are masked like the rest
     if ((p.causal && qbs < r0 + 31) || (qbs + 32 > s.n_q) || (r0 + 32 > s.n_kv) ||
         (win >= 0 && (qbs + 31 - r0 > win || r0 + 31 - qbs > win))) {
+      // lo <= qi <= hi for the lane's key; register r holds row qbs + 4hh + c(r), c(r) = 8 (r / 4) + r % 4
+      int lo = p.causal ? kcol : (win >= 0 ? kcol - win : 0);
+      lo = kcol < s.n_kv ? lo : 0x3fffffff;          // a key past the sequence keeps nothing
+      int hi = win >= 0 ? kcol + win : s.n_q - 1;
+      hi = hi < s.n_q - 1 ? hi : s.n_q - 1;
+      const int lo_rel = lo - qbs - 4 * hh, hi_rel = hi - qbs - 4 * hh;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int qi = qbs + 8 * (r >> 2) + 4 * hh + (r & 3);
-        const int dist = qi > kcol ? qi - kcol : kcol - qi;
-        const bool keep = (qi < s.n_q) && (kcol < s.n_kv) && (!p.causal || kcol <= qi) && (win < 0 || dist <= win);
+        const int c = 8 * (r >> 2) + (r & 3);
+        const bool keep = c >= lo_rel && c <= hi_rel;
         pv[r] = keep ? pv[r] : 0.f;
         ds[r] = keep ? ds[r] : 0.f;
       }

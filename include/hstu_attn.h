@@ -176,9 +176,11 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
  * (or passes null when the table gradient is not wanted).  fp32 or bf16
  * storage, every option of the forward, fp32 arithmetic; fp8 q/k is not
  * supported.  bf16 calls that meet the conditions of the
- * matrix-core forward, ask for no table gradient, pass 16-byte aligned
- * gradient buffers and bring the workspace run on the matrix cores instead
- * (bf16 products, fp32 accumulation); hstu_attn_bwd_variant tells which.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which
+ * matrix-core forward (without a dense mask or bias, and with keys and
+ * queries of one length), pass 16-byte aligned gradient buffers and bring
+ * the workspace run on the matrix cores instead (bf16 products, fp32
+ * accumulation, table gradients included); hstu_attn_bwd_variant tells
+ * which.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which
  * the reference reaches through jax.custom_vjp (hstu_ops.py:551-826), extended
  * by the table gradients that jax derives for recml/layers/keras/hstu.py:91-113,
  * 190-221. */

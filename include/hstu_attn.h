@@ -1,6 +1,6 @@
 /*
- * hstu_attn.h -- C ABI of the MI355X (gfx950) HSTU pointwise-SiLU attention
- * forward.
+ * hstu_attn.h -- C ABI of the MI355X (gfx950) HSTU pointwise-SiLU attention:
+ * the forward (below) and its backward (hstu_attn_bwd).
  *
  *   S[b,h,i,j] = alpha * sum_c q[b,i,h,c] k[b,j,h,c]
  *                (+ pos_tab[h|0][(L-1)+j-i]) (+ ts_tab[h|0][bucket(dt)])

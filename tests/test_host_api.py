@@ -38,3 +38,22 @@ def test_no_cpu_path():
     recml_amd.hstu_attention(z, z, z)
   with pytest.raises(TypeError):
     recml_amd.hstu_attention(np.zeros((1, 4, 1, 32)), z, z)
+
+
+def test_bench_refuses_more_than_one_gpu():
+  import subprocess
+  import sys
+  root = os.path.dirname(HERE)
+  res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, cwd=root)
+  assert res.returncode != 0
+  assert "one GPU" in (res.stderr + res.stdout)
+
+
+def test_product_package_does_not_use_the_oracle():
+  # the oracle is test infrastructure: nothing under recml_amd/ may import it
+  pkg = os.path.join(os.path.dirname(HERE), "recml_amd")
+  for dirpath, _, files in os.walk(pkg):
+    for name in files:
+      if name.endswith(".py"):
+        text = open(os.path.join(dirpath, name)).read()
+        assert "import oracle" not in text and "from oracle" not in text, os.path.join(dirpath, name)

@@ -351,12 +351,19 @@ def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
   if bias is not None:
     s = s + np.asarray(bias, dtype=dtype)[:, None]
   p = silu(s) / n
-  m = splash_mask(L, Lkv, causal=causal,
-                  explicit=None if (mask is None or np.ndim(mask) == 3) else mask,
+  # The explicit mask is one more factor of M here (the C ABI's meaning), for [L,Lkv] and [B,L,Lkv]
+  # alike; splash_mask's own `explicit` argument is the reference's mask_type array, which stands
+  # in place of the causal / full choice, and callers that mean that pass causal=False.
+  m = splash_mask(L, Lkv, causal=causal, explicit=None,
                   sliding_window_size=sliding_window_size,
                   q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids)
-  if mask is not None and np.ndim(mask) == 3:
-    m = m & np.asarray(mask).astype(bool)
+  if mask is not None:
+    mk = np.asarray(mask).astype(bool)
+    if mk.shape[-2:] != (L, Lkv):
+      raise ValueError(
+          f"Mask shape {mk.shape} does not match query and key length"
+          f" ({L}, {Lkv}).")
+    m = m & (mk if mk.ndim == 3 else mk[None])
   if seq_lens is not None:
     lens = np.asarray(seq_lens)
     vq = np.arange(L)[None, :] < lens[:, None]
@@ -396,12 +403,19 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
     s = s + tb.astype(dtype)
   if bias is not None:
     s = s + np.asarray(bias, dtype=dtype)[:, None]
-  m = splash_mask(L, Lkv, causal=causal,
-                  explicit=None if (mask is None or np.ndim(mask) == 3) else mask,
+  # The explicit mask is one more factor of M here (the C ABI's meaning), for [L,Lkv] and [B,L,Lkv]
+  # alike; splash_mask's own `explicit` argument is the reference's mask_type array, which stands
+  # in place of the causal / full choice, and callers that mean that pass causal=False.
+  m = splash_mask(L, Lkv, causal=causal, explicit=None,
                   sliding_window_size=sliding_window_size,
                   q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids)
-  if mask is not None and np.ndim(mask) == 3:
-    m = m & np.asarray(mask).astype(bool)
+  if mask is not None:
+    mk = np.asarray(mask).astype(bool)
+    if mk.shape[-2:] != (L, Lkv):
+      raise ValueError(
+          f"Mask shape {mk.shape} does not match query and key length"
+          f" ({L}, {Lkv}).")
+    m = m & (mk if mk.ndim == 3 else mk[None])
   if seq_lens is not None:
     lens = np.asarray(seq_lens)
     vq = np.arange(L)[None, :] < lens[:, None]

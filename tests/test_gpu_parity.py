@@ -737,3 +737,60 @@ def test_matrix_core_forward_on_random_option_mixes(gpu, seed):
   assert not edge.any() or err[edge].max() <= 1e-1, (c, err[edge].max())
   for b in range(B):
     assert (out[b, lens[b]:] == 0).all()
+
+
+@pytest.mark.parametrize("seed", list(range(3000, 3016)))
+def test_matrix_core_forward_on_random_dense_and_cross_length_mixes(gpu, seed):
+  """bf16 forward against the oracle over random mixes of dense mask / dense bias (shared or per
+  sequence), different key and query lengths, causal / full, window, lengths, head dim and heads
+  (fixed seeds; every mix stays on the matrix-core kernel)."""
+  rng = np.random.default_rng(seed)
+  B = int(rng.integers(1, 5))
+  H = int(rng.choice([1, 2, 3, 4, 8]))
+  d = int(rng.choice([32, 64, 128]))
+  Lq = 16 * int(rng.integers(1, 40))
+  cross = rng.random() < 0.4
+  Lk = 16 * int(rng.integers(1, 40)) if cross else Lq
+  use_mask = rng.random() < 0.6
+  use_bias = rng.random() < 0.6
+  if not (use_mask or use_bias or cross):
+    use_bias = True
+  causal = bool(rng.random() < 0.5)
+  window = int(rng.integers(0, 200)) if rng.random() < 0.3 else None
+  q = O.round_bf16(rng.standard_normal((B, Lq, H, d)).astype(np.float32) * 0.3)
+  k = O.round_bf16(rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.3)
+  v = O.round_bf16(rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.3)
+  kw, gk = dict(causal=causal), dict(causal=causal)
+  if window is not None:
+    kw["sliding_window_size"] = gk["sliding_window_size"] = window
+  if use_mask:
+    batched = rng.random() < 0.5
+    m = rng.random((B, Lq, Lk) if batched else (Lq, Lk)) < rng.choice([0.1, 0.5, 0.9])
+    if rng.random() < 0.3:
+      m[..., : Lq // 2, :] = False          # whole tiles masked out: the kernel skips their blocks
+    kw["mask"] = m
+    gk["mask"] = _dev(m.astype(np.uint8))
+  if use_bias:
+    batched = rng.random() < 0.5 and B > 1
+    bias = (rng.standard_normal((B, Lq, Lk) if batched else (1, Lq, Lk)) * 0.5).astype(np.float32)
+    kw["bias"] = bias
+    gk["bias"] = _dev(bias)
+  lens = None
+  if not cross and rng.random() < 0.5:
+    lens = rng.integers(1, Lq + 1, B).astype(np.int32)
+    kw["seq_lens"] = lens
+    gk["seq_lens"] = _dev(lens)
+  case = dict(seed=seed, B=B, H=H, d=d, Lq=Lq, Lk=Lk, mask=use_mask, bias=use_bias, causal=causal, window=window, lens=lens)
+  bf = torch.bfloat16
+  out = torch.full((B, Lq, H, d), float("nan"), dtype=bf, device="cuda:0")
+  a, keep = hstu_ops.build_args(_dev(q, bf), _dev(k, bf), _dev(v, bf), out, n=Lq, alpha=0.2, **gk)
+  assert hstu_ops.kernel_variant(a) == "hstu_fwd_mfma_bf16", case
+  hstu_ops._run(a, keep)
+  torch.cuda.synchronize()
+  ref = O.hstu_attention_ref(q, k, v, n=Lq, alpha=0.2, dtype=np.float32, **kw)
+  got = out.float().cpu().numpy()
+  assert np.isfinite(got).all(), case
+  assert _err(got, ref) <= BF16_TOL, (case, _err(got, ref))
+  if lens is not None:
+    for b in range(B):
+      assert (got[b, lens[b]:] == 0).all(), case

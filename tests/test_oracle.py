@@ -257,6 +257,15 @@ def test_explicit_mask_and_window():
   m = np.tril(np.ones((6, 6), dtype=bool))
   np.testing.assert_array_equal(O.hstu_attention_ref(q, k, v, causal=False, mask=m),
                                 O.hstu_attention_ref(q, k, v, causal=True))
+  # an explicit mask is one more factor of M, whatever its rank: with the causal flag on top, a mask that keeps
+  # exactly the pairs above the diagonal leaves nothing, one that keeps everything leaves the causal result
+  upper = np.triu(np.ones((6, 6), dtype=bool), 1)
+  assert not O.hstu_attention_ref(q, k, v, causal=True, mask=upper).any()
+  assert not O.hstu_attention_ref(q, k, v, causal=True, mask=upper[None]).any()
+  np.testing.assert_array_equal(O.hstu_attention_ref(q, k, v, causal=True, mask=np.ones((6, 6), dtype=bool)),
+                                O.hstu_attention_ref(q, k, v, causal=True))
+  dq, dk, dv, _, _ = O.hstu_attention_bwd_ref(q, k, v, np.ones_like(v), causal=True, mask=upper)
+  assert not dq.any() and not dk.any() and not dv.any()
   w = O.hstu_attention_ref(q, k, v, sliding_window_size=0)
   s = np.einsum("bthd,bthd->bth", q, k)
   np.testing.assert_allclose(w, (O.silu(s) / 6)[..., None] * v, rtol=1e-13)

@@ -794,3 +794,74 @@ def test_matrix_core_forward_on_random_dense_and_cross_length_mixes(gpu, seed):
   if lens is not None:
     for b in range(B):
       assert (got[b, lens[b]:] == 0).all(), case
+
+
+@pytest.mark.parametrize("seed", list(range(4000, 4016)))
+def test_general_kernel_on_random_option_mixes(gpu, seed):
+  """fp32 storage (the general kernel) against the oracle over random mixes of every option at once: lengths or
+  segment ids, explicit mask, dense bias, both table biases, window, causal / full, different key and query
+  lengths, odd head dims (fixed seeds)."""
+  rng = np.random.default_rng(seed)
+  B = int(rng.integers(1, 4))
+  H = int(rng.integers(1, 4))
+  d = int(rng.choice([8, 24, 32, 48, 72]))
+  dv = d if rng.random() < 0.7 else int(rng.choice([8, 40]))
+  Lq = int(rng.integers(1, 90))
+  cross = rng.random() < 0.3
+  Lk = int(rng.integers(1, 90)) if cross else Lq
+  causal = bool(rng.random() < 0.5)
+  q = rng.standard_normal((B, Lq, H, d)).astype(np.float32) * 0.5
+  k = rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.5
+  v = rng.standard_normal((B, Lk, H, dv)).astype(np.float32) * 0.5
+  kw, gk = dict(causal=causal), dict(causal=causal)
+  if rng.random() < 0.4:
+    kw["sliding_window_size"] = gk["sliding_window_size"] = int(rng.integers(0, 40))
+  if rng.random() < 0.5:
+    batched = rng.random() < 0.5
+    m = rng.random((B, Lq, Lk) if batched else (Lq, Lk)) < 0.6
+    kw["mask"], gk["mask"] = m, _dev(m.astype(np.uint8))
+  if rng.random() < 0.5:
+    batched = rng.random() < 0.5 and B > 1
+    bias = (rng.standard_normal((B, Lq, Lk) if batched else (1, Lq, Lk)) * 0.5).astype(np.float32)
+    kw["bias"], gk["bias"] = bias, _dev(bias)
+  lens = None
+  if rng.random() < 0.35:
+    cq, ck = np.sort(rng.integers(0, Lq + 1, 2)), np.sort(rng.integers(0, Lk + 1, 2))
+    qs = np.tile(np.searchsorted(cq, np.arange(Lq), side="right").astype(np.int32), (B, 1))
+    ks = np.tile(np.searchsorted(ck, np.arange(Lk), side="right").astype(np.int32), (B, 1))
+    kw["q_segment_ids"], kw["kv_segment_ids"] = qs, ks
+    gk["q_segment_ids"], gk["kv_segment_ids"] = _dev(qs), _dev(ks)
+  elif not cross and rng.random() < 0.6:
+    lens = rng.integers(0, Lq + 1, B).astype(np.int32)
+    kw["seq_lens"], gk["seq_lens"] = lens, _dev(lens)
+  if not cross and rng.random() < 0.5:
+    heads = H if rng.random() < 0.5 else 1
+    kw["pos_tab"] = (rng.standard_normal((heads, 2 * Lq - 1)) * 0.3).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  t = None
+  if not cross and rng.random() < 0.5:
+    heads = H if rng.random() < 0.5 else 1
+    nb = int(rng.choice([16, 64, 128]))
+    kw["ts_tab"] = (rng.standard_normal((heads, nb + 1)) * 0.3).astype(np.float32)
+    t = 1_700_000_000 + np.cumsum(np.ceil(rng.exponential(3000.0, (B, Lq))), axis=1).astype(np.int64)
+    kw["timestamps"] = t
+    gk["ts_bias"], gk["timestamps"] = _dev(kw["ts_tab"]), _dev(t)
+  out = torch.full((B, Lq, H, dv), float("nan"), dtype=torch.float32, device="cuda:0")
+  a, keep = hstu_ops.build_args(_dev(q), _dev(k), _dev(v), out, n=7.0, alpha=0.3, **gk)
+  assert hstu_ops.kernel_variant(a) == "hstu_fwd_general<float>"
+  hstu_ops._run(a, keep)
+  torch.cuda.synchronize()
+  ref = O.hstu_attention_ref(q, k, v, n=7.0, alpha=0.3, **kw)
+  got = out.cpu().numpy()
+  case = dict(seed=seed, B=B, H=H, d=d, dv=dv, Lq=Lq, Lk=Lk, causal=causal, keys=sorted(kw))
+  assert np.isfinite(got).all(), case
+  err = np.abs(got - ref).max(axis=(2, 3)) / max(np.abs(ref).max(), 1e-30)
+  edge = np.zeros((B, Lq), bool)
+  if t is not None:
+    for b in range(B):
+      near = O.near_bucket_boundary(O.time_delta(t[b:b + 1])[0], 0.301)
+      edge[b] = near.any(1)
+  assert err[~edge].max(initial=0.0) <= FP32_TOL, (case, err[~edge].max(initial=0.0))
+  if lens is not None:
+    for b in range(B):
+      assert (got[b, lens[b]:] == 0).all(), case

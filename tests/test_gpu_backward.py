@@ -333,3 +333,72 @@ def test_matrix_core_backward_on_random_option_mixes(gpu, seed):
     assert (g is None) == (w is None), nm
     if g is not None:
       assert _rel(g.cpu().numpy().reshape(w.shape), w) <= tol, (nm, seed)
+
+
+@pytest.mark.parametrize("seed", list(range(5000, 5014)))
+def test_general_backward_on_random_option_mixes(gpu, seed):
+  """fp32 storage (the general backward) against the oracle over random mixes of the options the
+  matrix-core pair does not take: explicit mask, dense bias, keys and queries of different lengths,
+  odd head dims, together with lengths or segment ids, window and the table biases (fixed seeds)."""
+  rng = np.random.default_rng(seed)
+  B = int(rng.integers(1, 4))
+  H = int(rng.integers(1, 4))
+  d = int(rng.choice([8, 24, 32, 48]))
+  dv = d if rng.random() < 0.7 else int(rng.choice([8, 40]))
+  Lq = int(rng.integers(1, 70))
+  cross = rng.random() < 0.3
+  Lk = int(rng.integers(1, 70)) if cross else Lq
+  causal = bool(rng.random() < 0.5)
+  q = rng.standard_normal((B, Lq, H, d)).astype(np.float32) * 0.5
+  k = rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.5
+  v = rng.standard_normal((B, Lk, H, dv)).astype(np.float32) * 0.5
+  dout = rng.standard_normal((B, Lq, H, dv)).astype(np.float32) * 0.5
+  kw, gk = dict(causal=causal, n=7.0, alpha=0.3), dict(causal=causal, n=7.0, alpha=0.3)
+  if rng.random() < 0.4:
+    kw["sliding_window_size"] = gk["sliding_window_size"] = int(rng.integers(0, 40))
+  if rng.random() < 0.5:
+    m = rng.random((B, Lq, Lk) if rng.random() < 0.5 else (Lq, Lk)) < 0.6
+    kw["mask"], gk["mask"] = m, _dev(m)
+  if rng.random() < 0.5:
+    bias = (rng.standard_normal((B if rng.random() < 0.5 else 1, Lq, Lk)) * 0.5).astype(np.float32)
+    kw["bias"], gk["bias"] = bias, _dev(bias)
+  lens = None
+  if rng.random() < 0.35:
+    cq, ck = np.sort(rng.integers(0, Lq + 1, 2)), np.sort(rng.integers(0, Lk + 1, 2))
+    qs = np.tile(np.searchsorted(cq, np.arange(Lq), side="right").astype(np.int32), (B, 1))
+    ks = np.tile(np.searchsorted(ck, np.arange(Lk), side="right").astype(np.int32), (B, 1))
+    kw["q_segment_ids"], kw["kv_segment_ids"] = qs, ks
+    gk["q_segment_ids"], gk["kv_segment_ids"] = _dev(qs), _dev(ks)
+  elif not cross and rng.random() < 0.6:
+    lens = rng.integers(0, Lq + 1, B).astype(np.int32)
+    kw["seq_lens"], gk["seq_lens"] = lens, _dev(lens)
+  if not cross and rng.random() < 0.5:
+    kw["pos_tab"] = (rng.standard_normal((H if rng.random() < 0.5 else 1, 2 * Lq - 1)) * 0.3).astype(np.float32)
+    gk["pos_bias"] = _dev(kw["pos_tab"])
+  t = None
+  if not cross and rng.random() < 0.5:
+    nb = int(rng.choice([16, 64, 128]))
+    kw["ts_tab"] = (rng.standard_normal((H if rng.random() < 0.5 else 1, nb + 1)) * 0.3).astype(np.float32)
+    t = 1_700_000_000 + np.cumsum(np.ceil(rng.exponential(3000.0, (B, Lq))), axis=1).astype(np.int64)
+    kw["timestamps"] = t
+    gk["ts_bias"], gk["timestamps"] = _dev(kw["ts_tab"]), _dev(t)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q), _dev(k), _dev(v), _dev(dout), _variant_out=variant, **gk)
+  torch.cuda.synchronize()
+  case = dict(seed=seed, B=B, H=H, d=d, dv=dv, Lq=Lq, Lk=Lk, causal=causal, keys=sorted(kw), variant=variant)
+  rows, cols = np.zeros((B, Lq), bool), np.zeros((B, Lk), bool)
+  if t is not None:
+    rows, cols = _boundary_flags(t, np.full((B,), Lq), False)
+  for nm, g, w, edge in zip(("dq", "dk", "dv"), got[:3], want[:3], (rows, cols, cols)):
+    g = g.cpu().numpy()
+    assert g.shape == w.shape and np.isfinite(g).all(), (nm, case)
+    err = np.abs(g - w).max(axis=(2, 3)) / max(np.abs(w).max(), 1e-30)
+    assert err[~edge].max(initial=0.0) <= 2e-5, (nm, case, err[~edge].max(initial=0.0))
+    if lens is not None:
+      for b in range(B):
+        assert (g[b, lens[b]:] == 0).all(), (nm, case)
+  for nm, g, w in (("dpos", got[3], want[3]), ("dts", got[4], want[4])):
+    assert (g is None) == (w is None), (nm, case)
+    if g is not None and not rows.any():
+      assert _rel(g.cpu().numpy().reshape(w.shape), w) <= 2e-5, (nm, case)

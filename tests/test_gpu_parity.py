@@ -148,6 +148,39 @@ def test_config3_full_size_bf16(gpu):
   assert np.isfinite(out).all()
 
 
+def _spot_check_jagged(w, q, k, v, out, pick, tol):
+  ref = oracle_workload(w, q, k, v, dtype=np.float32, sequences=pick)
+  scale = np.abs(ref).max()
+  for b in pick:
+    s, e = w.seq_offsets[b], w.seq_offsets[b + 1]
+    assert np.abs(out[s:e] - ref[s:e]).max() / scale <= tol, f"sequence {b}"
+  assert np.isfinite(out).all()
+
+
+def test_config4_attention_full_size_bf16(gpu):
+  # the attention call of the model configuration (B=128, L=1024, H=8, d=64, position bias only)
+  w = workloads.config4_attention()
+  q, k, v, out = run_workload(w, torch.bfloat16)
+  order = np.argsort(w.seq_lens)
+  _spot_check_jagged(w, q, k, v, out, [int(order[-1]), int(order[0]), int(order[len(order) // 2])], BF16_TOL)
+
+
+def test_config5_full_size_bf16_and_fp8(gpu):
+  # the long-sequence configuration (B=32, L=4096, H=8, d=128): bf16, then fp8 q / k against the oracle on
+  # exactly the dequantised values; oracle on the shortest and the median sequence
+  w = workloads.config5()
+  order = np.argsort(w.seq_lens)
+  pick = [int(order[0]), int(order[len(order) // 2])]
+  q, k, v, out = run_workload(w, torch.bfloat16)
+  _spot_check_jagged(w, q, k, v, out, pick, BF16_TOL)
+  q8, qs, qd = _quant(w.q)
+  k8, ks, kd = _quant(w.k)
+  out8 = recml_amd.hstu_attention(q8, k8, _dev(v, torch.bfloat16), q_scale=qs, k_scale=ks, seq_offsets=_dev(w.seq_offsets),
+                                  max_len=w.L, n=w.n, alpha=w.alpha, pos_bias=_dev(w.pos_tab))
+  torch.cuda.synchronize()
+  _spot_check_jagged(w, qd.astype(np.float32), kd.astype(np.float32), v, out8.float().cpu().numpy(), pick, BF16_TOL)
+
+
 @pytest.mark.parametrize("d", [32, 64, 128])
 @pytest.mark.parametrize("causal", [True, False])
 def test_mfma_head_dims_and_full_mask(gpu, d, causal):

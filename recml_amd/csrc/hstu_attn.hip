@@ -613,9 +613,10 @@ __global__ __launch_bounds__(256) void hstu_bwd_dkv(const Params p) {
 // One workgroup = 4 wavefronts = 128 query rows (32 per wavefront); two
 // workgroups per CU, i.e. two wavefronts per SIMD, so that one wavefront's
 // MFMAs can run while the other's SiLU arithmetic does.  Keys are streamed 32
-// at a time through a 4-stage LDS ring filled by direct global->LDS loads that
-// are issued three steps ahead (no staging registers, ~48 KB in flight per
-// workgroup).
+// at a time through a 4-stage LDS ring filled by direct global->LDS loads (no
+// staging registers): at d = 128 two steps at a time, one pair ahead, with one
+// barrier per pair (32-48 KB in flight per workgroup); with dense operands
+// three steps ahead, one barrier per step; at d <= 64 a 3-stage ring, two ahead.
 //
 //   S^T[kv, q] = K Q^T   A = K fragment (LDS, 16-byte reads), B = Q (registers)
 //   O^T[dv, q] = V^T P^T A = V fragment (LDS transpose reads), B = P (registers)
@@ -1246,7 +1247,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   };
 
   // prologue: the scaled bucket table (64 entries per wave, the last wave repeats the first), then
-  // three steps in flight before the first block
+  // the first steps in flight before the first block (two when the loop runs in pairs, else NSTAGE - 1)
   if (TS) {
     const int c = w < 3 ? w : 0;
     const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
@@ -1292,8 +1293,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     asm volatile("" ::"v"(tq), "v"(tq32));
   }
 
+  // With a four-stage ring and no dense operands the step loop below runs in pairs of steps: only
+  // the first pair is in flight before it (d = 128: 68.8 -> 64.9 us on the headline shape, 2-3 % on
+  // full-length batches).  Dense operands bring five to ten more loads per step and lose by pairs
+  // (490 -> 556 us), and so does a fourth stage bought for them at d <= 64 (110 -> 116 us).
+  constexpr bool PAIRS = NSTAGE == 4 && DENSE == 0;
   if (t_lo + 1 < nt) dma_step(t_lo + 1, std::integral_constant<int, 1>{});
-  if constexpr (NSTAGE > 3) {
+  if constexpr (NSTAGE > 3 && !PAIRS) {
     if (t_lo + 2 < nt) dma_step(t_lo + 2, std::integral_constant<int, 2>{});
   }
 
@@ -1507,28 +1513,53 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     else HSTU_WAIT_VMCNT(0);
   };
 
-  wait_step(t_lo);
-  __syncthreads();
-
-  // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
-  // which now receives step t+3; the block of step t is computed; then every
-  // wave makes sure its share of step t+1 has landed before the next barrier.
-  auto step = [&](int t, auto st_) {
-    constexpr int st = decltype(st_)::value;
-    if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1, std::integral_constant<int, (st + NSTAGE - 1) % NSTAGE>{});
-    if (t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0)) block(t, st_);
-    if (t + 1 < nt) wait_step(t + 1);
+  const auto live = [&](int t) { return t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0); };
+  if constexpr (PAIRS) {
+    // Steps in pairs, one barrier per pair.  The barrier that ended the pair (t-2, t-1) freed that
+    // pair's two ring stages, which now receive steps t+2 and t+3; the blocks of steps t and t+1
+    // are computed; then every wave makes sure that its share of the next pair has landed.  Between
+    // two barriers the waves of a workgroup drift apart by up to two blocks, which the diagonal
+    // tiles (where wave i has i+1 blocks to do) and the direct loads' issue stalls both use.
+    HSTU_WAIT_VMCNT(0);
     __syncthreads();
-  };
-  for (int t = t_lo; t < nt; t += NSTAGE) {
-    step(t, std::integral_constant<int, 0>{});
-    if (t + 1 >= nt) break;
-    step(t + 1, std::integral_constant<int, 1>{});
-    if (t + 2 >= nt) break;
-    step(t + 2, std::integral_constant<int, 2>{});
-    if constexpr (NSTAGE > 3) {
-      if (t + 3 >= nt) break;
-      step(t + 3, std::integral_constant<int, 3>{});
+    auto pair = [&](int t, auto st_) {
+      constexpr int st = decltype(st_)::value;
+      if (t + 2 < nt) dma_step(t + 2, std::integral_constant<int, (st + 2) % NSTAGE>{});
+      if (t + 3 < nt) dma_step(t + 3, std::integral_constant<int, (st + 3) % NSTAGE>{});
+      if (live(t)) block(t, st_);
+      if (t + 1 < nt && live(t + 1)) block(t + 1, std::integral_constant<int, (st + 1) % NSTAGE>{});
+      HSTU_WAIT_VMCNT(0);
+      __syncthreads();
+    };
+    for (int t = t_lo; t < nt; t += NSTAGE) {
+      pair(t, std::integral_constant<int, 0>{});
+      if (t + 2 >= nt) break;
+      pair(t + 2, std::integral_constant<int, 2>{});
+    }
+  } else {
+    wait_step(t_lo);
+    __syncthreads();
+
+    // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
+    // which now receives step t+NSTAGE-1; the block of step t is computed; then every
+    // wave makes sure its share of step t+1 has landed before the next barrier.
+    auto step = [&](int t, auto st_) {
+      constexpr int st = decltype(st_)::value;
+      if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1, std::integral_constant<int, (st + NSTAGE - 1) % NSTAGE>{});
+      if (live(t)) block(t, st_);
+      if (t + 1 < nt) wait_step(t + 1);
+      __syncthreads();
+    };
+    for (int t = t_lo; t < nt; t += NSTAGE) {
+      step(t, std::integral_constant<int, 0>{});
+      if (t + 1 >= nt) break;
+      step(t + 1, std::integral_constant<int, 1>{});
+      if (t + 2 >= nt) break;
+      step(t + 2, std::integral_constant<int, 2>{});
+      if constexpr (NSTAGE > 3) {
+        if (t + 3 >= nt) break;
+        step(t + 3, std::integral_constant<int, 3>{});
+      }
     }
   }
 

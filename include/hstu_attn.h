@@ -165,6 +165,26 @@ size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
  * recml/layers/keras/hstu.py:356-390. */
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
 
+/* Bytes of the scratch array built into the library that hstu_attn_fwd_noalloc
+ * uses in place of a caller workspace (one copy per GPU the library runs on,
+ * held until the process ends). */
+#define HSTU_ATTN_NOALLOC_SCRATCH_BYTES (4u << 20)
+
+/* hstu_attn_fwd for callers that cannot allocate device memory at all: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference (its op is a pure function under
+ * jax.jit and XLA owns every buffer).  Same arguments, kernels and results as
+ * hstu_attn_fwd, except that args->workspace / workspace_bytes are ignored:
+ * the scratch that call would need (hstu_attn_fwd_workspace_bytes) lives in
+ * a fixed array of HSTU_ATTN_NOALLOC_SCRATCH_BYTES inside the library.  The
+ * call allocates and frees nothing, on the device or through any library.
+ * Calls whose scratch need exceeds the array return HSTU_ERR_WORKSPACE (use
+ * hstu_attn_fwd with a caller buffer then).  Every call on a GPU shares that
+ * GPU's array: calls that overlap on one GPU (two streams, two threads) race;
+ * HSTU_FWD_WORKSPACE_PREPARED refers to what the previous call of this entry
+ * point on the same GPU prepared. */
+int hstu_attn_fwd_noalloc(const HstuAttnFwdArgs* args, void* stream);
+
 /* Backward of the same op: gradients of sum(out * dout) with respect to q, k, v
  * and the two bias tables.  `fwd` describes the forward call (its `out` is
  * not used; its `workspace`, sized by hstu_attn_fwd_workspace_bytes, is

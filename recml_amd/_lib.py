@@ -14,12 +14,14 @@ ABI_VERSION = 1
 LAYOUT_PADDED, LAYOUT_JAGGED = 0, 1
 DTYPE_FP32, DTYPE_BF16, DTYPE_FP8_E4M3FN = 0, 1, 2
 FWD_WORKSPACE_PREPARED = 1
+NOALLOC_SCRATCH_BYTES = 4 << 20   # HSTU_ATTN_NOALLOC_SCRATCH_BYTES
 MASK_NONE, MASK_LENGTH, MASK_SEGMENT = 0, 1, 2
 
 EXPORTS = (
     "hstu_attn_abi_version",
     "hstu_attn_fwd_workspace_bytes",
     "hstu_attn_fwd",
+    "hstu_attn_fwd_noalloc",
     "hstu_attn_last_error",
     "hstu_attn_fwd_variant",
     "hstu_attn_bwd",
@@ -98,6 +100,8 @@ def load():
     lib.hstu_attn_fwd_workspace_bytes.argtypes = [C.POINTER(HstuAttnFwdArgs)]
     lib.hstu_attn_fwd.restype = C.c_int
     lib.hstu_attn_fwd.argtypes = [C.POINTER(HstuAttnFwdArgs), C.c_void_p]
+    lib.hstu_attn_fwd_noalloc.restype = C.c_int
+    lib.hstu_attn_fwd_noalloc.argtypes = [C.POINTER(HstuAttnFwdArgs), C.c_void_p]
     lib.hstu_attn_last_error.restype = C.c_char_p
     lib.hstu_attn_last_error.argtypes = []
     lib.hstu_attn_fwd_variant.restype = C.c_char_p

@@ -3078,6 +3078,33 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
 
 }  // namespace
 
+// Scratch of hstu_attn_fwd_noalloc: the workspace of a forward call, built into the library so that
+// the call needs no allocation.  In host code this name is only a handle for hipGetSymbolAddress;
+// each GPU holds its own copy at its own address.
+static __device__ __align__(256) unsigned char scratch[HSTU_ATTN_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+// Device address of `scratch` on the current GPU, looked up once per device.
+int scratch_of_current_device(void** out) {
+  constexpr int kMaxDev = 64;
+  static void* ptrs[kMaxDev];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDev) return fail(HSTU_ERR_LAUNCH, "device index %d beyond the %d this library keeps scratch for", dev, kMaxDev);
+  void* ptr = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return fail(HSTU_ERR_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    __atomic_store_n(&ptrs[dev], ptr, __ATOMIC_RELEASE);   // two threads racing here store the same address
+  }
+  *out = ptr;
+  return HSTU_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 int hstu_attn_abi_version(void) { return HSTU_ATTN_ABI_VERSION; }
@@ -3130,6 +3157,25 @@ int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {
   hipStream_t st = (hipStream_t)stream;
   if (bwd_mfma_eligible(args)) return launch_bwd_mfma(args, p, st);
   return f->qk_dtype == HSTU_DTYPE_FP32 ? launch_bwd<float>(p, st) : launch_bwd<bf16_t>(p, st);
+}
+
+int hstu_attn_fwd_noalloc(const HstuAttnFwdArgs* args, void* stream) {
+  int rc = validate(args);
+  if (rc != HSTU_OK) return rc;
+  HstuAttnFwdArgs a = *args;
+  a.workspace = nullptr;
+  a.workspace_bytes = 0;
+  const size_t need = plan_workspace(&a).total();
+  if (need > (size_t)HSTU_ATTN_NOALLOC_SCRATCH_BYTES)
+    return fail(HSTU_ERR_WORKSPACE, "this call needs %zu bytes of scratch, the array built into the library holds %zu: "
+                "use hstu_attn_fwd with a caller workspace", need, (size_t)HSTU_ATTN_NOALLOC_SCRATCH_BYTES);
+  if (need) {
+    void* ptr = nullptr;
+    if ((rc = scratch_of_current_device(&ptr)) != HSTU_OK) return rc;
+    a.workspace = ptr;
+    a.workspace_bytes = HSTU_ATTN_NOALLOC_SCRATCH_BYTES;
+  }
+  return hstu_attn_fwd(&a, stream);
 }
 
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {

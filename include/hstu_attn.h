@@ -225,6 +225,20 @@ const char* hstu_attn_bwd_variant(const HstuAttnBwdArgs* args);
 /* Message for the last non-zero status on this thread ("" if none). */
 const char* hstu_attn_last_error(void);
 
+/* The timestamp bucket law every kernel here follows, as integer thresholds:
+ *   bucket(dt) = min(floor(ln(fl32(clip(|dt|, 1, 1e9))) / bucket_size), ts_num_buckets)
+ * -- recml/layers/keras/hstu.py:48-55 (float log and divide of the clipped
+ * difference, truncated) with the logarithm and the quotient taken in double,
+ * bucket_size being the float the caller passes.  thresholds[b], b < count,
+ * receives the smallest clipped |dt| whose bucket (before the clip to
+ * ts_num_buckets) is >= b, INT32_MAX where 1e9 does not reach b; thresholds[0]
+ * is 1.  Host-only (no GPU work).  Returns the number of buckets 1e9 reaches
+ * (its own bucket + 1), or a negative HstuStatus.  The reference evaluates
+ * the same expression in float inside XLA; within a few hundred of a
+ * threshold at the top of the range its rounding may differ, which no test
+ * of the reference pins. */
+int hstu_attn_bucket_thresholds(float bucket_size, int32_t* thresholds, int count);
+
 /* Name of the kernel variant hstu_attn_fwd would launch for `args`
  * (diagnostics for profiles and benchmarks; static storage). */
 const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args);

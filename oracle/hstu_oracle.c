@@ -8,7 +8,7 @@
  * Follows, per output row i of sequence b and head h:
  *   s_j  = alpha * <q_i, k_j>                      recml/layers/keras/hstu.py:365-371
  *        + pos_tab[(L-1) + j - i]                  hstu.py:91-113 (closed form)
- *        + ts_tab[clip(trunc(logf(clip(|ts[i+1]-ts[j]|,1,1e9)) / size), 0, nb)]
+ *        + ts_tab[clip(floor(log(fl32(clip(|ts[i+1]-ts[j]|,1,1e9))) / size), 0, nb)]   (log, divide in double)
  *                                                  hstu.py:33-55, 190-221
  *   p_j  = s_j * sigmoid(s_j) * inv_n              hstu.py:376-378
  *   keep j <= i (causal), j < n_b, i < n_b         recml/layers/keras/utils.py:29-41
@@ -45,7 +45,9 @@ static int bucket_of(int64_t dt, float size, int nb) {
   if (dt < 0) dt = -dt;
   if (dt < 1) dt = 1;
   if (dt > 1000000000LL) dt = 1000000000LL;
-  float lg = logf((float)dt) / size;
+  /* the bucket law: the reference's float log and divide (hstu.py:48-55) taken in double on the
+   * float-rounded difference and the float bucket size; the kernels follow it exactly */
+  double lg = log((double)(float)dt) / (double)size;
   int b = (int)lg;
   return b < 0 ? 0 : (b > nb ? nb : b);
 }

@@ -43,11 +43,16 @@ How each function is pinned (tests/test_oracle.py):
                                 (|i-j| <= w) comes from jax's splash-attention
                                 LocalMask, which is not vendored in the
                                 reference and cannot be run here.
-  default_bucketization at bucket boundaries  parity unpinned: the reference
-                                computes log and the divide in fp32 inside
-                                XLA; integers adjacent to e^(0.301 k) can land
-                                on either side.  `bucket_boundary_set` lists
-                                them; `bucketize_law` is the fp64 definition.
+  default_bucketization at bucket boundaries  parity unpinned against the
+                                reference: it computes log and the divide in
+                                fp32 inside XLA, and integers next to
+                                e^(0.301 k) can land on either side there.
+                                `bucketize_law` (the same expression with log
+                                and divide in fp64) is the definition every
+                                kernel and every reference output here follows
+                                exactly; `bucket_thresholds` are its integer
+                                thresholds, `bucket_boundary_set` lists where
+                                the literal fp32 recipe may differ from it.
 """
 
 from __future__ import annotations
@@ -73,29 +78,45 @@ def default_bucketization(delta, bucket_size: float = 0.301):
   return b.astype(np.int64)  # C-style truncation; values are >= 0
 
 
-def bucketize_law(delta, bucket_size: float = 0.301):
-  """The same law in fp64 on the fp32-rounded clipped |delta|.
+def _law_size(bucket_size) -> float:
+  """The bucket size as the float32 the reference's fp32 divide sees, widened to double."""
+  return float(np.float32(bucket_size))
 
-  This is the definition the kernel is held to away from the boundary set:
-  floor(ln(fl32(clip(|x|,1,1e9))) / bucket_size).
+
+def bucketize_law(delta, bucket_size: float = 0.301):
+  """THE bucket law: recml/layers/keras/hstu.py:48-55 with log and divide taken in fp64.
+
+    floor(ln(fl32(clip(|x|, 1, 1e9))) / fl32(bucket_size))
+
+  The reference casts the clipped integer to float32, takes a float32 log and
+  divides by the float32 bucket size; only the last two roundings are replaced
+  by fp64 here, which turns the law into a set of integer thresholds
+  (`bucket_thresholds`).  Every kernel and every reference output in this
+  repository follows it exactly, bucket boundaries included.
   """
   x = np.abs(np.asarray(delta).astype(np.int64))
   x = np.clip(x, 1, int(1e9)).astype(np.float32).astype(np.float64)
-  return np.floor(np.log(x) / float(bucket_size)).astype(np.int64)
+  return np.floor(np.log(x) / _law_size(bucket_size)).astype(np.int64)
 
 
-def bucket_thresholds(bucket_size: float = 0.301, x_max: float = 1e9):
-  """T_k = smallest integer x with floor(ln(x)/bucket_size) >= k, k=0..kmax."""
-  kmax = int(math.floor(math.log(x_max) / bucket_size))
+def bucket_thresholds(bucket_size: float = 0.301, x_max: int = 10 ** 9):
+  """T_k = smallest integer x in [1, x_max] with bucketize_law(x) >= k, k = 0..bucketize_law(x_max).
+
+  Found by bisection on the law itself (it is monotone in x), so that
+  bucketize_law(x) == number of k >= 1 with T_k <= x by construction.
+  """
+  law = lambda x: int(bucketize_law(np.asarray([x]), bucket_size)[0])
+  kmax = law(x_max)
   out = []
   for k in range(kmax + 1):
-    t = int(math.ceil(math.exp(bucket_size * k)))
-    # fix up by direct evaluation of the law
-    while t > 1 and math.floor(math.log(t - 1) / bucket_size) >= k:
-      t -= 1
-    while math.floor(math.log(t) / bucket_size) < k:
-      t += 1
-    out.append(t)
+    lo, hi = 1, int(x_max)
+    while lo < hi:
+      mid = (lo + hi) // 2
+      if law(mid) >= k:
+        hi = mid
+      else:
+        lo = mid + 1
+    out.append(lo)
   return np.asarray(out, dtype=np.int64)
 
 
@@ -122,7 +143,7 @@ def near_bucket_boundary(delta, bucket_size: float = 0.301, ulps: float = 8.0):
   """True where ln(fl32(clip|delta|))/bucket_size is within `ulps` fp32 ulps of an integer."""
   x = np.abs(np.asarray(delta).astype(np.int64))
   x = np.clip(x, 1, int(1e9)).astype(np.float32).astype(np.float64)
-  y = np.log(x) / float(bucket_size)
+  y = np.log(x) / _law_size(bucket_size)
   dist = np.abs(y - np.rint(y))
   tol = ulps * np.spacing(np.maximum(y, 1.0).astype(np.float32)).astype(np.float64)
   return (dist <= tol) & (np.rint(y) >= 1)
@@ -182,10 +203,13 @@ def time_delta(ts):
 
 
 def time_bias(ts, ts_w, num_buckets: int = 128, bucket_size: float = 0.301,
-              law: bool = False):
+              law: bool = True):
   """recml/layers/keras/hstu.py:190-221.  ts [B,n] ints, ts_w [num_buckets+1].
 
   The reference's one-hot matmul with ts_w is a gather ts_w[bucket].
+  law=True (the default) buckets by `bucketize_law`, law=False by the literal
+  float32 recipe `default_bucketization`; the two differ only on the
+  enumerated boundary set.
   """
   d = time_delta(ts)
   fn = bucketize_law if law else default_bucketization
@@ -320,7 +344,7 @@ def _bias_term(L, Lkv, H, pos_tab, timestamps, ts_tab, ts_bucket_size, law):
 
 def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
                        causal=True, pos_tab=None, timestamps=None,
-                       ts_tab=None, ts_bucket_size=0.301, bucket_law=False,
+                       ts_tab=None, ts_bucket_size=0.301, bucket_law=True,
                        q_segment_ids=None, kv_segment_ids=None,
                        sliding_window_size=None, mask=None, bias=None,
                        dtype=np.float64):
@@ -376,7 +400,7 @@ def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
 
 def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
                            causal=True, pos_tab=None, timestamps=None,
-                           ts_tab=None, ts_bucket_size=0.301, bucket_law=False,
+                           ts_tab=None, ts_bucket_size=0.301, bucket_law=True,
                            q_segment_ids=None, kv_segment_ids=None,
                            sliding_window_size=None, mask=None, bias=None,
                            dtype=np.float64):
@@ -594,7 +618,7 @@ def attention_flops(seq_lens, H, d_qk, d_v):
 def hstu_attention_jagged_ref(q, k, v, seq_offsets, max_len, *, n=None,
                               alpha=1.0, causal=True, pos_tab=None,
                               timestamps=None, ts_tab=None,
-                              ts_bucket_size=0.301, bucket_law=False,
+                              ts_bucket_size=0.301, bucket_law=True,
                               dtype=np.float64, sequences=None):
   """The op on jagged [T,H,d] inputs, one sequence at a time.
 

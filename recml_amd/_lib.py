@@ -26,6 +26,7 @@ EXPORTS = (
     "hstu_attn_fwd_variant",
     "hstu_attn_bwd",
     "hstu_attn_bwd_variant",
+    "hstu_attn_bucket_thresholds",
 )
 
 
@@ -110,6 +111,8 @@ def load():
     lib.hstu_attn_bwd.argtypes = [C.POINTER(HstuAttnBwdArgs), C.c_void_p]
     lib.hstu_attn_bwd_variant.restype = C.c_char_p
     lib.hstu_attn_bwd_variant.argtypes = [C.POINTER(HstuAttnBwdArgs)]
+    lib.hstu_attn_bucket_thresholds.restype = C.c_int
+    lib.hstu_attn_bucket_thresholds.argtypes = [C.c_float, C.POINTER(C.c_int32), C.c_int]
     ver = lib.hstu_attn_abi_version()
     if ver != ABI_VERSION:
       raise RuntimeError(f"libhstu_attn.so has ABI {ver}, expected {ABI_VERSION}")

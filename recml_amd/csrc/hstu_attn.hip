@@ -45,6 +45,7 @@
 
 #include <hip/hip_runtime.h>
 #include <type_traits>
+#include <math.h>
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -87,8 +88,7 @@ struct Params {
   const int32_t* ts_ok;
   const int32_t* ts_rel;
   const int32_t* ts_range;
-  const float* ts_scaled;    // workspace: log2(e) * ts_tab as [heads][TS_TAB_LEN], indices past the last bucket repeat it
-  const int32_t* ts_thr;     // workspace: [TS_TAB_LEN] smallest |dt| that the kernel's bucket function puts in bucket >= b
+  const int4* ts_keyed;      // workspace: the bucket tables [heads][3 KB], see TsKeys
   const void* ws_base;       // start of the workspace (all of the above lie within 4 GB of it)
   const float* q_scale;      // [H] or null: dequantisation scales of fp8 q / k
   const float* k_scale;
@@ -98,7 +98,6 @@ struct Params {
   int32_t mask_batched, dense_bias_batched, pos_heads, ts_heads;
   int32_t ts_nb;
   float ts_bucket_size;
-  float ts_log2_scale;  // ln(2) / ts_bucket_size
   float alpha, inv_n;
   int32_t n_qtiles;
   // Key-range splitting (MFMA kernel; off when split_steps == 0): a query tile with more than
@@ -210,8 +209,9 @@ __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
     if (dt < 0) dt = -dt;
     if (dt < 1) dt = 1;
     if (dt > 1000000000LL) dt = 1000000000LL;
-    // fp32 log then fp32 divide then truncation, as the dense layer does it
-    float lg = logf((float)dt) / p.ts_bucket_size;
+    // the bucket law: floor(ln(fl32(|dt|)) / size), evaluated in double so that every |dt| falls on the
+    // side of a bucket boundary that the law's integer thresholds (bucket_law below) put it on
+    const double lg = log((double)(float)dt) / (double)p.ts_bucket_size;
     int bk = (int)lg;
     bk = bk < 0 ? 0 : (bk > p.ts_nb ? p.ts_nb : bk);
     if (bucket) *bucket = bk;
@@ -634,7 +634,32 @@ constexpr int NSTAGE = 4;     // LDS ring depth
 constexpr int MFMA_THREADS = 256;
 constexpr int NWAVES = MFMA_THREADS / 64;
 constexpr int POS_PAD = 256;  // zero margin on both sides of the scaled position table
-constexpr int TS_TAB_LEN = 192;  // entries of the scaled bucket table (3 waves x 64 lanes of one direct load)
+constexpr int TS_TAB_LEN = 128;  // most timestamp buckets the matrix-core kernels index (the backward's histogram)
+// Timestamp buckets without a logarithm.  The bucket law is floor(ln(f) / size) of f = fl32(clip(|dt|, 1, 1e9));
+// it depends on dt only through the float f.  The key of f is its exponent and the top two bits of its
+// mantissa (four keys per octave, 120 keys up to 1e9).  When size > ln(1.25) a key's range of floats holds
+// at most one bucket boundary, so one entry per key {table value of the bucket the range starts in, first
+// float of the next bucket} decides the value with a single comparison; the value from the threshold on
+// is the next key's first field, so one 12-byte read brings all three -- exactly, boundaries included:
+// the thresholds are computed on the host in double.  The general kernels evaluate the law in double and
+// the CPU oracle is the same law, so all of them agree on every dt.
+// One head's table (TS_LDS_BYTES, copied to LDS by every workgroup):
+//   [(TS_KEYS + 2) x {float log2(e) * value, float threshold}]  by key (the per-pair path)
+//   [TS_KEYS x float: log2(e) * value of bucket b]  by bucket (the backward's table-gradient path)
+//   [TS_KEYS x int: smallest clipped |dt| that reaches the key's threshold]  [TS_KEYS x byte: bucket the
+//   key's range starts in]  by key (the per-tile shortcuts, table gradients)
+constexpr int TS_KEYS = 128;               // keys, and the most buckets the matrix-core kernels index
+constexpr int TS_KEY0 = 127 << 2;          // key of f = 1.0 before the offset is taken off
+constexpr int TS_DT_MAX = 1000000000;
+constexpr int TS_VAL_OFF = (TS_KEYS + 2) * 8, TS_INT_OFF = TS_VAL_OFF + TS_KEYS * 4, TS_BKT_OFF = TS_INT_OFF + TS_KEYS * 4;
+constexpr int TS_LDS_BYTES = TS_BKT_OFF + TS_KEYS;
+static_assert(TS_LDS_BYTES % 16 == 0 && TS_LDS_BYTES <= 3 * 1024, "table layout: at most three direct loads");
+struct TsKeys {                            // host-built part of the table, a kernel argument of hstu_prepare
+  float thr_f[TS_KEYS];                    // by key: first float of the bucket behind the one the key's range starts in
+  int32_t thr_i[TS_KEYS];                  // by key: smallest clipped |dt| that reaches thr_f
+  uint8_t bkt[TS_KEYS];                    // by key: bucket the key's range starts in
+};
+
 constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D, int KB>   // KB: bytes per q / k element (2 = bf16, 1 = fp8)
@@ -655,7 +680,7 @@ struct MfmaSmem {
   static constexpr int POS_BYTES = 4 * POS_COPY;    // 4 copies shifted by 0..3 floats
   static constexpr int TK_LANES = BN / 4 + 1;       // 16-byte pieces: 32 int32 key timestamps, then (min, max, -, -)
   static constexpr int TK_BYTES = TK_LANES * 16;
-  static constexpr int TAB_BYTES = 2 * TS_TAB_LEN * 4;   // scaled bucket table, then the bucket thresholds
+  static constexpr int TAB_BYTES = TS_LDS_BYTES;         // the bucket table of the workgroup's head
   static constexpr int SEG_BYTES = BN * 4;           // the step's 32 int32 key segment ids
   static constexpr int bias_stage(bool pos, bool ts, bool seg = false) {
     return (pos ? POS_BYTES : 0) + (ts ? TK_BYTES : 0) + (seg ? SEG_BYTES : 0);
@@ -820,12 +845,58 @@ __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, W
   return true;
 }
 
-// Timestamp bucket of a time difference already converted to float, as the MFMA kernel computes it:
-// trunc(log2(clamp(|f|, 1, 1e9)) * ln2 / bucket_size) by v_log_f32.
-__device__ __forceinline__ int ts_bucket_hw(float f, float log2_scale) {
-  f = __builtin_amdgcn_fmed3f(__builtin_fabsf(f), 1.0f, 1.0e9f);
-  return (int)(__builtin_amdgcn_logf(f) * log2_scale);
+// A 64-bit time difference clipped to [1, 1e9].
+__device__ __forceinline__ int ts_clip64(int64_t d) {
+  d = d < 0 ? -d : d;      // |INT64_MIN| stays negative and is clipped to 1; differences of real timestamps never get there
+  d = d < 1 ? 1 : d;
+  return (int)(d < TS_DT_MAX ? d : TS_DT_MAX);
 }
+// Lookup of a time difference in the head's table (in LDS): f = fl32(clip(|d|, 1, 1e9)), its key, and the
+// key's {value below the threshold, threshold, value from the threshold on}.
+struct TsLook { float f, lo, thr, hi; uint32_t key; };
+__device__ __forceinline__ TsLook ts_look(const unsigned char* tab, int d) {
+  TsLook l;
+  l.f = __builtin_amdgcn_fmed3f(__builtin_fabsf((float)d), 1.0f, (float)TS_DT_MAX);
+  l.key = (__builtin_bit_cast(uint32_t, l.f) >> 21) - (uint32_t)TS_KEY0;
+  const float* e = (const float*)(tab + (l.key << 3));
+  const float2 a = *(const float2*)e;
+  l.lo = a.x;
+  l.thr = a.y;
+  l.hi = e[2];
+  return l;
+}
+__device__ __forceinline__ float ts_value(const TsLook& l) { return l.f >= l.thr ? l.hi : l.lo; }
+__device__ __forceinline__ int ts_bucket(const unsigned char* tab, const TsLook& l) { return (int)tab[TS_BKT_OFF + l.key] + (l.f >= l.thr ? 1 : 0); }
+// The bucket alone (its value is then one more read, ts_bucket_value): fewer registers than ts_look,
+// for the kernel that also needs the bucket's index.
+__device__ __forceinline__ int ts_bucket_of(const unsigned char* tab, int d) {
+  const float f = __builtin_amdgcn_fmed3f(__builtin_fabsf((float)d), 1.0f, (float)TS_DT_MAX);
+  const uint32_t key = (__builtin_bit_cast(uint32_t, f) >> 21) - (uint32_t)TS_KEY0;
+  return (int)tab[TS_BKT_OFF + key] + (f >= *(const float*)(tab + (key << 3) + 4) ? 1 : 0);
+}
+// Both ends of a range of time differences [d_near, d_far]: their buckets and table values; `same` when
+// both are in one bucket and d_near >= 0 (then so is every difference between them); `two` when at most
+// one bucket boundary lies inside the range and one of the two entries holds it: differences >= thr are
+// then in the far end's bucket, the others in the near end's.
+struct TsEnds { int b_near, b_far, thr; float v_near, v_far; bool same, two; };
+__device__ __forceinline__ TsEnds ts_ends(const unsigned char* tab, int d_near, int d_far) {
+  const TsLook n = ts_look(tab, d_near), f = ts_look(tab, d_far);
+  TsEnds r;
+  r.b_near = ts_bucket(tab, n);
+  r.b_far = ts_bucket(tab, f);
+  r.v_near = ts_value(n);
+  r.v_far = ts_value(f);
+  const bool sorted = d_near >= 0;
+  r.same = sorted && r.b_near == r.b_far;
+  // the boundary is the near entry's when the near end lies below that, else the far entry's when the far
+  // end has passed it (a boundary that sits in a key's range between the two is in neither entry)
+  const bool n_up = n.f >= n.thr;
+  const bool held = n_up ? f.f >= f.thr : true;
+  r.thr = *(const int*)(tab + TS_INT_OFF + ((n_up ? f.key : n.key) << 2));
+  r.two = sorted && (r.b_near == r.b_far || (r.b_far == r.b_near + 1 && held));
+  return r;
+}
+__device__ __forceinline__ float ts_bucket_value(const unsigned char* tab, int b) { return *(const float*)(tab + TS_VAL_OFF + (b << 2)); }
 
 // Where sequence b starts in the int32 timestamp copy and in the per-tile range table.
 // Timestamps that follow the token axis are packed like it (tiles by an upper bound of
@@ -840,13 +911,14 @@ __device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_
 // What the main kernel reads from the workspace, rebuilt by every call:
 //  * the relative-position table scaled by log2(e) and zero-padded,
 //    [heads][POS_PAD + 2L-1 + POS_PAD]; the margins make every window read in-bounds;
-//  * the timestamp bucket table scaled by log2(e), [heads][TS_TAB_LEN];
+//  * the timestamp bucket tables (TsKeys above), [heads][TS_LDS_BYTES];
 //  * per sequence whose timestamps span less than 2^31: the timestamps minus their minimum
 //    as int32 (differences of two of them are then exact in 32 bits), and the (min, max)
 //    of those in each 32-key tile.  One workgroup per sequence.
-__global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __restrict__ pos_out, float* __restrict__ tab_out,
+__global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __restrict__ pos_out, int4* __restrict__ tab_out,
                                                     int32_t* __restrict__ ok_out, int32_t* __restrict__ rel_out,
-                                                    int32_t* __restrict__ range_out, int32_t* __restrict__ sched_out) {
+                                                    int32_t* __restrict__ range_out, int32_t* __restrict__ sched_out,
+                                                    const TsKeys keys) {
   const int tid = threadIdx.x;
   const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
   if (sched_out && blockIdx.x == gridDim.x - 1) {
@@ -936,31 +1008,20 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     }
   }
   if (tab_out) {
-    // bucket table times log2(e); indices past the last bucket repeat it (the clip of the bucket law)
-    for (int i = gtid; i < p.ts_heads * TS_TAB_LEN; i += gsz) {
-      const int hd = i / TS_TAB_LEN, e = i - hd * TS_TAB_LEN;
-      tab_out[i] = p.ts_tab[(int64_t)hd * (p.ts_nb + 1) + (e < p.ts_nb ? e : p.ts_nb)] * LOG2E;
-    }
-    // thr[b] = smallest |dt| >= 0 whose bucket, by the very instructions the main kernel uses, is >= b
-    // (INT_MAX when no 31-bit value reaches b): a bisection that relies on that function being monotone
-    int32_t* thr = (int32_t*)(tab_out + p.ts_heads * TS_TAB_LEN);
-    for (int bkt = gtid; bkt < TS_TAB_LEN; bkt += gsz) {
-      unsigned lo = 0, hi = 0x7fffffffu;          // invariant: bucket(hi) >= bkt or hi is the cap
-      if (ts_bucket_hw((float)(int)hi, p.ts_log2_scale) < bkt) { thr[bkt] = 0x7fffffff; continue; }
-      // the answer is near 2^(bkt / scale): try a window around it first (each bound is only taken when the
-      // function itself confirms it), which leaves 12 bisection steps instead of 31
-      const float guess = __builtin_amdgcn_exp2f((float)bkt / p.ts_log2_scale);
-      if (guess < 2.0e9f) {
-        const unsigned g = (unsigned)guess;
-        const unsigned a = g > 2048u ? g - 2048u : 0u, b = g + 2048u;
-        if (a > 0u && ts_bucket_hw((float)(int)(a - 1u), p.ts_log2_scale) < bkt) lo = a;
-        if (b < hi && ts_bucket_hw((float)(int)b, p.ts_log2_scale) >= bkt) hi = b;
+    // every head's bucket table: thresholds and buckets from the host, the table values times log2(e) with
+    // bucket indices clipped to the table's last entry (the clip of the bucket law)
+    for (int i = gtid; i < p.ts_heads * (TS_KEYS + 2); i += gsz) {
+      const int hd = i / (TS_KEYS + 2), e = i - hd * (TS_KEYS + 2);
+      unsigned char* out = (unsigned char*)tab_out + (int64_t)hd * (3 * 1024);
+      const float* tab = p.ts_tab + (int64_t)hd * (p.ts_nb + 1);
+      const int ek = e < TS_KEYS ? e : TS_KEYS - 1;      // the entries behind the last key repeat it
+      const int bk = keys.bkt[ek];
+      ((float2*)out)[e] = float2{tab[bk < p.ts_nb ? bk : p.ts_nb] * LOG2E, keys.thr_f[ek]};
+      if (e < TS_KEYS) {
+        ((float*)(out + TS_VAL_OFF))[e] = tab[e < p.ts_nb ? e : p.ts_nb] * LOG2E;
+        ((int*)(out + TS_INT_OFF))[e] = keys.thr_i[e];
+        out[TS_BKT_OFF + e] = (unsigned char)bk;
       }
-      while (lo < hi) {
-        const unsigned mid = lo + (hi - lo) / 2;
-        if (ts_bucket_hw((float)(int)mid, p.ts_log2_scale) >= bkt) hi = mid; else lo = mid + 1;
-      }
-      thr[bkt] = (int32_t)lo;
     }
   }
   if (pos_out) {
@@ -1076,8 +1137,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
-  float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
-  const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
+  const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   constexpr int DENSE_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
   constexpr int DENSE_STAGE = SM::dense_stage(DENSE);
   auto Db = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE; };
@@ -1246,13 +1306,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     }
   };
 
-  // prologue: the scaled bucket table (64 entries per wave, the last wave repeats the first), then
+  // prologue: the keyed bucket table, then
   // the first steps in flight before the first block (two when the loop runs in pairs, else NSTAGE - 1)
   if (TS) {
+    // three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
     const int c = w < 3 ? w : 0;
-    const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
-    lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
-    lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
+    if (1024 * c + 16 * lane < TS_LDS_BYTES)
+      lds_dma16((const unsigned char*)p.ts_keyed + (int64_t)(p.ts_heads > 1 ? h : 0) * (3 * 1024) + 1024 * c, (uint32_t)lane * 16u, TsKey + 1024 * c);
   }
   // The first step's tiles go out alone; the other two of the prologue follow behind the Q
   // fragments, whose wait below covers every load issued before it: behind all three steps it
@@ -1388,25 +1448,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
     if (TS) {
-      auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
       if (ts32) {
         const int32_t* tk = Tk(st);
         const int2 rg = *(const int2*)(tk + BN);
         // |tq - tk| grows as tk falls: when no key of the tile is later than tq and both ends of
         // the tile fall in the same bucket, so does everything between
-        const int d_near = tq32 - rg.y, d_far = tq32 - rg.x;
-        const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
-        const bool same = d_near >= 0 && b_near == b_far;
-        const bool two = d_near >= 0 && b_far - b_near <= 1;
-        if (__builtin_amdgcn_ballot_w64(!same) == 0) {
-          const float add = TsTab[b_near];
+        const TsEnds en = ts_ends(TsKey, tq32 - rg.y, tq32 - rg.x);
+        if (__builtin_amdgcn_ballot_w64(!en.same) == 0) {
+          const float add = en.v_near;
 #pragma unroll
           for (int r = 0; r < 16; ++r) u[r] += add;
-        } else if (__builtin_amdgcn_ballot_w64(!two) == 0) {
-          // at most one bucket boundary inside the tile for every lane: a key is in the farther
-          // bucket exactly when tq - tk >= thr[b_near + 1], i.e. tk <= tq - thr
-          const float add_near = TsTab[b_near], add_far = TsTab[b_near + 1];
-          const int cut = tq32 - TsThr[b_near + 1];
+        } else if (__builtin_amdgcn_ballot_w64(!en.two) == 0) {
+          // at most one bucket boundary inside the tile for every lane: a key is in the farther bucket
+          // exactly when tq - tk >= thr, i.e. tk <= tq - thr (lanes whose ends share a bucket: add_far == add_near)
+          const float add_near = en.v_near, add_far = en.v_far;
+          const int cut = tq32 - en.thr;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
@@ -1419,10 +1475,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
-            u[4 * g + 0] += TsTab[bucket_f((float)(tq32 - kk.x))];
-            u[4 * g + 1] += TsTab[bucket_f((float)(tq32 - kk.y))];
-            u[4 * g + 2] += TsTab[bucket_f((float)(tq32 - kk.z))];
-            u[4 * g + 3] += TsTab[bucket_f((float)(tq32 - kk.w))];
+            u[4 * g + 0] += ts_value(ts_look(TsKey, tq32 - kk.x));
+            u[4 * g + 1] += ts_value(ts_look(TsKey, tq32 - kk.y));
+            u[4 * g + 2] += ts_value(ts_look(TsKey, tq32 - kk.z));
+            u[4 * g + 3] += ts_value(ts_look(TsKey, tq32 - kk.w));
           }
         }
       } else {
@@ -1434,10 +1490,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
           for (int tt = 0; tt < 4; ++tt) {
             int j = kbs + 8 * g + 4 * hh + tt;
             j = j < s.n_ts ? j : s.n_ts - 1;
-            const int64_t dt = tq - tsg[j];
-            const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-            const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-            u[4 * g + tt] += TsTab[bucket_f((float)sat)];
+            u[4 * g + tt] += ts_value(ts_look(TsKey, ts_clip64(tq - tsg[j])));
           }
         }
       }
@@ -1811,8 +1864,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
-  float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
-  const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
+  const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   float* TgBase = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
   const bool want_dpos = TG && POS && p.dpos != nullptr, want_dts = TG && TS && p.dts != nullptr;
 
@@ -1908,10 +1960,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   };
 
   if (TS) {
+    // three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
     const int c = w < 3 ? w : 0;
-    const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
-    lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
-    lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
+    if (1024 * c + 16 * lane < TS_LDS_BYTES)
+      lds_dma16((const unsigned char*)p.ts_keyed + (int64_t)(p.ts_heads > 1 ? h : 0) * (3 * 1024) + 1024 * c, (uint32_t)lane * 16u, TsKey + 1024 * c);
   }
   // the first pair of steps in flight (the step loop runs in pairs, see there)
   if (t_lo < nt) dma_step(t_lo);
@@ -1945,14 +1997,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     qseg = p.q_seg[(int64_t)b * p.L + (qrow < p.L ? qrow : p.L - 1)];
     asm volatile("" ::"v"(qseg));
   }
-  int64_t tq = 0;
   int32_t tq32 = 0;
+  int iq_lane = 0;       // index of the timestamp this lane's row takes (the 64-bit path reads it from memory again)
   if (TS) {
     int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
-    iq = iq < 0 ? 0 : iq;
-    tq32 = trel[iq];
-    tq = tsg[iq];
-    asm volatile("" ::"v"(tq), "v"(tq32));
+    iq_lane = iq < 0 ? 0 : iq;
+    tq32 = trel[iq_lane];     // meaningless when !ts32, and then unused
+    asm volatile("" ::"v"(tq32));
   }
 
   floatx16 acc[DVB];
@@ -2019,24 +2070,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
     if (TS) {
-      auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
       if (ts32) {
         const int32_t* tk = Tk(st);
         const int2 rg = *(const int2*)(tk + BN);
-        const int d_near = tq32 - rg.y, d_far = tq32 - rg.x;
-        const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
-        const bool same = d_near >= 0 && b_near == b_far;
-        const bool two = d_near >= 0 && b_far - b_near <= 1;
-        if (__builtin_amdgcn_ballot_w64(!same) == 0) {
-          const float add = TsTab[b_near];
+        const TsEnds en = ts_ends(TsKey, tq32 - rg.y, tq32 - rg.x);
+        if (__builtin_amdgcn_ballot_w64(!en.same) == 0) {
+          const float add = en.v_near;
 #pragma unroll
           for (int r = 0; r < 16; ++r) u[r] += add;
-          bk_lane = b_near;
-        } else if (__builtin_amdgcn_ballot_w64(!two) == 0) {
+          bk_lane = en.b_near;
+        } else if (__builtin_amdgcn_ballot_w64(!en.two) == 0) {
           // at most one bucket boundary inside the tile for every lane: a key is in the farther
-          // bucket exactly when tq - tk >= thr[b_near + 1], i.e. tk <= tq - thr
-          const float add_near = TsTab[b_near], add_far = TsTab[b_near + 1];
-          const int cut = tq32 - TsThr[b_near + 1];
+          // bucket exactly when tq - tk >= thr, i.e. tk <= tq - thr (a lane whose ends share a bucket
+          // must not flag any key: the next bucket's sum would take its dS)
+          const float add_near = en.v_near, add_far = en.v_far;
+          const int cut = en.b_far != en.b_near ? tq32 - en.thr : (int)0x80000000;
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
@@ -2047,32 +2095,39 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
             u[4 * g + 3] += f3 ? add_far : add_near;
             if (TG) far_bits |= ((uint32_t)f0 | ((uint32_t)f1 << 1) | ((uint32_t)f2 << 2) | ((uint32_t)f3 << 3)) << (4 * g);
           }
-          bk_lane = b_near;
+          bk_lane = en.b_near;
         } else {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const int4 kk = *(const int4*)(tk + 8 * g + 4 * hh);
-            const int b0 = bucket_f((float)(tq32 - kk.x)), b1 = bucket_f((float)(tq32 - kk.y));
-            const int b2 = bucket_f((float)(tq32 - kk.z)), b3 = bucket_f((float)(tq32 - kk.w));
-            u[4 * g + 0] += TsTab[b0];
-            u[4 * g + 1] += TsTab[b1];
-            u[4 * g + 2] += TsTab[b2];
-            u[4 * g + 3] += TsTab[b3];
-            if (TG) bkp[g] = (uint32_t)b0 | ((uint32_t)b1 << 8) | ((uint32_t)b2 << 16) | ((uint32_t)b3 << 24);
+            if (TG) {
+              const int b0 = ts_bucket_of(TsKey, tq32 - kk.x), b1 = ts_bucket_of(TsKey, tq32 - kk.y);
+              const int b2 = ts_bucket_of(TsKey, tq32 - kk.z), b3 = ts_bucket_of(TsKey, tq32 - kk.w);
+              u[4 * g + 0] += ts_bucket_value(TsKey, b0);
+              u[4 * g + 1] += ts_bucket_value(TsKey, b1);
+              u[4 * g + 2] += ts_bucket_value(TsKey, b2);
+              u[4 * g + 3] += ts_bucket_value(TsKey, b3);
+              bkp[g] = (uint32_t)b0 | ((uint32_t)b1 << 8) | ((uint32_t)b2 << 16) | ((uint32_t)b3 << 24);
+            } else {
+              u[4 * g + 0] += ts_value(ts_look(TsKey, tq32 - kk.x));
+              u[4 * g + 1] += ts_value(ts_look(TsKey, tq32 - kk.y));
+              u[4 * g + 2] += ts_value(ts_look(TsKey, tq32 - kk.z));
+              u[4 * g + 3] += ts_value(ts_look(TsKey, tq32 - kk.w));
+            }
           }
         }
       } else {
+        // time span of the sequence beyond 31 bits: 64-bit differences of timestamps read straight
+        // from memory (rare; correctness over speed)
+        const int64_t tq = tsg[iq_lane];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
 #pragma unroll
           for (int tt = 0; tt < 4; ++tt) {
             int j = kbs + 8 * g + 4 * hh + tt;
             j = j < s.n_ts ? j : s.n_ts - 1;
-            const int64_t dt = tq - tsg[j];
-            const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-            const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-            const int bb = bucket_f((float)sat);
-            u[4 * g + tt] += TsTab[bb];
+            const int bb = ts_bucket_of(TsKey, ts_clip64(tq - tsg[j]));
+            u[4 * g + tt] += ts_bucket_value(TsKey, bb);
             if (TG) bkp[g] = tt == 0 ? (uint32_t)bb : bkp[g] | ((uint32_t)bb << (8 * tt));
           }
         }
@@ -2313,8 +2368,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0)); };
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
-  float* TsTab = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE);
-  const int32_t* TsThr = (const int32_t*)(TsTab + TS_TAB_LEN);
+  const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -2421,10 +2475,10 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   };
 
   if (TS) {
+    // three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
     const int c = w < 3 ? w : 0;
-    const float* tab = p.ts_scaled + (int64_t)(p.ts_heads > 1 ? h : 0) * TS_TAB_LEN + 64 * c;
-    lds_dma4(tab, (uint32_t)lane * 4u, TsTab + 64 * c);
-    lds_dma4(p.ts_thr + 64 * c, (uint32_t)lane * 4u, TsThr + 64 * c);
+    if (1024 * c + 16 * lane < TS_LDS_BYTES)
+      lds_dma16((const unsigned char*)p.ts_keyed + (int64_t)(p.ts_heads > 1 ? h : 0) * (3 * 1024) + 1024 * c, (uint32_t)lane * 16u, TsKey + 1024 * c);
   }
   // the first pair of steps in flight (the step loop runs in pairs, see there)
   if (t_lo < nt) dma_step(t_lo);
@@ -2528,7 +2582,6 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
     if (TS) {
-      auto bucket_f = [&](float f) { return ts_bucket_hw(f, p.ts_log2_scale); };
       const int32_t* tqs = Tq(st);
       // row i's logit takes the timestamp of row min(i + 1, last); index into this step's 36
       auto tq_at = [&](int r) {
@@ -2541,32 +2594,23 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
         // smallest and to the largest timestamp of the two tiles the rows come from
         const int4 rg = *(const int4*)(tqs + 4 * (TQ_LANES - 1));
         const int t_min = rg.x < rg.z ? rg.x : rg.z, t_max = rg.y > rg.w ? rg.y : rg.w;
-        const int d_near = t_min - tk32, d_far = t_max - tk32;
-        const int b_near = bucket_f((float)d_near), b_far = bucket_f((float)d_far);
-        const bool same = d_near >= 0 && b_near == b_far;
-        const bool two = d_near >= 0 && b_far - b_near <= 1;
-        if (__builtin_amdgcn_ballot_w64(!same) == 0) {
-          const float add = TsTab[b_near];
+        const TsEnds en = ts_ends(TsKey, t_min - tk32, t_max - tk32);
+        if (__builtin_amdgcn_ballot_w64(!en.same) == 0) {
+          const float add = en.v_near;
 #pragma unroll
           for (int r = 0; r < 16; ++r) u[r] += add;
-        } else if (__builtin_amdgcn_ballot_w64(!two) == 0) {
-          // one bucket boundary at most: the farther bucket exactly when tq - tk >= thr[b_near + 1]
-          const float add_near = TsTab[b_near], add_far = TsTab[b_near + 1];
-          const int thr = TsThr[b_near + 1];
+        } else if (__builtin_amdgcn_ballot_w64(!en.two) == 0) {
+          // one bucket boundary at most: the farther bucket exactly when tq - tk >= thr
+          const float add_near = en.v_near, add_far = en.v_far;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) u[r] += tqs[tq_at(r) - qbs] - tk32 >= thr ? add_far : add_near;
+          for (int r = 0; r < 16; ++r) u[r] += tqs[tq_at(r) - qbs] - tk32 >= en.thr ? add_far : add_near;
         } else {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) u[r] += TsTab[bucket_f((float)(tqs[tq_at(r) - qbs] - tk32))];
+          for (int r = 0; r < 16; ++r) u[r] += ts_value(ts_look(TsKey, tqs[tq_at(r) - qbs] - tk32));
         }
       } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int64_t dt = tsg[tq_at(r)] - tk;
-          const int32_t lo = (int32_t)dt, hi = (int32_t)(dt >> 32);
-          const int32_t sat = (hi == (lo >> 31)) ? lo : 0x7fffffff;
-          u[r] += TsTab[bucket_f((float)sat)];
-        }
+        for (int r = 0; r < 16; ++r) u[r] += ts_value(ts_look(TsKey, ts_clip64(tsg[tq_at(r)] - tk)));
       }
     }
     // transposed fragments of dO (for dV) and of Q (for dK)
@@ -2684,6 +2728,65 @@ int fail(int code, const char* fmt, ...) {
 
 enum Variant { V_INVALID = 0, V_GENERAL_F32, V_GENERAL_BF16, V_MFMA_BF16, V_MFMA_FP8 };
 
+// The timestamp bucket law on the host: bucket(dt) = floor(ln(fl32(clip(|dt|, 1, 1e9))) / size), the float
+// log and divide of recml/layers/keras/hstu.py:48-55 taken in double.  thr[b] is the smallest clipped
+// |dt| whose bucket is >= b (INT32_MAX when 1e9 does not reach b): the integer thresholds that the
+// kernels and the CPU oracle share.  `keys` is the part of the matrix-core kernels' keyed table that does
+// not depend on the bias values, `keyed_ok` whether that table can represent this bucket size (at most
+// one boundary per key range, bucket indices within the backward's histogram).
+constexpr int LAW_THR_LEN = 256;
+struct BucketLaw {
+  float size;
+  bool valid, keyed_ok;
+  int reach;                       // bucket of 1e9
+  int32_t thr[LAW_THR_LEN];
+  TsKeys keys;
+};
+int law_bucket(float f, double size) { return (int)floor(log((double)f) / size); }
+
+const BucketLaw& bucket_law(float size_f) {
+  thread_local BucketLaw law = {0.f, false, false, 0, {0}, {{0}, {0}, {0}}};
+  if (law.valid && law.size == size_f) return law;
+  const double size = (double)size_f;
+  law.size = size_f;
+  law.reach = law_bucket((float)TS_DT_MAX, size);
+  for (int b = 0; b < LAW_THR_LEN; ++b) {
+    if (b > law.reach) { law.thr[b] = 0x7fffffff; continue; }
+    int64_t lo = 1, hi = TS_DT_MAX;              // bucket(hi) >= b
+    while (lo < hi) {
+      const int64_t mid = lo + (hi - lo) / 2;
+      if (law_bucket((float)mid, size) >= b) hi = mid; else lo = mid + 1;
+    }
+    law.thr[b] = (int32_t)lo;
+  }
+  law.keyed_ok = law.reach + 1 < TS_KEYS && law.reach + 2 < LAW_THR_LEN;
+  for (int key = 0; key < TS_KEYS && law.keyed_ok; ++key) {
+    // floats of this key: [f_lo, f_next); the time differences behind them are integers
+    uint32_t bits_lo = (uint32_t)(TS_KEY0 + key) << 21, bits_next = (uint32_t)(TS_KEY0 + key + 1) << 21;
+    float f_lo, f_next;
+    memcpy(&f_lo, &bits_lo, 4);
+    memcpy(&f_next, &bits_next, 4);
+    float f_first = ceilf(f_lo);                 // first integer-valued float of the range
+    if (f_first > (float)TS_DT_MAX) f_first = (float)TS_DT_MAX;
+    float f_last = nextafterf(f_next, 0.f);
+    if (f_last > (float)TS_DT_MAX) f_last = (float)TS_DT_MAX;
+    const int b_lo = law_bucket(f_first, size);
+    law.keys.bkt[key] = (uint8_t)b_lo;
+    law.keys.thr_f[key] = (float)law.thr[b_lo + 1];      // INT32_MAX becomes 2^31: beyond every clipped difference
+    law.keys.thr_i[key] = law.thr[b_lo + 1];
+    if (f_first < f_next) {
+      // at most one boundary inside the key's range; and when there is one, the next key must start in
+      // the bucket behind it (the kernels take the value from the threshold on from the next key's entry)
+      const int b_last = law_bucket(f_last, size);
+      float f_after = ceilf(f_next);
+      if (f_after > (float)TS_DT_MAX) f_after = (float)TS_DT_MAX;
+      if (b_last > b_lo + 1 || (b_last == b_lo + 1 && key + 1 < TS_KEYS && law_bucket(f_after, size) != b_last)) law.keyed_ok = false;
+    }
+  }
+  law.valid = true;
+  return law;
+}
+
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
 // Whether the matrix-core kernel covers these arguments (dtype aside: bf16, or fp8 q/k).
@@ -2704,8 +2807,8 @@ bool mfma_eligible(const HstuAttnFwdArgs* a) {
   // keys and queries of different lengths: the padded layout without the table biases (whose geometry needs one length)
   const bool len_ok = a->L == a->Lkv || (a->layout == HSTU_LAYOUT_PADDED && !a->pos_tab && !a->ts_tab);
   const bool opts_ok = seg_ok && dense_ok && len_ok &&
-                       // every bucket index ln(1e9) / bucket_size can reach must be inside the kernel's table
-                       (!a->ts_tab || (a->ts_num_buckets <= 128 && a->ts_bucket_size >= 0.11f));
+                       // the keyed bucket table must be able to hold this bucket size (sizes above ln 1.25 = 0.2232)
+                       (!a->ts_tab || (a->ts_num_buckets <= 128 && bucket_law(a->ts_bucket_size).keyed_ok));
   auto s8 = [](int64_t x) { return (x & 7) == 0; };
   auto sq = [kb](int64_t x) { return (x * kb & 15) == 0; };
   const bool align_ok = aligned16(a->q) && aligned16(a->k) && aligned16(a->v) && aligned16(a->out) &&
@@ -2835,7 +2938,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) 
     const bool by_token = a->ts_stride_b == 0;
     const size_t n_ts = by_token ? (size_t)a->total_tokens : (size_t)a->B * (size_t)a->L;
     const size_t tiles = by_token ? (size_t)(a->total_tokens >> 5) + (size_t)a->B + tiles_per_seq : (size_t)a->B * tiles_per_seq;
-    w.tab_bytes = up(((size_t)a->ts_heads + 1) * TS_TAB_LEN * sizeof(float));   // scaled tables, then the thresholds
+    w.tab_bytes = up((size_t)a->ts_heads * 3 * 1024);   // the bucket tables (three direct loads of 1 KB per head)
     w.ok_bytes = up((size_t)a->B * sizeof(int32_t));
     // the kernels fetch whole 16-byte pieces: up to 35 timestamps and one range past the end
     w.rel_bytes = up(n_ts * sizeof(int32_t) + 160);
@@ -2865,7 +2968,6 @@ Params make_params(const HstuAttnFwdArgs* a) {
   p.pos_heads = a->pos_heads; p.ts_heads = a->ts_heads;
   p.ts_nb = a->ts_num_buckets;
   p.ts_bucket_size = a->ts_bucket_size;
-  p.ts_log2_scale = a->ts_tab ? (float)(0.6931471805599453 / (double)a->ts_bucket_size) : 0.f;
   p.alpha = a->alpha; p.inv_n = a->inv_n;
   p.q_scale = a->q_scale; p.k_scale = a->k_scale;
   p.n_qtiles = (a->L + BM - 1) / BM;
@@ -2964,11 +3066,17 @@ int launch_mfma_d(const Params& p, hipStream_t st) {
   return launch_mfma_inst<D, false, false, F8>(p, st);
 }
 
+// HSTU_ONLY_D128: a development build that compiles the d = 128 instances only (a quarter of the
+// compile time); other head dims then report an error instead of running.
 template <bool F8>
 int launch_mfma(const Params& p, hipStream_t st) {
   if (p.d_qk == 128) return launch_mfma_d<128, F8>(p, st);
+#ifndef HSTU_ONLY_D128
   if (p.d_qk == 64) return launch_mfma_d<64, F8>(p, st);
   return launch_mfma_d<32, F8>(p, st);
+#else
+  return fail(HSTU_ERR_SHAPE, "development build: d = 128 only");
+#endif
 }
 
 
@@ -2986,7 +3094,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   char* base = (char*)args->workspace;
   if (ws.bias_total() >= (1ull << 32)) return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes is beyond what the kernel addresses", ws.bias_total());
   float* pos_out = ws.pos_bytes ? (float*)base : nullptr;
-  float* tab_out = ws.tab_bytes ? (float*)(base + ws.pos_bytes) : nullptr;
+  int4* tab_out = ws.tab_bytes ? (int4*)(base + ws.pos_bytes) : nullptr;
   int32_t* ok_out = ws.ok_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes) : nullptr;
   int32_t* rel_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes);
   int32_t* range_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes);
@@ -2996,8 +3104,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   q.items_max = ws.items_max;
   q.split_max = ws.split_max;
   q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
-  q.ts_scaled = tab_out;
-  q.ts_thr = tab_out ? (const int32_t*)(tab_out + (size_t)q.ts_heads * TS_TAB_LEN) : nullptr;
+  q.ts_keyed = tab_out;
   q.pos_scaled = pos_out;
   q.ts_ok = ok_out;
   q.ts_rel = rel_out;
@@ -3008,7 +3115,9 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
   if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
   if ((ws.bias_total() || ws.sched_bytes) && !(args->flags & HSTU_FWD_WORKSPACE_PREPARED)) {
-    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out);
+    static const TsKeys no_keys = {{0}, {0}, {0}};
+    const TsKeys& keys = tab_out ? bucket_law(q.ts_bucket_size).keys : no_keys;
+    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out, keys);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
   }
@@ -3072,8 +3181,12 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
   Params q = p;
   if (int rc = setup_workspace(&f, ws, q, st)) return rc;
   if (q.d_qk == 128) return launch_bwd_mfma_d<128>(q, st);
+#ifndef HSTU_ONLY_D128
   if (q.d_qk == 64) return launch_bwd_mfma_d<64>(q, st);
   return launch_bwd_mfma_d<32>(q, st);
+#else
+  return fail(HSTU_ERR_SHAPE, "development build: d = 128 only");
+#endif
 }
 
 }  // namespace
@@ -3114,6 +3227,13 @@ const char* hstu_attn_last_error(void) { return g_err; }
 size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args) {
   if (validate(args) != HSTU_OK) return 0;
   return plan_workspace(args).total();
+}
+
+int hstu_attn_bucket_thresholds(float bucket_size, int32_t* thresholds, int count) {
+  if (!(bucket_size > 0.f) || (count > 0 && !thresholds)) return fail(HSTU_ERR_SHAPE, "bad bucket size or null output");
+  const BucketLaw& law = bucket_law(bucket_size);
+  for (int b = 0; b < count; ++b) thresholds[b] = b < LAW_THR_LEN ? law.thr[b] : 0x7fffffff;
+  return law.reach + 1;
 }
 
 const char* hstu_attn_fwd_variant(const HstuAttnFwdArgs* args) {

@@ -22,9 +22,16 @@ import torch
 
 
 def default_bucketization(x: torch.Tensor, bucket_size: float = 0.301) -> torch.Tensor:
-  """log(clip(|x|, 1, 1e9)) / 0.301 truncated to int (recml/layers/keras/hstu.py:33-55)."""
-  x = x.abs().clamp(1, int(1e9)).to(torch.float32)
-  return (torch.log(x) / bucket_size).to(torch.int64)
+  """log(clip(|x|, 1, 1e9)) / 0.301 truncated to int (recml/layers/keras/hstu.py:33-55).
+
+  The clipped difference and the bucket size are rounded to float32 as in the
+  reference; the logarithm and the quotient are taken in float64, which is the
+  bucket law the fused kernels follow on every time difference, boundaries of
+  buckets included.
+  """
+  x = x.abs().clamp(1, int(1e9)).to(torch.float32).to(torch.float64)
+  size = float(torch.tensor(bucket_size, dtype=torch.float32))
+  return torch.floor(torch.log(x) / size).to(torch.int64)
 
 
 class RelativePositionalBias(torch.nn.Module):

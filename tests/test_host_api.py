@@ -57,3 +57,23 @@ def test_product_package_does_not_use_the_oracle():
       if name.endswith(".py"):
         text = open(os.path.join(dirpath, name)).read()
         assert "import oracle" not in text and "from oracle" not in text, os.path.join(dirpath, name)
+
+
+def test_library_bucket_thresholds_equal_the_oracle_law():
+  """The integer thresholds the kernels bucket time differences by (computed on the host, no GPU
+  needed) are the oracle's, for the reference's bucket size and others."""
+  import ctypes as C
+  import numpy as np
+  from recml_amd import _lib
+  from oracle import hstu_oracle as O
+  lib = _lib.load()
+  for size in (0.301, 0.25, 0.4, 0.7, 1.0, 0.15):
+    want = O.bucket_thresholds(size)
+    out = (C.c_int32 * 256)()
+    reach = lib.hstu_attn_bucket_thresholds(C.c_float(size), out, 256)
+    assert reach == len(want), size
+    got = np.frombuffer(out, dtype=np.int32)
+    np.testing.assert_array_equal(got[:reach], want[:256])
+    if reach < 256:
+      assert (got[reach:] == 2**31 - 1).all()
+  assert lib.hstu_attn_bucket_thresholds(C.c_float(-1.0), None, 0) == -4

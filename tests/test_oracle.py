@@ -84,16 +84,37 @@ def test_bucketization_hand_cases():
 def test_bucket_thresholds_are_the_law():
   th = O.bucket_thresholds()
   assert len(th) == 69 and th[0] == 1 and th[-1] <= 10**9
+  # the textbook values ceil(e^(0.301 k)) where nothing is close: e^0.301 = 1.351, 1.826, 2.467, 3.333, 4.504,
+  # 6.086, 8.224, 11.11, 15.01, 20.29, 27.41, 37.04
+  assert list(th[:13]) == [1, 2, 2, 3, 4, 5, 7, 9, 12, 16, 21, 28, 38]
+  # by construction: T_k is where the law first reaches k
   for kk, t in enumerate(th):
-    assert math.floor(math.log(t) / 0.301) >= kk
+    assert O.bucketize_law(np.array([t]))[0] >= kk
     if t > 1:
-      assert math.floor(math.log(t - 1) / 0.301) < kk
-  # fp32 and fp64 evaluation agree away from the boundary set
+      assert O.bucketize_law(np.array([t - 1]))[0] < kk
+  # an independent evaluation of the same expression (python floats instead of numpy arrays)
+  size = float(np.float32(0.301))
+  for t in th[1:]:
+    for x in (int(t) - 1, int(t), int(t) + 1):
+      assert O.bucketize_law(np.array([x]))[0] == math.floor(math.log(float(np.float32(x))) / size)
+  # number of thresholds at or below x == the bucket of x
   rng = np.random.default_rng(1)
   x = np.concatenate([np.arange(1, 5000), rng.integers(1, 10**9, 200000)])
+  np.testing.assert_array_equal(np.searchsorted(th, x, side="right") - 1, O.bucketize_law(x))
+  # the literal float32 recipe agrees with the law away from the enumerated boundary set
   far = ~O.near_bucket_boundary(x)
   np.testing.assert_array_equal(O.default_bucketization(x)[far], O.bucketize_law(x)[far])
   assert far.mean() > 0.999
+
+
+def test_bucket_law_other_sizes_and_clip():
+  for size in (0.25, 0.301, 0.5, 1.0):
+    th = O.bucket_thresholds(size)
+    x = np.concatenate([th, th - 1, th + 1])
+    x = x[x >= 1]
+    np.testing.assert_array_equal(np.searchsorted(th, x, side="right") - 1, O.bucketize_law(x, size))
+  # beyond 1e9 the clip holds the bucket; the sign does not matter
+  assert O.bucketize_law(np.array([10**9, 10**9 + 5, 2 * 10**9, 5 * 10**12, -5 * 10**12])).tolist() == [68] * 5
 
 
 def test_time_delta_worked_example():

@@ -2789,6 +2789,13 @@ const BucketLaw& bucket_law(float size_f) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
 
+// The sliding window as the kernels take it: a window that reaches across the whole sequence restricts
+// nothing and is passed on as "no window" (the kernels add it to row indices in 32 bits).
+int effective_window(const HstuAttnFwdArgs* a) {
+  const int longest = a->L > a->Lkv ? a->L : a->Lkv;
+  return (a->window >= 0 && a->window < longest) ? a->window : -1;
+}
+
 // Whether the matrix-core kernel covers these arguments (dtype aside: bf16, or fp8 q/k).
 bool mfma_eligible(const HstuAttnFwdArgs* a) {
   const int kb = a->qk_dtype == HSTU_DTYPE_FP8_E4M3FN ? 1 : 2;   // bytes per q / k element
@@ -2904,7 +2911,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) 
   const bool jag = a->layout == HSTU_LAYOUT_JAGGED;
   const long long tiles_est = (long long)a->H * (jag ? (a->total_tokens / BM + a->B) : (long long)a->B * n_qtiles);
   w.entries_per_bh = n_qtiles;
-  if (allow_split && a->window < 0 && tiles_est < 1024 && steps_max > 16) {
+  if (allow_split && effective_window(a) < 0 && tiles_est < 1024 && steps_max > 16) {
     w.split_steps = (steps_max + MAX_CHUNKS - 1) / MAX_CHUNKS;
     w.split_steps = w.split_steps < 16 ? 16 : w.split_steps;
     // first tile with more steps than that (a causal tile qt has up to 4 (qt + 1) steps)
@@ -2963,7 +2970,7 @@ Params make_params(const HstuAttnFwdArgs* a) {
   p.jagged = a->layout == HSTU_LAYOUT_JAGGED;
   p.causal = a->causal != 0;
   p.mask_mode = p.jagged ? HSTU_MASK_LENGTH : a->mask_mode;
-  p.window = a->window;
+  p.window = effective_window(a);
   p.mask_batched = a->mask_batched; p.dense_bias_batched = a->dense_bias_batched;
   p.pos_heads = a->pos_heads; p.ts_heads = a->ts_heads;
   p.ts_nb = a->ts_num_buckets;

@@ -35,10 +35,19 @@ from recml_amd import hstu_ops
 from recml_amd import masks
 
 
+def _wants_grad(*tensors) -> bool:
+  return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
 def _attention(q, k, v, *, pos_bias=None, ts_bias=None, **kw):
-  """The attention op, differentiable when anything it reads wants a gradient."""
-  wants = torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (q, k, v, pos_bias, ts_bias))
-  if wants:
+  """The attention op, differentiable when anything it reads wants a gradient: through the HIP
+  backward kernels for q, k, v and the bias tables; through plain torch when a dense bias wants one
+  (the kernels return no gradient for it)."""
+  if _wants_grad(kw.get("bias")):
+    if q.dim() != 4:
+      raise ValueError("a dense bias that requires a gradient needs the padded layout")
+    return hstu_ops.dense_attention_torch(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
+  if _wants_grad(q, k, v, pos_bias, ts_bias):
     return hstu_ops.hstu_attention_autograd(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
   return hstu_ops.hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
 
@@ -110,7 +119,7 @@ class HSTUBlock(torch.nn.Module):
     """
     B, L, D = inputs.shape
     H, hd = self.num_heads, self.head_dim
-    fused = self._fused_inference(inputs)
+    fused = self._fused_inference(inputs, pos_bias, ts_bias, attention_bias)
     x = F.layer_norm(inputs, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
     w, b = self._uqkv_weights()
     if fused:
@@ -122,8 +131,13 @@ class HSTUBlock(torch.nn.Module):
       uqkv = F.silu(uqkv).reshape(B, L, 4, H, hd)
     u, q, k, v = uqkv.unbind(dim=2)
     if attention_mask is not None:
-      attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
-                                          scaled_pointwise_attn=self.scaled_pointwise_attn)
+      if _wants_grad(q, attention_bias):
+        # the reference's calling convention while training: dense mask and bias through plain torch
+        alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
+        attn = hstu_ops.dense_attention_torch(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
+      else:
+        attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
+                                            scaled_pointwise_attn=self.scaled_pointwise_attn)
     else:
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
@@ -143,9 +157,11 @@ class HSTUBlock(torch.nn.Module):
     return out.reshape(B, L, D) + inputs
 
 
-  def _fused_inference(self, t) -> bool:
-    """Whether the fused block steps apply: bf16 on a GPU, nothing asking for gradients."""
-    wants_grad = torch.is_grad_enabled() and (t.requires_grad or any(p.requires_grad for p in self.parameters()))
+  def _fused_inference(self, t, *bias_inputs) -> bool:
+    """Whether the fused block steps apply: bf16 on a GPU, nothing asking for gradients (the fused
+    steps are not differentiable: a bias table or dense bias that requires a gradient rules them out
+    like a parameter of the block would)."""
+    wants_grad = _wants_grad(t, *self.parameters(), *bias_inputs)
     return t.is_cuda and t.dtype == torch.bfloat16 and not wants_grad
 
   def _uqkv_weights(self):
@@ -162,7 +178,7 @@ class HSTUBlock(torch.nn.Module):
     residual as the C operand of the output product."""
     T, D = tokens.shape
     H, hd = self.num_heads, self.head_dim
-    fused = self._fused_inference(tokens)
+    fused = self._fused_inference(tokens, pos_bias, ts_bias)
     x = F.layer_norm(tokens, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
     w, b = self._uqkv_weights()
     if fused:

@@ -219,7 +219,7 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
   if sliding_window_size is not None:
     if int(sliding_window_size) < 0:
       raise ValueError("sliding_window_size must be >= 0")
-    a.window = int(sliding_window_size)
+    a.window = min(int(sliding_window_size), 2 ** 31 - 1)   # beyond the sequence it restricts nothing
 
   if mask is not None:
     if isinstance(mask, np.ndarray):
@@ -423,8 +423,55 @@ class _HstuAttentionFn(torch.autograd.Function):
 
 
 def hstu_attention_autograd(q, k, v, *, pos_bias=None, ts_bias=None, **kwargs):
-  """hstu_attention as a differentiable torch op (gradients for q, k, v, pos_bias, ts_bias)."""
+  """hstu_attention as a differentiable torch op (gradients for q, k, v, pos_bias, ts_bias).
+
+  A dense `bias` is taken as a constant: the backward kernels return no gradient
+  for it, so one that requires a gradient is refused here rather than silently
+  cut out of the graph (dense_attention_torch differentiates through it).
+  """
+  dense = kwargs.get("bias")
+  if isinstance(dense, torch.Tensor) and dense.requires_grad and torch.is_grad_enabled():
+    raise ValueError("the dense `bias` requires a gradient, which the fused backward does not compute: "
+                     "pass bias tables (pos_bias, ts_bias), or use dense_attention_torch")
   return _HstuAttentionFn.apply(q, k, v, pos_bias, ts_bias, kwargs)
+
+
+def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=True, pos_bias=None,
+                          timestamps=None, ts_bias=None, ts_bucket_size=0.301, bias=None, mask=None,
+                          sliding_window_size=None):
+  """The op in plain torch on padded [B, L, H, d] tensors (recml/layers/keras/hstu.py:356-390 with the
+  bias tables expanded): materialises [B, H, L, L], differentiable through everything it reads, any
+  device.  The slow path for what the fused backward cannot differentiate (a dense bias that requires
+  a gradient, e.g. from a custom bucketization function); not used otherwise."""
+  from recml_amd.hstu_bias import default_bucketization
+  B, L, H, d = q.shape
+  Lkv = k.shape[1]
+  n = L if n is None else n
+  s = alpha * torch.einsum("bihd,bjhd->bhij", q.float(), k.float())
+  i, j = torch.arange(L, device=q.device), torch.arange(Lkv, device=q.device)
+  if pos_bias is not None:
+    pt = pos_bias.float().reshape(-1, 2 * L - 1)
+    s = s + pt[:, (L - 1) + j[None, :] - i[:, None]][None]
+  if ts_bias is not None:
+    tt = ts_bias.float().reshape(-1, ts_bias.shape[-1])
+    ext = torch.cat([timestamps, timestamps[:, L - 1: L]], dim=1)
+    bucket = default_bucketization(ext[:, 1:, None] - ext[:, None, :-1], ts_bucket_size).clamp(0, tt.shape[1] - 1)
+    s = s + tt[:, bucket].transpose(0, 1)
+  if bias is not None:
+    bb = bias.float()
+    s = s + (bb if bb.dim() == 3 else bb[None])[:, None]
+  keep = torch.ones((1, L, Lkv), dtype=torch.bool, device=q.device)
+  if causal:
+    keep = keep & (j[None, None, :] <= i[None, :, None])
+  if sliding_window_size is not None:
+    keep = keep & ((i[None, :, None] - j[None, None, :]).abs() <= int(sliding_window_size))
+  if seq_lens is not None:
+    keep = keep & (i[None, :, None] < seq_lens[:, None, None]) & (j[None, None, :] < seq_lens[:, None, None])
+  if mask is not None:
+    mk = mask != 0
+    keep = keep & (mk if mk.dim() == 3 else mk[None])
+  p = torch.where(keep[:, None], torch.nn.functional.silu(s) / n, torch.zeros((), device=q.device))
+  return torch.einsum("bhij,bjhd->bihd", p, v.float()).to(v.dtype)
 
 
 def pointwise_splash_attention(

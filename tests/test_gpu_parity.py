@@ -134,51 +134,50 @@ def test_config3_reduced_fp32_and_bf16(gpu):
   assert _err(outb, oracle_workload(w, qb, kb, vb)) <= BF16_TOL
 
 
+def _check_all_sequences_c(w, q, k, v, out, tol):
+  """Every sequence of a jagged workload against the C oracle (double accumulation), plus the numpy
+  oracle on the shortest sequence so that the two restatements are seen to agree at this size."""
+  from oracle import c_oracle
+  ref = c_oracle.hstu_attention_c(q, k, v, seq_offsets=w.seq_offsets, max_len=w.L, n=w.n, alpha=w.alpha,
+                                  pos_tab=w.pos_tab, timestamps=w.timestamps, ts_tab=w.ts_tab, acc="f64")
+  scale = np.abs(ref).max()
+  assert np.isfinite(out).all()
+  per_seq = [np.abs(out[w.seq_offsets[b]:w.seq_offsets[b + 1]] - ref[w.seq_offsets[b]:w.seq_offsets[b + 1]]).max(initial=0.0) / scale
+             for b in range(w.B)]
+  worst = int(np.argmax(per_seq))
+  assert per_seq[worst] <= tol, f"sequence {worst} (length {w.seq_lens[worst]}): {per_seq[worst]}"
+  b = int(np.argmin(w.seq_lens))
+  ref_np = oracle_workload(w, q, k, v, dtype=np.float64, sequences=[b])
+  sl = slice(w.seq_offsets[b], w.seq_offsets[b + 1])
+  assert np.abs(ref_np[sl] - ref[sl]).max() / scale <= 1e-6
+
+
 def test_config3_full_size_bf16(gpu):
+  # the headline batch, all 64 sequences
   w = workloads.config3()
   q, k, v, out = run_workload(w, torch.bfloat16)
-  # oracle on the longest, the shortest and two middle sequences
-  order = np.argsort(w.seq_lens)
-  pick = [int(order[-1]), int(order[0]), int(order[len(order) // 2]), int(order[-2])]
-  ref = oracle_workload(w, q, k, v, dtype=np.float32, sequences=pick)
-  scale = np.abs(ref).max()
-  for b in pick:
-    s, e = w.seq_offsets[b], w.seq_offsets[b + 1]
-    assert np.abs(out[s:e] - ref[s:e]).max() / scale <= BF16_TOL, f"sequence {b}"
-  assert np.isfinite(out).all()
-
-
-def _spot_check_jagged(w, q, k, v, out, pick, tol):
-  ref = oracle_workload(w, q, k, v, dtype=np.float32, sequences=pick)
-  scale = np.abs(ref).max()
-  for b in pick:
-    s, e = w.seq_offsets[b], w.seq_offsets[b + 1]
-    assert np.abs(out[s:e] - ref[s:e]).max() / scale <= tol, f"sequence {b}"
-  assert np.isfinite(out).all()
+  _check_all_sequences_c(w, q, k, v, out, BF16_TOL)
 
 
 def test_config4_attention_full_size_bf16(gpu):
   # the attention call of the model configuration (B=128, L=1024, H=8, d=64, position bias only)
   w = workloads.config4_attention()
   q, k, v, out = run_workload(w, torch.bfloat16)
-  order = np.argsort(w.seq_lens)
-  _spot_check_jagged(w, q, k, v, out, [int(order[-1]), int(order[0]), int(order[len(order) // 2])], BF16_TOL)
+  _check_all_sequences_c(w, q, k, v, out, BF16_TOL)
 
 
 def test_config5_full_size_bf16_and_fp8(gpu):
   # the long-sequence configuration (B=32, L=4096, H=8, d=128): bf16, then fp8 q / k against the oracle on
-  # exactly the dequantised values; oracle on the shortest and the median sequence
+  # exactly the dequantised values; all 32 sequences, C oracle
   w = workloads.config5()
-  order = np.argsort(w.seq_lens)
-  pick = [int(order[0]), int(order[len(order) // 2])]
   q, k, v, out = run_workload(w, torch.bfloat16)
-  _spot_check_jagged(w, q, k, v, out, pick, BF16_TOL)
+  _check_all_sequences_c(w, q, k, v, out, BF16_TOL)
   q8, qs, qd = _quant(w.q)
   k8, ks, kd = _quant(w.k)
   out8 = recml_amd.hstu_attention(q8, k8, _dev(v, torch.bfloat16), q_scale=qs, k_scale=ks, seq_offsets=_dev(w.seq_offsets),
                                   max_len=w.L, n=w.n, alpha=w.alpha, pos_bias=_dev(w.pos_tab))
   torch.cuda.synchronize()
-  _spot_check_jagged(w, qd.astype(np.float32), kd.astype(np.float32), v, out8.float().cpu().numpy(), pick, BF16_TOL)
+  _check_all_sequences_c(w, qd.astype(np.float32), kd.astype(np.float32), v, out8.float().cpu().numpy(), BF16_TOL)
 
 
 @pytest.mark.parametrize("d", [32, 64, 128])
@@ -463,19 +462,22 @@ def test_dense_bias_with_lengths_on_matrix_cores(gpu):
 
 
 def test_dense_bias_large_on_matrix_cores(gpu):
-  # a longer case (several query tiles, the key range split over workgroups): against the general kernel,
-  # which the fp32 call takes, on the same bf16-rounded inputs
+  # a longer case (several query tiles, the key range split over workgroups) against the numpy oracle's
+  # dense layer form on the same bf16-rounded inputs; the general kernel (fp32 call) against it as well
   rng = np.random.default_rng(450)
   B, L, H, d = 2, 1040, 2, 64
   q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
   lens = np.array([1040, 333])
   pad = (np.arange(L)[None] < lens[:, None]).astype(np.float32)
-  mask = _dev(O.make_causal_mask(pad).astype(np.uint8))
-  bias = _dev(rng.standard_normal((B, L, L)).astype(np.float32) * 0.5)
+  mask_np = O.make_causal_mask(pad)
+  bias_np = rng.standard_normal((B, L, L)).astype(np.float32) * 0.5
+  mask, bias = _dev(mask_np.astype(np.uint8)), _dev(bias_np)
   got = recml_amd.pointwise_attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16), mask, bias)
-  ref = recml_amd.pointwise_attention(_dev(q), _dev(k), _dev(v), mask, bias)
+  gen = recml_amd.pointwise_attention(_dev(q), _dev(k), _dev(v), mask, bias)
   torch.cuda.synchronize()
-  assert _err(got.float().cpu().numpy(), ref.cpu().numpy()) <= BF16_TOL
+  ref = O.pointwise_attention_dense(q, k, v, mask_np, bias_np)
+  assert _err(got.float().cpu().numpy(), ref) <= BF16_TOL
+  assert _err(gen.cpu().numpy(), ref) <= FP32_TOL
   assert (got[1, 333:] == 0).all()
 
 
@@ -660,6 +662,21 @@ def test_sliding_window_on_the_matrix_core_kernel(gpu, d, L, window, causal, pos
   outj = recml_amd.hstu_attention(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), seq_offsets=_dev(off.astype(np.int32)), max_len=L,
                                   causal=causal, sliding_window_size=window, **gk)
   assert _err(O.jagged_to_padded(outj.float().cpu().numpy(), off, L), ref) <= BF16_TOL
+
+
+@pytest.mark.parametrize("window", [399, 400, 5000, 2 ** 31 - 1, 2 ** 40])
+def test_sliding_window_that_covers_everything(gpu, window):
+  """A window that reaches across the whole sequence restricts nothing (the reference's LocalMask
+  treats it so): same output as without a window, in both kernels, up to the largest values."""
+  rng = np.random.default_rng(7)
+  B, L, H, d = 2, 400, 2, 64
+  lens = np.array([L, 123], dtype=np.int32)
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  for dt_ in (torch.bfloat16, torch.float32):
+    for causal in (True, False):
+      run = lambda **kw: recml_amd.hstu_attention(_dev(q, dt_), _dev(k, dt_), _dev(v, dt_), seq_lens=_dev(lens), causal=causal, **kw)
+      plain, win = run(), run(sliding_window_size=window)
+      assert float(plain.float().abs().max()) > 0 and torch.equal(plain, win), (str(dt_), causal)
 
 
 @pytest.mark.parametrize("d,L,causal,window,pos", [

@@ -54,3 +54,43 @@ def test_fused_bias_and_table_gradients(gpu):
     a = dict(mod.named_parameters())[name].grad
     b = dict(ref_mod.named_parameters())[name].grad
     assert float((a - b).abs().max() / b.abs().max()) <= 2e-5, name
+
+
+def test_custom_bucketization_keeps_the_table_gradient():
+  """A custom bucketization function cannot be fused: the module hands the block a dense bias, and the
+  bias weights must still receive their gradient (through the plain torch form of the op), with frozen
+  block weights too.  Runs on the CPU: nothing here needs the HIP library."""
+  import torch
+  from recml_amd import hstu_bias, hstu_ops
+  from recml_amd.hstu_layer import HSTUBlock
+  torch.manual_seed(0)
+  B, L, D, H = 2, 12, 16, 2
+  sqrt_buckets = lambda x: torch.sqrt(x.abs().clamp(1, int(1e9)).double() / 3600.0).to(torch.int64)
+  mod = hstu_bias.RelativeBucketedTimeAndPositionBasedBias(L, num_buckets=16, bucketization_fn=sqrt_buckets)
+  ts = torch.cumsum(torch.randint(1, 20000, (B, L)), dim=1)
+  kw = mod.attention_kwargs(ts)
+  assert set(kw) == {"bias"} and kw["bias"].requires_grad
+  blk = HSTUBlock(D, H)
+  for p in blk.parameters():
+    p.requires_grad_(False)
+  x = torch.randn(B, L, D)
+  out = blk(x, seq_lens=torch.tensor([L, 7]), attention_bias=kw["bias"])
+  out.square().sum().backward()
+  assert mod._ts_w.grad is not None and float(mod._ts_w.grad.abs().max()) > 0
+  assert mod._positional_bias._pos_biases.grad is not None
+  # the fused autograd op refuses a dense bias it could not differentiate instead of dropping it
+  with pytest.raises(ValueError, match="requires a gradient"):
+    hstu_ops.hstu_attention_autograd(x.reshape(B, L, H, D // H), x.reshape(B, L, H, D // H), x.reshape(B, L, H, D // H),
+                                     bias=kw["bias"])
+  # and the torch form equals the dense oracle
+  from oracle import hstu_oracle as O
+  q, k, v = (torch.randn(B, L, H, 8) for _ in range(3))
+  lens = np.array([L, 7])
+  tsw, dense = torch.randn(17), torch.randn(B, L, L) * 0.1
+  pos = mod._positional_bias.table(L).detach()
+  got = hstu_ops.dense_attention_torch(q, k, v, seq_lens=torch.from_numpy(lens), pos_bias=pos, timestamps=ts, ts_bias=tsw,
+                                       bias=dense).numpy()
+  want = O.hstu_attention_ref(q.numpy(), k.numpy(), v.numpy(), seq_lens=lens, pos_tab=pos.numpy(), timestamps=ts.numpy(),
+                              ts_tab=tsw.numpy(), bias=dense.numpy())
+  assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+  assert (got[1, 7:] == 0).all()

@@ -155,6 +155,63 @@ def test_block_config4_shape_bf16(gpu):
   assert np.abs(got - ref).max() / np.abs(ref).max() <= 3e-2
 
 
+@pytest.mark.gpu
+def test_model_config4_full_size_bf16(gpu):
+  """BASELINE configuration 4 as a whole: 10 M x 512 bf16 embedding table (10.24 GB), Zipf(1.05) item ids,
+  4 blocks, D = 512, H = 8 (head dim 64), B = 128, L = 1024, lengths U{128..1024}, position bias; padded and
+  packed forward (recml/layers/keras/hstu.py:585-621), checked against the fp64 oracle on the longest, the
+  shortest and a median sequence, which also carry ids at the very end of the table (rows past 2^31 bytes /
+  row size would expose 32-bit addressing)."""
+  from recml_amd.hstu_layer import HSTU
+  free, _ = torch.cuda.mem_get_info()
+  if free < 16 << 30:
+    pytest.skip("needs 16 GB of free device memory")
+  rng = np.random.Generator(np.random.PCG64(4))
+  B, L, D, H, layers, vocab = 128, 1024, 512, 8, 4, 10_000_000
+  lens = rng.integers(128, L + 1, B).astype(np.int32)
+  lens[:2] = [L, 128]                                      # the longest and the shortest possible
+  ids = np.minimum(rng.zipf(1.05, (B, L)), vocab - 1).astype(np.int64)
+  order = np.argsort(lens, kind="stable")
+  pick = [int(order[-1]), int(order[0]), int(order[B // 2])]
+  for b in pick:                                           # ids near the end of the table in every checked sequence
+    ids[b, 5:9] = [vocab - 1, vocab - 2, vocab - 1000, 4_200_000]      # 4.2 M x 1 KB rows lies beyond 2^32 bytes
+  ids[np.arange(L)[None, :] >= lens[:, None]] = 0
+  dev = torch.device("cuda:0")
+  model = HSTU(vocab_size=8, max_positions=L, model_dim=D, num_heads=H, num_layers=layers, add_head=False,
+               dtype=torch.bfloat16, device=dev, seed=4)
+  table = torch.empty((vocab, D), dtype=torch.bfloat16, device=dev)
+  table.normal_(0.0, 0.01, generator=torch.Generator(device=dev).manual_seed(4))
+  model.item_embedding = torch.nn.Parameter(table, requires_grad=False)
+  pos = (torch.randn((2 * L - 1,), generator=torch.Generator().manual_seed(5)) * 0.02).to(dev)
+  ids_d, lens_d = torch.from_numpy(ids).to(dev), torch.from_numpy(lens).to(dev)
+  with torch.no_grad():
+    out = model(ids_d, seq_lens=lens_d, pos_bias=pos)
+    outj = model(ids_d, seq_lens=lens_d, pos_bias=pos, jagged=True)
+  torch.cuda.synchronize()
+  assert tuple(out.shape) == (B, L, D) and bool(torch.isfinite(out.float()).all())
+  # packed == padded on every valid position of the whole batch (the padded form carries the padding's own
+  # embeddings through the blocks, the packed form returns zeros there)
+  keep = (torch.arange(L, device=dev)[None, :] < lens_d[:, None])[:, :, None]
+  scale = float(out.float().abs().max())
+  assert float(((outj.float() - out.float()) * keep).abs().max()) / scale <= 2e-2
+  assert bool((outj.float() * ~keep == 0).all())
+  # the oracle on the three sequences: weights as stored (bf16 -> fp64), the table reduced to the rows they use
+  g = lambda t: t.detach().double().cpu().numpy()
+  sub = ids[pick]
+  uniq, inv = np.unique(sub, return_inverse=True)
+  w = {"item_embedding": g(table[torch.from_numpy(uniq).to(dev)]), "position_embedding": g(model.position_embedding),
+       "final_norm_gamma": g(model.final_norm_gamma), "final_norm_beta": g(model.final_norm_beta),
+       "blocks": [{n: g(p) for n, p in blk.named_parameters()} for blk in model.decoder_blocks]}
+  ref = BO.hstu_model(inv.reshape(sub.shape), w, num_heads=H, seq_lens=lens[pick], pos_tab=g(pos))
+  rs = np.abs(ref).max()
+  for row, b in enumerate(pick):
+    n = int(lens[b])
+    # bf16 activations between every step of four blocks: 3e-2 of the largest output (one block alone is held to 3e-2 too)
+    for name, got in (("padded", out), ("packed", outj)):
+      err = np.abs(got[b, :n].double().cpu().numpy() - ref[row, :n]).max() / rs
+      assert err <= 3e-2, (name, b, n, err)
+
+
 def _dense_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None, n=None, alpha=1.0, pos_bias=None, **_):
   """Differentiable dense torch form of the op (padded layout, causal, lengths, position table)."""
   B, L, H, d = q.shape

@@ -100,17 +100,18 @@ struct Params {
   float ts_bucket_size;
   float alpha, inv_n;
   int32_t n_qtiles;
-  // Key-range splitting (MFMA kernel; off when split_steps == 0): a query tile with more than
-  // split_steps 32-key steps is shared by up to MAX_CHUNKS workgroups, each covering a contiguous
-  // part of the keys and leaving its fp32 partial O^T in `partial`; hstu_combine sums them.
-  int32_t split_steps;
-  int32_t qt_split;          // first query tile that can be split
-  int32_t entries_per_bh;    // workgroups per (sequence, head): sum over query tiles of chunks_max
-  float* partial;            // [tile slot][head][chunk][BM x d_v floats in register order]
+  // Key-range splitting (MFMA forward; off when split_cap == 0): hstu_prepare, which sees the lengths,
+  // shares a query tile with more steps than a slot's average load between up to MAX_CHUNKS workgroups,
+  // each covering a contiguous part of the keys and leaving its fp32 partial O^T in `partial`; the
+  // workgroup that arrives last at the tile's counter sums them and writes the rows.
+  int32_t split_cap;         // chunk slots of the partial buffer (per head)
+  int32_t n_slots;           // workgroups that run at once per XCD (what the split decision balances for)
+  float* partial;            // [chunk slot][head][BM x d_v floats in register order]
+  uint32_t* ctr;             // workspace: [0, 16) reserved, then one arrival counter per (chunk slot, head)
   // Work list built on the device by hstu_prepare (MFMA kernel; null = workgroups enumerate every
-  // possible (sequence, tile, chunk) and most exit): sched[0] = number of items, then from
+  // possible (sequence, tile) and most exit): sched[0] = number of items, then from
   // sched[4] on one int4 per (sequence, query tile, chunk) that has work:
-  // {b, qt | chunk << 16, first token, stored length}.
+  // {b | first chunk slot << 14, qt | chunk << 16 | chunks << 24, first token, stored length}.
   const int32_t* sched;
   // backward pass: gradient of out in, gradients of q, k, v out (layouts of out, q, k, v), and
   // fp32 table gradients that are accumulated into (null = not wanted)
@@ -121,7 +122,6 @@ struct Params {
   float* dpos;
   float* dts;
   int64_t items_max;         // capacity of the list (sizes the grid)
-  int64_t split_max;         // capacity of the list of split tiles behind it: sched[1] int4s at sched + 4 + 4 items_max
 };
 
 // Per-sequence geometry shared by both kernels.
@@ -763,28 +763,8 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
 #define HSTU_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 15) | ((((n) >> 4) & 3) << 14)) | 0x0F70)
 
 constexpr int MAX_CHUNKS = 4;
+constexpr int CTR_RESERVED = 16;     // counters in front of the arrival counters
 
-// Most workgroups a query tile can be shared by (from its position alone), and how many share
-// it given its actual number of steps.
-__host__ __device__ __forceinline__ int chunks_max(int split_steps, int causal, int Lkv, int qt) {
-  if (split_steps <= 0) return 1;
-  const int all = (Lkv + BN - 1) / BN;
-  int nt = causal ? (qt + 1) * (BM / BN) : all;
-  nt = nt < all ? nt : all;
-  const int c = (nt + split_steps - 1) / split_steps;
-  return c < MAX_CHUNKS ? c : MAX_CHUNKS;
-}
-__device__ __forceinline__ int chunks_of(const Params& p, int nt) {
-  if (p.split_steps <= 0) return 1;
-  static_assert(MAX_CHUNKS == 4, "min(MAX_CHUNKS, ceil(nt / split_steps)) without a division");
-  const int s = p.split_steps;
-  return 1 + (nt > s ? 1 : 0) + (nt > 2 * s ? 1 : 0) + (nt > 3 * s ? 1 : 0);
-}
-// Slot of a split tile in the partial buffer: jagged sequences are packed by an upper bound of
-// the tiles before them.
-__device__ __forceinline__ int64_t partial_slot(const Params& p, int b, int64_t tok0, int qt) {
-  return (p.jagged ? (tok0 >> 7) + b : (int64_t)b * (p.n_qtiles - p.qt_split)) + (qt - p.qt_split);
-}
 // Steps of a tile: keys [0, kv_end) in 32-key steps
 __device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0) {
   int kv_end = s.n_kv;
@@ -800,14 +780,18 @@ __device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0)
 // launch order, the one with most keys first, so that the tiles running together stream the
 // same K/V rows and share them through that L2.  (Calls with a dense mask or bias are dealt
 // differently, see below.)  Returns false when there is nothing to do.
-struct Work { int b, h, qt, chunk; Seq s; };
-template <bool SPLIT_LIST = false>
+struct Work { int b, h, qt, chunk, n_chunks, pslot; Seq s; };
+__device__ __forceinline__ void work_from_item(const Params& p, const int4& item, int h, Work& wk) {
+  wk.b = item.x & 0x3fff; wk.pslot = (int)((uint32_t)item.x >> 14); wk.h = h;
+  wk.qt = item.y & 0xffff; wk.chunk = (item.y >> 16) & 0xff; wk.n_chunks = (int)((uint32_t)item.y >> 24);
+  wk.s = seq_from(p, wk.b, h, item.z, item.w);
+}
 __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, Work& wk) {
   const int xcd = block & 7, j = block >> 3;
   if (p.sched) {
     // from the work list: with H >= 8 head h runs on XCD h % 8, else 8 / H items share a round
     int it, h;
-    if (!SPLIT_LIST && (p.mask || p.dense_bias)) {
+    if (p.mask || p.dense_bias) {
       // Dense operands are shared by the heads, not by the query tiles: the H workgroups of an item
       // are neighbours on one XCD (they start together and fetch the same mask / bias tiles, so all
       // but the first find them in that L2), and runs of n_qtiles items -- the tiles of one full
@@ -822,25 +806,18 @@ __device__ __forceinline__ bool work_of_block(const Params& p, unsigned block, W
     // the item is read before the count is checked (the grid never reaches past the list's capacity):
     // both loads miss the cache, and one after the other they cost a workgroup twice the latency
     // (the dense mapping rounds its grid up to whole rounds of eight runs: indices past the capacity read item 0)
-    const int it_ld = (SPLIT_LIST || it < p.items_max) ? it : 0;
-    const int4 item = ((const int4*)(p.sched + 4))[(SPLIT_LIST ? p.items_max : 0) + it_ld];
-    if (it >= p.sched[SPLIT_LIST ? 1 : 0]) return false;
-    wk.b = item.x; wk.h = h; wk.qt = item.y & 0xffff; wk.chunk = item.y >> 16;
-    wk.s = seq_from(p, wk.b, h, item.z, item.w);
+    const int it_ld = it < p.items_max ? it : 0;
+    const int4 item = ((const int4*)(p.sched + 4))[it_ld];
+    if (it >= p.sched[0]) return false;
+    work_from_item(p, item, h, wk);
     return true;
   }
-  // without a list: entry -> (query tile, chunk of its key range), tiles from the last one down
-  const int bhk = j / p.entries_per_bh;
-  int qt = p.n_qtiles - 1, chunk = j - bhk * p.entries_per_bh;
-  for (;;) {
-    const int c = chunks_max(p.split_steps, p.causal, p.Lkv, qt);
-    if (chunk < c) break;
-    chunk -= c;
-    --qt;
-  }
+  // without a list: one entry per (sequence, head, query tile), tiles from the last one down, never split
+  const int bhk = j / p.n_qtiles;
+  const int qt = p.n_qtiles - 1 - (j - bhk * p.n_qtiles);
   const int bh = bhk * 8 + xcd;
   if (bh >= p.B * p.H) return false;
-  wk.b = bh / p.H; wk.h = bh - wk.b * p.H; wk.qt = qt; wk.chunk = chunk;
+  wk.b = bh / p.H; wk.h = bh - wk.b * p.H; wk.qt = qt; wk.chunk = 0; wk.n_chunks = 1; wk.pslot = 0;
   wk.s = seq_info(p, wk.b, wk.h);
   return true;
 }
@@ -922,14 +899,15 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
   const int tid = threadIdx.x;
   const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
   if (sched_out && blockIdx.x == gridDim.x - 1) {
-    // The work lists, by the last workgroup (the host launches one more than the rest needs).
+    // The work list, by the last workgroup (the host launches one more than the rest needs).
     // Sequences are taken longest first (batches of up to SORT_MAX sequences; larger ones in
     // batch order): the tiles with most keys start first and short ones fill in behind them.
-    // Thread t owns a run of sequences in that order, counts their items, finds where they start
-    // from the counts of the threads before it, and writes them out, last query tile (most keys)
-    // first within a sequence.  Items with chunk 1 also go to the list of split tiles.
+    // Thread t owns a run of sequences in that order.  Three walks over its tiles: the steps of all
+    // tiles (what decides which tiles are split), the chunk slots its split tiles ask for, and the
+    // items themselves, last query tile (most keys) first within a sequence; a prefix sum over the
+    // threads after the second and the third tells where a thread's slots and items start.
     constexpr int SORT_MAX = 1024;
-    __shared__ int counts[4], counts_split[4];
+    __shared__ int wave_sums[4];
     __shared__ int keys[SORT_MAX], firsts[SORT_MAX], order[SORT_MAX];
     const bool sorted = p.B <= SORT_MAX;
     if (sorted) {
@@ -952,60 +930,98 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     const int per = (p.B + 255) / 256;
     const int r_lo = tid * per < p.B ? tid * per : p.B, r_hi = r_lo + per < p.B ? r_lo + per : p.B;
     int4* items = (int4*)(sched_out + 4);
-    int4* split_items = items + p.items_max;
-    auto walk = [&](int b, int base, int base_split, bool write, int& n_split) {
-      int o0, nraw;
+    // sum over the workgroup and exclusive prefix of this thread's value (all 256 threads take part)
+    auto block_scan = [&](int v, int& total) {
+      int inc = v;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int a = __shfl_up(inc, d, 64);
+        if ((tid & 63) >= d) inc += a;
+      }
+      __syncthreads();            // the previous scan's readers are done with wave_sums
+      if ((tid & 63) == 63) wave_sums[tid >> 6] = inc;
+      __syncthreads();
+      int base = inc - v;
+      total = 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        base += i < (tid >> 6) ? wave_sums[i] : 0;
+        total += wave_sums[i];
+      }
+      return base;
+    };
+    auto seq_of = [&](int r, int& b, int& o0, int& nraw) {
+      b = sorted ? order[r] : r;
       if (sorted) { o0 = firsts[b]; nraw = keys[b]; }
       else seq_raw(p, b, o0, nraw);
-      const Seq sq = seq_from(p, b, 0, o0, nraw);
-      int n = 0;
-      n_split = 0;
-      if (!write && p.split_steps <= 0) return (sq.rows + BM - 1) / BM;   // one item per tile: no need to walk them to count
-      for (int qt = (sq.rows + BM - 1) / BM - 1; qt >= 0; --qt) {
-        const int c = qt * BM >= sq.n_q ? 1 : chunks_of(p, tile_steps(p, sq, qt * BM));
-        for (int k = 0; k < c; ++k, ++n) {
-          const int4 it = int4{b, qt | (k << 16), o0, nraw};
-          if (write && base + n < p.items_max) items[base + n] = it;
-          if (k == 1) {
-            if (write && base_split + n_split < p.split_max) split_items[base_split + n_split] = it;
-            ++n_split;
+      return seq_from(p, b, 0, o0, nraw);
+    };
+    // chunks of a tile of nt steps once the threshold is known: balanced parts of at most split_steps
+    auto chunks_of = [&](int nt, int split_steps) {
+      if (split_steps <= 0 || nt <= split_steps) return 1;
+      const int c = (nt + split_steps - 1) / split_steps;
+      return c < MAX_CHUNKS ? c : MAX_CHUNKS;
+    };
+    int split_steps = 0;
+    if (p.split_cap > 0) {
+      int steps = 0;
+      for (int r = r_lo; r < r_hi; ++r) {
+        int b, o0, nraw;
+        const Seq sq = seq_of(r, b, o0, nraw);
+        for (int q0 = 0; q0 < sq.n_q; q0 += BM) steps += tile_steps(p, sq, q0);
+      }
+      int total;
+      block_scan(steps, total);
+      // steps one slot of an XCD gets on average: with H >= 8 an XCD runs H / 8 heads of every item,
+      // else 8 / H XCDs share the items of one head
+      const long long per_xcd = p.H >= 8 ? (long long)total * (p.H >> 3) : (long long)total / (8 / p.H);
+      const long long avg = (per_xcd + p.n_slots - 1) / p.n_slots;
+      split_steps = avg < 8 ? 8 : (avg > 0x3fffffff ? 0x3fffffff : (int)avg);
+    }
+    // chunk slots this thread's split tiles ask for, then where they start
+    int want = 0;
+    for (int r = r_lo; r < r_hi && split_steps > 0; ++r) {
+      int b, o0, nraw;
+      const Seq sq = seq_of(r, b, o0, nraw);
+      for (int q0 = 0; q0 < sq.n_q; q0 += BM) {
+        const int c = chunks_of(tile_steps(p, sq, q0), split_steps);
+        want += c > 1 ? c : 0;
+      }
+    }
+    int total_slots = 0;
+    const int slot0 = split_steps > 0 ? block_scan(want, total_slots) : 0;
+    // one walk shared by the count and the write: a tile is split only while chunk slots last
+    auto walk = [&](int base, bool write) {
+      int n = 0, slot = slot0;
+      for (int r = r_lo; r < r_hi; ++r) {
+        int b, o0, nraw;
+        const Seq sq = seq_of(r, b, o0, nraw);
+        for (int qt = (sq.rows + BM - 1) / BM - 1; qt >= 0; --qt) {
+          int c = 1, ps = 0;
+          if (qt * BM < sq.n_q) {
+            c = chunks_of(tile_steps(p, sq, qt * BM), split_steps);
+            if (c > 1) {
+              ps = slot;
+              slot += c;
+              if (ps + c > p.split_cap) c = 1;      // the partial buffer is full: this tile stays whole
+            }
           }
+          for (int k = 0; k < c; ++k, ++n)
+            if (write && base + n < p.items_max) items[base + n] = int4{b | (ps << 14), qt | (k << 16) | (c << 24), o0, nraw};
         }
       }
       return n;
     };
-    int cnt = 0, cnt_split = 0;
-    for (int r = r_lo; r < r_hi; ++r) {
-      int ns;
-      cnt += walk(sorted ? order[r] : r, 0, 0, false, ns);
-      cnt_split += ns;
-    }
-    // exclusive prefix sums over the 256 threads: within the wave by shuffles, across the 4 waves by LDS
-    int inc = cnt, inc_split = cnt_split;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const int a = __shfl_up(inc, d, 64), c = __shfl_up(inc_split, d, 64);
-      if ((tid & 63) >= d) { inc += a; inc_split += c; }
-    }
-    if ((tid & 63) == 63) { counts[tid >> 6] = inc; counts_split[tid >> 6] = inc_split; }
-    __syncthreads();
-    int base = inc - cnt, total = 0, base_split = inc_split - cnt_split, total_split = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      base += i < (tid >> 6) ? counts[i] : 0;
-      total += counts[i];
-      base_split += i < (tid >> 6) ? counts_split[i] : 0;
-      total_split += counts_split[i];
-    }
-    for (int r = r_lo; r < r_hi; ++r) {
-      int ns;
-      base += walk(sorted ? order[r] : r, base, base_split, true, ns);
-      base_split += ns;
-    }
+    int total;
+    const int base = block_scan(walk(0, false), total);
+    walk(base, true);
     if (tid == 0) {
       sched_out[0] = total < p.items_max ? total : (int)p.items_max;
-      sched_out[1] = total_split < p.split_max ? total_split : (int)p.split_max;
+      sched_out[1] = split_steps;
     }
+    // the arrival counters of the split tiles start at zero (their last arriver leaves them so again)
+    if (p.ctr)
+      for (int i = tid; i < CTR_RESERVED + p.split_cap * p.H; i += 256) p.ctr[i] = 0u;
   }
   if (tab_out) {
     // every head's bucket table: thresholds and buckets from the host, the table values times log2(e) with
@@ -1103,6 +1119,7 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 // workgroups per CU to four (measured: 148 -> 139 us on the d = 64 benchmark shape).  At d = 128
 // registers allow two workgroups whatever the ring, and the depth makes no measurable difference.
 constexpr int fwd_stages(int d, int dense) { return (d <= 64 && dense == 0) ? 3 : 4; }
+constexpr int FWD_XCH_BYTES = 16;     // behind everything else in the forward kernel's LDS
 
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
@@ -1140,6 +1157,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   constexpr int DENSE_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
   constexpr int DENSE_STAGE = SM::dense_stage(DENSE);
+  constexpr int XCH_OFF = DENSE_OFF + NSTAGE * DENSE_STAGE;   // 16 bytes for values one lane hands to the workgroup
   auto Db = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE; };
   auto Dm = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE + ((DENSE & 1) ? SM::DB_BYTES : 0); };
 
@@ -1174,16 +1192,16 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const int qrow = r0 + m;             // this lane's query row
   const bool wave_live = r0 < s.n_q;
 
-  // this workgroup's steps [t_lo, nt) of the tile's
+  // this workgroup's steps [t_lo, nt) of the tile's: the whole tile, or balanced part `chunk` of n_chunks
+  // (a part can be empty only if the list were inconsistent; such a workgroup still arrives below)
   int nt = tile_steps(p, s, q0);
-  const int n_chunks = chunks_of(p, nt);
-  if (chunk >= n_chunks) return;
+  const int n_chunks = wk.n_chunks;
   int t_lo = 0;
   if (n_chunks > 1) {
     const int per = (nt + n_chunks - 1) / n_chunks;
     t_lo = chunk * per;
+    t_lo = t_lo < nt ? t_lo : nt;
     nt = t_lo + per < nt ? t_lo + per : nt;
-    if (t_lo >= nt) return;    // cannot happen for n_chunks = ceil(nt / split_steps) <= nt, kept as a guard
   }
   // a sliding window (never combined with key-range splitting) also drops the steps before the tile's first key
   const int win = p.window;
@@ -1619,13 +1637,56 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0.
   // The 1/log2(e) left out of the SiLU is folded into the output scale.
   if (n_chunks > 1) {
-    // fp32 partial in register order: float4 number (16 w + i) * 64 + lane of this (tile, head, chunk)
-    floatx4* dst = (floatx4*)(p.partial + ((partial_slot(p, b, s.tok0, qt) * p.H + h) * MAX_CHUNKS + chunk) * (int64_t)(BM * D)) +
-                   (w * (DVB * 4)) * 64 + lane;
+    // This workgroup covered part of the tile's keys.  It leaves its fp32 partial O^T (register order:
+    // 8-byte piece (16 w + i) * 128 + 2 lane + j of the chunk's slot) in the workspace and counts itself
+    // in at the tile's arrival counter; the workgroup that arrives last adds the others' partials to
+    // its own, always in the order of the chunks, and writes the rows.  Partials and counter go by
+    // device-scope atomic stores, loads and adds (which bypass the caches that are not coherent across
+    // the chip), ordered by waiting for the stores' completion before the count: no cache is flushed,
+    // and nothing depends on which workgroup runs where.  The result does not depend on the order of
+    // arrival.
+    constexpr int NPC = BM * D / 2;      // 8-byte pieces of a chunk's partial
+    uint64_t* slot0 = (uint64_t*)p.partial + ((int64_t)wk.pslot * p.H + h) * NPC;
+    uint64_t* mine = slot0 + (int64_t)chunk * p.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane;
 #pragma unroll
-    for (int i = 0; i < DVB * 4; ++i)
-      dst[i * 64] = floatx4{o[i >> 2][4 * (i & 3) + 0], o[i >> 2][4 * (i & 3) + 1], o[i >> 2][4 * (i & 3) + 2], o[i >> 2][4 * (i & 3) + 3]};
-    return;
+    for (int i = 0; i < DVB * 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        // (through named floats: a bit cast applied to a vector element directly reads element 0)
+        const float f0 = o[i >> 2][4 * (i & 3) + 2 * j], f1 = o[i >> 2][4 * (i & 3) + 2 * j + 1];
+        const uint64_t bits = (uint64_t)__builtin_bit_cast(uint32_t, f0) | ((uint64_t)__builtin_bit_cast(uint32_t, f1) << 32);
+        __hip_atomic_store(mine + i * 128 + j, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    HSTU_WAIT_VMCNT(0);                  // every store of this wave has been acknowledged
+    __syncthreads();
+    uint32_t* xch = (uint32_t*)(smem + XCH_OFF);
+    uint32_t* arrive = p.ctr + CTR_RESERVED + wk.pslot * p.H + h;
+    if (tid == 0) *xch = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    const uint32_t before = *xch;
+    if (before != (uint32_t)(n_chunks - 1)) return;
+    if (tid == 0) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next call
+#pragma unroll
+    for (int i = 0; i < DVB * 4; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float a0 = 0.f, a1 = 0.f;
+        for (int c = 0; c < n_chunks; ++c) {
+          float x0 = o[i >> 2][4 * (i & 3) + 2 * j], x1 = o[i >> 2][4 * (i & 3) + 2 * j + 1];
+          if (c != chunk) {
+            const uint64_t bits = __hip_atomic_load(slot0 + (int64_t)c * p.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane + i * 128 + j,
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            x0 = __builtin_bit_cast(float, (uint32_t)bits);
+            x1 = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+          }
+          a0 += x0;
+          a1 += x1;
+        }
+        o[i >> 2][4 * (i & 3) + 2 * j] = a0;
+        o[i >> 2][4 * (i & 3) + 2 * j + 1] = a1;
+      }
+    }
   }
   // Each wave turns its O^T fragment into whole output rows through LDS (the ring is free now: the
   // loop ended on a barrier and no load is in flight), so that global memory sees 16-byte stores that
@@ -1665,62 +1726,6 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
       const uintx4 vv = {val.x, val.y, val.z, val.w};
       __builtin_nontemporal_store(vv, (uintx4*)(og + (int64_t)grow * p.o_st + cc * 8));
-    }
-  }
-}
-
-// Sums the fp32 partials of the query tiles whose key range was split and writes their
-// output rows.  One workgroup per (sequence, head, splittable tile) with the lane roles of the
-// main kernel, so that each lane reads back exactly what lanes in its place wrote.
-template <int D>
-__global__ __launch_bounds__(MFMA_THREADS) void hstu_combine(const Params p) {
-  constexpr int DVB = D / 32;
-  // with a work list: one workgroup per entry of the list of split tiles; without: launched over
-  // the main kernel's grid, and the workgroup that has chunk 1 of a tile sums it
-  Work wk;
-  if (!work_of_block<true>(p, blockIdx.x, wk)) return;
-  if (wk.chunk != 1) return;
-  const int b = wk.b, h = wk.h, qt = wk.qt;
-  const Seq& s = wk.s;
-  const int q0 = qt * BM;
-  if (q0 >= s.n_q) return;
-  const int n_chunks = chunks_of(p, tile_steps(p, s, q0));
-  if (n_chunks <= 1) return;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int m = lane & 31, hh = lane >> 5;
-  const int qrow = q0 + 32 * w + m;
-  const floatx4* src = (const floatx4*)(p.partial + ((partial_slot(p, b, s.tok0, qt) * p.H + h) * MAX_CHUNKS) * (int64_t)(BM * D)) +
-                       (w * (DVB * 4)) * 64 + lane;
-  const float oscale = p.inv_n * (1.0f / LOG2E);
-  if (qrow >= s.rows) return;
-  const bool live = qrow < s.n_q;
-  bf16_t* orow = (bf16_t*)p.out + s.bo + (int64_t)qrow * p.o_st + 4 * hh;
-  // Every chunk slot is read, absent ones as a repeat of chunk 0 with weight 0, so that all the
-  // loads of a group are independent and in flight together.
-  constexpr int NP = DVB * 4, GRP = NP < 8 ? NP : 8;
-  const int c2 = n_chunks > 2 ? 2 : 0, c3 = n_chunks > 3 ? 3 : 0;
-  const float w2 = n_chunks > 2 ? 1.f : 0.f, w3 = n_chunks > 3 ? 1.f : 0.f;
-  constexpr int CS = BM * D / 4;   // float4s per chunk
-#pragma unroll
-  for (int g0 = 0; g0 < NP; g0 += GRP) {
-    floatx4 v0[GRP], v1[GRP], v2[GRP], v3[GRP];
-#pragma unroll
-    for (int i = 0; i < GRP; ++i) {
-      v0[i] = src[(g0 + i) * 64];
-      v1[i] = src[(g0 + i) * 64 + CS];
-      v2[i] = src[(g0 + i) * 64 + c2 * CS];
-      v3[i] = src[(g0 + i) * 64 + c3 * CS];
-    }
-#pragma unroll
-    for (int i = 0; i < GRP; ++i) {
-      const floatx4 a = v0[i] + v1[i] + v2[i] * w2 + v3[i] * w3;
-      uint2 pko = {0u, 0u};
-      if (live) {
-        pko.x = pack_bf16(a.x * oscale, a.y * oscale);
-        pko.y = pack_bf16(a.z * oscale, a.w * oscale);
-      }
-      const int ii = g0 + i;
-      *(uint2*)(orow + 32 * (ii >> 2) + 8 * (ii & 3)) = pko;
     }
   }
 }
@@ -2889,56 +2894,35 @@ Variant pick_variant(const HstuAttnFwdArgs* a) {
 // Workspace of the MFMA kernel: [scaled, padded position table][per-sequence int32-timestamp flag]
 // [int32 timestamps][their (min, max) per key tile], each part a multiple of 256 bytes.
 struct WorkspacePlan {
-  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes, sched_bytes, partial_bytes;
-  int split_steps, qt_split, entries_per_bh;
-  long long items_max, split_max;   // capacities of the work list and of the list of split tiles (0 = no list)
+  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes, sched_bytes, ctr_bytes, partial_bytes;
+  int split_cap;          // chunk slots of the partial buffer (0: no tile is split)
+  long long items_max;    // capacity of the work list (0 = no list)
   size_t bias_total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes; }
-  size_t total() const { return bias_total() + sched_bytes + partial_bytes; }
+  size_t total() const { return bias_total() + sched_bytes + ctr_bytes + partial_bytes; }
 };
 
-WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) {
-  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+// Chunk slots the partial buffer is sized for.  A tile is only split when it has more steps than a
+// slot's average load, so at most (slots per XCD) tiles per head ask for it, and few do in practice
+// (the headline batch: 14 tiles, 28 chunks); tiles beyond the capacity simply stay whole.
+constexpr int SPLIT_CAP_DEFAULT = 32;
+
+// max_bytes: a workspace this small must do (the split capacity is cut down to fit it).
+WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, size_t max_bytes = ~(size_t)0) {
+  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const Variant var = pick_variant(a);
   if (var != V_MFMA_BF16 && var != V_MFMA_FP8) return w;
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
-  // Key-range splitting pays when there are fewer query tiles than the GPU runs at once (512
-  // workgroups) or little more: then the tile with most keys sets the run time.  With more tiles,
-  // taking the longest sequences first keeps the GPU busy behind it and the extra pass that sums
-  // the partials costs more than it saves.  The lengths are on the device, so the decision rests
-  // on what the shapes allow.
   const int n_qtiles = (a->L + BM - 1) / BM;
-  const int steps_max = (a->Lkv + BN - 1) / BN;
   const bool jag = a->layout == HSTU_LAYOUT_JAGGED;
-  const long long tiles_est = (long long)a->H * (jag ? (a->total_tokens / BM + a->B) : (long long)a->B * n_qtiles);
-  w.entries_per_bh = n_qtiles;
-  if (allow_split && effective_window(a) < 0 && tiles_est < 1024 && steps_max > 16) {
-    w.split_steps = (steps_max + MAX_CHUNKS - 1) / MAX_CHUNKS;
-    w.split_steps = w.split_steps < 16 ? 16 : w.split_steps;
-    // first tile with more steps than that (a causal tile qt has up to 4 (qt + 1) steps)
-    w.qt_split = a->causal ? w.split_steps / (BM / BN) : 0;
-    if (w.qt_split >= n_qtiles) {
-      // causal with fewer query rows than keys: no tile reaches that many steps
-      w.split_steps = 0;
-      w.qt_split = 0;
-    } else {
-      w.entries_per_bh = 0;
-      for (int qt = 0; qt < n_qtiles; ++qt) w.entries_per_bh += chunks_max(w.split_steps, a->causal != 0, a->Lkv, qt);
-      const size_t slots = jag ? (size_t)(a->total_tokens / BM) + (size_t)a->B + 1 : (size_t)a->B * (size_t)(n_qtiles - w.qt_split);
-      w.partial_bytes = up(slots * (size_t)a->H * MAX_CHUNKS * (size_t)BM * (size_t)a->d_v * sizeof(float));
-    }
-  }
   // A work list built on the device spares the launch of workgroups that would find nothing to do
   // (a jagged batch with a long maximum length and mostly short sequences is mostly such).  Its
   // head mapping needs H to divide 8 or 8 to divide H; its builder is one workgroup.
-  if ((a->H % 8 == 0 || 8 % a->H == 0) && a->B <= 8192) {
-    const long long t128 = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
-    // every tile one item, plus up to MAX_CHUNKS - 1 more for each tile that can be split
-    const long long extra = w.split_steps ? (MAX_CHUNKS - 1) * (jag ? a->total_tokens / BM + 1 + (w.qt_split ? 0 : a->B)
-                                                                          : (long long)a->B * (n_qtiles - w.qt_split)) : 0;
-    w.items_max = t128 + extra;
-    w.split_max = extra / (MAX_CHUNKS - 1);
-    w.sched_bytes = up((size_t)(4 + 4 * (w.items_max + w.split_max)) * sizeof(int32_t));
-  }
+  const bool list = (a->H % 8 == 0 || 8 % a->H == 0) && a->B <= 8192;
+  // Key-range splitting (decided per tile by the preparation kernel, which sees the lengths) needs the list.
+  // (no tile of at most 8 steps is ever split; a tile takes at most MAX_CHUNKS slots)
+  const long long t128_all = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
+  if (list && allow_split && effective_window(a) < 0 && (a->Lkv + BN - 1) / BN > 8)
+    w.split_cap = (int)(t128_all * MAX_CHUNKS < SPLIT_CAP_DEFAULT ? t128_all * MAX_CHUNKS : SPLIT_CAP_DEFAULT);
   if (a->pos_tab) w.pos_bytes = up((size_t)a->pos_heads * (size_t)(2 * a->L - 1 + 2 * POS_PAD) * sizeof(float));
   if (a->ts_tab) {
     const size_t tiles_per_seq = (size_t)((a->L + BN - 1) / BN);
@@ -2950,6 +2934,20 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true) 
     // the kernels fetch whole 16-byte pieces: up to 35 timestamps and one range past the end
     w.rel_bytes = up(n_ts * sizeof(int32_t) + 160);
     w.range_bytes = up(tiles * 2 * sizeof(int32_t) + 16);
+  }
+  const long long t128 = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
+  const size_t chunk_bytes = (size_t)a->H * (size_t)BM * (size_t)a->d_v * sizeof(float);
+  for (;;) {
+    if (list) {
+      w.items_max = t128 + w.split_cap;     // every tile one item, and one more per chunk slot at most
+      w.sched_bytes = up((size_t)(4 + 4 * w.items_max) * sizeof(int32_t));
+    }
+    w.ctr_bytes = w.split_cap ? up((size_t)(CTR_RESERVED + (size_t)w.split_cap * a->H) * sizeof(uint32_t)) : 0;
+    w.partial_bytes = up((size_t)w.split_cap * chunk_bytes);
+    if (w.total() <= max_bytes || w.split_cap == 0) break;
+    const size_t over = w.total() - max_bytes;
+    const int fewer = (int)((over + chunk_bytes - 1) / chunk_bytes);
+    w.split_cap = w.split_cap - fewer >= 2 ? w.split_cap - fewer : 0;
   }
   return w;
 }
@@ -3008,18 +3006,18 @@ int launch_general(const Params& p, hipStream_t st) {
   return HSTU_OK;
 }
 
-// Workgroups of the main kernel (and of the combine kernel, which shares its mapping).
-long long mfma_grid(const Params& p, bool split_list = false) {
+// Workgroups of the main kernel.
+long long mfma_grid(const Params& p) {
   if (p.sched) {
-    const long long n = split_list ? p.split_max : p.items_max;
-    if (!split_list && (p.mask || p.dense_bias)) {
+    const long long n = p.items_max;
+    if (p.mask || p.dense_bias) {
       const long long groups = (n + p.n_qtiles - 1) / p.n_qtiles;     // runs of n_qtiles items, eight runs a round
       return 8LL * ((groups + 7) / 8) * p.n_qtiles * p.H;
     }
     const long long rounds = p.H >= 8 ? n * (p.H / 8) : (n + 8 / p.H - 1) / (8 / p.H);
     return 8LL * rounds;
   }
-  return 8LL * p.entries_per_bh * (((long long)p.B * p.H + 7) / 8);
+  return 8LL * p.n_qtiles * (((long long)p.B * p.H + 7) / 8);
 }
 
 template <typename T>
@@ -3041,7 +3039,7 @@ int launch_bwd(const Params& p, hipStream_t st) {
 
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE, fwd_stages(D, DENSE));
+  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE, fwd_stages(D, DENSE)) + FWD_XCH_BYTES;
   static int granted[64];
   if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE>, smem, granted)) return rc;
   hipError_t e;
@@ -3087,12 +3085,31 @@ int launch_mfma(const Params& p, hipStream_t st) {
 }
 
 
+// Workgroups of the forward kernel that run at once on one XCD (an eighth of the chip): what the
+// preparation kernel balances the split of long tiles for.  Two workgroups per compute unit at
+// d = 128, four below, one with dense operands; the count of compute units is read once per device.
+int slots_per_xcd(const Params& p, int32_t* out) {
+  constexpr int kMaxDev = 64;
+  static int cus[kMaxDev];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  int n = (dev >= 0 && dev < kMaxDev) ? __atomic_load_n(&cus[dev], __ATOMIC_ACQUIRE) : 0;
+  if (n <= 0) {
+    e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || n <= 0) return fail(HSTU_ERR_LAUNCH, "hipDeviceGetAttribute(multiprocessor count): %s", hipGetErrorString(e));
+    if (dev >= 0 && dev < kMaxDev) __atomic_store_n(&cus[dev], n, __ATOMIC_RELEASE);
+  }
+  const int per_cu = (p.mask || p.dense_bias) ? 1 : (p.d_qk <= 64 ? 4 : 2);
+  const int slots = n * per_cu / 8;
+  *out = slots > 0 ? slots : 1;
+  return HSTU_OK;
+}
+
 // Points the workspace fields of `q` into the caller's buffer as `ws` lays it out and enqueues the
 // kernel that fills it (unless the caller says it is filled already).
 int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params& q, hipStream_t st) {
-  q.split_steps = ws.split_steps;
-  q.qt_split = ws.qt_split;
-  q.entries_per_bh = ws.entries_per_bh;
+  q.split_cap = ws.split_cap;
   if (!ws.total()) return HSTU_OK;
   if (!args->workspace || args->workspace_bytes < ws.total())
     return fail(HSTU_ERR_WORKSPACE, "workspace of %zu bytes needed (see hstu_attn_fwd_workspace_bytes), got %zu",
@@ -3109,8 +3126,9 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
   q.sched = sched_out;
   q.items_max = ws.items_max;
-  q.split_max = ws.split_max;
-  q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
+  q.ctr = ws.ctr_bytes ? (uint32_t*)(base + ws.bias_total() + ws.sched_bytes) : nullptr;
+  q.partial = ws.partial_bytes ? (float*)(base + ws.bias_total() + ws.sched_bytes + ws.ctr_bytes) : nullptr;
+  if (int rc = slots_per_xcd(q, &q.n_slots)) return rc;
   q.ts_keyed = tab_out;
   q.pos_scaled = pos_out;
   q.ts_ok = ok_out;
@@ -3292,7 +3310,7 @@ int hstu_attn_fwd_noalloc(const HstuAttnFwdArgs* args, void* stream) {
   HstuAttnFwdArgs a = *args;
   a.workspace = nullptr;
   a.workspace_bytes = 0;
-  const size_t need = plan_workspace(&a).total();
+  const size_t need = plan_workspace(&a, true, (size_t)HSTU_ATTN_NOALLOC_SCRATCH_BYTES).total();
   if (need > (size_t)HSTU_ATTN_NOALLOC_SCRATCH_BYTES)
     return fail(HSTU_ERR_WORKSPACE, "this call needs %zu bytes of scratch, the array built into the library holds %zu: "
                 "use hstu_attn_fwd with a caller workspace", need, (size_t)HSTU_ATTN_NOALLOC_SCRATCH_BYTES);
@@ -3318,18 +3336,11 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
     case V_MFMA_BF16:
     case V_MFMA_FP8: {
       const bool f8 = args->qk_dtype == HSTU_DTYPE_FP8_E4M3FN;
-      const WorkspacePlan ws = plan_workspace(args);
+      // the split capacity adapts to the workspace the caller brought (never below what the call needs)
+      const WorkspacePlan ws = plan_workspace(args, true, args->workspace ? args->workspace_bytes : 0);
       Params q = p;
       if (int rc2 = setup_workspace(args, ws, q, st)) return rc2;
       if (int rc2 = f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st)) return rc2;
-      const long long cb = q.split_steps > 0 ? mfma_grid(q, true) : 0;
-      if (cb > 0) {
-        if (q.d_v == 128) hipLaunchKernelGGL(hstu_combine<128>, dim3((unsigned)cb), dim3(MFMA_THREADS), 0, st, q);
-        else if (q.d_v == 64) hipLaunchKernelGGL(hstu_combine<64>, dim3((unsigned)cb), dim3(MFMA_THREADS), 0, st, q);
-        else hipLaunchKernelGGL(hstu_combine<32>, dim3((unsigned)cb), dim3(MFMA_THREADS), 0, st, q);
-        hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "combine kernel launch: %s", hipGetErrorString(e));
-      }
       return HSTU_OK;
     }
     default: return fail(HSTU_ERR_SHAPE, "no kernel for these arguments");

@@ -150,6 +150,16 @@ def test_variant_and_workspace_query():
   # ... plus, with a position table, its scaled and padded copy
   a.pos_tab, a.pos_heads = 0x20000, 4
   assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == up(4 * (2 * 256 - 1 + 512) * 4) + sched
+  # longer sequences can have query tiles whose key range is split over workgroups: room for the fp32
+  # partial sums of up to 32 chunks per head, their arrival counters, and 32 more list entries
+  a.pos_tab, a.pos_heads = None, 0
+  a.L = a.Lkv = 1024
+  a.q_stride_b = a.k_stride_b = a.v_stride_b = a.o_stride_b = 1024 * 4 * 128
+  full = lib.hstu_attn_fwd_workspace_bytes(C.byref(a))
+  assert full == up(16 + 16 * (2 * 8 + 32)) + up(4 * (16 + 32 * 4)) + 32 * 4 * 128 * 128 * 4
+  a.L = a.Lkv = 256
+  a.q_stride_b = a.k_stride_b = a.v_stride_b = a.o_stride_b = 256 * 4 * 128
+  a.pos_tab, a.pos_heads = 0x20000, 4
   # general-kernel calls need none
   # a launch without the workspace is refused before anything is enqueued
   assert lib.hstu_attn_fwd(C.byref(a), None) == -5

@@ -676,7 +676,14 @@ def test_sliding_window_that_covers_everything(gpu, window):
     for causal in (True, False):
       run = lambda **kw: recml_amd.hstu_attention(_dev(q, dt_), _dev(k, dt_), _dev(v, dt_), seq_lens=_dev(lens), causal=causal, **kw)
       plain, win = run(), run(sliding_window_size=window)
-      assert float(plain.float().abs().max()) > 0 and torch.equal(plain, win), (str(dt_), causal)
+      assert float(plain.float().abs().max()) > 0
+      if window >= L:
+        assert torch.equal(plain, win), (str(dt_), causal)        # passed on as "no window": the very same launch
+      else:
+        # the widest real window keeps every pair too; the window path sums a long tile in one piece
+        # where the plain path may split its keys: equal up to the rounding of the output
+        tol = 2.0 ** -7 if dt_ == torch.bfloat16 else 1e-6
+        assert float((plain.float() - win.float()).abs().max()) <= tol * float(plain.float().abs().max()), (str(dt_), causal)
 
 
 @pytest.mark.parametrize("d,L,causal,window,pos", [

@@ -466,6 +466,10 @@ def main():
   ap.add_argument("--backward", action="store_true", help="measure the backward pass instead of the forward")
   ap.add_argument("--no-graph", dest="graph", action="store_false",
                   help="skip the variant that replays the timed calls as one HIP graph")
+  ap.add_argument("--one-item-per-workgroup", action="store_true",
+                  help="diagnostics: force one workgroup per work-list entry")
+  ap.add_argument("--resident-workgroups", action="store_true",
+                  help="diagnostics: force resident workgroups that loop over the work list")
   ap.add_argument("--calib-copy", action="store_true",
                   help="also run one 512 MiB device copy (reference point for HBM byte counters)")
   args = ap.parse_args()
@@ -495,6 +499,11 @@ def main():
   out = torch.empty_like(v)
   call_args, keep = hstu_ops.build_args(q, k, v, out, **kw)
   variant = hstu_ops.kernel_variant(call_args)
+  from recml_amd import _lib
+  if args.one_item_per_workgroup:
+    call_args.flags |= _lib.FWD_ONE_ITEM_PER_WORKGROUP
+  if args.resident_workgroups:
+    call_args.flags |= _lib.FWD_RESIDENT_WORKGROUPS
 
   def step():
     hstu_ops._run(call_args, keep)

@@ -62,7 +62,21 @@ enum HstuFwdFlags {
    * shapes, lengths / offsets, timestamps and bias tables (for example the
    * same call repeated, or a benchmark timing the main kernel alone): skip
    * the preparation kernel.  Undefined results if that does not hold. */
-  HSTU_FWD_WORKSPACE_PREPARED = 1
+  HSTU_FWD_WORKSPACE_PREPARED = 1,
+  /* Only prepare the workspace (the kernel that builds the work list, the scaled
+   * tables and the int32 timestamps) and return: a model whose layers share
+   * lengths, timestamps and bias tables prepares once per batch and then calls
+   * every layer with HSTU_FWD_WORKSPACE_PREPARED and the same workspace. */
+  HSTU_FWD_PREPARE_ONLY = 2,
+  /* How the matrix-core kernel takes the entries of its work list (bf16,
+   * d = 128, no dense operands, no segment ids; ignored elsewhere): one
+   * workgroup per entry, or two resident workgroups per compute unit that
+   * draw entry after entry and start the next one's loads under the last steps
+   * of the one at hand.  By default the library picks the second when the
+   * batch has at least 8 entries per resident workgroup.  These bits force one
+   * or the other (the first wins); the results are the same bit for bit. */
+  HSTU_FWD_ONE_ITEM_PER_WORKGROUP = 4,
+  HSTU_FWD_RESIDENT_WORKGROUPS = 8
 };
 
 /* Return codes (0 = launched). */

@@ -14,6 +14,9 @@ ABI_VERSION = 1
 LAYOUT_PADDED, LAYOUT_JAGGED = 0, 1
 DTYPE_FP32, DTYPE_BF16, DTYPE_FP8_E4M3FN = 0, 1, 2
 FWD_WORKSPACE_PREPARED = 1
+FWD_PREPARE_ONLY = 2
+FWD_ONE_ITEM_PER_WORKGROUP = 4
+FWD_RESIDENT_WORKGROUPS = 8
 NOALLOC_SCRATCH_BYTES = 4 << 20   # HSTU_ATTN_NOALLOC_SCRATCH_BYTES
 MASK_NONE, MASK_LENGTH, MASK_SEGMENT = 0, 1, 2
 

@@ -106,8 +106,10 @@ struct Params {
   // workgroup that arrives last at the tile's counter sums them and writes the rows.
   int32_t split_cap;         // chunk slots of the partial buffer (per head)
   int32_t n_slots;           // workgroups that run at once per XCD (what the split decision balances for)
+  int32_t persist;           // forward: resident workgroups that loop over the work list
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
-  uint32_t* ctr;             // workspace: [0, 16) reserved, then one arrival counter per (chunk slot, head)
+  uint32_t* ctr;             // workspace: [0, 8) draw counters of the XCDs, [8] workgroups done, then from
+                             // CTR_RESERVED on one arrival counter per (chunk slot, head); all zero between launches
   // Work list built on the device by hstu_prepare (MFMA kernel; null = workgroups enumerate every
   // possible (sequence, tile) and most exit): sched[0] = number of items, then from
   // sched[4] on one int4 per (sequence, query tile, chunk) that has work:
@@ -699,6 +701,12 @@ struct MfmaSmem {
 };
 
 typedef __attribute__((address_space(3))) unsigned char* lds_byte_ptr;
+// A pointer that is the same for every lane, taken from the first lane into scalar registers.
+__device__ __forceinline__ const void* scalar_ptr(const void* p_) {
+  const uint64_t v = (uint64_t)(uintptr_t)p_;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
 
 // Direct global -> LDS loads, 64 lanes x 16 (or 4) bytes: lane l of the wave
 // writes LDS bytes [lds_base + size*l, +size) with the bytes at gbase +
@@ -1121,7 +1129,7 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 constexpr int fwd_stages(int d, int dense) { return (d <= 64 && dense == 0) ? 3 : 4; }
 constexpr int FWD_XCH_BYTES = 16;     // behind everything else in the forward kernel's LDS
 
-template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
+template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0, bool PERSIST = false>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   constexpr int KB = F8 ? 1 : 2;       // bytes per q / k element
   using SM = MfmaSmem<D, KB>;
@@ -1161,70 +1169,68 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Db = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE; };
   auto Dm = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE + ((DENSE & 1) ? SM::DB_BYTES : 0); };
 
-  Work wk;
-  if (!work_of_block(p, blockIdx.x, wk)) return;
-  const int b = wk.b, h = wk.h, qt = wk.qt, chunk = wk.chunk;
-  const Seq& s = wk.s;
-  const int q0 = qt * BM;
-  if (q0 >= s.rows) return;
-  if (chunk > 0 && q0 >= s.n_q) return;
-
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave index, kept scalar
   const int m = lane & 31, hh = lane >> 5;
-  const char* __restrict__ kg = (const char*)p.k + s.bk * KB;
-  const bf16_t* __restrict__ vg = (const bf16_t*)p.v + s.bv;
-  bf16_t* __restrict__ og = (bf16_t*)p.out + s.bo;
-
-  if (q0 >= s.n_q) {
-    // padded rows of the padded layout: exact zeros
-    const int rows = (s.rows - q0) < BM ? (s.rows - q0) : BM;
-    const uint4 z = {0u, 0u, 0u, 0u};
-    for (int e = tid; e < rows * (D / 8); e += MFMA_THREADS) {
-      int r = e / (D / 8), c = e - r * (D / 8);
-      *(uint4*)(og + (int64_t)(q0 + r) * p.o_st + c * 8) = z;
-    }
-    return;
-  }
-
-  const int r0 = q0 + 32 * w;          // first query row of this wave
-  const int qrow = r0 + m;             // this lane's query row
-  const bool wave_live = r0 < s.n_q;
-
-  // this workgroup's steps [t_lo, nt) of the tile's: the whole tile, or balanced part `chunk` of n_chunks
-  // (a part can be empty only if the list were inconsistent; such a workgroup still arrives below)
-  int nt = tile_steps(p, s, q0);
-  const int n_chunks = wk.n_chunks;
-  int t_lo = 0;
-  if (n_chunks > 1) {
-    const int per = (nt + n_chunks - 1) / n_chunks;
-    t_lo = chunk * per;
-    t_lo = t_lo < nt ? t_lo : nt;
-    nt = t_lo + per < nt ? t_lo + per : nt;
-  }
-  // a sliding window (never combined with key-range splitting) also drops the steps before the tile's first key
+  constexpr bool PAIRS = NSTAGE == 4 && DENSE == 0;
+  static_assert(!PERSIST || (PAIRS && !SEG && !F8), "the loop over items is built on the paired step loop");
   const int win = p.window;
-  if (win >= 0 && q0 - win > 0) t_lo = (q0 - win) / BN;
-  // last key this wave needs (under a window without the causal mask: the last key its last row sees)
-  int wave_last = p.causal ? r0 + 31 : (win >= 0 ? r0 + 31 + win : s.n_kv - 1);
-  wave_last = wave_last < s.n_kv - 1 ? wave_last : s.n_kv - 1;
-  if (!wave_live) wave_last = -1;
-
-  // fp8 q and k carry per-head dequantisation scales: they multiply the logits
-  const float alpha2 = p.alpha * LOG2E * (F8 && p.q_scale ? p.q_scale[h] : 1.0f) * (F8 && p.k_scale ? p.k_scale[h] : 1.0f);
   const uint32_t kst_bytes = (uint32_t)p.k_st * (uint32_t)KB, vst_bytes = (uint32_t)p.v_st * 2u;
-  // Bias operands are fetched with 32-bit byte offsets from the start of the workspace.
-  // pos_off: this head's padded table; entry x of the unpadded table sits at float POS_PAD + x.
   const char* wsb = (const char*)p.ws_base;
-  const uint32_t pos_off = POS ? (uint32_t)((const char*)(p.pos_scaled + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1 + 2 * POS_PAD)) - wsb) : 0u;
-  const int64_t* tsg = TS ? p.ts + s.ts0 : nullptr;
-  // int32 timestamps of this sequence, valid when its time span allows them (ts_ok, same for the
-  // whole workgroup; read now, needed only when the first block is computed)
-  const int32_t* trel = TS ? p.ts_rel + ts_rel_base(p, b, s.tok0) : nullptr;
-  const int ts32 = TS ? p.ts_ok[b] : 0;
-  const uint32_t rel_off = TS ? (uint32_t)((const char*)trel - wsb) : 0u;
-  const uint32_t rng_off = TS ? (uint32_t)((const char*)(p.ts_range + 2 * ts_range_slot0(p, b, s.tok0)) - wsb) : 0u;
+  uint32_t* xch = (uint32_t*)(smem + XCH_OFF);
+
+  // What the direct loads of an item's steps need (everything here is the same for the whole workgroup).
+  // What an item's set-up needs of the arguments.  A workgroup that stays reads them again from the kernel
+  // argument segment at each item (scalar loads through a pointer the compiler cannot see through):
+  // kept in scalar registers across the step loop they would not fit beside what the loop itself holds.
+  auto fresh = [&]() -> Params {
+    if constexpr (PERSIST) {
+      typedef const __attribute__((address_space(4))) Params* KernArg;
+      KernArg ka = (KernArg)__builtin_amdgcn_kernarg_segment_ptr();
+      asm volatile("" : "+s"(ka));
+      return *(const Params*)ka;
+    } else {
+      return p;
+    }
+  };
+  struct DmaCtx { const char* kg; const bf16_t* vg; int n_kv, n_ts, q0, b; uint32_t pos_off, rel_off, rng_off; };
+  // Bias operands are fetched with 32-bit byte offsets from the start of the workspace.
+  // pos_off: the head's padded table; entry x of the unpadded table sits at float POS_PAD + x.
+  auto ctx_of = [&](const Work& k) {
+    const Params pf = fresh();
+    DmaCtx c;
+    c.kg = (const char*)pf.k + k.s.bk * KB;
+    c.vg = (const bf16_t*)pf.v + k.s.bv;
+    c.n_kv = k.s.n_kv; c.n_ts = k.s.n_ts; c.q0 = k.qt * BM; c.b = k.b;
+    c.pos_off = POS ? (uint32_t)((const char*)(pf.pos_scaled + (int64_t)(pf.pos_heads > 1 ? k.h : 0) * (2 * pf.L - 1 + 2 * POS_PAD)) - wsb) : 0u;
+    c.rel_off = TS ? (uint32_t)((const char*)(pf.ts_rel + ts_rel_base(pf, k.b, k.s.tok0)) - wsb) : 0u;
+    c.rng_off = TS ? (uint32_t)((const char*)(pf.ts_range + 2 * ts_range_slot0(pf, k.b, k.s.tok0)) - wsb) : 0u;
+    if constexpr (PERSIST) {
+      // (the same for every lane, and the direct loads want them in scalar registers: said outright, the
+      // compiler otherwise moves the arithmetic of an item drawn at run time to the vector unit)
+      c.kg = (const char*)scalar_ptr(c.kg);
+      c.vg = (const bf16_t*)scalar_ptr(c.vg);
+    }
+    return c;
+  };
+  // The steps [t_lo, nt) an item covers: the whole tile, or balanced part `chunk` of n_chunks (a part can be
+  // empty only if the list were inconsistent; such a workgroup still arrives at the tile's counter);
+  // nothing for a tile of padding rows.  A sliding window (never combined with key-range splitting) also
+  // drops the steps before the tile's first key.
+  auto range_of = [&](const Work& k, int& t_lo_, int& nt_) {
+    const Params pf = fresh();
+    const int q0_ = k.qt * BM;
+    t_lo_ = 0;
+    nt_ = q0_ < k.s.n_q ? tile_steps(pf, k.s, q0_) : 0;
+    if (k.n_chunks > 1) {
+      const int per = (nt_ + k.n_chunks - 1) / k.n_chunks;
+      t_lo_ = k.chunk * per;
+      t_lo_ = t_lo_ < nt_ ? t_lo_ : nt_;
+      nt_ = t_lo_ + per < nt_ ? t_lo_ + per : nt_;
+    }
+    if (win >= 0 && q0_ - win > 0 && nt_ > 0) t_lo_ = (q0_ - win) / BN;
+  };
 
   // Direct loads of step t into ring stage t % NSTAGE.  Wave w fills 1 KB
   // pieces w*LD .. w*LD+LD-1 of K and of V; lane l of piece j lands at chunk
@@ -1234,11 +1240,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // issues the same number of loads per step: the vmcnt arithmetic relies on it.
   // The ring stage is a compile-time constant everywhere (the step loop is unrolled over the ring):
   // LDS addresses are then a per-lane register plus an immediate, with no address arithmetic per step.
-  // Stage of step t: (t - t_lo) % NSTAGE.
-  auto dma_step = [&](int t, auto st_) {
+  auto dma_step = [&](const DmaCtx& c_, int t, auto st_) {
     constexpr int st = decltype(st_)::value;
     const int kv0 = t * BN;
-    const int last = s.n_kv - 1;
+    const int last = c_.n_kv - 1;
 #pragma unroll
     for (int r = 0; r < LDK; ++r) {
       const int j = (w * LDK + r) % NPIECE_K;   // small tiles: several waves repeat the same piece
@@ -1247,7 +1252,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       int grow = kv0 + row;
       grow = grow < last ? grow : last;
       const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
-      lds_dma16(kg, koff, (const unsigned char*)Ks(st) + j * 1024);
+      lds_dma16(c_.kg, koff, (const unsigned char*)Ks(st) + j * 1024);
     }
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
@@ -1257,7 +1262,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       int grow = kv0 + row;
       grow = grow < last ? grow : last;
       const uint32_t voff = (uint32_t)grow * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
-      lds_dma16(vg, voff, Vs(st) + j * 512);
+      lds_dma16(c_.vg, voff, Vs(st) + j * 512);
     }
     if (POS || TS) {
       // One more load per wave brings the bias operands.  Wave c writes position-window copy c:
@@ -1273,14 +1278,14 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       uint32_t off = 0;
       bool on = false;
       if (POS && lane < SM::POS_LANES) {
-        off = pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (q0 + BM - 1) + w + 4 * lane) * 4u;
+        off = c_.pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (c_.q0 + BM - 1) + w + 4 * lane) * 4u;
         on = true;
       }
       if (ts_wave && tl >= 0 && tl < SM::TK_LANES) {
         int tr = t;                                  // tiles past the last timestamp repeat the last tile's range
-        const int tr_last = (s.n_ts - 1) >> 5;
+        const int tr_last = (c_.n_ts - 1) >> 5;
         tr = tr < tr_last ? tr : tr_last;
-        off = tl < BN / 4 ? rel_off + (uint32_t)(kv0 + 4 * tl) * 4u : rng_off + (uint32_t)tr * 8u;
+        off = tl < BN / 4 ? c_.rel_off + (uint32_t)(kv0 + 4 * tl) * 4u : c_.rng_off + (uint32_t)tr * 8u;
         on = true;
       }
       if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
@@ -1291,7 +1296,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       if (lane < BN / 4) {
         int g4 = kv0 + 4 * lane;
         g4 = g4 < p.Lkv - 4 ? g4 : p.Lkv - 4;
-        lds_dma16_at(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
+        lds_dma16_at(p.kv_seg + (int64_t)c_.b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
       }
     }
     if (DENSE & 1) {
@@ -1300,12 +1305,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       // 4w .. 4w+3 (8 rows each); lane l of a piece lands at row l / 8, physical chunk l % 8.  Rows
       // past L and keys past Lkv re-read the last row / the last four keys: finite data for
       // logits that are masked by their index.
-      const float* dbg = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      const float* dbg = p.dense_bias + (p.dense_bias_batched ? (int64_t)c_.b * p.L * p.Lkv : 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int j = 4 * w + r;
         const int row = 8 * j + (lane >> 3), pc = lane & 7;
-        int gr = q0 + row;
+        int gr = c_.q0 + row;
         gr = gr < p.L - 1 ? gr : p.L - 1;
         int col = kv0 + 4 * (pc ^ (row & 7));
         col = col < p.Lkv - 4 ? col : p.Lkv - 4;
@@ -1314,9 +1319,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     }
     if (DENSE & 2) {
       // Mask tile: row r at LDS byte 32 r; wave w brings its own 32 rows, two lanes per row.
-      const uint8_t* mg = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      const uint8_t* mg = p.mask + (p.mask_batched ? (int64_t)c_.b * p.L * p.Lkv : 0);
       const int row = 32 * w + (lane >> 1);
-      int gr = q0 + row;
+      int gr = c_.q0 + row;
       gr = gr < p.L - 1 ? gr : p.L - 1;
       int col = kv0 + 16 * (lane & 1);
       col = col < p.Lkv - 16 ? col : p.Lkv - 16;
@@ -1324,68 +1329,84 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     }
   };
 
-  // prologue: the keyed bucket table, then
-  // the first steps in flight before the first block (two when the loop runs in pairs, else NSTAGE - 1)
-  if (TS) {
-    // three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
+
+  // ---- the item at hand: the same for the whole workgroup except where a lane's row enters
+  DmaCtx cx;
+  struct { int n_q, n_kv, rows, n_ts; } s;       // of the item's sequence
+  int h = 0, q0 = 0, r0 = 0, qrow = 0, wave_last = -1, nt = 0, t_lo = 0, n_chunks = 1, chunk = 0, pslot = 0, ts32 = 0;
+  float alpha2 = 0.f;
+  const int64_t* tsg = nullptr;
+  bf16_t* og = nullptr;
+  auto begin_item = [&](const Work& k) {
+    const Params pf = fresh();
+    s.n_q = k.s.n_q; s.n_kv = k.s.n_kv; s.rows = k.s.rows; s.n_ts = k.s.n_ts;
+    h = k.h; q0 = k.qt * BM; chunk = k.chunk; n_chunks = k.n_chunks; pslot = k.pslot;
+    cx = ctx_of(k);
+    range_of(k, t_lo, nt);
+    r0 = q0 + 32 * w;                    // first query row of this wave
+    qrow = r0 + m;                       // this lane's query row
+    // last key this wave needs (under a window without the causal mask: the last key its last row sees)
+    wave_last = pf.causal ? r0 + 31 : (win >= 0 ? r0 + 31 + win : s.n_kv - 1);
+    wave_last = wave_last < s.n_kv - 1 ? wave_last : s.n_kv - 1;
+    if (r0 >= s.n_q) wave_last = -1;
+    // fp8 q and k carry per-head dequantisation scales: they multiply the logits
+    alpha2 = pf.alpha * LOG2E * (F8 && pf.q_scale ? pf.q_scale[h] : 1.0f) * (F8 && pf.k_scale ? pf.k_scale[h] : 1.0f);
+    tsg = TS ? pf.ts + k.s.ts0 : nullptr;
+    // whether the sequence's int32 timestamps are valid (its time span allows them)
+    ts32 = TS ? pf.ts_ok[k.b] : 0;
+    og = (bf16_t*)pf.out + k.s.bo;
+  };
+  // the head's bucket table: three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
+  auto load_ts_table = [&](int head) {
+    const Params pf = fresh();
     const int c = w < 3 ? w : 0;
     if (1024 * c + 16 * lane < TS_LDS_BYTES)
-      lds_dma16((const unsigned char*)p.ts_keyed + (int64_t)(p.ts_heads > 1 ? h : 0) * (3 * 1024) + 1024 * c, (uint32_t)lane * 16u, TsKey + 1024 * c);
-  }
-  // The first step's tiles go out alone; the other two of the prologue follow behind the Q
-  // fragments, whose wait below covers every load issued before it: behind all three steps it
-  // held up the first block until the whole prologue had landed.
-  if (t_lo < nt) dma_step(t_lo, std::integral_constant<int, 0>{});
+      lds_dma16((const unsigned char*)pf.ts_keyed + (int64_t)(pf.ts_heads > 1 ? head : 0) * (3 * 1024) + 1024 * c, (uint32_t)lane * 16u, TsKey + 1024 * c);
+  };
 
   // Q fragments (B operand of S^T = K Q^T).  bf16: k-step ks of lane (row, hh) holds
   // q[qrow][16ks+8hh .. +7], i.e. 16-byte chunk 2ks+hh of the row.  fp8: the lane holds chunks
   // 2j+hh of the row, each feeding two k-steps (its low and its high 8 bytes); K is read the
-  // same way, and the order of the terms of a dot product is free.
+  // same way, and the order of the terms of a dot product is free.  With them the lane's segment id
+  // and the timestamp its row takes (that of the next row).
   uint4 qf[QCH];
-  {
-    const char* qg = (const char*)p.q + (s.bq + (int64_t)qrow * p.q_st) * KB + 16 * hh;
+  int32_t qseg = 0;
+  int64_t tq = 0;
+  int32_t tq32 = 0;
+  auto load_q = [&](const Work& k) {
+    const Params pf = fresh();
+    // (the lane's index enters through a register the compiler cannot see through: it would otherwise
+    // work the lane's share of every address out once, ahead of the loop over items, and keep it all in
+    // registers that loop does not have; the same in finish_item)
+    int m_ = m, hh_ = hh;
+    if (PERSIST) asm volatile("" : "+v"(m_), "+v"(hh_));
+    const int qr = k.qt * BM + 32 * w + m_;
+    const char* qg = (const char*)pf.q + (k.s.bq + (int64_t)qr * pf.q_st) * KB + 16 * hh_;
 #pragma unroll
     for (int ks = 0; ks < QCH; ++ks) {
       uint4 t4 = {0u, 0u, 0u, 0u};
-      if (qrow < s.n_q) t4 = *(const uint4*)(qg + 32 * ks);
+      if (qr < k.s.n_q) t4 = *(const uint4*)(qg + 32 * ks);
       qf[ks] = t4;
     }
-    // Use the fragments here so that the compiler's wait for these loads sits in the prologue.
-    // Left to the first use inside the loop it would be a vmcnt(0) on every step, which also
-    // waits for every direct load in flight and serialises the whole ring.
+    if (SEG) qseg = pf.q_seg[(int64_t)k.b * pf.L + (qr < pf.L ? qr : pf.L - 1)];
+    if (TS) {
+      int iq = qr + 1 < k.s.n_ts ? qr + 1 : k.s.n_ts - 1;
+      iq = iq < 0 ? 0 : iq;
+      tq32 = (pf.ts_rel + ts_rel_base(pf, k.b, k.s.tok0))[iq];     // meaningless when the sequence has no int32 timestamps, and then unused
+      tq = (pf.ts + k.s.ts0)[iq];
+    }
+  };
+  // Use what load_q fetched so that the compiler's wait for those loads sits here.  Left to the first
+  // use inside the loop it would be a vmcnt(0) on every step, which also waits for every direct
+  // load in flight and serialises the whole ring.
+  auto settle_q = [&]() {
 #pragma unroll
     for (int ks = 0; ks < QCH; ++ks) asm volatile("" ::"v"(qf[ks].x), "v"(qf[ks].y), "v"(qf[ks].z), "v"(qf[ks].w));
-  }
-  int32_t qseg = 0;
-  if (SEG) {
-    qseg = p.q_seg[(int64_t)b * p.L + (qrow < p.L ? qrow : p.L - 1)];
-    asm volatile("" ::"v"(qseg));
-  }
-  int64_t tq = 0;
-  int32_t tq32 = 0;
-  if (TS) {
-    int iq = qrow + 1 < s.n_ts ? qrow + 1 : s.n_ts - 1;
-    iq = iq < 0 ? 0 : iq;
-    tq32 = trel[iq];     // meaningless when !ts32, and then unused
-    tq = tsg[iq];
-    asm volatile("" ::"v"(tq), "v"(tq32));
-  }
-
-  // With a four-stage ring and no dense operands the step loop below runs in pairs of steps: only
-  // the first pair is in flight before it (d = 128: 68.8 -> 64.9 us on the headline shape, 2-3 % on
-  // full-length batches).  Dense operands bring five to ten more loads per step and lose by pairs
-  // (490 -> 556 us), and so does a fourth stage bought for them at d <= 64 (110 -> 116 us).
-  constexpr bool PAIRS = NSTAGE == 4 && DENSE == 0;
-  if (t_lo + 1 < nt) dma_step(t_lo + 1, std::integral_constant<int, 1>{});
-  if constexpr (NSTAGE > 3 && !PAIRS) {
-    if (t_lo + 2 < nt) dma_step(t_lo + 2, std::integral_constant<int, 2>{});
-  }
+    if (SEG) asm volatile("" ::"v"(qseg));
+    if (TS) asm volatile("" ::"v"(tq), "v"(tq32));
+  };
 
   floatx16 o[DVB];
-#pragma unroll
-  for (int i = 0; i < DVB; ++i)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
 
   // K: lane (row m, half hh) reads logical chunk 2ks+hh of row m
   const int gk = SM::swz_k(m);
@@ -1558,17 +1579,33 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 #pragma unroll
       for (int r = 0; r < 16; ++r) u[r] = ((mbits[r >> 2] >> (8 * (r & 3))) & 0xffu) ? u[r] : 0.f;
     }
-    float pv[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) pv[r] = silu_log2(u[r]);
+    // SiLU and P V in two halves of 8 keys, each in four phases of 8 independent operations with the order
+    // fixed by scheduling barriers: left to itself under register pressure, the compiler has run the 16
+    // exp -> add -> rcp -> mul chains one after another through one register, each link waiting for the last
+    // (the transcendental unit's latency 32 times per step).  The first half's matrix products run while the
+    // second half's vector work is issued.
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
+      float e[8];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) e[r] = __builtin_amdgcn_exp2f(-u[8 * cc + r]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) e[r] = 1.0f + e[r];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) e[r] = __builtin_amdgcn_rcpf(e[r]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) e[r] = u[8 * cc + r] * e[r];
       uint4 pk;
-      pk.x = pack_bf16(pv[8 * cc + 0], pv[8 * cc + 1]);
-      pk.y = pack_bf16(pv[8 * cc + 2], pv[8 * cc + 3]);
-      pk.z = pack_bf16(pv[8 * cc + 4], pv[8 * cc + 5]);
-      pk.w = pack_bf16(pv[8 * cc + 6], pv[8 * cc + 7]);
+      pk.x = pack_bf16(e[0], e[1]);
+      pk.y = pack_bf16(e[2], e[3]);
+      pk.z = pack_bf16(e[4], e[5]);
+      pk.w = pack_bf16(e[6], e[7]);
       const bf16x8 pb = __builtin_bit_cast(bf16x8, pk);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int dvb = 0; dvb < DVB; ++dvb)
         o[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[cc][dvb]), pb, o[dvb], 0, 0, 0);
@@ -1583,149 +1620,326 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     else if (younger == 1) HSTU_WAIT_VMCNT(NDMA);
     else HSTU_WAIT_VMCNT(0);
   };
-
   const auto live = [&](int t) { return t * BN <= wave_last && (win < 0 || t * BN + 31 + win >= r0); };
-  if constexpr (PAIRS) {
-    // Steps in pairs, one barrier per pair.  The barrier that ended the pair (t-2, t-1) freed that
-    // pair's two ring stages, which now receive steps t+2 and t+3; the blocks of steps t and t+1
-    // are computed; then every wave makes sure that its share of the next pair has landed.  Between
-    // two barriers the waves of a workgroup drift apart by up to two blocks, which the diagonal
-    // tiles (where wave i has i+1 blocks to do) and the direct loads' issue stalls both use.
-    HSTU_WAIT_VMCNT(0);
-    __syncthreads();
-    auto pair = [&](int t, auto st_) {
-      constexpr int st = decltype(st_)::value;
-      if (t + 2 < nt) dma_step(t + 2, std::integral_constant<int, (st + 2) % NSTAGE>{});
-      if (t + 3 < nt) dma_step(t + 3, std::integral_constant<int, (st + 3) % NSTAGE>{});
-      if (live(t)) block(t, st_);
-      if (t + 1 < nt && live(t + 1)) block(t + 1, std::integral_constant<int, (st + 1) % NSTAGE>{});
+
+  auto zero_o = [&]() {
+#pragma unroll
+    for (int i = 0; i < DVB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[i][r] = 0.f;
+  };
+
+  // The end of an item: its rows (or its partial sums) leave the workgroup.  `ot_base`: LDS bytes free
+  // for the waves' 32 x D staging tiles.
+  auto finish_item = [&](int ot_base) {
+    const Params pf = fresh();
+    int tid_ = tid;
+    if (PERSIST) asm volatile("" : "+v"(tid_));
+    const int tid = tid_, lane = tid_ & 63, m = lane & 31, hh = lane >> 5;     // shadow the kernel's: see load_q
+    const int qrow = r0 + m;
+    if (q0 >= s.n_q) {
+      // padded rows of the padded layout: exact zeros
+      const int rows = (s.rows - q0) < BM ? (s.rows - q0) : BM;
+      const uint4 z = {0u, 0u, 0u, 0u};
+      for (int e = tid; e < rows * (D / 8); e += MFMA_THREADS) {
+        int r = e / (D / 8), c = e - r * (D / 8);
+        *(uint4*)(og + (int64_t)(q0 + r) * pf.o_st + c * 8) = z;
+      }
+      return;
+    }
+    // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0.
+    // The 1/log2(e) left out of the SiLU is folded into the output scale.
+    if (n_chunks > 1) {
+      // This workgroup covered part of the tile's keys.  It leaves its fp32 partial O^T (register order:
+      // 8-byte piece (16 w + i) * 128 + 2 lane + j of the chunk's slot) in the workspace and counts itself
+      // in at the tile's arrival counter; the workgroup that arrives last adds the others' partials to
+      // its own, always in the order of the chunks, and writes the rows.  Partials and counter go by
+      // device-scope atomic stores, loads and adds (which bypass the caches that are not coherent across
+      // the chip), ordered by waiting for the stores' completion before the count: no cache is flushed,
+      // and nothing depends on which workgroup runs where.  The result does not depend on the order of
+      // arrival.
+      constexpr int NPC = BM * D / 2;      // 8-byte pieces of a chunk's partial
+      uint64_t* slot0 = (uint64_t*)pf.partial + ((int64_t)pslot * pf.H + h) * NPC;
+      uint64_t* mine = slot0 + (int64_t)chunk * pf.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane;
+#pragma unroll
+      for (int i = 0; i < DVB * 4; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          // (through named floats: a bit cast applied to a vector element directly reads element 0)
+          const float f0 = o[i >> 2][4 * (i & 3) + 2 * j], f1 = o[i >> 2][4 * (i & 3) + 2 * j + 1];
+          const uint64_t bits = (uint64_t)__builtin_bit_cast(uint32_t, f0) | ((uint64_t)__builtin_bit_cast(uint32_t, f1) << 32);
+          __hip_atomic_store(mine + i * 128 + j, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      HSTU_WAIT_VMCNT(0);                  // every store of this wave has been acknowledged
+      __syncthreads();
+      uint32_t* arrive = pf.ctr + CTR_RESERVED + pslot * pf.H + h;
+      if (tid == 0) xch[0] = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      const uint32_t before = xch[0];
+      if (before != (uint32_t)(n_chunks - 1)) return;
+      if (tid == 0) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next call
+      // (a chunk's pieces are asked for 16 at a time per lane and added once they are there: two round trips
+      // per chunk instead of one per piece)
+      auto add_chunk = [&](int c, floatx16 (&dst)[DVB]) {
+        const uint64_t* src = slot0 + (int64_t)c * pf.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane;
+#pragma unroll
+        for (int i0 = 0; i0 < DVB * 4; i0 += 8) {       // 16 pieces at a time
+          uint64_t bits[16];
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+              bits[2 * i + j] = __hip_atomic_load(src + (i0 + i) * 128 + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              const int ii = i0 + i;
+              dst[ii >> 2][4 * (ii & 3) + 2 * j] += __builtin_bit_cast(float, (uint32_t)bits[2 * i + j]);
+              dst[ii >> 2][4 * (ii & 3) + 2 * j + 1] += __builtin_bit_cast(float, (uint32_t)(bits[2 * i + j] >> 32));
+            }
+        }
+      };
+      // (its own partial comes back from the workspace like the others: one code path, no second accumulator)
+      zero_o();
+      for (int c = 0; c < n_chunks; ++c) add_chunk(c, o);
+    }
+    // Each wave turns its O^T fragment into whole output rows through LDS (those stages of the ring are
+    // free: the loop ended on a barrier and no load into them is in flight), so that global memory sees
+    // 16-byte stores that cover full rows instead of 8-byte pieces: lane (row m, half hh) writes 8 bytes
+    // of row m at a time, 16-byte chunks XOR-swizzled by row against bank conflicts, then reads 16 bytes
+    // per lane, 64 / (D/8) rows per instruction.  Only lanes of the same wave exchange data here and
+    // LDS executes a wave's operations in order: no barrier is needed.
+    const float oscale = pf.inv_n * (1.0f / LOG2E);
+    unsigned char* ot = smem + ot_base + w * (32 * D * 2);
+    auto oswz = [](int row) { return (row / SM::RPB) % CPR; };
+    {
+      const bool live_row = qrow < s.n_q;
+      unsigned char* orow = ot + m * (D * 2) + 8 * hh;
+#pragma unroll
+      for (int dvb = 0; dvb < DVB; ++dvb) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          uint2 pko = {0u, 0u};
+          if (live_row) {
+            pko.x = pack_bf16(o[dvb][4 * g + 0] * oscale, o[dvb][4 * g + 1] * oscale);
+            pko.y = pack_bf16(o[dvb][4 * g + 2] * oscale, o[dvb][4 * g + 3] * oscale);
+          }
+          *(uint2*)(orow + (((4 * dvb + g) ^ oswz(m)) * 16)) = pko;
+        }
+      }
+    }
+    constexpr int ROWS_PER_STORE = 64 / CPR;
+    const int rr = lane / CPR, cc = lane - rr * CPR;
+#pragma unroll
+    for (int r0s = 0; r0s < 32; r0s += ROWS_PER_STORE) {
+      const int row = r0s + rr;
+      const uint4 val = *(const uint4*)(ot + row * (D * 2) + ((cc ^ oswz(row)) * 16));
+      const int grow = r0 + row;
+      if (grow < s.rows) {
+        // streaming store: the output is not read again by this kernel, and K / V rows that other tiles of the
+        // sequence still need are worth more of the L2 than it is (d = 64 benchmark shape: 134 -> 122 us)
+        typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+        const uintx4 vv = {val.x, val.y, val.z, val.w};
+        __builtin_nontemporal_store(vv, (uintx4*)(og + (int64_t)grow * pf.o_st + cc * 8));
+      }
+    }
+  };
+  if constexpr (!PERSIST) {
+    // ---- one item per workgroup
+    Work first;
+    if (!work_of_block(p, blockIdx.x, first)) return;
+    if (first.qt * BM >= first.s.rows) return;
+    begin_item(first);
+    if (q0 >= s.n_q) {
+      if (chunk == 0) finish_item(0);
+      return;
+    }
+    // prologue: the bucket table, then the first steps in flight before the first block (two when the
+    // loop runs in pairs, else NSTAGE - 1).  The first step's tiles go out alone; the rest of the
+    // prologue follows behind the Q fragments, whose wait covers every load issued before it: behind
+    // all of the prologue it held up the first block until everything had landed.
+    if (TS) load_ts_table(h);
+    if (t_lo < nt) dma_step(cx, t_lo, std::integral_constant<int, 0>{});
+    load_q(first);
+    settle_q();
+    if (t_lo + 1 < nt) dma_step(cx, t_lo + 1, std::integral_constant<int, 1>{});
+    if constexpr (NSTAGE > 3 && !PAIRS) {
+      if (t_lo + 2 < nt) dma_step(cx, t_lo + 2, std::integral_constant<int, 2>{});
+    }
+    zero_o();
+    if constexpr (PAIRS) {
+      // Steps in pairs, one barrier per pair.  The barrier that ended the pair (t-2, t-1) freed that
+      // pair's two ring stages, which now receive steps t+2 and t+3; the blocks of steps t and t+1
+      // are computed; then every wave makes sure that its share of the next pair has landed.  Between
+      // two barriers the waves of a workgroup drift apart by up to two blocks, which the diagonal
+      // tiles (where wave i has i+1 blocks to do) and the direct loads' issue stalls both use.
+      // (With a four-stage ring and no dense operands only: d = 128 68.8 -> 64.9 us on the headline
+      // shape; dense operands bring five to ten more loads per step and lose by pairs, 490 -> 556 us,
+      // and so does a fourth stage bought for them at d <= 64, 110 -> 116 us.)
       HSTU_WAIT_VMCNT(0);
       __syncthreads();
-    };
-    for (int t = t_lo; t < nt; t += NSTAGE) {
-      pair(t, std::integral_constant<int, 0>{});
-      if (t + 2 >= nt) break;
-      pair(t + 2, std::integral_constant<int, 2>{});
-    }
-  } else {
-    wait_step(t_lo);
-    __syncthreads();
-
-    // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
-    // which now receives step t+NSTAGE-1; the block of step t is computed; then every
-    // wave makes sure its share of step t+1 has landed before the next barrier.
-    auto step = [&](int t, auto st_) {
-      constexpr int st = decltype(st_)::value;
-      if (t + NSTAGE - 1 < nt) dma_step(t + NSTAGE - 1, std::integral_constant<int, (st + NSTAGE - 1) % NSTAGE>{});
-      if (live(t)) block(t, st_);
-      if (t + 1 < nt) wait_step(t + 1);
+      auto pair = [&](int t, auto st_) {
+        constexpr int st = decltype(st_)::value;
+        if (t + 2 < nt) dma_step(cx, t + 2, std::integral_constant<int, (st + 2) % NSTAGE>{});
+        if (t + 3 < nt) dma_step(cx, t + 3, std::integral_constant<int, (st + 3) % NSTAGE>{});
+        if (live(t)) block(t, st_);
+        if (t + 1 < nt && live(t + 1)) block(t + 1, std::integral_constant<int, (st + 1) % NSTAGE>{});
+        HSTU_WAIT_VMCNT(0);
+        __syncthreads();
+      };
+      for (int t = t_lo; t < nt; t += NSTAGE) {
+        pair(t, std::integral_constant<int, 0>{});
+        if (t + 2 >= nt) break;
+        pair(t + 2, std::integral_constant<int, 2>{});
+      }
+    } else {
+      wait_step(t_lo);
       __syncthreads();
+      // Step t: the barrier that ended step t-1 freed the ring stage of step t-1,
+      // which now receives step t+NSTAGE-1; the block of step t is computed; then every
+      // wave makes sure its share of step t+1 has landed before the next barrier.
+      auto step = [&](int t, auto st_) {
+        constexpr int st = decltype(st_)::value;
+        if (t + NSTAGE - 1 < nt) dma_step(cx, t + NSTAGE - 1, std::integral_constant<int, (st + NSTAGE - 1) % NSTAGE>{});
+        if (live(t)) block(t, st_);
+        if (t + 1 < nt) wait_step(t + 1);
+        __syncthreads();
+      };
+      for (int t = t_lo; t < nt; t += NSTAGE) {
+        step(t, std::integral_constant<int, 0>{});
+        if (t + 1 >= nt) break;
+        step(t + 1, std::integral_constant<int, 1>{});
+        if (t + 2 >= nt) break;
+        step(t + 2, std::integral_constant<int, 2>{});
+        if constexpr (NSTAGE > 3) {
+          if (t + 3 >= nt) break;
+          step(t + 3, std::integral_constant<int, 3>{});
+        }
+      }
+    }
+    finish_item(0);
+  } else {
+    // ---- a workgroup that stays: it takes item after item of its XCD's part of the work list.  Job j of
+    // an XCD is (item, head) as in work_of_block; a workgroup's first job is j = slot, every later one is
+    // drawn from the XCD's counter (the list is in order of falling work, so whoever is free takes the
+    // longest job left).  The draw is made late, when at most two pairs of steps of the item at hand are
+    // left: a job drawn early would wait for a workgroup that may still be busy for long while others
+    // run dry.  While an item's last pair of steps is computed, the next item's first pair of tiles is
+    // already on its way into the two ring stages that pair does not use, and its Q rows follow as soon
+    // as the last logits are done: the latencies of an item's start hide behind the item before it.
+    const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
+    const int n_items = p.sched[0];
+    const int4* items = (const int4*)(p.sched + 4);
+    auto job_item = [&](int job, int& head) {
+      const int H = fresh().H;
+      int it;
+      if (H >= 8) { const int hx = H >> 3; it = job / hx; head = (job - it * hx) * 8 + xcd; }
+      else        { const int r = 8 / H;   it = job * r + xcd / H; head = xcd % H; }
+      return it;
     };
-    for (int t = t_lo; t < nt; t += NSTAGE) {
-      step(t, std::integral_constant<int, 0>{});
-      if (t + 1 >= nt) break;
-      step(t + 1, std::integral_constant<int, 1>{});
-      if (t + 2 >= nt) break;
-      step(t + 2, std::integral_constant<int, 2>{});
-      if constexpr (NSTAGE > 3) {
-        if (t + 3 >= nt) break;
-        step(t + 3, std::integral_constant<int, 3>{});
-      }
+    int head_now = 0;
+    int it_now = job_item(blockIdx.x >> 3, head_now);
+    bool have = it_now < n_items;
+    if (have) {
+      Work first;
+      work_from_item(p, items[it_now], head_now, first);
+      begin_item(first);
+      if (TS) load_ts_table(h);
+      if (t_lo < nt) dma_step(cx, t_lo, std::integral_constant<int, 0>{});
+      load_q(first);
+      settle_q();
+      if (t_lo + 1 < nt) dma_step(cx, t_lo + 1, std::integral_constant<int, 1>{});
     }
-  }
-
-  // O^T[dv = 32 dvb + 8g + 4hh + t][q = qrow]; rows past the sequence are 0.
-  // The 1/log2(e) left out of the SiLU is folded into the output scale.
-  if (n_chunks > 1) {
-    // This workgroup covered part of the tile's keys.  It leaves its fp32 partial O^T (register order:
-    // 8-byte piece (16 w + i) * 128 + 2 lane + j of the chunk's slot) in the workspace and counts itself
-    // in at the tile's arrival counter; the workgroup that arrives last adds the others' partials to
-    // its own, always in the order of the chunks, and writes the rows.  Partials and counter go by
-    // device-scope atomic stores, loads and adds (which bypass the caches that are not coherent across
-    // the chip), ordered by waiting for the stores' completion before the count: no cache is flushed,
-    // and nothing depends on which workgroup runs where.  The result does not depend on the order of
-    // arrival.
-    constexpr int NPC = BM * D / 2;      // 8-byte pieces of a chunk's partial
-    uint64_t* slot0 = (uint64_t*)p.partial + ((int64_t)wk.pslot * p.H + h) * NPC;
-    uint64_t* mine = slot0 + (int64_t)chunk * p.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane;
-#pragma unroll
-    for (int i = 0; i < DVB * 4; ++i) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        // (through named floats: a bit cast applied to a vector element directly reads element 0)
-        const float f0 = o[i >> 2][4 * (i & 3) + 2 * j], f1 = o[i >> 2][4 * (i & 3) + 2 * j + 1];
-        const uint64_t bits = (uint64_t)__builtin_bit_cast(uint32_t, f0) | ((uint64_t)__builtin_bit_cast(uint32_t, f1) << 32);
-        __hip_atomic_store(mine + i * 128 + j, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    HSTU_WAIT_VMCNT(0);                  // every store of this wave has been acknowledged
-    __syncthreads();
-    uint32_t* xch = (uint32_t*)(smem + XCH_OFF);
-    uint32_t* arrive = p.ctr + CTR_RESERVED + wk.pslot * p.H + h;
-    if (tid == 0) *xch = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    const uint32_t before = *xch;
-    if (before != (uint32_t)(n_chunks - 1)) return;
-    if (tid == 0) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next call
-#pragma unroll
-    for (int i = 0; i < DVB * 4; ++i) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        float a0 = 0.f, a1 = 0.f;
-        for (int c = 0; c < n_chunks; ++c) {
-          float x0 = o[i >> 2][4 * (i & 3) + 2 * j], x1 = o[i >> 2][4 * (i & 3) + 2 * j + 1];
-          if (c != chunk) {
-            const uint64_t bits = __hip_atomic_load(slot0 + (int64_t)c * p.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane + i * 128 + j,
-                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            x0 = __builtin_bit_cast(float, (uint32_t)bits);
-            x1 = __builtin_bit_cast(float, (uint32_t)(bits >> 32));
+    while (have) {
+      zero_o();
+      HSTU_WAIT_VMCNT(0);                  // the item's first pair of tiles, its Q rows, the stores of the item before
+      __syncthreads();
+      // the next item: known from the draw on
+      bool have_next = false, drew = false;
+      int head_next = 0;
+      int4 entry = {0, 0, 0, 0};
+      // The next item's scalars are worked out from its list entry each time they are needed (its first
+      // tiles, its Q rows, its turn): kept across the last pair they would not fit the scalar registers.
+      auto prefetch_next = [&]() {
+        Work k;
+        work_from_item(fresh(), entry, head_next, k);
+        const DmaCtx ncx = ctx_of(k);
+        int n_tlo, n_nt;
+        range_of(k, n_tlo, n_nt);
+        if (n_tlo < n_nt) dma_step(ncx, n_tlo, std::integral_constant<int, 0>{});
+        if (n_tlo + 1 < n_nt) dma_step(ncx, n_tlo + 1, std::integral_constant<int, 1>{});
+      };
+      // Every item starts at ring stage 0 (the stage is a compile-time constant everywhere; a stage picked at
+      // run time costs the block code 60 registers).  Its steps go in pairs through stages (0, 1) and (2, 3) in
+      // turn, an even number of pairs: with an odd number of real ones the last pair at (2, 3) has no steps.
+      // That last pair is where the next item's first tiles are sent for (into stages (0, 1), free since the
+      // barrier before it) and, once the last logits are done, its Q rows; it ends without waiting for
+      // them: the item's rows are written while they arrive.
+      for (int t = t_lo;; t += 4) {
+        // stages (0, 1)
+        const bool draw = !drew && t + 8 >= nt;
+        if (t + 2 < nt) dma_step(cx, t + 2, std::integral_constant<int, 2>{});
+        if (t + 3 < nt) dma_step(cx, t + 3, std::integral_constant<int, 3>{});
+        uint32_t drawn = 0u;
+        if (draw && tid == 0) drawn = __hip_atomic_fetch_add(p.ctr + xcd, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (t < nt && live(t)) block(t, std::integral_constant<int, 0>{});
+        if (t + 1 < nt && live(t + 1)) block(t + 1, std::integral_constant<int, 1>{});
+        HSTU_WAIT_VMCNT(0);
+        if (draw && tid == 0) xch[1] = drawn;
+        __syncthreads();
+        // stages (2, 3)
+        if (draw) {
+          drew = true;
+          const int job_next = slots + __builtin_amdgcn_readfirstlane((int)xch[1]);
+          const int it_next = job_item(job_next, head_next);
+          have_next = it_next < n_items;
+          if (have_next) {
+            // (a scalar load by hand: this kernel also writes memory, so the compiler would fetch the entry
+            // once per lane into vector registers)
+            typedef int intx4 __attribute__((ext_vector_type(4)));
+            intx4 e4;
+            asm volatile("s_load_dwordx4 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(e4) : "s"(items + it_next));
+            entry.x = e4.x; entry.y = e4.y; entry.z = e4.z; entry.w = e4.w;
           }
-          a0 += x0;
-          a1 += x1;
         }
-        o[i >> 2][4 * (i & 3) + 2 * j] = a0;
-        o[i >> 2][4 * (i & 3) + 2 * j + 1] = a1;
+        const bool last = t + 4 >= nt;
+        if (!last) {
+          dma_step(cx, t + 4, std::integral_constant<int, 0>{});
+          if (t + 5 < nt) dma_step(cx, t + 5, std::integral_constant<int, 1>{});
+        } else if (have_next) {
+          prefetch_next();
+        }
+        if (t + 2 < nt && live(t + 2)) block(t + 2, std::integral_constant<int, 2>{});
+        if (t + 3 < nt && live(t + 3)) block(t + 3, std::integral_constant<int, 3>{});
+        if (last && have_next) {             // the Q registers are free: this item's last logits are done
+          Work k;
+          work_from_item(fresh(), entry, head_next, k);
+          load_q(k);
+        }
+        if (!last) HSTU_WAIT_VMCNT(0);
+        __syncthreads();
+        if (last) break;
+      }
+      // stages (2, 3) are free now (the next item's tiles are landing in (0, 1)): they take the waves' staging tiles
+      finish_item(2 * SM::STAGE);
+      have = have_next;
+      if (have) {
+        const int head_before = h;
+        Work k;
+        work_from_item(fresh(), entry, head_next, k);
+        begin_item(k);
+        settle_q();
+        if (TS && h != head_before) load_ts_table(h);
       }
     }
-  }
-  // Each wave turns its O^T fragment into whole output rows through LDS (the ring is free now: the
-  // loop ended on a barrier and no load is in flight), so that global memory sees 16-byte stores that
-  // cover full rows instead of 8-byte pieces: lane (row m, half hh) writes 8 bytes of row m at a
-  // time, 16-byte chunks XOR-swizzled by row against bank conflicts, then reads 16 bytes per lane,
-  // 64 / (D/8) rows per instruction.  Only lanes of the same wave exchange data here and LDS
-  // executes a wave's operations in order: no barrier is needed.
-  const float oscale = p.inv_n * (1.0f / LOG2E);
-  unsigned char* ot = smem + w * (32 * D * 2);
-  auto oswz = [](int row) { return (row / SM::RPB) % CPR; };
-  {
-    const bool live = qrow < s.n_q;
-    unsigned char* orow = ot + m * (D * 2) + 8 * hh;
-#pragma unroll
-    for (int dvb = 0; dvb < DVB; ++dvb) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint2 pko = {0u, 0u};
-        if (live) {
-          pko.x = pack_bf16(o[dvb][4 * g + 0] * oscale, o[dvb][4 * g + 1] * oscale);
-          pko.y = pack_bf16(o[dvb][4 * g + 2] * oscale, o[dvb][4 * g + 3] * oscale);
-        }
-        *(uint2*)(orow + (((4 * dvb + g) ^ oswz(m)) * 16)) = pko;
+    // the last workgroup out leaves the draw counters at zero for the next launch
+    if (tid == 0) {
+      const uint32_t done = __hip_atomic_fetch_add(p.ctr + 8, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (done == gridDim.x - 1) {
+        for (int i = 0; i < 9; ++i) __hip_atomic_store(p.ctr + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-    }
-  }
-  constexpr int ROWS_PER_STORE = 64 / CPR;
-  const int rr = lane / CPR, cc = lane - rr * CPR;
-#pragma unroll
-  for (int r0s = 0; r0s < 32; r0s += ROWS_PER_STORE) {
-    const int row = r0s + rr;
-    const uint4 val = *(const uint4*)(ot + row * (D * 2) + ((cc ^ oswz(row)) * 16));
-    const int grow = r0 + row;
-    if (grow < s.rows) {
-      // streaming store: the output is not read again by this kernel, and K / V rows that other tiles of the
-      // sequence still need are worth more of the L2 than it is (d = 64 benchmark shape: 134 -> 122 us)
-      typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
-      const uintx4 vv = {val.x, val.y, val.z, val.w};
-      __builtin_nontemporal_store(vv, (uintx4*)(og + (int64_t)grow * p.o_st + cc * 8));
     }
   }
 }
@@ -2942,7 +3156,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, 
       w.items_max = t128 + w.split_cap;     // every tile one item, and one more per chunk slot at most
       w.sched_bytes = up((size_t)(4 + 4 * w.items_max) * sizeof(int32_t));
     }
-    w.ctr_bytes = w.split_cap ? up((size_t)(CTR_RESERVED + (size_t)w.split_cap * a->H) * sizeof(uint32_t)) : 0;
+    w.ctr_bytes = list ? up((size_t)(CTR_RESERVED + (size_t)w.split_cap * a->H) * sizeof(uint32_t)) : 0;
     w.partial_bytes = up((size_t)w.split_cap * chunk_bytes);
     if (w.total() <= max_bytes || w.split_cap == 0) break;
     const size_t over = w.total() - max_bytes;
@@ -3037,15 +3251,17 @@ int launch_bwd(const Params& p, hipStream_t st) {
   return HSTU_OK;
 }
 
-template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0>
+template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0, bool PERSIST = false>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE, fwd_stages(D, DENSE)) + FWD_XCH_BYTES;
   static int granted[64];
-  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE>, smem, granted)) return rc;
+  if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE, PERSIST>, smem, granted)) return rc;
   hipError_t e;
-  const long long blocks = mfma_grid(p);
+  long long blocks = mfma_grid(p);
+  // resident workgroups: as many as run at once, fewer when the list cannot be longer than that
+  if (PERSIST && blocks > 8LL * p.n_slots) blocks = 8LL * p.n_slots;
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
+  hipLaunchKernelGGL((hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE, PERSIST>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "mfma kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
@@ -3064,6 +3280,14 @@ int launch_mfma_d(const Params& p, hipStream_t st) {
     if (pos) return launch_mfma_inst<D, true, false, false, true>(p, st);
     if (ts) return launch_mfma_inst<D, false, true, false, true>(p, st);
     return launch_mfma_inst<D, false, false, false, true>(p, st);
+  }
+  if constexpr (D == 128 && !F8) {
+    if (p.persist) {
+      if (pos && ts) return launch_mfma_inst<D, true, true, false, false, 0, true>(p, st);
+      if (pos) return launch_mfma_inst<D, true, false, false, false, 0, true>(p, st);
+      if (ts) return launch_mfma_inst<D, false, true, false, false, 0, true>(p, st);
+      return launch_mfma_inst<D, false, false, false, false, 0, true>(p, st);
+    }
   }
   if (pos && ts) return launch_mfma_inst<D, true, true, F8>(p, st);
   if (pos) return launch_mfma_inst<D, true, false, F8>(p, st);
@@ -3139,7 +3363,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
   blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
   if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
-  if ((ws.bias_total() || ws.sched_bytes) && !(args->flags & HSTU_FWD_WORKSPACE_PREPARED)) {
+  if ((ws.bias_total() || ws.sched_bytes) && (!(args->flags & HSTU_FWD_WORKSPACE_PREPARED) || (args->flags & HSTU_FWD_PREPARE_ONLY))) {
     static const TsKeys no_keys = {{0}, {0}, {0}};
     const TsKeys& keys = tab_out ? bucket_law(q.ts_bucket_size).keys : no_keys;
     hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out, keys);
@@ -3340,6 +3564,19 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
       const WorkspacePlan ws = plan_workspace(args, true, args->workspace ? args->workspace_bytes : 0);
       Params q = p;
       if (int rc2 = setup_workspace(args, ws, q, st)) return rc2;
+      if (args->flags & HSTU_FWD_PREPARE_ONLY) return HSTU_OK;
+      // Resident workgroups over the work list, where that loop is built (d = 128 in bf16, lengths or no mask)
+      // and where it pays: with many items per resident workgroup.  (B = 64, L = 2048, H = 8, every sequence
+      // full, 17 items each: 0.962 -> 0.924 ms.  The jagged headline shape has under 3 items each; there the
+      // end of the launch, where each workgroup finishes whatever it drew last, costs more than the items'
+      // starts save: 69 -> 77 us.)  The padded layout with lengths leaves the host guessing the number of
+      // items: one workgroup per item there.
+      const bool can_stay = q.sched && q.ctr && q.d_qk == 128 && !f8 && !q.mask && !q.dense_bias && q.mask_mode != HSTU_MASK_SEGMENT;
+      const bool count_known = q.jagged || !q.seq_lens;
+      const long long tiles = q.jagged ? args->total_tokens / BM + args->B : (long long)args->B * q.n_qtiles;
+      const long long jobs_per_xcd = q.H >= 8 ? tiles * (q.H >> 3) : tiles / (8 / q.H);
+      q.persist = can_stay && !(args->flags & HSTU_FWD_ONE_ITEM_PER_WORKGROUP) &&
+                  ((args->flags & HSTU_FWD_RESIDENT_WORKGROUPS) || (count_known && jobs_per_xcd >= 8LL * q.n_slots));
       if (int rc2 = f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st)) return rc2;
       return HSTU_OK;
     }
@@ -3348,3 +3585,4 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
 }
 
 }  // extern "C"
+

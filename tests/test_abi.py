@@ -143,9 +143,9 @@ def test_variant_and_workspace_query():
   a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
   # the matrix-core kernel always wants a workspace: a work list of one int4 per query tile
-  # (2 sequences x 2 tiles here) behind a 16-byte header ...
+  # (2 sequences x 2 tiles here) behind a 16-byte header and 16 counters behind that ...
   up = lambda x: (x + 255) // 256 * 256
-  sched = up(16 + 16 * 2 * 2)
+  sched = up(16 + 16 * 2 * 2) + up(4 * 16)
   assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == sched
   # ... plus, with a position table, its scaled and padded copy
   a.pos_tab, a.pos_heads = 0x20000, 4

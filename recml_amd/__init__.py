@@ -7,6 +7,7 @@ HSTU block and model forward (recml/layers/keras/hstu.py:240-621).
 """
 
 from recml_amd.hstu_ops import (  # noqa: F401
+    AttentionBatch,
     MaskType,
     hstu_attention,
     hstu_attention_autograd,

@@ -908,35 +908,17 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
   const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
   if (sched_out && blockIdx.x == gridDim.x - 1) {
     // The work list, by the last workgroup (the host launches one more than the rest needs).
-    // Sequences are taken longest first (batches of up to SORT_MAX sequences; larger ones in
-    // batch order): the tiles with most keys start first and short ones fill in behind them.
-    // Thread t owns a run of sequences in that order.  Three walks over its tiles: the steps of all
-    // tiles (what decides which tiles are split), the chunk slots its split tiles ask for, and the
-    // items themselves, last query tile (most keys) first within a sequence; a prefix sum over the
-    // threads after the second and the third tells where a thread's slots and items start.
-    constexpr int SORT_MAX = 1024;
+    // Sequences are taken longest first (batches of up to SEG sequences; larger ones in batch order,
+    // SEG at a time): the tiles with most keys start first and short ones fill in behind them.  Within
+    // a sequence the last query tile (most keys) comes first.  The tiles of the sequences at hand are
+    // numbered in that order and dealt to the threads 256 at a time (a thread finds its tile's
+    // sequence by bisection over the prefix sums of the tiles per sequence); prefix sums over the
+    // threads tell each tile where its chunk slots and its items start.  Two passes: the steps of all
+    // tiles (what decides which tiles are split), then the items.
+    constexpr int SEG = 1024;
     __shared__ int wave_sums[4];
-    __shared__ int keys[SORT_MAX], firsts[SORT_MAX], order[SORT_MAX];
-    const bool sorted = p.B <= SORT_MAX;
-    if (sorted) {
-      for (int b = tid; b < p.B; b += 256) {
-        int o0, nraw;
-        seq_raw(p, b, o0, nraw);
-        keys[b] = nraw;
-        firsts[b] = o0;
-      }
-      __syncthreads();
-      for (int b = tid; b < p.B; b += 256) {
-        const int kb = keys[b];
-        int rank = 0;
-#pragma unroll 8
-        for (int c = 0; c < p.B; ++c) rank += (keys[c] > kb || (keys[c] == kb && c < b)) ? 1 : 0;
-        order[rank] = b;
-      }
-      __syncthreads();
-    }
-    const int per = (p.B + 255) / 256;
-    const int r_lo = tid * per < p.B ? tid * per : p.B, r_hi = r_lo + per < p.B ? r_lo + per : p.B;
+    __shared__ int keys[SEG], firsts[SEG], order[SEG], tbase[SEG + 1];
+    const bool sorted = p.B <= SEG;
     int4* items = (int4*)(sched_out + 4);
     // sum over the workgroup and exclusive prefix of this thread's value (all 256 threads take part)
     auto block_scan = [&](int v, int& total) {
@@ -958,11 +940,73 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       }
       return base;
     };
-    auto seq_of = [&](int r, int& b, int& o0, int& nraw) {
-      b = sorted ? order[r] : r;
-      if (sorted) { o0 = firsts[b]; nraw = keys[b]; }
-      else seq_raw(p, b, o0, nraw);
-      return seq_from(p, b, 0, o0, nraw);
+    // rows with output, keys and rows of the tile space of a sequence of stored length nraw (as seq_from)
+    auto dims = [&](int nraw, int& nq, int& nk, int& rows) {
+      if (p.jagged) {
+        const int n = nraw < 0 ? 0 : (nraw > p.L ? p.L : nraw);
+        nq = n; nk = n; rows = n;
+      } else {
+        nq = p.L; nk = p.Lkv; rows = p.L;
+        if (p.mask_mode == HSTU_MASK_LENGTH) {
+          const int n = nraw < 0 ? 0 : nraw;
+          nq = n < p.L ? n : p.L;
+          nk = n < p.Lkv ? n : p.Lkv;
+        }
+      }
+    };
+    auto steps_of = [&](int nq, int nk, int q0) {       // as tile_steps
+      if (q0 >= nq) return 0;
+      int kv_end = nk;
+      const int row_end = q0 + BM < nq ? q0 + BM : nq;
+      if (p.causal) kv_end = row_end < kv_end ? row_end : kv_end;
+      if (p.window >= 0 && row_end - 1 + p.window + 1 < kv_end) kv_end = row_end + p.window;
+      return (kv_end + BN - 1) / BN;
+    };
+    // Sequences [s0, s0 + cnt) into LDS: stored lengths and first tokens, their order, the prefix sums of
+    // their tiles.  Returns the number of tiles.
+    auto load_segment = [&](int s0, int cnt) {
+      __syncthreads();            // the readers of the segment before are done
+      for (int i = tid; i < cnt; i += 256) {
+        int o0, nraw;
+        seq_raw(p, s0 + i, o0, nraw);
+        keys[i] = nraw;
+        firsts[i] = o0;
+      }
+      __syncthreads();
+      for (int i = tid; i < cnt; i += 256) {
+        int rank = i;
+        if (sorted) {
+          const int kb = keys[i];
+          rank = 0;
+#pragma unroll 8
+          for (int c = 0; c < cnt; ++c) rank += (keys[c] > kb || (keys[c] == kb && c < i)) ? 1 : 0;
+        }
+        order[rank] = i;
+      }
+      __syncthreads();
+      int c[SEG / 256], sum = 0;
+#pragma unroll
+      for (int k = 0; k < SEG / 256; ++k) {
+        const int r = tid * (SEG / 256) + k;
+        c[k] = 0;
+        if (r < cnt) {
+          int nq, nk, rows;
+          dims(keys[order[r]], nq, nk, rows);
+          c[k] = (rows + BM - 1) / BM;
+        }
+        sum += c[k];
+      }
+      int total;
+      int base = block_scan(sum, total);
+#pragma unroll
+      for (int k = 0; k < SEG / 256; ++k) {
+        const int r = tid * (SEG / 256) + k;
+        if (r < cnt) tbase[r] = base;
+        base += c[k];
+      }
+      if (tid == 0) tbase[cnt] = total;
+      __syncthreads();
+      return total;
     };
     // chunks of a tile of nt steps once the threshold is known: balanced parts of at most split_steps
     auto chunks_of = [&](int nt, int split_steps) {
@@ -970,13 +1014,35 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       const int c = (nt + split_steps - 1) / split_steps;
       return c < MAX_CHUNKS ? c : MAX_CHUNKS;
     };
-    int split_steps = 0;
+    // A thread's run of the segment's tiles, [f_lo, f_hi): one bisection finds the first tile's sequence, the
+    // rest follow in order.  fn(i, qt, nq, nk): index of the sequence within the segment, query tile, dimensions.
+    auto walk = [&](int cnt, int f_lo, int f_hi, auto&& fn) {
+      if (f_lo >= f_hi) return;
+      int lo = 0, hi = cnt;       // the last r with tbase[r] <= f_lo (those before it with the same value have no tiles)
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tbase[mid] <= f_lo) lo = mid; else hi = mid;
+      }
+      int r = lo;
+      for (int f = f_lo; f < f_hi;) {
+        while (f >= tbase[r + 1]) ++r;
+        const int i = order[r], t0 = tbase[r], t1 = tbase[r + 1];
+        int nq, nk, rows;
+        dims(keys[i], nq, nk, rows);
+        const int last = f_hi < t1 ? f_hi : t1;
+        for (; f < last; ++f) fn(i, (t1 - t0) - 1 - (f - t0), nq, nk);
+      }
+    };
+    const int nseg = (p.B + SEG - 1) / SEG;
+    int split_steps = 0, tiles = -1;
     if (p.split_cap > 0) {
       int steps = 0;
-      for (int r = r_lo; r < r_hi; ++r) {
-        int b, o0, nraw;
-        const Seq sq = seq_of(r, b, o0, nraw);
-        for (int q0 = 0; q0 < sq.n_q; q0 += BM) steps += tile_steps(p, sq, q0);
+      for (int sg = 0; sg < nseg; ++sg) {
+        const int cnt = p.B - sg * SEG < SEG ? p.B - sg * SEG : SEG;
+        tiles = load_segment(sg * SEG, cnt);
+        const int per = (tiles + 255) / 256;
+        walk(cnt, tid * per < tiles ? tid * per : tiles, (tid + 1) * per < tiles ? (tid + 1) * per : tiles,
+             [&](int, int qt, int nq, int nk) { steps += steps_of(nq, nk, qt * BM); });
       }
       int total;
       block_scan(steps, total);
@@ -986,45 +1052,44 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       const long long avg = (per_xcd + p.n_slots - 1) / p.n_slots;
       split_steps = avg < 8 ? 8 : (avg > 0x3fffffff ? 0x3fffffff : (int)avg);
     }
-    // chunk slots this thread's split tiles ask for, then where they start
-    int want = 0;
-    for (int r = r_lo; r < r_hi && split_steps > 0; ++r) {
-      int b, o0, nraw;
-      const Seq sq = seq_of(r, b, o0, nraw);
-      for (int q0 = 0; q0 < sq.n_q; q0 += BM) {
-        const int c = chunks_of(tile_steps(p, sq, q0), split_steps);
-        want += c > 1 ? c : 0;
-      }
-    }
-    int total_slots = 0;
-    const int slot0 = split_steps > 0 ? block_scan(want, total_slots) : 0;
-    // one walk shared by the count and the write: a tile is split only while chunk slots last
-    auto walk = [&](int base, bool write) {
-      int n = 0, slot = slot0;
-      for (int r = r_lo; r < r_hi; ++r) {
-        int b, o0, nraw;
-        const Seq sq = seq_of(r, b, o0, nraw);
-        for (int qt = (sq.rows + BM - 1) / BM - 1; qt >= 0; --qt) {
-          int c = 1, ps = 0;
-          if (qt * BM < sq.n_q) {
-            c = chunks_of(tile_steps(p, sq, qt * BM), split_steps);
-            if (c > 1) {
-              ps = slot;
-              slot += c;
-              if (ps + c > p.split_cap) c = 1;      // the partial buffer is full: this tile stays whole
-            }
+    int item_base = 0, slot_base = 0;
+    for (int sg = 0; sg < nseg; ++sg) {
+      const int cnt = p.B - sg * SEG < SEG ? p.B - sg * SEG : SEG;
+      if (nseg > 1 || tiles < 0) tiles = load_segment(sg * SEG, cnt);     // (a single segment is still there from the first pass)
+      const int per = (tiles + 255) / 256;
+      const int f_lo = tid * per < tiles ? tid * per : tiles, f_hi = (tid + 1) * per < tiles ? (tid + 1) * per : tiles;
+      // the chunk slots this thread's tiles ask for, and where they start: a tile is split only while slots last
+      int want = 0, asked = 0;
+      if (split_steps > 0)
+        walk(cnt, f_lo, f_hi, [&](int, int qt, int nq, int nk) {
+          const int c = chunks_of(steps_of(nq, nk, qt * BM), split_steps);
+          want += c > 1 ? c : 0;
+        });
+      const int slot0 = split_steps > 0 ? slot_base + block_scan(want, asked) : 0;
+      // one walk shared by the count and the write
+      auto emit = [&](int base, bool write) {
+        int n = 0, slot = slot0;
+        walk(cnt, f_lo, f_hi, [&](int i, int qt, int nq, int nk) {
+          int c = chunks_of(steps_of(nq, nk, qt * BM), split_steps), ps = 0;
+          if (c > 1) {
+            ps = slot;
+            slot += c;
+            if (ps + c > p.split_cap) { c = 1; ps = 0; }      // the partial buffer is full: this tile stays whole
           }
           for (int k = 0; k < c; ++k, ++n)
-            if (write && base + n < p.items_max) items[base + n] = int4{b | (ps << 14), qt | (k << 16) | (c << 24), o0, nraw};
-        }
-      }
-      return n;
-    };
-    int total;
-    const int base = block_scan(walk(0, false), total);
-    walk(base, true);
+            if (write && base + n < p.items_max)
+              items[base + n] = int4{(sg * SEG + i) | (ps << 14), qt | (k << 16) | (c << 24), firsts[i], keys[i]};
+        });
+        return n;
+      };
+      int made;
+      const int at = item_base + block_scan(emit(0, false), made);
+      emit(at, true);
+      slot_base += asked;
+      item_base += made;
+    }
     if (tid == 0) {
-      sched_out[0] = total < p.items_max ? total : (int)p.items_max;
+      sched_out[0] = item_base < p.items_max ? item_base : (int)p.items_max;
       sched_out[1] = split_steps;
     }
     // the arrival counters of the split tiles start at zero (their last arriver leaves them so again)
@@ -1069,11 +1134,20 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       continue;
     }
     const int64_t* ts = p.ts + s.ts0;
+    // (eight loads in flight per thread: one memory round trip per 2048 timestamps instead of eight)
     int64_t lo_v = ts[0], hi_v = lo_v;
-    for (int j = tid; j < n; j += 256) {
-      const int64_t x = ts[j];
-      lo_v = x < lo_v ? x : lo_v;
-      hi_v = x > hi_v ? x : hi_v;
+    for (int j0 = 0; j0 < n; j0 += 2048) {
+      int64_t x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int j = j0 + i * 256 + tid;
+        x[i] = ts[j < n ? j : n - 1];
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        lo_v = x[i] < lo_v ? x[i] : lo_v;
+        hi_v = x[i] > hi_v ? x[i] : hi_v;
+      }
     }
 #pragma unroll
     for (int d = 32; d >= 1; d >>= 1) {
@@ -1094,20 +1168,28 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     int32_t* rel = rel_out + ts_rel_base(p, b, s.tok0);
     int32_t* rng = range_out + 2 * ts_range_slot0(p, b, s.tok0);
     const int tiles = (n + BN - 1) / BN;
-    for (int t = tid >> 5; t < tiles; t += 8) {   // one half-wave per tile
-      int j = t * BN + l32;
-      const bool live = j < n;
-      j = live ? j : n - 1;
-      const int32_t r = (int32_t)(ts[j] - lo_v);
-      if (live) rel[j] = r;
-      int32_t mn = r, mx = r;
+    for (int t0 = 0; t0 < tiles; t0 += 64) {      // one half-wave per tile, eight tiles in flight per half-wave
+      int64_t x[8];
 #pragma unroll
-      for (int d = 16; d >= 1; d >>= 1) {
-        const int32_t a = __shfl_xor(mn, d, 32), c = __shfl_xor(mx, d, 32);
-        mn = a < mn ? a : mn;
-        mx = c > mx ? c : mx;
+      for (int i = 0; i < 8; ++i) {
+        const int j = (t0 + 8 * i + (tid >> 5)) * BN + l32;
+        x[i] = ts[j < n ? j : n - 1];
       }
-      if (l32 == 0) { rng[2 * t] = mn; rng[2 * t + 1] = mx; }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int t = t0 + 8 * i + (tid >> 5);
+        const int j = t * BN + l32;
+        const int32_t r = (int32_t)(x[i] - lo_v);
+        if (j < n) rel[j] = r;
+        int32_t mn = r, mx = r;
+#pragma unroll
+        for (int d = 16; d >= 1; d >>= 1) {
+          const int32_t a = __shfl_xor(mn, d, 32), c = __shfl_xor(mx, d, 32);
+          mn = a < mn ? a : mn;
+          mx = c > mx ? c : mx;
+        }
+        if (l32 == 0 && t < tiles) { rng[2 * t] = mn; rng[2 * t + 1] = mx; }
+      }
     }
   }
 }

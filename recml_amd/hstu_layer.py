@@ -39,17 +39,18 @@ def _wants_grad(*tensors) -> bool:
   return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
 
 
-def _attention(q, k, v, *, pos_bias=None, ts_bias=None, **kw):
+def _attention(q, k, v, *, pos_bias=None, ts_bias=None, batch=None, **kw):
   """The attention op, differentiable when anything it reads wants a gradient: through the HIP
   backward kernels for q, k, v and the bias tables; through plain torch when a dense bias wants one
-  (the kernels return no gradient for it)."""
+  (the kernels return no gradient for it).  `batch`: the per-batch preparation shared by the layers
+  (inference only)."""
   if _wants_grad(kw.get("bias")):
     if q.dim() != 4:
       raise ValueError("a dense bias that requires a gradient needs the padded layout")
     return hstu_ops.dense_attention_torch(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
   if _wants_grad(q, k, v, pos_bias, ts_bias):
     return hstu_ops.hstu_attention_autograd(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
-  return hstu_ops.hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
+  return hstu_ops.hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, batch=batch, **kw)
 
 
 def _glorot_uniform(shape, fan_in, fan_out, generator, dtype, device):
@@ -108,14 +109,15 @@ class HSTUBlock(torch.nn.Module):
     return shape[-2] * rf, shape[-1] * rf
 
   def forward(self, inputs, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None,
-              attention_mask=None, attention_bias=None):
+              attention_mask=None, attention_bias=None, batch=None):
     """inputs [B, L, D] -> [B, L, D].
 
     Give `seq_lens` [B] (keys and rows at or past the length are masked, as
     make_causal_mask does for an end-padded batch) with optional bias tables;
     or, for the reference's calling convention, a dense `attention_mask`
     [B, L, L] and optional `attention_bias` [B, L, L]
-    (recml/layers/keras/hstu.py:422-440).
+    (recml/layers/keras/hstu.py:422-440).  `batch`: an `hstu_ops.AttentionBatch` shared with the
+    other blocks that see the same lengths, timestamps and tables.
     """
     B, L, D = inputs.shape
     H, hd = self.num_heads, self.head_dim
@@ -141,7 +143,7 @@ class HSTUBlock(torch.nn.Module):
     else:
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
-                        timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias)
+                        timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias, batch=batch)
     if fused:
       gated = hstu_block_ops.norm_gate(attn.reshape(B * L, H * hd), u.reshape(B * L, H * hd), self.attn_ln_gamma.reshape(-1),
                                        self.attn_ln_beta.reshape(-1), self.eps)
@@ -169,7 +171,7 @@ class HSTUBlock(torch.nn.Module):
     b = torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1) if self.use_bias else None
     return w, b
 
-  def forward_jagged(self, tokens, seq_offsets, max_len, *, pos_bias=None, timestamps=None, ts_bias=None):
+  def forward_jagged(self, tokens, seq_offsets, max_len, *, pos_bias=None, timestamps=None, ts_bias=None, batch=None):
     """The block on packed tokens [T, D] (sequence b = rows seq_offsets[b]..seq_offsets[b+1]):
     no work at all for padding, in the projections either.  `timestamps` is jagged [T].
 
@@ -191,7 +193,7 @@ class HSTUBlock(torch.nn.Module):
     u, q, k, v = uqkv.unbind(dim=1)
     alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
     attn = _attention(q, k, v, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
-                      pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
+                      pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, batch=batch)
     if fused:
       gated = hstu_block_ops.norm_gate(attn.reshape(T, H * hd), u.reshape(T, H * hd), self.attn_ln_gamma.reshape(-1),
                                        self.attn_ln_beta.reshape(-1), self.eps)
@@ -276,8 +278,10 @@ class HSTU(torch.nn.Module):
       if self.position_embedding is not None:
         x = x + self.position_embedding[: x.shape[1]]
       x = self._final_norm(x)
+    # every block sees the same lengths, timestamps and tables: the attention prepares them once
+    batch = hstu_ops.AttentionBatch()
     for block in self.decoder_blocks:
-      x = block(x, seq_lens=seq_lens, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias)
+      x = block(x, seq_lens=seq_lens, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, batch=batch)
     x = self._final_norm(x)
     if self.reverse_embedding is None:
       return x
@@ -303,8 +307,9 @@ class HSTU(torch.nn.Module):
         x = x + self.position_embedding[pos_idx]
       x = self._final_norm(x)
     ts = None if timestamps is None else timestamps[valid]
+    batch = hstu_ops.AttentionBatch()
     for block in self.decoder_blocks:
-      x = block.forward_jagged(x, offsets, L, pos_bias=pos_bias, timestamps=ts, ts_bias=ts_bias)
+      x = block.forward_jagged(x, offsets, L, pos_bias=pos_bias, timestamps=ts, ts_bias=ts_bias, batch=batch)
     x = self._final_norm(x)
     if self.reverse_embedding is not None:
       x = x @ self.reverse_embedding

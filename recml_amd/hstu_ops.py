@@ -77,6 +77,58 @@ def _attach_workspace(args, keep):
     args.workspace_bytes = ws
 
 
+class AttentionBatch:
+  """What the attention prepares from a batch before its kernel runs -- the work list, the timestamps
+  as 32-bit offsets with their per-tile ranges, the scaled bias tables -- kept for every call on that
+  batch: a model hands one of these to all its layers, and only the first call pays the preparation
+  (`HSTU.forward` does).  It also keeps the device scratch, so no call after the first allocates.
+
+  The preparation is reused when the call's shapes and options are the same and the tensors it was
+  built from (`seq_lens` / `seq_offsets`, `timestamps`, `pos_bias`, `ts_bias`) are the same objects,
+  unmodified since (torch's version counter); anything else prepares again.  q, k, v, `alpha` and `n`
+  may differ from call to call.  Not for concurrent use on several streams.
+  """
+
+  def __init__(self):
+    self._buf = None
+    self._prepared = None     # signature the workspace was prepared for
+    self._pending = None
+    self._tensors = ()        # keeps the signature's tensors alive (their addresses are part of it)
+    self.prepared_calls = 0   # calls that skipped the preparation
+
+  @staticmethod
+  def _ident(t):
+    if t is None:
+      return None
+    if not isinstance(t, torch.Tensor):
+      return False            # not a tensor: never reused
+    return (t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride()), t.dtype)
+
+  def _attach(self, args, keep, sig, tensors):
+    ws = _lib.load().hstu_attn_fwd_workspace_bytes(C.byref(args))
+    if not ws:
+      return
+    dev = keep[0].device
+    if self._buf is None or self._buf.numel() != ws or self._buf.device != dev:
+      self._buf = torch.empty(ws, dtype=torch.uint8, device=dev)
+      self._prepared = None
+    keep.append(self._buf)
+    args.workspace = self._buf.data_ptr()
+    args.workspace_bytes = ws
+    self._pending = None
+    if sig is not None and sig == self._prepared:
+      args.flags |= _lib.FWD_WORKSPACE_PREPARED
+      self.prepared_calls += 1
+    else:
+      self._prepared = None
+      self._pending = (sig, tensors)
+
+  def _commit(self):
+    if self._pending is not None:
+      self._prepared, self._tensors = self._pending
+      self._pending = None
+
+
 def _passed_inputs(keep):
   """The q, k, v tensors whose pointers build_args put into the struct (after any copy)."""
   return keep[0], keep[1], keep[2]
@@ -102,8 +154,9 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
                timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                q_segment_ids=None, kv_segment_ids=None,
                sliding_window_size=None, mask=None, bias=None,
-               q_scale=None, k_scale=None):
+               q_scale=None, k_scale=None, batch=None):
   """Validates the call and fills an HstuAttnFwdArgs.  Returns (args, keepalive)."""
+  given = (seq_lens, seq_offsets, timestamps, pos_bias, ts_bias)
   for name, t in (("q", q), ("k", k), ("v", v)):
     _check_gpu(name, t)
   if q.dtype not in _DTYPES:
@@ -272,7 +325,17 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
     a.ts_num_buckets = tt.shape[1] - 1
     a.ts_bucket_size = float(ts_bucket_size)
   if q.is_cuda:
-    _attach_workspace(a, keep)
+    if batch is None:
+      _attach_workspace(a, keep)
+    else:
+      # everything the preparation reads or the workspace layout depends on; dense operands and segment
+      # ids (not part of it, but of the choice of kernel) rule the reuse out
+      sig = None
+      idents = tuple(AttentionBatch._ident(t) for t in given)
+      if mask is None and bias is None and q_segment_ids is None and False not in idents:
+        sig = (tuple(q.shape), tuple(k.shape), int(v.shape[-1]), q.dtype, max_len, bool(causal),
+               sliding_window_size, float(ts_bucket_size), idents)
+      batch._attach(a, keep, sig, given)
   return a, keep
 
 
@@ -281,7 +344,7 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
                    timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                    q_segment_ids=None, kv_segment_ids=None,
                    sliding_window_size=None, mask=None, bias=None, out=None,
-                   q_scale=None, k_scale=None):
+                   q_scale=None, k_scale=None, batch=None):
   """out = (silu(alpha * q k^T + bias) / n, masked) v.
 
   Args:
@@ -310,6 +373,8 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
     bias: dense additive logit bias [L, Lkv] or [B, L, Lkv] shared by heads
       (hstu.py:373-374).
     out: optional preallocated output.
+    batch: optional AttentionBatch shared by the calls on one batch (a model's layers): the first
+      call prepares the work list, timestamps and tables, the later ones reuse them.
 
   Returns:
     Tensor shaped like q with v's head dim and v's dtype.
@@ -325,9 +390,11 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
       timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
       q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids,
       sliding_window_size=sliding_window_size, mask=mask, bias=bias,
-      q_scale=q_scale, k_scale=k_scale)
+      q_scale=q_scale, k_scale=k_scale, batch=batch)
   with torch.cuda.device(q.device):
     _run(args, keep)
+  if batch is not None:
+    batch._commit()
   return out
 
 

@@ -163,14 +163,23 @@ int hstu_attn_abi_version(void);
 /* Bytes of device scratch the call needs for these arguments; pass a buffer of
  * at least that size, 256-byte aligned, in args->workspace.  0 for calls the
  * general kernel serves.  For the matrix-core kernel it holds what a small
- * preparation kernel rebuilds on every call: the work list of (sequence,
- * query tile) items, the scaled position and bucket tables, int32 timestamps
- * with their per-tile ranges and, when few long sequences underfill the GPU,
- * fp32 partial outputs of query tiles whose key range is split.  The size
+ * preparation kernel builds (on every call, or once per batch, see
+ * HSTU_FWD_PREPARE_ONLY): the work list of (sequence, query tile, key chunk)
+ * items, the scaled position table, the timestamp bucket tables, int32
+ * timestamps with their per-tile ranges; and what the main kernel itself
+ * uses: the counters it draws work from and, for query tiles whose keys are
+ * split between workgroups (decided on the device from the lengths, when few
+ * long tiles would otherwise finish long after the rest), the arrival counters
+ * and up to 32 fp32 partial outputs of 128 rows x H heads x d_v, summed in a
+ * fixed order by whichever workgroup of the tile arrives last: the result does
+ * not depend on the order of arrival.  A larger buffer than asked for is fine;
+ * a smaller one that still holds everything but the partial outputs makes the
+ * library split fewer tiles (none below two) instead of failing.  The size
  * depends on shapes, options and total_tokens only, never on device data.
- * The contents mean nothing between calls; two calls that overlap on one GPU
- * need two buffers.  No reference counterpart: the reference's op is a pure
- * function under jax.jit. */
+ * Counters are left at zero by every call; the rest means nothing between
+ * calls unless HSTU_FWD_WORKSPACE_PREPARED says so; two calls that overlap on
+ * one GPU need two buffers.  No reference counterpart: the reference's op is a
+ * pure function under jax.jit. */
 size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
 
 /* Validate `args` and enqueue the forward on `stream` (a hipStream_t passed
@@ -192,8 +201,9 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
  * the scratch that call would need (hstu_attn_fwd_workspace_bytes) lives in
  * a fixed array of HSTU_ATTN_NOALLOC_SCRATCH_BYTES inside the library.  The
  * call allocates and frees nothing, on the device or through any library.
- * Calls whose scratch need exceeds the array return HSTU_ERR_WORKSPACE (use
- * hstu_attn_fwd with a caller buffer then).  Every call on a GPU shares that
+ * Calls whose scratch need exceeds the array even with no tile split return
+ * HSTU_ERR_WORKSPACE (use hstu_attn_fwd with a caller buffer then); between
+ * that and the full need, fewer tiles are split, as with any small workspace.  Every call on a GPU shares that
  * GPU's array: calls that overlap on one GPU (two streams, two threads) race;
  * HSTU_FWD_WORKSPACE_PREPARED refers to what the previous call of this entry
  * point on the same GPU prepared. */
@@ -207,7 +217,9 @@ int hstu_attn_fwd_noalloc(const HstuAttnFwdArgs* args, void* stream);
  * dq, dk, dv those of q, k, v and are fully written (rows past a sequence's
  * length as zeros).  dpos_tab / dts_tab are fp32 tables shaped like pos_tab /
  * ts_tab that are ACCUMULATED into by atomic adds: the caller zero-fills them
- * (or passes null when the table gradient is not wanted).  fp32 or bf16
+ * (or passes null when the table gradient is not wanted).  Those float atomic
+ * adds arrive in no fixed order, so the table gradients may differ in their
+ * last bits from run to run; out, dq, dk and dv are the same bits every run.  fp32 or bf16
  * storage, every option of the forward, fp32 arithmetic; fp8 q/k is not
  * supported.  bf16 calls that meet the conditions of the
  * matrix-core forward (without a dense mask or bias, and with keys and

@@ -70,7 +70,9 @@ int hstu_norm_gate_fwd(const HstuNormGateArgs* args, void* stream);
  * [M, N] contiguous.  fp32 accumulation.  `workspace` (device memory, may be
  * null) is handed to hipBLASLt; hstu_gemm_silu_workspace_bytes() says how much
  * it would like.  The descriptor and the chosen algorithm of a shape are kept
- * by the library after the first call with it. */
+ * by the library after the first call with it: every call must therefore offer
+ * what the first did, so x, w, bias, out and workspace must be 16-byte aligned
+ * and x_stride a multiple of 8 elements (HSTU_BLOCK_ERR_SHAPE otherwise). */
 typedef struct HstuGemmSiluArgs {
   uint32_t struct_size;   /* sizeof(HstuGemmSiluArgs)  */
   uint32_t version;       /* HSTU_BLOCK_ABI_VERSION    */

@@ -342,6 +342,10 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
   g_err[0] = 0;
   if (a->M == 0) return HSTU_BLOCK_OK;
   if (!a->x || !a->w || !a->out) return fail(HSTU_BLOCK_ERR_NULL, "x, w and out must be non-null");
+  // the kernel picked for a shape is kept and reused for every later call of that shape: it may assume what
+  // the first call's pointers offered, so every call has to offer it
+  if (!aligned16(a->x) || !aligned16(a->w) || !aligned16(a->out) || !aligned16(a->bias) || !aligned16(a->workspace) || (a->x_stride & 7))
+    return fail(HSTU_BLOCK_ERR_SHAPE, "x, w, out, bias and workspace must be 16-byte aligned and x_stride a multiple of 8 elements");
   if (a->workspace_bytes && !a->workspace) return fail(HSTU_BLOCK_ERR_WORKSPACE, "workspace_bytes without a workspace");
   int dev = 0;
   hipError_t he = hipGetDevice(&dev);
@@ -363,37 +367,55 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
     if (it == bs.plans.end()) {
       // row-major out[M, N] = x[M, K] w[K, N] is, in the column-major terms of the library,
       // out^T [N x M] = w^T [N x K] x^T [K x M] with leading dimensions N, x_stride and N
-      GemmPlan np;
+      // (built in a holder that frees whatever exists of the plan on every early return)
+      struct Partial {
+        GemmPlan p{};
+        hipblasLtMatmulPreference_t pref = nullptr;
+        bool keep = false;
+        ~Partial() {
+          if (pref) hipblasLtMatmulPreferenceDestroy(pref);
+          if (keep) return;
+          if (p.la) hipblasLtMatrixLayoutDestroy(p.la);
+          if (p.lb) hipblasLtMatrixLayoutDestroy(p.lb);
+          if (p.lc) hipblasLtMatrixLayoutDestroy(p.lc);
+          if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+        }
+      } part;
+      GemmPlan& np = part.p;
       hipblasStatus_t st = hipblasLtMatmulDescCreate(&np.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F);
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulDescCreate: %s", blas_str(st));
+      // every attribute is checked: a rejected epilogue or bias type would otherwise come back as "no kernel",
+      // or as a product without its epilogue
+      auto set_desc = [&](hipblasLtMatmulDescAttributes_t attr, const void* val, size_t bytes) {
+        return hipblasLtMatmulDescSetAttribute(np.desc, attr, val, bytes);
+      };
       const hipblasOperation_t op_n = HIPBLAS_OP_N;
-      hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_n, sizeof(op_n));
-      hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n));
+      st = set_desc(HIPBLASLT_MATMUL_DESC_TRANSA, &op_n, sizeof(op_n));
+      if (st == HIPBLAS_STATUS_SUCCESS) st = set_desc(HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof(op_n));
       hipblasLtEpilogue_t epi = HIPBLASLT_EPILOGUE_DEFAULT;
       if (a->activation == 1) epi = a->bias ? HIPBLASLT_EPILOGUE_SWISH_BIAS_EXT : HIPBLASLT_EPILOGUE_SWISH_EXT;
       else if (a->bias) epi = HIPBLASLT_EPILOGUE_BIAS;
-      hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi));
-      if (a->bias) {
+      if (st == HIPBLAS_STATUS_SUCCESS) st = set_desc(HIPBLASLT_MATMUL_DESC_EPILOGUE, &epi, sizeof(epi));
+      if (st == HIPBLAS_STATUS_SUCCESS && a->bias) {
         const hipDataType bt = HIP_R_16BF;
-        hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt));
+        st = set_desc(HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bt, sizeof(bt));
+        // the heuristic looks at the pointer's presence; the real one is set on every call below
+        if (st == HIPBLAS_STATUS_SUCCESS) st = set_desc(HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
       }
+      if (st != HIPBLAS_STATUS_SUCCESS)
+        return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulDescSetAttribute (epilogue %d, bias %d): %s", (int)epi, a->bias ? 1 : 0, blas_str(st));
       st = hipblasLtMatrixLayoutCreate(&np.la, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->K, (int64_t)a->N);
       if (st == HIPBLAS_STATUS_SUCCESS) st = hipblasLtMatrixLayoutCreate(&np.lb, HIP_R_16BF, (uint64_t)a->K, (uint64_t)a->M, a->x_stride);
       if (st == HIPBLAS_STATUS_SUCCESS) st = hipblasLtMatrixLayoutCreate(&np.lc, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->M, (int64_t)a->N);
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatrixLayoutCreate: %s", blas_str(st));
-      hipblasLtMatmulPreference_t pref;
-      st = hipblasLtMatmulPreferenceCreate(&pref);
+      st = hipblasLtMatmulPreferenceCreate(&part.pref);
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulPreferenceCreate: %s", blas_str(st));
       const uint64_t ws = a->workspace_bytes;
-      hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
-      if (a->bias) {
-        // the heuristic looks at the pointer's presence; the real one is set on every call below
-        hipblasLtMatmulDescSetAttribute(np.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
-      }
+      st = hipblasLtMatmulPreferenceSetAttribute(part.pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &ws, sizeof(ws));
+      if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulPreferenceSetAttribute: %s", blas_str(st));
       hipblasLtMatmulHeuristicResult_t res[1];
       int found = 0;
-      st = hipblasLtMatmulAlgoGetHeuristic(handle, np.desc, np.la, np.lb, np.lc, np.lc, pref, 1, res, &found);
-      hipblasLtMatmulPreferenceDestroy(pref);
+      st = hipblasLtMatmulAlgoGetHeuristic(handle, np.desc, np.la, np.lb, np.lc, np.lc, part.pref, 1, res, &found);
       if (st != HIPBLAS_STATUS_SUCCESS || found < 1)
         return fail(HSTU_BLOCK_ERR_BLAS, "hipBLASLt has no kernel for M=%lld N=%d K=%d with this epilogue (%s)",
                     (long long)a->M, a->N, a->K, blas_str(st));
@@ -409,11 +431,15 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
         bs.plans.clear();
       }
       it = bs.plans.emplace(key, np).first;
+      part.keep = true;
     }
     plan = it->second;
     // the descriptor is shared by every call of this shape: the bias pointer is set under the lock
     // and the product is enqueued before it is released
-    if (a->bias) hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
+    if (a->bias) {
+      const hipblasStatus_t sb = hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
+      if (sb != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulDescSetAttribute (bias pointer): %s", blas_str(sb));
+    }
     const float alpha = 1.0f, beta = 0.0f;
     const hipblasStatus_t st = hipblasLtMatmul(handle, plan.desc, &alpha, a->w, plan.la, a->x, plan.lb, &beta, a->out, plan.lc,
                                                a->out, plan.lc, &plan.algo, a->workspace, a->workspace_bytes, (hipStream_t)stream);

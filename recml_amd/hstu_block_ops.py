@@ -80,9 +80,12 @@ def gemm_silu(x, w, bias=None, activation: bool = True):
   _check("w", w)
   if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[0]:
     raise ValueError(f"x [M, K] and w [K, N] expected, got {tuple(x.shape)} and {tuple(w.shape)}")
-  if x.stride(1) != 1:
+  # the library wants 16-byte aligned operands and a row stride that keeps rows so
+  if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
     x = x.contiguous()
   w = w.contiguous()
+  if w.data_ptr() % 16:
+    w = w.clone()
   M, K = x.shape
   N = w.shape[1]
   out = torch.empty((M, N), dtype=x.dtype, device=x.device)
@@ -101,6 +104,8 @@ def gemm_silu(x, w, bias=None, activation: bool = True):
     bias = bias.reshape(-1).contiguous()
     if bias.numel() != N:
       raise ValueError(f"bias must have {N} entries")
+    if bias.data_ptr() % 16:
+      bias = bias.clone()
     a.bias = bias.data_ptr()
   a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
   with torch.cuda.device(x.device):

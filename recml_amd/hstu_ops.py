@@ -419,20 +419,16 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   exp = tuple(q.shape[:-1]) + (v.shape[-1],)
   if tuple(dout.shape) != exp or dout.dtype != q.dtype:
     raise ValueError(f"dout must be a {q.dtype} tensor of shape {exp}")
-  out_like = torch.empty_strided(dout.shape, dout.stride(), dtype=dout.dtype, device=dout.device) \
-      if dout.stride(-1) == 1 else torch.empty_like(dout.contiguous())
-  dout = dout if dout.stride() == out_like.stride() else dout.contiguous()
+  dout = dout if dout.stride(-1) == 1 else dout.contiguous()
+  # (the forward struct's `out` is not read by the backward, which takes dout's strides from it: dout stands in)
   fa, keep = build_args(
-      q, k, v, out_like, seq_lens=seq_lens, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
+      q, k, v, dout, seq_lens=seq_lens, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
       causal=causal, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
       q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids, sliding_window_size=sliding_window_size,
       mask=mask, bias=bias)
   # build_args may have made q, k, v contiguous in d: the gradients take the layout it passed on
   qi, ki, vi = _passed_inputs(keep)
-  # the kernels write dq, dk, dv with the strides of q, k, v: mirror them exactly (empty_like would
-  # compact a view with gaps, e.g. one slice of a fused projection)
-  like = lambda t: torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device=t.device)
-  dq, dk, dv = like(qi), like(ki), like(vi)
+  dq, dk, dv = _grad_buffers(qi, ki, vi)
   ba = _lib.HstuAttnBwdArgs()
   ba.struct_size = C.sizeof(_lib.HstuAttnBwdArgs)
   ba.version = _lib.ABI_VERSION
@@ -462,6 +458,23 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   if dts is not None:
     dts = dts.reshape(ts_bias.shape)
   return dq, dk, dv, dpos, dts
+
+
+def _grad_buffers(q, k, v):
+  """dq, dk, dv with exactly the strides of q, k, v (the kernels write them so).  Slices of one fused
+  projection (same storage, interleaved) get slices of ONE buffer laid out like that projection;
+  mirrored one by one, each would span nearly the whole projection."""
+  def extent(t):
+    return sum((n - 1) * st for n, st in zip(t.shape, t.stride())) + 1 if t.numel() else 0
+  ts = (q, k, v)
+  if q.dtype == k.dtype == v.dtype and len({t.untyped_storage().data_ptr() for t in ts}) == 1 and all(t.numel() for t in ts):
+    lo = min(t.storage_offset() for t in ts)
+    hi = max(t.storage_offset() + extent(t) for t in ts)
+    if hi - lo <= 2 * sum(t.numel() for t in ts):
+      buf = torch.empty(hi - lo, dtype=q.dtype, device=q.device)
+      return tuple(buf.as_strided(t.shape, t.stride(), t.storage_offset() - lo) for t in ts)
+  # otherwise mirror each (empty_like would compact a view with gaps)
+  return tuple(torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device=t.device) for t in ts)
 
 
 class _HstuAttentionFn(torch.autograd.Function):

@@ -378,3 +378,26 @@ def test_general_backward_on_random_option_mixes(gpu, seed):
     assert (g is None) == (w is None), (nm, case)
     if g is not None:
       assert _rel(g.cpu().numpy().reshape(w.shape), w) <= 2e-5, (nm, case)
+
+
+def test_gradients_of_fused_projection_slices_share_one_buffer(gpu):
+  """q, k, v cut out of one [T, 4, H, d] projection (as the block does): the gradients come back as
+  slices of one buffer laid out like the projection, not three buffers that each span it, and equal
+  those of separate tensors."""
+  rng = np.random.default_rng(77)
+  T, H, d = 300, 2, 128
+  off = np.array([0, 130, 300], dtype=np.int32)
+  uqkv = torch.from_numpy(O.round_bf16(rng.standard_normal((T, 4, H, d)).astype(np.float32) * 0.4)).to("cuda:0", torch.bfloat16)
+  dout = torch.from_numpy(O.round_bf16(rng.standard_normal((T, H, d)).astype(np.float32) * 0.4)).to("cuda:0", torch.bfloat16)
+  _, q, k, v = uqkv.unbind(dim=1)
+  kw = dict(seq_offsets=torch.from_numpy(off).to("cuda:0"), max_len=170)
+  variant = []
+  dq, dk, dv, _, _ = recml_amd.hstu_attention_bwd(q, k, v, dout, _variant_out=variant, **kw)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  assert dq.stride() == q.stride() and dk.stride() == k.stride() and dv.stride() == v.stride()
+  store = {t.untyped_storage().data_ptr() for t in (dq, dk, dv)}
+  assert len(store) == 1
+  assert dq.untyped_storage().nbytes() <= 1.4 * 3 * q.numel() * 2
+  want = recml_amd.hstu_attention_bwd(q.contiguous(), k.contiguous(), v.contiguous(), dout, **kw)
+  for g, w_ in zip((dq, dk, dv), want[:3]):
+    assert torch.equal(g.contiguous(), w_)

@@ -1050,7 +1050,13 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       // else 8 / H XCDs share the items of one head
       const long long per_xcd = p.H >= 8 ? (long long)total * (p.H >> 3) : (long long)total / (8 / p.H);
       const long long avg = (per_xcd + p.n_slots - 1) / p.n_slots;
-      split_steps = avg < 8 ? 8 : (avg > 0x3fffffff ? 0x3fffffff : (int)avg);
+      // A tile is split when it alone is more than twice that average: its chunks cost a round trip of
+      // fp32 partial sums through memory, so tiles near the average are left whole.  (Measured, kernel
+      // time with the threshold at 1x / 1.5x / 2x the average / never: one sequence of 2048 tokens
+      // 40 / 37 / 34 / 55 us; two 65 / 60 / 46 / 56; two long among 60 short 62 / 46 / 48 / 57; the
+      // headline shape of 64 jagged sequences 72 / 68 / 69 / 69.)
+      const long long thr = 2 * avg;
+      split_steps = thr < 8 ? 8 : (thr > 0x3fffffff ? 0x3fffffff : (int)thr);
     }
     int item_base = 0, slot_base = 0;
     for (int sg = 0; sg < nseg; ++sg) {

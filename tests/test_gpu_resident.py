@@ -117,3 +117,36 @@ def test_headline_shape(gpu):
   one, res = _both(t(w.q).to(bf), t(w.k).to(bf), t(w.v).to(bf), seq_offsets=t(w.seq_offsets), max_len=w.L,
                    n=w.n, alpha=w.alpha, pos_bias=t(w.pos_tab), ts_bias=t(w.ts_tab), timestamps=t(w.timestamps))
   assert np.array_equal(one, res)
+
+
+@pytest.mark.parametrize("d", [128, 64])
+def test_more_sequences_than_one_list_segment(gpu, d):
+  """2600 sequences: the list builder takes them 1024 at a time, in batch order (no sorting), with the
+  item and chunk-slot counts carried from one segment to the next; one long sequence in the third segment
+  has tiles that are split."""
+  rng = np.random.default_rng(1600 + d)
+  H, L, B = 8, 1024, 2600
+  lens = rng.integers(0, 150, B).astype(np.int32)
+  lens[2100] = 1024
+  lens[7] = 700
+  off = np.zeros(B + 1, dtype=np.int32)
+  off[1:] = np.cumsum(lens)
+  T = int(off[-1])
+  q, k, v = (O.round_bf16(rng.standard_normal((T, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.2).astype(np.float32)
+  if d == 128:
+    one, res = _both(_dev(q, bf), _dev(k, bf), _dev(v, bf), seq_offsets=_dev(off), max_len=L, pos_bias=_dev(pos))
+    assert np.array_equal(one, res)
+  else:
+    import recml_amd
+    res = recml_amd.hstu_attention(_dev(q, bf), _dev(k, bf), _dev(v, bf), seq_offsets=_dev(off), max_len=L,
+                                   pos_bias=_dev(pos)).float().cpu().numpy()
+  for b in [0, 7, 1023, 1024, 1025, 2047, 2048, 2100, 2599] + list(rng.integers(0, B, 12)):
+    sl = slice(int(off[b]), int(off[b + 1]))
+    if lens[b] == 0:
+      continue
+    o1 = np.array([0, lens[b]], dtype=np.int32)
+    ref = O.hstu_attention_jagged_ref(q[sl], k[sl], v[sl], o1, L, pos_tab=pos)
+    assert _rel(res[sl], ref) <= BF16_TOL, b
+  # every row was written by someone: nothing is left of the fill
+  assert np.isfinite(res).all()

@@ -157,7 +157,7 @@ def test_block_config4_shape_bf16(gpu):
 
 @pytest.mark.gpu
 def test_model_config4_full_size_bf16(gpu):
-  """BASELINE configuration 4 as a whole: 10 M x 512 bf16 embedding table (10.24 GB), Zipf(1.05) item ids,
+  """Benchmark configuration 4 as a whole: 10 M x 512 bf16 embedding table (10.24 GB), Zipf(1.05) item ids,
   4 blocks, D = 512, H = 8 (head dim 64), B = 128, L = 1024, lengths U{128..1024}, position bias; padded and
   packed forward (recml/layers/keras/hstu.py:585-621), checked against the fp64 oracle on the longest, the
   shortest and a median sequence, which also carry ids at the very end of the table (rows past 2^31 bytes /

@@ -15,12 +15,16 @@
 //                        fp32 bias streamed through the same ring.  Computes
 //                        S^T = K Q^T so that the
 //                        accumulator layout of S^T is already the B-operand
-//                        layout of O^T = V^T P^T: P never touches LDS.
-//   hstu_prepare         runs before it: work list of (sequence, tile) items,
-//                        longest sequences first; scaled bias tables; int32
-//                        timestamps and their per-tile ranges.
-//   hstu_combine         runs after it when query tiles were split over
-//                        several workgroups by key range: sums the partials.
+//                        layout of O^T = V^T P^T: P never touches LDS.  Its
+//                        work list is taken one workgroup per item or by
+//                        resident workgroups that draw item after item; query
+//                        tiles that alone would outlast the rest are split by
+//                        key range between workgroups, and the one that
+//                        arrives last at the tile's counter sums the parts.
+//   hstu_prepare         runs before it, once per batch: work list of
+//                        (sequence, tile, key chunk) items, longest sequences
+//                        first; scaled bias tables; the timestamp bucket
+//                        tables; int32 timestamps and their per-tile ranges.
 //   hstu_fwd_general     every option of the op (segment ids, explicit mask,
 //                        sliding window, dense bias, cross lengths, any head
 //                        dim <= 256, fp32 or bf16 storage) in plain fp32 FMA
@@ -44,7 +48,6 @@
 // hstu.py:33-55, 190-221 (timestamp buckets).
 
 #include <hip/hip_runtime.h>
-#include <type_traits>
 #include <math.h>
 #include <stdarg.h>
 #include <stdint.h>
@@ -101,7 +104,7 @@ struct Params {
   float alpha, inv_n;
   int32_t n_qtiles;
   // Key-range splitting (MFMA forward; off when split_cap == 0): hstu_prepare, which sees the lengths,
-  // shares a query tile with more steps than a slot's average load between up to MAX_CHUNKS workgroups,
+  // shares a query tile with more steps than twice a slot's average load between up to MAX_CHUNKS workgroups,
   // each covering a contiguous part of the keys and leaving its fp32 partial O^T in `partial`; the
   // workgroup that arrives last at the tile's counter sums them and writes the rows.
   int32_t split_cap;         // chunk slots of the partial buffer (per head)
@@ -782,7 +785,7 @@ __device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0)
   return (kv_end + BN - 1) / BN;
 }
 
-// Which (sequence, head, query tile, chunk) a workgroup of the main (or combine) kernel has.
+// Which (sequence, head, query tile, chunk) a workgroup of the main kernels has.
 // Workgroups are dealt round-robin to the 8 XCDs (blockIdx % 8), each with its own L2: every
 // tile of one (sequence, head) goes to the same XCD, and tiles of a sequence are adjacent in
 // launch order, the one with most keys first, so that the tiles running together stream the

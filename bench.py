@@ -524,6 +524,8 @@ def main():
                   help="diagnostics: force one workgroup per work-list entry")
   ap.add_argument("--resident-workgroups", action="store_true",
                   help="diagnostics: force resident workgroups that loop over the work list")
+  ap.add_argument("--ramp-ms", type=float, default=300.0,
+                  help="untimed calls for this long before anything is measured (clock ramp from idle)")
   ap.add_argument("--calib-copy", action="store_true",
                   help="also run one 512 MiB device copy (reference point for HBM byte counters)")
   args = ap.parse_args()
@@ -583,6 +585,14 @@ def main():
       ends[i].record()
     torch.cuda.synchronize()
     return np.array([s.elapsed_time(e) for s, e in zip(starts, ends)])
+
+  # The GPU's clocks take tens of milliseconds of work to come up from idle: untimed calls for a fixed
+  # time first, so that a run with few steps measures the same machine state as one with many.
+  t_ramp = time.perf_counter()
+  while (time.perf_counter() - t_ramp) * 1e3 < args.ramp_ms:
+    for _ in range(50):
+      step()
+    torch.cuda.synchronize()
 
   # Calls that carry their own preparation (work list, 32-bit timestamps, scaled tables: one more kernel).
   for _ in range(args.warmup):

@@ -3144,6 +3144,9 @@ int validate(const HstuAttnFwdArgs* a) {
   if (a->struct_size != sizeof(HstuAttnFwdArgs) || a->version != HSTU_ATTN_ABI_VERSION)
     return fail(HSTU_ERR_VERSION, "args struct_size/version (%u/%u) do not match this library (%zu/%d)",
                 a->struct_size, a->version, sizeof(HstuAttnFwdArgs), HSTU_ATTN_ABI_VERSION);
+  constexpr uint32_t known_flags = HSTU_FWD_WORKSPACE_PREPARED | HSTU_FWD_PREPARE_ONLY | HSTU_FWD_ONE_ITEM_PER_WORKGROUP |
+                                   HSTU_FWD_RESIDENT_WORKGROUPS;
+  if ((uint32_t)a->flags & ~known_flags) return fail(HSTU_ERR_SHAPE, "unknown bits in flags: 0x%x", (unsigned)a->flags);
   const bool empty = a->B == 0 || (a->layout == HSTU_LAYOUT_JAGGED && a->total_tokens == 0);
   if (!empty && (!a->q || !a->k || !a->v || !a->out))
     return fail(HSTU_ERR_NULL, "q, k, v and out must be non-null");

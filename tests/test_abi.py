@@ -116,6 +116,10 @@ def test_validation_errors_without_gpu():
   a.d_qk = 512
   assert lib.hstu_attn_fwd(C.byref(a), None) == -4           # HSTU_ERR_SHAPE
   a.d_qk = 32
+  a.flags = 64                                               # a bit no flag has
+  assert lib.hstu_attn_fwd(C.byref(a), None) == -4
+  assert b"flags" in lib.hstu_attn_last_error()
+  a.flags = 0
   a.qk_dtype, a.v_dtype, a.out_dtype = 0, 1, 1
   assert lib.hstu_attn_fwd(C.byref(a), None) == -3           # HSTU_ERR_DTYPE
   a.qk_dtype = a.v_dtype = a.out_dtype = 1

@@ -20,6 +20,7 @@ import torch
 
 import recml_amd
 from recml_amd import workloads
+from oracle import hstu_oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -172,3 +173,38 @@ def test_backward_identities_at_full_size(c3):
     assert torch.equal(_bits((2 * a.float()).to(torch.bfloat16)), _bits(b))
   for a, b in ((dpos, dpos2), (dts, dts2)):
     assert (2 * a - b).abs().max().item() <= 1e-3 * b.abs().max().item()
+
+
+def test_backward_at_full_size_against_the_oracle(c3):
+  """The matrix-core backward on the whole of configuration 3, sequence by sequence against the numpy
+  oracle: every sequence of up to 320 tokens in fp64 and the longest one (1655 tokens) in fp32.  A
+  sequence alone with its slice of the position table is the same problem as the sequence in the batch."""
+  w = c3.w
+  g = torch.Generator(device="cuda:0").manual_seed(3)
+  dout = (torch.randn(c3.v.shape, device="cuda:0", generator=g) * 0.1).to(torch.bfloat16)
+  kw = c3.kwargs()
+  kw.pop("n")
+  variant = []
+  dq, dk, dv, _, _ = recml_amd.hstu_attention_bwd(c3.q, c3.k, c3.v, dout, n=w.n, table_grads=False, _variant_out=variant, **kw)
+  torch.cuda.synchronize()
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  got = [t.float().cpu().numpy() for t in (dq, dk, dv)]
+  host = [t.float().cpu().numpy() for t in (c3.q, c3.k, c3.v, dout)]
+  L = w.L
+  lens = np.asarray(w.seq_lens)
+  longest = int(np.argmax(lens))
+  checked = 0
+  for b in range(w.B):
+    n = int(lens[b])
+    if n == 0 or (n > 320 and b != longest):
+      continue
+    sl = slice(int(w.seq_offsets[b]), int(w.seq_offsets[b]) + n)
+    qb, kb, vb, db = (x[sl][None] for x in host)
+    pos = w.pos_tab[:, (L - 1) - (n - 1): (L - 1) + n]          # entries (L-1) + j - i for |j - i| < n
+    want = O.hstu_attention_bwd_ref(qb, kb, vb, db, n=w.n, alpha=w.alpha, pos_tab=pos, ts_tab=w.ts_tab,
+                                    timestamps=w.timestamps[sl][None], dtype=np.float64 if n <= 320 else np.float32)
+    for name, gt, wt in zip(("dq", "dk", "dv"), got, want[:3]):
+      err = np.abs(gt[sl] - wt[0]).max() / max(np.abs(wt).max(), 1e-30)
+      assert err <= 2e-2, (b, n, name, err)
+    checked += 1
+  assert checked >= 40

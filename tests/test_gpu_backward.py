@@ -401,3 +401,18 @@ def test_gradients_of_fused_projection_slices_share_one_buffer(gpu):
   want = recml_amd.hstu_attention_bwd(q.contiguous(), k.contiguous(), v.contiguous(), dout, **kw)
   for g, w_ in zip((dq, dk, dv), want[:3]):
     assert torch.equal(g.contiguous(), w_)
+
+
+def test_backward_work_list_over_two_segments_of_sequences(gpu):
+  """1500 sequences: the work list (built without key-range splits for the backward) takes them 1024 at a time."""
+  rng = np.random.default_rng(34)
+  B, L, H, d = 1500, 40, 8, 32
+  bf = torch.bfloat16
+  lens = rng.integers(0, L + 1, B).astype(np.int32)
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, seq_lens=lens)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), seq_lens=_dev(lens), _variant_out=variant)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(g.float().cpu().numpy(), w) <= 2e-2, nm

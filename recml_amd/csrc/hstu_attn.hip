@@ -651,8 +651,9 @@ constexpr int TS_TAB_LEN = 128;  // most timestamp buckets the matrix-core kerne
 // One head's table (TS_LDS_BYTES, copied to LDS by every workgroup):
 //   [(TS_KEYS + 2) x {float log2(e) * value, float threshold}]  by key (the per-pair path)
 //   [TS_KEYS x float: log2(e) * value of bucket b]  by bucket (the backward's table-gradient path)
-//   [TS_KEYS x int: smallest clipped |dt| that reaches the key's threshold]  [TS_KEYS x byte: bucket the
-//   key's range starts in]  by key (the per-tile shortcuts, table gradients)
+//   [TS_KEYS x int: smallest clipped |dt| of bucket b, INT32_MAX for buckets nothing reaches]  by bucket (the
+//   per-tile shortcuts)
+//   [TS_KEYS x byte: bucket the key's range starts in]  by key (the per-tile shortcuts, table gradients)
 constexpr int TS_KEYS = 128;               // keys, and the most buckets the matrix-core kernels index
 constexpr int TS_KEY0 = 127 << 2;          // key of f = 1.0 before the offset is taken off
 constexpr int TS_DT_MAX = 1000000000;
@@ -661,7 +662,7 @@ constexpr int TS_LDS_BYTES = TS_BKT_OFF + TS_KEYS;
 static_assert(TS_LDS_BYTES % 16 == 0 && TS_LDS_BYTES <= 3 * 1024, "table layout: at most three direct loads");
 struct TsKeys {                            // host-built part of the table, a kernel argument of hstu_prepare
   float thr_f[TS_KEYS];                    // by key: first float of the bucket behind the one the key's range starts in
-  int32_t thr_i[TS_KEYS];                  // by key: smallest clipped |dt| that reaches thr_f
+  int32_t thr_b[TS_KEYS];                  // by bucket: smallest clipped |dt| in bucket b or a later one
   uint8_t bkt[TS_KEYS];                    // by key: bucket the key's range starts in
 };
 
@@ -862,26 +863,26 @@ __device__ __forceinline__ int ts_bucket_of(const unsigned char* tab, int d) {
   const uint32_t key = (__builtin_bit_cast(uint32_t, f) >> 21) - (uint32_t)TS_KEY0;
   return (int)tab[TS_BKT_OFF + key] + (f >= *(const float*)(tab + (key << 3) + 4) ? 1 : 0);
 }
-// Both ends of a range of time differences [d_near, d_far]: their buckets and table values; `same` when
-// both are in one bucket and d_near >= 0 (then so is every difference between them); `two` when at most
-// one bucket boundary lies inside the range and one of the two entries holds it: differences >= thr are
-// then in the far end's bucket, the others in the near end's.
+// A range of time differences [d_near, d_far], d_near <= d_far: the near end's bucket b and its table value
+// by one lookup, then the integer thresholds of the next two buckets tell where the far end lies: `same`
+// when it is still in b and d_near >= 0 (then so is every difference between them); `two` when it is in
+// b or b + 1: differences >= thr are then in b + 1 (value v_far), the others in b.
 struct TsEnds { int b_near, b_far, thr; float v_near, v_far; bool same, two; };
 __device__ __forceinline__ TsEnds ts_ends(const unsigned char* tab, int d_near, int d_far) {
-  const TsLook n = ts_look(tab, d_near), f = ts_look(tab, d_far);
+  const TsLook n = ts_look(tab, d_near);
   TsEnds r;
   r.b_near = ts_bucket(tab, n);
-  r.b_far = ts_bucket(tab, f);
   r.v_near = ts_value(n);
-  r.v_far = ts_value(f);
+  const int* next = (const int*)(tab + TS_INT_OFF) + r.b_near;
+  const int t1 = next[1], t2 = next[2];          // first differences of buckets b + 1 and b + 2
+  int far = d_far < 0 ? -d_far : d_far;
+  far = far < 1 ? 1 : (far > TS_DT_MAX ? TS_DT_MAX : far);
   const bool sorted = d_near >= 0;
-  r.same = sorted && r.b_near == r.b_far;
-  // the boundary is the near entry's when the near end lies below that, else the far entry's when the far
-  // end has passed it (a boundary that sits in a key's range between the two is in neither entry)
-  const bool n_up = n.f >= n.thr;
-  const bool held = n_up ? f.f >= f.thr : true;
-  r.thr = *(const int*)(tab + TS_INT_OFF + ((n_up ? f.key : n.key) << 2));
-  r.two = sorted && (r.b_near == r.b_far || (r.b_far == r.b_near + 1 && held));
+  r.same = sorted && far < t1;
+  r.two = sorted && far < t2;
+  r.b_far = far < t1 ? r.b_near : r.b_near + 1;
+  r.thr = t1;
+  r.v_far = *(const float*)(tab + TS_VAL_OFF + ((r.b_near + 1) << 2));
   return r;
 }
 __device__ __forceinline__ float ts_bucket_value(const unsigned char* tab, int b) { return *(const float*)(tab + TS_VAL_OFF + (b << 2)); }
@@ -1117,7 +1118,7 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       ((float2*)out)[e] = float2{tab[bk < p.ts_nb ? bk : p.ts_nb] * LOG2E, keys.thr_f[ek]};
       if (e < TS_KEYS) {
         ((float*)(out + TS_VAL_OFF))[e] = tab[e < p.ts_nb ? e : p.ts_nb] * LOG2E;
-        ((int*)(out + TS_INT_OFF))[e] = keys.thr_i[e];
+        ((int*)(out + TS_INT_OFF))[e] = e <= p.ts_nb ? keys.thr_b[e] : 0x7fffffff;    // buckets are clipped to ts_nb
         out[TS_BKT_OFF + e] = (unsigned char)bk;
       }
     }
@@ -3069,7 +3070,8 @@ const BucketLaw& bucket_law(float size_f) {
     }
     law.thr[b] = (int32_t)lo;
   }
-  law.keyed_ok = law.reach + 1 < TS_KEYS && law.reach + 2 < LAW_THR_LEN;
+  law.keyed_ok = law.reach + 2 < TS_KEYS && law.reach + 2 < LAW_THR_LEN;     // the kernels read thresholds up to bucket reach + 2
+  for (int b = 0; b < TS_KEYS; ++b) law.keys.thr_b[b] = b < LAW_THR_LEN ? law.thr[b] : 0x7fffffff;
   for (int key = 0; key < TS_KEYS && law.keyed_ok; ++key) {
     // floats of this key: [f_lo, f_next); the time differences behind them are integers
     uint32_t bits_lo = (uint32_t)(TS_KEY0 + key) << 21, bits_next = (uint32_t)(TS_KEY0 + key + 1) << 21;
@@ -3083,7 +3085,6 @@ const BucketLaw& bucket_law(float size_f) {
     const int b_lo = law_bucket(f_first, size);
     law.keys.bkt[key] = (uint8_t)b_lo;
     law.keys.thr_f[key] = (float)law.thr[b_lo + 1];      // INT32_MAX becomes 2^31: beyond every clipped difference
-    law.keys.thr_i[key] = law.thr[b_lo + 1];
     if (f_first < f_next) {
       // at most one boundary inside the key's range; and when there is one, the next key must start in
       // the bucket behind it (the kernels take the value from the threshold on from the next key's entry)

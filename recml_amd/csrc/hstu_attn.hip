@@ -109,6 +109,7 @@ struct Params {
   // workgroup that arrives last at the tile's counter sums them and writes the rows.
   int32_t split_cap;         // chunk slots of the partial buffer (per head)
   int32_t n_slots;           // workgroups that run at once per XCD (what the split decision balances for)
+  const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
   uint32_t* ctr;             // workspace: [0, 8) draw counters of the XCDs, [8] workgroups done, then from
@@ -695,8 +696,9 @@ struct MfmaSmem {
   static constexpr int DB_BYTES = BM * BN * 4;
   static constexpr int DM_BYTES = BM * BN;
   static constexpr int dense_stage(int dense) { return ((dense & 1) ? DB_BYTES : 0) + ((dense & 2) ? DM_BYTES : 0); }
+  // (the dense operands have one stage: each wave owns the rows of its 32 queries and refills them itself)
   static constexpr int total(bool pos, bool ts, bool seg = false, int dense = 0, int nst = NSTAGE) {
-    return nst * (STAGE + bias_stage(pos, ts, seg) + dense_stage(dense)) + (ts ? TAB_BYTES : 0);
+    return nst * (STAGE + bias_stage(pos, ts, seg)) + dense_stage(dense) + (ts ? TAB_BYTES : 0);
   }
   // K is read one row per lane, 16 bytes at a time: 16 consecutive rows must hit 16 different chunks
   __device__ static constexpr int swz_k(int row) { return (row / KRPB) % KCPR; }
@@ -903,11 +905,12 @@ __device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_
 //  * the timestamp bucket tables (TsKeys above), [heads][TS_LDS_BYTES];
 //  * per sequence whose timestamps span less than 2^31: the timestamps minus their minimum
 //    as int32 (differences of two of them are then exact in 32 bits), and the (min, max)
-//    of those in each 32-key tile.  One workgroup per sequence.
+//    of those in each 32-key tile.  One workgroup per sequence;
+//  * with a dense keep-mask: per query tile the range of 32-key steps that hold a kept pair.
 __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __restrict__ pos_out, int4* __restrict__ tab_out,
                                                     int32_t* __restrict__ ok_out, int32_t* __restrict__ rel_out,
                                                     int32_t* __restrict__ range_out, int32_t* __restrict__ sched_out,
-                                                    const TsKeys keys) {
+                                                    int32_t* __restrict__ mrange_out, const TsKeys keys) {
   const int tid = threadIdx.x;
   const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
   if (sched_out && blockIdx.x == gridDim.x - 1) {
@@ -1132,6 +1135,58 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       pos_out[i] = (j >= 0 && j < len) ? p.pos_tab[(int64_t)hd * len + j] * LOG2E : 0.f;
     }
   }
+  if (mrange_out) {
+    // The dense keep-mask, per query tile of 128 rows: the range of 32-key steps outside of which no pair
+    // of the tile is kept (a causal or length mask handed over as a matrix keeps a prefix of the keys: the
+    // main kernel then leaves the other steps out altogether, loads included).  One workgroup per tile, 16
+    // bytes per lane and load, eight loads in flight; rows are whole 16-byte pieces (Lkv is a multiple of 16).
+    __shared__ int mr_lo[4], mr_hi[4];
+    const int nb = p.mask_batched ? p.B : 1;
+    const int ppr = p.Lkv / 16;
+    for (int tile = blockIdx.x; tile < nb * p.n_qtiles; tile += gridDim.x) {
+      const int b = tile / p.n_qtiles, qt = tile - b * p.n_qtiles;
+      const int r0 = qt * BM;
+      const int rows = p.L - r0 < BM ? p.L - r0 : BM;
+      const uint4* mg = (const uint4*)(p.mask + ((int64_t)b * p.L + r0) * p.Lkv);
+      const int n = rows * ppr;
+      int lo = 0x7fffffff, hi = 0;
+      for (int i0 = 0; i0 < n; i0 += 8 * 256) {
+        uint4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          const int i = i0 + 256 * k + tid;
+          v[k] = i < n ? mg[i] : uint4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          if ((v[k].x | v[k].y | v[k].z | v[k].w) != 0u) {
+            const int i = i0 + 256 * k + tid;
+            const int step = (i % ppr) >> 1;
+            lo = step < lo ? step : lo;
+            hi = step + 1 > hi ? step + 1 : hi;
+          }
+        }
+      }
+#pragma unroll
+      for (int d = 32; d >= 1; d >>= 1) {
+        const int a = __shfl_xor(lo, d, 64), c = __shfl_xor(hi, d, 64);
+        lo = a < lo ? a : lo;
+        hi = c > hi ? c : hi;
+      }
+      __syncthreads();            // the readers of the tile before are done
+      if ((tid & 63) == 0) { mr_lo[tid >> 6] = lo; mr_hi[tid >> 6] = hi; }
+      __syncthreads();
+      if (tid == 0) {
+#pragma unroll
+        for (int i = 1; i < 4; ++i) {
+          lo = mr_lo[i] < lo ? mr_lo[i] : lo;
+          hi = mr_hi[i] > hi ? mr_hi[i] : hi;
+        }
+        mrange_out[2 * tile] = hi > 0 ? lo : 0;
+        mrange_out[2 * tile + 1] = hi;
+      }
+    }
+  }
   if (!ok_out) return;
   static_assert(BN == 32, "one lane per key of a tile");
   __shared__ int64_t red_lo[4], red_hi[4];
@@ -1210,15 +1265,18 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 //
 // DENSE (bit 0: additive bias, bit 1: keep-mask; the layer-side call of
 // recml/layers/keras/hstu.py:356-390): the step's 128 x 32 tile of the [L, Lkv] fp32 bias and / or
-// of the byte mask comes through the ring like K and V (four more direct loads per wave for the
-// bias, one for the mask).  16 KB + 4 KB a stage: one workgroup per CU.  A block whose mask tile is
-// all zero is skipped.
+// of the byte mask comes by direct loads like K and V (four per wave for the bias, one for the mask),
+// but into a single 16 KB + 4 KB buffer instead of a ring: a wave reads only the 32 rows of its own
+// queries, and the loads that bring those rows are its own, so each wave takes its part of step t into
+// registers at the start of the step and at once asks for step t + 1 into the same bytes -- no other
+// wave is involved, and the loads have the whole block and the barrier to land.  With a three-stage K / V
+// ring that is 68 KB at d = 128: two workgroups per CU.  A block whose mask tile is all zero is skipped.
 // Ring depth of the forward kernel.  Up to d = 64 a wave needs at most 128 registers, so four
 // workgroups fit a CU once their LDS does: three stages (two steps in flight behind the one being
 // computed) instead of four take the d = 64 kernel with a position table from 43 KB to 32 KB, three
 // workgroups per CU to four (measured: 148 -> 139 us on the d = 64 benchmark shape).  At d = 128
 // registers allow two workgroups whatever the ring, and the depth makes no measurable difference.
-constexpr int fwd_stages(int d, int dense) { return (d <= 64 && dense == 0) ? 3 : 4; }
+constexpr int fwd_stages(int d, int dense) { return (d <= 64 || dense != 0) ? 3 : 4; }
 constexpr int FWD_XCH_BYTES = 16;     // behind everything else in the forward kernel's LDS
 
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0, bool PERSIST = false>
@@ -1238,13 +1296,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   constexpr int NSTAGE = fwd_stages(D, DENSE);   // the ring depth of this kernel (shadows the backward kernels' constant)
   static_assert(BM * BN * 4 / 1024 == 4 * NWAVES && BM * BN / 1024 == NWAVES, "dense tiles: 4 + 1 pieces per wave");
   // direct loads per wave per step
-  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + ((DENSE & 1) ? 4 : 0) + ((DENSE & 2) ? 1 : 0);
-  static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
+  constexpr int NDMA = LDK + LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);
+  constexpr int NDENSE = ((DENSE & 1) ? 4 : 0) + ((DENSE & 2) ? 1 : 0);     // the dense operands' loads, counted apart
+  static_assert((NSTAGE - 1) * NDMA + NDENSE <= 63, "vmcnt range");
+  static_assert(DENSE == 0 || (!POS && !TS && !SEG && !F8), "dense operands come without table biases, segment ids and fp8");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
   // LDS map: [ring: NSTAGE x (K | V)][bias operands x NSTAGE: 4 pos windows | key timestamps][ts table]
-  // [dense operands x NSTAGE: bias tile | mask tile].
+  // [dense operands: bias tile | mask tile].
   // The key timestamps sit right behind the last position window so that one direct load of the
   // last wave can fill both.
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
@@ -1257,9 +1317,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   constexpr int DENSE_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
   constexpr int DENSE_STAGE = SM::dense_stage(DENSE);
-  constexpr int XCH_OFF = DENSE_OFF + NSTAGE * DENSE_STAGE;   // 16 bytes for values one lane hands to the workgroup
-  auto Db = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE; };
-  auto Dm = [&](int st) { return smem + DENSE_OFF + st * DENSE_STAGE + ((DENSE & 1) ? SM::DB_BYTES : 0); };
+  constexpr int XCH_OFF = DENSE_OFF + DENSE_STAGE;   // 16 bytes for values one lane hands to the workgroup
+  auto Db = [&]() { return smem + DENSE_OFF; };
+  auto Dm = [&]() { return smem + DENSE_OFF + ((DENSE & 1) ? SM::DB_BYTES : 0); };
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -1322,6 +1382,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       nt_ = t_lo_ + per < nt_ ? t_lo_ + per : nt_;
     }
     if (win >= 0 && q0_ - win > 0 && nt_ > 0) t_lo_ = (q0_ - win) / BN;
+    if constexpr ((DENSE & 2) != 0) {
+      // the steps in which the keep-mask keeps a pair of this tile at all (found by the preparation kernel)
+      const int2 mr = ((const int2*)pf.mask_range)[(pf.mask_batched ? k.b : 0) * pf.n_qtiles + k.qt];
+      t_lo_ = t_lo_ > mr.x ? t_lo_ : mr.x;
+      nt_ = nt_ < mr.y ? nt_ : mr.y;
+      nt_ = nt_ > t_lo_ ? nt_ : t_lo_;
+    }
   };
 
   // Direct loads of step t into ring stage t % NSTAGE.  Wave w fills 1 KB
@@ -1391,12 +1458,16 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         lds_dma16_at(p.kv_seg + (int64_t)c_.b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
       }
     }
+  };
+  // The dense operands of step t, each wave its own rows (the same number of loads whatever the step).
+  auto dense_refill = [&](const DmaCtx& c_, int t) {
+    const int kv0 = t * BN;
     if (DENSE & 1) {
       // Bias tile: row r of the tile at LDS byte 128 r, its 16-byte chunks XOR-swizzled by r & 7
-      // (the block reads one chunk per lane from 16 consecutive rows).  Wave w brings 1 KB pieces
-      // 4w .. 4w+3 (8 rows each); lane l of a piece lands at row l / 8, physical chunk l % 8.  Rows
-      // past L and keys past Lkv re-read the last row / the last four keys: finite data for
-      // logits that are masked by their index.
+      // (the wave reads one chunk per lane from 16 consecutive rows).  Wave w brings 1 KB pieces
+      // 4w .. 4w+3 (8 rows each, the rows of its own queries); lane l of a piece lands at row l / 8,
+      // physical chunk l % 8.  Rows past L and keys past Lkv re-read the last row / the last four keys:
+      // finite data for logits that are masked by their index.
       const float* dbg = p.dense_bias + (p.dense_bias_batched ? (int64_t)c_.b * p.L * p.Lkv : 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -1406,7 +1477,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         gr = gr < p.L - 1 ? gr : p.L - 1;
         int col = kv0 + 4 * (pc ^ (row & 7));
         col = col < p.Lkv - 4 ? col : p.Lkv - 4;
-        lds_dma16(dbg, ((uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col) * 4u, Db(st) + j * 1024);
+        lds_dma16(dbg, ((uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col) * 4u, Db() + j * 1024);
       }
     }
     if (DENSE & 2) {
@@ -1417,7 +1488,28 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       gr = gr < p.L - 1 ? gr : p.L - 1;
       int col = kv0 + 16 * (lane & 1);
       col = col < p.Lkv - 16 ? col : p.Lkv - 16;
-      lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Dm(st) + w * 1024);
+      lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Dm() + w * 1024);
+    }
+  };
+  // The lane's share of the dense operands that have landed: 16 bias values (keys 8g + 4hh .. +3 of its
+  // row) and their 16 mask bytes.  The empty statement at the end makes the compiler wait for the values
+  // here: once it is passed, the buffer may be refilled.
+  float4 dbv[4];
+  uint32_t mbits[4] = {0u, 0u, 0u, 0u};
+  auto dense_take = [&]() {
+    if (DENSE & 2) {
+      const unsigned char* mrow = Dm() + (32 * w + m) * 32 + 4 * hh;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) mbits[g] = *(const uint32_t*)(mrow + 8 * g);
+      asm volatile("" : "+v"(mbits[0]), "+v"(mbits[1]), "+v"(mbits[2]), "+v"(mbits[3]));
+    }
+    if (DENSE & 1) {
+      const int row = 32 * w + m;
+      const unsigned char* brow = Db() + row * 128;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) dbv[g] = *(const float4*)(brow + (((2 * g + hh) ^ (row & 7)) * 16));
+#pragma unroll
+      for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(dbv[g].x), "+v"(dbv[g].y), "+v"(dbv[g].z), "+v"(dbv[g].w));
     }
   };
 
@@ -1516,12 +1608,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto block = [&](int t, auto st_) {
     constexpr int st = decltype(st_)::value;
     const int kbs = t * BN;
-    uint32_t mbits[4] = {0u, 0u, 0u, 0u};
     if (DENSE & 2) {
-      // the lane's 16 mask bytes: keys 8g + 4hh .. +3 of its row; nothing to do when the wave's whole tile is 0
-      const unsigned char* mrow = Dm(st) + (32 * w + m) * 32 + 4 * hh;
-#pragma unroll
-      for (int g = 0; g < 4; ++g) mbits[g] = *(const uint32_t*)(mrow + 8 * g);
+      // nothing to do when the wave's whole mask tile is 0
       if (__builtin_amdgcn_ballot_w64((mbits[0] | mbits[1] | mbits[2] | mbits[3]) != 0u) == 0) return;
     }
     floatx16 sacc;
@@ -1627,11 +1715,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
     }
     if (DENSE & 1) {
-      const int row = 32 * w + m;
-      const unsigned char* brow = Db(st) + row * 128;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const float4 bv = *(const float4*)(brow + (((2 * g + hh) ^ (row & 7)) * 16));
+        const float4 bv = dbv[g];
         u[4 * g + 0] = __builtin_fmaf(bv.x, LOG2E, u[4 * g + 0]);
         u[4 * g + 1] = __builtin_fmaf(bv.y, LOG2E, u[4 * g + 1]);
         u[4 * g + 2] = __builtin_fmaf(bv.z, LOG2E, u[4 * g + 2]);
@@ -1854,6 +1940,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     // all of the prologue it held up the first block until everything had landed.
     if (TS) load_ts_table(h);
     if (t_lo < nt) dma_step(cx, t_lo, std::integral_constant<int, 0>{});
+    if (DENSE != 0 && t_lo < nt) dense_refill(cx, t_lo);
     load_q(first);
     settle_q();
     if (t_lo + 1 < nt) dma_step(cx, t_lo + 1, std::integral_constant<int, 1>{});
@@ -1885,6 +1972,32 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         pair(t, std::integral_constant<int, 0>{});
         if (t + 2 >= nt) break;
         pair(t + 2, std::integral_constant<int, 2>{});
+      }
+    } else if constexpr (DENSE != 0) {
+      // Step t with dense operands: the wave takes its rows of the step's bias and mask tiles into registers,
+      // asks for the next step's into the same bytes, then for the K / V tiles of step t + 2 (into the ring
+      // stage that the barrier before freed), and computes its block.  Before the barrier, everything of
+      // step t + 1 has landed: the loads are counted in the order of their issue, so only the K / V tiles of
+      // step t + 2, the youngest, stay in flight.
+      static_assert(NSTAGE == 3, "two steps of K / V tiles in flight");
+      if (t_lo + 1 < nt) HSTU_WAIT_VMCNT(NDMA); else HSTU_WAIT_VMCNT(0);      // all of step t_lo
+      __syncthreads();
+      auto step = [&](int t, auto st_) {
+        constexpr int st = decltype(st_)::value;
+        const bool lv = live(t);
+        if (lv) dense_take();
+        if (t + 1 < nt) dense_refill(cx, t + 1);
+        if (t + 2 < nt) dma_step(cx, t + 2, std::integral_constant<int, (st + 2) % NSTAGE>{});
+        if (lv) block(t, st_);
+        if (t + 2 < nt) HSTU_WAIT_VMCNT(NDMA); else HSTU_WAIT_VMCNT(0);
+        __syncthreads();
+      };
+      for (int t = t_lo; t < nt; t += NSTAGE) {
+        step(t, std::integral_constant<int, 0>{});
+        if (t + 1 >= nt) break;
+        step(t + 1, std::integral_constant<int, 1>{});
+        if (t + 2 >= nt) break;
+        step(t + 2, std::integral_constant<int, 2>{});
       }
     } else {
       wait_step(t_lo);
@@ -3203,10 +3316,10 @@ Variant pick_variant(const HstuAttnFwdArgs* a) {
 // Workspace of the MFMA kernel: [scaled, padded position table][per-sequence int32-timestamp flag]
 // [int32 timestamps][their (min, max) per key tile], each part a multiple of 256 bytes.
 struct WorkspacePlan {
-  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes, sched_bytes, ctr_bytes, partial_bytes;
+  size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes, mrange_bytes, sched_bytes, ctr_bytes, partial_bytes;
   int split_cap;          // chunk slots of the partial buffer (0: no tile is split)
   long long items_max;    // capacity of the work list (0 = no list)
-  size_t bias_total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes; }
+  size_t bias_total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes + mrange_bytes; }
   size_t total() const { return bias_total() + sched_bytes + ctr_bytes + partial_bytes; }
 };
 
@@ -3217,7 +3330,7 @@ constexpr int SPLIT_CAP_DEFAULT = 32;
 
 // max_bytes: a workspace this small must do (the split capacity is cut down to fit it).
 WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, size_t max_bytes = ~(size_t)0) {
-  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const Variant var = pick_variant(a);
   if (var != V_MFMA_BF16 && var != V_MFMA_FP8) return w;
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
@@ -3244,6 +3357,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, 
     w.rel_bytes = up(n_ts * sizeof(int32_t) + 160);
     w.range_bytes = up(tiles * 2 * sizeof(int32_t) + 16);
   }
+  if (a->mask) w.mrange_bytes = up((size_t)(a->mask_batched ? a->B : 1) * (size_t)n_qtiles * 2 * sizeof(int32_t));
   const long long t128 = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
   const size_t chunk_bytes = (size_t)a->H * (size_t)BM * (size_t)a->d_v * sizeof(float);
   for (;;) {
@@ -3419,7 +3533,9 @@ int slots_per_xcd(const Params& p, int32_t* out) {
     if (e != hipSuccess || n <= 0) return fail(HSTU_ERR_LAUNCH, "hipDeviceGetAttribute(multiprocessor count): %s", hipGetErrorString(e));
     if (dev >= 0 && dev < kMaxDev) __atomic_store_n(&cus[dev], n, __ATOMIC_RELEASE);
   }
-  const int per_cu = (p.mask || p.dense_bias) ? 1 : (p.d_qk <= 64 ? 4 : 2);
+  // (by registers and LDS: with dense operands the d = 64 kernel takes 153 registers, three waves per SIMD)
+  const bool dense = p.mask || p.dense_bias;
+  const int per_cu = p.d_qk > 64 ? 2 : (dense && p.d_qk > 32 ? 3 : 4);
   const int slots = n * per_cu / 8;
   *out = slots > 0 ? slots : 1;
   return HSTU_OK;
@@ -3441,6 +3557,8 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   int32_t* ok_out = ws.ok_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes) : nullptr;
   int32_t* rel_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes);
   int32_t* range_out = (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes);
+  int32_t* mrange_out = ws.mrange_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes + ws.range_bytes) : nullptr;
+  q.mask_range = mrange_out;
   q.ws_base = base;
   int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
   q.sched = sched_out;
@@ -3456,12 +3574,14 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   const long long blocks_pos = ws.pos_bytes ? ((long long)q.pos_heads * (2 * q.L - 1 + 2 * POS_PAD) + 255) / 256 : 0;
   const long long blocks_ts = ws.ok_bytes ? q.B : 0;
   long long blocks = blocks_pos > blocks_ts ? blocks_pos : blocks_ts;
+  const long long blocks_mask = ws.mrange_bytes ? (long long)(q.mask_batched ? q.B : 1) * q.n_qtiles : 0;
+  blocks = blocks > blocks_mask ? blocks : blocks_mask;
   blocks = blocks < 1 ? 1 : (blocks > 4096 ? 4096 : blocks);
   if (ws.sched_bytes) ++blocks;   // the last workgroup builds the work lists
   if ((ws.bias_total() || ws.sched_bytes) && (!(args->flags & HSTU_FWD_WORKSPACE_PREPARED) || (args->flags & HSTU_FWD_PREPARE_ONLY))) {
     static const TsKeys no_keys = {{0}, {0}, {0}};
     const TsKeys& keys = tab_out ? bucket_law(q.ts_bucket_size).keys : no_keys;
-    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out, keys);
+    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out, mrange_out, keys);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
   }

@@ -481,6 +481,50 @@ def test_dense_bias_large_on_matrix_cores(gpu):
   assert (got[1, 333:] == 0).all()
 
 
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("shape", ["band", "blocks", "lower-left", "nothing", "one pair"])
+@pytest.mark.parametrize("batched", [True, False])
+def test_dense_mask_step_ranges(gpu, d, shape, batched):
+  # The preparation kernel finds, per tile of 128 query rows, the range of 32-key steps in which the mask keeps
+  # anything, and the main kernel runs only those.  Masks whose kept pairs start late, end early, leave whole
+  # tiles or whole sequences empty, or keep one single pair; 3 query tiles (the last one partial), keys of
+  # another length than the queries, with and without a bias.
+  rng = np.random.default_rng(460 + d + len(shape))
+  B, L, Lkv, H = 3, 300, 464, 2
+  q = O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3)
+  k, v = (O.round_bf16(rng.standard_normal((B, Lkv, H, d)).astype(np.float32) * 0.3) for _ in range(2))
+  nb = B if batched else 1
+  mask = np.zeros((nb, L, Lkv), dtype=np.uint8)
+  i, j = np.arange(L)[:, None], np.arange(Lkv)[None, :]
+  if shape == "band":
+    for b in range(nb):
+      mask[b] = (np.abs(j - i - 40 * b) <= 45) & (rng.random((L, Lkv)) < 0.8)
+  elif shape == "blocks":
+    for b in range(nb):
+      mask[b, 128:256, 64 + 32 * b:96 + 32 * b] = 1      # one step of the second tile; the other tiles keep nothing
+      mask[b, 290:, 400:] = rng.random((10, 64)) < 0.5   # the partial last tile: its last two steps
+  elif shape == "lower-left":
+    mask[:, 200:, :33] = 1
+  elif shape == "one pair":
+    mask[nb - 1, 129, 463] = 1
+  bias = rng.standard_normal((B, L, Lkv)).astype(np.float32) * 0.5 if d == 128 else None
+  qd, kd, vd = (_dev(t, torch.bfloat16) for t in (q, k, v))
+  out = torch.full((B, L, H, d), float("nan"), dtype=torch.bfloat16, device="cuda:0")
+  args, keep = hstu_ops.build_args(qd, kd, vd, out, n=L, alpha=1.0, causal=False,
+                                   mask=_dev(mask if batched else mask[0]), bias=_dev(bias))
+  assert hstu_ops.kernel_variant(args) == "hstu_fwd_mfma_bf16"
+  hstu_ops._run(args, keep)
+  torch.cuda.synchronize()
+  got = out.float().cpu().numpy()
+  full = np.broadcast_to(mask.astype(np.float64), (B, L, Lkv))
+  ref = O.pointwise_attention_dense(q, k, v, full, bias)      # (divides by the query length, like n = L)
+  assert np.isfinite(got).all()
+  assert np.abs(got - ref).max() <= BF16_TOL * max(np.abs(ref).max(), 1e-3)
+  # rows that keep no key: exact zeros
+  empty = full.sum(axis=2) == 0
+  assert (got[empty] == 0).all()
+
+
 def test_shared_tables_and_strided_inputs(gpu):
   rng = np.random.default_rng(45)
   B, L, H, d = 2, 130, 4, 64

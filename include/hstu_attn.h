@@ -59,9 +59,10 @@ enum HstuMaskMode {
 /* Bits of HstuAttnFwdArgs.flags. */
 enum HstuFwdFlags {
   /* The workspace still holds what an earlier call prepared from the same
-   * shapes, lengths / offsets, timestamps and bias tables (for example the
-   * same call repeated, or a benchmark timing the main kernel alone): skip
-   * the preparation kernel.  Undefined results if that does not hold. */
+   * shapes, lengths / offsets, timestamps, bias tables and dense mask (for
+   * example the same call repeated, or a benchmark timing the main kernel
+   * alone): skip the preparation kernel.  Undefined results if that does not
+   * hold. */
   HSTU_FWD_WORKSPACE_PREPARED = 1,
   /* Only prepare the workspace (the kernel that builds the work list, the scaled
    * tables and the int32 timestamps) and return: a model whose layers share
@@ -134,7 +135,8 @@ typedef struct HstuAttnFwdArgs {
   /* Dense operands (the layer-side call of recml/layers/keras/hstu.py:356-390).  bf16 calls take
    * them on the matrix cores when Lkv is a multiple of 16 (mask) / 4 (bias), the arrays are
    * 16-byte aligned and no table bias or segment ids come with them; any other call on the
-   * general kernel. */
+   * general kernel.  Key steps in which the mask keeps no pair of a query tile cost nothing
+   * (a causal mask given as a matrix costs what the causal flag costs, plus reading it). */
   const uint8_t* mask;    /* explicit keep-mask (non-zero = keep) or null     */
   int32_t mask_batched;   /* 0: [L, Lkv] shared; 1: [B, L, Lkv]               */
   int32_t dense_bias_batched; /* 0: [L, Lkv] shared; 1: [B, L, Lkv]           */
@@ -166,7 +168,9 @@ int hstu_attn_abi_version(void);
  * preparation kernel builds (on every call, or once per batch, see
  * HSTU_FWD_PREPARE_ONLY): the work list of (sequence, query tile, key chunk)
  * items, the scaled position table, the timestamp bucket tables, int32
- * timestamps with their per-tile ranges; and what the main kernel itself
+ * timestamps with their per-tile ranges, for a dense mask the range of key
+ * steps in which it keeps anything per tile of 128 query rows (the mask is
+ * read once for that); and what the main kernel itself
  * uses: the counters it draws work from and, for query tiles whose keys are
  * split between workgroups (decided on the device from the lengths, when few
  * long tiles would otherwise finish long after the rest), the arrival counters

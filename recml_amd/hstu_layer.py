@@ -139,7 +139,7 @@ class HSTUBlock(torch.nn.Module):
         attn = hstu_ops.dense_attention_torch(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
       else:
         attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
-                                            scaled_pointwise_attn=self.scaled_pointwise_attn)
+                                            scaled_pointwise_attn=self.scaled_pointwise_attn, batch=batch)
     else:
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,

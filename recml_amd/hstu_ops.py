@@ -84,7 +84,7 @@ class AttentionBatch:
   (`HSTU.forward` does).  It also keeps the device scratch, so no call after the first allocates.
 
   The preparation is reused when the call's shapes and options are the same and the tensors it was
-  built from (`seq_lens` / `seq_offsets`, `timestamps`, `pos_bias`, `ts_bias`) are the same objects,
+  built from (`seq_lens` / `seq_offsets`, `timestamps`, `pos_bias`, `ts_bias`, a dense `mask`) are the same objects,
   unmodified since (torch's version counter); anything else prepares again.  q, k, v, `alpha` and `n`
   may differ from call to call.  Not for concurrent use on several streams.
   """
@@ -156,7 +156,7 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
                sliding_window_size=None, mask=None, bias=None,
                q_scale=None, k_scale=None, batch=None):
   """Validates the call and fills an HstuAttnFwdArgs.  Returns (args, keepalive)."""
-  given = (seq_lens, seq_offsets, timestamps, pos_bias, ts_bias)
+  given = (seq_lens, seq_offsets, timestamps, pos_bias, ts_bias, mask)
   for name, t in (("q", q), ("k", k), ("v", v)):
     _check_gpu(name, t)
   if q.dtype not in _DTYPES:
@@ -286,7 +286,13 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
       a.mask_batched = 1
     else:
       raise ValueError(f"mask must be [{L}, {Lkv}] or [{B}, {L}, {Lkv}], got {tuple(mask.shape)}")
-    m8 = (mask != 0).to(torch.uint8).contiguous()
+    # the kernels keep a pair where the byte is non-zero: bool and uint8 masks go as they are
+    if mask.dtype == torch.bool:
+      m8 = mask.contiguous().view(torch.uint8)
+    elif mask.dtype == torch.uint8:
+      m8 = mask.contiguous()
+    else:
+      m8 = (mask != 0).to(torch.uint8).contiguous()
     keep.append(m8)
     a.mask = m8.data_ptr()
   if bias is not None:
@@ -328,13 +334,13 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
     if batch is None:
       _attach_workspace(a, keep)
     else:
-      # everything the preparation reads or the workspace layout depends on; dense operands and segment
-      # ids (not part of it, but of the choice of kernel) rule the reuse out
+      # everything the preparation reads (the dense mask included: its key-step ranges) or the workspace
+      # layout depends on; segment ids (not part of it, but of the choice of kernel) rule the reuse out
       sig = None
       idents = tuple(AttentionBatch._ident(t) for t in given)
-      if mask is None and bias is None and q_segment_ids is None and False not in idents:
+      if q_segment_ids is None and False not in idents:
         sig = (tuple(q.shape), tuple(k.shape), int(v.shape[-1]), q.dtype, max_len, bool(causal),
-               sliding_window_size, float(ts_bucket_size), idents)
+               sliding_window_size, float(ts_bucket_size), bias is not None, idents)
       batch._attach(a, keep, sig, given)
   return a, keep
 
@@ -600,7 +606,7 @@ def pointwise_splash_attention(
 
 
 def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
-                        scaled_pointwise_attn=False, seq_lens=None):
+                        scaled_pointwise_attn=False, seq_lens=None, batch=None):
   """Layer-side call, recml/layers/keras/hstu.py:356-390 (inference).
 
   `attention_mask` is the [B, L, L] 0/1 mask the layer builds with
@@ -608,7 +614,9 @@ def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
   shared by heads.  scaled_pointwise_attn=True divides q by sqrt(d) and skips
   the 1/L (hstu.py:365-378).  A caller that knows its batch is end-padded and
   causal can pass `seq_lens` with attention_mask=None: same result without
-  ever building the [B, L, L] mask.
+  ever building the [B, L, L] mask.  `batch`: an AttentionBatch shared by the
+  calls that bring the same mask (the layers of a model): the mask is then
+  scanned for its key-step ranges once, by the first of them.
   """
   d = q.shape[-1]
   alpha = 1.0 / math.sqrt(d) if scaled_pointwise_attn else 1.0
@@ -617,6 +625,6 @@ def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
     if seq_lens is None:
       raise ValueError("pass attention_mask or seq_lens")
     return hstu_attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha,
-                          causal=True, bias=attention_bias)
+                          causal=True, bias=attention_bias, batch=batch)
   return hstu_attention(q, k, v, n=n, alpha=alpha, causal=False,
-                        mask=attention_mask, bias=attention_bias)
+                        mask=attention_mask, bias=attention_bias, batch=batch)

@@ -108,3 +108,31 @@ def test_model_prepares_once_for_its_blocks(gpu, monkeypatch):
       ref = model(ids, seq_lens=lens, pos_bias=pos, jagged=jagged)
       monkeypatch.setattr(hstu_ops, "AttentionBatch", Counting)
       assert torch.equal(out, ref), jagged
+
+
+def test_layers_share_the_scan_of_a_dense_mask(gpu):
+  """The layer-side call with a [B, L, L] mask: the preparation reads the mask for each query tile's range of
+  key steps; calls on the same batch reuse it, and a mask edited in place is read again."""
+  rng = np.random.default_rng(1503)
+  B, L, H, d = 3, 400, 2, 128
+  q, k, v = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.3) for _ in range(3))
+  lens = np.array([400, 150, 31])
+  pad = (np.arange(L)[None] < lens[:, None]).astype(np.float32)
+  mask_np = O.make_causal_mask(pad).astype(bool)
+  bias_np = (rng.standard_normal((B, L, L)) * 0.5).astype(np.float32)
+  mask, bias = _dev(mask_np), _dev(bias_np)
+  qd, kd, vd = (_dev(t, bf) for t in (q, k, v))
+  batch = hstu_ops.AttentionBatch()
+  outs = [recml_amd.pointwise_attention(qd, kd, vd, mask, bias, batch=batch) for _ in range(3)]
+  assert batch.prepared_calls == 2
+  alone = recml_amd.pointwise_attention(qd, kd, vd, mask, bias)
+  for o in outs:
+    assert torch.equal(o, alone)
+  ref = O.pointwise_attention_dense(q, k, v, mask_np, bias_np)
+  assert np.abs(alone.float().cpu().numpy() - ref).max() <= 2e-2 * np.abs(ref).max()
+  # the mask opened up in place (every pair kept): ranges found for the causal mask would drop most of it
+  mask.fill_(True)
+  again = recml_amd.pointwise_attention(qd, kd, vd, mask, bias, batch=batch)
+  assert batch.prepared_calls == 2
+  ref = O.pointwise_attention_dense(q, k, v, np.ones((B, L, L)), bias_np)
+  assert np.abs(again.float().cpu().numpy() - ref).max() <= 2e-2 * np.abs(ref).max()

@@ -428,7 +428,7 @@ def bench_dense(args, dev):
       "config": {"workload": f"A1-dense: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",
                  "kernel": variant},
       "roofline": {"bound": "hbm", "achieved": nbytes / (ker * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                   "frac": nbytes / (ker * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": None, "kernel_ms_avg": ker,
+                   "frac": nbytes / (ker * 1e-3) / 1e9 / PEAK_HBM_GBS, "traffic": measured_traffic("a1-dense"), "kernel_ms_avg": ker,
                    "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
                    "dense_operand_bytes_as_read_by_all_heads": H * B * steps_run * 128 * 32 * 5,
                    "prepare_ms": with_prepare_ms - ms,

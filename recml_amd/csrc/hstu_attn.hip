@@ -109,6 +109,7 @@ struct Params {
   // workgroup that arrives last at the tile's counter sums them and writes the rows.
   int32_t split_cap;         // chunk slots of the partial buffer (per head)
   int32_t n_slots;           // workgroups that run at once per XCD (what the split decision balances for)
+  int32_t g_rows;            // general forward: query rows per workgroup
   const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
@@ -198,6 +199,7 @@ __device__ __forceinline__ void stf(bf16_t* p, float x) { *p = (bf16_t)x; }
 // General kernel: fp32 FMA arithmetic, every option.
 // ---------------------------------------------------------------------------
 
+constexpr float LOG2E = 1.4426950408889634f;
 constexpr int GT = 32;       // query rows and keys per tile
 constexpr int GMAXX = 32;    // d_v / 8 accumulators per thread, d_v <= 256
 
@@ -249,101 +251,308 @@ __device__ __forceinline__ bool general_keep(const Params& p, const Seq& s,
   return keep;
 }
 
-template <typename T>
-__global__ __launch_bounds__(256) void hstu_fwd_general(const Params p) {
-  extern __shared__ float gsm[];
-  const int dq = p.d_qk, dv = p.d_v;
-  const int kp = dq + 1;                   // odd pitch: column reads of K
-  float* Qs = gsm;                         // [GT][dq]
-  float* Ks = Qs + GT * dq;                // [GT][kp]
-  float* Vs = Ks + GT * kp;                // [GT][dv]
-  float* Ps = Vs + GT * dv;                // [GT][GT+1]
+// The general forward: fp32 arithmetic on the matrix cores (v_mfma_f32_32x32x2_f32: fp32 products, fp32
+// sums), every option, any head dims up to 256, fp32 or bf16 storage, any strides.  A workgroup takes up
+// to 128 query rows of one (sequence, head), 32 per wave, and streams the keys 32 at a time through LDS:
+//   S^T = K Q^T        A = K rows, B = Q rows, both read from LDS two floats per lane and pair of steps;
+//   pointwise          on the accumulators, one (query, key) pair per value, through general_keep / general_bias;
+//   O^T += V^T P^T     A = V rows from LDS, B = the accumulators of S^T as they are (fp32: no packing).
+// The order of the terms of a dot product is free, so slot l / 32 of step s of a pair takes channel
+// 4 (s / 2) + 2 (l / 32) + s % 2: the two channels of a lane are neighbours in memory.  Row pitches keep the
+// reads free of bank conflicts: twice an odd number of floats for Q and K (rows 0 .. 31 then start on the 32
+// even banks), 8 more than a multiple of 32 for V (rows k and k + 4, read by the two halves of a wave, then
+// lie 32 banks apart).
+__host__ __device__ inline int general_pitch_qk(int d) { const int d4 = (d + 3) & ~3; return ((d4 >> 1) & 1) ? d4 : d4 + 2; }
+__host__ __device__ inline int general_pitch_v(int d) { return ((d + 31) & ~31) + 8; }
+constexpr int GMAXB = 8;     // 32-channel blocks of the output, d_v <= 256
 
-  const int qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+// Four consecutive elements of a row as floats, zeros where the row or the column is out of range; one
+// 16-byte (fp32) or 8-byte (bf16) load when the caller says the address is aligned for it.
+__device__ __forceinline__ float4 general_load4(const float* row, int c, int d, bool row_ok, bool vec) {
+  float4 r = {0.f, 0.f, 0.f, 0.f};
+  if (!row_ok || c >= d) return r;
+  if (vec && c + 4 <= d) return *(const float4*)(row + c);
+  r.x = row[c];
+  if (c + 1 < d) r.y = row[c + 1];
+  if (c + 2 < d) r.z = row[c + 2];
+  if (c + 3 < d) r.w = row[c + 3];
+  return r;
+}
+__device__ __forceinline__ float4 general_load4(const bf16_t* row, int c, int d, bool row_ok, bool vec) {
+  float4 r = {0.f, 0.f, 0.f, 0.f};
+  if (!row_ok || c >= d) return r;
+  if (vec && c + 4 <= d) {
+    const uint2 u = *(const uint2*)(row + c);
+    r.x = __builtin_bit_cast(float, u.x << 16);
+    r.y = __builtin_bit_cast(float, u.x & 0xffff0000u);
+    r.z = __builtin_bit_cast(float, u.y << 16);
+    r.w = __builtin_bit_cast(float, u.y & 0xffff0000u);
+    return r;
+  }
+  r.x = (float)row[c];
+  if (c + 1 < d) r.y = (float)row[c + 1];
+  if (c + 2 < d) r.z = (float)row[c + 2];
+  if (c + 3 < d) r.w = (float)row[c + 3];
+  return r;
+}
+
+// SMALL (head dims up to 128): the wave's Q rows stay in registers instead of LDS, 64 accumulators instead of
+// 128: two waves per SIMD and 34 KB of LDS, several workgroups per CU, so that one workgroup's loads, barriers
+// and pointwise work run under another's products.
+template <typename T, bool SMALL>
+__global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Params p) {
+  extern __shared__ __attribute__((aligned(16))) float gsm[];
+  constexpr int NB = SMALL ? 4 : GMAXB;    // 32-channel blocks of the output
+  const int dq = p.d_qk, dv = p.d_v;
+  const int GQ = p.g_rows;                 // query rows of this workgroup: 128, or fewer when LDS is short
+  const int dq4 = (dq + 3) & ~3;
+  const int qp_ = general_pitch_qk(dq), vp_ = general_pitch_v(dv);
+  const int nblk = (dv + 31) >> 5;
+  float* Qs = gsm;                         // [GQ][qp_] (not SMALL)
+  float* Ks = Qs + (SMALL ? 0 : GQ * qp_); // [32][qp_]
+  float* Vs = Ks + GT * qp_;               // [32][vp_]
+
+  // Workgroups are handed to the eight XCDs in turn by their linear index: with the head fastest and the query
+  // tile slowest every XCD sees every tile position (under the causal mask the last tiles have many times the
+  // work of the first), a sequence's tiles of one head meet its K and V rows in one L2, and the longest
+  // tiles start first.
+  const int h = blockIdx.x, b = blockIdx.y, qt = gridDim.z - 1 - blockIdx.z;
   const Seq s = seq_info(p, b, h);
-  const int q0 = qt * GT;
+  const int q0 = qt * GQ;
   if (q0 >= s.rows) return;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, m = lane & 31, hh = lane >> 5;
   const T* __restrict__ qp = (const T*)p.q;
   const T* __restrict__ kp_ = (const T*)p.k;
   const T* __restrict__ vp = (const T*)p.v;
   T* __restrict__ op = (T*)p.out;
+  const bool wave_on = 32 * w < GQ;        // waves beyond the tile's rows only help with the loads
+  const int r0 = q0 + 32 * w;
+  const int qi = r0 + m;                   // this lane's query row
+  // whole groups of four elements can be fetched by one load when bases and row strides allow
+  constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
+  const bool kvec = (((uintptr_t)(kp_ + s.bk) & VMASK) == 0) && (p.k_st & 3) == 0;
+  const bool vvec = (((uintptr_t)(vp + s.bv) & VMASK) == 0) && (p.v_st & 3) == 0;
+  const bool qvec = (((uintptr_t)(qp + s.bq) & VMASK) == 0) && (p.q_st & 3) == 0;
 
-  const int oi = tid >> 3, ocg = tid & 7;  // output row / column group
-  const int nx = (dv + 7) >> 3;
-  float acc[GMAXX];
+  floatx16 o[NB];
 #pragma unroll
-  for (int x = 0; x < GMAXX; ++x) acc[x] = 0.f;
+  for (int x = 0; x < NB; ++x)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[x][r] = 0.f;
 
   if (q0 < s.n_q) {
-    for (int e = tid; e < GT * dq; e += 256) {
-      int r = e / dq, c = e - r * dq;
-      int i = q0 + r;
-      Qs[e] = (i < s.n_q) ? ldf(qp + s.bq + (int64_t)i * p.q_st + c) : 0.f;
+    // tiles are brought by eight threads per row, four channels per thread and turn
+    const int lr = tid >> 3, lc = (tid & 7) * 4;
+    // SMALL: the lane's share of its query row, channels 4u + 2hh and 4u + 2hh + 1 for the pair of steps u
+    float2 qf[SMALL ? 32 : 1];
+    if constexpr (SMALL) {
+      const T* qrow_g = qp + s.bq + (int64_t)qi * p.q_st;
+#pragma unroll
+      for (int u = 0; u < 32; ++u) {
+        qf[u] = float2{0.f, 0.f};
+        if (4 * u < dq4 && qi < s.n_q) {
+          const int c = 4 * u + 2 * hh;
+          if (c < dq) qf[u].x = ldf(qrow_g + c);
+          if (c + 1 < dq) qf[u].y = ldf(qrow_g + c + 1);
+        }
+      }
+    } else {
+      for (int r = lr; r < GQ; r += 32) {
+        const int i = q0 + r;
+        for (int c = lc; c < dq4; c += 32) {
+          // (rows of Q and K start on 8-byte, not 16-byte boundaries: two stores)
+          const float4 t4 = general_load4(qp + s.bq + (int64_t)i * p.q_st, c, dq, i < s.n_q, qvec);
+          *(float2*)(Qs + r * qp_ + c) = float2{t4.x, t4.y};
+          *(float2*)(Qs + r * qp_ + c + 2) = float2{t4.z, t4.w};
+        }
+      }
     }
     int kv_end = s.n_kv;
-    if (p.causal && q0 + GT < kv_end) kv_end = q0 + GT;
-    if (p.window >= 0 && q0 + GT + p.window < kv_end) kv_end = q0 + GT + p.window;
+    if (p.causal && q0 + GQ < kv_end) kv_end = q0 + GQ;
+    if (p.window >= 0 && q0 + GQ + p.window < kv_end) kv_end = q0 + GQ + p.window;
     int kv_begin = 0;
     if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
+    const int vcols = nblk * 32;
+    // The next tile travels in registers while this one is computed on: up to 8 + 8 groups of four per thread
+    // (head dims up to 256).  When bases and strides allow whole groups and the head dims are multiples of four,
+    // the loads are unconditional (rows past the sequence re-read its last key, columns past the head dim the
+    // last group) and what must be zero is zeroed on the way into LDS: nothing then uses a loaded value before
+    // the tile is staged, and the loads stay in flight behind the products.  Otherwise element by element.
+    constexpr int NG = SMALL ? 4 : 8;
+    typedef typename std::conditional<sizeof(T) == 4, float4, uint2>::type Raw;
+    const bool fast = kvec && vvec && (dq & 3) == 0 && (dv & 3) == 0;
+    const int ngk = (dq4 + 31) >> 5, ngv = (vcols + 31) >> 5;
+    Raw kraw[NG], vraw[NG];
+    auto widen = [](const Raw& u) -> float4 {
+      if constexpr (sizeof(T) == 4) {
+        return u;
+      } else {
+        return float4{__builtin_bit_cast(float, u.x << 16), __builtin_bit_cast(float, u.x & 0xffff0000u),
+                      __builtin_bit_cast(float, u.y << 16), __builtin_bit_cast(float, u.y & 0xffff0000u)};
+      }
+    };
+    // (the element-by-element path leaves the same registers: bf16 elements packed again, nothing is lost)
+    auto narrow = [](const float4& f) -> Raw {
+      if constexpr (sizeof(T) == 4) {
+        return f;
+      } else {
+        return uint2{(__builtin_bit_cast(uint32_t, f.x) >> 16) | (__builtin_bit_cast(uint32_t, f.y) & 0xffff0000u),
+                     (__builtin_bit_cast(uint32_t, f.z) >> 16) | (__builtin_bit_cast(uint32_t, f.w) & 0xffff0000u)};
+      }
+    };
+    auto fetch_k = [&](int kv0) {
+      const int j = kv0 + lr;
+      const int jc = fast && j >= s.n_kv ? s.n_kv - 1 : j;
+      const T* krow = kp_ + s.bk + (int64_t)jc * p.k_st;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int c = lc + 32 * g;
+        if (g < ngk) {
+          if (fast) kraw[g] = *(const Raw*)(krow + (c < dq ? c : dq - 4));
+          else kraw[g] = narrow(general_load4(krow, c, dq, j < s.n_kv, false));
+        }
+      }
+    };
+    auto fetch_v = [&](int kv0) {
+      const int j = kv0 + lr;
+      const int jc = fast && j >= s.n_kv ? s.n_kv - 1 : j;
+      const T* vrow = vp + s.bv + (int64_t)jc * p.v_st;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int c = lc + 32 * g;
+        if (g < ngv) {
+          if (fast) vraw[g] = *(const Raw*)(vrow + (c < dv ? c : dv - 4));
+          else vraw[g] = narrow(general_load4(vrow, c, dv, j < s.n_kv, false));
+        }
+      }
+    };
+    auto stage = [&](int kv0) {
+      const bool row_ok = kv0 + lr < s.n_kv;
+      const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int c = lc + 32 * g;
+        if (g < ngk && c < dq4) {
+          const float4 t4 = (!fast || (row_ok && c < dq)) ? widen(kraw[g]) : zero4;
+          // (rows of Q and K start on 8-byte, not 16-byte boundaries: two stores)
+          *(float2*)(Ks + lr * qp_ + c) = float2{t4.x, t4.y};
+          *(float2*)(Ks + lr * qp_ + c + 2) = float2{t4.z, t4.w};
+        }
+        if (g < ngv && c < vcols) *(float4*)(Vs + lr * vp_ + c) = (!fast || (row_ok && c < dv)) ? widen(vraw[g]) : zero4;
+      }
+    };
+    if constexpr (SMALL) {
+      // the slack behind a row's channels is read by the logit loop when the head dim is no multiple of 16
+      for (int e = tid; e < GT * (qp_ - dq4); e += 256) Ks[(e / (qp_ - dq4)) * qp_ + dq4 + e % (qp_ - dq4)] = 0.f;
+    }
+    if (kv_begin < kv_end) {
+      fetch_k(kv_begin);
+      fetch_v(kv_begin);
+    }
 
     for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
+      __syncthreads();                     // everyone is done with the tile before
+      stage(kv0);
       __syncthreads();
-      for (int e = tid; e < GT * dq; e += 256) {
-        int r = e / dq, c = e - r * dq;
-        int j = kv0 + r;
-        Ks[r * kp + c] = (j < s.n_kv) ? ldf(kp_ + s.bk + (int64_t)j * p.k_st + c) : 0.f;
+      // the next tile: its K rows are asked for now, its V rows once the pointwise part is done (fewer
+      // registers held across it)
+      const bool more = kv0 + GT < kv_end;
+      if (more) fetch_k(kv0 + GT);
+      // nothing for a wave whose rows all lie before these keys (causal) or outside the window
+      bool live = wave_on && r0 < s.n_q;
+      if (p.causal && kv0 > r0 + 31) live = false;
+      if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
+      if (!live) {
+        if (more) fetch_v(kv0 + GT);
+        continue;
       }
-      for (int e = tid; e < GT * dv; e += 256) {
-        int r = e / dv, c = e - r * dv;
-        int j = kv0 + r;
-        Vs[e] = (j < s.n_kv) ? ldf(vp + s.bv + (int64_t)j * p.v_st + c) : 0.f;
-      }
-      __syncthreads();
-      {
-        const int tx = tid & 31, ty = tid >> 5;
-        float sacc[4] = {0.f, 0.f, 0.f, 0.f};
-        const float* krow = Ks + tx * kp;
-        for (int c = 0; c < dq; ++c) {
-          float kvv = krow[c];
+      floatx16 sacc;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) sacc[r] = fmaf(Qs[(ty + 8 * r) * dq + c], kvv, sacc[r]);
-        }
-        const int j = kv0 + tx;
+      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+      const float* krow = Ks + m * qp_ + 2 * hh;
+      const float* qrow = Qs + (32 * w + m) * qp_ + 2 * hh;
+      // (sixteen channels at a time, their eight reads ahead of the eight products)
+      int c = 0;
+      if constexpr (SMALL) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = q0 + ty + 8 * r;
-          float pval = 0.f;
-          if (general_keep(p, s, b, i, j)) {
-            float x = p.alpha * sacc[r] + general_bias(p, s, b, h, i, j);
-            pval = x / (1.0f + expf(-x));
+        for (int u0 = 0; u0 < 32; u0 += 4) {
+          if (4 * u0 < dq4) {       // (sixteen channels at a time; head dims that are no multiple of 16 read up to 12 floats
+            float2 kk[4];           // of the pitch's slack or of the next row, and multiply them by zeros of Q)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) kk[u] = *(const float2*)(krow + 4 * (u0 + u));
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].x, qf[u0 + u].x, sacc, 0, 0, 0);
+              sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].y, qf[u0 + u].y, sacc, 0, 0, 0);
+            }
           }
-          Ps[(ty + 8 * r) * (GT + 1) + tx] = pval;
+        }
+        c = dq4;
+      }
+      for (; c + 16 <= dq4; c += 16) {
+        float2 kk[4], qq[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          kk[u] = *(const float2*)(krow + c + 4 * u);
+          qq[u] = *(const float2*)(qrow + c + 4 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].x, qq[u].x, sacc, 0, 0, 0);
+          sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].y, qq[u].y, sacc, 0, 0, 0);
         }
       }
-      __syncthreads();
-      for (int jj = 0; jj < GT; ++jj) {
-        float pv = Ps[oi * (GT + 1) + jj];
-        const float* vrow = Vs + jj * dv;
+      for (; c < dq4; c += 4) {
+        const float2 kk = *(const float2*)(krow + c), qq = *(const float2*)(qrow + c);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.x, qq.x, sacc, 0, 0, 0);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.y, qq.y, sacc, 0, 0, 0);
+      }
+      // lane holds S^T[key kv0 + 8g + 4hh + tt][query qi], r = 4g + tt.  The index masks are two bounds per
+      // lane; segment ids, an explicit mask and the biases go through the per-pair helpers only when present.
+      int hi = s.n_kv - 1, lo = 0;
+      if (p.causal) hi = qi < hi ? qi : hi;
+      if (p.window >= 0) {
+        hi = qi + p.window < hi ? qi + p.window : hi;
+        lo = qi - p.window;
+      }
+      if (qi >= s.n_q) hi = -1;
+      const bool by_pair = p.mask_mode == HSTU_MASK_SEGMENT || p.mask != nullptr;
+      const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
 #pragma unroll
-        for (int x = 0; x < GMAXX; ++x) {
-          if (x < nx) {
-            int c = ocg + 8 * x;
-            if (c < dv) acc[x] = fmaf(pv, vrow[c], acc[x]);
-          }
+      for (int r = 0; r < 16; ++r) {
+        const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+        bool keep = j >= lo && j <= hi;
+        if (by_pair) keep = keep && general_keep(p, s, b, qi, j);
+        float x = p.alpha * sacc[r];
+        if (biased && keep) x += general_bias(p, s, b, h, qi, j);
+        // silu(x) = x / (1 + e^-x), by the hardware's exp2 and reciprocal (1 ulp each)
+        const float val = x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
+        sacc[r] = keep ? val : 0.f;      // P^T in place of S^T
+      }
+      // (key by key across the output blocks: consecutive products go to different accumulators)
+      if (more) fetch_v(kv0 + GT);
+      const float* vcol = Vs + (4 * hh) * vp_ + m;
+#pragma unroll
+      for (int x = 0; x < NB; ++x) {
+        if (x < nblk) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            o[x] = __builtin_amdgcn_mfma_f32_32x32x2f32(vcol[(8 * (r >> 2) + (r & 3)) * vp_ + 32 * x], sacc[r], o[x], 0, 0, 0);
         }
       }
     }
   }
-  // rows past the sequence are written as exact zeros (padded layout)
-  const int i = q0 + oi;
-  if (i < s.rows) {
-    const bool live = i < s.n_q;
+  // O^T[channel 32x + 8g + 4hh + tt][query qi]; rows past the sequence are written as exact zeros (padded layout)
+  if (wave_on && qi < s.rows) {
+    const bool live_row = qi < s.n_q;
 #pragma unroll
-    for (int x = 0; x < GMAXX; ++x) {
-      if (x < nx) {
-        int c = ocg + 8 * x;
-        if (c < dv) stf(op + s.bo + (int64_t)i * p.o_st + c, live ? acc[x] * p.inv_n : 0.f);
+    for (int x = 0; x < NB; ++x) {
+      if (x < nblk) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c = 32 * x + 8 * (r >> 2) + 4 * hh + (r & 3);
+          if (c < dv) stf(op + s.bo + (int64_t)qi * p.o_st + c, live_row ? o[x][r] * p.inv_n : 0.f);
+        }
       }
     }
   }
@@ -382,7 +591,8 @@ __global__ __launch_bounds__(256) void hstu_bwd_dq(const Params p) {
   float* Hist = Ds + GT * (GT + 1);        // [ts_nb + 1] timestamp-bucket sums of this tile
   int* Bk = (int*)(Hist + 132);            // [GT][GT] bucket of each pair
 
-  const int qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // (head fastest, tile slowest and longest first: see hstu_fwd_general)
+  const int h = blockIdx.x, b = blockIdx.y, qt = gridDim.z - 1 - blockIdx.z;
   const Seq s = seq_info(p, b, h);
   const int q0 = qt * GT;
   if (q0 >= s.rows) return;
@@ -517,7 +727,8 @@ __global__ __launch_bounds__(256) void hstu_bwd_dkv(const Params p) {
   float* Ds = Os + GT * dv;                // [GT][GT+1] dS   [row][key]
   float* Ps = Ds + GT * (GT + 1);          // [GT][GT+1] P
 
-  const int kt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // (head fastest, tile slowest; under the causal mask the first key tile has the most rows behind it)
+  const int h = blockIdx.x, b = blockIdx.y, kt = blockIdx.z;
   const Seq s = seq_info(p, b, h);
   const int kv0 = kt * GT;
   const int krows = p.jagged ? s.n_kv : p.Lkv;      // rows of dk / dv that exist
@@ -667,7 +878,6 @@ struct TsKeys {                            // host-built part of the table, a ke
   uint8_t bkt[TS_KEYS];                    // by key: bucket the key's range starts in
 };
 
-constexpr float LOG2E = 1.4426950408889634f;
 
 template <int D, int KB>   // KB: bytes per q / k element (2 = bf16, 1 = fp8)
 struct MfmaSmem {
@@ -3417,13 +3627,27 @@ int allow_lds(const void* fn, int bytes, int* granted /* [kMaxDev] */) {
 }
 
 template <typename T>
-int launch_general(const Params& p, hipStream_t st) {
-  size_t smem = sizeof(float) * ((size_t)GT * p.d_qk + (size_t)GT * (p.d_qk + 1) + (size_t)GT * p.d_v + GT * (GT + 1));
-  static int granted[64];
-  if (int rc = allow_lds((const void*)hstu_fwd_general<T>, (int)smem, granted)) return rc;
+int launch_general(const Params& p_in, hipStream_t st) {
+  Params p = p_in;
+  const bool small = p.d_qk <= 128 && p.d_v <= 128;
+  // 128 query rows per workgroup; with head dims beyond 128 fewer where their fp32 rows would not fit the LDS
+  // beside the K and V tiles
+  auto lds_bytes = [&](int rows) {
+    return sizeof(float) * ((size_t)((small ? 0 : rows) + GT) * general_pitch_qk(p.d_qk) + (size_t)GT * general_pitch_v(p.d_v));
+  };
+  p.g_rows = 128;
+  while (p.g_rows > 32 && lds_bytes(p.g_rows) > 150 * 1024) p.g_rows >>= 1;
+  if (p.L < p.g_rows) p.g_rows = p.L <= 32 ? 32 : (p.L <= 64 ? 64 : 128);
+  const size_t smem = lds_bytes(p.g_rows);
+  if (smem > 160 * 1024) return fail(HSTU_ERR_SHAPE, "head dims %d / %d are beyond the general kernel's LDS", p.d_qk, p.d_v);
+  static int granted_small[64], granted_large[64];
+  if (int rc = small ? allow_lds((const void*)hstu_fwd_general<T, true>, (int)smem, granted_small)
+                     : allow_lds((const void*)hstu_fwd_general<T, false>, (int)smem, granted_large)) return rc;
   hipError_t e;
-  dim3 grid((p.L + GT - 1) / GT, p.H, p.B);
-  hipLaunchKernelGGL(hstu_fwd_general<T>, grid, dim3(256), smem, st, p);
+  if (p.B > 65535) return fail(HSTU_ERR_SHAPE, "the general kernel takes at most 65535 sequences per call, got %d", p.B);
+  dim3 grid(p.H, p.B, (p.L + p.g_rows - 1) / p.g_rows);
+  if (small) hipLaunchKernelGGL((hstu_fwd_general<T, true>), grid, dim3(256), smem, st, p);
+  else hipLaunchKernelGGL((hstu_fwd_general<T, false>), grid, dim3(256), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "general kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
@@ -3451,10 +3675,12 @@ int launch_bwd(const Params& p, hipStream_t st) {
   static int granted_q[64], granted_kv[64];
   if (int rc = allow_lds((const void*)hstu_bwd_dq<T>, (int)smem_q, granted_q)) return rc;
   if (int rc = allow_lds((const void*)hstu_bwd_dkv<T>, (int)smem_kv, granted_kv)) return rc;
-  hipLaunchKernelGGL(hstu_bwd_dq<T>, dim3((p.L + GT - 1) / GT, p.H, p.B), dim3(256), smem_q, st, p);
+  if (p.B > 65535 || (p.L + GT - 1) / GT > 65535 || (p.Lkv + GT - 1) / GT > 65535)
+    return fail(HSTU_ERR_SHAPE, "the general backward takes at most 65535 sequences and 65535 tiles of 32 rows per call");
+  hipLaunchKernelGGL(hstu_bwd_dq<T>, dim3(p.H, p.B, (p.L + GT - 1) / GT), dim3(256), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL(hstu_bwd_dkv<T>, dim3((p.Lkv + GT - 1) / GT, p.H, p.B), dim3(256), smem_kv, st, p);
+  hipLaunchKernelGGL(hstu_bwd_dkv<T>, dim3(p.H, p.B, (p.Lkv + GT - 1) / GT), dim3(256), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;

@@ -956,3 +956,48 @@ def test_general_kernel_on_random_option_mixes(gpu, seed):
   if lens is not None:
     for b in range(B):
       assert (got[b, lens[b]:] == 0).all(), case
+
+
+@pytest.mark.parametrize("d,dv", [(1, 1), (3, 5), (20, 20), (36, 100), (100, 36), (128, 128), (129, 64), (160, 160),
+                                  (200, 256), (256, 256)])
+@pytest.mark.parametrize("storage", ["fp32", "fp32 views", "bf16"])
+def test_general_kernel_head_dims_and_storage(gpu, d, dv, storage):
+  """The general kernel over head dims that are no multiple of 4 or 16, differ between q/k and v, or go beyond 128
+  (its Q rows then sit in LDS and a workgroup takes fewer rows), with rows that allow 16-byte loads, rows that do
+  not (views with an odd offset and stride), and bf16 storage; several 128-row tiles, a partial last key tile,
+  lengths, causal, a position table."""
+  rng = np.random.default_rng(4700 + 7 * d + dv)
+  B, L, H = 2, 300, 2
+  lens = np.array([300, 77], dtype=np.int32)
+  mk = lambda dd: rng.standard_normal((B, L, H, dd)).astype(np.float32) * 0.4
+  q, k, v = mk(d), mk(d), mk(dv)
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+  if storage == "bf16":
+    q, k, v = (O.round_bf16(t) for t in (q, k, v))
+    dt = torch.bfloat16
+  else:
+    dt = torch.float32
+  def place(t):
+    x = _dev(t, dt)
+    if storage != "fp32 views":
+      return x
+    # the same values inside a larger buffer: every row starts at an odd element offset
+    buf = torch.zeros((B, L, H, t.shape[-1] + 3), dtype=dt, device="cuda:0")
+    buf[..., 1:1 + t.shape[-1]] = x
+    return buf[..., 1:1 + t.shape[-1]]
+  qd, kd, vd = place(q), place(k), place(v)
+  out = torch.full((B, L, H, dv), float("nan"), dtype=dt, device="cuda:0")
+  a, keep = hstu_ops.build_args(qd, kd, vd, out, n=float(L), alpha=0.25, causal=True, seq_lens=_dev(lens), pos_bias=_dev(pos))
+  variant = hstu_ops.kernel_variant(a)
+  if storage == "bf16" and d == dv and d == 128:
+    assert variant == "hstu_fwd_mfma_bf16"       # (the one case here that the bf16 matrix-core kernel takes)
+  else:
+    assert variant.startswith("hstu_fwd_general")
+  hstu_ops._run(a, keep)
+  torch.cuda.synchronize()
+  got = out.float().cpu().numpy()
+  ref = O.hstu_attention_ref(q, k, v, n=float(L), alpha=0.25, causal=True, seq_lens=lens, pos_tab=pos)
+  tol = FP32_TOL if storage != "bf16" else BF16_TOL
+  assert np.isfinite(got).all()
+  assert np.abs(got - ref).max() <= tol * np.abs(ref).max()
+  assert (got[1, 77:] == 0).all()

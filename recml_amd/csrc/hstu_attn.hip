@@ -27,10 +27,10 @@
 //                        tables; int32 timestamps and their per-tile ranges.
 //   hstu_fwd_general     every option of the op (segment ids, explicit mask,
 //                        sliding window, dense bias, cross lengths, any head
-//                        dim <= 256, fp32 or bf16 storage) in plain fp32 FMA
-//                        arithmetic.  Correctness path for the options the
-//                        MFMA kernel does not cover and the fp32 reference
-//                        configuration.
+//                        dim <= 256, fp32 or bf16 storage, any strides) in
+//                        fp32 arithmetic on the fp32 matrix cores.  The path of
+//                        fp32 callers (the reference's default dtype) and of
+//                        the options the bf16 kernel does not cover.
 //
 // Backward (dq, dk, dv and the gradients of the two bias tables):
 //

@@ -202,6 +202,8 @@ __device__ __forceinline__ void stf(bf16_t* p, float x) { *p = (bf16_t)x; }
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr int GT = 32;       // query rows and keys per tile
 constexpr int GMAXX = 32;    // d_v / 8 accumulators per thread, d_v <= 256
+// floats of the general backward's timestamp-bucket histogram in LDS: one per table entry, a multiple of four
+__host__ __device__ inline int general_hist_len(int ts_nb) { return ts_nb < 0 ? 4 : ((ts_nb + 4) & ~3); }
 
 __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
                                               int b, int h, int i, int j, int* bucket = nullptr) {
@@ -294,6 +296,34 @@ __device__ __forceinline__ float4 general_load4(const bf16_t* row, int c, int d,
   if (c + 2 < d) r.z = (float)row[c + 2];
   if (c + 3 < d) r.w = (float)row[c + 3];
   return r;
+}
+
+// acc += A B^T over the channels: A rows from LDS (`arow` = the lane's row + 2 hh, pitch twice an odd number),
+// B = a register fragment; sixteen channels at a time, their reads ahead of their products, then what is left
+// four at a time (nothing past d4 is read).
+__device__ __forceinline__ void general_dot_rows(floatx16& acc, const float* arow, const float2 (&bf)[32], int d4) {
+#pragma unroll
+  for (int u0 = 0; u0 < 32; u0 += 4) {
+    if (4 * (u0 + 4) <= d4) {
+      float2 a[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) a[u] = *(const float2*)(arow + 4 * (u0 + u));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].x, bf[u0 + u].x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u].y, bf[u0 + u].y, acc, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (4 * (u0 + u) < d4) {
+          const float2 a = *(const float2*)(arow + 4 * (u0 + u));
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bf[u0 + u].x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bf[u0 + u].y, acc, 0, 0, 0);
+        }
+      }
+    }
+  }
 }
 
 // SMALL (head dims up to 128): the wave's Q rows stay in registers instead of LDS, 64 accumulators instead of
@@ -443,6 +473,7 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
     };
     if constexpr (SMALL) {
       // the slack behind a row's channels is read by the logit loop when the head dim is no multiple of 16
+      // (what lies behind the slack is tile data: finite)
       for (int e = tid; e < GT * (qp_ - dq4); e += 256) Ks[(e / (qp_ - dq4)) * qp_ + dq4 + e % (qp_ - dq4)] = 0.f;
     }
     if (kv_begin < kv_end) {
@@ -477,7 +508,7 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
 #pragma unroll
         for (int u0 = 0; u0 < 32; u0 += 4) {
           if (4 * u0 < dq4) {       // (sixteen channels at a time; head dims that are no multiple of 16 read up to 12 floats
-            float2 kk[4];           // of the pitch's slack or of the next row, and multiply them by zeros of Q)
+            float2 kk[4];           // of the pitch's slack or of the rows behind, and multiply them by zeros of Q)
 #pragma unroll
             for (int u = 0; u < 4; ++u) kk[u] = *(const float2*)(krow + 4 * (u0 + u));
 #pragma unroll
@@ -589,7 +620,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_dq(const Params p) {
   float* Vs = Ks + GT * kp;                // [GT][vp_]
   float* Ds = Vs + GT * vp_;               // [GT][GT+1] dS
   float* Hist = Ds + GT * (GT + 1);        // [ts_nb + 1] timestamp-bucket sums of this tile
-  int* Bk = (int*)(Hist + 132);            // [GT][GT] bucket of each pair
+  int* Bk = (int*)(Hist + general_hist_len(p.ts_nb));   // [GT][GT] bucket of each pair
 
   // (head fastest, tile slowest and longest first: see hstu_fwd_general)
   const int h = blockIdx.x, b = blockIdx.y, qt = gridDim.z - 1 - blockIdx.z;
@@ -820,6 +851,368 @@ __global__ __launch_bounds__(256) void hstu_bwd_dkv(const Params p) {
       const int c = ocg + 8 * x;
       if (x < nxk && c < dq) stf(dkp + s.bk + (int64_t)j * p.k_st + c, live ? acck[x] * p.alpha : 0.f);
       if (x < nxv && c < dv) stf(dvp + s.bv + (int64_t)j * p.v_st + c, live ? accv[x] : 0.f);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The general backward on the fp32 matrix cores (head dims up to 128; beyond that the two kernels above).
+// Same products, masks and biases as above; tiles of 32 rows travel through registers into LDS as in
+// hstu_fwd_general, each in up to two layouts: pitch twice an odd number where its rows are the A operand of
+// a product over the channels (two floats per lane and pair of steps), pitch 8 more than a multiple of 32
+// where its rows are read across the channels (A operand of a product over the tile's 32 rows).
+// ---------------------------------------------------------------------------
+
+typedef __attribute__((address_space(3))) float* general_lds_float_ptr;   // (a float atomic on LDS named as such)
+
+// A tile of 32 rows x d channels of a [row][channel] array, rows `row0 ..` of at most `nrows`: eight threads per
+// row, four channels per thread and turn, held in registers between fetch and stage.
+template <typename T, int NG>
+struct GeneralTile {
+  typedef typename std::conditional<sizeof(T) == 4, float4, uint2>::type Raw;
+  Raw raw[NG];
+  static __device__ __forceinline__ float4 widen(const Raw& u) {
+    if constexpr (sizeof(T) == 4) {
+      return u;
+    } else {
+      return float4{__builtin_bit_cast(float, u.x << 16), __builtin_bit_cast(float, u.x & 0xffff0000u),
+                    __builtin_bit_cast(float, u.y << 16), __builtin_bit_cast(float, u.y & 0xffff0000u)};
+    }
+  }
+  static __device__ __forceinline__ Raw narrow(const float4& f) {
+    if constexpr (sizeof(T) == 4) {
+      return f;
+    } else {
+      return uint2{(__builtin_bit_cast(uint32_t, f.x) >> 16) | (__builtin_bit_cast(uint32_t, f.y) & 0xffff0000u),
+                   (__builtin_bit_cast(uint32_t, f.z) >> 16) | (__builtin_bit_cast(uint32_t, f.w) & 0xffff0000u)};
+    }
+  }
+  // fast: whole groups of four can be loaded (aligned base and row stride, d a multiple of four); then the loads
+  // are unconditional (rows past the end re-read the last row) and stage() writes the zeros
+  __device__ __forceinline__ void fetch(const T* base, int64_t row_stride, int row0, int nrows, int d, bool fast, int tid) {
+    const int lr = tid >> 3, lc = (tid & 7) * 4;
+    const int d4 = (d + 3) & ~3;
+    const int ng = (d4 + 31) >> 5;
+    const int j = row0 + lr;
+    const int jc = fast && j >= nrows ? nrows - 1 : j;
+    const T* row = base + (int64_t)jc * row_stride;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const int c = lc + 32 * g;
+      if (g < ng) {
+        if (fast) raw[g] = *(const Raw*)(row + (c < d ? c : d - 4));
+        else raw[g] = narrow(general_load4(row, c, d, j < nrows, false));
+      }
+    }
+  }
+  // into LDS: `by_row` (pitch twice an odd number: 8-byte stores) and / or `by_col` (pitch a multiple of four)
+  __device__ __forceinline__ void stage(int row0, int nrows, int d, bool fast, int tid, float* by_row, int pitch_row, float* by_col,
+                                        int pitch_col) const {
+    const int lr = tid >> 3, lc = (tid & 7) * 4;
+    const int d4 = (d + 3) & ~3;
+    const int ng = (d4 + 31) >> 5;
+    const bool row_ok = row0 + lr < nrows;
+    const float4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const int c = lc + 32 * g;
+      if (g < ng && c < d4) {
+        const float4 t4 = (!fast || (row_ok && c < d)) ? widen(raw[g]) : zero4;
+        if (by_row) {
+          *(float2*)(by_row + lr * pitch_row + c) = float2{t4.x, t4.y};
+          *(float2*)(by_row + lr * pitch_row + c + 2) = float2{t4.z, t4.w};
+        }
+        if (by_col) *(float4*)(by_col + lr * pitch_col + c) = t4;
+      }
+    }
+  }
+};
+
+// The lane's share of row `row` as the B operand of a product over the channels: channels 4u + 2hh and
+// 4u + 2hh + 1 for the pair of steps u; zeros past d or when the row does not exist.
+template <typename T>
+__device__ __forceinline__ void general_row_frag(float2 (&f)[32], const T* row, int d, bool row_ok, int hh) {
+  const int d4 = (d + 3) & ~3;
+#pragma unroll
+  for (int u = 0; u < 32; ++u) {
+    f[u] = float2{0.f, 0.f};
+    if (4 * u < d4 && row_ok) {
+      const int c = 4 * u + 2 * hh;
+      if (c < d) f[u].x = ldf(row + c);
+      if (c + 1 < d) f[u].y = ldf(row + c + 1);
+    }
+  }
+}
+
+// out[x]^T += A^T B over the tile's 32 rows: A = LDS tile read across the channels (`acol` = tile + 4 hh rows + m,
+// pitch 8 more than a multiple of 32), B = the 16 values of an accumulator (row 8g + 4hh + tt, r = 4g + tt).
+template <int NB>
+__device__ __forceinline__ void general_dot_cols(floatx16 (&out)[NB], const float* acol, int pitch, const floatx16& bv, int nblk) {
+#pragma unroll
+  for (int x = 0; x < NB; ++x) {
+    if (x < nblk) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        out[x] = __builtin_amdgcn_mfma_f32_32x32x2f32(acol[(8 * (r >> 2) + (r & 3)) * pitch + 32 * x], bv[r], out[x], 0, 0, 0);
+    }
+  }
+}
+
+// LDS floats of the two kernels (host and device agree through these)
+__host__ __device__ inline int general_bwd_dq_lds(int dq, int dv, bool want_pos, int ts_nb) {
+  return GT * (general_pitch_qk(dq) + general_pitch_v(dq) + general_pitch_qk(dv)) + (want_pos ? 4 * GT * (GT + 1) : 0) + general_hist_len(ts_nb);
+}
+__host__ __device__ inline int general_bwd_dkv_lds(int dq, int dv) {
+  return GT * (general_pitch_qk(dq) + general_pitch_v(dq) + general_pitch_qk(dv) + general_pitch_v(dv));
+}
+
+// dQ and the table gradients: one workgroup per 128 query rows of one (sequence, head), 32 per wave, keys streamed.
+//   S^T = K Q^T, dP^T = V dO^T (A = K / V rows, B = the wave's Q / dO rows in registers), dS^T pointwise,
+//   dQ^T += K^T dS^T (A = K read across the channels, B = dS^T as it leaves the pointwise part).
+template <typename T>
+__global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
+  extern __shared__ __attribute__((aligned(16))) float gsm[];
+  const int dq = p.d_qk, dv = p.d_v;
+  const int dq4 = (dq + 3) & ~3, dv4 = (dv + 3) & ~3;
+  const int pk = general_pitch_qk(dq), pc = general_pitch_v(dq), pv = general_pitch_qk(dv);
+  const bool want_ts = p.dts != nullptr && p.ts_tab != nullptr;
+  const bool want_pos = p.dpos != nullptr && p.pos_tab != nullptr;
+  float* Kr = gsm;                         // [32][pk]  K rows for S^T
+  float* Kc = Kr + GT * pk;                // [32][pc]  K read across the channels for dQ^T
+  float* Vr = Kc + GT * pc;                // [32][pv]  V rows for dP^T
+  float* Hist = Vr + GT * pv;              // [buckets] timestamp-bucket sums of this workgroup
+  float* Ds = Hist + general_hist_len(p.ts_nb);   // [4][32][33] dS of each wave's block, [query][key] (position gradient only)
+
+  const int h = blockIdx.x, b = blockIdx.y, qt = gridDim.z - 1 - blockIdx.z;
+  const Seq s = seq_info(p, b, h);
+  const int q0 = qt * 128;
+  if (q0 >= s.rows) return;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, m = lane & 31, hh = lane >> 5;
+  const T* __restrict__ qp = (const T*)p.q + s.bq;
+  const T* __restrict__ kp_ = (const T*)p.k + s.bk;
+  const T* __restrict__ vp = (const T*)p.v + s.bv;
+  const T* __restrict__ dop = (const T*)p.dout + s.bo;
+  T* __restrict__ dqp = (T*)p.dq + s.bq;
+  const int r0 = q0 + 32 * w, qi = r0 + m;
+  constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
+  const bool kfast = (((uintptr_t)kp_ & VMASK) == 0) && (p.k_st & 3) == 0 && (dq & 3) == 0;
+  const bool vfast = (((uintptr_t)vp & VMASK) == 0) && (p.v_st & 3) == 0 && (dv & 3) == 0;
+
+  constexpr int NB = 4;
+  const int nblk = (dq + 31) >> 5;
+  floatx16 o[NB];
+#pragma unroll
+  for (int x = 0; x < NB; ++x)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[x][r] = 0.f;
+
+  if (q0 < s.n_q) {
+    float2 qf[32], dof[32];
+    general_row_frag(qf, qp + (int64_t)qi * p.q_st, dq, qi < s.n_q, hh);
+    general_row_frag(dof, dop + (int64_t)qi * p.o_st, dv, qi < s.n_q, hh);
+    if (want_ts) for (int e = tid; e <= p.ts_nb; e += 256) Hist[e] = 0.f;
+    int kv_end = s.n_kv;
+    if (p.causal && q0 + 128 < kv_end) kv_end = q0 + 128;
+    if (p.window >= 0 && q0 + 128 + p.window < kv_end) kv_end = q0 + 128 + p.window;
+    int kv_begin = 0;
+    if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
+    GeneralTile<T, 4> kt_, vt_;
+    if (kv_begin < kv_end) {
+      kt_.fetch(kp_, p.k_st, kv_begin, s.n_kv, dq, kfast, tid);
+      vt_.fetch(vp, p.v_st, kv_begin, s.n_kv, dv, vfast, tid);
+    }
+    int hi = s.n_kv - 1, lo = 0;
+    if (p.causal) hi = qi < hi ? qi : hi;
+    if (p.window >= 0) {
+      hi = qi + p.window < hi ? qi + p.window : hi;
+      lo = qi - p.window;
+    }
+    if (qi >= s.n_q) hi = -1;
+    const bool by_pair = p.mask_mode == HSTU_MASK_SEGMENT || p.mask != nullptr;
+    const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
+    float* dsw = Ds + w * (GT * (GT + 1));
+
+    for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
+      __syncthreads();
+      kt_.stage(kv0, s.n_kv, dq, kfast, tid, Kr, pk, Kc, pc);
+      vt_.stage(kv0, s.n_kv, dv, vfast, tid, Vr, pv, nullptr, 0);
+      __syncthreads();
+      if (kv0 + GT < kv_end) {
+        kt_.fetch(kp_, p.k_st, kv0 + GT, s.n_kv, dq, kfast, tid);
+        vt_.fetch(vp, p.v_st, kv0 + GT, s.n_kv, dv, vfast, tid);
+      }
+      bool live = r0 < s.n_q;
+      if (p.causal && kv0 > r0 + 31) live = false;
+      if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
+      if (!live) continue;
+      floatx16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+      general_dot_rows(sacc, Kr + m * pk + 2 * hh, qf, dq4);
+      general_dot_rows(dpacc, Vr + m * pv + 2 * hh, dof, dv4);
+      // lane holds pair (query qi, key kv0 + 8g + 4hh + tt), r = 4g + tt
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+        bool keep = j >= lo && j <= hi;
+        if (by_pair) keep = keep && general_keep(p, s, b, qi, j);
+        float x = p.alpha * sacc[r];
+        int bk = 0;
+        if (biased && keep) x += general_bias(p, s, b, h, qi, j, &bk);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
+        const float ds = keep ? dpacc[r] * sg * (1.0f + x * (1.0f - sg)) * p.inv_n : 0.f;
+        sacc[r] = ds;                      // dS^T in place of S^T
+        if (want_ts && ds != 0.f) __hip_atomic_fetch_add((general_lds_float_ptr)(Hist + bk), ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (want_pos) dsw[m * (GT + 1) + 8 * (r >> 2) + 4 * hh + (r & 3)] = ds;
+      }
+      if (want_pos) {
+        // one sum per diagonal of the wave's 32 x 32 block (the wave's own LDS: its operations run in order)
+        const int dd = lane - (GT - 1);          // key - query inside the block; lane 63 has none
+        if (lane < 2 * GT - 1) {
+          float sum = 0.f;
+          for (int r = 0; r < GT; ++r) {
+            const int c = r + dd;
+            if (c >= 0 && c < GT) sum += dsw[r * (GT + 1) + c];
+          }
+          const int idx = (p.L - 1) + (kv0 - r0) + dd;
+          if (sum != 0.f && idx >= 0 && idx < 2 * p.L - 1)
+            atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, sum);
+        }
+      }
+      general_dot_cols<NB>(o, Kc + (4 * hh) * pc + m, pc, sacc, nblk);
+    }
+    if (want_ts) {
+      __syncthreads();
+      for (int e = tid; e <= p.ts_nb; e += 256)
+        if (Hist[e] != 0.f) atomicAdd(p.dts + (int64_t)(p.ts_heads > 1 ? h : 0) * (p.ts_nb + 1) + e, Hist[e]);
+    }
+  }
+  // dQ^T[channel 32x + 8g + 4hh + tt][query qi]; rows past the sequence are written as zeros
+  if (qi < s.rows) {
+    const bool live_row = qi < s.n_q;
+#pragma unroll
+    for (int x = 0; x < NB; ++x) {
+      if (x < nblk) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c = 32 * x + 8 * (r >> 2) + 4 * hh + (r & 3);
+          if (c < dq) stf(dqp + (int64_t)qi * p.q_st + c, live_row ? o[x][r] * p.alpha : 0.f);
+        }
+      }
+    }
+  }
+}
+
+// dK and dV: one workgroup per 128 keys of one (sequence, head), 32 per wave, query rows streamed 32 at a time.
+//   S = Q K^T, dP = dO V^T (A = Q / dO rows, B = the wave's K / V rows in registers), P and dS pointwise,
+//   dV^T += dO^T P, dK^T += Q^T dS (A = dO / Q read across the channels, B = P / dS as they leave the pointwise part).
+template <typename T>
+__global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
+  extern __shared__ __attribute__((aligned(16))) float gsm[];
+  const int dq = p.d_qk, dv = p.d_v;
+  const int dq4 = (dq + 3) & ~3, dv4 = (dv + 3) & ~3;
+  const int pqr = general_pitch_qk(dq), pqc = general_pitch_v(dq), por = general_pitch_qk(dv), poc = general_pitch_v(dv);
+  float* Qr = gsm;                         // [32][pqr] Q rows for S
+  float* Qc = Qr + GT * pqr;               // [32][pqc] Q read across the channels for dK^T
+  float* Or = Qc + GT * pqc;               // [32][por] dO rows for dP
+  float* Oc = Or + GT * por;               // [32][poc] dO read across the channels for dV^T
+
+  const int h = blockIdx.x, b = blockIdx.y, kt = blockIdx.z;
+  const Seq s = seq_info(p, b, h);
+  const int k0 = kt * 128;
+  const int krows = p.jagged ? s.n_kv : p.Lkv;      // rows of dk / dv that exist
+  if (k0 >= krows) return;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, m = lane & 31, hh = lane >> 5;
+  const T* __restrict__ qp = (const T*)p.q + s.bq;
+  const T* __restrict__ kp_ = (const T*)p.k + s.bk;
+  const T* __restrict__ vp = (const T*)p.v + s.bv;
+  const T* __restrict__ dop = (const T*)p.dout + s.bo;
+  T* __restrict__ dkp = (T*)p.dk + s.bk;
+  T* __restrict__ dvp = (T*)p.dv + s.bv;
+  const int c0 = k0 + 32 * w, kj = c0 + m;          // the wave's first key, this lane's key
+  constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
+  const bool qfast = (((uintptr_t)qp & VMASK) == 0) && (p.q_st & 3) == 0 && (dq & 3) == 0;
+  const bool ofast = (((uintptr_t)dop & VMASK) == 0) && (p.o_st & 3) == 0 && (dv & 3) == 0;
+
+  constexpr int NB = 4;
+  const int nbk = (dq + 31) >> 5, nbv = (dv + 31) >> 5;
+  floatx16 ak[NB], av[NB];
+#pragma unroll
+  for (int x = 0; x < NB; ++x)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { ak[x][r] = 0.f; av[x][r] = 0.f; }
+
+  if (k0 < s.n_kv) {
+    float2 kf[32], vf[32];
+    general_row_frag(kf, kp_ + (int64_t)kj * p.k_st, dq, kj < s.n_kv, hh);
+    general_row_frag(vf, vp + (int64_t)kj * p.v_st, dv, kj < s.n_kv, hh);
+    // query rows that can see these keys
+    int q_begin = 0, q_end = s.n_q;
+    if (p.causal) q_begin = k0;
+    if (p.window >= 0 && k0 - p.window > q_begin) q_begin = k0 - p.window;
+    if (p.window >= 0 && k0 + 128 + p.window < q_end) q_end = k0 + 128 + p.window;
+    q_begin = (q_begin / GT) * GT;
+    GeneralTile<T, 4> qt_, ot_;
+    if (q_begin < q_end) {
+      qt_.fetch(qp, p.q_st, q_begin, s.n_q, dq, qfast, tid);
+      ot_.fetch(dop, p.o_st, q_begin, s.n_q, dv, ofast, tid);
+    }
+    // the query rows this lane's key keeps: lo <= i <= hi
+    int lo = p.causal ? kj : 0, hi = s.n_q - 1;
+    if (p.window >= 0) {
+      lo = kj - p.window > lo ? kj - p.window : lo;
+      hi = kj + p.window < hi ? kj + p.window : hi;
+    }
+    if (kj >= s.n_kv) hi = -1;
+    const bool by_pair = p.mask_mode == HSTU_MASK_SEGMENT || p.mask != nullptr;
+    const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
+
+    for (int i0 = q_begin; i0 < q_end; i0 += GT) {
+      __syncthreads();
+      qt_.stage(i0, s.n_q, dq, qfast, tid, Qr, pqr, Qc, pqc);
+      ot_.stage(i0, s.n_q, dv, ofast, tid, Or, por, Oc, poc);
+      __syncthreads();
+      if (i0 + GT < q_end) {
+        qt_.fetch(qp, p.q_st, i0 + GT, s.n_q, dq, qfast, tid);
+        ot_.fetch(dop, p.o_st, i0 + GT, s.n_q, dv, ofast, tid);
+      }
+      // nothing for a wave whose keys all lie behind these rows (causal) or outside the window
+      bool live = c0 < s.n_kv;
+      if (p.causal && c0 > i0 + 31) live = false;
+      if (p.window >= 0 && (c0 > i0 + 31 + p.window || c0 + 31 + p.window < i0)) live = false;
+      if (!live) continue;
+      floatx16 sacc, dpacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
+      general_dot_rows(sacc, Qr + m * pqr + 2 * hh, kf, dq4);
+      general_dot_rows(dpacc, Or + m * por + 2 * hh, vf, dv4);
+      // MFMA rows are the A operand's rows: lane holds pair (query i0 + 8g + 4hh + tt, key ... ) -- see below
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = i0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+        bool keep = i >= lo && i <= hi;
+        if (by_pair) keep = keep && general_keep(p, s, b, i, kj);
+        float x = p.alpha * sacc[r];
+        if (biased && keep) x += general_bias(p, s, b, h, i, kj);
+        const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
+        const float ds = keep ? dpacc[r] * sg * (1.0f + x * (1.0f - sg)) * p.inv_n : 0.f;
+        sacc[r] = keep ? x * sg * p.inv_n : 0.f;    // P in place of S
+        dpacc[r] = ds;                              // dS in place of dP
+      }
+      general_dot_cols<NB>(av, Oc + (4 * hh) * poc + m, poc, sacc, nbv);
+      general_dot_cols<NB>(ak, Qc + (4 * hh) * pqc + m, pqc, dpacc, nbk);
+    }
+  }
+  if (kj < krows) {
+    const bool live_row = kj < s.n_kv;
+#pragma unroll
+    for (int x = 0; x < NB; ++x) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = 32 * x + 8 * (r >> 2) + 4 * hh + (r & 3);
+        if (x < nbk && c < dq) stf(dkp + (int64_t)kj * p.k_st + c, live_row ? ak[x][r] * p.alpha : 0.f);
+        if (x < nbv && c < dv) stf(dvp + (int64_t)kj * p.v_st + c, live_row ? av[x][r] : 0.f);
+      }
     }
   }
 }
@@ -3667,10 +4060,26 @@ long long mfma_grid(const Params& p) {
   return 8LL * p.n_qtiles * (((long long)p.B * p.H + 7) / 8);
 }
 
+// The general backward: head dims up to 128 on the fp32 matrix cores, larger ones by the FMA kernels.
 template <typename T>
 int launch_bwd(const Params& p, hipStream_t st) {
+  if (p.B > 65535) return fail(HSTU_ERR_SHAPE, "the general backward takes at most 65535 sequences per call, got %d", p.B);
+  if (p.d_qk <= 128 && p.d_v <= 128) {
+    const bool want_pos = p.dpos != nullptr && p.pos_tab != nullptr;
+    const int smem_q = 4 * general_bwd_dq_lds(p.d_qk, p.d_v, want_pos, p.ts_nb), smem_kv = 4 * general_bwd_dkv_lds(p.d_qk, p.d_v);
+    static int granted_q[64], granted_kv[64];
+    if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T>, smem_q, granted_q)) return rc;
+    if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T>, smem_kv, granted_kv)) return rc;
+    hipLaunchKernelGGL(hstu_bwd_dq_mm<T>, dim3(p.H, p.B, (p.L + 127) / 128), dim3(256), smem_q, st, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
+    hipLaunchKernelGGL(hstu_bwd_dkv_mm<T>, dim3(p.H, p.B, (p.Lkv + 127) / 128), dim3(256), smem_kv, st, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
+    return HSTU_OK;
+  }
   const size_t tile = (size_t)GT * p.d_qk + (size_t)GT * p.d_v + (size_t)GT * (p.d_qk + 1) + (size_t)GT * (p.d_v + 1);
-  const size_t smem_q = sizeof(float) * (tile + GT * (GT + 1) + 132 + GT * GT);
+  const size_t smem_q = sizeof(float) * (tile + GT * (GT + 1) + general_hist_len(p.ts_nb) + GT * GT);
   const size_t smem_kv = sizeof(float) * (tile + 2 * GT * (GT + 1));
   static int granted_q[64], granted_kv[64];
   if (int rc = allow_lds((const void*)hstu_bwd_dq<T>, (int)smem_q, granted_q)) return rc;
@@ -3966,6 +4375,9 @@ int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {
   p.dpos = args->dpos_tab; p.dts = args->dts_tab;
   hipStream_t st = (hipStream_t)stream;
   if (bwd_mfma_eligible(args)) return launch_bwd_mfma(args, p, st);
+  // (the general kernels sum the bucket table's gradient in LDS first, one float per entry)
+  if (p.dts && p.ts_tab && p.ts_nb > 4095)
+    return fail(HSTU_ERR_SHAPE, "the gradient of a timestamp table of more than 4096 entries is not supported, got %d", p.ts_nb + 1);
   return f->qk_dtype == HSTU_DTYPE_FP32 ? launch_bwd<float>(p, st) : launch_bwd<bf16_t>(p, st);
 }
 

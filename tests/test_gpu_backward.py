@@ -416,3 +416,40 @@ def test_backward_work_list_over_two_segments_of_sequences(gpu):
   assert variant == ["hstu_bwd_mfma_bf16"]
   for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
     assert _rel(g.float().cpu().numpy(), w) <= 2e-2, nm
+
+
+@pytest.mark.parametrize("d,dv", [(3, 5), (20, 20), (36, 100), (128, 128), (129, 64), (160, 160)])
+@pytest.mark.parametrize("storage", ["fp32", "fp32 views"])
+def test_general_backward_head_dims_and_storage(gpu, d, dv, storage):
+  """The general backward over head dims that are no multiple of 4 or 16, differ between q/k and v, or go beyond
+  128 (those stay on the FMA kernels), with rows that allow 16-byte loads and rows that do not; three tiles of 128
+  rows with a partial last one, lengths, causal, both table biases with their gradients."""
+  rng = np.random.default_rng(5700 + 7 * d + dv)
+  B, L, H = 2, 300, 2
+  lens = np.array([300, 77], dtype=np.int32)
+  mk = lambda dd: rng.standard_normal((B, L, H, dd)).astype(np.float32) * 0.4
+  q, k, v, dout = mk(d), mk(d), mk(dv), mk(dv)
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+  tab = (rng.standard_normal((1, 65)) * 0.3).astype(np.float32)
+  t = 1_700_000_000 + np.cumsum(np.ceil(rng.exponential(3000.0, (B, L))), axis=1).astype(np.int64)
+  def place(x):
+    xd = _dev(x)
+    if storage != "fp32 views":
+      return xd
+    buf = torch.zeros((B, L, H, x.shape[-1] + 3), dtype=torch.float32, device="cuda:0")
+    buf[..., 1:1 + x.shape[-1]] = xd
+    return buf[..., 1:1 + x.shape[-1]]
+  kw = dict(n=float(L), alpha=0.25, causal=True, seq_lens=lens, pos_tab=pos, ts_tab=tab, timestamps=t)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(place(q), place(k), place(v), place(dout), _variant_out=variant, n=float(L), alpha=0.25,
+                                     causal=True, seq_lens=_dev(lens), pos_bias=_dev(pos), ts_bias=_dev(tab), timestamps=_dev(t))
+  torch.cuda.synchronize()
+  assert variant[-1].startswith("hstu_bwd_general"), variant
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    g = g.cpu().numpy()
+    assert g.shape == w.shape and np.isfinite(g).all(), nm
+    assert np.abs(g - w).max() <= 2e-5 * np.abs(w).max(), (nm, np.abs(g - w).max() / np.abs(w).max())
+    assert (g[1, 77:] == 0).all(), nm
+  for nm, g, w in (("dpos", got[3], want[3]), ("dts", got[4], want[4])):
+    assert _rel(g.cpu().numpy().reshape(w.shape), w) <= 2e-5, nm

@@ -133,10 +133,14 @@ class HSTUBlock(torch.nn.Module):
       uqkv = F.silu(uqkv).reshape(B, L, 4, H, hd)
     u, q, k, v = uqkv.unbind(dim=2)
     if attention_mask is not None:
-      if _wants_grad(q, attention_bias):
-        # the reference's calling convention while training: dense mask and bias through plain torch
-        alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
+      # the reference's calling convention: a dense [B, L, L] mask and bias
+      alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
+      if _wants_grad(attention_bias):
+        # a dense bias that is being trained: the one gradient the kernels do not return, through plain torch
         attn = hstu_ops.dense_attention_torch(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
+      elif _wants_grad(q, k, v):
+        # training with the mask (and a constant bias, if any): forward and backward kernels
+        attn = hstu_ops.hstu_attention_autograd(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
       else:
         attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
                                             scaled_pointwise_attn=self.scaled_pointwise_attn, batch=batch)

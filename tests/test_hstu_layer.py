@@ -261,3 +261,44 @@ def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
   for name in want:
     err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
     assert err <= tol, (name, err)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,hd,tol", [(torch.float32, 16, 2e-4), (torch.bfloat16, 64, 6e-2)])
+def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol):
+  """Training a block the way the reference calls it -- a dense [B, L, L] mask and a constant dense bias:
+  the attention's forward and backward kernels take the mask and the bias as they are (no gradient is asked
+  for the bias); against the same block with the attention in plain torch."""
+  from recml_amd import hstu_ops
+  from recml_amd.hstu_layer import HSTUBlock
+  dev = torch.device("cuda:0")
+  B, L, H = 2, 144, 2
+  D = H * hd
+  gen = torch.Generator().manual_seed(6)
+  blk = HSTUBlock(D, H, dtype=dtype, device=dev, generator=gen)
+  blk.requires_grad_(True)
+  x = (torch.randn((B, L, D), generator=gen) * 0.5).to(dev).to(dtype).requires_grad_(True)
+  lens = torch.tensor([144, 50], device=dev)
+  i = torch.arange(L, device=dev)
+  mask = ((i[None, :] <= i[:, None])[None] & (i[None, None, :] < lens[:, None, None]) & (i[None, :, None] < lens[:, None, None]))
+  bias = (torch.randn((B, L, L), generator=gen) * 0.3).to(dev)
+  dout = torch.randn((B, L, D), generator=gen).to(dev).to(dtype)
+
+  def grads(fused):
+    saved = hstu_ops.hstu_attention_autograd
+    if not fused:
+      hstu_ops.hstu_attention_autograd = lambda q, k, v, **kw: hstu_ops.dense_attention_torch(q, k, v, **kw)
+    try:
+      for t in [x, *blk.parameters()]:
+        t.grad = None
+      out = blk(x, attention_mask=mask, attention_bias=bias)
+      (out.float() * dout.float()).sum().backward()
+      return {"x": x.grad.float().clone(), **{n: p.grad.float().clone() for n, p in blk.named_parameters() if p.grad is not None}}
+    finally:
+      hstu_ops.hstu_attention_autograd = saved
+
+  got, want = grads(True), grads(False)
+  assert set(got) == set(want) and "q_kernel" in got and "output_kernel" in got
+  for name in want:
+    err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
+    assert err <= tol, (name, err)

@@ -188,6 +188,8 @@ size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args);
 
 /* Validate `args` and enqueue the forward on `stream` (a hipStream_t passed
  * as void* so that C callers need no HIP headers).  Returns an HstuStatus.
+ * (Calls that the general kernel serves -- fp32 storage, head dims other than
+ * 32 / 64 / 128, unaligned rows -- take at most 65535 sequences.)
  * Replaces recml/core/ops/hstu_ops.py:829-1046 and the dense path of
  * recml/layers/keras/hstu.py:356-390. */
 int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream);
@@ -223,7 +225,9 @@ int hstu_attn_fwd_noalloc(const HstuAttnFwdArgs* args, void* stream);
  * ts_tab that are ACCUMULATED into by atomic adds: the caller zero-fills them
  * (or passes null when the table gradient is not wanted).  Those float atomic
  * adds arrive in no fixed order, so the table gradients may differ in their
- * last bits from run to run; out, dq, dk and dv are the same bits every run.  fp32 or bf16
+ * last bits from run to run; out, dq, dk and dv are the same bits every run.  (Outside
+ * the bf16 matrix-core pair: at most 65535 sequences per call, and a dts_tab of
+ * at most 4096 entries.)  fp32 or bf16
  * storage, every option of the forward, fp32 arithmetic; fp8 q/k is not
  * supported.  bf16 calls that meet the conditions of the
  * matrix-core forward (without a dense mask or bias, and with keys and

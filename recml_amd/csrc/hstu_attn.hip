@@ -39,7 +39,9 @@
 //                        K and V, one per 128 keys streaming Q and dO; both
 //                        recompute the logits; the first also sums the table
 //                        gradients.
-//   hstu_bwd_dq,         every option, fp32 FMA arithmetic.
+//   hstu_bwd_dq_mm,      every option and storage form in fp32 arithmetic on the
+//   hstu_bwd_dkv_mm      fp32 matrix cores, head dims up to 128.
+//   hstu_bwd_dq,         the same by fp32 FMA loops for head dims up to 256.
 //   hstu_bwd_dkv
 //
 // The math follows recml/layers/keras/hstu.py:356-390 (dense formulation),

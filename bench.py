@@ -476,16 +476,18 @@ def bench_backward(args, w, q, k, v, kw, dev):
   mfma = variant[-1] == "hstu_bwd_mfma_bf16"
   peak = PEAK_BF16_TFLOPS if mfma else PEAK_FP32_TFLOPS
   rec = {
-      "metric": "HSTU attn bwd TFLOP/s (unmasked), L=%d bf16" % w.L, "value": flops / (ms * 1e-3) / 1e12,
+      "metric": "HSTU attn bwd TFLOP/s (unmasked), L=%d %s" % (w.L, "fp32" if w.dtype == "fp32" else "bf16"), "value": flops / (ms * 1e-3) / 1e12,
       "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-      "dtype": "bf16" if mfma else "bf16 storage, fp32 arithmetic",
+      "dtype": "bf16" if mfma else ("f32" if w.dtype == "fp32" else "bf16 storage, fp32 arithmetic"),
       "data": "synthetic",
       "config": {"workload": w.name + " backward",
-                 "kernel": "hstu_bwd_dq_mfma + hstu_bwd_dkv_mfma" if mfma else "hstu_bwd_dq + hstu_bwd_dkv"},
+                 "kernel": "hstu_bwd_dq_mfma + hstu_bwd_dkv_mfma" if mfma else
+                           ("hstu_bwd_dq_mm + hstu_bwd_dkv_mm" if w.d <= 128 else "hstu_bwd_dq + hstu_bwd_dkv")},
       "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                    "frac": flops / (ms * 1e-3) / 1e12 / peak, "traffic": None,
-                   "note": ("matrix-core kernels" if mfma else "fp32 FMA kernels") +
+                   "note": ("bf16 matrix-core kernels" if mfma else "general kernels, fp32 arithmetic" +
+                            (" on the fp32 matrix cores" if w.d <= 128 else " by FMA loops")) +
                            "; time covers both kernels, the preparation kernel, the table memsets and the host call"},
   }
   if not args.no_cpu and w.layout == "jagged":
@@ -533,6 +535,9 @@ def main():
   ap.add_argument("--no-cold", dest="cold", action="store_false",
                   help="skip the cold-cache variant (a 1 GiB fill between launches)")
   ap.add_argument("--backward", action="store_true", help="measure the backward pass instead of the forward")
+  ap.add_argument("--fp32", action="store_true",
+                  help="fp32 storage (Keras' default dtype): the general kernels on the fp32 matrix cores; a profiling aid, "
+                       "not the contract's workload")
   ap.add_argument("--no-graph", dest="graph", action="store_false",
                   help="skip the variant that replays the timed calls as one HIP graph")
   ap.add_argument("--one-item-per-workgroup", action="store_true",
@@ -563,6 +568,11 @@ def main():
     return bench_dense(args, dev)
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
+  if args.fp32:
+    if w.dtype == "fp8":
+      raise SystemExit("--fp32 goes with the bf16 workloads")
+    q, k, v = (torch.from_numpy(np.ascontiguousarray(x)).to(dev) for x in (w.q, w.k, w.v))
+    w.dtype = "fp32"
   if args.backward:
     if w.dtype == "fp8":
       raise SystemExit("the backward takes fp32 or bf16 storage")
@@ -656,7 +666,7 @@ def main():
   shared = hstu_ops.AttentionBatch()
   recml_amd.hstu_attention(q, k, v, out=out, batch=shared, **api_kw)
   api_batch_ms = timed(lambda: recml_amd.hstu_attention(q, k, v, out=out, batch=shared, **api_kw), args.steps)
-  assert shared.prepared_calls >= args.steps
+  assert shared.prepared_calls >= args.steps or not call_args.workspace_bytes     # (the general kernel prepares nothing)
 
   # Cold variant: a 1 GiB fill between launches pushes the inputs out of L2 and the memory-side cache.
   cold_ms = None
@@ -679,18 +689,20 @@ def main():
   flops = w.flops
   tflops = flops / (ms_per_step * 1e-3) / 1e12
   achieved = flops / (kernel_ms * 1e-3) / 1e12
-  bytes_alg = w.bytes_moved(2, 1 if w.dtype == "fp8" else None)
+  bytes_alg = w.bytes_moved(4 if w.dtype == "fp32" else 2, 1 if w.dtype == "fp8" else None)
   ai = flops / bytes_alg
   # fp8 q/k: half of the flops (q k^T) run at the fp8 rate, half (P V) at the bf16 rate
   peak = PEAK_BF16_TFLOPS if w.dtype != "fp8" else 1.0 / (0.5 / PEAK_FP8_TFLOPS + 0.5 / PEAK_BF16_TFLOPS)
+  if w.dtype == "fp32":
+    peak = PEAK_FP32_TFLOPS
   capped_peak = min(peak, ai * PEAK_HBM_GBS / 1e3)
 
   rec = {
-      "metric": "HSTU attn fwd TFLOP/s (unmasked), L=%d %s" % (w.L, "fp8" if w.dtype == "fp8" else "bf16"),
+      "metric": "HSTU attn fwd TFLOP/s (unmasked), L=%d %s" % (w.L, {"fp8": "fp8", "fp32": "fp32"}.get(w.dtype, "bf16")),
       "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
       "warmup": args.warmup, "ms_per_step": ms_per_step,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-      "dtype": "fp8 q/k, bf16 v/out" if w.dtype == "fp8" else "bf16", "data": "synthetic",
+      "dtype": {"fp8": "fp8 q/k, bf16 v/out", "fp32": "f32"}.get(w.dtype, "bf16"), "data": "synthetic",
       "config": {"workload": f"{w.name}: B={w.B} max_len={w.L} H={w.H} d={w.d} {w.layout} "
                              f"lens mean {w.seq_lens.mean():.0f} max {w.seq_lens.max()}, causal, "
                              f"pos_bias={'yes' if w.pos_tab is not None else 'no'} "

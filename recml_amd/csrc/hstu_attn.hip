@@ -4410,8 +4410,9 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
   const Params p = make_params(args);
   hipStream_t st = (hipStream_t)stream;
   switch (pick_variant(args)) {
-    case V_GENERAL_F32: return launch_general<float>(p, st);
-    case V_GENERAL_BF16: return launch_general<bf16_t>(p, st);
+    // (the general kernel has nothing to prepare)
+    case V_GENERAL_F32: return (args->flags & HSTU_FWD_PREPARE_ONLY) ? HSTU_OK : launch_general<float>(p, st);
+    case V_GENERAL_BF16: return (args->flags & HSTU_FWD_PREPARE_ONLY) ? HSTU_OK : launch_general<bf16_t>(p, st);
     case V_MFMA_BF16:
     case V_MFMA_FP8: {
       const bool f8 = args->qk_dtype == HSTU_DTYPE_FP8_E4M3FN;

@@ -237,6 +237,51 @@ __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
   return bias;
 }
 
+// The explicit mask's bytes for the 16 pairs (row i, keys j0 + 8g + 4hh .. +3, g < 4) a lane holds after a
+// product with the query row fixed: one 32-bit word per g (byte tt = key j0 + 8g + 4hh + tt).  Row and keys are
+// clamped into the matrix: bytes of pairs outside it are never looked at (their indices drop them).
+__device__ __forceinline__ void general_mask_words(const Params& p, int b, int i, int j0, int hh, uint32_t (&w)[4]) {
+  const uint8_t* mrow = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)(i < p.L - 1 ? i : p.L - 1) * p.Lkv;
+  if ((p.Lkv & 3) == 0 && ((uintptr_t)p.mask & 3) == 0) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int j = j0 + 8 * g + 4 * hh;
+      j = j < p.Lkv - 4 ? j : p.Lkv - 4;
+      w[g] = *(const uint32_t*)(mrow + j);
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      uint32_t v = 0u;
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        int j = j0 + 8 * g + 4 * hh + tt;
+        j = j < p.Lkv - 1 ? j : p.Lkv - 1;
+        v |= (uint32_t)mrow[j] << (8 * tt);
+      }
+      w[g] = v;
+    }
+  }
+}
+// The same for a product with the key fixed: pairs (rows i0 + 8g + 4hh + tt, key j), bytes a row apart.
+__device__ __forceinline__ void general_mask_words_col(const Params& p, int b, int i0, int j, int hh, uint32_t (&w)[4]) {
+  const uint8_t* mcol = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0) + (j < p.Lkv - 1 ? j : p.Lkv - 1);
+  uint8_t v[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    int i = i0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+    i = i < p.L - 1 ? i : p.L - 1;
+    v[r] = mcol[(int64_t)i * p.Lkv];
+  }
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+    w[g] = (uint32_t)v[4 * g] | ((uint32_t)v[4 * g + 1] << 8) | ((uint32_t)v[4 * g + 2] << 16) | ((uint32_t)v[4 * g + 3] << 24);
+}
+// pair (i, j) under the segment ids alone (SEGMENT mode)
+__device__ __forceinline__ bool general_same_segment(const Params& p, int b, int i, int j) {
+  return p.q_seg[(int64_t)b * p.L + i] == p.kv_seg[(int64_t)b * p.Lkv + j];
+}
+
 __device__ __forceinline__ bool general_keep(const Params& p, const Seq& s,
                                              int b, int i, int j) {
   bool keep = (i < s.n_q) && (j < s.n_kv);
@@ -484,6 +529,14 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
     }
 
     for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
+      // nothing for a wave whose rows all lie before these keys (causal) or outside the window
+      bool live = wave_on && r0 < s.n_q;
+      if (p.causal && kv0 > r0 + 31) live = false;
+      if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
+      // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers below; a block they
+      // all drop is left out altogether
+      uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
+      if (live && p.mask) general_mask_words(p, b, qi, kv0, hh, mw);
       __syncthreads();                     // everyone is done with the tile before
       stage(kv0);
       __syncthreads();
@@ -491,10 +544,7 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
       // registers held across it)
       const bool more = kv0 + GT < kv_end;
       if (more) fetch_k(kv0 + GT);
-      // nothing for a wave whose rows all lie before these keys (causal) or outside the window
-      bool live = wave_on && r0 < s.n_q;
-      if (p.causal && kv0 > r0 + 31) live = false;
-      if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
+      if (live && p.mask && __builtin_amdgcn_ballot_w64((mw[0] | mw[1] | mw[2] | mw[3]) != 0u) == 0) live = false;
       if (!live) {
         if (more) fetch_v(kv0 + GT);
         continue;
@@ -549,13 +599,13 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
         lo = qi - p.window;
       }
       if (qi >= s.n_q) hi = -1;
-      const bool by_pair = p.mask_mode == HSTU_MASK_SEGMENT || p.mask != nullptr;
+      const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
       const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
-        bool keep = j >= lo && j <= hi;
-        if (by_pair) keep = keep && general_keep(p, s, b, qi, j);
+        bool keep = j >= lo && j <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
+        if (by_seg) keep = keep && general_same_segment(p, b, qi, j);
         float x = p.alpha * sacc[r];
         if (biased && keep) x += general_bias(p, s, b, h, qi, j);
         // silu(x) = x / (1 + e^-x), by the hardware's exp2 and reciprocal (1 ulp each)
@@ -1030,11 +1080,18 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
       lo = qi - p.window;
     }
     if (qi >= s.n_q) hi = -1;
-    const bool by_pair = p.mask_mode == HSTU_MASK_SEGMENT || p.mask != nullptr;
+    const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
     const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
     float* dsw = Ds + w * (GT * (GT + 1));
 
     for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
+      bool live = r0 < s.n_q;
+      if (p.causal && kv0 > r0 + 31) live = false;
+      if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
+      // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers; a block they all
+      // drop is left out
+      uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
+      if (live && p.mask) general_mask_words(p, b, qi, kv0, hh, mw);
       __syncthreads();
       kt_.stage(kv0, s.n_kv, dq, kfast, tid, Kr, pk, Kc, pc);
       vt_.stage(kv0, s.n_kv, dv, vfast, tid, Vr, pv, nullptr, 0);
@@ -1043,9 +1100,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
         kt_.fetch(kp_, p.k_st, kv0 + GT, s.n_kv, dq, kfast, tid);
         vt_.fetch(vp, p.v_st, kv0 + GT, s.n_kv, dv, vfast, tid);
       }
-      bool live = r0 < s.n_q;
-      if (p.causal && kv0 > r0 + 31) live = false;
-      if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
+      if (live && p.mask && __builtin_amdgcn_ballot_w64((mw[0] | mw[1] | mw[2] | mw[3]) != 0u) == 0) live = false;
       if (!live) continue;
       floatx16 sacc, dpacc;
 #pragma unroll
@@ -1056,8 +1111,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
-        bool keep = j >= lo && j <= hi;
-        if (by_pair) keep = keep && general_keep(p, s, b, qi, j);
+        bool keep = j >= lo && j <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
+        if (by_seg) keep = keep && general_same_segment(p, b, qi, j);
         float x = p.alpha * sacc[r];
         int bk = 0;
         if (biased && keep) x += general_bias(p, s, b, h, qi, j, &bk);
@@ -1166,10 +1221,17 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
       hi = kj + p.window < hi ? kj + p.window : hi;
     }
     if (kj >= s.n_kv) hi = -1;
-    const bool by_pair = p.mask_mode == HSTU_MASK_SEGMENT || p.mask != nullptr;
+    const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
     const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
 
     for (int i0 = q_begin; i0 < q_end; i0 += GT) {
+      // nothing for a wave whose keys all lie behind these rows (causal) or outside the window
+      bool live = c0 < s.n_kv;
+      if (p.causal && c0 > i0 + 31) live = false;
+      if (p.window >= 0 && (c0 > i0 + 31 + p.window || c0 + 31 + p.window < i0)) live = false;
+      // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers
+      uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
+      if (live && p.mask) general_mask_words_col(p, b, i0, kj, hh, mw);
       __syncthreads();
       qt_.stage(i0, s.n_q, dq, qfast, tid, Qr, pqr, Qc, pqc);
       ot_.stage(i0, s.n_q, dv, ofast, tid, Or, por, Oc, poc);
@@ -1178,10 +1240,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
         qt_.fetch(qp, p.q_st, i0 + GT, s.n_q, dq, qfast, tid);
         ot_.fetch(dop, p.o_st, i0 + GT, s.n_q, dv, ofast, tid);
       }
-      // nothing for a wave whose keys all lie behind these rows (causal) or outside the window
-      bool live = c0 < s.n_kv;
-      if (p.causal && c0 > i0 + 31) live = false;
-      if (p.window >= 0 && (c0 > i0 + 31 + p.window || c0 + 31 + p.window < i0)) live = false;
+      if (live && p.mask && __builtin_amdgcn_ballot_w64((mw[0] | mw[1] | mw[2] | mw[3]) != 0u) == 0) live = false;
       if (!live) continue;
       floatx16 sacc, dpacc;
 #pragma unroll
@@ -1192,8 +1251,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int i = i0 + 8 * (r >> 2) + 4 * hh + (r & 3);
-        bool keep = i >= lo && i <= hi;
-        if (by_pair) keep = keep && general_keep(p, s, b, i, kj);
+        bool keep = i >= lo && i <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
+        if (by_seg) keep = keep && general_same_segment(p, b, i, kj);
         float x = p.alpha * sacc[r];
         if (biased && keep) x += general_bias(p, s, b, h, i, kj);
         const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));

@@ -453,3 +453,40 @@ def test_general_backward_head_dims_and_storage(gpu, d, dv, storage):
     assert (g[1, 77:] == 0).all(), nm
   for nm, g, w in (("dpos", got[3], want[3]), ("dts", got[4], want[4])):
     assert _rel(g.cpu().numpy().reshape(w.shape), w) <= 2e-5, nm
+
+
+def test_general_kernels_on_a_jagged_batch(gpu):
+  """fp32 storage in the jagged layout (forward and backward on the fp32 matrix cores): sequences of 0, 1, 129 and
+  300 tokens (empty, one row, one row past a tile, two tiles and a partial one), both table biases and gradients."""
+  rng = np.random.default_rng(5900)
+  H, d, L = 2, 64, 320
+  lens = np.array([300, 0, 1, 129, 64], dtype=np.int32)
+  off = np.zeros(len(lens) + 1, dtype=np.int32)
+  off[1:] = np.cumsum(lens)
+  T = int(off[-1])
+  q, k, v, dout = (rng.standard_normal((T, H, d)).astype(np.float32) * 0.4 for _ in range(4))
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+  tab = (rng.standard_normal((H, 129)) * 0.3).astype(np.float32)
+  ts = np.concatenate([1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, n)).astype(np.int64)) for n in lens])
+  gk = dict(seq_offsets=_dev(off), max_len=L, n=float(L), alpha=0.3, pos_bias=_dev(pos), ts_bias=_dev(tab), timestamps=_dev(ts))
+  out = recml_amd.hstu_attention(_dev(q), _dev(k), _dev(v), **gk).cpu().numpy()
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q), _dev(k), _dev(v), _dev(dout), _variant_out=variant, **gk)
+  torch.cuda.synchronize()
+  assert variant[-1] == "hstu_bwd_general<float>"
+  dpos = np.zeros_like(pos, dtype=np.float64)
+  dts = np.zeros_like(tab, dtype=np.float64)
+  for b, n in enumerate(lens):
+    if n == 0:
+      continue
+    sl = slice(int(off[b]), int(off[b + 1]))
+    kw = dict(n=float(L), alpha=0.3, pos_tab=pos[:, L - n: L + n - 1], ts_tab=tab, timestamps=ts[sl][None])
+    ref = O.hstu_attention_ref(q[sl][None], k[sl][None], v[sl][None], **kw)
+    assert np.abs(out[sl] - ref[0]).max() <= 1e-5 * max(np.abs(ref).max(), 1e-30), b
+    want = O.hstu_attention_bwd_ref(q[sl][None], k[sl][None], v[sl][None], dout[sl][None], **kw)
+    for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+      assert np.abs(g[sl].cpu().numpy() - w[0]).max() <= 2e-5 * max(np.abs(w).max(), 1e-30), (nm, b)
+    dpos[:, L - n: L + n - 1] += want[3]
+    dts += want[4]
+  assert _rel(got[3].cpu().numpy().reshape(dpos.shape), dpos) <= 2e-5
+  assert _rel(got[4].cpu().numpy().reshape(dts.shape), dts) <= 2e-5

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HSTU_ATTN_ABI_VERSION 1
+#define HSTU_ATTN_ABI_VERSION 2
 
 /* Tensor layouts of q, k, v, out. */
 enum HstuLayout {
@@ -248,6 +248,12 @@ typedef struct HstuAttnBwdArgs {
   void* dv;
   float* dpos_tab;
   float* dts_tab;
+  /* Gradient of fwd.dense_bias, fp32, shaped like it ([L, Lkv] or [B, L, Lkv] by
+   * fwd.dense_bias_batched): dS summed over the heads (and over the batch for a
+   * shared bias), ACCUMULATED into by atomic adds like the table gradients (the
+   * caller zero-fills; null = not wanted; needs fwd.dense_bias).  jax's derivative
+   * of recml/layers/keras/hstu.py:373-374. */
+  float* ddense_bias;
 } HstuAttnBwdArgs;
 
 int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream);

@@ -403,7 +403,7 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
                            ts_tab=None, ts_bucket_size=0.301, bucket_law=True,
                            q_segment_ids=None, kv_segment_ids=None,
                            sliding_window_size=None, mask=None, bias=None,
-                           dtype=np.float64):
+                           bias_grad=False, dtype=np.float64):
   """Gradients of sum(out * dout) for hstu_attention_ref, dense, on padded inputs.
 
   The math of the reference's backward kernel (recml/core/ops/hstu_ops.py:461-517):
@@ -412,7 +412,9 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
   extended by the bias terms of the forward: every (i, j) adds dS to the table entry it
   read (position entry (L-1)+j-i, timestamp entry bucket(i, j)), summed over heads when
   the table has one row for all heads.  Returns dq, dk, dv, dpos_tab (or None),
-  dts_tab (or None) with the shapes of the inputs.
+  dts_tab (or None) with the shapes of the inputs; with bias_grad=True also the gradient
+  of the dense `bias` (dS summed over the heads, and over the batch when the bias is
+  shared by it: jax's derivative of recml/layers/keras/hstu.py:373-374), shaped like it.
   """
   q = np.asarray(q, dtype=dtype)
   k = np.asarray(k, dtype=dtype)
@@ -471,6 +473,12 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
     for h in range(H):
       np.add.at(dts[h if tt.shape[0] > 1 else 0], bucket, ds[:, h])
     dts = dts.reshape(np.asarray(ts_tab).shape)
+  if bias_grad:
+    bshape = np.asarray(bias).shape
+    dbias = ds.sum(axis=1)                                                     # [B, L, Lkv]
+    if len(bshape) == 2 or bshape[0] == 1:
+      dbias = dbias.sum(axis=0, keepdims=len(bshape) == 3)
+    return dq, dk, dv, dpos, dts, dbias.reshape(bshape)
   return dq, dk, dv, dpos, dts
 
 

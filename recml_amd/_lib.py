@@ -9,7 +9,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RECML_AMD_LIB") or os.path.join(_HERE, "lib", "libhstu_attn.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 LAYOUT_PADDED, LAYOUT_JAGGED = 0, 1
 DTYPE_FP32, DTYPE_BF16, DTYPE_FP8_E4M3FN = 0, 1, 2
@@ -74,7 +74,7 @@ class HstuAttnBwdArgs(C.Structure):
       ("struct_size", C.c_uint32), ("version", C.c_uint32),
       ("fwd", HstuAttnFwdArgs),
       ("dout", C.c_void_p), ("dq", C.c_void_p), ("dk", C.c_void_p), ("dv", C.c_void_p),
-      ("dpos_tab", C.c_void_p), ("dts_tab", C.c_void_p),
+      ("dpos_tab", C.c_void_p), ("dts_tab", C.c_void_p), ("ddense_bias", C.c_void_p),
   ]
 
 

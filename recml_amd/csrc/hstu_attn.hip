@@ -130,6 +130,7 @@ struct Params {
   void* dv;
   float* dpos;
   float* dts;
+  float* dbias;              // gradient of the dense bias (general backward), or null
   int64_t items_max;         // capacity of the list (sizes the grid)
 };
 
@@ -748,6 +749,13 @@ __global__ __launch_bounds__(256) void hstu_bwd_dq(const Params p) {
         }
       }
       __syncthreads();
+      if (p.dbias) {
+        float* db = p.dbias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0);
+        for (int e = tid; e < GT * GT; e += 256) {
+          const float ds = Ds[(e >> 5) * (GT + 1) + (e & 31)];
+          if (ds != 0.f) atomicAdd(db + (int64_t)(q0 + (e >> 5)) * p.Lkv + kv0 + (e & 31), ds);
+        }
+      }
       // table gradients of this tile: one sum per diagonal (position), one LDS histogram (time)
       if (want_pos && tid < 2 * GT - 1) {
         const int dd = tid - (GT - 1);           // j - i inside the tile
@@ -1119,6 +1127,9 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
         const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
         const float ds = keep ? dpacc[r] * sg * (1.0f + x * (1.0f - sg)) * p.inv_n : 0.f;
         sacc[r] = ds;                      // dS^T in place of S^T
+        // (dense-bias gradient: the heads' workgroups, and the sequences' for a shared bias, add into one matrix)
+        if (p.dbias && ds != 0.f)
+          atomicAdd(p.dbias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)qi * p.Lkv + j, ds);
         if (want_ts && ds != 0.f) __hip_atomic_fetch_add((general_lds_float_ptr)(Hist + bk), ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         if (want_pos) dsw[m * (GT + 1) + 8 * (r >> 2) + 4 * hh + (r & 3)] = ds;
       }
@@ -4434,6 +4445,8 @@ int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {
   Params p = make_params(f);
   p.dout = args->dout; p.dq = args->dq; p.dk = args->dk; p.dv = args->dv;
   p.dpos = args->dpos_tab; p.dts = args->dts_tab;
+  p.dbias = args->ddense_bias;
+  if (p.dbias && !p.dense_bias) return fail(HSTU_ERR_NULL, "ddense_bias needs the forward's dense_bias");
   hipStream_t st = (hipStream_t)stream;
   if (bwd_mfma_eligible(args)) return launch_bwd_mfma(args, p, st);
   // (the general kernels sum the bucket table's gradient in LDS first, one float per entry)

@@ -41,14 +41,9 @@ def _wants_grad(*tensors) -> bool:
 
 def _attention(q, k, v, *, pos_bias=None, ts_bias=None, batch=None, **kw):
   """The attention op, differentiable when anything it reads wants a gradient: through the HIP
-  backward kernels for q, k, v and the bias tables; through plain torch when a dense bias wants one
-  (the kernels return no gradient for it).  `batch`: the per-batch preparation shared by the layers
-  (inference only)."""
-  if _wants_grad(kw.get("bias")):
-    if q.dim() != 4:
-      raise ValueError("a dense bias that requires a gradient needs the padded layout")
-    return hstu_ops.dense_attention_torch(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
-  if _wants_grad(q, k, v, pos_bias, ts_bias):
+  backward kernels for q, k, v, the bias tables and a dense bias.  `batch`: the per-batch preparation
+  shared by the layers (inference only)."""
+  if _wants_grad(q, k, v, pos_bias, ts_bias, kw.get("bias")):
     return hstu_ops.hstu_attention_autograd(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kw)
   return hstu_ops.hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, batch=batch, **kw)
 
@@ -135,11 +130,8 @@ class HSTUBlock(torch.nn.Module):
     if attention_mask is not None:
       # the reference's calling convention: a dense [B, L, L] mask and bias
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
-      if _wants_grad(attention_bias):
-        # a dense bias that is being trained: the one gradient the kernels do not return, through plain torch
-        attn = hstu_ops.dense_attention_torch(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
-      elif _wants_grad(q, k, v):
-        # training with the mask (and a constant bias, if any): forward and backward kernels
+      if _wants_grad(q, k, v, attention_bias):
+        # training: forward and backward kernels, the gradient of a dense bias included
         attn = hstu_ops.hstu_attention_autograd(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
       else:
         attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,

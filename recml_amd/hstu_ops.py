@@ -409,14 +409,16 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
                        timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                        q_segment_ids=None, kv_segment_ids=None,
                        sliding_window_size=None, mask=None, bias=None,
-                       table_grads=True, _variant_out=None):
+                       table_grads=True, bias_grad=False, _variant_out=None):
   """Gradients of sum(hstu_attention(q, k, v, ...) * dout).
 
   Same arguments as hstu_attention (fp32 or bf16; not fp8).  Returns
   (dq, dk, dv, dpos_bias, dts_bias): dq, dk, dv shaped and typed like q, k, v;
   the table gradients fp32 and shaped like the tables (None for a table that
-  was not given, and for both with table_grads=False).  Math of the reference's
-  backward kernel (recml/core/ops/hstu_ops.py:417-548).
+  was not given, and for both with table_grads=False).  With bias_grad=True a
+  sixth value: the gradient of the dense `bias`, fp32, shaped like it (summed
+  over the heads, and over the batch when the bias is shared by it).  Math of
+  the reference's backward kernel (recml/core/ops/hstu_ops.py:417-548).
   """
   for name, t in (("q", q), ("k", k), ("v", v), ("dout", dout)):
     _check_gpu(name, t)
@@ -447,6 +449,12 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   if ts_bias is not None and table_grads:
     dts = torch.zeros((fa.ts_heads, fa.ts_num_buckets + 1), dtype=torch.float32, device=q.device)
     ba.dts_tab = dts.data_ptr()
+  dbias = None
+  if bias_grad:
+    if bias is None:
+      raise ValueError("bias_grad=True needs a dense `bias`")
+    dbias = torch.zeros((fa.B if fa.dense_bias_batched else 1, fa.L, fa.Lkv), dtype=torch.float32, device=q.device)
+    ba.ddense_bias = dbias.data_ptr()
   lib = _lib.load()
   if _variant_out is not None:
     _variant_out.append(lib.hstu_attn_bwd_variant(C.byref(ba)).decode())
@@ -463,6 +471,8 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
     dpos = dpos.reshape(pos_bias.shape)
   if dts is not None:
     dts = dts.reshape(ts_bias.shape)
+  if bias_grad:
+    return dq, dk, dv, dpos, dts, dbias.reshape(bias.shape)
   return dq, dk, dv, dpos, dts
 
 
@@ -484,14 +494,14 @@ def _grad_buffers(q, k, v):
 
 
 class _HstuAttentionFn(torch.autograd.Function):
-  """hstu_attention with gradients for q, k, v and the two bias tables."""
+  """hstu_attention with gradients for q, k, v, the two bias tables and the dense bias."""
 
   @staticmethod
-  def forward(ctx, q, k, v, pos_bias, ts_bias, kwargs):
+  def forward(ctx, q, k, v, pos_bias, ts_bias, bias, kwargs):
     ctx.kwargs = kwargs
-    ctx.save_for_backward(q, k, v, *(t for t in (pos_bias, ts_bias) if t is not None))
-    ctx.has = (pos_bias is not None, ts_bias is not None)
-    return hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, **kwargs)
+    ctx.save_for_backward(q, k, v, *(t for t in (pos_bias, ts_bias, bias) if t is not None))
+    ctx.has = (pos_bias is not None, ts_bias is not None, bias is not None)
+    return hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, bias=bias, **kwargs)
 
   @staticmethod
   def backward(ctx, dout):
@@ -500,26 +510,23 @@ class _HstuAttentionFn(torch.autograd.Function):
     rest = saved[3:]
     pos = rest.pop(0) if ctx.has[0] else None
     ts = rest.pop(0) if ctx.has[1] else None
-    # needs_input_grad follows forward's arguments: q, k, v, pos_bias, ts_bias, kwargs
+    bias = rest.pop(0) if ctx.has[2] else None
+    # needs_input_grad follows forward's arguments: q, k, v, pos_bias, ts_bias, bias, kwargs
     want_tables = (pos is not None and ctx.needs_input_grad[3]) or (ts is not None and ctx.needs_input_grad[4])
-    dq, dk, dv, dpos, dts = hstu_attention_bwd(q, k, v, dout.contiguous(), pos_bias=pos, ts_bias=ts,
-                                               table_grads=want_tables, **ctx.kwargs)
+    want_bias = bias is not None and ctx.needs_input_grad[5]
+    got = hstu_attention_bwd(q, k, v, dout.contiguous(), pos_bias=pos, ts_bias=ts, bias=bias,
+                             table_grads=want_tables, bias_grad=want_bias, **ctx.kwargs)
+    dq, dk, dv, dpos, dts = got[:5]
     cast = lambda g, t: None if g is None else g.to(t.dtype)
-    return dq, dk, dv, cast(dpos, pos) if pos is not None else None, cast(dts, ts) if ts is not None else None, None
+    return (dq, dk, dv, cast(dpos, pos) if pos is not None else None, cast(dts, ts) if ts is not None else None,
+            cast(got[5], bias) if want_bias else None, None)
 
 
-def hstu_attention_autograd(q, k, v, *, pos_bias=None, ts_bias=None, **kwargs):
-  """hstu_attention as a differentiable torch op (gradients for q, k, v, pos_bias, ts_bias).
-
-  A dense `bias` is taken as a constant: the backward kernels return no gradient
-  for it, so one that requires a gradient is refused here rather than silently
-  cut out of the graph (dense_attention_torch differentiates through it).
-  """
-  dense = kwargs.get("bias")
-  if isinstance(dense, torch.Tensor) and dense.requires_grad and torch.is_grad_enabled():
-    raise ValueError("the dense `bias` requires a gradient, which the fused backward does not compute: "
-                     "pass bias tables (pos_bias, ts_bias), or use dense_attention_torch")
-  return _HstuAttentionFn.apply(q, k, v, pos_bias, ts_bias, kwargs)
+def hstu_attention_autograd(q, k, v, *, pos_bias=None, ts_bias=None, bias=None, **kwargs):
+  """hstu_attention as a differentiable torch op: gradients for q, k, v, the bias tables pos_bias
+  and ts_bias, and a dense `bias` (its gradient is dS summed over the heads, and over the batch
+  when the bias is shared by it)."""
+  return _HstuAttentionFn.apply(q, k, v, pos_bias, ts_bias, bias, kwargs)
 
 
 def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=True, pos_bias=None,

@@ -490,3 +490,40 @@ def test_general_kernels_on_a_jagged_batch(gpu):
     dts += want[4]
   assert _rel(got[3].cpu().numpy().reshape(dpos.shape), dpos) <= 2e-5
   assert _rel(got[4].cpu().numpy().reshape(dts.shape), dts) <= 2e-5
+
+
+@pytest.mark.parametrize("d", [32, 160])
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("storage", ["fp32", "bf16"])
+def test_dense_bias_gradient(gpu, d, shared, storage):
+  """The gradient of a dense [B | 1, L, Lkv] bias (dS summed over the heads, and over the batch when shared)
+  from the general backward -- matrix-core kernels at d = 32, FMA kernels at d = 160 -- with an explicit
+  mask, lengths and keys of another length than the queries; dq, dk, dv alongside."""
+  rng = np.random.default_rng(6100 + d + shared)
+  B, L, Lk, H = 3, 150, 170, 2
+  q = rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.4
+  k, v = (rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.4 for _ in range(2))
+  dout = rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.4
+  mask = rng.random((B, L, Lk)) < 0.7
+  bias = (rng.standard_normal((1 if shared else B, L, Lk)) * 0.4).astype(np.float32)
+  tol = 2e-5
+  dt = torch.float32
+  if storage == "bf16":
+    q, k, v, dout = (O.round_bf16(t) for t in (q, k, v, dout))
+    dt = torch.bfloat16
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, n=9.0, alpha=0.3, causal=False, mask=mask, bias=bias, bias_grad=True)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, dt), _dev(k, dt), _dev(v, dt), _dev(dout, dt), n=9.0, alpha=0.3, causal=False,
+                                     mask=_dev(mask), bias=_dev(bias), bias_grad=True, _variant_out=variant)
+  torch.cuda.synchronize()
+  assert variant[-1].startswith("hstu_bwd_general")
+  assert got[5].shape == bias.shape and got[5].dtype == torch.float32
+  assert _rel(got[5].cpu().numpy(), want[5]) <= (tol if storage == "fp32" else 2e-2)
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(g.float().cpu().numpy(), w) <= (tol if storage == "fp32" else 2e-2), nm
+  # through autograd: the same gradient reaches a bias that requires it
+  bt = _dev(bias).requires_grad_(True)
+  out = recml_amd.hstu_attention_autograd(_dev(q, dt), _dev(k, dt), _dev(v, dt), n=9.0, alpha=0.3, causal=False,
+                                          mask=_dev(mask), bias=bt)
+  (out.float() * _dev(dout)).sum().backward()
+  assert _rel(bt.grad.cpu().numpy(), want[5]) <= (tol if storage == "fp32" else 2e-2)

@@ -56,33 +56,55 @@ def test_fused_bias_and_table_gradients(gpu):
     assert float((a - b).abs().max() / b.abs().max()) <= 2e-5, name
 
 
-def test_custom_bucketization_keeps_the_table_gradient():
-  """A custom bucketization function cannot be fused: the module hands the block a dense bias, and the
-  bias weights must still receive their gradient (through the plain torch form of the op), with frozen
-  block weights too.  Runs on the CPU: nothing here needs the HIP library."""
+@pytest.mark.gpu
+def test_custom_bucketization_keeps_the_table_gradient(gpu):
+  """A custom bucketization function cannot be fused as a table: the module hands the block a dense bias, and
+  the bias weights still receive their gradient -- through the attention's backward kernels, which return the
+  gradient of a dense bias -- with frozen block weights too; against the same block with the op in plain torch."""
   import torch
   from recml_amd import hstu_bias, hstu_ops
   from recml_amd.hstu_layer import HSTUBlock
-  torch.manual_seed(0)
-  B, L, D, H = 2, 12, 16, 2
+  dev = torch.device("cuda:0")
+  gen = torch.Generator().manual_seed(0)
+  B, L, D, H = 2, 140, 32, 2
   sqrt_buckets = lambda x: torch.sqrt(x.abs().clamp(1, int(1e9)).double() / 3600.0).to(torch.int64)
-  mod = hstu_bias.RelativeBucketedTimeAndPositionBasedBias(L, num_buckets=16, bucketization_fn=sqrt_buckets)
-  ts = torch.cumsum(torch.randint(1, 20000, (B, L)), dim=1)
-  kw = mod.attention_kwargs(ts)
-  assert set(kw) == {"bias"} and kw["bias"].requires_grad
-  blk = HSTUBlock(D, H)
+  mod = hstu_bias.RelativeBucketedTimeAndPositionBasedBias(L, num_buckets=16, bucketization_fn=sqrt_buckets, device=dev,
+                                                           generator=gen)
+  ts = torch.cumsum(torch.randint(1, 20000, (B, L), generator=gen), dim=1).to(dev)
+  blk = HSTUBlock(D, H, device=dev, generator=gen)
   for p in blk.parameters():
     p.requires_grad_(False)
-  x = torch.randn(B, L, D)
-  out = blk(x, seq_lens=torch.tensor([L, 7]), attention_bias=kw["bias"])
-  out.square().sum().backward()
-  assert mod._ts_w.grad is not None and float(mod._ts_w.grad.abs().max()) > 0
-  assert mod._positional_bias._pos_biases.grad is not None
-  # the fused autograd op refuses a dense bias it could not differentiate instead of dropping it
-  with pytest.raises(ValueError, match="requires a gradient"):
-    hstu_ops.hstu_attention_autograd(x.reshape(B, L, H, D // H), x.reshape(B, L, H, D // H), x.reshape(B, L, H, D // H),
-                                     bias=kw["bias"])
-  # and the torch form equals the dense oracle
+  x = torch.randn((B, L, D), generator=gen).to(dev)
+  lens = torch.tensor([L, 77], device=dev)
+
+  def grads(fused):
+    saved = hstu_ops.hstu_attention_autograd
+    if not fused:
+      hstu_ops.hstu_attention_autograd = lambda q, k, v, **kw: hstu_ops.dense_attention_torch(q, k, v, **kw)
+    try:
+      for p in mod.parameters():
+        p.grad = None
+      kw = mod.attention_kwargs(ts)
+      assert set(kw) == {"bias"} and kw["bias"].requires_grad
+      out = blk(x, seq_lens=lens, attention_bias=kw["bias"])
+      out.square().sum().backward()
+      return mod._ts_w.grad.clone(), mod._positional_bias._pos_biases.grad.clone()
+    finally:
+      hstu_ops.hstu_attention_autograd = saved
+
+  got, want = grads(True), grads(False)
+  for g, w in zip(got, want):
+    assert float(w.abs().max()) > 0
+    assert float((g - w).abs().max() / w.abs().max()) <= 2e-4
+
+
+def test_dense_attention_in_plain_torch_equals_the_oracle():
+  import torch
+  from recml_amd import hstu_bias, hstu_ops
+  B, L, H = 2, 12, 2
+  torch.manual_seed(0)
+  mod = hstu_bias.RelativeBucketedTimeAndPositionBasedBias(L, num_buckets=16)
+  ts = torch.cumsum(torch.randint(1, 20000, (B, L)), dim=1)
   from oracle import hstu_oracle as O
   q, k, v = (torch.randn(B, L, H, 8) for _ in range(3))
   lens = np.array([L, 7])

@@ -378,7 +378,7 @@ def _fd_grad(f, x, eps=1e-6):
   return g
 
 
-@pytest.mark.parametrize("case", ["lengths_bias", "segments_window", "full_mask_dense_bias"])
+@pytest.mark.parametrize("case", ["lengths_bias", "segments_window", "full_mask_dense_bias", "shared_dense_bias"])
 def test_backward_oracle_against_finite_differences(case):
   rng = np.random.default_rng(11)
   B, L, H, d, dv = 2, 6, 2, 4, 3
@@ -397,9 +397,16 @@ def test_backward_oracle_against_finite_differences(case):
     kw.update(q_segment_ids=seg, kv_segment_ids=seg, sliding_window_size=2, pos_tab=pos)
   else:
     m = rng.random((B, L, L)) > 0.3
-    kw.update(causal=False, mask=m, bias=rng.standard_normal((B, L, L)))
+    kw.update(causal=case == "shared_dense_bias", mask=m,
+              bias=rng.standard_normal((B, L, L) if case == "full_mask_dense_bias" else (1, L, L)))
   loss = lambda: float((O.hstu_attention_ref(q, k, v, **kw) * dout).sum())
-  dq, dk, dvv, dpos, dts = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  if "bias" in kw:
+    dq, dk, dvv, dpos, dts, dbias = O.hstu_attention_bwd_ref(q, k, v, dout, bias_grad=True, **kw)
+    fd = _fd_grad(loss, kw["bias"])
+    assert dbias.shape == kw["bias"].shape and np.abs(fd - dbias).max() <= 1e-7 * max(1.0, np.abs(fd).max())
+    assert np.abs(dbias).max() > 0
+  else:
+    dq, dk, dvv, dpos, dts = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
   for name, x, g in (("q", q, dq), ("k", k, dk), ("v", v, dvv)):
     fd = _fd_grad(loss, x)
     assert np.abs(fd - g).max() <= 1e-7 * max(1.0, np.abs(fd).max()), name

@@ -12,8 +12,10 @@ and for callers that want the dense form.  The fast path never builds it:
 `attention_kwargs(timestamps)` hands the tables themselves to
 `recml_amd.hstu_attention` / `hstu_attention_autograd`, which fuse the
 gathers into the kernel and return the table gradients.  A custom
-`bucketization_fn` cannot be fused (the kernel implements the default law);
-`attention_kwargs` then falls back to the dense bias.
+`bucketization_fn` cannot be fused as a table (the kernels implement the
+default law); `attention_kwargs` then hands over the dense bias, which the
+kernels take as it is and whose gradient their backward returns, so the
+weights behind it train all the same.
 """
 
 from __future__ import annotations

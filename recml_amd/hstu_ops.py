@@ -534,8 +534,8 @@ def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=T
                           sliding_window_size=None):
   """The op in plain torch on padded [B, L, H, d] tensors (recml/layers/keras/hstu.py:356-390 with the
   bias tables expanded): materialises [B, H, L, L], differentiable through everything it reads, any
-  device.  The slow path for what the fused backward cannot differentiate (a dense bias that requires
-  a gradient, e.g. from a custom bucketization function); not used otherwise."""
+  device.  A plain statement of the op for tests and comparisons: no code path of the package calls it
+  (the backward kernels return every gradient, the dense bias's included)."""
   from recml_amd.hstu_bias import default_bucketization
   B, L, H, d = q.shape
   Lkv = k.shape[1]

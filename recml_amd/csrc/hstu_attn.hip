@@ -111,7 +111,6 @@ struct Params {
   // workgroup that arrives last at the tile's counter sums them and writes the rows.
   int32_t split_cap;         // chunk slots of the partial buffer (per head)
   int32_t n_slots;           // workgroups that run at once per XCD (what the split decision balances for)
-  int32_t g_rows;            // general forward: query rows per workgroup
   const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
@@ -314,7 +313,6 @@ __device__ __forceinline__ bool general_keep(const Params& p, const Seq& s,
 // lie 32 banks apart).
 __host__ __device__ inline int general_pitch_qk(int d) { const int d4 = (d + 3) & ~3; return ((d4 >> 1) & 1) ? d4 : d4 + 2; }
 __host__ __device__ inline int general_pitch_v(int d) { return ((d + 31) & ~31) + 8; }
-constexpr int GMAXB = 8;     // 32-channel blocks of the output, d_v <= 256
 
 // Four consecutive elements of a row as floats, zeros where the row or the column is out of range; one
 // 16-byte (fp32) or 8-byte (bf16) load when the caller says the address is aligned for it.
@@ -374,20 +372,20 @@ __device__ __forceinline__ void general_dot_rows(floatx16& acc, const float* aro
   }
 }
 
-// SMALL (head dims up to 128): the wave's Q rows stay in registers instead of LDS, 64 accumulators instead of
-// 128: two waves per SIMD and 34 KB of LDS, several workgroups per CU, so that one workgroup's loads, barriers
-// and pointwise work run under another's products.
-template <typename T, bool SMALL>
-__global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Params p) {
+// DMAX (128 or 256): the head dims the instance holds.  The wave's Q row shares live in DMAX / 2 registers and
+// its output in DMAX / 2 accumulators: up to 128, 255 registers in all and two waves per SIMD, so that one
+// workgroup's loads, barriers and pointwise work run under another's products; up to 256, one wave per SIMD.
+template <typename T, int DMAX>
+__global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(const Params p) {
   extern __shared__ __attribute__((aligned(16))) float gsm[];
-  constexpr int NB = SMALL ? 4 : GMAXB;    // 32-channel blocks of the output
+  constexpr int NB = DMAX / 32;            // 32-channel blocks of the output
+  constexpr int NU = DMAX / 4;             // pairs of steps of a product over the channels
+  constexpr int GQ = 128;                  // query rows of a workgroup
   const int dq = p.d_qk, dv = p.d_v;
-  const int GQ = p.g_rows;                 // query rows of this workgroup: 128, or fewer when LDS is short
   const int dq4 = (dq + 3) & ~3;
   const int qp_ = general_pitch_qk(dq), vp_ = general_pitch_v(dv);
   const int nblk = (dv + 31) >> 5;
-  float* Qs = gsm;                         // [GQ][qp_] (not SMALL)
-  float* Ks = Qs + (SMALL ? 0 : GQ * qp_); // [32][qp_]
+  float* Ks = gsm;                         // [32][qp_]
   float* Vs = Ks + GT * qp_;               // [32][vp_]
 
   // Workgroups are handed to the eight XCDs in turn by their linear index: with the head fastest and the query
@@ -403,14 +401,12 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
   const T* __restrict__ kp_ = (const T*)p.k;
   const T* __restrict__ vp = (const T*)p.v;
   T* __restrict__ op = (T*)p.out;
-  const bool wave_on = 32 * w < GQ;        // waves beyond the tile's rows only help with the loads
   const int r0 = q0 + 32 * w;
   const int qi = r0 + m;                   // this lane's query row
   // whole groups of four elements can be fetched by one load when bases and row strides allow
   constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
   const bool kvec = (((uintptr_t)(kp_ + s.bk) & VMASK) == 0) && (p.k_st & 3) == 0;
   const bool vvec = (((uintptr_t)(vp + s.bv) & VMASK) == 0) && (p.v_st & 3) == 0;
-  const bool qvec = (((uintptr_t)(qp + s.bq) & VMASK) == 0) && (p.q_st & 3) == 0;
 
   floatx16 o[NB];
 #pragma unroll
@@ -421,27 +417,17 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
   if (q0 < s.n_q) {
     // tiles are brought by eight threads per row, four channels per thread and turn
     const int lr = tid >> 3, lc = (tid & 7) * 4;
-    // SMALL: the lane's share of its query row, channels 4u + 2hh and 4u + 2hh + 1 for the pair of steps u
-    float2 qf[SMALL ? 32 : 1];
-    if constexpr (SMALL) {
+    // the lane's share of its query row: channels 4u + 2hh and 4u + 2hh + 1 for the pair of steps u
+    float2 qf[NU];
+    {
       const T* qrow_g = qp + s.bq + (int64_t)qi * p.q_st;
 #pragma unroll
-      for (int u = 0; u < 32; ++u) {
+      for (int u = 0; u < NU; ++u) {
         qf[u] = float2{0.f, 0.f};
         if (4 * u < dq4 && qi < s.n_q) {
           const int c = 4 * u + 2 * hh;
           if (c < dq) qf[u].x = ldf(qrow_g + c);
           if (c + 1 < dq) qf[u].y = ldf(qrow_g + c + 1);
-        }
-      }
-    } else {
-      for (int r = lr; r < GQ; r += 32) {
-        const int i = q0 + r;
-        for (int c = lc; c < dq4; c += 32) {
-          // (rows of Q and K start on 8-byte, not 16-byte boundaries: two stores)
-          const float4 t4 = general_load4(qp + s.bq + (int64_t)i * p.q_st, c, dq, i < s.n_q, qvec);
-          *(float2*)(Qs + r * qp_ + c) = float2{t4.x, t4.y};
-          *(float2*)(Qs + r * qp_ + c + 2) = float2{t4.z, t4.w};
         }
       }
     }
@@ -451,12 +437,12 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
     int kv_begin = 0;
     if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
     const int vcols = nblk * 32;
-    // The next tile travels in registers while this one is computed on: up to 8 + 8 groups of four per thread
-    // (head dims up to 256).  When bases and strides allow whole groups and the head dims are multiples of four,
-    // the loads are unconditional (rows past the sequence re-read its last key, columns past the head dim the
-    // last group) and what must be zero is zeroed on the way into LDS: nothing then uses a loaded value before
-    // the tile is staged, and the loads stay in flight behind the products.  Otherwise element by element.
-    constexpr int NG = SMALL ? 4 : 8;
+    // The next tile travels in registers while this one is computed on.  When bases and strides allow whole
+    // groups and the head dims are multiples of four, the loads are unconditional (rows past the sequence
+    // re-read its last key, columns past the head dim the last group) and what must be zero is zeroed on the way
+    // into LDS: nothing then uses a loaded value before the tile is staged, and the loads stay in flight behind
+    // the products.  Otherwise element by element (bf16 elements packed again: nothing is lost).
+    constexpr int NG = DMAX / 32;
     typedef typename std::conditional<sizeof(T) == 4, float4, uint2>::type Raw;
     const bool fast = kvec && vvec && (dq & 3) == 0 && (dv & 3) == 0;
     const int ngk = (dq4 + 31) >> 5, ngv = (vcols + 31) >> 5;
@@ -469,7 +455,6 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
                       __builtin_bit_cast(float, u.y << 16), __builtin_bit_cast(float, u.y & 0xffff0000u)};
       }
     };
-    // (the element-by-element path leaves the same registers: bf16 elements packed again, nothing is lost)
     auto narrow = [](const float4& f) -> Raw {
       if constexpr (sizeof(T) == 4) {
         return f;
@@ -512,18 +497,16 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
         const int c = lc + 32 * g;
         if (g < ngk && c < dq4) {
           const float4 t4 = (!fast || (row_ok && c < dq)) ? widen(kraw[g]) : zero4;
-          // (rows of Q and K start on 8-byte, not 16-byte boundaries: two stores)
+          // (rows of K start on 8-byte, not 16-byte boundaries: two stores)
           *(float2*)(Ks + lr * qp_ + c) = float2{t4.x, t4.y};
           *(float2*)(Ks + lr * qp_ + c + 2) = float2{t4.z, t4.w};
         }
         if (g < ngv && c < vcols) *(float4*)(Vs + lr * vp_ + c) = (!fast || (row_ok && c < dv)) ? widen(vraw[g]) : zero4;
       }
     };
-    if constexpr (SMALL) {
-      // the slack behind a row's channels is read by the logit loop when the head dim is no multiple of 16
-      // (what lies behind the slack is tile data: finite)
-      for (int e = tid; e < GT * (qp_ - dq4); e += 256) Ks[(e / (qp_ - dq4)) * qp_ + dq4 + e % (qp_ - dq4)] = 0.f;
-    }
+    // the slack behind a row's channels is read by the logit loop when the head dim is no multiple of 16
+    // (what lies behind the slack is tile data: finite)
+    for (int e = tid; e < GT * (qp_ - dq4); e += 256) Ks[(e / (qp_ - dq4)) * qp_ + dq4 + e % (qp_ - dq4)] = 0.f;
     if (kv_begin < kv_end) {
       fetch_k(kv_begin);
       fetch_v(kv_begin);
@@ -531,7 +514,7 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
 
     for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
       // nothing for a wave whose rows all lie before these keys (causal) or outside the window
-      bool live = wave_on && r0 < s.n_q;
+      bool live = r0 < s.n_q;
       if (p.causal && kv0 > r0 + 31) live = false;
       if (p.window >= 0 && (kv0 > r0 + 31 + p.window || kv0 + 31 + p.window < r0)) live = false;
       // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers below; a block they
@@ -554,45 +537,21 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
 #pragma unroll
       for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
       const float* krow = Ks + m * qp_ + 2 * hh;
-      const float* qrow = Qs + (32 * w + m) * qp_ + 2 * hh;
-      // (sixteen channels at a time, their eight reads ahead of the eight products)
-      int c = 0;
-      if constexpr (SMALL) {
 #pragma unroll
-        for (int u0 = 0; u0 < 32; u0 += 4) {
-          if (4 * u0 < dq4) {       // (sixteen channels at a time; head dims that are no multiple of 16 read up to 12 floats
-            float2 kk[4];           // of the pitch's slack or of the rows behind, and multiply them by zeros of Q)
+      for (int u0 = 0; u0 < NU; u0 += 4) {
+        if (4 * u0 < dq4) {       // (sixteen channels at a time; head dims that are no multiple of 16 read up to 12 floats
+          float2 kk[4];           // of the pitch's slack or of the rows behind, and multiply them by zeros of Q)
 #pragma unroll
-            for (int u = 0; u < 4; ++u) kk[u] = *(const float2*)(krow + 4 * (u0 + u));
+          for (int u = 0; u < 4; ++u) kk[u] = *(const float2*)(krow + 4 * (u0 + u));
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].x, qf[u0 + u].x, sacc, 0, 0, 0);
-              sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].y, qf[u0 + u].y, sacc, 0, 0, 0);
-            }
+          for (int u = 0; u < 4; ++u) {
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].x, qf[u0 + u].x, sacc, 0, 0, 0);
+            sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].y, qf[u0 + u].y, sacc, 0, 0, 0);
           }
         }
-        c = dq4;
-      }
-      for (; c + 16 <= dq4; c += 16) {
-        float2 kk[4], qq[4];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          kk[u] = *(const float2*)(krow + c + 4 * u);
-          qq[u] = *(const float2*)(qrow + c + 4 * u);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].x, qq[u].x, sacc, 0, 0, 0);
-          sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk[u].y, qq[u].y, sacc, 0, 0, 0);
-        }
-      }
-      for (; c < dq4; c += 4) {
-        const float2 kk = *(const float2*)(krow + c), qq = *(const float2*)(qrow + c);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.x, qq.x, sacc, 0, 0, 0);
-        sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(kk.y, qq.y, sacc, 0, 0, 0);
       }
       // lane holds S^T[key kv0 + 8g + 4hh + tt][query qi], r = 4g + tt.  The index masks are two bounds per
-      // lane; segment ids, an explicit mask and the biases go through the per-pair helpers only when present.
+      // lane; segment ids and the biases go through the per-pair helpers only when present.
       int hi = s.n_kv - 1, lo = 0;
       if (p.causal) hi = qi < hi ? qi : hi;
       if (p.window >= 0) {
@@ -613,7 +572,6 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
         const float val = x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
         sacc[r] = keep ? val : 0.f;      // P^T in place of S^T
       }
-      // (key by key across the output blocks: consecutive products go to different accumulators)
       if (more) fetch_v(kv0 + GT);
       const float* vcol = Vs + (4 * hh) * vp_ + m;
 #pragma unroll
@@ -627,7 +585,7 @@ __global__ __launch_bounds__(256, SMALL ? 2 : 1) void hstu_fwd_general(const Par
     }
   }
   // O^T[channel 32x + 8g + 4hh + tt][query qi]; rows past the sequence are written as exact zeros (padded layout)
-  if (wave_on && qi < s.rows) {
+  if (qi < s.rows) {
     const bool live_row = qi < s.n_q;
 #pragma unroll
     for (int x = 0; x < NB; ++x) {
@@ -4092,27 +4050,18 @@ int allow_lds(const void* fn, int bytes, int* granted /* [kMaxDev] */) {
 }
 
 template <typename T>
-int launch_general(const Params& p_in, hipStream_t st) {
-  Params p = p_in;
+int launch_general(const Params& p, hipStream_t st) {
   const bool small = p.d_qk <= 128 && p.d_v <= 128;
-  // 128 query rows per workgroup; with head dims beyond 128 fewer where their fp32 rows would not fit the LDS
-  // beside the K and V tiles
-  auto lds_bytes = [&](int rows) {
-    return sizeof(float) * ((size_t)((small ? 0 : rows) + GT) * general_pitch_qk(p.d_qk) + (size_t)GT * general_pitch_v(p.d_v));
-  };
-  p.g_rows = 128;
-  while (p.g_rows > 32 && lds_bytes(p.g_rows) > 150 * 1024) p.g_rows >>= 1;
-  if (p.L < p.g_rows) p.g_rows = p.L <= 32 ? 32 : (p.L <= 64 ? 64 : 128);
-  const size_t smem = lds_bytes(p.g_rows);
-  if (smem > 160 * 1024) return fail(HSTU_ERR_SHAPE, "head dims %d / %d are beyond the general kernel's LDS", p.d_qk, p.d_v);
+  if (p.B > 65535 || (p.L + 127) / 128 > 65535)
+    return fail(HSTU_ERR_SHAPE, "the general kernel takes at most 65535 sequences and 65535 tiles of 128 rows per call (B = %d, L = %d)", p.B, p.L);
+  const size_t smem = sizeof(float) * ((size_t)GT * general_pitch_qk(p.d_qk) + (size_t)GT * general_pitch_v(p.d_v));
   static int granted_small[64], granted_large[64];
-  if (int rc = small ? allow_lds((const void*)hstu_fwd_general<T, true>, (int)smem, granted_small)
-                     : allow_lds((const void*)hstu_fwd_general<T, false>, (int)smem, granted_large)) return rc;
+  if (int rc = small ? allow_lds((const void*)hstu_fwd_general<T, 128>, (int)smem, granted_small)
+                     : allow_lds((const void*)hstu_fwd_general<T, 256>, (int)smem, granted_large)) return rc;
   hipError_t e;
-  if (p.B > 65535) return fail(HSTU_ERR_SHAPE, "the general kernel takes at most 65535 sequences per call, got %d", p.B);
-  dim3 grid(p.H, p.B, (p.L + p.g_rows - 1) / p.g_rows);
-  if (small) hipLaunchKernelGGL((hstu_fwd_general<T, true>), grid, dim3(256), smem, st, p);
-  else hipLaunchKernelGGL((hstu_fwd_general<T, false>), grid, dim3(256), smem, st, p);
+  dim3 grid(p.H, p.B, (p.L + 127) / 128);
+  if (small) hipLaunchKernelGGL((hstu_fwd_general<T, 128>), grid, dim3(256), smem, st, p);
+  else hipLaunchKernelGGL((hstu_fwd_general<T, 256>), grid, dim3(256), smem, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "general kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;

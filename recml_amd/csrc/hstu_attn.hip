@@ -207,8 +207,9 @@ constexpr int GMAXX = 32;    // d_v / 8 accumulators per thread, d_v <= 256
 // floats of the general backward's timestamp-bucket histogram in LDS: one per table entry, a multiple of four
 __host__ __device__ inline int general_hist_len(int ts_nb) { return ts_nb < 0 ? 4 : ((ts_nb + 4) & ~3); }
 
-__device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
-                                              int b, int h, int i, int j, int* bucket = nullptr) {
+// the table biases of pair (i, j): position and timestamp
+__device__ __forceinline__ float general_table_bias(const Params& p, const Seq& s,
+                                                    int b, int h, int i, int j, int* bucket = nullptr) {
   float bias = 0.f;
   if (p.pos_tab) {
     int hh = p.pos_heads > 1 ? h : 0;
@@ -230,6 +231,12 @@ __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
     int hh = p.ts_heads > 1 ? h : 0;
     bias += p.ts_tab[(int64_t)hh * (p.ts_nb + 1) + bk];
   }
+  return bias;
+}
+// every bias of pair (i, j)
+__device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
+                                              int b, int h, int i, int j, int* bucket = nullptr) {
+  float bias = general_table_bias(p, s, b, h, i, j, bucket);
   if (p.dense_bias) {
     int64_t o = p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0;
     bias += p.dense_bias[o + (int64_t)i * p.Lkv + j];
@@ -276,6 +283,34 @@ __device__ __forceinline__ void general_mask_words_col(const Params& p, int b, i
 #pragma unroll
   for (int g = 0; g < 4; ++g)
     w[g] = (uint32_t)v[4 * g] | ((uint32_t)v[4 * g + 1] << 8) | ((uint32_t)v[4 * g + 2] << 16) | ((uint32_t)v[4 * g + 3] << 24);
+}
+// The dense bias of the same 16 pairs (query row fixed / key fixed), fetched together ahead of their use: four
+// 16-byte loads where the rows allow, else one load per pair; indices clamped into the matrix like the mask's.
+__device__ __forceinline__ void general_dense_row(const Params& p, int b, int i, int j0, int hh, float (&v)[16]) {
+  const float* row = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)(i < p.L - 1 ? i : p.L - 1) * p.Lkv;
+  if ((p.Lkv & 3) == 0 && ((uintptr_t)p.dense_bias & 15) == 0) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      int j = j0 + 8 * g + 4 * hh;
+      j = j < p.Lkv - 4 ? j : p.Lkv - 4;
+      const float4 t4 = *(const float4*)(row + j);
+      v[4 * g] = t4.x; v[4 * g + 1] = t4.y; v[4 * g + 2] = t4.z; v[4 * g + 3] = t4.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int j = j0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+      v[r] = row[j < p.Lkv - 1 ? j : p.Lkv - 1];
+    }
+  }
+}
+__device__ __forceinline__ void general_dense_col(const Params& p, int b, int i0, int j, int hh, float (&v)[16]) {
+  const float* col = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (j < p.Lkv - 1 ? j : p.Lkv - 1);
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    int i = i0 + 8 * (r >> 2) + 4 * hh + (r & 3);
+    v[r] = col[(int64_t)(i < p.L - 1 ? i : p.L - 1) * p.Lkv];
+  }
 }
 // pair (i, j) under the segment ids alone (SEGMENT mode)
 __device__ __forceinline__ bool general_same_segment(const Params& p, int b, int i, int j) {
@@ -1047,7 +1082,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
     }
     if (qi >= s.n_q) hi = -1;
     const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
-    const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
+    const bool tabled = p.pos_tab != nullptr || p.ts_tab != nullptr;
     float* dsw = Ds + w * (GT * (GT + 1));
 
     for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
@@ -1058,6 +1093,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
       // drop is left out
       uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
       if (live && p.mask) general_mask_words(p, b, qi, kv0, hh, mw);
+      float db[16];
+      if (live && p.dense_bias) general_dense_row(p, b, qi, kv0, hh, db);
       __syncthreads();
       kt_.stage(kv0, s.n_kv, dq, kfast, tid, Kr, pk, Kc, pc);
       vt_.stage(kv0, s.n_kv, dv, vfast, tid, Vr, pv, nullptr, 0);
@@ -1081,7 +1118,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
         if (by_seg) keep = keep && general_same_segment(p, b, qi, j);
         float x = p.alpha * sacc[r];
         int bk = 0;
-        if (biased && keep) x += general_bias(p, s, b, h, qi, j, &bk);
+        if (tabled && keep) x += general_table_bias(p, s, b, h, qi, j, &bk);
+        if (p.dense_bias) x += db[r];
         const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
         const float ds = keep ? dpacc[r] * sg * (1.0f + x * (1.0f - sg)) * p.inv_n : 0.f;
         sacc[r] = ds;                      // dS^T in place of S^T
@@ -1191,7 +1229,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
     }
     if (kj >= s.n_kv) hi = -1;
     const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
-    const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
+    const bool tabled = p.pos_tab != nullptr || p.ts_tab != nullptr;
 
     for (int i0 = q_begin; i0 < q_end; i0 += GT) {
       // nothing for a wave whose keys all lie behind these rows (causal) or outside the window
@@ -1201,6 +1239,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
       // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers
       uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
       if (live && p.mask) general_mask_words_col(p, b, i0, kj, hh, mw);
+      float db[16];
+      if (live && p.dense_bias) general_dense_col(p, b, i0, kj, hh, db);
       __syncthreads();
       qt_.stage(i0, s.n_q, dq, qfast, tid, Qr, pqr, Qc, pqc);
       ot_.stage(i0, s.n_q, dv, ofast, tid, Or, por, Oc, poc);
@@ -1223,7 +1263,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
         bool keep = i >= lo && i <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
         if (by_seg) keep = keep && general_same_segment(p, b, i, kj);
         float x = p.alpha * sacc[r];
-        if (biased && keep) x += general_bias(p, s, b, h, i, kj);
+        if (tabled && keep) x += general_table_bias(p, s, b, h, i, kj);
+        if (p.dense_bias) x += db[r];
         const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
         const float ds = keep ? dpacc[r] * sg * (1.0f + x * (1.0f - sg)) * p.inv_n : 0.f;
         sacc[r] = keep ? x * sg * p.inv_n : 0.f;    // P in place of S

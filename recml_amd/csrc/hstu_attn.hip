@@ -556,6 +556,12 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
       // all drop is left out altogether
       uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
       if (live && p.mask) general_mask_words(p, b, qi, kv0, hh, mw);
+      // (the block's dense-bias values likewise, where there are registers for them: one wave per SIMD)
+      constexpr bool DENSE_AHEAD = DMAX > 128;
+      float db[DENSE_AHEAD ? 16 : 1];
+      if constexpr (DENSE_AHEAD) {
+        if (live && p.dense_bias) general_dense_row(p, b, qi, kv0, hh, db);
+      }
       __syncthreads();                     // everyone is done with the tile before
       stage(kv0);
       __syncthreads();
@@ -595,14 +601,20 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
       }
       if (qi >= s.n_q) hi = -1;
       const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
-      const bool biased = p.pos_tab != nullptr || p.ts_tab != nullptr || p.dense_bias != nullptr;
+      const bool tabled = p.pos_tab != nullptr || p.ts_tab != nullptr;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
         bool keep = j >= lo && j <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
         if (by_seg) keep = keep && general_same_segment(p, b, qi, j);
         float x = p.alpha * sacc[r];
-        if (biased && keep) x += general_bias(p, s, b, h, qi, j);
+        if (tabled && keep) x += general_table_bias(p, s, b, h, qi, j);
+        if constexpr (DENSE_AHEAD) {
+          if (p.dense_bias) x += db[r];
+        } else {
+          if (p.dense_bias && keep)
+            x += p.dense_bias[(p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)qi * p.Lkv + j];
+        }
         // silu(x) = x / (1 + e^-x), by the hardware's exp2 and reciprocal (1 ulp each)
         const float val = x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
         sacc[r] = keep ? val : 0.f;      // P^T in place of S^T

@@ -662,6 +662,8 @@ def main():
   # The public entry point as a user calls it (arguments checked and the struct built on every call):
   # on its own (scratch allocated and prepared per call), and with one AttentionBatch for all calls.
   api_kw = dict(kw)
+  for _ in range(max(3, args.warmup)):      # (the first calls pay torch's allocator for the scratch buffer)
+    recml_amd.hstu_attention(q, k, v, out=out, **api_kw)
   api_ms = timed(lambda: recml_amd.hstu_attention(q, k, v, out=out, **api_kw), args.steps)
   shared = hstu_ops.AttentionBatch()
   recml_amd.hstu_attention(q, k, v, out=out, batch=shared, **api_kw)

@@ -381,9 +381,12 @@ def bench_dense(args, dev):
   from oracle import hstu_oracle as O
   B, L, H, d = 16, 2048, 8, 128
   gen = torch.Generator(device=dev).manual_seed(11)
-  q, k, v = (torch.randn((B, L, H, d), device=dev, generator=gen).mul_(0.3).to(torch.bfloat16) for _ in range(3))
+  dt = torch.float32 if args.fp32 else torch.bfloat16
+  q, k, v = (torch.randn((B, L, H, d), device=dev, generator=gen).mul_(0.3).to(dt) for _ in range(3))
   mask = torch.tril(torch.ones((L, L), device=dev, dtype=torch.uint8))[None].expand(B, L, L).contiguous()
   bias = torch.randn((B, L, L), device=dev, generator=gen).mul_(0.3)
+  if args.backward:
+    return bench_dense_backward(args, q, k, v, mask, bias)
   out = torch.empty_like(v)
   call_args, keep = hstu_ops.build_args(q, k, v, out, n=L, alpha=1.0, causal=False, mask=mask, bias=bias)
   variant = hstu_ops.kernel_variant(call_args)
@@ -421,10 +424,11 @@ def bench_dense(args, dev):
   flops = 4.0 * d * H * B * L * (L + 1) / 2
   nbytes = 4 * B * L * H * d * 2 + B * L * L * 5
   rec = {
-      "metric": "HSTU attn fwd TFLOP/s (kept pairs), dense mask + bias, L=%d bf16" % L, "value": flops / (ms * 1e-3) / 1e12,
+      "metric": "HSTU attn fwd TFLOP/s (kept pairs), dense mask + bias, L=%d %s" % (L, "fp32" if args.fp32 else "bf16"),
+      "value": flops / (ms * 1e-3) / 1e12,
       "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
       "ms_per_step_with_prepare": with_prepare_ms,
-      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if args.fp32 else "bf16", "data": "synthetic",
       "config": {"workload": f"A1-dense: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",
                  "kernel": variant},
       "roofline": {"bound": "hbm", "achieved": nbytes / (ker * 1e-3) / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -432,7 +436,7 @@ def bench_dense(args, dev):
                    "algorithmic_bytes": nbytes, "algorithmic_flops": flops,
                    "dense_operand_bytes_as_read_by_all_heads": H * B * steps_run * 128 * 32 * 5,
                    "prepare_ms": with_prepare_ms - ms,
-                   "mfma_frac": flops / (ker * 1e-3) / 1e12 / PEAK_BF16_TFLOPS},
+                   "mfma_frac": flops / (ker * 1e-3) / 1e12 / (PEAK_FP32_TFLOPS if args.fp32 else PEAK_BF16_TFLOPS)},
   }
   if not args.no_cpu:
     # the numpy restatement on the first sequence's first 256 rows and keys (the causal mask keeps earlier keys only)
@@ -450,6 +454,45 @@ def bench_dense(args, dev):
     if not err <= 2e-2:
       raise SystemExit(f"parity failed in the benchmark run: {err}")
   print(json.dumps(rec))
+
+
+def bench_dense_backward(args, q, k, v, mask, bias):
+  """The backward of the layer-side call (dense mask + bias), without and with the gradient of the dense bias:
+  one JSON line.  FLOPs: four products over the pairs the mask keeps."""
+  import torch
+  import recml_amd
+  B, L, H, d = q.shape
+  dout = torch.randn_like(q)
+  variant = []
+  steps, warm = max(1, args.steps // 10), max(1, args.warmup // 10)
+
+  def timed(bias_grad):
+    run = lambda: recml_amd.hstu_attention_bwd(q, k, v, dout, n=L, alpha=1.0, causal=False, mask=mask, bias=bias,
+                                               bias_grad=bias_grad, _variant_out=variant)
+    for _ in range(warm):
+      run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+      run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+  ms, ms_bias = timed(False), timed(True)
+  flops = 8.0 * d * H * B * L * (L + 1) / 2
+  fp32 = q.dtype == torch.float32
+  print(json.dumps({
+      "metric": "HSTU attn bwd TFLOP/s (kept pairs), dense mask + bias, L=%d %s" % (L, "fp32" if fp32 else "bf16"),
+      "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
+      "ms_per_step_with_bias_gradient": ms_bias,
+      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+      "dtype": "f32" if fp32 else "bf16 storage, fp32 arithmetic", "data": "synthetic",
+      "config": {"workload": f"A1-dense backward: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",
+                 "kernel": variant[-1]},
+      "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                   "frac": flops / (ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, "traffic": None,
+                   "note": "general kernels on the fp32 matrix cores; time covers both kernels, the memsets and the host call"},
+  }))
 
 
 def bench_backward(args, w, q, k, v, kw, dev):

@@ -12,6 +12,12 @@
  *   hstu_norm_gate_fwd    out = u * layer_norm(attn): the layer norm over
  *                         (heads, head_dim) of the attention output and the U
  *                         gate (hstu.py:471-472) in one pass over memory.
+ *   hstu_norm_gate_bwd    the gradients of that step for training: of the
+ *                         attention output, of U, of the norm's scale and
+ *                         offset (what the framework's autodiff derives from
+ *                         hstu.py:471-472); without a gate, the gradients of a
+ *                         plain layer norm (the block's input norm,
+ *                         hstu.py:442, and the model's final_norm).
  *   hstu_embed_norm_fwd   out = layer_norm(scale * table[ids] + pos_table[positions]):
  *                         the model's front end (hstu.py:593-601: item
  *                         embedding, optional sqrt(D) scale, position
@@ -30,7 +36,7 @@
 extern "C" {
 #endif
 
-#define HSTU_BLOCK_ABI_VERSION 1
+#define HSTU_BLOCK_ABI_VERSION 2
 
 typedef enum HstuBlockStatus {
   HSTU_BLOCK_OK = 0,
@@ -48,7 +54,8 @@ typedef enum HstuBlockStatus {
  * hstu.py:340-346 and :471-472).  a, u, out: bf16 [rows, width] with the given
  * row strides in elements (u is usually a slice of the fused projection);
  * gamma, beta: bf16 [width].  width a multiple of 8 up to 8192; pointers and
- * row strides multiples of 8 elements (16 bytes). */
+ * row strides multiples of 8 elements (16 bytes).  u may be null: then
+ * out = layer_norm(a), the plain norm (u_stride is ignored). */
 typedef struct HstuNormGateArgs {
   uint32_t struct_size;   /* sizeof(HstuNormGateArgs)  */
   uint32_t version;       /* HSTU_BLOCK_ABI_VERSION    */
@@ -64,6 +71,43 @@ typedef struct HstuNormGateArgs {
 } HstuNormGateArgs;
 
 int hstu_norm_gate_fwd(const HstuNormGateArgs* args, void* stream);
+
+/* Gradients of hstu_norm_gate_fwd for the gradient `dout` of its result (the
+ * reference leaves these to autodiff of hstu.py:471-472 and of keras
+ * LayerNormalization):
+ *   da     bf16 [rows, width]  gradient of a
+ *   du     bf16 [rows, width]  gradient of u (usually a slice of the gradient
+ *                              of the fused projection: du_stride)
+ *   dgamma, dbeta  fp32 [width], overwritten: sums over the rows, added in a
+ *                              fixed order (the same bits on every run)
+ * a, u, gamma, beta, eps as in the forward call; u and du null together: the
+ * gradients of a plain layer norm.  width a multiple of 8 up to 2048; pointers
+ * and row strides multiples of 8 elements.  `workspace`: device memory of
+ * hstu_norm_gate_bwd_workspace_bytes(rows, width) bytes (one partial row of
+ * column sums per workgroup), owned by the caller; the library allocates
+ * nothing.  rows = 0 writes zeros to dgamma and dbeta. */
+typedef struct HstuNormGateBwdArgs {
+  uint32_t struct_size;   /* sizeof(HstuNormGateBwdArgs) */
+  uint32_t version;       /* HSTU_BLOCK_ABI_VERSION      */
+  int64_t rows;
+  int32_t width;
+  float eps;
+  const void* a;
+  const void* u;
+  const void* dout;
+  void* da;
+  void* du;
+  int64_t a_stride, u_stride, dout_stride, da_stride, du_stride;
+  const void* gamma;
+  const void* beta;
+  float* dgamma;
+  float* dbeta;
+  void* workspace;
+  size_t workspace_bytes;
+} HstuNormGateBwdArgs;
+
+size_t hstu_norm_gate_bwd_workspace_bytes(int64_t rows, int32_t width);
+int hstu_norm_gate_bwd(const HstuNormGateBwdArgs* args, void* stream);
 
 /* out[m, n] = silu(sum_k x[m, k] w[k, n] + bias[n]); x: bf16 [M, K] (row stride
  * x_stride), w: bf16 [K, N] contiguous, bias: bf16 [N] or null, out: bf16

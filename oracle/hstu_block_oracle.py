@@ -22,6 +22,9 @@ Restates, in plain numpy:
                        hstu.py:593-601.
                        These three are compositions of layer_norm and hstu_oracle.silu,
                        both pinned, with a product / a row lookup.
+  norm_gate_bwd        the gradients of norm_gate (and of layer_norm alone): the
+                       reference leaves them to autodiff; pinned by central
+                       differences of norm_gate in fp64 (tests/test_block_ops.py).
 
 Pinning (tests/test_hstu_layer.py): layer_norm against the textbook definition
 on hand-sized inputs and against torch's CPU layer_norm; the dense layers are
@@ -112,6 +115,26 @@ def hstu_param_count(vocab_size, max_positions, model_dim, num_layers, add_head=
 def norm_gate(attn, u, gamma, beta, eps=1e-6):
   """u * layer_norm(attn) over the last axis (recml/layers/keras/hstu.py:471-472)."""
   return np.asarray(u, np.float64) * layer_norm(attn, gamma, beta, eps)
+
+
+def norm_gate_bwd(attn, u, gamma, beta, dout, eps=1e-6):
+  """Gradients of sum(norm_gate(attn, u, gamma, beta) * dout): (d_attn, d_u, d_gamma, d_beta); u=None: of
+  sum(layer_norm(attn) * dout), d_u None.  The layer norm's textbook backward: with xh the normalised row
+  and g the gradient at the norm's output times gamma, d_attn = rstd (g - mean(g) - xh mean(g xh))."""
+  a, do = np.asarray(attn, np.float64), np.asarray(dout, np.float64)
+  gm, bt = np.asarray(gamma, np.float64), np.asarray(beta, np.float64)
+  mean = a.mean(-1, keepdims=True)
+  rstd = 1.0 / np.sqrt(((a - mean) ** 2).mean(-1, keepdims=True) + eps)
+  xh = (a - mean) * rstd
+  du = None
+  gn = do
+  if u is not None:
+    du = do * (xh * gm + bt)
+    gn = do * np.asarray(u, np.float64)
+  g = gn * gm
+  da = rstd * (g - g.mean(-1, keepdims=True) - xh * (g * xh).mean(-1, keepdims=True))
+  red = tuple(range(a.ndim - 1))
+  return da, du, (gn * xh).sum(red), gn.sum(red)
 
 
 def gemm_silu(x, w, bias=None, activation=True):

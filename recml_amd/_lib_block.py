@@ -9,12 +9,14 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RECML_AMD_BLOCK_LIB") or os.path.join(_HERE, "lib", "libhstu_block.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EXPORTS = (
     "hstu_block_abi_version",
     "hstu_block_last_error",
     "hstu_norm_gate_fwd",
+    "hstu_norm_gate_bwd",
+    "hstu_norm_gate_bwd_workspace_bytes",
     "hstu_gemm_silu_fwd",
     "hstu_gemm_silu_workspace_bytes",
     "hstu_embed_norm_fwd",
@@ -30,6 +32,20 @@ class HstuNormGateArgs(C.Structure):
       ("a", C.c_void_p), ("u", C.c_void_p), ("out", C.c_void_p),
       ("a_stride", C.c_int64), ("u_stride", C.c_int64), ("out_stride", C.c_int64),
       ("gamma", C.c_void_p), ("beta", C.c_void_p),
+  ]
+
+
+class HstuNormGateBwdArgs(C.Structure):
+  """Field-for-field image of `struct HstuNormGateBwdArgs`."""
+
+  _fields_ = [
+      ("struct_size", C.c_uint32), ("version", C.c_uint32),
+      ("rows", C.c_int64), ("width", C.c_int32), ("eps", C.c_float),
+      ("a", C.c_void_p), ("u", C.c_void_p), ("dout", C.c_void_p), ("da", C.c_void_p), ("du", C.c_void_p),
+      ("a_stride", C.c_int64), ("u_stride", C.c_int64), ("dout_stride", C.c_int64),
+      ("da_stride", C.c_int64), ("du_stride", C.c_int64),
+      ("gamma", C.c_void_p), ("beta", C.c_void_p), ("dgamma", C.c_void_p), ("dbeta", C.c_void_p),
+      ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
   ]
 
 
@@ -82,6 +98,10 @@ def load():
     lib.hstu_block_last_error.argtypes = []
     lib.hstu_norm_gate_fwd.restype = C.c_int
     lib.hstu_norm_gate_fwd.argtypes = [C.POINTER(HstuNormGateArgs), C.c_void_p]
+    lib.hstu_norm_gate_bwd.restype = C.c_int
+    lib.hstu_norm_gate_bwd.argtypes = [C.POINTER(HstuNormGateBwdArgs), C.c_void_p]
+    lib.hstu_norm_gate_bwd_workspace_bytes.restype = C.c_size_t
+    lib.hstu_norm_gate_bwd_workspace_bytes.argtypes = [C.c_int64, C.c_int32]
     lib.hstu_gemm_silu_fwd.restype = C.c_int
     lib.hstu_gemm_silu_fwd.argtypes = [C.POINTER(HstuGemmSiluArgs), C.c_void_p]
     lib.hstu_gemm_silu_workspace_bytes.restype = C.c_size_t

@@ -5,6 +5,9 @@
 //                    one wavefront per token row, 16 bytes per lane and trip: the row is read once,
 //                    kept in registers for the two reductions (mean, then centred sum of squares) and
 //                    written once: 3 x width x 2 bytes of HBM traffic per row, which is the bound.
+//   hstu_norm_gate_bwd  the gradients of that step (and, without a gate, of a plain layer norm): one
+//                    pass over the row, its gradient and the gate; column sums for dgamma / dbeta in
+//                    registers, one partial row per workgroup, added in a fixed order by hstu_colsum.
 //   gemm + silu      out = silu(x W + bias)       (hstu.py:444-449)
 //                    hipBLASLt matrix product with the activation in its epilogue.
 //   hstu_embed_norm  out = layer_norm(scale * table[ids] + pos_table[positions])   (hstu.py:593-601)
@@ -79,7 +82,7 @@ __global__ __launch_bounds__(256) void hstu_norm_gate(const NormGateParams p) {
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= p.rows) return;
   const bf16_t* ar = p.a + row * p.a_stride;
-  const bf16_t* ur = p.u + row * p.u_stride;
+  const bf16_t* ur = p.u ? p.u + row * p.u_stride : nullptr;   // no gate: the plain layer norm
   bf16_t* orow = p.out + row * p.out_stride;
   float x[CH][8];
   float sum = 0.f;
@@ -116,7 +119,12 @@ __global__ __launch_bounds__(256) void hstu_norm_gate(const NormGateParams p) {
       float g[8], b[8], uu[8];
       unpack8(*(const uint4*)(p.gamma + e), g);
       unpack8(*(const uint4*)(p.beta + e), b);
-      unpack8(*(const uint4*)(ur + e), uu);
+      if (ur) {
+        unpack8(*(const uint4*)(ur + e), uu);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) uu[i] = 1.f;
+      }
       float y[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) y[i] = uu[i] * __builtin_fmaf((x[c][i] - mean) * rstd, g[i], b[i]);
@@ -128,6 +136,165 @@ __global__ __launch_bounds__(256) void hstu_norm_gate(const NormGateParams p) {
       *(uint4*)(orow + e) = o;
     }
   }
+}
+
+struct NormGateBwdParams {
+  const bf16_t* a;
+  const bf16_t* u;
+  const bf16_t* dout;
+  const bf16_t* gamma;
+  const bf16_t* beta;
+  bf16_t* da;
+  bf16_t* du;
+  float* partial;          // [gridDim.x][2 * width]: each workgroup's sums for dgamma, then for dbeta
+  int64_t rows, a_stride, u_stride, dout_stride, da_stride, du_stride;
+  int32_t width;
+  float eps;
+};
+
+// Backward of out = u * (gamma * xhat + beta), xhat = (a - mean) * rstd, for the gradient g of out:
+//   du = g * (gamma * xhat + beta),  gn = g * u  (the gradient at the normalised row; gn = g without a gate)
+//   dgamma += gn * xhat,  dbeta += gn           (summed over the rows)
+//   da = rstd * (gn gamma - mean_w(gn gamma) - xhat * mean_w(gn gamma xhat))
+// One wavefront per row as in the forward, a workgroup walking over rows with the grid's stride: the row,
+// its gradient and the gate are read once, da and du written once (5 x width x 2 bytes per row, the
+// bound).  The two column sums stay in registers over a wave's rows, are added across the workgroup's
+// four waves through LDS and leave as one partial row per workgroup; hstu_colsum adds those in a fixed
+// order, so the result does not depend on the timing of the run.
+template <int CH>
+__global__ __launch_bounds__(256) void hstu_norm_gate_bwd(const NormGateBwdParams p) {
+  __shared__ float red[4][CH * 512];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const float inv_w = 1.f / (float)p.width;
+  float dg[CH][8], db[CH][8];
+#pragma unroll
+  for (int c = 0; c < CH; ++c)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dg[c][i] = db[c][i] = 0.f;
+  for (int64_t row = (int64_t)blockIdx.x * 4 + w; row < p.rows; row += (int64_t)gridDim.x * 4) {
+    const bf16_t* ar = p.a + row * p.a_stride;
+    const bf16_t* gr = p.dout + row * p.dout_stride;
+    float x[CH][8], g[CH][8];
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int e = (c * 64 + lane) * 8;
+      if (e < p.width) {
+        unpack8(*(const uint4*)(ar + e), x[c]);
+        unpack8(*(const uint4*)(gr + e), g[c]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += x[c][i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[c][i] = g[c][i] = 0.f;
+      }
+    }
+    const float mean = wave_sum(sum) * inv_w;
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int e = (c * 64 + lane) * 8;
+      if (e < p.width) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float d = x[c][i] - mean;
+          ss += d * d;
+        }
+      }
+    }
+    const float rstd = __builtin_amdgcn_rsqf(wave_sum(ss) * inv_w + p.eps);
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int e = (c * 64 + lane) * 8;
+      if (e < p.width) {
+        float gm[8];
+        unpack8(*(const uint4*)(p.gamma + e), gm);
+        if (p.u) {
+          float bt[8], uu[8], y[8];
+          unpack8(*(const uint4*)(p.beta + e), bt);
+          unpack8(*(const uint4*)(p.u + row * p.u_stride + e), uu);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            y[i] = g[c][i] * __builtin_fmaf((x[c][i] - mean) * rstd, gm[i], bt[i]);
+            g[c][i] *= uu[i];
+          }
+          uint4 o;
+          o.x = pack2(y[0], y[1]);
+          o.y = pack2(y[2], y[3]);
+          o.z = pack2(y[4], y[5]);
+          o.w = pack2(y[6], y[7]);
+          *(uint4*)(p.du + row * p.du_stride + e) = o;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xh = (x[c][i] - mean) * rstd;
+          const float gn = g[c][i];
+          x[c][i] = xh;
+          dg[c][i] = __builtin_fmaf(gn, xh, dg[c][i]);
+          db[c][i] += gn;
+          const float gx = gn * gm[i];
+          g[c][i] = gx;
+          s1 += gx;
+          s2 = __builtin_fmaf(gx, xh, s2);
+        }
+      }
+    }
+    const float c1 = wave_sum(s1) * inv_w, c2 = wave_sum(s2) * inv_w;
+    bf16_t* dr = p.da + row * p.da_stride;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int e = (c * 64 + lane) * 8;
+      if (e < p.width) {
+        float y[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = rstd * (g[c][i] - c1 - x[c][i] * c2);
+        uint4 o;
+        o.x = pack2(y[0], y[1]);
+        o.y = pack2(y[2], y[3]);
+        o.z = pack2(y[4], y[5]);
+        o.w = pack2(y[6], y[7]);
+        *(uint4*)(dr + e) = o;
+      }
+    }
+  }
+  // the workgroup's column sums: every wave gets here, whatever rows it had
+  float* part = p.partial + (int64_t)blockIdx.x * (2 * p.width);
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) red[w][(c * 64 + lane) * 8 + i] = half == 0 ? dg[c][i] : db[c][i];
+    __syncthreads();
+    for (int col = threadIdx.x; col < p.width; col += 256)
+      part[half * p.width + col] = (red[0][col] + red[1][col]) + (red[2][col] + red[3][col]);
+    __syncthreads();
+  }
+}
+
+// out[col] = sum over the nb partial rows of part[.][col], rows added in a fixed order; columns
+// [0, width) go to dgamma, [width, 2 width) to dbeta.  nb = 0 writes zeros.
+__global__ __launch_bounds__(256) void hstu_colsum(const float* __restrict__ part, int nb, int width, float* __restrict__ dgamma,
+                                                   float* __restrict__ dbeta) {
+  __shared__ float red[4][64];
+  const int cl = threadIdx.x & 63, rg = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + cl, n2 = 2 * width;
+  float s = 0.f;
+  if (col < n2)
+    for (int r = rg; r < nb; r += 4) s += part[(int64_t)r * n2 + col];
+  red[rg][cl] = s;
+  __syncthreads();
+  if (rg == 0 && col < n2) {
+    s = (red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl]);
+    if (col < width) dgamma[col] = s; else dbeta[col - width] = s;
+  }
+}
+
+// workgroups of the backward kernel for this many rows (each walks over rows with the grid's stride)
+int norm_gate_bwd_blocks(int64_t rows) {
+  const int64_t nb = (rows + 3) / 4;
+  return (int)(nb < 1 ? 1 : (nb > 1024 ? 1024 : nb));
 }
 
 struct EmbedNormParams {
@@ -271,10 +438,10 @@ int hstu_norm_gate_fwd(const HstuNormGateArgs* a, void* stream) {
                 (long long)a->rows, a->width);
   g_err[0] = 0;
   if (a->rows == 0) return HSTU_BLOCK_OK;
-  if (!a->a || !a->u || !a->out || !a->gamma || !a->beta) return fail(HSTU_BLOCK_ERR_NULL, "a, u, out, gamma and beta must be non-null");
+  if (!a->a || !a->out || !a->gamma || !a->beta) return fail(HSTU_BLOCK_ERR_NULL, "a, out, gamma and beta must be non-null");
   if (!aligned16(a->a) || !aligned16(a->u) || !aligned16(a->out) || !aligned16(a->gamma) || !aligned16(a->beta) ||
-      (a->a_stride & 7) || (a->u_stride & 7) || (a->out_stride & 7) ||
-      a->a_stride < a->width || a->u_stride < a->width || a->out_stride < a->width)
+      (a->a_stride & 7) || (a->out_stride & 7) || a->a_stride < a->width || a->out_stride < a->width ||
+      (a->u && ((a->u_stride & 7) || a->u_stride < a->width)))
     return fail(HSTU_BLOCK_ERR_SHAPE, "pointers must be 16-byte aligned, row strides multiples of 8 elements and >= width");
   if ((a->rows + 3) / 4 > 0x7fffffffLL) return fail(HSTU_BLOCK_ERR_SHAPE, "too many rows");
   NormGateParams p;
@@ -291,6 +458,57 @@ int hstu_norm_gate_fwd(const HstuNormGateArgs* a, void* stream) {
   else hipLaunchKernelGGL(hstu_norm_gate<16>, grid, block, 0, st, p);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "norm-gate kernel launch: %s", hipGetErrorString(e));
+  return HSTU_BLOCK_OK;
+}
+
+size_t hstu_norm_gate_bwd_workspace_bytes(int64_t rows, int32_t width) {
+  if (rows < 0 || width < 8) return 0;
+  return (size_t)norm_gate_bwd_blocks(rows) * 2u * (size_t)width * sizeof(float);
+}
+
+int hstu_norm_gate_bwd(const HstuNormGateBwdArgs* a, void* stream) {
+  if (!a) return fail(HSTU_BLOCK_ERR_NULL, "args is null");
+  if (a->struct_size != sizeof(HstuNormGateBwdArgs) || a->version != HSTU_BLOCK_ABI_VERSION)
+    return fail(HSTU_BLOCK_ERR_VERSION, "norm-gate backward args struct_size/version (%u/%u) do not match this library (%zu/%d)",
+                a->struct_size, a->version, sizeof(HstuNormGateBwdArgs), HSTU_BLOCK_ABI_VERSION);
+  if (a->rows < 0 || a->width < 8 || a->width > 2048 || (a->width & 7))
+    return fail(HSTU_BLOCK_ERR_SHAPE, "rows >= 0 and width a multiple of 8 in [8, 2048] expected, got rows=%lld width=%d",
+                (long long)a->rows, a->width);
+  g_err[0] = 0;
+  if (!a->dgamma || !a->dbeta) return fail(HSTU_BLOCK_ERR_NULL, "dgamma and dbeta must be non-null");
+  hipStream_t st = (hipStream_t)stream;
+  const int nb = a->rows == 0 ? 0 : norm_gate_bwd_blocks(a->rows);
+  if (nb > 0) {
+    if (!a->a || !a->dout || !a->da || !a->gamma || !a->beta) return fail(HSTU_BLOCK_ERR_NULL, "a, dout, da, gamma and beta must be non-null");
+    if ((a->u == nullptr) != (a->du == nullptr)) return fail(HSTU_BLOCK_ERR_NULL, "u and du go together (both null: the plain layer norm)");
+    if (!aligned16(a->a) || !aligned16(a->u) || !aligned16(a->dout) || !aligned16(a->da) || !aligned16(a->du) ||
+        !aligned16(a->gamma) || !aligned16(a->beta) ||
+        (a->a_stride & 7) || (a->dout_stride & 7) || (a->da_stride & 7) ||
+        a->a_stride < a->width || a->dout_stride < a->width || a->da_stride < a->width ||
+        (a->u && ((a->u_stride & 7) || (a->du_stride & 7) || a->u_stride < a->width || a->du_stride < a->width)))
+      return fail(HSTU_BLOCK_ERR_SHAPE, "pointers must be 16-byte aligned, row strides multiples of 8 elements and >= width");
+    const size_t need = hstu_norm_gate_bwd_workspace_bytes(a->rows, a->width);
+    if (!a->workspace || a->workspace_bytes < need || ((uintptr_t)a->workspace & 3u))
+      return fail(HSTU_BLOCK_ERR_WORKSPACE, "workspace of %zu bytes needed (hstu_norm_gate_bwd_workspace_bytes), got %zu", need,
+                  a->workspace ? a->workspace_bytes : (size_t)0);
+    NormGateBwdParams p;
+    p.a = (const bf16_t*)a->a; p.u = (const bf16_t*)a->u; p.dout = (const bf16_t*)a->dout;
+    p.gamma = (const bf16_t*)a->gamma; p.beta = (const bf16_t*)a->beta;
+    p.da = (bf16_t*)a->da; p.du = (bf16_t*)a->du; p.partial = (float*)a->workspace;
+    p.rows = a->rows; p.a_stride = a->a_stride; p.u_stride = a->u_stride; p.dout_stride = a->dout_stride;
+    p.da_stride = a->da_stride; p.du_stride = a->du_stride; p.width = a->width; p.eps = a->eps;
+    const dim3 grid((unsigned)nb), block(256);
+    const int ch = (a->width + 511) / 512;
+    if (ch <= 1) hipLaunchKernelGGL(hstu_norm_gate_bwd<1>, grid, block, 0, st, p);
+    else if (ch <= 2) hipLaunchKernelGGL(hstu_norm_gate_bwd<2>, grid, block, 0, st, p);
+    else hipLaunchKernelGGL(hstu_norm_gate_bwd<4>, grid, block, 0, st, p);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "norm-gate backward kernel launch: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(hstu_colsum, dim3((unsigned)((2 * a->width + 63) / 64)), dim3(256), 0, st, (const float*)a->workspace, nb, a->width,
+                     a->dgamma, a->dbeta);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "column-sum kernel launch: %s", hipGetErrorString(e));
   return HSTU_BLOCK_OK;
 }
 

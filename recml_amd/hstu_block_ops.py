@@ -1,6 +1,8 @@
 """Host side of the fused block steps (libhstu_block.so): torch tensors in, HIP kernels behind the C ABI.
 
   norm_gate(attn, u, gamma, beta, eps)     u * layer_norm(attn)       recml/layers/keras/hstu.py:471-472
+  layer_norm(x, gamma, beta, eps)          the same kernels without the gate                     hstu.py:442
+  norm_gate_bwd(...)                       their gradients (norm_gate and layer_norm are differentiable)
   gemm_silu(x, w, bias, activation)        silu(x @ w + bias)          recml/layers/keras/hstu.py:444-449
   embed_norm(ids, table, ...)              layer_norm(scale * table[ids] + pos_table[positions])   hstu.py:593-601
 
@@ -32,22 +34,23 @@ def _raise(lib, rc, what):
   raise RuntimeError(f"{what} failed ({rc}): {msg}")
 
 
-def norm_gate(attn, u, gamma, beta, eps: float = 1e-6):
-  """u * layer_norm(attn) over the last axis.  attn, u: [..., W] bf16 whose last axis is contiguous
-  and whose leading axes collapse to one row stride (a slice of a fused projection does);
-  gamma, beta: [W]."""
-  for n, t in (("attn", attn), ("u", u), ("gamma", gamma), ("beta", beta)):
+def _norm_gate_fwd(attn, u, gamma, beta, eps):
+  """The forward kernel: u * layer_norm(attn), or layer_norm(attn) with u=None."""
+  for n, t in (("attn", attn), ("gamma", gamma), ("beta", beta)) + ((("u", u),) if u is not None else ()):
     _check(n, t)
-  if attn.shape != u.shape:
+  if u is not None and attn.shape != u.shape:
     raise ValueError(f"attn {tuple(attn.shape)} and u {tuple(u.shape)} differ in shape")
   W = attn.shape[-1]
-  a2, u2 = _rows(attn, "attn"), _rows(u, "u")
+  a2 = _rows(attn, "attn")
+  u2 = _rows(u, "u") if u is not None else None
   out = torch.empty(attn.shape, dtype=attn.dtype, device=attn.device)
   a = _lib_block.HstuNormGateArgs()
   a.struct_size, a.version = C.sizeof(_lib_block.HstuNormGateArgs), _lib_block.ABI_VERSION
   a.rows, a.width, a.eps = a2.shape[0], W, float(eps)
-  a.a, a.u, a.out = a2.data_ptr(), u2.data_ptr(), out.data_ptr()
-  a.a_stride, a.u_stride, a.out_stride = a2.stride(0), u2.stride(0), W
+  a.a, a.out = a2.data_ptr(), out.data_ptr()
+  a.a_stride, a.out_stride = a2.stride(0), W
+  if u2 is not None:
+    a.u, a.u_stride = u2.data_ptr(), u2.stride(0)
   g, b = gamma.reshape(-1).contiguous(), beta.reshape(-1).contiguous()
   if g.numel() != W or b.numel() != W:
     raise ValueError(f"gamma and beta must have {W} entries")
@@ -58,6 +61,91 @@ def norm_gate(attn, u, gamma, beta, eps: float = 1e-6):
   if rc != 0:
     _raise(lib, rc, "hstu_norm_gate_fwd")
   return out
+
+
+def norm_gate_bwd(attn, u, gamma, beta, dout, eps: float = 1e-6, *, du_out=None):
+  """Gradients of u * layer_norm(attn) (of layer_norm(attn) with u=None) for the gradient `dout` of the
+  result: (d_attn, d_u, d_gamma, d_beta); d_attn and d_u bf16 shaped like attn, d_gamma and d_beta fp32
+  [W], summed over the rows in a fixed order.  `du_out`: where to write d_u (a slice of the gradient
+  of a fused projection, say) instead of a new tensor.  W up to 2048."""
+  for n, t in (("attn", attn), ("gamma", gamma), ("beta", beta), ("dout", dout)) + ((("u", u),) if u is not None else ()):
+    _check(n, t)
+  if dout.shape != attn.shape or (u is not None and u.shape != attn.shape):
+    raise ValueError(f"attn {tuple(attn.shape)}, u and dout must have one shape")
+  W = attn.shape[-1]
+  a2, g2 = _rows(attn, "attn"), _rows(dout, "dout")
+  da = torch.empty(attn.shape, dtype=attn.dtype, device=attn.device)
+  a = _lib_block.HstuNormGateBwdArgs()
+  a.struct_size, a.version = C.sizeof(_lib_block.HstuNormGateBwdArgs), _lib_block.ABI_VERSION
+  a.rows, a.width, a.eps = a2.shape[0], W, float(eps)
+  a.a, a.dout, a.da = a2.data_ptr(), g2.data_ptr(), da.data_ptr()
+  a.a_stride, a.dout_stride, a.da_stride = a2.stride(0), g2.stride(0), W
+  du = None
+  if u is not None:
+    u2 = _rows(u, "u")
+    if du_out is None:
+      du = torch.empty(attn.shape, dtype=attn.dtype, device=attn.device)
+    else:
+      _check("du_out", du_out)
+      du = du_out
+      if du.shape != attn.shape or du.stride(-1) != 1:
+        raise ValueError("du_out must be shaped like attn with a contiguous last axis")
+    d2 = du if du.dim() == 2 else du.view(-1, W)     # raises if the leading axes do not collapse: a copy would lose the writes
+    a.u, a.u_stride, a.du, a.du_stride = u2.data_ptr(), u2.stride(0), d2.data_ptr(), d2.stride(0)
+  g, b = gamma.reshape(-1).contiguous(), beta.reshape(-1).contiguous()
+  if g.numel() != W or b.numel() != W:
+    raise ValueError(f"gamma and beta must have {W} entries")
+  a.gamma, a.beta = g.data_ptr(), b.data_ptr()
+  dgb = torch.empty((2, W), dtype=torch.float32, device=attn.device)
+  a.dgamma, a.dbeta = dgb[0].data_ptr(), dgb[1].data_ptr()
+  lib = _lib_block.load()
+  ws = torch.empty(max(lib.hstu_norm_gate_bwd_workspace_bytes(a2.shape[0], W), 16), dtype=torch.uint8, device=attn.device)
+  a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+  with torch.cuda.device(attn.device):
+    rc = lib.hstu_norm_gate_bwd(C.byref(a), C.c_void_p(torch.cuda.current_stream(attn.device).cuda_stream))
+  if rc != 0:
+    _raise(lib, rc, "hstu_norm_gate_bwd")
+  return da, du, dgb[0], dgb[1]
+
+
+class _NormGateFn(torch.autograd.Function):
+  """u * layer_norm(attn) (u=None: layer_norm(attn)) with its gradients, both through the HIP kernels."""
+
+  @staticmethod
+  def forward(ctx, attn, u, gamma, beta, eps):
+    ctx.eps = eps
+    ctx.gated = u is not None
+    ctx.save_for_backward(attn, gamma, beta, *((u,) if u is not None else ()))
+    return _norm_gate_fwd(attn, u, gamma, beta, eps)
+
+  @staticmethod
+  def backward(ctx, dout):
+    attn, gamma, beta, *rest = ctx.saved_tensors
+    u = rest[0] if ctx.gated else None
+    dout = dout if dout.stride(-1) == 1 else dout.contiguous()
+    da, du, dg, db = norm_gate_bwd(attn, u, gamma, beta, dout, ctx.eps)
+    return da, du, dg.to(gamma.dtype).reshape(gamma.shape), db.to(beta.dtype).reshape(beta.shape), None
+
+
+def _wants_grad(*ts):
+  return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in ts)
+
+
+def norm_gate(attn, u, gamma, beta, eps: float = 1e-6):
+  """u * layer_norm(attn) over the last axis.  attn, u: [..., W] bf16 whose last axis is contiguous
+  and whose leading axes collapse to one row stride (a slice of a fused projection does);
+  gamma, beta: [W].  Differentiable in all four (W up to 2048 then)."""
+  if _wants_grad(attn, u, gamma, beta):
+    return _NormGateFn.apply(attn, u, gamma, beta, eps)
+  return _norm_gate_fwd(attn, u, gamma, beta, eps)
+
+
+def layer_norm(x, gamma, beta, eps: float = 1e-6):
+  """layer_norm(x) over the last axis (keras LayerNormalization as the block's input norm uses it,
+  recml/layers/keras/hstu.py:442): the same kernels without the gate.  Differentiable in x, gamma, beta."""
+  if _wants_grad(x, gamma, beta):
+    return _NormGateFn.apply(x, None, gamma, beta, eps)
+  return _norm_gate_fwd(x, None, gamma, beta, eps)
 
 
 def _rows(t, name):

@@ -409,7 +409,7 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
                        timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                        q_segment_ids=None, kv_segment_ids=None,
                        sliding_window_size=None, mask=None, bias=None,
-                       table_grads=True, bias_grad=False, _variant_out=None):
+                       table_grads=True, bias_grad=False, grads_out=None, _variant_out=None):
   """Gradients of sum(hstu_attention(q, k, v, ...) * dout).
 
   Same arguments as hstu_attention (fp32 or bf16; not fp8).  Returns
@@ -417,8 +417,11 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   the table gradients fp32 and shaped like the tables (None for a table that
   was not given, and for both with table_grads=False).  With bias_grad=True a
   sixth value: the gradient of the dense `bias`, fp32, shaped like it (summed
-  over the heads, and over the batch when the bias is shared by it).  Math of
-  the reference's backward kernel (recml/core/ops/hstu_ops.py:417-548).
+  over the heads, and over the batch when the bias is shared by it).
+  `grads_out`: three tensors to take dq, dk, dv instead of new ones, each with
+  the shape, dtype and strides of its input (the slices of the gradient of a
+  fused projection, say).  Math of the reference's backward kernel
+  (recml/core/ops/hstu_ops.py:417-548).
   """
   for name, t in (("q", q), ("k", k), ("v", v), ("dout", dout)):
     _check_gpu(name, t)
@@ -436,7 +439,14 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
       mask=mask, bias=bias)
   # build_args may have made q, k, v contiguous in d: the gradients take the layout it passed on
   qi, ki, vi = _passed_inputs(keep)
-  dq, dk, dv = _grad_buffers(qi, ki, vi)
+  if grads_out is None:
+    dq, dk, dv = _grad_buffers(qi, ki, vi)
+  else:
+    dq, dk, dv = grads_out
+    for name, g, t in (("dq", dq, qi), ("dk", dk, ki), ("dv", dv, vi)):
+      if g.shape != t.shape or g.dtype != t.dtype or g.stride() != t.stride() or g.device != t.device:
+        raise ValueError(f"grads_out: {name} must have the shape, dtype and strides of its input as the kernels read it "
+                         f"({tuple(t.shape)}, {t.dtype}, strides {t.stride()})")
   ba = _lib.HstuAttnBwdArgs()
   ba.struct_size = C.sizeof(_lib.HstuAttnBwdArgs)
   ba.version = _lib.ABI_VERSION

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
   assert lib.hstu_block_abi_version() == _lib_block.ABI_VERSION
 
 
-@pytest.mark.parametrize("name", ["HstuNormGateArgs", "HstuGemmSiluArgs", "HstuEmbedNormArgs"])
+@pytest.mark.parametrize("name", ["HstuNormGateArgs", "HstuNormGateBwdArgs", "HstuGemmSiluArgs", "HstuEmbedNormArgs"])
 def test_struct_layout_matches_header(name):
   struct = getattr(_lib_block, name)
   fields = [f[0] for f in struct._fields_]
@@ -62,6 +62,21 @@ def test_validation_errors_without_gpu():
   assert b"stride" in lib.hstu_block_last_error()
   a.rows = 0
   assert lib.hstu_norm_gate_fwd(C.byref(a), None) == 0           # nothing to do
+  nb = _lib_block.HstuNormGateBwdArgs()
+  assert lib.hstu_norm_gate_bwd(None, None) == -1
+  assert lib.hstu_norm_gate_bwd(C.byref(nb), None) == -2
+  nb.struct_size, nb.version = C.sizeof(nb), _lib_block.ABI_VERSION
+  nb.rows, nb.width = 4, 4096
+  assert lib.hstu_norm_gate_bwd(C.byref(nb), None) == -4         # the backward stops at width 2048
+  nb.width = 64
+  assert lib.hstu_norm_gate_bwd(C.byref(nb), None) == -1         # null outputs
+  nb.a = nb.dout = nb.da = nb.gamma = nb.beta = nb.dgamma = nb.dbeta = nb.u = 0x1000
+  nb.a_stride = nb.dout_stride = nb.da_stride = nb.u_stride = nb.du_stride = 64
+  assert lib.hstu_norm_gate_bwd(C.byref(nb), None) == -1         # a gate without a place for its gradient
+  nb.du = 0x1000
+  assert lib.hstu_norm_gate_bwd(C.byref(nb), None) == -5         # no workspace
+  assert lib.hstu_norm_gate_bwd_workspace_bytes(4, 64) == 1 * 2 * 64 * 4
+  assert lib.hstu_norm_gate_bwd_workspace_bytes(10 ** 6, 512) == 1024 * 2 * 512 * 4
   g = _lib_block.HstuGemmSiluArgs()
   assert lib.hstu_gemm_silu_fwd(C.byref(g), None) == -2
   g.struct_size, g.version = C.sizeof(g), _lib_block.ABI_VERSION
@@ -90,6 +105,34 @@ def test_oracle_compositions_on_a_hand_case():
   assert np.allclose(got, np.stack([z[0], z[0]]), atol=1e-15)      # scale 2 and the shift both cancel in the norm
 
 
+@pytest.mark.parametrize("gated", [True, False])
+def test_oracle_norm_gate_gradients_by_central_differences(gated):
+  """Pins oracle.norm_gate_bwd: every entry of each gradient against a central difference of the forward
+  restatement in fp64 (a dropped mean term, a wrong sign or a missing gamma shows at 1e-3 or more)."""
+  rng = np.random.default_rng(3)
+  R, W, eps = 3, 8, 1e-3
+  a, u, do = rng.normal(size=(R, W)), rng.normal(size=(R, W)), rng.normal(size=(R, W))
+  gm, bt = 1 + 0.3 * rng.normal(size=W), 0.2 * rng.normal(size=W)
+  f = lambda a_, u_, g_, b_: float(((BO.norm_gate(a_, u_, g_, b_, eps) if gated else BO.layer_norm(a_, g_, b_, eps)) * do).sum())
+  da, du, dg, db = BO.norm_gate_bwd(a, u if gated else None, gm, bt, do, eps)
+  h = 1e-6
+  def fd(which):
+    base = [a, u, gm, bt]
+    out = np.zeros_like(base[which])
+    for idx in np.ndindex(out.shape):
+      hi = [t.copy() for t in base]; lo = [t.copy() for t in base]
+      hi[which][idx] += h; lo[which][idx] -= h
+      out[idx] = (f(*hi) - f(*lo)) / (2 * h)
+    return out
+  assert np.allclose(da, fd(0), rtol=1e-6, atol=1e-7)
+  assert np.allclose(dg, fd(2), rtol=1e-6, atol=1e-7)
+  assert np.allclose(db, fd(3), rtol=1e-6, atol=1e-7)
+  if gated:
+    assert np.allclose(du, fd(1), rtol=1e-6, atol=1e-7)
+  else:
+    assert du is None
+
+
 def _rel(a, b):
   return float((a - b).abs().max() / b.abs().max().clamp_min(1e-30))
 
@@ -111,6 +154,50 @@ def test_norm_gate_parity(gpu, rows, width):
   ref = torch.from_numpy(BO.norm_gate(n(attn), n(u), n(gamma), n(beta), 1e-6))
   assert out.shape == attn.shape and out.dtype == bf
   assert _rel(out.double().cpu(), ref) <= 8e-3                 # bf16 rounding of the result: 2^-8
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,width,gated", [(1, 8, True), (37, 64, True), (5000, 512, True), (4099, 512, False),
+                                              (64, 1000, True), (131, 2048, True), (9, 1536, False)])
+def test_norm_gate_gradients_parity(gpu, rows, width, gated):
+  """The backward kernel against the fp64 oracle on the same bf16 inputs; the column sums bit for bit
+  the same on a second run; the plain layer norm as the kernel without a gate; and through autograd."""
+  from recml_amd import hstu_block_ops as B
+  gen = torch.Generator().manual_seed(rows * 11 + width)
+  dev, bf = "cuda:0", torch.bfloat16
+  fused = (torch.randn((rows, 4, width), generator=gen) * 0.7).to(dev).to(bf)
+  u = fused[:, 1] if gated else None
+  attn = (torch.randn((rows, width), generator=gen) * 3e-3 + 1e-3).to(dev).to(bf)
+  dout = (torch.randn((rows, width), generator=gen) * 0.5).to(dev).to(bf)
+  gamma = (1 + 0.2 * torch.randn(width, generator=gen)).to(dev).to(bf)
+  beta = (0.1 * torch.randn(width, generator=gen)).to(dev).to(bf)
+  dfused = torch.zeros_like(fused)
+  da, du, dg, db = B.norm_gate_bwd(attn, u, gamma, beta, dout, 1e-6, du_out=dfused[:, 1] if gated else None)
+  n = lambda t: t.float().cpu().numpy()
+  rda, rdu, rdg, rdb = BO.norm_gate_bwd(n(attn), n(u) if gated else None, n(gamma), n(beta), n(dout), 1e-6)
+  assert da.dtype == bf and dg.dtype == torch.float32 and dg.shape == (width,)
+  assert _rel(da.double().cpu(), torch.from_numpy(rda)) <= 8e-3          # one bf16 rounding at the end
+  assert _rel(dg.double().cpu(), torch.from_numpy(rdg)) <= 1e-4          # fp32 sums of fp32 products
+  assert _rel(db.double().cpu(), torch.from_numpy(rdb)) <= 1e-4
+  if gated:
+    assert du.data_ptr() == dfused[:, 1].data_ptr()
+    assert _rel(du.double().cpu(), torch.from_numpy(rdu)) <= 8e-3
+    assert float(dfused[:, 0].abs().max()) == 0 and float(dfused[:, 2:].abs().max()) == 0   # only the slice is written
+  else:
+    assert du is None
+  again = B.norm_gate_bwd(attn, u, gamma, beta, dout, 1e-6)
+  assert torch.equal(again[2], dg) and torch.equal(again[3], db) and torch.equal(again[0], da)
+  # the differentiable ops
+  leaves = [t.clone().requires_grad_(True) for t in ((attn, u, gamma, beta) if gated else (attn, gamma, beta))]
+  out = B.norm_gate(*leaves, 1e-6) if gated else B.layer_norm(*leaves, 1e-6)
+  ref_out = BO.norm_gate(n(attn), n(u), n(gamma), n(beta), 1e-6) if gated else BO.layer_norm(n(attn), n(gamma), n(beta), 1e-6)
+  assert _rel(out.detach().double().cpu(), torch.from_numpy(ref_out)) <= 8e-3
+  out.backward(dout)
+  assert torch.equal(leaves[0].grad, da)
+  assert _rel(leaves[-2].grad.double().cpu(), torch.from_numpy(rdg)) <= 8e-3 and leaves[-2].grad.dtype == bf
+  assert _rel(leaves[-1].grad.double().cpu(), torch.from_numpy(rdb)) <= 8e-3
+  if gated:
+    assert torch.equal(leaves[1].grad, du)
 
 
 @pytest.mark.gpu

@@ -242,9 +242,11 @@ def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
   pos = (torch.randn((H, 2 * L - 1), generator=gen) * 0.3).to(dev).requires_grad_(True)
   dout = torch.randn((B, L, D), generator=gen).to(dev).to(dtype)
 
-  def grads(attention):
+  def grads(attention, fused_training):
     saved = hstu_layer._attention
     hstu_layer._attention = attention
+    if not fused_training:
+      blk._fused_training = lambda *a: False          # torch's layer norms and gate, the attention as a function of its own
     try:
       for t in [x, pos, *blk.parameters()]:
         t.grad = None
@@ -254,13 +256,71 @@ def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
               **{n: p.grad.float().clone() for n, p in blk.named_parameters() if p.grad is not None}}
     finally:
       hstu_layer._attention = saved
+      blk.__dict__.pop("_fused_training", None)
 
-  got = grads(hstu_layer._attention)
-  want = grads(_dense_attention)
-  assert set(got) == set(want) and "q_kernel" in got and "output_kernel" in got
+  # the block as it trains (in bf16: norms, gate and attention through the kernels, the projection's
+  # gradient written in place) against plain torch everywhere with a dense torch attention
+  got = grads(hstu_layer._attention, True)
+  want = grads(_dense_attention, False)
+  assert set(got) == set(want) and "q_kernel" in got and "output_kernel" in got and "attn_ln_gamma" in got
   for name in want:
     err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
     assert err <= tol, (name, err)
+
+
+@pytest.mark.gpu
+def test_packed_block_trains_through_the_fused_steps(gpu):
+  """forward_jagged in bf16 with gradients: the fused training steps (kernel layer norms, attention + norm
+  + gate as one function) against the same block with torch's norms and gate around the attention
+  function, on packed tokens with timestamps and both tables; and the fused path is the one taken."""
+  from recml_amd import hstu_layer, hstu_block_ops
+  from recml_amd.hstu_layer import HSTUBlock
+  dev, bf = torch.device("cuda:0"), torch.bfloat16
+  H, hd = 4, 64
+  D = H * hd
+  gen = torch.Generator().manual_seed(9)
+  lens = [200, 1, 77, 130]
+  T, L = sum(lens), 256
+  offsets = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=dev)
+  blk = HSTUBlock(D, H, dtype=bf, device=dev, generator=gen)
+  blk.requires_grad_(True)
+  x = (torch.randn((T, D), generator=gen) * 0.5).to(dev).to(bf).requires_grad_(True)
+  pos = (torch.randn((H, 2 * L - 1), generator=gen) * 0.3).to(dev).requires_grad_(True)
+  tsb = (torch.randn((H, 33), generator=gen) * 0.3).to(dev).requires_grad_(True)
+  stamps = torch.cat([torch.cumsum(torch.randint(1, 5000, (n,), generator=gen), 0) for n in lens]).to(dev)
+  dout = torch.randn((T, D), generator=gen).to(dev).to(bf)
+  calls = []
+  real = hstu_block_ops.norm_gate_bwd
+
+  def counted(*a, **k):
+    calls.append(k.get("du_out") is not None)
+    return real(*a, **k)
+
+  def grads(fused_training):
+    if not fused_training:
+      blk._fused_training = lambda *a: False
+    try:
+      for t in [x, pos, tsb, *blk.parameters()]:
+        t.grad = None
+      out = blk.forward_jagged(x, offsets, L, pos_bias=pos, timestamps=stamps, ts_bias=tsb)
+      (out.float() * dout.float()).sum().backward()
+      return out.detach().float(), {"x": x.grad.float().clone(), "pos": pos.grad.float().clone(), "ts": tsb.grad.float().clone(),
+                                   **{n: p.grad.float().clone() for n, p in blk.named_parameters() if p.grad is not None}}
+    finally:
+      blk.__dict__.pop("_fused_training", None)
+
+  hstu_block_ops.norm_gate_bwd = counted
+  try:
+    out_f, got = grads(True)
+  finally:
+    hstu_block_ops.norm_gate_bwd = real
+  assert calls == [True, False]                       # the gate's backward writing in place, then the input norm's
+  out_t, want = grads(False)
+  assert float((out_f - out_t).abs().max() / out_t.abs().max()) <= 2e-2
+  assert set(got) == set(want) and {"u_kernel", "attn_ln_beta", "input_ln_gamma"} <= set(got)
+  for name in want:
+    err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
+    assert err <= 4e-2, (name, err)                   # bf16 activations on both sides, rounded at different points
 
 
 @pytest.mark.gpu

@@ -274,19 +274,32 @@ __global__ __launch_bounds__(256) void hstu_norm_gate_bwd(const NormGateBwdParam
 }
 
 // out[col] = sum over the nb partial rows of part[.][col], rows added in a fixed order; columns
-// [0, width) go to dgamma, [width, 2 width) to dbeta.  nb = 0 writes zeros.
-__global__ __launch_bounds__(256) void hstu_colsum(const float* __restrict__ part, int nb, int width, float* __restrict__ dgamma,
-                                                   float* __restrict__ dbeta) {
-  __shared__ float red[4][64];
-  const int cl = threadIdx.x & 63, rg = threadIdx.x >> 6;
-  const int col = blockIdx.x * 64 + cl, n2 = 2 * width;
-  float s = 0.f;
-  if (col < n2)
-    for (int r = rg; r < nb; r += 4) s += part[(int64_t)r * n2 + col];
-  red[rg][cl] = s;
+// [0, width) go to dgamma, [width, 2 width) to dbeta.  nb = 0 writes zeros.  A workgroup of 1024
+// threads takes 32 columns: 32 groups of threads each add every 32nd row (four sums in flight per
+// thread: the loop is nothing but dependent loads otherwise), then the groups' sums are added through LDS.
+__global__ __launch_bounds__(1024) void hstu_colsum(const float* __restrict__ part, int nb, int width, float* __restrict__ dgamma,
+                                                    float* __restrict__ dbeta) {
+  __shared__ float red[32][33];
+  const int cl = threadIdx.x & 31, rg = threadIdx.x >> 5;
+  const int col = blockIdx.x * 32 + cl, n2 = 2 * width;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (col < n2) {
+    const float* pc = part + col;
+    int r = rg;
+    for (; r + 96 < nb; r += 128) {
+      s0 += pc[(int64_t)r * n2];
+      s1 += pc[(int64_t)(r + 32) * n2];
+      s2 += pc[(int64_t)(r + 64) * n2];
+      s3 += pc[(int64_t)(r + 96) * n2];
+    }
+    for (; r < nb; r += 32) s0 += pc[(int64_t)r * n2];
+  }
+  red[rg][cl] = (s0 + s1) + (s2 + s3);
   __syncthreads();
   if (rg == 0 && col < n2) {
-    s = (red[0][cl] + red[1][cl]) + (red[2][cl] + red[3][cl]);
+    float s = 0.f;
+#pragma unroll
+    for (int g = 0; g < 32; ++g) s += red[g][cl];
     if (col < width) dgamma[col] = s; else dbeta[col - width] = s;
   }
 }
@@ -505,7 +518,7 @@ int hstu_norm_gate_bwd(const HstuNormGateBwdArgs* a, void* stream) {
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "norm-gate backward kernel launch: %s", hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(hstu_colsum, dim3((unsigned)((2 * a->width + 63) / 64)), dim3(256), 0, st, (const float*)a->workspace, nb, a->width,
+  hipLaunchKernelGGL(hstu_colsum, dim3((unsigned)((2 * a->width + 31) / 32)), dim3(1024), 0, st, (const float*)a->workspace, nb, a->width,
                      a->dgamma, a->dbeta);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_BLOCK_ERR_LAUNCH, "column-sum kernel launch: %s", hipGetErrorString(e));

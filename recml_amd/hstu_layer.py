@@ -167,7 +167,7 @@ class HSTUBlock(torch.nn.Module):
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       return self._train_steps(inputs.reshape(B * L, D), (B, L), pos_bias, ts_bias, batch,
                                dict(seq_lens=seq_lens, n=n, alpha=alpha, timestamps=timestamps)).reshape(B, L, D)
-    x = F.layer_norm(inputs, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
+    x = self._input_norm(inputs, fused)
     w, b = self._uqkv_weights()
     if fused:
       uqkv = hstu_block_ops.gemm_silu(x.reshape(B * L, D), w, b, True).reshape(B, L, 4, H, hd)
@@ -212,6 +212,12 @@ class HSTUBlock(torch.nn.Module):
     wants_grad = _wants_grad(t, *self.parameters(), *bias_inputs)
     return t.is_cuda and t.dtype == torch.bfloat16 and not wants_grad
 
+  def _input_norm(self, t, fused):
+    D = self.hidden_dim
+    if fused and D % 8 == 0 and D <= 8192:
+      return hstu_block_ops.layer_norm(t, self.input_ln_gamma, self.input_ln_beta, self.eps)   # one wave per row, one pass
+    return F.layer_norm(t, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
+
   def _fused_training(self, t, *bias_inputs) -> bool:
     """Whether the training form of the fused steps applies: bf16 on a GPU, something asking for a
     gradient, widths the norm kernels' backward takes."""
@@ -254,7 +260,7 @@ class HSTUBlock(torch.nn.Module):
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
       return self._train_steps(tokens, (T,), pos_bias, ts_bias, batch,
                                dict(seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha, timestamps=timestamps))
-    x = F.layer_norm(tokens, (D,), self.input_ln_gamma, self.input_ln_beta, self.eps)
+    x = self._input_norm(tokens, fused)
     w, b = self._uqkv_weights()
     if fused:
       uqkv = hstu_block_ops.gemm_silu(x, w, b, True).reshape(T, 4, H, hd)
@@ -310,8 +316,9 @@ class HSTU(torch.nn.Module):
 
   def _final_norm(self, x):
     D = self.model_dim
-    if x.is_cuda and x.dtype == torch.bfloat16 and D % 8 == 0 and D <= 2048 and _wants_grad(x, self.final_norm_gamma, self.final_norm_beta):
-      # training in bf16: the norm and its gradients in one pass each
+    training = _wants_grad(x, self.final_norm_gamma, self.final_norm_beta)
+    if x.is_cuda and x.dtype == torch.bfloat16 and D % 8 == 0 and D <= (2048 if training else 8192):
+      # bf16 on a GPU: the norm (and its gradients) in one pass each
       return hstu_block_ops.layer_norm(x, self.final_norm_gamma, self.final_norm_beta, self.eps)
     return F.layer_norm(x, (D,), self.final_norm_gamma, self.final_norm_beta, self.eps)
 

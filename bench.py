@@ -315,6 +315,18 @@ def bench_block_steps(args, dev):
   wall_t, _ = timed(lambda: u * torch.nn.functional.layer_norm(attn, (D,), gamma, beta, 1e-6))
   wall_g, ker_g = timed(lambda: recml_amd.gemm_silu(x, w, None, True))
   wall_gt, _ = timed(lambda: torch.nn.functional.silu(x @ w))
+  # the same step's gradients (training): 5 x T x D x 2 bytes (row, gate and gradient in; d_attn and d_u out),
+  # d_u into a slice of a projection-shaped tensor as the block's backward has it; and torch's autograd of the same
+  from recml_amd import hstu_block_ops
+  dout = torch.randn((T, D), device=dev, dtype=bf, generator=gen)
+  dfused = torch.empty_like(fused)
+  wall_nb, ker_nb = timed(lambda: hstu_block_ops.norm_gate_bwd(attn, u, gamma, beta, dout, 1e-6, du_out=dfused[:, 0]))
+  leaves = [t.detach().clone().requires_grad_(True) for t in (attn, u.contiguous(), gamma, beta)]
+  def torch_bwd():
+    for t in leaves:
+      t.grad = None
+    (leaves[1] * torch.nn.functional.layer_norm(leaves[0], (D,), leaves[2], leaves[3], 1e-6)).backward(dout)
+  wall_nbt, _ = timed(torch_bwd)
   # the front end: 10 M x 512 table, Zipf(1.05) ids as in the model workload, position table of 1024 rows
   vocab = 10_000_000
   table = torch.empty((vocab, D), dtype=bf, device=dev)
@@ -338,6 +350,9 @@ def bench_block_steps(args, dev):
                    "frac": nbytes / (ker_ng * 1e-3) / 1e9 / 8000.0, "traffic": None, "kernel_ms_avg": ker_ng,
                    "algorithmic_bytes": nbytes},
       "torch_layer_norm_then_mul_ms": wall_t,
+      "norm_gate_bwd": {"ms_per_call": wall_nb, "event_ms": ker_nb, "gb_per_s": 5 * T * D * 2 / (ker_nb * 1e-3) / 1e9,
+                        "frac_of_hbm_peak": 5 * T * D * 2 / (ker_nb * 1e-3) / 1e9 / 8000.0, "algorithmic_bytes": 5 * T * D * 2,
+                        "torch_forward_and_autograd_ms": wall_nbt},
       "embed_norm": {"ms_per_call": wall_e, "event_ms": ker_e, "torch_gather_add_layer_norm_ms": wall_et,
                      "unique_ids": uniq, "gb_per_s_rows_read_and_written": 2 * T * D * 2 / (ker_e * 1e-3) / 1e9},
       "gemm_silu": {"ms_per_call": wall_g, "event_ms": ker_g, "tflops": gflop / ker_g, "torch_mm_then_silu_ms": wall_gt,

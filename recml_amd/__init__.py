@@ -15,7 +15,7 @@ from recml_amd.hstu_ops import (  # noqa: F401
     pointwise_attention,
     pointwise_splash_attention,
 )
-from recml_amd.hstu_block_ops import embed_norm, gemm_silu, norm_gate  # noqa: F401
+from recml_amd.hstu_block_ops import embed_norm, gemm_silu, layer_norm, norm_gate, norm_gate_bwd  # noqa: F401
 from recml_amd.masks import make_attention_mask, make_causal_mask  # noqa: F401
 from recml_amd.hstu_layer import HSTU, HSTUBlock  # noqa: F401
 from recml_amd.hstu_bias import (  # noqa: F401

@@ -1046,7 +1046,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
   float* Kc = Kr + GT * pk;                // [32][pc]  K read across the channels for dQ^T
   float* Vr = Kc + GT * pc;                // [32][pv]  V rows for dP^T
   float* Hist = Vr + GT * pv;              // [buckets] timestamp-bucket sums of this workgroup
-  float* Ds = Hist + general_hist_len(p.ts_nb);   // [4][32][33] dS of each wave's block, [query][key] (position gradient only)
+  float* Ds = Hist + general_hist_len(p.ts_nb);   // [4][32][33] dS of each wave's block, [query][key] (position and dense-bias gradients only)
 
   const int h = blockIdx.x, b = blockIdx.y, qt = gridDim.z - 1 - blockIdx.z;
   const Seq s = seq_info(p, b, h);
@@ -1135,11 +1135,21 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
         const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-x * LOG2E));
         const float ds = keep ? dpacc[r] * sg * (1.0f + x * (1.0f - sg)) * p.inv_n : 0.f;
         sacc[r] = ds;                      // dS^T in place of S^T
-        // (dense-bias gradient: the heads' workgroups, and the sequences' for a shared bias, add into one matrix)
-        if (p.dbias && ds != 0.f)
-          atomicAdd(p.dbias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)qi * p.Lkv + j, ds);
         if (want_ts && ds != 0.f) __hip_atomic_fetch_add((general_lds_float_ptr)(Hist + bk), ds, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (want_pos) dsw[m * (GT + 1) + 8 * (r >> 2) + 4 * hh + (r & 3)] = ds;
+        if (want_pos || p.dbias) dsw[m * (GT + 1) + 8 * (r >> 2) + 4 * hh + (r & 3)] = ds;
+      }
+      if (p.dbias) {
+        // Dense-bias gradient: the heads' workgroups, and the sequences' for a shared bias, add into one matrix.
+        // A lane's own 16 pairs lie in one row of it, so added from the accumulators one instruction would touch
+        // 32 rows; read back from the wave's LDS by rows (its operations run in order), an instruction adds two
+        // whole rows of the block: two cache lines instead of 32.
+        float* dbp = p.dbias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)r0 * p.Lkv + kv0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int row = 2 * i + (lane >> 5), col = lane & 31;
+          const float v = dsw[row * (GT + 1) + col];
+          if (v != 0.f) atomicAdd(dbp + (int64_t)row * p.Lkv + col, v);      // zero wherever the pair is masked or outside
+        }
       }
       if (want_pos) {
         // one sum per diagonal of the wave's 32 x 32 block (the wave's own LDS: its operations run in order)
@@ -4139,7 +4149,8 @@ template <typename T>
 int launch_bwd(const Params& p, hipStream_t st) {
   if (p.B > 65535) return fail(HSTU_ERR_SHAPE, "the general backward takes at most 65535 sequences per call, got %d", p.B);
   if (p.d_qk <= 128 && p.d_v <= 128) {
-    const bool want_pos = p.dpos != nullptr && p.pos_tab != nullptr;
+    // (each wave's block of dS goes through LDS for the position table's diagonal sums and for the dense bias's row-wise adds)
+    const bool want_pos = (p.dpos != nullptr && p.pos_tab != nullptr) || p.dbias != nullptr;
     const int smem_q = 4 * general_bwd_dq_lds(p.d_qk, p.d_v, want_pos, p.ts_nb), smem_kv = 4 * general_bwd_dkv_lds(p.d_qk, p.d_v);
     static int granted_q[64], granted_kv[64];
     if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T>, smem_q, granted_q)) return rc;

@@ -284,6 +284,76 @@ __device__ __forceinline__ void general_mask_words_col(const Params& p, int b, i
   for (int g = 0; g < 4; ++g)
     w[g] = (uint32_t)v[4 * g] | ((uint32_t)v[4 * g + 1] << 8) | ((uint32_t)v[4 * g + 2] << 16) | ((uint32_t)v[4 * g + 3] << 24);
 }
+// The explicit mask's live steps for one workgroup's tile, found by one pass of its 256 threads over the tile's
+// bytes before the step loop (an L x Lkv mask is mostly zeros when it carries the causal rule, and a step the mask
+// empties still costs its tile loads and barriers):
+//   ROWS:  rows [t0, t0 + 128) -> the 32-key steps [lo, hi) outside of which every byte of those rows is zero;
+//   !ROWS: keys [t0, t0 + 128) -> the 32-row steps likewise.
+// Reads 16 bytes per lane: where Lkv or the pointer does not allow that, the full range comes back.  Every
+// thread of the workgroup must call it (one barrier inside).
+template <bool ROWS>
+__device__ __forceinline__ void general_mask_live_steps(const Params& p, int b, int t0, int tid, int& lo, int& hi) {
+  // (lo, hi come in as the range of steps the other rules leave: only that part of the mask is looked at)
+  __shared__ int ends[4][2];
+  const int s_lo = lo, s_hi = hi;
+  if ((p.Lkv & 15) != 0 || ((uintptr_t)p.mask & 15) != 0 || s_lo >= s_hi) return;
+  const uint8_t* mb = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0);
+  const int lane = tid & 63, w = tid >> 6;
+  int mn = 0x7fffffff, mx = -1;
+  if (ROWS) {
+    // wave w: rows t0 + 32 w .. + 31 (clamped into the matrix); lane: 16-byte chunks lane, lane + 64, ... of a row
+    const int n_chunks = (p.Lkv >> 4) < 2 * s_hi ? (p.Lkv >> 4) : 2 * s_hi;
+    for (int c = 2 * s_lo + lane; c < n_chunks; c += 64) {
+      uint32_t any = 0u;
+#pragma unroll 8
+      for (int rr = 0; rr < 32; ++rr) {
+        int r = t0 + 32 * w + rr;
+        r = r < p.L - 1 ? r : p.L - 1;
+        const uint4 v = *(const uint4*)(mb + (int64_t)r * p.Lkv + 16 * c);
+        any |= v.x | v.y | v.z | v.w;
+      }
+      if (any != 0u) {
+        mn = mn < (c >> 1) ? mn : (c >> 1);
+        mx = mx > (c >> 1) ? mx : (c >> 1);
+      }
+    }
+  } else {
+    // 8 chunks per row cover the 128 keys; a wave's instruction reads 8 rows: wave w takes rows 32 i + 8 w + lane / 8
+    const int ch = lane & 7;
+    const bool col_ok = t0 + 16 * ch < p.Lkv;
+#pragma unroll 4
+    for (int i = s_lo; i < s_hi; ++i) {
+      const int r = 32 * i + 8 * w + (lane >> 3);
+      if (col_ok && r < p.L) {
+        const uint4 v = *(const uint4*)(mb + (int64_t)r * p.Lkv + t0 + 16 * ch);
+        if ((v.x | v.y | v.z | v.w) != 0u) {
+          mn = mn < i ? mn : i;
+          mx = mx > i ? mx : i;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int dl = 32; dl >= 1; dl >>= 1) {
+    const int on = __shfl_xor(mn, dl, 64), ox = __shfl_xor(mx, dl, 64);
+    mn = mn < on ? mn : on;
+    mx = mx > ox ? mx : ox;
+  }
+  if (lane == 0) {
+    ends[w][0] = mn;
+    ends[w][1] = mx;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    mn = mn < ends[x][0] ? mn : ends[x][0];
+    mx = mx > ends[x][1] ? mx : ends[x][1];
+  }
+  // (the same in every lane, and said so: loop bounds derived from these must stay scalar)
+  lo = __builtin_amdgcn_readfirstlane(mx < 0 ? s_lo : mn);
+  hi = __builtin_amdgcn_readfirstlane(mx < 0 ? s_lo : mx + 1);             // nothing kept at all: an empty range
+}
+
 // The dense bias of the same 16 pairs (query row fixed / key fixed), fetched together ahead of their use: four
 // 16-byte loads where the rows allow, else one load per pair; indices clamped into the matrix like the mask's.
 __device__ __forceinline__ void general_dense_row(const Params& p, int b, int i, int j0, int hh, float (&v)[16]) {
@@ -443,6 +513,20 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
   const bool kvec = (((uintptr_t)(kp_ + s.bk) & VMASK) == 0) && (p.k_st & 3) == 0;
   const bool vvec = (((uintptr_t)(vp + s.bv) & VMASK) == 0) && (p.v_st & 3) == 0;
 
+  // the key steps of this tile (found first, while nothing else is held in registers)
+  int kv_end = s.n_kv;
+  if (p.causal && q0 + GQ < kv_end) kv_end = q0 + GQ;
+  if (p.window >= 0 && q0 + GQ + p.window < kv_end) kv_end = q0 + GQ + p.window;
+  int kv_begin = 0;
+  if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
+  if (p.mask && q0 < s.n_q) {
+    // the steps before the first and after the last key the mask keeps for these rows are left out
+    int t_lo = kv_begin / GT, t_hi = (kv_end + GT - 1) / GT;
+    general_mask_live_steps<true>(p, b, q0, tid, t_lo, t_hi);
+    kv_begin = t_lo * GT > kv_begin ? t_lo * GT : kv_begin;
+    kv_end = t_hi * GT < kv_end ? t_hi * GT : kv_end;
+  }
+
   floatx16 o[NB];
 #pragma unroll
   for (int x = 0; x < NB; ++x)
@@ -466,11 +550,6 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
         }
       }
     }
-    int kv_end = s.n_kv;
-    if (p.causal && q0 + GQ < kv_end) kv_end = q0 + GQ;
-    if (p.window >= 0 && q0 + GQ + p.window < kv_end) kv_end = q0 + GQ + p.window;
-    int kv_begin = 0;
-    if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
     const int vcols = nblk * 32;
     // The next tile travels in registers while this one is computed on.  When bases and strides allow whole
     // groups and the head dims are multiples of four, the loads are unconditional (rows past the sequence
@@ -1081,6 +1160,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
     if (p.window >= 0 && q0 + 128 + p.window < kv_end) kv_end = q0 + 128 + p.window;
     int kv_begin = 0;
     if (p.window >= 0 && q0 - p.window > 0) kv_begin = ((q0 - p.window) / GT) * GT;
+    if (p.mask) {
+      // the steps before the first and after the last key the mask keeps for these rows are left out
+      int t_lo = kv_begin / GT, t_hi = (kv_end + GT - 1) / GT;
+      general_mask_live_steps<true>(p, b, q0, tid, t_lo, t_hi);
+      kv_begin = t_lo * GT > kv_begin ? t_lo * GT : kv_begin;
+      kv_end = t_hi * GT < kv_end ? t_hi * GT : kv_end;
+    }
     GeneralTile<T, 4> kt_, vt_;
     if (kv_begin < kv_end) {
       kt_.fetch(kp_, p.k_st, kv_begin, s.n_kv, dq, kfast, tid);
@@ -1238,6 +1324,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
     if (p.window >= 0 && k0 - p.window > q_begin) q_begin = k0 - p.window;
     if (p.window >= 0 && k0 + 128 + p.window < q_end) q_end = k0 + 128 + p.window;
     q_begin = (q_begin / GT) * GT;
+    if (p.mask) {
+      // the steps before the first and after the last row for which the mask keeps one of these keys are left out
+      int t_lo = q_begin / GT, t_hi = (q_end + GT - 1) / GT;
+      general_mask_live_steps<false>(p, b, k0, tid, t_lo, t_hi);
+      q_begin = t_lo * GT > q_begin ? t_lo * GT : q_begin;
+      q_end = t_hi * GT < q_end ? t_hi * GT : q_end;
+    }
     GeneralTile<T, 4> qt_, ot_;
     if (q_begin < q_end) {
       qt_.fetch(qp, p.q_st, q_begin, s.n_q, dq, qfast, tid);

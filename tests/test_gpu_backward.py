@@ -527,3 +527,50 @@ def test_dense_bias_gradient(gpu, d, shared, storage):
                                           mask=_dev(mask), bias=bt)
   (out.float() * _dev(dout)).sum().backward()
   assert _rel(bt.grad.cpu().numpy(), want[5]) <= (tol if storage == "fp32" else 2e-2)
+
+
+@pytest.mark.parametrize("shape", ["band", "blocks", "ragged16", "offset_view", "empty_tile"])
+def test_general_kernels_leave_out_the_steps_a_mask_empties(gpu, shape):
+  """The general kernels find, per tile, the first and last step an explicit mask keeps anything in and run
+  only those.  Masks whose live range is cut on both sides, per row tile and per key tile: a band, diagonal
+  blocks, a tile the mask empties altogether; and the two layouts that switch the search off (a key length
+  that is no multiple of 16, a mask view that starts off a 16-byte boundary).  Forward and backward in fp32
+  against the oracle, the dense bias's gradient included."""
+  rng = np.random.default_rng(7300 + len(shape))
+  B, L, H, d = 2, 400, 2, 32
+  Lk = 400 if shape != "ragged16" else 390
+  i, j = np.arange(L)[:, None], np.arange(Lk)[None, :]
+  if shape in ("band", "ragged16", "offset_view"):
+    mask = (j <= i) & (j >= i - 70)                      # a band: live keys start late and end early for most tiles
+  elif shape == "blocks":
+    mask = (i // 96) == (j // 96)                        # diagonal blocks that straddle the 128-row tiles
+  else:
+    mask = (j <= i) & ~((i >= 128) & (i < 256))          # rows 128..255 keep nothing: one whole row tile is empty
+    mask &= ~((j >= 256) & (j < 384))                    # and so is one whole key tile
+  mask = np.broadcast_to(mask, (B, L, Lk)) & (rng.random((B, L, Lk)) < 0.9)
+  q = rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.4
+  k, v = (rng.standard_normal((B, Lk, H, d)).astype(np.float32) * 0.4 for _ in range(2))
+  dout = rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.4
+  bias = (rng.standard_normal((B, L, Lk)) * 0.4).astype(np.float32)
+  want_out = O.hstu_attention_ref(q, k, v, n=7.0, alpha=0.3, causal=False, mask=mask, bias=bias)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, n=7.0, alpha=0.3, causal=False, mask=mask, bias=bias, bias_grad=True)
+  md = _dev(mask.astype(np.uint8))
+  if shape == "offset_view":
+    flat = torch.zeros(B * L * Lk + 16, dtype=torch.uint8, device=md.device)
+    flat[5: 5 + B * L * Lk] = md.reshape(-1)
+    md = flat[5: 5 + B * L * Lk].view(B, L, Lk)
+    assert md.data_ptr() % 16 != 0
+  args = [_dev(t) for t in (q, k, v)]
+  out = recml_amd.hstu_attention(*args, n=7.0, alpha=0.3, causal=False, mask=md, bias=_dev(bias))
+  variant = []
+  got = recml_amd.hstu_attention_bwd(*args, _dev(dout), n=7.0, alpha=0.3, causal=False, mask=md, bias=_dev(bias),
+                                     bias_grad=True, _variant_out=variant)
+  torch.cuda.synchronize()
+  assert variant[-1].startswith("hstu_bwd_general")
+  assert _rel(out.cpu().numpy(), want_out) <= 2e-5
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(g.cpu().numpy(), w) <= 2e-5, nm
+  assert _rel(got[5].cpu().numpy(), want[5]) <= 2e-5
+  if shape == "empty_tile":
+    assert float(out[:, 128:256].abs().max()) == 0 and float(got[0][:, 128:256].abs().max()) == 0
+    assert float(got[1][:, 256:384].abs().max()) == 0 and float(got[2][:, 256:384].abs().max()) == 0

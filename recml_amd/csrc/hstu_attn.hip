@@ -3018,6 +3018,7 @@ __device__ __forceinline__ void store_rows(const floatx16 (&acc)[D / 32], float 
 // wave, then one sum per bucket for the workgroup.  Kept this small on purpose: with both biases at
 // d = 128 the kernel's LDS is 78 KB, and two workgroups must still fit a CU's 160 KB.
 constexpr int TG_RING = 128;
+constexpr int TG_WG_RING = 256;      // the workgroup's ring of diagonal sums (within the NWAVES * TG_RING floats set aside)
 constexpr int BWD_TG_BYTES = (NWAVES * TG_RING + TS_TAB_LEN) * 4;
 
 // v of the lane `CTRL` names (data-parallel-primitive controls of the vector ALU: 0x110 + n = n lanes
@@ -3046,13 +3047,13 @@ __device__ __forceinline__ void lds_atomic_add(float* lds_location, float v) {
 }
 
 // TG: also accumulate the table gradients.  Every pair adds its dS to the entry of each table its
-// logit read; LDS float atomics turned out to cost about 4 cycles per lane, so the sums are formed
-// in registers first and each wave keeps its own LDS accumulators, updated without atomics.
-// Position table: pair (q, key) of a wave lies on diagonal X = key - q + (r0 + 31) >= 0.  A block's
+// logit read; LDS float atomics with many lanes on one address turned out to cost about 4 cycles per
+// lane, so the sums are formed in registers first and reach LDS one lane per address.
+// Position table: pair (q, key) of a workgroup lies on diagonal X = key - q + (q0 + 127) >= 0.  A block's
 // 32 x 32 pairs are brought onto their 63 diagonals by lane permutes (see the block), one value per
-// lane, and added to the wave's ring of sums.  Block t only touches X in [32 t, 32 t + 63), so
-// everything below 32 (t + 1) is final after it: every second block the wave adds 64 finished
-// diagonals to the table in memory and clears them.
+// lane, and added to the workgroup's ring of sums.  The blocks of a pair of steps (t, t + 1) only touch
+// X in [32 t, 32 t + 192), so everything below 32 (t + 2) is final after the pair's barrier: at the start
+// of the next pair one wave adds those 64 diagonals to the table in memory and clears them.
 // Bucket table: where each lane has one bucket for the whole block (or two neighbours), lanes with
 // the same bucket are summed across the wave and one lane adds the sum to the workgroup's
 // histogram (an LDS atomic, but of one lane); only blocks with more buckets per lane use one
@@ -3386,7 +3387,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       // keep the 16 permute addresses of the loop below in registers across the whole key loop, which
       // this kernel does not have)
       int jj = m + 4 * hh;
-      asm volatile("" : "+v"(jj));
+      if (D == 128) asm volatile("" : "+v"(jj));        // (smaller head dims have the 16 registers)
       const int half4 = (lane & 32) << 2;
       float s_all = 0.f, s_low = 0.f;
 #pragma unroll
@@ -3400,8 +3401,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       const float s_high = s_all - s_low;
       const float mine = hh ? s_high : s_low, theirs = hh ? s_low : s_high;
       const float got = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, theirs)));
-      float* slot = TgBase + w * TG_RING + ((kbs + 31 - m + 32 * hh) & (TG_RING - 1));
-      *slot += mine + got;
+      // the workgroup's ring of diagonal sums: this wave's diagonal X is the workgroup's X + 96 - 32 w (a lane per
+      // slot within the instruction; other waves may add to the same slots, hence the atomic form)
+      lds_atomic_add(TgBase + ((kbs + 127 - m + 32 * hh - 32 * w) & (TG_WG_RING - 1)), mine + got);
     }
     if (want_dts) {
       float* hist = TgBase + NWAVES * TG_RING;
@@ -3474,12 +3476,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
     }
   };
 
-  // adds diagonals [x0, x0 + 64) of this wave's ring to the table in memory and clears them
+  // adds diagonals [x0, x0 + 64) of the workgroup's ring to the table in memory and clears them (one wave's job)
   auto flush_diag = [&](int x0) {
-    float* slot = TgBase + w * TG_RING + ((x0 + lane) & (TG_RING - 1));
+    float* slot = TgBase + ((x0 + lane) & (TG_WG_RING - 1));
     const float val = *slot;
     *slot = 0.f;
-    const int idx = (p.L - 1) + (x0 + lane) - 31 - r0;
+    const int idx = (p.L - 1) + (x0 + lane) - (BM - 1) - q0;
     if (val != 0.f && idx >= 0 && idx < 2 * p.L - 1)
       atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, val * p.inv_n);
   };
@@ -3490,24 +3492,27 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   static_assert(NSTAGE == 4, "two pairs of stages");
   HSTU_WAIT_VMCNT(0);
   __syncthreads();
+  // Position-table gradient: the four waves add their blocks' diagonal sums into ONE ring of the workgroup
+  // (diagonal X = key - row + q0 + 127; the blocks of step pair (t, t + 1) touch [32 t, 32 t + 192)), and what a
+  // pair has completed -- [32 t, 32 t + 64), final once every wave is past the pair's barrier -- goes to memory
+  // at the start of the next pair, by one wave in turn.  Every workgroup of the launch adds into the one table:
+  // with a ring per wave, each flushing its own 64 diagonals per pair, those adds (four times as many) cost a
+  // config-4 layer 0.19 of the 0.31 ms the table gradient took.
   for (int t = t_lo; t < nt; t += 2) {
+    if (want_dpos && t > t_lo && w == ((t >> 1) & 3)) flush_diag(32 * (t - 2));
     if (t + 2 < nt) dma_step(t + 2);
     if (t + 3 < nt) dma_step(t + 3);
 #pragma unroll
     for (int u = t; u < t + 2; ++u) {
-      if (u < nt && u * BN <= wave_last && (win < 0 || u * BN + 31 + win >= r0)) {
-        block(u);
-        if (want_dpos && (u & 1) == 1) flush_diag(32 * (u - 1));
-      }
+      if (u < nt && u * BN <= wave_last && (win < 0 || u * BN + 31 + win >= r0)) block(u);
     }
     HSTU_WAIT_VMCNT(0);
     __syncthreads();
   }
-
-  if (want_dpos && wave_last >= 0) {
-    // what the wave has not written out: the diagonals of its last block if their number is odd, then 31 more
-    const int t_done = wave_last / BN + 1;
-    flush_diag(32 * (t_done & ~1));
+  if (want_dpos && t_lo < nt && w < 3) {
+    // what the last pair left in the ring (every wave is past the loop's last barrier)
+    const int t_last = t_lo + ((nt - 1 - t_lo) & ~1);
+    flush_diag(32 * t_last + 64 * w);
   }
   if (want_dts) {
     // every wave is past the loop's last barrier: the histogram is complete

@@ -260,6 +260,28 @@ def bench_model(args, dev):
   torch.cuda.synchronize()
   train_ms = (time.perf_counter() - t0) * 1e3 / steps
   assert bool(torch.isfinite(pos_t.grad).all()) and float(pos_t.grad.abs().max()) > 0
+  # the same step with torch left to pick each matrix product's kernel by timing the candidates once
+  # (torch.cuda.tunable: the products are torch's, and the library's first choice for the weight
+  # gradients' shapes -- a small output, 70 k rows to sum over -- leaves most of the chip idle)
+  train_tuned_ms = None
+  try:
+    import torch.cuda.tunable as tunable
+    import tempfile
+    tunable.enable(True)
+    tunable.set_filename(os.path.join(tempfile.gettempdir(), "recml_amd_bench_tuned_products.csv"))   # (it writes its choices at exit)
+    tunable.set_max_tuning_duration(15)
+    tunable.set_max_tuning_iterations(10)
+    for _ in range(warm):
+      train_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+      train_step()
+    torch.cuda.synchronize()
+    train_tuned_ms = (time.perf_counter() - t0) * 1e3 / steps
+    tunable.enable(False)
+  except Exception as e:   # an older torch without the module, or a tuning failure: the plain figure stands
+    print(f"tunable products not measured: {e}", file=sys.stderr)
   nn = lens.astype(np.int64)
   attn_flops = int((H * (nn * (nn + 1) // 2) * 4 * (D // H)).sum()) * layers
   proj_flops = B * L * (2 * D * 4 * D + 2 * D * D) * layers
@@ -271,6 +293,7 @@ def bench_model(args, dev):
       "ms_per_step_packed_tokens": ms_jagged, "seqs_per_s_packed_tokens": B / (ms_jagged * 1e-3),
       "packed_vs_padded_max_abs_over_max": jag_err,
       "train_fwd_bwd_ms_packed_tokens": train_ms,
+      "train_fwd_bwd_ms_packed_tokens_tuned_products": train_tuned_ms,
       "attention_ms_per_layer": att_ms, "attention_share": layers * att_ms / ms,
       "attention_gflop_unmasked": attn_flops / 1e9, "projection_gflop_padded": proj_flops / 1e9,
       "model_tflops": (attn_flops + proj_flops) / (ms * 1e-3) / 1e12}))

@@ -377,10 +377,11 @@ class HSTU(torch.nn.Module):
     valid = torch.arange(L, device=inputs.device)[None, :] < lens[:, None]          # [B, L]
     offsets = torch.zeros(B + 1, dtype=torch.int32, device=inputs.device)
     offsets[1:] = torch.cumsum(lens, 0)
-    ids = inputs[valid]                                                              # [T], sequence-major
-    pos_idx = None
-    if self.position_embedding is not None:
-      pos_idx = torch.arange(L, device=inputs.device)[None, :].expand(B, L)[valid]
+    # the flat positions of the valid tokens, sequence-major: found once (the one host wait of the packing:
+    # the token count) and used for every gather and for the scatter at the end
+    where = valid.reshape(-1).nonzero().squeeze(1)                                   # [T]
+    ids = inputs.reshape(-1)[where]
+    pos_idx = where % L if self.position_embedding is not None else None
     if self._fused_front_end():
       x = self._embed_norm(ids, pos_idx)
     else:
@@ -390,13 +391,12 @@ class HSTU(torch.nn.Module):
       if pos_idx is not None:
         x = x + self.position_embedding[pos_idx]
       x = self._final_norm(x)
-    ts = None if timestamps is None else timestamps[valid]
+    ts = None if timestamps is None else timestamps.reshape(-1)[where]
     batch = hstu_ops.AttentionBatch()
     for block in self.decoder_blocks:
       x = block.forward_jagged(x, offsets, L, pos_bias=pos_bias, timestamps=ts, ts_bias=ts_bias, batch=batch)
     x = self._final_norm(x)
     if self.reverse_embedding is not None:
       x = x @ self.reverse_embedding
-    out = torch.zeros((B, L, x.shape[-1]), dtype=x.dtype, device=x.device)
-    out[valid] = x
-    return out
+    out = torch.zeros((B * L, x.shape[-1]), dtype=x.dtype, device=x.device)
+    return out.index_copy(0, where, x).reshape(B, L, x.shape[-1])

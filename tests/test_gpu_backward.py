@@ -574,3 +574,31 @@ def test_general_kernels_leave_out_the_steps_a_mask_empties(gpu, shape):
   if shape == "empty_tile":
     assert float(out[:, 128:256].abs().max()) == 0 and float(got[0][:, 128:256].abs().max()) == 0
     assert float(got[1][:, 256:384].abs().max()) == 0 and float(got[2][:, 256:384].abs().max()) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gradients_written_into_given_slices(gpu, dtype):
+  """grads_out: dq, dk, dv land in the slices of one tensor laid out like a fused projection (what the block's
+  backward hands over), bit for bit what the call returns on its own, and nothing else of that tensor is
+  touched; buffers of another layout are refused."""
+  rng = np.random.default_rng(8100)
+  B, L, H, d = 2, 200, 2, 64
+  fused = _dev(rng.standard_normal((B, L, 4, H, d)).astype(np.float32) * 0.4, dtype)
+  q, k, v = fused[:, :, 1], fused[:, :, 2], fused[:, :, 3]
+  dout = _dev(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.4, dtype)
+  lens = _dev(np.array([200, 77], np.int32))
+  pos = _dev((rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32))
+  want = recml_amd.hstu_attention_bwd(q, k, v, dout, seq_lens=lens, pos_bias=pos)
+  grad = torch.full_like(fused, 7.0)
+  got = recml_amd.hstu_attention_bwd(q, k, v, dout, seq_lens=lens, pos_bias=pos,
+                                     grads_out=(grad[:, :, 1], grad[:, :, 2], grad[:, :, 3]))
+  torch.cuda.synchronize()
+  for i in range(3):
+    assert got[i].data_ptr() == grad[:, :, 1 + i].data_ptr()
+    assert torch.equal(grad[:, :, 1 + i], want[i])
+  assert bool((grad[:, :, 0] == 7.0).all())
+  # the position table's gradient is summed by atomic adds in an order that varies: equal to rounding
+  assert _rel(got[3].cpu().numpy(), want[3].cpu().numpy()) <= 1e-5
+  with pytest.raises(ValueError, match="grads_out"):
+    recml_amd.hstu_attention_bwd(q, k, v, dout, seq_lens=lens, pos_bias=pos,
+                                 grads_out=(torch.empty_like(q), grad[:, :, 2], grad[:, :, 3]))

@@ -1102,6 +1102,65 @@ __device__ __forceinline__ void general_dot_cols(floatx16 (&out)[NB], const floa
   }
 }
 
+// ---- the same products on the bf16 matrix cores, for tensors stored in bf16 (BP instances of the two kernels) ----
+// Every operand of the first two products is then a bf16 value, so v_mfma_f32_32x32x16_bf16 forms the same
+// products and fp32 sums in one instruction per 16 channels instead of eight per 16; P and dS are rounded to
+// bf16 for the last products, as the forward rounds P.  The instruction leaves its result in the same lanes and
+// registers as the fp32 one, so everything between the products is shared.  Tiles stay in LDS as they are
+// (fp32, both layouts) and are packed on the way into the instruction.
+__device__ __forceinline__ uint32_t general_pack_bf16(float lo, float hi) {
+  floatx2 f = {lo, hi};
+  typedef bf16_t bf16x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+// The lane's share of a bf16 row as the B operand: channels 16 ks + 8 hh .. + 7 (16-byte reads: d a multiple
+// of 16, rows on 16-byte boundaries); zeros when the row does not exist.
+__device__ __forceinline__ void general_row_frag_bf16(bf16x8 (&f)[8], const bf16_t* row, int d, bool row_ok, int hh) {
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    uint4 v = {0u, 0u, 0u, 0u};
+    if (16 * ks < d && row_ok) v = *(const uint4*)(row + 16 * ks + 8 * hh);
+    f[ks] = __builtin_bit_cast(bf16x8, v);
+  }
+}
+// acc += A B^T over the channels: `arow` = the lane's row of the fp32 tile + 8 hh (8-byte reads)
+__device__ __forceinline__ void general_dot_rows_bf16(floatx16& acc, const float* arow, const bf16x8 (&bf)[8], int d) {
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    if (16 * ks < d) {
+      const float2 a0 = *(const float2*)(arow + 16 * ks), a1 = *(const float2*)(arow + 16 * ks + 2);
+      const float2 a2 = *(const float2*)(arow + 16 * ks + 4), a3 = *(const float2*)(arow + 16 * ks + 6);
+      const uint4 pa = {general_pack_bf16(a0.x, a0.y), general_pack_bf16(a1.x, a1.y), general_pack_bf16(a2.x, a2.y),
+                        general_pack_bf16(a3.x, a3.y)};
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pa), bf[ks], acc, 0, 0, 0);
+    }
+  }
+}
+// out[x]^T += A^T B over the tile's 32 rows, 16 at a time: B = the accumulator's values 8 cc .. 8 cc + 7 (rows
+// 16 cc + 4 hh + tt and 16 cc + 8 + 4 hh + tt), A = channel 32 x + m of the same rows (`acol` = tile + 4 hh rows + m)
+template <int NB>
+__device__ __forceinline__ void general_dot_cols_bf16(floatx16 (&out)[NB], const float* acol, int pitch, const floatx16& bv, int nblk) {
+#pragma unroll
+  for (int cc = 0; cc < 2; ++cc) {
+    const uint4 pb = {general_pack_bf16(bv[8 * cc + 0], bv[8 * cc + 1]), general_pack_bf16(bv[8 * cc + 2], bv[8 * cc + 3]),
+                      general_pack_bf16(bv[8 * cc + 4], bv[8 * cc + 5]), general_pack_bf16(bv[8 * cc + 6], bv[8 * cc + 7])};
+#pragma unroll
+    for (int x = 0; x < NB; ++x) {
+      if (x < nblk) {
+        float a[8];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          a[tt] = acol[(16 * cc + tt) * pitch + 32 * x];
+          a[4 + tt] = acol[(16 * cc + 8 + tt) * pitch + 32 * x];
+        }
+        const uint4 pa = {general_pack_bf16(a[0], a[1]), general_pack_bf16(a[2], a[3]), general_pack_bf16(a[4], a[5]),
+                          general_pack_bf16(a[6], a[7])};
+        out[x] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pa), __builtin_bit_cast(bf16x8, pb), out[x], 0, 0, 0);
+      }
+    }
+  }
+}
+
 // LDS floats of the two kernels (host and device agree through these)
 __host__ __device__ inline int general_bwd_dq_lds(int dq, int dv, bool want_pos, int ts_nb) {
   return GT * (general_pitch_qk(dq) + general_pitch_v(dq) + general_pitch_qk(dv)) + (want_pos ? 4 * GT * (GT + 1) : 0) + general_hist_len(ts_nb);
@@ -1113,7 +1172,7 @@ __host__ __device__ inline int general_bwd_dkv_lds(int dq, int dv) {
 // dQ and the table gradients: one workgroup per 128 query rows of one (sequence, head), 32 per wave, keys streamed.
 //   S^T = K Q^T, dP^T = V dO^T (A = K / V rows, B = the wave's Q / dO rows in registers), dS^T pointwise,
 //   dQ^T += K^T dS^T (A = K read across the channels, B = dS^T as it leaves the pointwise part).
-template <typename T>
+template <typename T, bool BP = false>
 __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
   extern __shared__ __attribute__((aligned(16))) float gsm[];
   const int dq = p.d_qk, dv = p.d_v;
@@ -1151,9 +1210,15 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
     for (int r = 0; r < 16; ++r) o[x][r] = 0.f;
 
   if (q0 < s.n_q) {
-    float2 qf[32], dof[32];
-    general_row_frag(qf, qp + (int64_t)qi * p.q_st, dq, qi < s.n_q, hh);
-    general_row_frag(dof, dop + (int64_t)qi * p.o_st, dv, qi < s.n_q, hh);
+    float2 qf[BP ? 1 : 32], dof[BP ? 1 : 32];
+    bf16x8 qb[BP ? 8 : 1], dob[BP ? 8 : 1];
+    if constexpr (BP) {
+      general_row_frag_bf16(qb, (const bf16_t*)(qp + (int64_t)qi * p.q_st), dq, qi < s.n_q, hh);
+      general_row_frag_bf16(dob, (const bf16_t*)(dop + (int64_t)qi * p.o_st), dv, qi < s.n_q, hh);
+    } else {
+      general_row_frag(qf, qp + (int64_t)qi * p.q_st, dq, qi < s.n_q, hh);
+      general_row_frag(dof, dop + (int64_t)qi * p.o_st, dv, qi < s.n_q, hh);
+    }
     if (want_ts) for (int e = tid; e <= p.ts_nb; e += 256) Hist[e] = 0.f;
     int kv_end = s.n_kv;
     if (p.causal && q0 + 128 < kv_end) kv_end = q0 + 128;
@@ -1206,8 +1271,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
       floatx16 sacc, dpacc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
-      general_dot_rows(sacc, Kr + m * pk + 2 * hh, qf, dq4);
-      general_dot_rows(dpacc, Vr + m * pv + 2 * hh, dof, dv4);
+      if constexpr (BP) {
+        general_dot_rows_bf16(sacc, Kr + m * pk + 8 * hh, qb, dq);
+        general_dot_rows_bf16(dpacc, Vr + m * pv + 8 * hh, dob, dv);
+      } else {
+        general_dot_rows(sacc, Kr + m * pk + 2 * hh, qf, dq4);
+        general_dot_rows(dpacc, Vr + m * pv + 2 * hh, dof, dv4);
+      }
       // lane holds pair (query qi, key kv0 + 8g + 4hh + tt), r = 4g + tt
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -1251,7 +1321,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
             atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, sum);
         }
       }
-      general_dot_cols<NB>(o, Kc + (4 * hh) * pc + m, pc, sacc, nblk);
+      if constexpr (BP) general_dot_cols_bf16<NB>(o, Kc + (4 * hh) * pc + m, pc, sacc, nblk);
+      else general_dot_cols<NB>(o, Kc + (4 * hh) * pc + m, pc, sacc, nblk);
     }
     if (want_ts) {
       __syncthreads();
@@ -1278,7 +1349,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
 // dK and dV: one workgroup per 128 keys of one (sequence, head), 32 per wave, query rows streamed 32 at a time.
 //   S = Q K^T, dP = dO V^T (A = Q / dO rows, B = the wave's K / V rows in registers), P and dS pointwise,
 //   dV^T += dO^T P, dK^T += Q^T dS (A = dO / Q read across the channels, B = P / dS as they leave the pointwise part).
-template <typename T>
+template <typename T, bool BP = false>
 __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
   extern __shared__ __attribute__((aligned(16))) float gsm[];
   const int dq = p.d_qk, dv = p.d_v;
@@ -1315,9 +1386,15 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
     for (int r = 0; r < 16; ++r) { ak[x][r] = 0.f; av[x][r] = 0.f; }
 
   if (k0 < s.n_kv) {
-    float2 kf[32], vf[32];
-    general_row_frag(kf, kp_ + (int64_t)kj * p.k_st, dq, kj < s.n_kv, hh);
-    general_row_frag(vf, vp + (int64_t)kj * p.v_st, dv, kj < s.n_kv, hh);
+    float2 kf[BP ? 1 : 32], vf[BP ? 1 : 32];
+    bf16x8 kb[BP ? 8 : 1], vb[BP ? 8 : 1];
+    if constexpr (BP) {
+      general_row_frag_bf16(kb, (const bf16_t*)(kp_ + (int64_t)kj * p.k_st), dq, kj < s.n_kv, hh);
+      general_row_frag_bf16(vb, (const bf16_t*)(vp + (int64_t)kj * p.v_st), dv, kj < s.n_kv, hh);
+    } else {
+      general_row_frag(kf, kp_ + (int64_t)kj * p.k_st, dq, kj < s.n_kv, hh);
+      general_row_frag(vf, vp + (int64_t)kj * p.v_st, dv, kj < s.n_kv, hh);
+    }
     // query rows that can see these keys
     int q_begin = 0, q_end = s.n_q;
     if (p.causal) q_begin = k0;
@@ -1369,8 +1446,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
       floatx16 sacc, dpacc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
-      general_dot_rows(sacc, Qr + m * pqr + 2 * hh, kf, dq4);
-      general_dot_rows(dpacc, Or + m * por + 2 * hh, vf, dv4);
+      if constexpr (BP) {
+        general_dot_rows_bf16(sacc, Qr + m * pqr + 8 * hh, kb, dq);
+        general_dot_rows_bf16(dpacc, Or + m * por + 8 * hh, vb, dv);
+      } else {
+        general_dot_rows(sacc, Qr + m * pqr + 2 * hh, kf, dq4);
+        general_dot_rows(dpacc, Or + m * por + 2 * hh, vf, dv4);
+      }
       // MFMA rows are the A operand's rows: lane holds pair (query i0 + 8g + 4hh + tt, key ... ) -- see below
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -1385,8 +1467,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
         sacc[r] = keep ? x * sg * p.inv_n : 0.f;    // P in place of S
         dpacc[r] = ds;                              // dS in place of dP
       }
-      general_dot_cols<NB>(av, Oc + (4 * hh) * poc + m, poc, sacc, nbv);
-      general_dot_cols<NB>(ak, Qc + (4 * hh) * pqc + m, pqc, dpacc, nbk);
+      if constexpr (BP) {
+        general_dot_cols_bf16<NB>(av, Oc + (4 * hh) * poc + m, poc, sacc, nbv);
+        general_dot_cols_bf16<NB>(ak, Qc + (4 * hh) * pqc + m, pqc, dpacc, nbk);
+      } else {
+        general_dot_cols<NB>(av, Oc + (4 * hh) * poc + m, poc, sacc, nbv);
+        general_dot_cols<NB>(ak, Qc + (4 * hh) * pqc + m, pqc, dpacc, nbk);
+      }
     }
   }
   if (kj < krows) {
@@ -4242,7 +4329,18 @@ long long mfma_grid(const Params& p) {
   return 8LL * p.n_qtiles * (((long long)p.B * p.H + 7) / 8);
 }
 
-// The general backward: head dims up to 128 on the fp32 matrix cores, larger ones by the FMA kernels.
+// Whether a bf16 call of the general backward takes its products to the bf16 matrix cores: head dims up to 128
+// in multiples of 16, every row of q, k, v and dout on a 16-byte boundary.
+bool general_bwd_bf16_products(const Params& p) {
+  auto rows16 = [](const void* base, int64_t row, int64_t head, int64_t batch) {
+    return ((uintptr_t)base & 15u) == 0 && ((row | head | batch) & 7) == 0;
+  };
+  return p.d_qk <= 128 && p.d_v <= 128 && (p.d_qk & 15) == 0 && (p.d_v & 15) == 0 && rows16(p.q, p.q_st, p.q_sh, p.q_sb) &&
+         rows16(p.k, p.k_st, p.k_sh, p.k_sb) && rows16(p.v, p.v_st, p.v_sh, p.v_sb) && rows16(p.dout, p.o_st, p.o_sh, p.o_sb);
+}
+
+// The general backward: head dims up to 128 on the matrix cores (fp32 products; bf16 products for bf16 storage
+// where the rows allow), larger ones by the FMA kernels.
 template <typename T>
 int launch_bwd(const Params& p, hipStream_t st) {
   if (p.B > 65535) return fail(HSTU_ERR_SHAPE, "the general backward takes at most 65535 sequences per call, got %d", p.B);
@@ -4250,6 +4348,21 @@ int launch_bwd(const Params& p, hipStream_t st) {
     // (each wave's block of dS goes through LDS for the position table's diagonal sums and for the dense bias's row-wise adds)
     const bool want_pos = (p.dpos != nullptr && p.pos_tab != nullptr) || p.dbias != nullptr;
     const int smem_q = 4 * general_bwd_dq_lds(p.d_qk, p.d_v, want_pos, p.ts_nb), smem_kv = 4 * general_bwd_dkv_lds(p.d_qk, p.d_v);
+    if constexpr (sizeof(T) == 2) {
+      // bf16 storage whose rows can be fetched 16 bytes at a time: the products on the bf16 matrix cores
+      if (general_bwd_bf16_products(p)) {
+        static int granted_qb[64], granted_kvb[64];
+        if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, true>, smem_q, granted_qb)) return rc;
+        if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T, true>, smem_kv, granted_kvb)) return rc;
+        hipLaunchKernelGGL((hstu_bwd_dq_mm<T, true>), dim3(p.H, p.B, (p.L + 127) / 128), dim3(256), smem_q, st, p);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
+        hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true>), dim3(p.H, p.B, (p.Lkv + 127) / 128), dim3(256), smem_kv, st, p);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
+        return HSTU_OK;
+      }
+    }
     static int granted_q[64], granted_kv[64];
     if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T>, smem_q, granted_q)) return rc;
     if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T>, smem_kv, granted_kv)) return rc;
@@ -4535,7 +4648,10 @@ const char* hstu_attn_bwd_variant(const HstuAttnBwdArgs* args) {
   if (!probe.out) probe.out = (void*)args->dout;
   if (validate(&probe) != HSTU_OK || probe.qk_dtype == HSTU_DTYPE_FP8_E4M3FN) return "invalid";
   if (bwd_mfma_eligible(args)) return "hstu_bwd_mfma_bf16";
-  return probe.qk_dtype == HSTU_DTYPE_FP32 ? "hstu_bwd_general<float>" : "hstu_bwd_general<bf16>";
+  if (probe.qk_dtype == HSTU_DTYPE_FP32) return "hstu_bwd_general<float>";
+  Params p = make_params(&probe);
+  p.dout = args->dout;
+  return general_bwd_bf16_products(p) ? "hstu_bwd_general<bf16, bf16 products>" : "hstu_bwd_general<bf16>";
 }
 
 int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream) {

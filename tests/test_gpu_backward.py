@@ -602,3 +602,56 @@ def test_gradients_written_into_given_slices(gpu, dtype):
   with pytest.raises(ValueError, match="grads_out"):
     recml_amd.hstu_attention_bwd(q, k, v, dout, seq_lens=lens, pos_bias=pos,
                                  grads_out=(torch.empty_like(q), grad[:, :, 2], grad[:, :, 3]))
+
+
+@pytest.mark.parametrize("d,dv,view,products,layout", [
+    (16, 16, False, True, "padded"), (48, 80, False, True, "padded"), (48, 80, False, True, "jagged"), (64, 32, False, True, "padded"),
+    (128, 128, False, True, "padded + zero bias"),          # (a dense bias keeps d = 128 off the hand-scheduled pair)
+    (40, 40, False, False, "padded"), (40, 40, False, False, "jagged"), (64, 64, True, False, "padded"), (160, 160, False, False, "padded")])
+def test_general_backward_in_bf16_storage(gpu, d, dv, view, products, layout):
+  """bf16 tensors on the general backward: head dims in multiples of 16 with rows on 16-byte boundaries take the
+  bf16 products, everything else -- other head dims, rows that start off a boundary, head dims beyond 128 -- the
+  fp32 ones; both against the oracle on the same bf16 inputs, table gradients included."""
+  rng = np.random.default_rng(8300 + 3 * d + dv + view)
+  bf = torch.bfloat16
+  B, L, Lk, H = 3, 200, 200, 2
+  lens = np.array([200, 77, 130], dtype=np.int32)
+  mk = lambda dd: O.round_bf16(rng.standard_normal((B, L, H, dd)).astype(np.float32) * 0.4)
+  q, k, v, dout = mk(d), mk(d), mk(dv), mk(dv)
+  pos = (rng.standard_normal((H, 2 * L - 1)) * 0.3).astype(np.float32)
+  tab = (rng.standard_normal((1, 33)) * 0.3).astype(np.float32)
+  t = 1_700_000_000 + np.cumsum(np.ceil(rng.exponential(3000.0, (B, L))), axis=1).astype(np.int64)
+  for b in range(B):
+    t[b, lens[b]:] = t[b, lens[b] - 1]
+  kw = dict(n=float(L), alpha=0.25, causal=True, seq_lens=lens, pos_tab=pos, ts_tab=tab, timestamps=t, sliding_window_size=150)
+  zero_bias = np.zeros((1, L, L), np.float32) if layout.endswith("zero bias") else None
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, bias=zero_bias, **kw)
+
+  def place(x):
+    if layout == "jagged":
+      x = O.padded_to_jagged(x, lens)[0]
+    xd = _dev(x, bf)
+    if not view:
+      return xd
+    buf = torch.zeros(xd.shape[:-1] + (x.shape[-1] + 8,), dtype=bf, device="cuda:0")
+    buf[..., 1:1 + x.shape[-1]] = xd
+    return buf[..., 1:1 + x.shape[-1]]                # rows start two bytes off a 16-byte boundary
+  gk = dict(n=float(L), alpha=0.25, causal=True, pos_bias=_dev(pos), ts_bias=_dev(tab), sliding_window_size=150)
+  if layout == "jagged":
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    gk.update(seq_offsets=_dev(off), max_len=L, timestamps=_dev(O.padded_to_jagged(t[..., None, None], lens)[0].reshape(-1)))
+  else:
+    gk.update(seq_lens=_dev(lens), timestamps=_dev(t))
+  if zero_bias is not None:
+    gk.update(bias=_dev(zero_bias))
+  variant = []
+  got = recml_amd.hstu_attention_bwd(place(q), place(k), place(v), place(dout), _variant_out=variant, **gk)
+  torch.cuda.synchronize()
+  assert variant[-1] == ("hstu_bwd_general<bf16, bf16 products>" if products else "hstu_bwd_general<bf16>"), variant
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    g = g.float().cpu().numpy()
+    if layout == "jagged":
+      g = O.jagged_to_padded(g, off, L)
+    assert np.isfinite(g).all() and _rel(g, w) <= 2e-2, (nm, _rel(g, w))
+  for nm, g, w in (("dpos", got[3], want[3]), ("dts", got[4], want[4])):
+    assert _rel(g.cpu().numpy().reshape(w.shape), w) <= 2e-2, nm

@@ -519,17 +519,20 @@ def bench_dense_backward(args, q, k, v, mask, bias):
   ms, ms_bias = timed(False), timed(True)
   flops = 8.0 * d * H * B * L * (L + 1) / 2
   fp32 = q.dtype == torch.float32
+  bf16_products = "bf16 products" in variant[-1]
+  peak = PEAK_BF16_TFLOPS if bf16_products else PEAK_FP32_TFLOPS
   print(json.dumps({
       "metric": "HSTU attn bwd TFLOP/s (kept pairs), dense mask + bias, L=%d %s" % (L, "fp32" if fp32 else "bf16"),
       "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
       "ms_per_step_with_bias_gradient": ms_bias,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-      "dtype": "f32" if fp32 else "bf16 storage, fp32 arithmetic", "data": "synthetic",
+      "dtype": "f32" if fp32 else ("bf16" if bf16_products else "bf16 storage, fp32 arithmetic"), "data": "synthetic",
       "config": {"workload": f"A1-dense backward: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",
                  "kernel": variant[-1]},
-      "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                   "frac": flops / (ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, "traffic": None,
-                   "note": "general kernels on the fp32 matrix cores; time covers both kernels, the memsets and the host call"},
+      "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
+                   "frac": flops / (ms * 1e-3) / 1e12 / peak, "traffic": None,
+                   "note": "general kernels, products on the %s matrix cores; time covers both kernels, the memsets and the host call"
+                           % ("bf16" if bf16_products else "fp32")},
   }))
 
 
@@ -560,7 +563,7 @@ def bench_backward(args, w, q, k, v, kw, dev):
       "metric": "HSTU attn bwd TFLOP/s (unmasked), L=%d %s" % (w.L, "fp32" if w.dtype == "fp32" else "bf16"), "value": flops / (ms * 1e-3) / 1e12,
       "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-      "dtype": "bf16" if mfma else ("f32" if w.dtype == "fp32" else "bf16 storage, fp32 arithmetic"),
+      "dtype": "bf16" if (mfma or "bf16 products" in variant[-1]) else ("f32" if w.dtype == "fp32" else "bf16 storage, fp32 arithmetic"),
       "data": "synthetic",
       "config": {"workload": w.name + " backward",
                  "kernel": "hstu_bwd_dq_mfma + hstu_bwd_dkv_mfma" if mfma else

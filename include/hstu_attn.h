@@ -233,7 +233,11 @@ int hstu_attn_fwd_noalloc(const HstuAttnFwdArgs* args, void* stream);
  * matrix-core forward (without a dense mask or bias, and with keys and
  * queries of one length), pass 16-byte aligned gradient buffers and bring
  * the workspace run on the matrix cores instead (bf16 products, fp32
- * accumulation, table gradients included); hstu_attn_bwd_variant tells
+ * accumulation, table gradients included); every other bf16 call whose head
+ * dims are multiples of 16 up to 128 and whose q, k, v, dout rows lie on
+ * 16-byte boundaries keeps the general kernels but forms its products on the
+ * bf16 matrix cores too (P and dS rounded to bf16 for the last products, as the
+ * forward rounds P); hstu_attn_bwd_variant tells
  * which.  Math of recml/core/ops/hstu_ops.py:417-548 (dq, dk, dv), which
  * the reference reaches through jax.custom_vjp (hstu_ops.py:551-826), extended
  * by the table gradients that jax derives for recml/layers/keras/hstu.py:91-113,
@@ -259,7 +263,8 @@ typedef struct HstuAttnBwdArgs {
 int hstu_attn_bwd(const HstuAttnBwdArgs* args, void* stream);
 
 /* Name of the kernel pair hstu_attn_bwd would launch for `args` (diagnostics;
- * static storage): "hstu_bwd_mfma_bf16", "hstu_bwd_general<...>" or "invalid". */
+ * static storage): "hstu_bwd_mfma_bf16", "hstu_bwd_general<float>", "hstu_bwd_general<bf16>",
+ * "hstu_bwd_general<bf16, bf16 products>" or "invalid". */
 const char* hstu_attn_bwd_variant(const HstuAttnBwdArgs* args);
 
 /* Message for the last non-zero status on this thread ("" if none). */

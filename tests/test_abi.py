@@ -82,21 +82,24 @@ def test_backward_variant_query():
   f.alpha, f.inv_n, f.causal = 1.0, 1.0 / 256, 1
   f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_BF16
   b.dout = b.dq = b.dk = b.dv = 0x20000
-  # bf16 at a matrix-core head dim, but no workspace: the general pair
+  # bf16 at a matrix-core head dim, but no workspace: the general pair (bf16 products: rows on 16-byte boundaries)
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16, bf16 products>"
+  f.q = 0x10002                                                       # rows off a boundary: fp32 products
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  f.q = 0x10000
   f.out = 0x30000                                                     # the size query validates a forward call
   f.workspace, f.workspace_bytes = 0x40000, lib.hstu_attn_fwd_workspace_bytes(C.byref(f))
   f.out = None                                                        # the backward does not need it
   assert f.workspace_bytes > 0
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
   b.dq = 0x20004                                                      # gradient buffers must be 16-byte aligned for it
-  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16, bf16 products>"
   b.dq = 0x20000
   f.window = 8                                                        # a sliding window stays on the matrix cores
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
   f.window = -1
   f.mask = 0x50000                                                    # an explicit mask does not (the forward would)
-  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16>"
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16, bf16 products>"
   f.mask = None
   f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_FP32
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<float>"

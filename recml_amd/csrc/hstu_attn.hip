@@ -1070,6 +1070,33 @@ struct GeneralTile {
       }
     }
   }
+  // bf16 storage, kept as bf16 in LDS (the instances with bf16 products; `fast` loads only): rows at `by_row`
+  // (pitch in bytes, a multiple of 16) and / or transposed at `by_chan`: [channel][row of the tile], pitch in bytes
+  __device__ __forceinline__ void stage_bf16(int row0, int nrows, int d, int tid, unsigned char* by_row, int pitch_row,
+                                             unsigned char* by_chan, int pitch_chan) const {
+    static_assert(sizeof(T) == 2 || sizeof(T) == 4, "");
+    if constexpr (sizeof(T) == 2) {
+      const int lr = tid >> 3, lc = (tid & 7) * 4;
+      const int ng = (d + 31) >> 5;
+      const bool row_ok = row0 + lr < nrows;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const int c = lc + 32 * g;
+        if (g < ng && c < d) {
+          const uint2 v = row_ok ? raw[g] : uint2{0u, 0u};
+          if (by_row) *(uint2*)(by_row + lr * pitch_row + 2 * c) = v;
+          if (by_chan) {
+            unsigned short* col = (unsigned short*)(by_chan + c * pitch_chan) + lr;
+            const int ps = pitch_chan >> 1;
+            col[0] = (unsigned short)(v.x & 0xffffu);
+            col[ps] = (unsigned short)(v.x >> 16);
+            col[2 * ps] = (unsigned short)(v.y & 0xffffu);
+            col[3 * ps] = (unsigned short)(v.y >> 16);
+          }
+        }
+      }
+    }
+  }
 };
 
 // The lane's share of row `row` as the B operand of a product over the channels: channels 4u + 2hh and
@@ -1106,8 +1133,9 @@ __device__ __forceinline__ void general_dot_cols(floatx16 (&out)[NB], const floa
 // Every operand of the first two products is then a bf16 value, so v_mfma_f32_32x32x16_bf16 forms the same
 // products and fp32 sums in one instruction per 16 channels instead of eight per 16; P and dS are rounded to
 // bf16 for the last products, as the forward rounds P.  The instruction leaves its result in the same lanes and
-// registers as the fp32 one, so everything between the products is shared.  Tiles stay in LDS as they are
-// (fp32, both layouts) and are packed on the way into the instruction.
+// registers as the fp32 one, so everything between the products is shared.  The tiles are kept in LDS as bf16:
+// by rows for the products over the channels (16-byte reads), transposed for the products over the tile's rows
+// (a lane's eight rows of a product are two 8-byte reads).
 __device__ __forceinline__ uint32_t general_pack_bf16(float lo, float hi) {
   floatx2 f = {lo, hi};
   typedef bf16_t bf16x2_t __attribute__((ext_vector_type(2)));
@@ -1123,23 +1151,21 @@ __device__ __forceinline__ void general_row_frag_bf16(bf16x8 (&f)[8], const bf16
     f[ks] = __builtin_bit_cast(bf16x8, v);
   }
 }
-// acc += A B^T over the channels: `arow` = the lane's row of the fp32 tile + 8 hh (8-byte reads)
-__device__ __forceinline__ void general_dot_rows_bf16(floatx16& acc, const float* arow, const bf16x8 (&bf)[8], int d) {
+// acc += A B^T over the channels: `arow` = the lane's row of the bf16 tile + 16 hh bytes (16-byte reads)
+__device__ __forceinline__ void general_dot_rows_bf16(floatx16& acc, const unsigned char* arow, const bf16x8 (&bf)[8], int d) {
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) {
     if (16 * ks < d) {
-      const float2 a0 = *(const float2*)(arow + 16 * ks), a1 = *(const float2*)(arow + 16 * ks + 2);
-      const float2 a2 = *(const float2*)(arow + 16 * ks + 4), a3 = *(const float2*)(arow + 16 * ks + 6);
-      const uint4 pa = {general_pack_bf16(a0.x, a0.y), general_pack_bf16(a1.x, a1.y), general_pack_bf16(a2.x, a2.y),
-                        general_pack_bf16(a3.x, a3.y)};
+      const uint4 pa = *(const uint4*)(arow + 32 * ks);
       acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pa), bf[ks], acc, 0, 0, 0);
     }
   }
 }
 // out[x]^T += A^T B over the tile's 32 rows, 16 at a time: B = the accumulator's values 8 cc .. 8 cc + 7 (rows
-// 16 cc + 4 hh + tt and 16 cc + 8 + 4 hh + tt), A = channel 32 x + m of the same rows (`acol` = tile + 4 hh rows + m)
+// 16 cc + 4 hh + tt and 16 cc + 8 + 4 hh + tt), A = channel 32 x + m of the same rows: two 8-byte reads of the
+// transposed tile (`acol` = its channel m + 8 hh bytes, `pitch` bytes per channel)
 template <int NB>
-__device__ __forceinline__ void general_dot_cols_bf16(floatx16 (&out)[NB], const float* acol, int pitch, const floatx16& bv, int nblk) {
+__device__ __forceinline__ void general_dot_cols_bf16(floatx16 (&out)[NB], const unsigned char* acol, int pitch, const floatx16& bv, int nblk) {
 #pragma unroll
   for (int cc = 0; cc < 2; ++cc) {
     const uint4 pb = {general_pack_bf16(bv[8 * cc + 0], bv[8 * cc + 1]), general_pack_bf16(bv[8 * cc + 2], bv[8 * cc + 3]),
@@ -1147,18 +1173,24 @@ __device__ __forceinline__ void general_dot_cols_bf16(floatx16 (&out)[NB], const
 #pragma unroll
     for (int x = 0; x < NB; ++x) {
       if (x < nblk) {
-        float a[8];
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          a[tt] = acol[(16 * cc + tt) * pitch + 32 * x];
-          a[4 + tt] = acol[(16 * cc + 8 + tt) * pitch + 32 * x];
-        }
-        const uint4 pa = {general_pack_bf16(a[0], a[1]), general_pack_bf16(a[2], a[3]), general_pack_bf16(a[4], a[5]),
-                          general_pack_bf16(a[6], a[7])};
+        const unsigned char* ap = acol + 32 * x * pitch + 32 * cc;
+        const uint2 lo = *(const uint2*)ap, hi = *(const uint2*)(ap + 16);
+        const uint4 pa = {lo.x, lo.y, hi.x, hi.y};
         out[x] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, pa), __builtin_bit_cast(bf16x8, pb), out[x], 0, 0, 0);
       }
     }
   }
+}
+// Pitches of the bf16 tiles in bytes: rows of d channels + 16 bytes (16 consecutive rows then sweep the banks once
+// under 16-byte reads); a channel's 32 keys + 8 bytes (72: consecutive channels 18 banks apart, 8-byte reads).
+__host__ __device__ inline int general_bf16_row_pitch(int d) { return 2 * d + 16; }
+constexpr int GENERAL_BF16_CHAN_PITCH = 72;
+__host__ __device__ inline int general_bwd_dq_lds_bf16(int dq, int dv, bool want_ds, int ts_nb) {   // bytes
+  return GT * general_bf16_row_pitch(dq) + dq * GENERAL_BF16_CHAN_PITCH + GT * general_bf16_row_pitch(dv) +
+         4 * ((want_ds ? 4 * GT * (GT + 1) : 0) + general_hist_len(ts_nb));
+}
+__host__ __device__ inline int general_bwd_dkv_lds_bf16(int dq, int dv) {                            // bytes
+  return GT * general_bf16_row_pitch(dq) + dq * GENERAL_BF16_CHAN_PITCH + GT * general_bf16_row_pitch(dv) + dv * GENERAL_BF16_CHAN_PITCH;
 }
 
 // LDS floats of the two kernels (host and device agree through these)
@@ -1183,7 +1215,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
   float* Kr = gsm;                         // [32][pk]  K rows for S^T
   float* Kc = Kr + GT * pk;                // [32][pc]  K read across the channels for dQ^T
   float* Vr = Kc + GT * pc;                // [32][pv]  V rows for dP^T
-  float* Hist = Vr + GT * pv;              // [buckets] timestamp-bucket sums of this workgroup
+  // (bf16 products: [32][prk bytes] K rows | [dq][72 bytes] K transposed | [32][prv bytes] V rows)
+  unsigned char* const smb = (unsigned char*)gsm;
+  const int prk = general_bf16_row_pitch(dq), prv = general_bf16_row_pitch(dv);
+  unsigned char* const Krb = smb;
+  unsigned char* const Ktb = Krb + GT * prk;
+  unsigned char* const Vrb = Ktb + dq * GENERAL_BF16_CHAN_PITCH;
+  float* Hist = BP ? (float*)(Vrb + GT * prv) : Vr + GT * pv;   // [buckets] timestamp-bucket sums of this workgroup
   float* Ds = Hist + general_hist_len(p.ts_nb);   // [4][32][33] dS of each wave's block, [query][key] (position and dense-bias gradients only)
 
   const int h = blockIdx.x, b = blockIdx.y, qt = gridDim.z - 1 - blockIdx.z;
@@ -1259,8 +1297,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
       float db[16];
       if (live && p.dense_bias) general_dense_row(p, b, qi, kv0, hh, db);
       __syncthreads();
-      kt_.stage(kv0, s.n_kv, dq, kfast, tid, Kr, pk, Kc, pc);
-      vt_.stage(kv0, s.n_kv, dv, vfast, tid, Vr, pv, nullptr, 0);
+      if constexpr (BP) {
+        kt_.stage_bf16(kv0, s.n_kv, dq, tid, Krb, prk, Ktb, GENERAL_BF16_CHAN_PITCH);
+        vt_.stage_bf16(kv0, s.n_kv, dv, tid, Vrb, prv, nullptr, 0);
+      } else {
+        kt_.stage(kv0, s.n_kv, dq, kfast, tid, Kr, pk, Kc, pc);
+        vt_.stage(kv0, s.n_kv, dv, vfast, tid, Vr, pv, nullptr, 0);
+      }
       __syncthreads();
       if (kv0 + GT < kv_end) {
         kt_.fetch(kp_, p.k_st, kv0 + GT, s.n_kv, dq, kfast, tid);
@@ -1272,8 +1315,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
       if constexpr (BP) {
-        general_dot_rows_bf16(sacc, Kr + m * pk + 8 * hh, qb, dq);
-        general_dot_rows_bf16(dpacc, Vr + m * pv + 8 * hh, dob, dv);
+        general_dot_rows_bf16(sacc, Krb + m * prk + 16 * hh, qb, dq);
+        general_dot_rows_bf16(dpacc, Vrb + m * prv + 16 * hh, dob, dv);
       } else {
         general_dot_rows(sacc, Kr + m * pk + 2 * hh, qf, dq4);
         general_dot_rows(dpacc, Vr + m * pv + 2 * hh, dof, dv4);
@@ -1321,7 +1364,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
             atomicAdd(p.dpos + (int64_t)(p.pos_heads > 1 ? h : 0) * (2 * p.L - 1) + idx, sum);
         }
       }
-      if constexpr (BP) general_dot_cols_bf16<NB>(o, Kc + (4 * hh) * pc + m, pc, sacc, nblk);
+      if constexpr (BP) general_dot_cols_bf16<NB>(o, Ktb + m * GENERAL_BF16_CHAN_PITCH + 8 * hh, GENERAL_BF16_CHAN_PITCH, sacc, nblk);
       else general_dot_cols<NB>(o, Kc + (4 * hh) * pc + m, pc, sacc, nblk);
     }
     if (want_ts) {
@@ -1359,6 +1402,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
   float* Qc = Qr + GT * pqr;               // [32][pqc] Q read across the channels for dK^T
   float* Or = Qc + GT * pqc;               // [32][por] dO rows for dP
   float* Oc = Or + GT * por;               // [32][poc] dO read across the channels for dV^T
+  // (bf16 products: Q rows | Q transposed | dO rows | dO transposed, pitches in bytes)
+  unsigned char* const smb = (unsigned char*)gsm;
+  const int prq = general_bf16_row_pitch(dq), pro = general_bf16_row_pitch(dv);
+  unsigned char* const Qrb = smb;
+  unsigned char* const Qtb = Qrb + GT * prq;
+  unsigned char* const Orb = Qtb + dq * GENERAL_BF16_CHAN_PITCH;
+  unsigned char* const Otb = Orb + GT * pro;
 
   const int h = blockIdx.x, b = blockIdx.y, kt = blockIdx.z;
   const Seq s = seq_info(p, b, h);
@@ -1434,8 +1484,13 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
       float db[16];
       if (live && p.dense_bias) general_dense_col(p, b, i0, kj, hh, db);
       __syncthreads();
-      qt_.stage(i0, s.n_q, dq, qfast, tid, Qr, pqr, Qc, pqc);
-      ot_.stage(i0, s.n_q, dv, ofast, tid, Or, por, Oc, poc);
+      if constexpr (BP) {
+        qt_.stage_bf16(i0, s.n_q, dq, tid, Qrb, prq, Qtb, GENERAL_BF16_CHAN_PITCH);
+        ot_.stage_bf16(i0, s.n_q, dv, tid, Orb, pro, Otb, GENERAL_BF16_CHAN_PITCH);
+      } else {
+        qt_.stage(i0, s.n_q, dq, qfast, tid, Qr, pqr, Qc, pqc);
+        ot_.stage(i0, s.n_q, dv, ofast, tid, Or, por, Oc, poc);
+      }
       __syncthreads();
       if (i0 + GT < q_end) {
         qt_.fetch(qp, p.q_st, i0 + GT, s.n_q, dq, qfast, tid);
@@ -1447,8 +1502,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) { sacc[r] = 0.f; dpacc[r] = 0.f; }
       if constexpr (BP) {
-        general_dot_rows_bf16(sacc, Qr + m * pqr + 8 * hh, kb, dq);
-        general_dot_rows_bf16(dpacc, Or + m * por + 8 * hh, vb, dv);
+        general_dot_rows_bf16(sacc, Qrb + m * prq + 16 * hh, kb, dq);
+        general_dot_rows_bf16(dpacc, Orb + m * pro + 16 * hh, vb, dv);
       } else {
         general_dot_rows(sacc, Qr + m * pqr + 2 * hh, kf, dq4);
         general_dot_rows(dpacc, Or + m * por + 2 * hh, vf, dv4);
@@ -1468,8 +1523,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
         dpacc[r] = ds;                              // dS in place of dP
       }
       if constexpr (BP) {
-        general_dot_cols_bf16<NB>(av, Oc + (4 * hh) * poc + m, poc, sacc, nbv);
-        general_dot_cols_bf16<NB>(ak, Qc + (4 * hh) * pqc + m, pqc, dpacc, nbk);
+        general_dot_cols_bf16<NB>(av, Otb + m * GENERAL_BF16_CHAN_PITCH + 8 * hh, GENERAL_BF16_CHAN_PITCH, sacc, nbv);
+        general_dot_cols_bf16<NB>(ak, Qtb + m * GENERAL_BF16_CHAN_PITCH + 8 * hh, GENERAL_BF16_CHAN_PITCH, dpacc, nbk);
       } else {
         general_dot_cols<NB>(av, Oc + (4 * hh) * poc + m, poc, sacc, nbv);
         general_dot_cols<NB>(ak, Qc + (4 * hh) * pqc + m, pqc, dpacc, nbk);
@@ -4351,13 +4406,14 @@ int launch_bwd(const Params& p, hipStream_t st) {
     if constexpr (sizeof(T) == 2) {
       // bf16 storage whose rows can be fetched 16 bytes at a time: the products on the bf16 matrix cores
       if (general_bwd_bf16_products(p)) {
+        const int smem_qb = general_bwd_dq_lds_bf16(p.d_qk, p.d_v, want_pos, p.ts_nb), smem_kvb = general_bwd_dkv_lds_bf16(p.d_qk, p.d_v);
         static int granted_qb[64], granted_kvb[64];
-        if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, true>, smem_q, granted_qb)) return rc;
-        if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T, true>, smem_kv, granted_kvb)) return rc;
-        hipLaunchKernelGGL((hstu_bwd_dq_mm<T, true>), dim3(p.H, p.B, (p.L + 127) / 128), dim3(256), smem_q, st, p);
+        if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, true>, smem_qb, granted_qb)) return rc;
+        if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T, true>, smem_kvb, granted_kvb)) return rc;
+        hipLaunchKernelGGL((hstu_bwd_dq_mm<T, true>), dim3(p.H, p.B, (p.L + 127) / 128), dim3(256), smem_qb, st, p);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-        hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true>), dim3(p.H, p.B, (p.Lkv + 127) / 128), dim3(256), smem_kv, st, p);
+        hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true>), dim3(p.H, p.B, (p.Lkv + 127) / 128), dim3(256), smem_kvb, st, p);
         e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
         return HSTU_OK;

@@ -1204,14 +1204,15 @@ __host__ __device__ inline int general_bwd_dkv_lds(int dq, int dv) {
 // dQ and the table gradients: one workgroup per 128 query rows of one (sequence, head), 32 per wave, keys streamed.
 //   S^T = K Q^T, dP^T = V dO^T (A = K / V rows, B = the wave's Q / dO rows in registers), dS^T pointwise,
 //   dQ^T += K^T dS^T (A = K read across the channels, B = dS^T as it leaves the pointwise part).
-template <typename T, bool BP = false>
-__global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
+template <typename T, bool BP = false, bool TAB = true>
+__global__ __launch_bounds__(256, (BP && !TAB) ? 2 : 1) void hstu_bwd_dq_mm(const Params p) {
   extern __shared__ __attribute__((aligned(16))) float gsm[];
   const int dq = p.d_qk, dv = p.d_v;
   const int dq4 = (dq + 3) & ~3, dv4 = (dv + 3) & ~3;
   const int pk = general_pitch_qk(dq), pc = general_pitch_v(dq), pv = general_pitch_qk(dv);
-  const bool want_ts = p.dts != nullptr && p.ts_tab != nullptr;
-  const bool want_pos = p.dpos != nullptr && p.pos_tab != nullptr;
+  // (TAB = false: an instance for calls without bias tables, which then carries none of their code)
+  const bool want_ts = TAB && p.dts != nullptr && p.ts_tab != nullptr;
+  const bool want_pos = TAB && p.dpos != nullptr && p.pos_tab != nullptr;
   float* Kr = gsm;                         // [32][pk]  K rows for S^T
   float* Kc = Kr + GT * pk;                // [32][pc]  K read across the channels for dQ^T
   float* Vr = Kc + GT * pc;                // [32][pv]  V rows for dP^T
@@ -1283,7 +1284,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
     }
     if (qi >= s.n_q) hi = -1;
     const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
-    const bool tabled = p.pos_tab != nullptr || p.ts_tab != nullptr;
+    const bool tabled = TAB && (p.pos_tab != nullptr || p.ts_tab != nullptr);
     float* dsw = Ds + w * (GT * (GT + 1));
 
     for (int kv0 = kv_begin; kv0 < kv_end; kv0 += GT) {
@@ -1392,7 +1393,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dq_mm(const Params p) {
 // dK and dV: one workgroup per 128 keys of one (sequence, head), 32 per wave, query rows streamed 32 at a time.
 //   S = Q K^T, dP = dO V^T (A = Q / dO rows, B = the wave's K / V rows in registers), P and dS pointwise,
 //   dV^T += dO^T P, dK^T += Q^T dS (A = dO / Q read across the channels, B = P / dS as they leave the pointwise part).
-template <typename T, bool BP = false>
+template <typename T, bool BP = false, bool TAB = true>
 __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
   extern __shared__ __attribute__((aligned(16))) float gsm[];
   const int dq = p.d_qk, dv = p.d_v;
@@ -1471,7 +1472,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
     }
     if (kj >= s.n_kv) hi = -1;
     const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
-    const bool tabled = p.pos_tab != nullptr || p.ts_tab != nullptr;
+    const bool tabled = TAB && (p.pos_tab != nullptr || p.ts_tab != nullptr);
 
     for (int i0 = q_begin; i0 < q_end; i0 += GT) {
       // nothing for a wave whose keys all lie behind these rows (causal) or outside the window
@@ -4407,13 +4408,28 @@ int launch_bwd(const Params& p, hipStream_t st) {
       // bf16 storage whose rows can be fetched 16 bytes at a time: the products on the bf16 matrix cores
       if (general_bwd_bf16_products(p)) {
         const int smem_qb = general_bwd_dq_lds_bf16(p.d_qk, p.d_v, want_pos, p.ts_nb), smem_kvb = general_bwd_dkv_lds_bf16(p.d_qk, p.d_v);
-        static int granted_qb[64], granted_kvb[64];
+        static int granted_qb[64], granted_kvb[64], granted_qn[64], granted_kvn[64];
+        const bool tables = p.pos_tab != nullptr || p.ts_tab != nullptr;
+        const dim3 grid_q(p.H, p.B, (p.L + 127) / 128), grid_kv(p.H, p.B, (p.Lkv + 127) / 128);
+        if (!tables) {
+          // no bias tables (the layer's dense operands, or no bias at all): instances without the tables' code,
+          // which fit two workgroups per CU
+          if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, true, false>, smem_qb, granted_qn)) return rc;
+          if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T, true, false>, smem_kvb, granted_kvn)) return rc;
+          hipLaunchKernelGGL((hstu_bwd_dq_mm<T, true, false>), grid_q, dim3(256), smem_qb, st, p);
+          hipError_t e = hipGetLastError();
+          if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
+          hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true, false>), grid_kv, dim3(256), smem_kvb, st, p);
+          e = hipGetLastError();
+          if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
+          return HSTU_OK;
+        }
         if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, true>, smem_qb, granted_qb)) return rc;
         if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T, true>, smem_kvb, granted_kvb)) return rc;
-        hipLaunchKernelGGL((hstu_bwd_dq_mm<T, true>), dim3(p.H, p.B, (p.L + 127) / 128), dim3(256), smem_qb, st, p);
+        hipLaunchKernelGGL((hstu_bwd_dq_mm<T, true>), grid_q, dim3(256), smem_qb, st, p);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-        hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true>), dim3(p.H, p.B, (p.Lkv + 127) / 128), dim3(256), smem_kvb, st, p);
+        hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true>), grid_kv, dim3(256), smem_kvb, st, p);
         e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
         return HSTU_OK;

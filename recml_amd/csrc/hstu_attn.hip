@@ -247,9 +247,11 @@ __device__ __forceinline__ float general_bias(const Params& p, const Seq& s,
 // The explicit mask's bytes for the 16 pairs (row i, keys j0 + 8g + 4hh .. +3, g < 4) a lane holds after a
 // product with the query row fixed: one 32-bit word per g (byte tt = key j0 + 8g + 4hh + tt).  Row and keys are
 // clamped into the matrix: bytes of pairs outside it are never looked at (their indices drop them).
+// (WORDS_ONLY: the caller has checked that whole words can be fetched; the byte-wise form is then left out)
+template <bool WORDS_ONLY = false>
 __device__ __forceinline__ void general_mask_words(const Params& p, int b, int i, int j0, int hh, uint32_t (&w)[4]) {
   const uint8_t* mrow = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)(i < p.L - 1 ? i : p.L - 1) * p.Lkv;
-  if ((p.Lkv & 3) == 0 && ((uintptr_t)p.mask & 3) == 0) {
+  if (WORDS_ONLY || ((p.Lkv & 3) == 0 && ((uintptr_t)p.mask & 3) == 0)) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       int j = j0 + 8 * g + 4 * hh;
@@ -356,9 +358,10 @@ __device__ __forceinline__ void general_mask_live_steps(const Params& p, int b, 
 
 // The dense bias of the same 16 pairs (query row fixed / key fixed), fetched together ahead of their use: four
 // 16-byte loads where the rows allow, else one load per pair; indices clamped into the matrix like the mask's.
+template <bool WORDS_ONLY = false>
 __device__ __forceinline__ void general_dense_row(const Params& p, int b, int i, int j0, int hh, float (&v)[16]) {
   const float* row = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)(i < p.L - 1 ? i : p.L - 1) * p.Lkv;
-  if ((p.Lkv & 3) == 0 && ((uintptr_t)p.dense_bias & 15) == 0) {
+  if (WORDS_ONLY || ((p.Lkv & 3) == 0 && ((uintptr_t)p.dense_bias & 15) == 0)) {
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       int j = j0 + 8 * g + 4 * hh;
@@ -1237,8 +1240,10 @@ __global__ __launch_bounds__(256, (BP && !TAB) ? 2 : 1) void hstu_bwd_dq_mm(cons
   T* __restrict__ dqp = (T*)p.dq + s.bq;
   const int r0 = q0 + 32 * w, qi = r0 + m;
   constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
-  const bool kfast = (((uintptr_t)kp_ & VMASK) == 0) && (p.k_st & 3) == 0 && (dq & 3) == 0;
-  const bool vfast = (((uintptr_t)vp & VMASK) == 0) && (p.v_st & 3) == 0 && (dv & 3) == 0;
+  // (bf16 products are only taken with rows on 16-byte boundaries and head dims in multiples of 16)
+  const bool kfast = BP || ((((uintptr_t)kp_ & VMASK) == 0) && (p.k_st & 3) == 0 && (dq & 3) == 0);
+  const bool vfast = BP || ((((uintptr_t)vp & VMASK) == 0) && (p.v_st & 3) == 0 && (dv & 3) == 0);
+  constexpr bool LEAN = BP && !TAB;      // also: mask and dense bias fetched by whole words (checked at the launch)
 
   constexpr int NB = 4;
   const int nblk = (dq + 31) >> 5;
@@ -1294,9 +1299,9 @@ __global__ __launch_bounds__(256, (BP && !TAB) ? 2 : 1) void hstu_bwd_dq_mm(cons
       // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers; a block they all
       // drop is left out
       uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
-      if (live && p.mask) general_mask_words(p, b, qi, kv0, hh, mw);
+      if (live && p.mask) general_mask_words<LEAN>(p, b, qi, kv0, hh, mw);
       float db[16];
-      if (live && p.dense_bias) general_dense_row(p, b, qi, kv0, hh, db);
+      if (live && p.dense_bias) general_dense_row<LEAN>(p, b, qi, kv0, hh, db);
       __syncthreads();
       if constexpr (BP) {
         kt_.stage_bf16(kv0, s.n_kv, dq, tid, Krb, prk, Ktb, GENERAL_BF16_CHAN_PITCH);
@@ -1425,8 +1430,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
   T* __restrict__ dvp = (T*)p.dv + s.bv;
   const int c0 = k0 + 32 * w, kj = c0 + m;          // the wave's first key, this lane's key
   constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
-  const bool qfast = (((uintptr_t)qp & VMASK) == 0) && (p.q_st & 3) == 0 && (dq & 3) == 0;
-  const bool ofast = (((uintptr_t)dop & VMASK) == 0) && (p.o_st & 3) == 0 && (dv & 3) == 0;
+  const bool qfast = BP || ((((uintptr_t)qp & VMASK) == 0) && (p.q_st & 3) == 0 && (dq & 3) == 0);
+  const bool ofast = BP || ((((uintptr_t)dop & VMASK) == 0) && (p.o_st & 3) == 0 && (dv & 3) == 0);
 
   constexpr int NB = 4;
   const int nbk = (dq + 31) >> 5, nbv = (dv + 31) >> 5;
@@ -4411,7 +4416,9 @@ int launch_bwd(const Params& p, hipStream_t st) {
         static int granted_qb[64], granted_kvb[64], granted_qn[64], granted_kvn[64];
         const bool tables = p.pos_tab != nullptr || p.ts_tab != nullptr;
         const dim3 grid_q(p.H, p.B, (p.L + 127) / 128), grid_kv(p.H, p.B, (p.Lkv + 127) / 128);
-        if (!tables) {
+        const bool words = (!p.mask || ((p.Lkv & 3) == 0 && ((uintptr_t)p.mask & 3) == 0)) &&
+                           (!p.dense_bias || ((p.Lkv & 3) == 0 && ((uintptr_t)p.dense_bias & 15) == 0));
+        if (!tables && words) {
           // no bias tables (the layer's dense operands, or no bias at all): instances without the tables' code,
           // which fit two workgroups per CU
           if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, true, false>, smem_qb, granted_qn)) return rc;

@@ -62,6 +62,7 @@ class _AttentionGateFn(torch.autograd.Function):
 
   @staticmethod
   def forward(ctx, uqkv, gamma, beta, pos_bias, ts_bias, eps, batch, kwargs):
+    uqkv = uqkv.contiguous()            # (the backward mirrors this layout for the gradient)
     u, q, k, v = uqkv.unbind(dim=-3)
     attn = hstu_ops.hstu_attention(q, k, v, pos_bias=pos_bias, ts_bias=ts_bias, batch=batch, **kwargs)
     W = q.shape[-2] * q.shape[-1]

@@ -1241,9 +1241,10 @@ __global__ __launch_bounds__(256, (BP && !TAB) ? 2 : 1) void hstu_bwd_dq_mm(cons
   const int r0 = q0 + 32 * w, qi = r0 + m;
   constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
   // (bf16 products are only taken with rows on 16-byte boundaries and head dims in multiples of 16)
-  const bool kfast = BP || ((((uintptr_t)kp_ & VMASK) == 0) && (p.k_st & 3) == 0 && (dq & 3) == 0);
-  const bool vfast = BP || ((((uintptr_t)vp & VMASK) == 0) && (p.v_st & 3) == 0 && (dv & 3) == 0);
-  constexpr bool LEAN = BP && !TAB;      // also: mask and dense bias fetched by whole words (checked at the launch)
+  // (and the instances without tables, fp32 ones included, are only launched where whole groups of four can be fetched)
+  const bool kfast = BP || !TAB || ((((uintptr_t)kp_ & VMASK) == 0) && (p.k_st & 3) == 0 && (dq & 3) == 0);
+  const bool vfast = BP || !TAB || ((((uintptr_t)vp & VMASK) == 0) && (p.v_st & 3) == 0 && (dv & 3) == 0);
+  constexpr bool LEAN = !TAB;            // also: mask and dense bias fetched by whole words (checked at the launch)
 
   constexpr int NB = 4;
   const int nblk = (dq + 31) >> 5;
@@ -1430,8 +1431,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
   T* __restrict__ dvp = (T*)p.dv + s.bv;
   const int c0 = k0 + 32 * w, kj = c0 + m;          // the wave's first key, this lane's key
   constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
-  const bool qfast = BP || ((((uintptr_t)qp & VMASK) == 0) && (p.q_st & 3) == 0 && (dq & 3) == 0);
-  const bool ofast = BP || ((((uintptr_t)dop & VMASK) == 0) && (p.o_st & 3) == 0 && (dv & 3) == 0);
+  const bool qfast = BP || !TAB || ((((uintptr_t)qp & VMASK) == 0) && (p.q_st & 3) == 0 && (dq & 3) == 0);
+  const bool ofast = BP || !TAB || ((((uintptr_t)dop & VMASK) == 0) && (p.o_st & 3) == 0 && (dv & 3) == 0);
 
   constexpr int NB = 4;
   const int nbk = (dq + 31) >> 5, nbv = (dv + 31) >> 5;
@@ -4437,6 +4438,29 @@ int launch_bwd(const Params& p, hipStream_t st) {
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
         hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, true>), grid_kv, dim3(256), smem_kvb, st, p);
+        e = hipGetLastError();
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
+        return HSTU_OK;
+      }
+    }
+    if constexpr (sizeof(T) == 4) {
+      // fp32 calls without bias tables whose rows, mask and dense bias can be fetched whole: instances with those
+      // fetches fixed at compile time (none of the tables' code, none of the element-wise fallbacks)
+      auto whole = [&](const void* base, int64_t row, int64_t head, int64_t batch) {
+        return ((uintptr_t)base & 15u) == 0 && ((row | head | batch) & 3) == 0;
+      };
+      const bool words = (!p.mask || ((p.Lkv & 3) == 0 && ((uintptr_t)p.mask & 3) == 0)) &&
+                         (!p.dense_bias || ((p.Lkv & 3) == 0 && ((uintptr_t)p.dense_bias & 15) == 0));
+      if (p.pos_tab == nullptr && p.ts_tab == nullptr && words && (p.d_qk & 3) == 0 && (p.d_v & 3) == 0 &&
+          whole(p.q, p.q_st, p.q_sh, p.q_sb) && whole(p.k, p.k_st, p.k_sh, p.k_sb) && whole(p.v, p.v_st, p.v_sh, p.v_sb) &&
+          whole(p.dout, p.o_st, p.o_sh, p.o_sb)) {
+        static int granted_ql[64], granted_kvl[64];
+        if (int rc = allow_lds((const void*)hstu_bwd_dq_mm<T, false, false>, smem_q, granted_ql)) return rc;
+        if (int rc = allow_lds((const void*)hstu_bwd_dkv_mm<T, false, false>, smem_kv, granted_kvl)) return rc;
+        hipLaunchKernelGGL((hstu_bwd_dq_mm<T, false, false>), dim3(p.H, p.B, (p.L + 127) / 128), dim3(256), smem_q, st, p);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
+        hipLaunchKernelGGL((hstu_bwd_dkv_mm<T, false, false>), dim3(p.H, p.B, (p.Lkv + 127) / 128), dim3(256), smem_kv, st, p);
         e = hipGetLastError();
         if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
         return HSTU_OK;

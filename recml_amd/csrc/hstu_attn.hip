@@ -483,7 +483,9 @@ __device__ __forceinline__ void general_dot_rows(floatx16& acc, const float* aro
 // DMAX (128 or 256): the head dims the instance holds.  The wave's Q row shares live in DMAX / 2 registers and
 // its output in DMAX / 2 accumulators: up to 128, 255 registers in all and two waves per SIMD, so that one
 // workgroup's loads, barriers and pointwise work run under another's products; up to 256, one wave per SIMD.
-template <typename T, int DMAX>
+// TAB = false: an instance for calls without bias tables whose rows, mask and dense bias can be fetched whole (the
+// launch checks): none of the tables' code and none of the element-wise fetches in it.
+template <typename T, int DMAX, bool TAB = true>
 __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(const Params p) {
   extern __shared__ __attribute__((aligned(16))) float gsm[];
   constexpr int NB = DMAX / 32;            // 32-channel blocks of the output
@@ -513,8 +515,8 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
   const int qi = r0 + m;                   // this lane's query row
   // whole groups of four elements can be fetched by one load when bases and row strides allow
   constexpr uintptr_t VMASK = sizeof(T) * 4 - 1;
-  const bool kvec = (((uintptr_t)(kp_ + s.bk) & VMASK) == 0) && (p.k_st & 3) == 0;
-  const bool vvec = (((uintptr_t)(vp + s.bv) & VMASK) == 0) && (p.v_st & 3) == 0;
+  const bool kvec = !TAB || ((((uintptr_t)(kp_ + s.bk) & VMASK) == 0) && (p.k_st & 3) == 0);
+  const bool vvec = !TAB || ((((uintptr_t)(vp + s.bv) & VMASK) == 0) && (p.v_st & 3) == 0);
 
   // the key steps of this tile (found first, while nothing else is held in registers)
   int kv_end = s.n_kv;
@@ -561,7 +563,7 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
     // the products.  Otherwise element by element (bf16 elements packed again: nothing is lost).
     constexpr int NG = DMAX / 32;
     typedef typename std::conditional<sizeof(T) == 4, float4, uint2>::type Raw;
-    const bool fast = kvec && vvec && (dq & 3) == 0 && (dv & 3) == 0;
+    const bool fast = !TAB || (kvec && vvec && (dq & 3) == 0 && (dv & 3) == 0);
     const int ngk = (dq4 + 31) >> 5, ngv = (vcols + 31) >> 5;
     Raw kraw[NG], vraw[NG];
     auto widen = [](const Raw& u) -> float4 {
@@ -637,12 +639,12 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
       // an explicit mask: the bytes of the lane's 16 pairs, asked for ahead of the barriers below; a block they
       // all drop is left out altogether
       uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
-      if (live && p.mask) general_mask_words(p, b, qi, kv0, hh, mw);
+      if (live && p.mask) general_mask_words<!TAB>(p, b, qi, kv0, hh, mw);
       // (the block's dense-bias values likewise, where there are registers for them: one wave per SIMD)
       constexpr bool DENSE_AHEAD = DMAX > 128;
       float db[DENSE_AHEAD ? 16 : 1];
       if constexpr (DENSE_AHEAD) {
-        if (live && p.dense_bias) general_dense_row(p, b, qi, kv0, hh, db);
+        if (live && p.dense_bias) general_dense_row<!TAB>(p, b, qi, kv0, hh, db);
       }
       __syncthreads();                     // everyone is done with the tile before
       stage(kv0);
@@ -683,7 +685,7 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
       }
       if (qi >= s.n_q) hi = -1;
       const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
-      const bool tabled = p.pos_tab != nullptr || p.ts_tab != nullptr;
+      const bool tabled = TAB && (p.pos_tab != nullptr || p.ts_tab != nullptr);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
@@ -4370,6 +4372,22 @@ int launch_general(const Params& p, hipStream_t st) {
                      : allow_lds((const void*)hstu_fwd_general<T, 256>, (int)smem, granted_large)) return rc;
   hipError_t e;
   dim3 grid(p.H, p.B, (p.L + 127) / 128);
+  {
+    auto whole = [&](const void* base, int64_t row, int64_t head, int64_t batch) {
+      return ((uintptr_t)base & (4 * sizeof(T) - 1)) == 0 && ((row | head | batch) & 3) == 0;
+    };
+    const bool words = (!p.mask || ((p.Lkv & 3) == 0 && ((uintptr_t)p.mask & 3) == 0)) &&
+                       (!p.dense_bias || ((p.Lkv & 3) == 0 && ((uintptr_t)p.dense_bias & 15) == 0));
+    if (small && p.pos_tab == nullptr && p.ts_tab == nullptr && words && (p.d_qk & 3) == 0 && (p.d_v & 3) == 0 &&
+        whole(p.k, p.k_st, p.k_sh, p.k_sb) && whole(p.v, p.v_st, p.v_sh, p.v_sb)) {
+      static int granted_lean[64];
+      if (int rc = allow_lds((const void*)hstu_fwd_general<T, 128, false>, (int)smem, granted_lean)) return rc;
+      hipLaunchKernelGGL((hstu_fwd_general<T, 128, false>), grid, dim3(256), smem, st, p);
+      e = hipGetLastError();
+      if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "general kernel launch: %s", hipGetErrorString(e));
+      return HSTU_OK;
+    }
+  }
   if (small) hipLaunchKernelGGL((hstu_fwd_general<T, 128>), grid, dim3(256), smem, st, p);
   else hipLaunchKernelGGL((hstu_fwd_general<T, 256>), grid, dim3(256), smem, st, p);
   e = hipGetLastError();

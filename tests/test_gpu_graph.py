@@ -116,3 +116,40 @@ def test_backward_replays_in_a_graph(gpu):
       scale = b.abs().max().item()
       assert scale > 0
       assert (a - b).abs().max().item() <= 1e-4 * scale, f"replay {rep}: {name}"
+
+
+def test_norm_gate_and_its_gradients_replay_in_a_graph(gpu):
+  """The block's norm + gate step and its backward (two kernels: the rows' pass, then the column sums added in a
+  fixed order, no memset) recorded into one graph: every replay, with the inputs changed in place between them,
+  gives the bits of an eager call -- the column sums included."""
+  from recml_amd import hstu_block_ops as B
+  bf = torch.bfloat16
+  gen = torch.Generator(device="cuda:0").manual_seed(77)
+  rows, width = 3001, 512
+  fused = torch.randn((rows, 4, width), device="cuda:0", generator=gen).to(bf)
+  attn = (torch.randn((rows, width), device="cuda:0", generator=gen) * 3e-3).to(bf)
+  dout = torch.randn((rows, width), device="cuda:0", generator=gen).to(bf)
+  gamma = (1 + 0.2 * torch.randn(width, device="cuda:0", generator=gen)).to(bf)
+  beta = (0.1 * torch.randn(width, device="cuda:0", generator=gen)).to(bf)
+  dfused = torch.zeros_like(fused)
+
+  def call():
+    out = B.norm_gate(attn, fused[:, 0], gamma, beta, 1e-6)
+    return (out,) + B.norm_gate_bwd(attn, fused[:, 0], gamma, beta, dout, 1e-6, du_out=dfused[:, 0])
+
+  call()                                # (library loaded before capture)
+  torch.cuda.synchronize()
+  graph = torch.cuda.CUDAGraph()
+  with torch.cuda.graph(graph):
+    recorded = call()
+  for rep in range(3):
+    attn.mul_(1.5 if rep else 1.0).add_(1e-3 * rep)
+    dout.neg_()
+    fused.mul_(0.5)
+    graph.replay()
+    torch.cuda.synchronize()
+    replayed = [t.clone() for t in recorded]
+    eager = call()
+    torch.cuda.synchronize()
+    for name, a, b in zip(("out", "d_attn", "d_u", "d_gamma", "d_beta"), replayed, eager):
+      assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager call"

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define HSTU_BLOCK_ABI_VERSION 2
+#define HSTU_BLOCK_ABI_VERSION 3
 
 typedef enum HstuBlockStatus {
   HSTU_BLOCK_OK = 0,
@@ -111,7 +111,8 @@ int hstu_norm_gate_bwd(const HstuNormGateBwdArgs* args, void* stream);
 
 /* out[m, n] = silu(sum_k x[m, k] w[k, n] + bias[n]); x: bf16 [M, K] (row stride
  * x_stride), w: bf16 [K, N] contiguous, bias: bf16 [N] or null, out: bf16
- * [M, N] contiguous.  fp32 accumulation.  `workspace` (device memory, may be
+ * [M, N] contiguous; with `c` (bf16 [M, N], row stride c_stride, 16-byte aligned,
+ * c_stride a multiple of 8) out = act(x w + c + bias).  fp32 accumulation.  `workspace` (device memory, may be
  * null) is handed to hipBLASLt; hstu_gemm_silu_workspace_bytes() says how much
  * it would like.  The descriptor and the chosen algorithm of a shape are kept
  * by the library after the first call with it: every call must therefore offer
@@ -131,6 +132,8 @@ typedef struct HstuGemmSiluArgs {
   void* out;
   void* workspace;
   size_t workspace_bytes;
+  const void* c;          /* bf16 [M, N] added to the product before bias and activation, or null: the block's */
+  int64_t c_stride;       /* residual as the product's C operand (hstu.py:474), no pass of its own; row stride */
 } HstuGemmSiluArgs;
 
 size_t hstu_gemm_silu_workspace_bytes(void);

@@ -137,9 +137,12 @@ def norm_gate_bwd(attn, u, gamma, beta, dout, eps=1e-6):
   return da, du, (gn * xh).sum(red), gn.sum(red)
 
 
-def gemm_silu(x, w, bias=None, activation=True):
-  """silu(x w + bias): the block's projections with their activation (hstu.py:444-449)."""
+def gemm_silu(x, w, bias=None, activation=True, residual=None):
+  """silu(x w + bias): the block's projections with their activation (hstu.py:444-449); without the
+  activation and with `residual`, the output projection plus the block's input (hstu.py:473-474)."""
   y = np.asarray(x, np.float64) @ np.asarray(w, np.float64)
+  if residual is not None:
+    y = y + np.asarray(residual, np.float64)
   if bias is not None:
     y = y + np.asarray(bias, np.float64)
   return O.silu(y) if activation else y

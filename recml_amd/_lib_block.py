@@ -9,7 +9,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RECML_AMD_BLOCK_LIB") or os.path.join(_HERE, "lib", "libhstu_block.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 EXPORTS = (
     "hstu_block_abi_version",
@@ -59,6 +59,7 @@ class HstuGemmSiluArgs(C.Structure):
       ("x", C.c_void_p), ("x_stride", C.c_int64),
       ("w", C.c_void_p), ("bias", C.c_void_p), ("out", C.c_void_p),
       ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+      ("c", C.c_void_p), ("c_stride", C.c_int64),
   ]
 
 

@@ -404,7 +404,7 @@ constexpr size_t kBlasWorkspace = 32u << 20;
 
 struct GemmPlan {
   hipblasLtMatmulDesc_t desc = nullptr;
-  hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr;
+  hipblasLtMatrixLayout_t la = nullptr, lb = nullptr, lc = nullptr, lres = nullptr;   // lres: the C operand when it is not the output
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
 };
@@ -412,8 +412,8 @@ struct GemmPlan {
 struct BlasState {
   std::mutex mu;
   hipblasLtHandle_t handle[64] = {};
-  // (device, M, N, K, x_stride, bias?, activation, workspace offered) -> plan
-  std::map<std::tuple<int, int64_t, int, int, int64_t, int, int, size_t>, GemmPlan> plans;
+  // (device, M, N, K, x_stride, bias?, activation, workspace offered, row stride of c or 0) -> plan
+  std::map<std::tuple<int, int64_t, int, int, int64_t, int, int, size_t, int64_t>, GemmPlan> plans;
 };
 
 BlasState& blas() {
@@ -577,6 +577,8 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
   // the first call's pointers offered, so every call has to offer it
   if (!aligned16(a->x) || !aligned16(a->w) || !aligned16(a->out) || !aligned16(a->bias) || !aligned16(a->workspace) || (a->x_stride & 7))
     return fail(HSTU_BLOCK_ERR_SHAPE, "x, w, out, bias and workspace must be 16-byte aligned and x_stride a multiple of 8 elements");
+  if (a->c && (!aligned16(a->c) || (a->c_stride & 7) || a->c_stride < a->N))
+    return fail(HSTU_BLOCK_ERR_SHAPE, "c must be 16-byte aligned with a row stride that is a multiple of 8 elements and >= N");
   if (a->workspace_bytes && !a->workspace) return fail(HSTU_BLOCK_ERR_WORKSPACE, "workspace_bytes without a workspace");
   int dev = 0;
   hipError_t he = hipGetDevice(&dev);
@@ -593,7 +595,8 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtCreate: %s", blas_str(st));
     }
     handle = bs.handle[dev];
-    const auto key = std::make_tuple(dev, a->M, a->N, a->K, a->x_stride, a->bias ? 1 : 0, a->activation, a->workspace_bytes);
+    const auto key = std::make_tuple(dev, a->M, a->N, a->K, a->x_stride, a->bias ? 1 : 0, a->activation, a->workspace_bytes,
+                                     a->c ? a->c_stride : (int64_t)0);
     auto it = bs.plans.find(key);
     if (it == bs.plans.end()) {
       // row-major out[M, N] = x[M, K] w[K, N] is, in the column-major terms of the library,
@@ -609,6 +612,7 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
           if (p.la) hipblasLtMatrixLayoutDestroy(p.la);
           if (p.lb) hipblasLtMatrixLayoutDestroy(p.lb);
           if (p.lc) hipblasLtMatrixLayoutDestroy(p.lc);
+          if (p.lres) hipblasLtMatrixLayoutDestroy(p.lres);
           if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
         }
       } part;
@@ -638,6 +642,8 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
       st = hipblasLtMatrixLayoutCreate(&np.la, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->K, (int64_t)a->N);
       if (st == HIPBLAS_STATUS_SUCCESS) st = hipblasLtMatrixLayoutCreate(&np.lb, HIP_R_16BF, (uint64_t)a->K, (uint64_t)a->M, a->x_stride);
       if (st == HIPBLAS_STATUS_SUCCESS) st = hipblasLtMatrixLayoutCreate(&np.lc, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->M, (int64_t)a->N);
+      if (st == HIPBLAS_STATUS_SUCCESS && a->c)
+        st = hipblasLtMatrixLayoutCreate(&np.lres, HIP_R_16BF, (uint64_t)a->N, (uint64_t)a->M, a->c_stride);
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatrixLayoutCreate: %s", blas_str(st));
       st = hipblasLtMatmulPreferenceCreate(&part.pref);
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulPreferenceCreate: %s", blas_str(st));
@@ -646,7 +652,7 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
       if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulPreferenceSetAttribute: %s", blas_str(st));
       hipblasLtMatmulHeuristicResult_t res[1];
       int found = 0;
-      st = hipblasLtMatmulAlgoGetHeuristic(handle, np.desc, np.la, np.lb, np.lc, np.lc, part.pref, 1, res, &found);
+      st = hipblasLtMatmulAlgoGetHeuristic(handle, np.desc, np.la, np.lb, a->c ? np.lres : np.lc, np.lc, part.pref, 1, res, &found);
       if (st != HIPBLAS_STATUS_SUCCESS || found < 1)
         return fail(HSTU_BLOCK_ERR_BLAS, "hipBLASLt has no kernel for M=%lld N=%d K=%d with this epilogue (%s)",
                     (long long)a->M, a->N, a->K, blas_str(st));
@@ -657,6 +663,7 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
           hipblasLtMatrixLayoutDestroy(kv.second.la);
           hipblasLtMatrixLayoutDestroy(kv.second.lb);
           hipblasLtMatrixLayoutDestroy(kv.second.lc);
+          if (kv.second.lres) hipblasLtMatrixLayoutDestroy(kv.second.lres);
           hipblasLtMatmulDescDestroy(kv.second.desc);
         }
         bs.plans.clear();
@@ -671,9 +678,11 @@ int hstu_gemm_silu_fwd(const HstuGemmSiluArgs* a, void* stream) {
       const hipblasStatus_t sb = hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &a->bias, sizeof(void*));
       if (sb != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmulDescSetAttribute (bias pointer): %s", blas_str(sb));
     }
-    const float alpha = 1.0f, beta = 0.0f;
-    const hipblasStatus_t st = hipblasLtMatmul(handle, plan.desc, &alpha, a->w, plan.la, a->x, plan.lb, &beta, a->out, plan.lc,
-                                               a->out, plan.lc, &plan.algo, a->workspace, a->workspace_bytes, (hipStream_t)stream);
+    // (with c: D = alpha A B + beta C with C = c and beta = 1, the output written elsewhere)
+    const float alpha = 1.0f, beta = a->c ? 1.0f : 0.0f;
+    const hipblasStatus_t st = hipblasLtMatmul(handle, plan.desc, &alpha, a->w, plan.la, a->x, plan.lb, &beta, a->c ? a->c : a->out,
+                                               a->c ? plan.lres : plan.lc, a->out, plan.lc, &plan.algo, a->workspace, a->workspace_bytes,
+                                               (hipStream_t)stream);
     if (st != HIPBLAS_STATUS_SUCCESS) return fail(HSTU_BLOCK_ERR_BLAS, "hipblasLtMatmul: %s", blas_str(st));
   }
   return HSTU_BLOCK_OK;

@@ -161,9 +161,10 @@ def _rows(t, name):
   return t.reshape(-1, W)
 
 
-def gemm_silu(x, w, bias=None, activation: bool = True):
+def gemm_silu(x, w, bias=None, activation: bool = True, residual=None):
   """silu(x @ w + bias) (or without the activation): x [M, K] bf16 (row stride free), w [K, N] contiguous,
-  bias [N] or None -> [M, N] bf16."""
+  bias [N] or None -> [M, N] bf16.  `residual` [M, N] bf16 (row stride free) is added to the product as
+  its C operand, before bias and activation: the block's `+ inputs` without a pass (or a copy) of its own."""
   _check("x", x)
   _check("w", w)
   if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[0]:
@@ -196,6 +197,13 @@ def gemm_silu(x, w, bias=None, activation: bool = True):
       bias = bias.clone()
     a.bias = bias.data_ptr()
   a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+  if residual is not None:
+    _check("residual", residual)
+    if tuple(residual.shape) != (M, N):
+      raise ValueError(f"residual must be [{M}, {N}], got {tuple(residual.shape)}")
+    if residual.stride(1) != 1 or residual.stride(0) % 8 or residual.data_ptr() % 16:
+      residual = residual.contiguous()
+    a.c, a.c_stride = residual.data_ptr(), residual.stride(0)
   with torch.cuda.device(x.device):
     rc = lib.hstu_gemm_silu_fwd(C.byref(a), C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream))
   if rc != 0:

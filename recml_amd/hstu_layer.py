@@ -194,9 +194,8 @@ class HSTUBlock(torch.nn.Module):
     if fused:
       gated = hstu_block_ops.norm_gate(attn.reshape(B * L, H * hd), u.reshape(B * L, H * hd), self.attn_ln_gamma.reshape(-1),
                                        self.attn_ln_beta.reshape(-1), self.eps)
-      res = inputs.reshape(B * L, D)
-      res = res if self.output_bias is None else res + self.output_bias
-      return torch.addmm(res, gated, self.output_kernel.reshape(H * hd, D)).reshape(B, L, D)
+      return hstu_block_ops.gemm_silu(gated, self.output_kernel.reshape(H * hd, D), self.output_bias, False,
+                                      residual=inputs.reshape(B * L, D)).reshape(B, L, D)
     normed = F.layer_norm(attn.reshape(B, L, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
                           self.attn_ln_beta.reshape(-1), self.eps)
     gated = u.reshape(B, L, H * hd) * normed
@@ -277,8 +276,7 @@ class HSTUBlock(torch.nn.Module):
     if fused:
       gated = hstu_block_ops.norm_gate(attn.reshape(T, H * hd), u.reshape(T, H * hd), self.attn_ln_gamma.reshape(-1),
                                        self.attn_ln_beta.reshape(-1), self.eps)
-      res = tokens if self.output_bias is None else tokens + self.output_bias
-      return torch.addmm(res, gated, self.output_kernel.reshape(H * hd, D))
+      return hstu_block_ops.gemm_silu(gated, self.output_kernel.reshape(H * hd, D), self.output_bias, False, residual=tokens)
     normed = F.layer_norm(attn.reshape(T, H * hd), (H * hd,), self.attn_ln_gamma.reshape(-1),
                           self.attn_ln_beta.reshape(-1), self.eps)
     out = (u.reshape(T, H * hd) * normed) @ self.output_kernel.reshape(H * hd, D)

@@ -99,6 +99,7 @@ def test_oracle_compositions_on_a_hand_case():
   y = np.array([[0.0, 3.0]]) + np.array([0.5, -1.0])              # x w + bias = [0.5, 2.0]
   assert np.allclose(BO.gemm_silu(x, w, np.array([0.5, -1.0]), False), y, atol=1e-15)
   assert np.allclose(BO.gemm_silu(x, w, np.array([0.5, -1.0])), y / (1 + np.exp(-y)), atol=1e-15)
+  assert np.allclose(BO.gemm_silu(x, w, np.array([0.5, -1.0]), False, residual=np.array([[10.0, 20.0]])), y + [10.0, 20.0], atol=1e-15)
   table = np.array([[0.0, 0.0, 0.0, 0.0], [1.0, 2.0, 3.0, 4.0]])
   pos = np.array([[0.0, 0.0, 0.0, 0.0], [1.0, 1.0, 1.0, 1.0]])    # a constant row shifts the mean only
   got = BO.embed_norm(np.array([1, 1]), table, np.ones(4), np.zeros(4), 0.0, 2.0, np.array([0, 1]), pos)
@@ -219,6 +220,15 @@ def test_gemm_silu_parity(gpu, M, K, N, bias, act):
   wide = torch.zeros((M, 2 * K), device=dev, dtype=bf)
   wide[:, :K] = x
   assert torch.equal(B.gemm_silu(wide[:, :K], w, b, act), out)
+  # a residual as the product's C operand (a strided one too): added before bias and activation, and left as it was
+  res = (torch.randn((M, N), generator=gen) * 0.5).to(dev).to(bf)
+  keep = res.clone()
+  got = B.gemm_silu(x, w, b, act, residual=res)
+  ref = torch.from_numpy(BO.gemm_silu(n(x), n(w), n(b) if bias else None, act, residual=n(res)))
+  assert _rel(got.double().cpu(), ref) <= 8e-3 and torch.equal(res, keep)
+  wide_res = torch.zeros((M, 2 * N), device=dev, dtype=bf)
+  wide_res[:, :N] = res
+  assert torch.equal(B.gemm_silu(x, w, b, act, residual=wide_res[:, :N]), got)
 
 
 @pytest.mark.gpu

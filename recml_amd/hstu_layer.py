@@ -95,6 +95,26 @@ class _AttentionGateFn(torch.autograd.Function):
             cast(dpos, pos) if pos is not None else None, cast(dts, ts) if ts is not None else None, None, None, None)
 
 
+class _OutputProjectionFn(torch.autograd.Function):
+  """gated @ W (+ bias) + residual with the residual as the product's C operand (recml/layers/keras/hstu.py:473-474):
+  torch's addmm copies the residual into the output before the product.  The gradients are two plain products."""
+
+  @staticmethod
+  def forward(ctx, gated, w, bias, residual):
+    ctx.save_for_backward(gated, w)
+    ctx.has_bias = bias is not None
+    return hstu_block_ops.gemm_silu(gated, w, bias, False, residual=residual)
+
+  @staticmethod
+  def backward(ctx, dout):
+    gated, w = ctx.saved_tensors
+    need = ctx.needs_input_grad
+    d_gated = dout @ w.t() if need[0] else None
+    d_w = gated.t() @ dout if need[1] else None
+    d_bias = dout.sum(0) if (ctx.has_bias and need[2]) else None
+    return d_gated, d_w, d_bias, dout if need[3] else None
+
+
 def _glorot_uniform(shape, fan_in, fan_out, generator, dtype, device):
   limit = math.sqrt(6.0 / (fan_in + fan_out))
   w = torch.empty(shape, dtype=torch.float32)
@@ -238,8 +258,8 @@ class HSTUBlock(torch.nn.Module):
       uqkv = uqkv + b
     uqkv = F.silu(uqkv).reshape(*lead, 4, H, hd)
     gated = _AttentionGateFn.apply(uqkv, self.attn_ln_gamma, self.attn_ln_beta, pos_bias, ts_bias, self.eps, batch, attn_kw)
-    res = tokens if self.output_bias is None else tokens + self.output_bias
-    return torch.addmm(res, gated.reshape(-1, H * hd), self.output_kernel.reshape(H * hd, self.hidden_dim))
+    return _OutputProjectionFn.apply(gated.reshape(-1, H * hd), self.output_kernel.reshape(H * hd, self.hidden_dim),
+                                     self.output_bias, tokens)
 
   def _uqkv_weights(self):
     w = torch.cat([self.u_kernel, self.q_kernel, self.k_kernel, self.v_kernel], dim=1).reshape(self.hidden_dim, -1)

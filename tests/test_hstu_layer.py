@@ -269,7 +269,8 @@ def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
 
 
 @pytest.mark.gpu
-def test_packed_block_trains_through_the_fused_steps(gpu):
+@pytest.mark.parametrize("use_bias", [False, True])
+def test_packed_block_trains_through_the_fused_steps(gpu, use_bias):
   """forward_jagged in bf16 with gradients: the fused training steps (kernel layer norms, attention + norm
   + gate as one function) against the same block with torch's norms and gate around the attention
   function, on packed tokens with timestamps and both tables; and the fused path is the one taken."""
@@ -282,7 +283,12 @@ def test_packed_block_trains_through_the_fused_steps(gpu):
   lens = [200, 1, 77, 130]
   T, L = sum(lens), 256
   offsets = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=dev)
-  blk = HSTUBlock(D, H, dtype=bf, device=dev, generator=gen)
+  blk = HSTUBlock(D, H, use_bias=use_bias, dtype=bf, device=dev, generator=gen)
+  if use_bias:
+    with torch.no_grad():
+      for name, prm in blk.named_parameters():
+        if name.endswith("_bias"):
+          prm.copy_((torch.randn(prm.shape, generator=gen) * 0.1).to(dev).to(bf))
   blk.requires_grad_(True)
   x = (torch.randn((T, D), generator=gen) * 0.5).to(dev).to(bf).requires_grad_(True)
   pos = (torch.randn((H, 2 * L - 1), generator=gen) * 0.3).to(dev).requires_grad_(True)
@@ -318,6 +324,7 @@ def test_packed_block_trains_through_the_fused_steps(gpu):
   out_t, want = grads(False)
   assert float((out_f - out_t).abs().max() / out_t.abs().max()) <= 2e-2
   assert set(got) == set(want) and {"u_kernel", "attn_ln_beta", "input_ln_gamma"} <= set(got)
+  assert ("output_bias" in got and "q_bias" in got) == use_bias
   for name in want:
     err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
     assert err <= 4e-2, (name, err)                   # bf16 activations on both sides, rounded at different points

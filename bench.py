@@ -265,6 +265,8 @@ def bench_model(args, dev):
   # gradients' shapes -- a small output, 70 k rows to sum over -- leaves most of the chip idle)
   train_tuned_ms = None
   try:
+    if not args.tuned:
+      raise RuntimeError("switched off (--no-tuned-products)")
     import torch.cuda.tunable as tunable
     import tempfile
     tunable.enable(True)
@@ -630,6 +632,9 @@ def main():
                   help="diagnostics: force resident workgroups that loop over the work list")
   ap.add_argument("--ramp-ms", type=float, default=300.0,
                   help="untimed calls for this long before anything is measured (clock ramp from idle)")
+  ap.add_argument("--no-tuned-products", dest="tuned", action="store_false",
+                  help="c4-model: skip the training step with torch's tuned matrix products (its search runs hundreds of "
+                       "candidate kernels: leave it out under a profiler)")
   ap.add_argument("--calib-copy", action="store_true",
                   help="also run one 512 MiB device copy (reference point for HBM byte counters)")
   args = ap.parse_args()

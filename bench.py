@@ -630,6 +630,8 @@ def main():
                   help="diagnostics: force one workgroup per work-list entry")
   ap.add_argument("--resident-workgroups", action="store_true",
                   help="diagnostics: force resident workgroups that loop over the work list")
+  ap.add_argument("--compiler-scheduled-blocks", action="store_true",
+                  help="diagnostics: interior steps through the compiler-scheduled block code instead of the hand-scheduled stream")
   ap.add_argument("--ramp-ms", type=float, default=300.0,
                   help="untimed calls for this long before anything is measured (clock ramp from idle)")
   ap.add_argument("--no-tuned-products", dest="tuned", action="store_false",
@@ -674,6 +676,8 @@ def main():
     call_args.flags |= _lib.FWD_ONE_ITEM_PER_WORKGROUP
   if args.resident_workgroups:
     call_args.flags |= _lib.FWD_RESIDENT_WORKGROUPS
+  if args.compiler_scheduled_blocks:
+    call_args.flags |= _lib.FWD_COMPILER_SCHEDULED_BLOCKS
 
   def step():
     hstu_ops._run(call_args, keep)

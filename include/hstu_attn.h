@@ -77,7 +77,13 @@ enum HstuFwdFlags {
    * batch has at least 8 entries per resident workgroup.  These bits force one
    * or the other (the first wins); the results are the same bit for bit. */
   HSTU_FWD_ONE_ITEM_PER_WORKGROUP = 4,
-  HSTU_FWD_RESIDENT_WORKGROUPS = 8
+  HSTU_FWD_RESIDENT_WORKGROUPS = 8,
+  /* The matrix-core kernel at d = 128 in bf16 runs the steps that no mask touches
+   * as one hand-scheduled instruction stream (software-pipelined across steps).
+   * This bit sends those steps through the compiler-scheduled code that handles
+   * every other step instead: a comparison switch; same arithmetic in the same
+   * order, the same bits out. */
+  HSTU_FWD_COMPILER_SCHEDULED_BLOCKS = 16
 };
 
 /* Return codes (0 = launched). */

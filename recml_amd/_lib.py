@@ -17,6 +17,7 @@ FWD_WORKSPACE_PREPARED = 1
 FWD_PREPARE_ONLY = 2
 FWD_ONE_ITEM_PER_WORKGROUP = 4
 FWD_RESIDENT_WORKGROUPS = 8
+FWD_COMPILER_SCHEDULED_BLOCKS = 16
 NOALLOC_SCRATCH_BYTES = 4 << 20   # HSTU_ATTN_NOALLOC_SCRATCH_BYTES
 MASK_NONE, MASK_LENGTH, MASK_SEGMENT = 0, 1, 2
 

@@ -16,6 +16,9 @@ BLOCK_LIB_PATH = os.path.join(LIB_DIR, "libhstu_block.so")
 BLOCK_SOURCES = [os.path.join(_HERE, "csrc", "hstu_block.hip")]
 BLOCK_LINK = ["-lhipblaslt"]
 INCLUDE = os.path.join(ROOT, "include")
+# the block's microbenchmark: a stand-alone program (its own main), evidence for what bounds the kernel
+MICRO_PATH = os.path.join(LIB_DIR, "micro_fwd_stream")
+MICRO_SOURCES = [os.path.join(_HERE, "csrc", "micro_fwd_stream.hip")]
 
 # -packed-fp32-ops is switched off for the device pass: packed fp32
 # instructions are not wanted in these kernels.  The host pass does not know
@@ -56,6 +59,22 @@ def build_block_library(verbose: bool = False) -> str:
   return _compile(BLOCK_SOURCES, BLOCK_LIB_PATH, BLOCK_LINK, verbose=verbose)
 
 
+def build_microbench(verbose: bool = False) -> str:
+  """Compiles the forward block's microbenchmark into recml_amd/lib/micro_fwd_stream (an executable)."""
+  os.makedirs(LIB_DIR, exist_ok=True)
+  tmp = MICRO_PATH + ".tmp"
+  flags = [f for f in HIPCC_FLAGS if f not in ("-fPIC", "-shared")]
+  cmd = [hipcc(), *flags, "-o", tmp, *MICRO_SOURCES]
+  res = subprocess.run(cmd, capture_output=True, text=True)
+  if res.returncode != 0:
+    raise RuntimeError("hipcc failed:\n" + res.stdout + res.stderr)
+  if verbose:
+    print(res.stderr)
+  os.replace(tmp, MICRO_PATH)
+  return MICRO_PATH
+
+
 if __name__ == "__main__":
   print(build_library(verbose=True))
   print(build_block_library(verbose=True))
+  print(build_microbench(verbose=True))

@@ -113,6 +113,7 @@ struct Params {
   int32_t n_slots;           // workgroups that run at once per XCD (what the split decision balances for)
   const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
+  int32_t no_stream;         // forward: interior steps through the compiler-scheduled block code too (a comparison switch)
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
   uint32_t* ctr;             // workspace: [0, 8) draw counters of the XCDs, [8] workgroups done, then from
                              // CTR_RESERVED on one arrival counter per (chunk slot, head); all zero between launches
@@ -2219,6 +2220,8 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 constexpr int fwd_stages(int d, int dense) { return (d <= 64 || dense != 0) ? 3 : 4; }
 constexpr int FWD_XCH_BYTES = 16;     // behind everything else in the forward kernel's LDS
 
+#include "hstu_fwd_stream_d128.inc"   // (the variants' names; the statements are expanded inside the kernel)
+
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0, bool PERSIST = false>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
   constexpr int KB = F8 ? 1 : 2;       // bytes per q / k element
@@ -2339,10 +2342,14 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // issues the same number of loads per step: the vmcnt arithmetic relies on it.
   // The ring stage is a compile-time constant everywhere (the step loop is unrolled over the ring):
   // LDS addresses are then a per-lane register plus an immediate, with no address arithmetic per step.
-  auto dma_step = [&](const DmaCtx& c_, int t, auto st_) {
+  // `part_`: 3 = the whole step, 1 = its K tile and bias operands only, 2 = its V tile only (the hand-scheduled
+  // stream of the interior steps keeps the K side of the ring one step ahead of the V side).
+  auto dma_part = [&](const DmaCtx& c_, int t, auto st_, auto part_) {
     constexpr int st = decltype(st_)::value;
+    constexpr int part = decltype(part_)::value;
     const int kv0 = t * BN;
     const int last = c_.n_kv - 1;
+    if constexpr ((part & 1) != 0) {
 #pragma unroll
     for (int r = 0; r < LDK; ++r) {
       const int j = (w * LDK + r) % NPIECE_K;   // small tiles: several waves repeat the same piece
@@ -2353,6 +2360,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       const uint32_t koff = (uint32_t)grow * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
       lds_dma16(c_.kg, koff, (const unsigned char*)Ks(st) + j * 1024);
     }
+    }
+    if constexpr ((part & 2) != 0) {
 #pragma unroll
     for (int r = 0; r < LD; ++r) {
       const int j = (w * LD + r) % NPIECE;
@@ -2363,7 +2372,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       const uint32_t voff = (uint32_t)grow * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
       lds_dma16(c_.vg, voff, Vs(st) + j * 512);
     }
-    if (POS || TS) {
+    }
+    if ((POS || TS) && (part & 1) != 0) {
       // One more load per wave brings the bias operands.  Wave c writes position-window copy c:
       // window[x + c], window[x] = pos[(L-1) + kv0 - (q0+127) + x]; the table index is
       // >= POS_PAD - 127 > 0 and inside the padded table (the offset register is unsigned: a
@@ -2389,7 +2399,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
       if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
     }
-    if (SEG) {
+    if (SEG && (part & 1) != 0) {
       // every wave brings the same 32 ids (each wave must issue the same number of loads); groups of 4
       // past the row repeat the last group (L is a multiple of 4; those keys are masked by their index)
       if (lane < BN / 4) {
@@ -2399,6 +2409,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
     }
   };
+  auto dma_step = [&](const DmaCtx& c_, int t, auto st_) { dma_part(c_, t, st_, std::integral_constant<int, 3>{}); };
   // The dense operands of step t, each wave its own rows (the same number of loads whatever the step).
   auto dense_refill = [&](const DmaCtx& c_, int t) {
     const int kv0 = t * BN;
@@ -2864,6 +2875,76 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
     }
   };
+  // ---- The interior steps as one hand-scheduled instruction stream (d = 128 in bf16, no timestamps, segment ids
+  // or dense operands; hstu_fwd_stream_d128.inc, written by gen_fwd_stream.py).  A step is interior when every key
+  // of it is kept for every row of the tile: under the causal mask the steps below the tile's first row, without
+  // it those that lie whole inside the sequence.  The stream takes them four at a time from the item's first step
+  // on (ring stage 0), software-pipelined across steps, with the K side of the ring one step ahead of the V side.
+  // It starts where a pair of the loops below would start (the first two steps' tiles in the ring and published,
+  // nothing else in flight) and sends for the K side of the third step itself; on exit, n quads later, the tiles of
+  // the next two steps are in the ring and published (and the K side of the one after), so the paired loop takes
+  // over where the stream stops.  The stream's last pair asks for K tiles up to two steps past its end and for V
+  // tiles up to one: those steps must exist and lie whole inside the sequence (no row to clamp).  The arithmetic
+  // and its order are those of `block`: the same bits either way.
+  constexpr bool STREAM = D == 128 && !TS && !F8 && !SEG && DENSE == 0 && PAIRS;
+  auto stream_quads = [&]() -> int {
+    if constexpr (!STREAM) return 0;
+    const Params pf = fresh();
+    if (pf.no_stream || win >= 0) return 0;
+    int keys = s.n_kv;
+    if (pf.causal) keys = q0 < keys ? q0 : keys;
+    const int t_int = keys / BN;                 // steps [0, t_int) are interior for all four waves
+    int n = (t_int - t_lo) >> 2;
+    // lookahead: steps up to t_lo + 4n + 2 exist and are whole
+    const int whole = s.n_kv / BN;
+    while (n > 0 && !(t_lo + 4 * n + 2 < nt && t_lo + 4 * n + 3 <= whole)) --n;
+    return n > 0 ? n : 0;
+  };
+  auto run_stream = [&](int n_quads) {
+    if constexpr (STREAM) {
+      typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+      uintx4 hs_q[8];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) hs_q[ks] = uintx4{qf[ks].x, qf[ks].y, qf[ks].z, qf[ks].w};
+      uint32_t hs_ka[8], hs_va[4];
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) hs_ka[ks] = smem_lds + (uint32_t)(m * 256 + (((2 * ks + hh) ^ gk) * 16));
+#pragma unroll
+      for (int d = 0; d < 4; ++d) hs_va[d] = smem_lds + (uint32_t)(SM::K_BYTES + vrow * 256 + 8 * (gi & 1) + vc2 * 16 + ((d ^ gq) & 3) * 64);
+      const int xb = 4 * hh + (BM - 1) - 32 * w - m, sft = xb & 3;
+      const uint32_t hs_pa = smem_lds + (uint32_t)(BIAS_OFF + sft * SM::POS_COPY + (xb - sft) * 4);
+      uint32_t hs_koff[2], hs_voff[2];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int c = 64 * (2 * w + r) + lane, row = c / 16, pc = c - row * 16;
+        hs_koff[r] = (uint32_t)row * kst_bytes + (uint32_t)((pc ^ SM::swz_k(row)) * 16);
+        hs_voff[r] = (uint32_t)row * vst_bytes + (uint32_t)((pc ^ SM::swz_v(row)) * 16);
+      }
+      const uint32_t hs_kdst = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(2 * w * 1024));
+      const uint32_t hs_vdst = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(SM::K_BYTES + 2 * w * 1024));
+      const uint32_t hs_kstep = (uint32_t)BN * kst_bytes, hs_vstep = (uint32_t)BN * vst_bytes;
+      const char* hs_kp = cx.kg + (size_t)(t_lo + 2) * hs_kstep;
+      const char* hs_vp = (const char*)cx.vg + (size_t)(t_lo + 2) * hs_vstep;
+      const uint32_t hs_bdst = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(BIAS_OFF + w * SM::POS_COPY));
+      const uint32_t hs_boff = (uint32_t)(w + 4 * lane) * 4u;
+      const uint64_t hs_bexec = (1ull << SM::POS_LANES) - 1ull;
+      // the window of step t starts at table entry POS_PAD + (L - 1) + 32 t - (q0 + 127) of the head's padded table
+      const char* hs_bp = wsb + cx.pos_off + (int64_t)(POS_PAD + (fresh().L - 1) + BN * (t_lo + 2) - (q0 + BM - 1)) * 4;
+      const float hs_alpha = alpha2;
+      int hs_n = n_quads;
+      floatx16 (&hs_o)[DVB] = o;
+      if constexpr (POS) {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_FULL_POS
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+      } else {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_FULL
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+        (void)hs_pa; (void)hs_bdst; (void)hs_boff; (void)hs_bexec; (void)hs_bp;
+      }
+    }
+  };
   if constexpr (!PERSIST) {
     // ---- one item per workgroup
     Work first;
@@ -2887,6 +2968,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     if constexpr (NSTAGE > 3 && !PAIRS) {
       if (t_lo + 2 < nt) dma_step(cx, t_lo + 2, std::integral_constant<int, 2>{});
     }
+    const int n_quads = stream_quads();
     zero_o();
     if constexpr (PAIRS) {
       // Steps in pairs, one barrier per pair.  The barrier that ended the pair (t-2, t-1) freed that
@@ -2899,6 +2981,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       // and so does a fourth stage bought for them at d <= 64, 110 -> 116 us.)
       HSTU_WAIT_VMCNT(0);
       __syncthreads();
+      if (n_quads > 0) run_stream(n_quads);
       auto pair = [&](int t, auto st_) {
         constexpr int st = decltype(st_)::value;
         if (t + 2 < nt) dma_step(cx, t + 2, std::integral_constant<int, (st + 2) % NSTAGE>{});
@@ -2908,7 +2991,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         HSTU_WAIT_VMCNT(0);
         __syncthreads();
       };
-      for (int t = t_lo; t < nt; t += NSTAGE) {
+      for (int t = t_lo + 4 * n_quads; t < nt; t += NSTAGE) {
         pair(t, std::integral_constant<int, 0>{});
         if (t + 2 >= nt) break;
         pair(t + 2, std::integral_constant<int, 2>{});
@@ -3001,6 +3084,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       zero_o();
       HSTU_WAIT_VMCNT(0);                  // the item's first pair of tiles, its Q rows, the stores of the item before
       __syncthreads();
+      // the item's interior steps, four at a time, as the hand-scheduled stream; the loop below takes the rest
+      const int n_quads = stream_quads();
+      if (n_quads > 0) run_stream(n_quads);
+      const int t_first = t_lo + 4 * n_quads;
       // the next item: known from the draw on
       bool have_next = false, drew = false;
       int head_next = 0;
@@ -3022,7 +3109,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       // That last pair is where the next item's first tiles are sent for (into stages (0, 1), free since the
       // barrier before it) and, once the last logits are done, its Q rows; it ends without waiting for
       // them: the item's rows are written while they arrive.
-      for (int t = t_lo;; t += 4) {
+      for (int t = t_first;; t += 4) {
         // stages (0, 1)
         const bool draw = !drew && t + 8 >= nt;
         if (t + 2 < nt) dma_step(cx, t + 2, std::integral_constant<int, 2>{});
@@ -4204,7 +4291,7 @@ int validate(const HstuAttnFwdArgs* a) {
     return fail(HSTU_ERR_VERSION, "args struct_size/version (%u/%u) do not match this library (%zu/%d)",
                 a->struct_size, a->version, sizeof(HstuAttnFwdArgs), HSTU_ATTN_ABI_VERSION);
   constexpr uint32_t known_flags = HSTU_FWD_WORKSPACE_PREPARED | HSTU_FWD_PREPARE_ONLY | HSTU_FWD_ONE_ITEM_PER_WORKGROUP |
-                                   HSTU_FWD_RESIDENT_WORKGROUPS;
+                                   HSTU_FWD_RESIDENT_WORKGROUPS | HSTU_FWD_COMPILER_SCHEDULED_BLOCKS;
   if ((uint32_t)a->flags & ~known_flags) return fail(HSTU_ERR_SHAPE, "unknown bits in flags: 0x%x", (unsigned)a->flags);
   const bool empty = a->B == 0 || (a->layout == HSTU_LAYOUT_JAGGED && a->total_tokens == 0);
   if (!empty && (!a->q || !a->k || !a->v || !a->out))
@@ -4851,6 +4938,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
       const bool count_known = q.jagged || !q.seq_lens;
       const long long tiles = q.jagged ? args->total_tokens / BM + args->B : (long long)args->B * q.n_qtiles;
       const long long jobs_per_xcd = q.H >= 8 ? tiles * (q.H >> 3) : tiles / (8 / q.H);
+      q.no_stream = (args->flags & HSTU_FWD_COMPILER_SCHEDULED_BLOCKS) ? 1 : 0;
       q.persist = can_stay && !(args->flags & HSTU_FWD_ONE_ITEM_PER_WORKGROUP) &&
                   ((args->flags & HSTU_FWD_RESIDENT_WORKGROUPS) || (count_known && jobs_per_xcd >= 8LL * q.n_slots));
       if (int rc2 = f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st)) return rc2;

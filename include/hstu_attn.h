@@ -65,7 +65,7 @@ enum HstuFwdFlags {
    * hold. */
   HSTU_FWD_WORKSPACE_PREPARED = 1,
   /* Only prepare the workspace (the kernel that builds the work list, the scaled
-   * tables and the int32 timestamps) and return: a model whose layers share
+   * tables, the int32 timestamps and the timestamp descriptors) and return: a model whose layers share
    * lengths, timestamps and bias tables prepares once per batch and then calls
    * every layer with HSTU_FWD_WORKSPACE_PREPARED and the same workspace. */
   HSTU_FWD_PREPARE_ONLY = 2,
@@ -174,7 +174,13 @@ int hstu_attn_abi_version(void);
  * preparation kernel builds (on every call, or once per batch, see
  * HSTU_FWD_PREPARE_ONLY): the work list of (sequence, query tile, key chunk)
  * items, the scaled position table, the timestamp bucket tables, int32
- * timestamps with their per-tile ranges, for a dense mask the range of key
+ * timestamps with their per-tile ranges, for a timestamp bias at d = 128 in
+ * bf16 under the causal mask one 16-bit descriptor per (query row, step of 32
+ * keys) -- the bucket of the step's nearest key and how many of its keys lie one
+ * bucket further, or a flag that says the step needs the per-pair lookup --
+ * written by a second small kernel (2 bytes x rows x ceil(L/32); left out, and
+ * the per-pair lookup used throughout, for L above 16384, above 256 MiB, or
+ * when the buffer is too small for them), for a dense mask the range of key
  * steps in which it keeps anything per tile of 128 query rows (the mask is
  * read once for that); and what the main kernel itself
  * uses: the counters it draws work from and, for query tiles whose keys are

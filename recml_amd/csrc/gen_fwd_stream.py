@@ -53,7 +53,7 @@ class Regs:
   """The stream's own registers from v[base] up.  With `alias` the K fragments share registers with
   the V fragments of keys 0..15 and with the position window (96 registers), else 128."""
 
-  def __init__(self, base: int, alias: bool, lag: bool = False):
+  def __init__(self, base: int, alias: bool, lag: bool = False, ts: bool = False):
     assert base % 4 == 0
     self.base = base
     b = base
@@ -82,6 +82,9 @@ class Regs:
     else:
       self.vfa = b; b += 16
       self.posw = b; b += 16
+    # timestamp bias: the lane's descriptor, its count of far keys (less 4 * half), the two table values, two scratch
+    if ts:
+      self.dsc = b; self.cp = b + 1; self.vn = b + 2; self.vf = b + 3; self.sel = b + 4; b += 6
     self.end = b
     assert self.end <= 256
 
@@ -151,13 +154,14 @@ LDS_SLOTS_DEEP = {-1: ["k0", "k1"], 1: ["va0"], 2: ["va1"], 5: ["vb0"], 6: ["vb1
 
 class Gen:
   def __init__(self, pos: bool, dma: bool, base: int = 160, alias: bool = True, lds_slots=None, valu: str = "phases", ablate=(),
-               lag: bool = False, pos_slot: int = 11):
+               lag: bool = False, pos_slot: int = 11, ts: bool = False):
     self.pos = pos
+    self.ts = ts
     self.dma = dma
     self.lag = lag
     self.pos_slot = pos_slot
     self.parity = 0               # lag schedule: which P buffer the iteration at hand writes
-    self.R = Regs(140 if lag else base, alias, lag)
+    self.R = Regs(140 if lag else base, alias, lag, ts)
     self.S = Stream(ablate)
     self.alias = alias
     self.lds_slots = lds_slots or (LDS_SLOTS_ALIAS if alias else LDS_SLOTS_DEEP)
@@ -172,7 +176,36 @@ class Gen:
 
   @property
   def bias_stage(self):
+    """Bytes of one ring stage's bias operands (the kernel's BIAS_STAGE).  With timestamps: four times (window
+    copy | 64 bytes of descriptors), then 144 bytes of key timestamps."""
+    if self.ts: return 4 * ((656 if self.pos else 0) + 64) + 144
     return POS_BYTES if self.pos else 0
+
+  # ---- timestamp bias from descriptors
+  def desc_read(self, kst: int):
+    R, S = self.R, self.S
+    S.lds(f"ds_read_u16 {R.r(R.dsc)}, %[dsa] offset:{kst * self.bias_stage}", "dsc")
+
+  def desc_unpack(self):
+    """bucket -> address of its table value; count of far keys less 4 * half."""
+    R, S = self.R, self.S
+    S.need("dsc")
+    S.emit(f"v_and_b32 {R.r(R.sel)}, 127, {R.r(R.dsc)}")
+    S.emit(f"v_bfe_u32 {R.r(R.cp)}, {R.r(R.dsc)}, 7, 6")
+    S.emit(f"v_lshl_add_u32 {R.r(R.sel)}, {R.r(R.sel)}, 2, %[tva]")
+    S.emit(f"v_sub_u32 {R.r(R.cp)}, {R.r(R.cp)}, %[hh4]")
+
+  def value_read(self):
+    R, S = self.R, self.S
+    S.lds(f"ds_read2_b32 {R.r(R.vn, 2)}, {R.r(R.sel)} offset1:1", "tsv")
+
+  def ts_ops(self, r: int):
+    """u[r] += the far value when the key's index in the step, 4 half + 8 (r / 4) + r % 4, is below the count."""
+    R = self.R
+    sel = R.sel + (r & 1)
+    return [(f"v_cmp_lt_i32 vcc, {8 * (r >> 2) + (r & 3)}, {R.r(R.cp)}", ("tsv",)),
+            (f"v_cndmask_b32 {R.r(sel)}, {R.r(R.vn)}, {R.r(R.vf)}, vcc", ()),
+            (f"v_add_f32 {R.r(R.u + r)}, {R.r(R.u + r)}, {R.r(sel)}", ())]
 
   # ---- the pieces of an iteration
   def k_reads(self, kst: int, lo: int, hi: int):
@@ -230,9 +263,12 @@ class Gen:
       p = R.p0 if cc == 0 else R.p1
       P.append([(f"v_cvt_pk_bf16_f32 {R.r(p + j)}, {R.r(R.e + 2 * j)}, {R.r(R.e + 2 * j + 1)}", ()) for j in range(4)])
     if self.valu == "phases":
-      # scale + bias of all 16, then per half: 8 exp2, 8 add, 8 rcp, 8 mul, 4 pack
+      # scale + bias of all 16, then per half: (the timestamp bias of its 8,) 8 exp2, 8 add, 8 rcp, 8 mul, 4 pack
       ops = list(U)
-      for cc in range(2): ops += E[cc] + A[cc] + RC[cc] + M[cc] + P[cc]
+      for cc in range(2):
+        if self.ts:
+          for r in range(8 * cc, 8 * cc + 8): ops += self.ts_ops(r)
+        ops += E[cc] + A[cc] + RC[cc] + M[cc] + P[cc]
       return ops
     raise ValueError(self.valu)
 
@@ -242,7 +278,7 @@ class Gen:
     kst = (vst + 1) % NSTAGE
     ops = self.valu_ops() if "novalu" not in self.ablate else []
     n_ops = len(ops)
-    # vector instructions per slot, as even as 88 over 16 goes
+    # vector instructions per slot, as even as 88 (136 with timestamps) over 16 goes
     per_slot = [(n_ops * (s + 1)) // 16 - (n_ops * s) // 16 for s in range(16)]
     pos_in_ops = 0
     if first_of_pair:
@@ -273,6 +309,14 @@ class Gen:
       for g in self.lds_slots.get(slot, ()):
         if g == "k1" and self.alias and n_ops: assert pos_in_ops >= 16   # the window's registers are free
         self.lds_group(g, vst, kst, last)
+      if self.ts and not last:
+        # the next block's descriptor: read early, unpacked once this block's timestamp instructions are out
+        # (they use the same registers), its two table values asked for right behind
+        if slot == 3: self.desc_read(kst)
+        if slot == 11:
+          assert pos_in_ops >= 16 + 48 + 36
+          self.desc_unpack()
+          self.value_read()
     assert pos_in_ops == n_ops
 
   def valu_ops_lag(self, pcur: int):
@@ -399,7 +443,13 @@ class Gen:
     for r in range(2): self._load(L, "%[kdst]", st * STAGE + r * 1024, f"%[koff{r}]", "s[90:91]")
     L.append("s_add_u32 s90, s90, %[kstep]")
     L.append("s_addc_u32 s91, s91, 0")
-    if self.pos:
+    if self.ts:
+      # window, descriptors and key timestamps move on by different strides: a per-lane increment
+      L.append("s_mov_b64 exec, %[bexec]")
+      self._load(L, "%[bdst]", st * self.bias_stage, "%[boff]", "s[94:95]")
+      L.append("v_add_u32 %[boff], %[boff], %[binc]")
+      L.append("s_mov_b64 exec, -1")
+    elif self.pos:
       L.append("s_mov_b64 exec, %[bexec]")
       self._load(L, "%[bdst]", st * self.bias_stage, "%[boff]", "s[94:95]")
       L.append("s_mov_b64 exec, -1")
@@ -437,6 +487,10 @@ class Gen:
       S.need(f"k{ks}")
       S.emit(mfma(R.r(R.sacc, 16), R.r(R.kf + 4 * ks, 4), self.q(ks), "0" if ks == 0 else R.r(R.sacc, 16)))
     if self.pos: self.pos_reads(kst)
+    if self.ts:
+      self.desc_read(kst)
+      self.desc_unpack()
+      self.value_read()
     # the scale + bias instructions read the accumulator: 11 wait states behind the last matrix instruction
     S.emit("s_nop 7")
     S.emit("s_nop 3")
@@ -484,7 +538,7 @@ def full_variant(pos: bool, base: int, **kw) -> Gen:
   S = g.S
   S.emit("s_mov_b64 s[90:91], %[kp]")
   S.emit("s_mov_b64 s[92:93], %[vp]")
-  if pos: S.emit("s_mov_b64 s[94:95], %[bp]")
+  if pos or g.ts: S.emit("s_mov_b64 s[94:95], %[bp]")
   (g.prologue_lag if g.lag else g.prologue)(0)
   # The first pair's loads overwrite ring stage 0 on the K side (the tile and window of step 4), which every
   # wave has just read for the first block's logits: they wait for each other before any of them sends for it.
@@ -501,7 +555,7 @@ def full_variant(pos: bool, base: int, **kw) -> Gen:
       it(vst, first_of_pair=True, dma_lines=lines)
       if first and pair == 0:
         # this wave's share of step 2's K side has landed once at most the pair's own loads are in flight
-        own = (3 if pos else 2) * 2 + 2 * 2
+        own = (3 if (pos or g.ts) else 2) * 2 + 2 * 2
         S.emit(f"s_waitcnt vmcnt({own})")
         S.emit("s_barrier")
       else:
@@ -528,14 +582,22 @@ def asm_statement(g: Gen) -> str:
   ins += [f'[ka{ks}] "v"(hs_ka[{ks}])' for ks in range(8)]
   ins += [f'[va{d}] "v"(hs_va[{d}])' for d in range(4)]
   if g.pos: ins.append('[pa] "v"(hs_pa)')
+  if g.ts:
+    ins += ['[dsa] "v"(hs_dsa)', '[tva] "s"(hs_tva)', '[hh4] "v"(hs_hh4)']
+    clob_extra = ['"vcc"']
+  else:
+    clob_extra = []
   outs = [f'[o{d}] "+v"(hs_o[{d}])' for d in range(4)] + ['[n] "+s"(hs_n)']
-  clob = ['"memory"', '"scc"'] + [f'"{c}"' for c in g.R.clobbers()]
+  clob = ['"memory"', '"scc"'] + clob_extra + [f'"{c}"' for c in g.R.clobbers()]
   if g.dma:
     ins += ['[kdst] "s"(hs_kdst)', '[vdst] "s"(hs_vdst)', '[kstep] "s"(hs_kstep)', '[vstep] "s"(hs_vstep)']
     ins += [f'[koff{r}] "v"(hs_koff[{r}])' for r in range(2)] + [f'[voff{r}] "v"(hs_voff[{r}])' for r in range(2)]
     ins += ['[kp] "s"(hs_kp)', '[vp] "s"(hs_vp)']
     clob += ['"m0"'] + [f'"s{i}"' for i in range(90, 96)]
-    if g.pos:
+    if g.ts:
+      ins += ['[bdst] "s"(hs_bdst)', '[binc] "v"(hs_binc)', '[bexec] "s"(hs_bexec)', '[bp] "s"(hs_bp)']
+      outs.append('[boff] "+v"(hs_boff)')
+    elif g.pos:
       ins += ['[bdst] "s"(hs_bdst)', '[boff] "v"(hs_boff)', '[bexec] "s"(hs_bexec)', '[bp] "s"(hs_bp)']
   return (f"  asm volatile(\n{g.S.text()}"
           f"      : {', '.join(outs)}\n      : {', '.join(ins)}\n      : {', '.join(clob)});\n")
@@ -590,11 +652,14 @@ def main():
   ap.add_argument("--experiments", default=None, help="also write the sweep's variants (for micro_fwd_stream.hip -DHSTU_STREAM_EXPERIMENTS) to this file")
   a = ap.parse_args()
   parts = ["// Generated by gen_fwd_stream.py: do not edit.  The hand-scheduled stream of the forward kernel's interior blocks.\n",
-           "#define HSTU_STREAM_COMPUTE_ONLY 1\n#define HSTU_STREAM_COMPUTE_ONLY_POS 2\n#define HSTU_STREAM_FULL 3\n#define HSTU_STREAM_FULL_POS 4\n"]
+           "#define HSTU_STREAM_COMPUTE_ONLY 1\n#define HSTU_STREAM_COMPUTE_ONLY_POS 2\n#define HSTU_STREAM_FULL 3\n#define HSTU_STREAM_FULL_POS 4\n"
+           "#define HSTU_STREAM_FULL_TS 5\n#define HSTU_STREAM_FULL_POS_TS 6\n"]
   parts.append(statement(compute_only_variant(False, a.base, **PRODUCT), "HSTU_STREAM_COMPUTE_ONLY"))
   parts.append(statement(compute_only_variant(True, a.base, **PRODUCT), "HSTU_STREAM_COMPUTE_ONLY_POS"))
   parts.append(statement(full_variant(False, a.base, **PRODUCT), "HSTU_STREAM_FULL"))
   parts.append(statement(full_variant(True, a.base, **PRODUCT), "HSTU_STREAM_FULL_POS"))
+  parts.append(statement(full_variant(False, a.base - 8, ts=True, **PRODUCT), "HSTU_STREAM_FULL_TS"))
+  parts.append(statement(full_variant(True, a.base - 8, ts=True, **PRODUCT), "HSTU_STREAM_FULL_POS_TS"))
   with open(a.out, "w") as f:
     f.write("".join(parts))
   print("wrote", a.out)

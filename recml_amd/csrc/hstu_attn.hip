@@ -114,6 +114,13 @@ struct Params {
   const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
   int32_t no_stream;         // forward: interior steps through the compiler-scheduled block code too (a comparison switch)
+  // Timestamp descriptors (matrix-core forward at d = 128; null = none): one 16-bit word per (32-key step, query
+  // row), [step][row] with `ts_desc_pitch` rows per step, built by hstu_prepare_ts_desc for every head and layer of
+  // a batch; and per 128-row tile the number of leading quads of steps in which no row needs the per-pair lookup.
+  const uint16_t* ts_desc;
+  const int32_t* ts_tquads;
+  int32_t ts_desc_pitch;
+  int32_t ts_desc_tiles;     // entries of ts_tquads
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
   uint32_t* ctr;             // workspace: [0, 8) draw counters of the XCDs, [8] workgroups done, then from
                              // CTR_RESERVED on one arrival counter per (chunk slot, head); all zero between launches
@@ -2050,6 +2057,11 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     if (p.ctr)
       for (int i = tid; i < CTR_RESERVED + p.split_cap * p.H; i += 256) p.ctr[i] = 0u;
   }
+  if (p.ts_tquads) {
+    // the descriptor kernel, which follows, takes each tile's first flagged step as a minimum over its workgroups
+    int32_t* tg = const_cast<int32_t*>(p.ts_tquads);
+    for (int i = gtid; i < p.ts_desc_tiles; i += gsz) tg[i] = 0x7fffffff;
+  }
   if (tab_out) {
     // every head's bucket table: thresholds and buckets from the host, the table values times log2(e) with
     // bucket indices clipped to the table's last entry (the clip of the bucket law)
@@ -2200,6 +2212,165 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
   }
 }
 
+// ---------------------------------------------------------------------------
+// Timestamp descriptors.  The bucket of a pair depends on the sequence's timestamps alone: not on the head, not
+// on the layer.  With sorted timestamps the buckets of one row fall from key to key, and away from the diagonal
+// a step of 32 keys holds one bucket or two for a row.  This kernel works that out once per batch: for every
+// query row and every 32-key step at or below its diagonal one 16-bit word
+//   bits 0..6   bucket b of the step's last key the row keeps (the nearest in time)
+//   bits 7..12  c: the step's first c keys are one bucket further (b + 1), the others in b (0: one bucket)
+//   bit 15      neither holds (three buckets or more, timestamps out of order in the step, a key later than the
+//               row's own time, buckets past the table): the kernel looks every pair of the block up
+// laid out [step][row] (ts_desc_pitch rows per step; a sequence's rows start at ts_desc_row0), so that the 32
+// rows of a wave are 64 contiguous bytes per step.  Rows past the sequence get 0.  The main kernel's blocks then
+// read one word per lane instead of testing the tile's time range against the bucket thresholds, and the steps
+// before a tile's first flagged one can run as the hand-scheduled stream (ts_tquads: how many quads of them).
+// One workgroup per 128-row tile; the tile's part of the sequence's timestamps sits in LDS.
+// ---------------------------------------------------------------------------
+constexpr int TS_DESC_MAX_L = 16384;      // longest sequence descriptors are built for (table size)
+constexpr uint32_t TS_DESC_GENERAL = 0x8000u;
+__device__ __host__ __forceinline__ int64_t ts_desc_row0(int jagged, int L, int b, int64_t tok0) {
+  return jagged ? 8 * ((tok0 >> 3) + b) : (int64_t)b * ((L + 7) & ~7);
+}
+__device__ __host__ __forceinline__ int64_t ts_desc_tile0(int jagged, int n_qtiles, int b, int64_t tok0) {
+  return jagged ? (tok0 >> 7) + b : (int64_t)b * n_qtiles;
+}
+
+constexpr int TS_DESC_CHUNK = 8;          // steps per workgroup of the descriptor kernel
+__global__ __launch_bounds__(256) void hstu_prepare_ts_desc(const Params p, uint16_t* __restrict__ desc, int32_t* __restrict__ tgen,
+                                                           int n_chunks, const TsKeys keys) {
+  // One workgroup per (128-row tile, chunk of 32 steps): the rows' own times and the chunk's 1024 key timestamps in LDS.
+  // tgen[tile] (set to INT32_MAX by hstu_prepare beforehand) ends up as the tile's first flagged step.
+  __shared__ int64_t tq_l[BM], k_l[TS_DESC_CHUNK * BN];
+  __shared__ float thr_f[TS_KEYS];
+  __shared__ int32_t thr_b[TS_KEYS];
+  __shared__ unsigned char bkt[TS_KEYS];
+  __shared__ int sorted_to[TS_DESC_CHUNK];
+  const int tid = threadIdx.x;
+  const int64_t slot = blockIdx.x / n_chunks;
+  const int chunk = blockIdx.x - (int)slot * n_chunks;
+  int b, qt;
+  Seq s;
+  bool have_seq = false;
+  if (p.sched) {
+    // from the work list that hstu_prepare has just built: one entry per (sequence, tile, key chunk), with the
+    // sequence's first token and length in it (no second trip to memory for the offsets)
+    const int4 item = ((const int4*)(p.sched + 4))[slot < p.items_max ? slot : 0];
+    if (slot >= p.sched[0]) return;
+    if (((item.y >> 16) & 0xff) != 0) return;       // a split tile's later chunks: the first one's workgroups do the tile
+    b = item.x & 0x3fff;
+    qt = item.y & 0xffff;
+    s = seq_from(p, b, 0, item.z, item.w);
+    have_seq = true;
+  } else if (p.jagged) {
+    int lo = 0, hi = p.B;            // the last b with tile0(b) <= slot
+    while (hi - lo > 1) {
+      const int mid = (lo + hi) >> 1;
+      if (ts_desc_tile0(1, 0, mid, p.seq_offsets[mid]) <= slot) lo = mid; else hi = mid;
+    }
+    b = lo;
+    qt = (int)(slot - ts_desc_tile0(1, 0, b, p.seq_offsets[b]));
+  } else {
+    b = (int)(slot / p.n_qtiles);
+    qt = (int)(slot - (int64_t)b * p.n_qtiles);
+  }
+  if (b >= p.B) return;
+  if (!have_seq) s = seq_info(p, b, 0);
+  const int q0 = qt * BM;
+  if (q0 >= s.rows) return;
+  const int n_steps_tile = (((q0 + BM < s.n_kv ? q0 + BM : s.n_kv) + BN - 1) / BN);   // steps a causal tile can touch
+  const int t0 = chunk * TS_DESC_CHUNK;
+  if (t0 >= n_steps_tile) return;
+  const int t1 = t0 + TS_DESC_CHUNK < n_steps_tile ? t0 + TS_DESC_CHUNK : n_steps_tile;
+  const int64_t row0 = ts_desc_row0(p.jagged, p.L, b, s.tok0);
+  // (the next sequence's first token: this one's plus its stored rows)
+  const int64_t row_end = b + 1 < p.B ? ts_desc_row0(p.jagged, p.L, b + 1, p.jagged ? s.tok0 + s.rows : 0) : (int64_t)p.ts_desc_pitch;
+  const int n_ts = s.n_ts;
+  const int64_t* tsg = p.ts + s.ts0;
+  if (tid < BM) {
+    // the time a row takes: that of the next row (its own for the last)
+    int iq = q0 + tid + 1;
+    iq = iq < n_ts ? iq : n_ts - 1;
+    tq_l[tid] = tsg[iq < 0 ? 0 : iq];
+  }
+#pragma unroll
+  for (int e = 0; e < TS_DESC_CHUNK * BN / 256; ++e) {
+    int j = t0 * BN + e * 256 + tid;
+    j = j < n_ts ? j : n_ts - 1;
+    k_l[e * 256 + tid] = (t0 * BN + e * 256 < (t1 * BN)) ? tsg[j < 0 ? 0 : j] : 0;
+  }
+  if (tid < TS_KEYS) {
+    thr_f[tid] = keys.thr_f[tid];
+    thr_b[tid] = tid <= p.ts_nb ? keys.thr_b[tid] : 0x7fffffff;
+    bkt[tid] = keys.bkt[tid];
+  }
+  __syncthreads();
+  {
+    // up to which key of a step the timestamps are in order: every thread compares one neighbouring pair, a
+    // wave's ballot covers two steps
+    static_assert(TS_DESC_CHUNK * BN == 256, "one key per thread");
+    const int l32 = tid & 31;
+    const int j_last = (n_ts - 1) - t0 * BN;                 // the last timestamp there is, as an index into k_l
+    const bool breaks = l32 < BN - 1 && tid + 1 <= j_last && k_l[tid + 1] < k_l[tid];
+    const uint64_t mask = __builtin_amdgcn_ballot_w64(breaks);
+    if (l32 == 0) {
+      const uint32_t mine = (uint32_t)(mask >> (tid & 32));
+      int e = mine ? __builtin_ctz(mine) : BN - 1;           // the step is in order up to its key e
+      e = tid + e < j_last ? tid + e : j_last;
+      sorted_to[tid >> 5] = e;
+    }
+  }
+  __syncthreads();
+  auto bucket = [&](int64_t d) {       // the bucket law on a difference >= 0, clipped to the table
+    const int dc = d < 1 ? 1 : (d < TS_DT_MAX ? (int)d : TS_DT_MAX);
+    const float f = (float)dc;
+    const uint32_t key = (__builtin_bit_cast(uint32_t, f) >> 21) - (uint32_t)TS_KEY0;
+    const int bk = (int)bkt[key] + (f >= thr_f[key] ? 1 : 0);
+    return bk < p.ts_nb ? bk : p.ts_nb;
+  };
+  int my_general = 0x7fffffff;
+  for (int idx = tid; idx < BM * (t1 - t0); idx += 256) {
+    const int r = idx & (BM - 1), tl = idx >> 7, t = t0 + tl;
+    const int i = q0 + r;
+    uint32_t word = 0u;
+    const int j0 = t * BN;
+    int j1 = j0 + BN - 1;
+    j1 = j1 < s.n_kv - 1 ? j1 : s.n_kv - 1;
+    j1 = j1 < i ? j1 : i;                // (the causal mask: later keys are masked whatever their bucket)
+    if (i < s.n_q && j1 >= j0) {
+      const int l0 = tl * BN, l1 = j1 - t0 * BN;     // the step's first key and the row's last, as indices into k_l
+      const int64_t tq = tq_l[r];
+      const int64_t k_first = k_l[l0], k_last = k_l[l1];
+      bool general = sorted_to[tl] < l1 || tq < k_last;
+      if (!general) {
+        const int bn = bucket(tq - k_last), bf = bucket(tq - k_first);
+        if (bf == bn && bn < TS_KEYS) {
+          word = (uint32_t)bn;
+        } else if (bf == bn + 1 && bf < TS_KEYS) {
+          // keys in order: those with tq - ts >= thr, i.e. ts <= tq - thr, are the first c of the step
+          const int64_t cut = tq - (int64_t)thr_b[bf];
+          int lo = l0, hi = l1;        // k[lo] <= cut < k[hi]: the first and last key are on different sides
+          while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (k_l[mid] <= cut) lo = mid; else hi = mid;
+          }
+          word = (uint32_t)bn | ((uint32_t)(lo + 1 - l0) << 7);
+        } else {
+          general = true;
+        }
+      }
+      if (general) {
+        word = TS_DESC_GENERAL;
+        my_general = t < my_general ? t : my_general;
+      }
+    }
+    // (a tile's last rows may lie past the sequence: those up to the next sequence's first row are this
+    // workgroup's to clear, the rest are that sequence's own)
+    if (row0 + i < row_end) desc[(int64_t)t * p.ts_desc_pitch + row0 + i] = (uint16_t)word;
+  }
+  if (my_general != 0x7fffffff) atomicMin(&tgen[ts_desc_tile0(p.jagged, p.n_qtiles, b, s.tok0) + qt], my_general);
+}
+
 // SEG: segment ids (padded layout, L a multiple of 4): a pair is kept when its row's and its key's
 // ids are equal.  The step's 32 key ids arrive by one more direct load per wave and every block
 // compares them with the lane's row id.
@@ -2219,6 +2390,8 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
 // registers allow two workgroups whatever the ring, and the depth makes no measurable difference.
 constexpr int fwd_stages(int d, int dense) { return (d <= 64 || dense != 0) ? 3 : 4; }
 constexpr int FWD_XCH_BYTES = 16;     // behind everything else in the forward kernel's LDS
+// which instances of the forward kernel are laid out for timestamp descriptors (64 bytes per wave and ring stage)
+constexpr bool fwd_takes_ts_desc(int d, bool ts, bool f8, bool seg, int dense) { return ts && d == 128 && !f8 && !seg && dense == 0; }
 
 #include "hstu_fwd_stream_d128.inc"   // (the variants' names; the statements are expanded inside the kernel)
 
@@ -2253,9 +2426,15 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG);
+  // TSD: the kernel can take timestamp descriptors (hstu_prepare_ts_desc).  The bias operands of a stage are then
+  // [4 x (window copy w | the 32 descriptors of wave w's rows)][key timestamps]: each wave's one bias load brings
+  // its window copy and, in the four lanes behind it, its own rows' descriptors.
+  constexpr bool TSD = fwd_takes_ts_desc(D, TS, F8, SEG, DENSE);
+  constexpr int DESC_WAVE = 64;                                      // 32 descriptors of 2 bytes
+  constexpr int CS = TSD ? (POS ? SM::POS_COPY : 0) + DESC_WAVE : SM::POS_COPY;   // from one wave's copy to the next
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG) + (TSD ? NWAVES * DESC_WAVE : 0);
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
-  auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
+  auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (TSD ? NWAVES * CS : (POS ? SM::POS_BYTES : 0))); };
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   constexpr int DENSE_OFF = BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0);
@@ -2289,7 +2468,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       return p;
     }
   };
-  struct DmaCtx { const char* kg; const bf16_t* vg; int n_kv, n_ts, q0, b; uint32_t pos_off, rel_off, rng_off; };
+  struct DmaCtx { const char* kg; const bf16_t* vg; int n_kv, n_ts, q0, b; uint32_t pos_off, rel_off, rng_off, desc_off; };
   // Bias operands are fetched with 32-bit byte offsets from the start of the workspace.
   // pos_off: the head's padded table; entry x of the unpadded table sits at float POS_PAD + x.
   auto ctx_of = [&](const Work& k) {
@@ -2301,6 +2480,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     c.pos_off = POS ? (uint32_t)((const char*)(pf.pos_scaled + (int64_t)(pf.pos_heads > 1 ? k.h : 0) * (2 * pf.L - 1 + 2 * POS_PAD)) - wsb) : 0u;
     c.rel_off = TS ? (uint32_t)((const char*)(pf.ts_rel + ts_rel_base(pf, k.b, k.s.tok0)) - wsb) : 0u;
     c.rng_off = TS ? (uint32_t)((const char*)(pf.ts_range + 2 * ts_range_slot0(pf, k.b, k.s.tok0)) - wsb) : 0u;
+    // (descriptor of row i at step t: entry t * pitch + i from here; 0 = no descriptors)
+    c.desc_off = (TSD && pf.ts_desc) ? (uint32_t)((const char*)(pf.ts_desc + ts_desc_row0(pf.jagged, pf.L, k.b, k.s.tok0)) - wsb) : 0u;
     if constexpr (PERSIST) {
       // (the same for every lane, and the direct loads want them in scalar registers: said outright, the
       // compiler otherwise moves the arithmetic of an item drawn at run time to the vector unit)
@@ -2342,6 +2523,39 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // issues the same number of loads per step: the vmcnt arithmetic relies on it.
   // The ring stage is a compile-time constant everywhere (the step loop is unrolled over the ring):
   // LDS addresses are then a per-lane register plus an immediate, with no address arithmetic per step.
+  // What a lane of the step's one bias load per wave fetches: byte offset from the workspace base, and whether the
+  // lane takes part.  Wave c writes position-window copy c: window[x + c], window[x] = pos[(L-1) + kv0 - (q0+127) + x];
+  // the table index is >= POS_PAD - 127 > 0 and inside the padded table (the offset register is unsigned: a negative
+  // index would address 4 GB past the base).  With descriptors the four lanes behind the window bring the wave's own
+  // 32 rows of the step's descriptors.  The lanes behind those on the last wave (or the first lanes of every wave
+  // when there is neither window nor descriptors) bring 32 int32 key timestamps, 4 per lane, and the tile's (min, max).
+  // Keys past the sequence read whatever follows in the workspace: their logits are masked.
+  auto bias_lane = [&](const DmaCtx& c_, int t, bool& on, int lane) -> uint32_t {
+    constexpr int DESC_LANE0 = POS ? SM::POS_LANES : 0;
+    constexpr int TS_LANE0 = DESC_LANE0 + (TSD ? DESC_WAVE / 16 : 0);
+    const int kv0 = t * BN;
+    const bool ts_wave = TS && ((!POS && !TSD) || w == NWAVES - 1);
+    const int tl = lane - TS_LANE0;
+    uint32_t off = 0;
+    on = false;
+    if (POS && lane < SM::POS_LANES) {
+      off = c_.pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (c_.q0 + BM - 1) + w + 4 * lane) * 4u;
+      on = true;
+    }
+    if (TSD && c_.desc_off != 0u && lane >= DESC_LANE0 && lane < TS_LANE0) {
+      // the wave's own 32 rows of the step's descriptors: 8 rows per lane
+      off = c_.desc_off + ((uint32_t)t * (uint32_t)p.ts_desc_pitch + (uint32_t)(c_.q0 + 32 * w + 8 * (lane - DESC_LANE0))) * 2u;
+      on = true;
+    }
+    if (ts_wave && tl >= 0 && tl < SM::TK_LANES) {
+      int tr = t;                                  // tiles past the last timestamp repeat the last tile's range
+      const int tr_last = (c_.n_ts - 1) >> 5;
+      tr = tr < tr_last ? tr : tr_last;
+      off = tl < BN / 4 ? c_.rel_off + (uint32_t)(kv0 + 4 * tl) * 4u : c_.rng_off + (uint32_t)tr * 8u;
+      on = true;
+    }
+    return off;
+  };
   // `part_`: 3 = the whole step, 1 = its K tile and bias operands only, 2 = its V tile only (the hand-scheduled
   // stream of the interior steps keeps the K side of the ring one step ahead of the V side).
   auto dma_part = [&](const DmaCtx& c_, int t, auto st_, auto part_) {
@@ -2374,30 +2588,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     }
     }
     if ((POS || TS) && (part & 1) != 0) {
-      // One more load per wave brings the bias operands.  Wave c writes position-window copy c:
-      // window[x + c], window[x] = pos[(L-1) + kv0 - (q0+127) + x]; the table index is
-      // >= POS_PAD - 127 > 0 and inside the padded table (the offset register is unsigned: a
-      // negative index would address 4 GB past the base).  The lanes behind the last wave's copy
-      // (or the first lanes of every wave when there is no position bias) bring 32 int32 key
-      // timestamps, 4 per lane, and the tile's (min, max).  Keys past the sequence read whatever
-      // follows in the workspace: their logits are masked.
-      constexpr int TS_LANE0 = POS ? SM::POS_LANES : 0;
-      const bool ts_wave = TS && (!POS || w == NWAVES - 1);
-      const int tl = lane - TS_LANE0;
-      uint32_t off = 0;
-      bool on = false;
-      if (POS && lane < SM::POS_LANES) {
-        off = c_.pos_off + (uint32_t)(POS_PAD + (p.L - 1) + kv0 - (c_.q0 + BM - 1) + w + 4 * lane) * 4u;
-        on = true;
-      }
-      if (ts_wave && tl >= 0 && tl < SM::TK_LANES) {
-        int tr = t;                                  // tiles past the last timestamp repeat the last tile's range
-        const int tr_last = (c_.n_ts - 1) >> 5;
-        tr = tr < tr_last ? tr : tr_last;
-        off = tl < BN / 4 ? c_.rel_off + (uint32_t)(kv0 + 4 * tl) * 4u : c_.rng_off + (uint32_t)tr * 8u;
-        on = true;
-      }
-      if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + (POS ? w * SM::POS_COPY : 0));
+      // one more load per wave brings the bias operands (bias_lane)
+      bool on;
+      const uint32_t off = bias_lane(c_, t, on, lane);
+      if (on) lds_dma16(wsb, off, (const unsigned char*)Wc(st) + ((POS || TSD) ? w * CS : 0));
     }
     if (SEG && (part & 1) != 0) {
       // every wave brings the same 32 ids (each wave must issue the same number of loads); groups of 4
@@ -2469,6 +2663,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   DmaCtx cx;
   struct { int n_q, n_kv, rows, n_ts; } s;       // of the item's sequence
   int h = 0, q0 = 0, r0 = 0, qrow = 0, wave_last = -1, nt = 0, t_lo = 0, n_chunks = 1, chunk = 0, pslot = 0, ts32 = 0;
+  int has_desc = 0, desc_quads = 0;         // descriptors at hand; leading quads of steps none of whose rows is flagged
   float alpha2 = 0.f;
   const int64_t* tsg = nullptr;
   bf16_t* og = nullptr;
@@ -2489,6 +2684,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     tsg = TS ? pf.ts + k.s.ts0 : nullptr;
     // whether the sequence's int32 timestamps are valid (its time span allows them)
     ts32 = TS ? pf.ts_ok[k.b] : 0;
+    if constexpr (TSD) {
+      has_desc = pf.ts_desc != nullptr;
+      desc_quads = has_desc ? (pf.ts_tquads[ts_desc_tile0(pf.jagged, pf.n_qtiles, k.b, k.s.tok0) + k.qt] >> 2) : 0;
+    }
     og = (bf16_t*)pf.out + k.s.bo;
   };
   // the head's bucket table: three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
@@ -2604,7 +2803,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     if (POS) {
       const int xb = 4 * hh + (BM - 1) - 32 * w - m;
       const int sft = xb & 3;
-      const float* wrow = (const float*)((const unsigned char*)Wc(st) + sft * SM::POS_COPY) + (xb - sft);
+      const float* wrow = (const float*)((const unsigned char*)Wc(st) + sft * CS) + (xb - sft);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         float4 bv = *(const float4*)(wrow + 8 * g);
@@ -2616,6 +2815,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     } else {
 #pragma unroll
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
+      if constexpr (TSD) {
+        // (the product rounded by itself, as the hand-scheduled stream has it: the compiler would otherwise fuse it
+        // with the timestamp bias's addition below, and the two paths would differ in the last bit)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) asm volatile("" : "+v"(u[r]));
+      }
     }
     if (TS) {
       if (ts32) {
@@ -2875,8 +3080,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       }
     }
   };
-  // ---- The interior steps as one hand-scheduled instruction stream (d = 128 in bf16, no timestamps, segment ids
-  // or dense operands; hstu_fwd_stream_d128.inc, written by gen_fwd_stream.py).  A step is interior when every key
+  // ---- The interior steps as one hand-scheduled instruction stream (d = 128 in bf16, no segment ids or dense
+  // operands; hstu_fwd_stream_d128.inc, written by gen_fwd_stream.py).  With timestamps it takes each (row, step)'s
+  // bias from the descriptors that hstu_prepare_ts_desc wrote (the bucket of the step's nearest key and how many of
+  // its keys are one bucket further), and only the leading steps in which no row of the tile is flagged.  A step is interior when every key
   // of it is kept for every row of the tile: under the causal mask the steps below the tile's first row, without
   // it those that lie whole inside the sequence.  The stream takes them four at a time from the item's first step
   // on (ring stage 0), software-pipelined across steps, with the K side of the ring one step ahead of the V side.
@@ -2886,7 +3093,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   // over where the stream stops.  The stream's last pair asks for K tiles up to two steps past its end and for V
   // tiles up to one: those steps must exist and lie whole inside the sequence (no row to clamp).  The arithmetic
   // and its order are those of `block`: the same bits either way.
-  constexpr bool STREAM = D == 128 && !TS && !F8 && !SEG && DENSE == 0 && PAIRS;
+  // (Not in the resident-workgroup instances with timestamps: what those keep across their loop over items and
+  // what the stream clobbers do not fit the register file together, and the compiler's spills cost the block code
+  // more than the stream gains.  Calls with timestamp descriptors take one workgroup per item instead.)
+  constexpr bool STREAM = D == 128 && !F8 && !SEG && DENSE == 0 && PAIRS && !(TS && PERSIST);
   auto stream_quads = [&]() -> int {
     if constexpr (!STREAM) return 0;
     const Params pf = fresh();
@@ -2895,6 +3105,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     if (pf.causal) keys = q0 < keys ? q0 : keys;
     const int t_int = keys / BN;                 // steps [0, t_int) are interior for all four waves
     int n = (t_int - t_lo) >> 2;
+    if constexpr (TS) {
+      // with timestamps: only on descriptors, and only the leading steps in which no row of the tile is flagged
+      if (!ts32 || !has_desc) return 0;
+      const int nd = desc_quads - (t_lo >> 2);
+      n = (t_lo & 3) != 0 ? 0 : (n < nd ? n : nd);
+    }
     // lookahead: steps up to t_lo + 4n + 2 exist and are whole
     const int whole = s.n_kv / BN;
     while (n > 0 && !(t_lo + 4 * n + 2 < nt && t_lo + 4 * n + 3 <= whole)) --n;
@@ -2902,6 +3118,14 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   };
   auto run_stream = [&](int n_quads) {
     if constexpr (STREAM) {
+      // (the lane's index enters through a register the compiler cannot see through: it would otherwise work the
+      // lane's share of the stream's two dozen addresses out once, ahead of the loop over items, and keep them in
+      // registers the block code needs)
+      int tid_ = tid;
+      asm volatile("" : "+v"(tid_));
+      const int lane = tid_ & 63, m = lane & 31, hh = lane >> 5;
+      const int gk = SM::swz_k(m), gi = lane & 15, vrow = 4 * hh + (gi >> 2), gq = SM::swz_v(vrow) >> 2;
+      const int vc2 = 2 * ((lane >> 4) & 1) + ((gi & 3) >> 1);
       typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
       uintx4 hs_q[8];
 #pragma unroll
@@ -2912,7 +3136,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 #pragma unroll
       for (int d = 0; d < 4; ++d) hs_va[d] = smem_lds + (uint32_t)(SM::K_BYTES + vrow * 256 + 8 * (gi & 1) + vc2 * 16 + ((d ^ gq) & 3) * 64);
       const int xb = 4 * hh + (BM - 1) - 32 * w - m, sft = xb & 3;
-      const uint32_t hs_pa = smem_lds + (uint32_t)(BIAS_OFF + sft * SM::POS_COPY + (xb - sft) * 4);
+      const uint32_t hs_pa = smem_lds + (uint32_t)(BIAS_OFF + sft * CS + (xb - sft) * 4);
       uint32_t hs_koff[2], hs_voff[2];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
@@ -2925,15 +3149,38 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       const uint32_t hs_kstep = (uint32_t)BN * kst_bytes, hs_vstep = (uint32_t)BN * vst_bytes;
       const char* hs_kp = cx.kg + (size_t)(t_lo + 2) * hs_kstep;
       const char* hs_vp = (const char*)cx.vg + (size_t)(t_lo + 2) * hs_vstep;
-      const uint32_t hs_bdst = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(BIAS_OFF + w * SM::POS_COPY));
-      const uint32_t hs_boff = (uint32_t)(w + 4 * lane) * 4u;
-      const uint64_t hs_bexec = (1ull << SM::POS_LANES) - 1ull;
+      const uint32_t hs_bdst = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(BIAS_OFF + w * CS));
+      // the bias load: without timestamps one scalar pointer walks along the table, 128 bytes a step; with them
+      // window, descriptors and key timestamps move on by different strides, so each lane's offset from the
+      // workspace base takes a per-lane step (the differences of two steps' offsets)
+      uint32_t hs_boff = (uint32_t)(w + 4 * lane) * 4u, hs_binc = 0u;
+      uint64_t hs_bexec = (1ull << SM::POS_LANES) - 1ull;
       // the window of step t starts at table entry POS_PAD + (L - 1) + 32 t - (q0 + 127) of the head's padded table
       const char* hs_bp = wsb + cx.pos_off + (int64_t)(POS_PAD + (fresh().L - 1) + BN * (t_lo + 2) - (q0 + BM - 1)) * 4;
+      uint32_t hs_dsa = 0u, hs_hh4 = 0u, hs_tva = 0u;
+      if constexpr (TS) {
+        bool on2, on3;
+        const uint32_t o2 = bias_lane(cx, t_lo + 2, on2, lane), o3 = bias_lane(cx, t_lo + 3, on3, lane);
+        hs_boff = o2;
+        hs_binc = o3 - o2;
+        hs_bexec = __builtin_amdgcn_ballot_w64(on2);
+        hs_bp = wsb;
+        hs_dsa = smem_lds + (uint32_t)(BIAS_OFF + w * CS + (POS ? SM::POS_COPY : 0) + 2 * m);
+        hs_hh4 = (uint32_t)(4 * hh);
+        hs_tva = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(BIAS_OFF + NSTAGE * BIAS_STAGE + TS_VAL_OFF));
+      }
       const float hs_alpha = alpha2;
       int hs_n = n_quads;
       floatx16 (&hs_o)[DVB] = o;
-      if constexpr (POS) {
+      if constexpr (POS && TS) {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_FULL_POS_TS
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+      } else if constexpr (TS) {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_FULL_TS
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+      } else if constexpr (POS) {
 #define HSTU_STREAM_VARIANT HSTU_STREAM_FULL_POS
 #include "hstu_fwd_stream_d128.inc"
 #undef HSTU_STREAM_VARIANT
@@ -2941,8 +3188,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
 #define HSTU_STREAM_VARIANT HSTU_STREAM_FULL
 #include "hstu_fwd_stream_d128.inc"
 #undef HSTU_STREAM_VARIANT
-        (void)hs_pa; (void)hs_bdst; (void)hs_boff; (void)hs_bexec; (void)hs_bp;
       }
+      (void)hs_pa; (void)hs_bdst; (void)hs_boff; (void)hs_binc; (void)hs_bexec; (void)hs_bp; (void)hs_dsa; (void)hs_hh4; (void)hs_tva;
     }
   };
   if constexpr (!PERSIST) {
@@ -4351,7 +4598,9 @@ struct WorkspacePlan {
   size_t pos_bytes, tab_bytes, ok_bytes, rel_bytes, range_bytes, mrange_bytes, sched_bytes, ctr_bytes, partial_bytes;
   int split_cap;          // chunk slots of the partial buffer (0: no tile is split)
   long long items_max;    // capacity of the work list (0 = no list)
-  size_t bias_total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes + mrange_bytes; }
+  size_t desc_bytes, tquad_bytes;   // timestamp descriptors and the tiles' stream quads (forward, d = 128; 0 = none)
+  long long desc_pitch, desc_tiles; // rows per step of the descriptor table, tile slots
+  size_t bias_total() const { return pos_bytes + tab_bytes + ok_bytes + rel_bytes + range_bytes + mrange_bytes + desc_bytes + tquad_bytes; }
   size_t total() const { return bias_total() + sched_bytes + ctr_bytes + partial_bytes; }
 };
 
@@ -4361,8 +4610,8 @@ struct WorkspacePlan {
 constexpr int SPLIT_CAP_DEFAULT = 32;
 
 // max_bytes: a workspace this small must do (the split capacity is cut down to fit it).
-WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, size_t max_bytes = ~(size_t)0) {
-  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, size_t max_bytes = ~(size_t)0, bool want_desc = true) {
+  WorkspacePlan w = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const Variant var = pick_variant(a);
   if (var != V_MFMA_BF16 && var != V_MFMA_FP8) return w;
   auto up = [](size_t x) { return (x + 255) / 256 * 256; };
@@ -4390,6 +4639,20 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, 
     w.range_bytes = up(tiles * 2 * sizeof(int32_t) + 16);
   }
   if (a->mask) w.mrange_bytes = up((size_t)(a->mask_batched ? a->B : 1) * (size_t)n_qtiles * 2 * sizeof(int32_t));
+  // Timestamp descriptors: the forward at d = 128 in bf16 under the causal mask with lengths (what the descriptor
+  // kernel's LDS holds; tables small enough to be worth their memory), when the caller's workspace has the room.
+  if (want_desc && a->ts_tab && var == V_MFMA_BF16 && a->d_qk == 128 && a->causal && effective_window(a) < 0 && a->L == a->Lkv &&
+      a->L <= TS_DESC_MAX_L && !a->mask && !a->dense_bias && (jag || a->mask_mode != HSTU_MASK_SEGMENT)) {
+    const long long rows = jag ? 8 * ((a->total_tokens >> 3) + a->B) + BM : (long long)a->B * ((a->L + 7) & ~7) + BM;
+    const long long steps = (a->L + BN - 1) / BN;
+    const size_t bytes = up((size_t)rows * (size_t)steps * sizeof(uint16_t));
+    if (bytes <= ((size_t)256 << 20)) {
+      w.desc_pitch = rows;
+      w.desc_tiles = jag ? (a->total_tokens >> 7) + a->B + 1 : (long long)a->B * n_qtiles;
+      w.desc_bytes = bytes;
+      w.tquad_bytes = up((size_t)w.desc_tiles * sizeof(int32_t));
+    }
+  }
   const long long t128 = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
   const size_t chunk_bytes = (size_t)a->H * (size_t)BM * (size_t)a->d_v * sizeof(float);
   for (;;) {
@@ -4399,7 +4662,13 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, 
     }
     w.ctr_bytes = list ? up((size_t)(CTR_RESERVED + (size_t)w.split_cap * a->H) * sizeof(uint32_t)) : 0;
     w.partial_bytes = up((size_t)w.split_cap * chunk_bytes);
-    if (w.total() <= max_bytes || w.split_cap == 0) break;
+    if (w.total() <= max_bytes) break;
+    if (w.split_cap == 0) {
+      // still too large without any chunk slot: the descriptors go (every block then looks its pairs up)
+      if (!w.desc_bytes) break;
+      w.desc_bytes = w.tquad_bytes = 0; w.desc_pitch = w.desc_tiles = 0;
+      continue;
+    }
     const size_t over = w.total() - max_bytes;
     const int fewer = (int)((over + chunk_bytes - 1) / chunk_bytes);
     w.split_cap = w.split_cap - fewer >= 2 ? w.split_cap - fewer : 0;
@@ -4601,7 +4870,8 @@ int launch_bwd(const Params& p, hipStream_t st) {
 
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0, bool PERSIST = false>
 int launch_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE, fwd_stages(D, DENSE)) + FWD_XCH_BYTES;
+  const int smem = MfmaSmem<D, F8 ? 1 : 2>::total(POS, TS, SEG, DENSE, fwd_stages(D, DENSE)) + FWD_XCH_BYTES +
+                   (fwd_takes_ts_desc(D, TS, F8, SEG, DENSE) ? fwd_stages(D, DENSE) * NWAVES * 64 : 0);
   static int granted[64];
   if (int rc = allow_lds((const void*)hstu_fwd_mfma_bf16<D, POS, TS, F8, SEG, DENSE, PERSIST>, smem, granted)) return rc;
   hipError_t e;
@@ -4699,6 +4969,12 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   int32_t* mrange_out = ws.mrange_bytes ? (int32_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes + ws.range_bytes) : nullptr;
   q.mask_range = mrange_out;
   q.ws_base = base;
+  uint16_t* desc_out = ws.desc_bytes ? (uint16_t*)(base + ws.pos_bytes + ws.tab_bytes + ws.ok_bytes + ws.rel_bytes + ws.range_bytes + ws.mrange_bytes) : nullptr;
+  int32_t* tquad_out = ws.desc_bytes ? (int32_t*)((char*)desc_out + ws.desc_bytes) : nullptr;
+  q.ts_desc = desc_out;
+  q.ts_tquads = tquad_out;
+  q.ts_desc_pitch = (int32_t)ws.desc_pitch;
+  q.ts_desc_tiles = (int32_t)ws.desc_tiles;
   int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
   q.sched = sched_out;
   q.items_max = ws.items_max;
@@ -4723,6 +4999,13 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
     hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out, mrange_out, keys);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
+    if (desc_out) {
+      const int n_chunks = ((q.L + BN - 1) / BN + TS_DESC_CHUNK - 1) / TS_DESC_CHUNK;
+      const long long slots = q.sched ? q.items_max : ws.desc_tiles;     // by work-list entry, else by tile slot
+      hipLaunchKernelGGL(hstu_prepare_ts_desc, dim3((unsigned)(slots * n_chunks)), dim3(256), 0, st, q, desc_out, tquad_out, n_chunks, keys);
+      e = hipGetLastError();
+      if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "descriptor kernel launch: %s", hipGetErrorString(e));
+    }
   }
   return HSTU_OK;
 }
@@ -4738,7 +5021,7 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
       f.q_stride_t <= 0 || f.o_stride_t <= 0) return false;
-  const WorkspacePlan ws = plan_workspace(&f, false);
+  const WorkspacePlan ws = plan_workspace(&f, false, ~(size_t)0, false);
   return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
 }
 
@@ -4780,7 +5063,7 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
   f.flags &= ~HSTU_FWD_WORKSPACE_PREPARED;   // the backward lays the work list out without key-range splits
-  const WorkspacePlan ws = plan_workspace(&f, false);
+  const WorkspacePlan ws = plan_workspace(&f, false, ~(size_t)0, false);
   Params q = p;
   if (int rc = setup_workspace(&f, ws, q, st)) return rc;
   if (q.d_qk == 128) return launch_bwd_mfma_d<128>(q, st);
@@ -4939,8 +5222,10 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
       const long long tiles = q.jagged ? args->total_tokens / BM + args->B : (long long)args->B * q.n_qtiles;
       const long long jobs_per_xcd = q.H >= 8 ? tiles * (q.H >> 3) : tiles / (8 / q.H);
       q.no_stream = (args->flags & HSTU_FWD_COMPILER_SCHEDULED_BLOCKS) ? 1 : 0;
+      // (with timestamp descriptors the interior steps run as the hand-scheduled stream, which the resident instances
+      // with timestamps do not have: one workgroup per item there)
       q.persist = can_stay && !(args->flags & HSTU_FWD_ONE_ITEM_PER_WORKGROUP) &&
-                  ((args->flags & HSTU_FWD_RESIDENT_WORKGROUPS) || (count_known && jobs_per_xcd >= 8LL * q.n_slots));
+                  ((args->flags & HSTU_FWD_RESIDENT_WORKGROUPS) || (count_known && jobs_per_xcd >= 8LL * q.n_slots && !q.ts_desc));
       if (int rc2 = f8 ? launch_mfma<true>(q, st) : launch_mfma<false>(q, st)) return rc2;
       return HSTU_OK;
     }

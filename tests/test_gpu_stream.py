@@ -1,7 +1,10 @@
 """The hand-scheduled instruction stream of the forward kernel's interior steps (d = 128, bf16): the same
 arithmetic in the same order as the compiler-scheduled block code, so a call with
 HSTU_FWD_COMPILER_SCHEDULED_BLOCKS must give the same bits, for both ways through the work list; and the
-stream itself against the oracle on shapes where nearly every step is an interior one."""
+stream itself against the oracle on shapes where nearly every step is an interior one.  With a timestamp
+bias the stream reads the per-(row, step) descriptors that a kernel of their own builds once per batch
+(bucket of the nearest key, how many of the step's keys are one bucket further): timestamps a second and a
+million seconds apart, out of order, and spans beyond 31 bits against the oracle as well."""
 
 import numpy as np
 import pytest
@@ -73,6 +76,68 @@ def test_stream_gives_the_bits_of_the_block_code(gpu, walk, name, lens, L, H, po
   got = _run(q, k, v, mode, **kw)
   assert not torch.isnan(got.float()).any()
   assert torch.equal(ref.view(torch.int16), got.view(torch.int16))
+
+
+TS_CASES = [
+    # name, lengths, L, H, position table
+    ("one long sequence, timestamps", [2048], 2048, 8, False),
+    ("one long sequence, table + timestamps", [2048], 2048, 8, True),
+    ("mixed lengths, table + timestamps", [2048, 1655, 1000, 777, 513, 512, 511, 385, 384, 256, 129, 128, 127, 16, 1], 2048, 8, True),
+    ("two long sequences (tiles split by keys), table + timestamps", [2048, 2048], 2048, 8, True),
+    ("three sequences, two heads", [2048, 1300, 700], 2048, 2, True),
+]
+
+
+@pytest.mark.parametrize("name,lens,L,H,pos", TS_CASES, ids=[c[0] for c in TS_CASES])
+@pytest.mark.parametrize("walk", ["one item per workgroup", "resident workgroups"])
+def test_stream_with_timestamps_gives_the_bits_of_the_block_code(gpu, walk, name, lens, L, H, pos):
+  q, k, v, kw = _inputs(lens, L, H, pos, True, True, timestamps=True)
+  mode = _lib.FWD_ONE_ITEM_PER_WORKGROUP if walk == "one item per workgroup" else _lib.FWD_RESIDENT_WORKGROUPS
+  for _ in range(2):      # (twice: a race between the workgroups that write the descriptors would not show every time)
+    ref = _run(q, k, v, mode | _lib.FWD_COMPILER_SCHEDULED_BLOCKS, **kw)
+    got = _run(q, k, v, mode, **kw)
+    assert not torch.isnan(got.float()).any()
+    assert torch.equal(ref.view(torch.int16), got.view(torch.int16))
+
+
+def _ts_oracle_case(lens, L, H, pos, ts, seed):
+  g = torch.Generator(device="cuda:0").manual_seed(seed)
+  offs = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+  shape = (int(offs[-1]), H, 128)
+  q, k, v = (torch.randn(shape, device="cuda:0", generator=g).mul_(0.3).to(torch.bfloat16) for _ in range(3))
+  ts_tab = torch.randn((H, 129), device="cuda:0", generator=g) * 0.2
+  kw = dict(max_len=L, n=L, causal=True, seq_offsets=torch.from_numpy(offs).to("cuda:0"),
+            timestamps=torch.from_numpy(ts).to("cuda:0"), ts_bias=ts_tab)
+  okw = dict(timestamps=ts, ts_tab=ts_tab.cpu().numpy())
+  if pos:
+    kw["pos_bias"] = torch.randn((H, 2 * L - 1), device="cuda:0", generator=g) * 0.05
+    okw["pos_tab"] = kw["pos_bias"].cpu().numpy()
+  got = _run(q, k, v, 0, **kw).float().cpu().numpy()
+  f = lambda t: t.float().cpu().numpy()
+  ref = O.hstu_attention_jagged_ref(f(q), f(k), f(v), offs, L, n=L, **okw)
+  return np.abs(got - ref).max() / np.abs(ref).max()
+
+
+@pytest.mark.parametrize("mean_dt", [1.0, 3600.0, 1e6])
+@pytest.mark.parametrize("pos", [False, True])
+def test_stream_with_timestamps_against_the_oracle(gpu, mean_dt, pos):
+  rng = np.random.default_rng(int(mean_dt) + pos)
+  lens = np.asarray([1536, 900, 2048], np.int32)
+  ts = np.concatenate([1_600_000_000 + np.cumsum(np.ceil(rng.exponential(mean_dt, n)).astype(np.int64)) for n in lens])
+  assert _ts_oracle_case(lens, 2048, 2, pos, ts, seed=11) <= BF16_TOL
+
+
+def test_timestamps_out_of_order_and_wide_spans_with_descriptors(gpu):
+  # one sequence in order, one shuffled (every step flagged: the per-pair lookup), one with equal timestamps, one
+  # whose span needs more than 31 bits (no 32-bit timestamps: the kernel's 64-bit path, descriptors unused)
+  rng = np.random.default_rng(5)
+  lens = np.asarray([1024, 1024, 700, 640], np.int32)
+  a = 1_600_000_000 + np.cumsum(np.ceil(rng.exponential(3600.0, 1024)).astype(np.int64))
+  b = rng.permutation(a)
+  c = np.full(700, 1_700_000_000, np.int64)
+  d = np.cumsum(rng.integers(1, 2**24, 640).astype(np.int64)) * 1000
+  ts = np.concatenate([a, b, c, d])
+  assert _ts_oracle_case(lens, 1024, 2, True, ts, seed=12) <= BF16_TOL
 
 
 @pytest.mark.parametrize("pos", [False, True])

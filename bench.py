@@ -465,9 +465,12 @@ def bench_dense(args, dev):
   nbytes = 4 * B * L * H * d * 2 + B * L * L * 5
   rec = {
       "metric": "HSTU attn fwd TFLOP/s (kept pairs), dense mask + bias, L=%d %s" % (L, "fp32" if args.fp32 else "bf16"),
-      "value": flops / (ms * 1e-3) / 1e12,
-      "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms,
+      "value": flops / (with_prepare_ms * 1e-3) / 1e12,
+      "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": with_prepare_ms,
+      "timed_call": "hstu_attn_fwd, self-contained: every call runs the preparation kernel (which reads the mask once) and "
+                    "the main kernel.  *_prepared_batch: the batch prepared once, as the layers of a model after the first call it",
       "ms_per_step_with_prepare": with_prepare_ms,
+      "ms_per_step_prepared_batch": ms, "value_prepared_batch": flops / (ms * 1e-3) / 1e12,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32" if args.fp32 else "bf16", "data": "synthetic",
       "config": {"workload": f"A1-dense: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",
                  "kernel": variant},
@@ -712,22 +715,24 @@ def main():
       step()
     torch.cuda.synchronize()
 
-  # Calls that carry their own preparation (work list, 32-bit timestamps, scaled tables: one more kernel).
+  # The timed region: the call as the reference's op is called -- a function of its arguments that does all of
+  # its work every time: the preparation kernel (work list, 32-bit timestamps, scaled tables, timestamp
+  # descriptors) and the main kernel.  Exactly `steps` calls between two synchronisations, nothing else on
+  # the stream.
   for _ in range(args.warmup):
     step()
-  self_contained_ms = timed(step, args.steps)
+  wall = timed(step, args.steps) * 1e-3 * args.steps
   # The preparation alone.
   call_args.flags |= _lib.FWD_PREPARE_ONLY
   prepare_ms = float(evented(step).mean())
   call_args.flags &= ~_lib.FWD_PREPARE_ONLY
 
-  # The timed region: the call as a layer of a model makes it -- the batch was prepared once (above),
-  # every layer's call reuses that.  Exactly `steps` calls between two synchronisations, nothing else
-  # on the stream.
+  # The call as a layer of a model makes it: the batch was prepared once (above), every layer's call reuses
+  # that (lengths, timestamps and tables are the same for all layers).  A secondary figure.
   call_args.flags |= _lib.FWD_WORKSPACE_PREPARED
   for _ in range(args.warmup):
     step()
-  wall = timed(step, args.steps) * 1e-3 * args.steps
+  prepared_ms = timed(step, args.steps)
 
   # the same calls again with a pair of HIP events around each one, on the launch stream: the kernel
   # alone (the roofline figure)
@@ -804,14 +809,19 @@ def main():
                              f"ts_bias={'yes' if w.ts_tab is not None else 'no'} N={w.n} alpha={w.alpha}",
                  "kernel": variant},
       "seqs_per_s": w.B / (ms_per_step * 1e-3),
-      "timed_call": "hstu_attn_fwd on a batch prepared once (HSTU_FWD_WORKSPACE_PREPARED), as every layer of a model "
-                    "calls it; ms_per_step_with_prepare: each call prepares for itself",
-      "ms_per_step_with_prepare": self_contained_ms,
-      "value_with_prepare": flops / (self_contained_ms * 1e-3) / 1e12,
+      "timed_call": "hstu_attn_fwd, self-contained: every call runs the preparation kernel and the main kernel (value, "
+                    "ms_per_step; the same as *_with_prepare).  *_prepared_batch: the batch prepared once "
+                    "(HSTU_FWD_WORKSPACE_PREPARED), as the layers of a model after the first call it",
+      "ms_per_step_with_prepare": ms_per_step,
+      "value_with_prepare": tflops,
+      "ms_per_step_prepared_batch": prepared_ms,
+      "value_prepared_batch": flops / (prepared_ms * 1e-3) / 1e12,
       "api_ms_per_step": api_ms, "api_shared_batch_ms_per_step": api_batch_ms,
       "roofline": {
           "bound": "mfma", "achieved": achieved, "peak": peak,
           "unit": "TFLOP/s", "frac": achieved / peak, "traffic": measured_traffic(args.workload),
+          "traffic_source": "profiles/traffic.json (rocprofv3 --pmc runs of this command, scaled by a copy of known size)"
+                            if measured_traffic(args.workload) is not None else None,
           "kernel": variant, "kernel_ms_avg": kernel_ms, "kernel_ms_min": float(main_ms.min()),
           "kernel_ms_median": float(np.median(main_ms)),
           "step_ms_avg": step_ms, "step_ms_cold_avg": cold_ms,

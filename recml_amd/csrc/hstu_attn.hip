@@ -120,7 +120,8 @@ struct Params {
   const uint16_t* ts_desc;
   const int32_t* ts_tquads;
   int32_t ts_desc_pitch;
-  int32_t ts_desc_tiles;     // entries of ts_tquads
+  int32_t ts_desc_tiles;     // tile slots of ts_tquads
+  int32_t ts_desc_chunks;    // entries per tile slot: chunks of TS_DESC_CHUNK steps
   float* partial;            // [chunk slot][head][BM x d_v floats in register order]
   uint32_t* ctr;             // workspace: [0, 8) draw counters of the XCDs, [8] workgroups done, then from
                              // CTR_RESERVED on one arrival counter per (chunk slot, head); all zero between launches
@@ -1847,6 +1848,171 @@ __device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_
   return p.ts_sb != 0 ? (int64_t)b * ((p.L + BN - 1) / BN) : (tok0 >> 5) + b;
 }
 
+// ---------------------------------------------------------------------------
+// Timestamp descriptors.  The bucket of a pair depends on the sequence's timestamps alone: not on the head, not
+// on the layer.  With sorted timestamps the buckets of one row fall from key to key, and away from the diagonal
+// a step of 32 keys holds one bucket or two for a row.  This kernel works that out once per batch: for every
+// query row and every 32-key step at or below its diagonal one 16-bit word
+//   bits 0..6   bucket b of the step's last key the row keeps (the nearest in time)
+//   bits 7..12  c: the step's first c keys are one bucket further (b + 1), the others in b (0: one bucket)
+//   bit 15      neither holds (three buckets or more, timestamps out of order in the step, a key later than the
+//               row's own time, buckets past the table): the kernel looks every pair of the block up
+// laid out [step][row] (ts_desc_pitch rows per step; a sequence's rows start at ts_desc_row0), so that the 32
+// rows of a wave are 64 contiguous bytes per step.  Rows past the sequence get 0.  The main kernel's blocks then
+// read one word per lane instead of testing the tile's time range against the bucket thresholds, and the steps
+// before a tile's first flagged one can run as the hand-scheduled stream (ts_tquads: per tile and chunk of
+// TS_DESC_CHUNK steps the first flagged step of the chunk, or INT32_MAX).
+// The work of extra workgroups of hstu_prepare's launch, one per (128-row tile slot, chunk of steps): it depends
+// on nothing else that launch writes, and so hides behind the work list, which one workgroup builds.
+// ---------------------------------------------------------------------------
+constexpr int TS_DESC_MAX_L = 16384;      // longest sequence descriptors are built for (table size)
+constexpr uint32_t TS_DESC_GENERAL = 0x8000u;
+__device__ __host__ __forceinline__ int64_t ts_desc_row0(int jagged, int L, int b, int64_t tok0) {
+  return jagged ? 8 * ((tok0 >> 3) + b) : (int64_t)b * ((L + 7) & ~7);
+}
+__device__ __host__ __forceinline__ int64_t ts_desc_tile0(int jagged, int n_qtiles, int b, int64_t tok0) {
+  return jagged ? (tok0 >> 7) + b : (int64_t)b * n_qtiles;
+}
+
+constexpr int TS_DESC_CHUNK = 8;          // steps per workgroup of the descriptor build
+__device__ __host__ __forceinline__ int ts_desc_chunks(int L) { return ((L + BN - 1) / BN + TS_DESC_CHUNK - 1) / TS_DESC_CHUNK; }
+__device__ __forceinline__ void ts_desc_block(const Params& p, uint16_t* __restrict__ desc, int32_t* __restrict__ tgen,
+                                              const int block, const int n_chunks, const TsKeys& keys) {
+  // The rows' own times and the chunk's 256 key timestamps in LDS.
+  __shared__ int64_t tq_l[BM], k_l[TS_DESC_CHUNK * BN];
+  __shared__ float thr_f[TS_KEYS];
+  __shared__ int32_t thr_b[TS_KEYS];
+  __shared__ unsigned char bkt[TS_KEYS];
+  __shared__ int sorted_to[TS_DESC_CHUNK];
+  __shared__ int found_b, found_o0, found_o1, first_general;
+  const int tid = threadIdx.x;
+  const int64_t slot = block / n_chunks;
+  const int chunk = block - (int)slot * n_chunks;
+  int b, qt, o0 = 0, nraw = 0;
+  if (p.jagged) {
+    // the sequence whose tile slots hold this one: every thread tries the sequences tid, tid + 256, ...; the
+    // slots of sequence b start at (its first token >> 7) + b, so exactly one sequence has
+    // tile0(b) <= slot < tile0(b + 1), or none (a slot past the last sequence's).  The thread that finds it
+    // hands its offsets on with it: one trip to memory for both.
+    if (tid == 0) { found_b = -1; first_general = 0x7fffffff; }
+    __syncthreads();
+    for (int c = tid; c < p.B; c += 256) {
+      const int f0 = p.seq_offsets[c], f1 = p.seq_offsets[c + 1];
+      if (ts_desc_tile0(1, 0, c, f0) <= slot && slot < ts_desc_tile0(1, 0, c + 1, f1)) { found_b = c; found_o0 = f0; found_o1 = f1; }
+    }
+    __syncthreads();
+    b = found_b;
+    if (b < 0) return;
+    o0 = found_o0;
+    nraw = found_o1 - o0;
+    qt = (int)(slot - ts_desc_tile0(1, 0, b, o0));
+  } else {
+    if (tid == 0) first_general = 0x7fffffff;
+    b = (int)(slot / p.n_qtiles);
+    qt = (int)(slot - (int64_t)b * p.n_qtiles);
+    if (b >= p.B) return;
+    seq_raw(p, b, o0, nraw);
+  }
+  const Seq s = seq_from(p, b, 0, o0, nraw);
+  const int q0 = qt * BM;
+  if (q0 >= s.rows) return;
+  const int n_steps_tile = (((q0 + BM < s.n_kv ? q0 + BM : s.n_kv) + BN - 1) / BN);   // steps a causal tile can touch
+  const int t0 = chunk * TS_DESC_CHUNK;
+  if (t0 >= n_steps_tile) return;
+  const int t1 = t0 + TS_DESC_CHUNK < n_steps_tile ? t0 + TS_DESC_CHUNK : n_steps_tile;
+  const int64_t row0 = ts_desc_row0(p.jagged, p.L, b, s.tok0);
+  // (the next sequence's first token: this one's plus its stored rows)
+  const int64_t row_end = b + 1 < p.B ? ts_desc_row0(p.jagged, p.L, b + 1, p.jagged ? s.tok0 + s.rows : 0) : (int64_t)p.ts_desc_pitch;
+  const int n_ts = s.n_ts;
+  const int64_t* tsg = p.ts + s.ts0;
+  if (tid < BM) {
+    // the time a row takes: that of the next row (its own for the last)
+    int iq = q0 + tid + 1;
+    iq = iq < n_ts ? iq : n_ts - 1;
+    tq_l[tid] = tsg[iq < 0 ? 0 : iq];
+  }
+#pragma unroll
+  for (int e = 0; e < TS_DESC_CHUNK * BN / 256; ++e) {
+    int j = t0 * BN + e * 256 + tid;
+    j = j < n_ts ? j : n_ts - 1;
+    k_l[e * 256 + tid] = (t0 * BN + e * 256 < (t1 * BN)) ? tsg[j < 0 ? 0 : j] : 0;
+  }
+  if (tid < TS_KEYS) {
+    thr_f[tid] = keys.thr_f[tid];
+    thr_b[tid] = tid <= p.ts_nb ? keys.thr_b[tid] : 0x7fffffff;
+    bkt[tid] = keys.bkt[tid];
+  }
+  __syncthreads();
+  {
+    // up to which key of a step the timestamps are in order: every thread compares one neighbouring pair, a
+    // wave's ballot covers two steps
+    static_assert(TS_DESC_CHUNK * BN == 256, "one key per thread");
+    const int l32 = tid & 31;
+    const int j_last = (n_ts - 1) - t0 * BN;                 // the last timestamp there is, as an index into k_l
+    const bool breaks = l32 < BN - 1 && tid + 1 <= j_last && k_l[tid + 1] < k_l[tid];
+    const uint64_t mask = __builtin_amdgcn_ballot_w64(breaks);
+    if (l32 == 0) {
+      const uint32_t mine = (uint32_t)(mask >> (tid & 32));
+      int e = mine ? __builtin_ctz(mine) : BN - 1;           // the step is in order up to its key e
+      e = tid + e < j_last ? tid + e : j_last;
+      sorted_to[tid >> 5] = e;
+    }
+  }
+  __syncthreads();
+  auto bucket = [&](int64_t d) {       // the bucket law on a difference >= 0, clipped to the table
+    const int dc = d < 1 ? 1 : (d < TS_DT_MAX ? (int)d : TS_DT_MAX);
+    const float f = (float)dc;
+    const uint32_t key = (__builtin_bit_cast(uint32_t, f) >> 21) - (uint32_t)TS_KEY0;
+    const int bk = (int)bkt[key] + (f >= thr_f[key] ? 1 : 0);
+    return bk < p.ts_nb ? bk : p.ts_nb;
+  };
+  int my_general = 0x7fffffff;
+  for (int idx = tid; idx < BM * (t1 - t0); idx += 256) {
+    const int r = idx & (BM - 1), tl = idx >> 7, t = t0 + tl;
+    const int i = q0 + r;
+    uint32_t word = 0u;
+    const int j0 = t * BN;
+    int j1 = j0 + BN - 1;
+    j1 = j1 < s.n_kv - 1 ? j1 : s.n_kv - 1;
+    j1 = j1 < i ? j1 : i;                // (the causal mask: later keys are masked whatever their bucket)
+    if (i < s.n_q && j1 >= j0) {
+      const int l0 = tl * BN, l1 = j1 - t0 * BN;     // the step's first key and the row's last, as indices into k_l
+      const int64_t tq = tq_l[r];
+      const int64_t k_first = k_l[l0], k_last = k_l[l1];
+      bool general = sorted_to[tl] < l1 || tq < k_last;
+      if (!general) {
+        const int bn = bucket(tq - k_last), bf = bucket(tq - k_first);
+        if (bf == bn && bn < TS_KEYS) {
+          word = (uint32_t)bn;
+        } else if (bf == bn + 1 && bf < TS_KEYS) {
+          // keys in order: those with tq - ts >= thr, i.e. ts <= tq - thr, are the first c of the step
+          const int64_t cut = tq - (int64_t)thr_b[bf];
+          int lo = l0, hi = l1;        // k[lo] <= cut < k[hi]: the first and last key are on different sides
+          while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (k_l[mid] <= cut) lo = mid; else hi = mid;
+          }
+          word = (uint32_t)bn | ((uint32_t)(lo + 1 - l0) << 7);
+        } else {
+          general = true;
+        }
+      }
+      if (general) {
+        word = TS_DESC_GENERAL;
+        my_general = t < my_general ? t : my_general;
+      }
+    }
+    // (a tile's last rows may lie past the sequence: those up to the next sequence's first row are this
+    // workgroup's to clear, the rest are that sequence's own)
+    if (row0 + i < row_end) desc[(int64_t)t * p.ts_desc_pitch + row0 + i] = (uint16_t)word;
+  }
+  // the chunk's first flagged step, INT32_MAX when it has none: a slot of its own per (tile, chunk), written every time
+  if (my_general != 0x7fffffff) atomicMin(&first_general, my_general);
+  __syncthreads();
+  if (tid == 0) tgen[(ts_desc_tile0(p.jagged, p.n_qtiles, b, s.tok0) + qt) * n_chunks + chunk] = first_general;
+}
+
+
 // What the main kernel reads from the workspace, rebuilt by every call:
 //  * the relative-position table scaled by log2(e) and zero-padded,
 //    [heads][POS_PAD + 2L-1 + POS_PAD]; the margins make every window read in-bounds;
@@ -1858,11 +2024,18 @@ __device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_
 __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __restrict__ pos_out, int4* __restrict__ tab_out,
                                                     int32_t* __restrict__ ok_out, int32_t* __restrict__ rel_out,
                                                     int32_t* __restrict__ range_out, int32_t* __restrict__ sched_out,
-                                                    int32_t* __restrict__ mrange_out, const TsKeys keys) {
+                                                    int32_t* __restrict__ mrange_out, uint16_t* __restrict__ desc_out,
+                                                    int32_t* __restrict__ tgen_out, const int n_prep, const int desc_chunks,
+                                                    const TsKeys keys) {
+  // workgroups [0, n_prep): what this comment lists; those behind them: the timestamp descriptors
+  if ((int)blockIdx.x >= n_prep) {
+    ts_desc_block(p, desc_out, tgen_out, (int)blockIdx.x - n_prep, desc_chunks, keys);
+    return;
+  }
   const int tid = threadIdx.x;
-  const int gtid = blockIdx.x * blockDim.x + tid, gsz = gridDim.x * blockDim.x;
-  if (sched_out && blockIdx.x == gridDim.x - 1) {
-    // The work list, by the last workgroup (the host launches one more than the rest needs).
+  const int gtid = blockIdx.x * blockDim.x + tid, gsz = n_prep * blockDim.x;
+  if (sched_out && (int)blockIdx.x == n_prep - 1) {
+    // The work list, by the last of these workgroups (the host launches one more than the rest needs).
     // Sequences are taken longest first (batches of up to SEG sequences; larger ones in batch order,
     // SEG at a time): the tiles with most keys start first and short ones fill in behind them.  Within
     // a sequence the last query tile (most keys) comes first.  The tiles of the sequences at hand are
@@ -2057,11 +2230,6 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     if (p.ctr)
       for (int i = tid; i < CTR_RESERVED + p.split_cap * p.H; i += 256) p.ctr[i] = 0u;
   }
-  if (p.ts_tquads) {
-    // the descriptor kernel, which follows, takes each tile's first flagged step as a minimum over its workgroups
-    int32_t* tg = const_cast<int32_t*>(p.ts_tquads);
-    for (int i = gtid; i < p.ts_desc_tiles; i += gsz) tg[i] = 0x7fffffff;
-  }
   if (tab_out) {
     // every head's bucket table: thresholds and buckets from the host, the table values times log2(e) with
     // bucket indices clipped to the table's last entry (the clip of the bucket law)
@@ -2096,7 +2264,7 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     __shared__ int mr_lo[4], mr_hi[4];
     const int nb = p.mask_batched ? p.B : 1;
     const int ppr = p.Lkv / 16;
-    for (int tile = blockIdx.x; tile < nb * p.n_qtiles; tile += gridDim.x) {
+    for (int tile = blockIdx.x; tile < nb * p.n_qtiles; tile += n_prep) {
       const int b = tile / p.n_qtiles, qt = tile - b * p.n_qtiles;
       const int r0 = qt * BM;
       const int rows = p.L - r0 < BM ? p.L - r0 : BM;
@@ -2144,7 +2312,7 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
   static_assert(BN == 32, "one lane per key of a tile");
   __shared__ int64_t red_lo[4], red_hi[4];
   const int lane = tid & 63, wv = tid >> 6, l32 = tid & 31;
-  for (int b = blockIdx.x; b < p.B; b += gridDim.x) {
+  for (int b = blockIdx.x; b < p.B; b += n_prep) {
     const Seq s = seq_info(p, b, 0);
     const int n = s.n_ts;
     if (n <= 0) {
@@ -2210,165 +2378,6 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       }
     }
   }
-}
-
-// ---------------------------------------------------------------------------
-// Timestamp descriptors.  The bucket of a pair depends on the sequence's timestamps alone: not on the head, not
-// on the layer.  With sorted timestamps the buckets of one row fall from key to key, and away from the diagonal
-// a step of 32 keys holds one bucket or two for a row.  This kernel works that out once per batch: for every
-// query row and every 32-key step at or below its diagonal one 16-bit word
-//   bits 0..6   bucket b of the step's last key the row keeps (the nearest in time)
-//   bits 7..12  c: the step's first c keys are one bucket further (b + 1), the others in b (0: one bucket)
-//   bit 15      neither holds (three buckets or more, timestamps out of order in the step, a key later than the
-//               row's own time, buckets past the table): the kernel looks every pair of the block up
-// laid out [step][row] (ts_desc_pitch rows per step; a sequence's rows start at ts_desc_row0), so that the 32
-// rows of a wave are 64 contiguous bytes per step.  Rows past the sequence get 0.  The main kernel's blocks then
-// read one word per lane instead of testing the tile's time range against the bucket thresholds, and the steps
-// before a tile's first flagged one can run as the hand-scheduled stream (ts_tquads: how many quads of them).
-// One workgroup per 128-row tile; the tile's part of the sequence's timestamps sits in LDS.
-// ---------------------------------------------------------------------------
-constexpr int TS_DESC_MAX_L = 16384;      // longest sequence descriptors are built for (table size)
-constexpr uint32_t TS_DESC_GENERAL = 0x8000u;
-__device__ __host__ __forceinline__ int64_t ts_desc_row0(int jagged, int L, int b, int64_t tok0) {
-  return jagged ? 8 * ((tok0 >> 3) + b) : (int64_t)b * ((L + 7) & ~7);
-}
-__device__ __host__ __forceinline__ int64_t ts_desc_tile0(int jagged, int n_qtiles, int b, int64_t tok0) {
-  return jagged ? (tok0 >> 7) + b : (int64_t)b * n_qtiles;
-}
-
-constexpr int TS_DESC_CHUNK = 8;          // steps per workgroup of the descriptor kernel
-__global__ __launch_bounds__(256) void hstu_prepare_ts_desc(const Params p, uint16_t* __restrict__ desc, int32_t* __restrict__ tgen,
-                                                           int n_chunks, const TsKeys keys) {
-  // One workgroup per (128-row tile, chunk of 32 steps): the rows' own times and the chunk's 1024 key timestamps in LDS.
-  // tgen[tile] (set to INT32_MAX by hstu_prepare beforehand) ends up as the tile's first flagged step.
-  __shared__ int64_t tq_l[BM], k_l[TS_DESC_CHUNK * BN];
-  __shared__ float thr_f[TS_KEYS];
-  __shared__ int32_t thr_b[TS_KEYS];
-  __shared__ unsigned char bkt[TS_KEYS];
-  __shared__ int sorted_to[TS_DESC_CHUNK];
-  const int tid = threadIdx.x;
-  const int64_t slot = blockIdx.x / n_chunks;
-  const int chunk = blockIdx.x - (int)slot * n_chunks;
-  int b, qt;
-  Seq s;
-  bool have_seq = false;
-  if (p.sched) {
-    // from the work list that hstu_prepare has just built: one entry per (sequence, tile, key chunk), with the
-    // sequence's first token and length in it (no second trip to memory for the offsets)
-    const int4 item = ((const int4*)(p.sched + 4))[slot < p.items_max ? slot : 0];
-    if (slot >= p.sched[0]) return;
-    if (((item.y >> 16) & 0xff) != 0) return;       // a split tile's later chunks: the first one's workgroups do the tile
-    b = item.x & 0x3fff;
-    qt = item.y & 0xffff;
-    s = seq_from(p, b, 0, item.z, item.w);
-    have_seq = true;
-  } else if (p.jagged) {
-    int lo = 0, hi = p.B;            // the last b with tile0(b) <= slot
-    while (hi - lo > 1) {
-      const int mid = (lo + hi) >> 1;
-      if (ts_desc_tile0(1, 0, mid, p.seq_offsets[mid]) <= slot) lo = mid; else hi = mid;
-    }
-    b = lo;
-    qt = (int)(slot - ts_desc_tile0(1, 0, b, p.seq_offsets[b]));
-  } else {
-    b = (int)(slot / p.n_qtiles);
-    qt = (int)(slot - (int64_t)b * p.n_qtiles);
-  }
-  if (b >= p.B) return;
-  if (!have_seq) s = seq_info(p, b, 0);
-  const int q0 = qt * BM;
-  if (q0 >= s.rows) return;
-  const int n_steps_tile = (((q0 + BM < s.n_kv ? q0 + BM : s.n_kv) + BN - 1) / BN);   // steps a causal tile can touch
-  const int t0 = chunk * TS_DESC_CHUNK;
-  if (t0 >= n_steps_tile) return;
-  const int t1 = t0 + TS_DESC_CHUNK < n_steps_tile ? t0 + TS_DESC_CHUNK : n_steps_tile;
-  const int64_t row0 = ts_desc_row0(p.jagged, p.L, b, s.tok0);
-  // (the next sequence's first token: this one's plus its stored rows)
-  const int64_t row_end = b + 1 < p.B ? ts_desc_row0(p.jagged, p.L, b + 1, p.jagged ? s.tok0 + s.rows : 0) : (int64_t)p.ts_desc_pitch;
-  const int n_ts = s.n_ts;
-  const int64_t* tsg = p.ts + s.ts0;
-  if (tid < BM) {
-    // the time a row takes: that of the next row (its own for the last)
-    int iq = q0 + tid + 1;
-    iq = iq < n_ts ? iq : n_ts - 1;
-    tq_l[tid] = tsg[iq < 0 ? 0 : iq];
-  }
-#pragma unroll
-  for (int e = 0; e < TS_DESC_CHUNK * BN / 256; ++e) {
-    int j = t0 * BN + e * 256 + tid;
-    j = j < n_ts ? j : n_ts - 1;
-    k_l[e * 256 + tid] = (t0 * BN + e * 256 < (t1 * BN)) ? tsg[j < 0 ? 0 : j] : 0;
-  }
-  if (tid < TS_KEYS) {
-    thr_f[tid] = keys.thr_f[tid];
-    thr_b[tid] = tid <= p.ts_nb ? keys.thr_b[tid] : 0x7fffffff;
-    bkt[tid] = keys.bkt[tid];
-  }
-  __syncthreads();
-  {
-    // up to which key of a step the timestamps are in order: every thread compares one neighbouring pair, a
-    // wave's ballot covers two steps
-    static_assert(TS_DESC_CHUNK * BN == 256, "one key per thread");
-    const int l32 = tid & 31;
-    const int j_last = (n_ts - 1) - t0 * BN;                 // the last timestamp there is, as an index into k_l
-    const bool breaks = l32 < BN - 1 && tid + 1 <= j_last && k_l[tid + 1] < k_l[tid];
-    const uint64_t mask = __builtin_amdgcn_ballot_w64(breaks);
-    if (l32 == 0) {
-      const uint32_t mine = (uint32_t)(mask >> (tid & 32));
-      int e = mine ? __builtin_ctz(mine) : BN - 1;           // the step is in order up to its key e
-      e = tid + e < j_last ? tid + e : j_last;
-      sorted_to[tid >> 5] = e;
-    }
-  }
-  __syncthreads();
-  auto bucket = [&](int64_t d) {       // the bucket law on a difference >= 0, clipped to the table
-    const int dc = d < 1 ? 1 : (d < TS_DT_MAX ? (int)d : TS_DT_MAX);
-    const float f = (float)dc;
-    const uint32_t key = (__builtin_bit_cast(uint32_t, f) >> 21) - (uint32_t)TS_KEY0;
-    const int bk = (int)bkt[key] + (f >= thr_f[key] ? 1 : 0);
-    return bk < p.ts_nb ? bk : p.ts_nb;
-  };
-  int my_general = 0x7fffffff;
-  for (int idx = tid; idx < BM * (t1 - t0); idx += 256) {
-    const int r = idx & (BM - 1), tl = idx >> 7, t = t0 + tl;
-    const int i = q0 + r;
-    uint32_t word = 0u;
-    const int j0 = t * BN;
-    int j1 = j0 + BN - 1;
-    j1 = j1 < s.n_kv - 1 ? j1 : s.n_kv - 1;
-    j1 = j1 < i ? j1 : i;                // (the causal mask: later keys are masked whatever their bucket)
-    if (i < s.n_q && j1 >= j0) {
-      const int l0 = tl * BN, l1 = j1 - t0 * BN;     // the step's first key and the row's last, as indices into k_l
-      const int64_t tq = tq_l[r];
-      const int64_t k_first = k_l[l0], k_last = k_l[l1];
-      bool general = sorted_to[tl] < l1 || tq < k_last;
-      if (!general) {
-        const int bn = bucket(tq - k_last), bf = bucket(tq - k_first);
-        if (bf == bn && bn < TS_KEYS) {
-          word = (uint32_t)bn;
-        } else if (bf == bn + 1 && bf < TS_KEYS) {
-          // keys in order: those with tq - ts >= thr, i.e. ts <= tq - thr, are the first c of the step
-          const int64_t cut = tq - (int64_t)thr_b[bf];
-          int lo = l0, hi = l1;        // k[lo] <= cut < k[hi]: the first and last key are on different sides
-          while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (k_l[mid] <= cut) lo = mid; else hi = mid;
-          }
-          word = (uint32_t)bn | ((uint32_t)(lo + 1 - l0) << 7);
-        } else {
-          general = true;
-        }
-      }
-      if (general) {
-        word = TS_DESC_GENERAL;
-        my_general = t < my_general ? t : my_general;
-      }
-    }
-    // (a tile's last rows may lie past the sequence: those up to the next sequence's first row are this
-    // workgroup's to clear, the rest are that sequence's own)
-    if (row0 + i < row_end) desc[(int64_t)t * p.ts_desc_pitch + row0 + i] = (uint16_t)word;
-  }
-  if (my_general != 0x7fffffff) atomicMin(&tgen[ts_desc_tile0(p.jagged, p.n_qtiles, b, s.tok0) + qt], my_general);
 }
 
 // SEG: segment ids (padded layout, L a multiple of 4): a pair is kept when its row's and its key's
@@ -2663,7 +2672,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   DmaCtx cx;
   struct { int n_q, n_kv, rows, n_ts; } s;       // of the item's sequence
   int h = 0, q0 = 0, r0 = 0, qrow = 0, wave_last = -1, nt = 0, t_lo = 0, n_chunks = 1, chunk = 0, pslot = 0, ts32 = 0;
-  int has_desc = 0, desc_quads = 0;         // descriptors at hand; leading quads of steps none of whose rows is flagged
+  int has_desc = 0, desc_first = 0x7fffffff;   // descriptors at hand; per lane, a chunk's first step with a flagged row
   float alpha2 = 0.f;
   const int64_t* tsg = nullptr;
   bf16_t* og = nullptr;
@@ -2685,8 +2694,13 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     // whether the sequence's int32 timestamps are valid (its time span allows them)
     ts32 = TS ? pf.ts_ok[k.b] : 0;
     if constexpr (TSD) {
+      // (each lane takes one chunk's first flagged step, of the chunks that hold interior steps; the first lane
+      // that has one holds the tile's: stream_quads reads it, behind the loads that go out in between)
       has_desc = pf.ts_desc != nullptr;
-      desc_quads = has_desc ? (pf.ts_tquads[ts_desc_tile0(pf.jagged, pf.n_qtiles, k.b, k.s.tok0) + k.qt] >> 2) : 0;
+      const int interior = (q0 < s.n_kv ? q0 : s.n_kv) / BN;
+      desc_first = 0x7fffffff;
+      if (has_desc && lane * TS_DESC_CHUNK < interior)
+        desc_first = pf.ts_tquads[(ts_desc_tile0(pf.jagged, pf.n_qtiles, k.b, k.s.tok0) + k.qt) * pf.ts_desc_chunks + lane];
     }
     og = (bf16_t*)pf.out + k.s.bo;
   };
@@ -2989,9 +3003,12 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       // in at the tile's arrival counter; the workgroup that arrives last adds the others' partials to
       // its own, always in the order of the chunks, and writes the rows.  Partials and counter go by
       // device-scope atomic stores, loads and adds (which bypass the caches that are not coherent across
-      // the chip), ordered by waiting for the stores' completion before the count: no cache is flushed,
-      // and nothing depends on which workgroup runs where.  The result does not depend on the order of
-      // arrival.
+      // the chip).  The order is the memory model's: every wave's stores, then the workgroup barrier, then
+      // thread 0's count as a release-acquire add at device scope (the barrier makes the other waves' stores
+      // part of what it releases); the last arriver's count reads the others' releases, its barrier hands
+      // that on to its other waves, and each of them takes an acquire fence before it loads.  (The wait for
+      // the stores' acknowledgement stays: it costs nothing once the release is there.)  Nothing depends on
+      // which workgroup runs where, and the result does not depend on the order of arrival.
       constexpr int NPC = BM * D / 2;      // 8-byte pieces of a chunk's partial
       uint64_t* slot0 = (uint64_t*)pf.partial + ((int64_t)pslot * pf.H + h) * NPC;
       uint64_t* mine = slot0 + (int64_t)chunk * pf.H * NPC + (w * (DVB * 4)) * 128 + 2 * lane;
@@ -3008,10 +3025,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       HSTU_WAIT_VMCNT(0);                  // every store of this wave has been acknowledged
       __syncthreads();
       uint32_t* arrive = pf.ctr + CTR_RESERVED + pslot * pf.H + h;
-      if (tid == 0) xch[0] = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid == 0) xch[0] = __hip_atomic_fetch_add(arrive, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
       __syncthreads();
       const uint32_t before = xch[0];
       if (before != (uint32_t)(n_chunks - 1)) return;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
       if (tid == 0) __hip_atomic_store(arrive, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next call
       // (a chunk's pieces are asked for 16 at a time per lane and added once they are there: two round trips
       // per chunk instead of one per piece)
@@ -3108,7 +3126,9 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     if constexpr (TS) {
       // with timestamps: only on descriptors, and only the leading steps in which no row of the tile is flagged
       if (!ts32 || !has_desc) return 0;
-      const int nd = desc_quads - (t_lo >> 2);
+      const uint64_t flagged = __builtin_amdgcn_ballot_w64(desc_first != 0x7fffffff);
+      const int first = flagged ? __builtin_amdgcn_readlane(desc_first, (int)__builtin_ctzll(flagged)) : 0x7fffffff;
+      const int nd = (first >> 2) - (t_lo >> 2);
       n = (t_lo & 3) != 0 ? 0 : (n < nd ? n : nd);
     }
     // lookahead: steps up to t_lo + 4n + 2 exist and are whole
@@ -4650,7 +4670,7 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, 
       w.desc_pitch = rows;
       w.desc_tiles = jag ? (a->total_tokens >> 7) + a->B + 1 : (long long)a->B * n_qtiles;
       w.desc_bytes = bytes;
-      w.tquad_bytes = up((size_t)w.desc_tiles * sizeof(int32_t));
+      w.tquad_bytes = up((size_t)w.desc_tiles * (size_t)ts_desc_chunks(a->L) * sizeof(int32_t));
     }
   }
   const long long t128 = jag ? a->total_tokens / BM + a->B : (long long)a->B * n_qtiles;
@@ -4975,6 +4995,7 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   q.ts_tquads = tquad_out;
   q.ts_desc_pitch = (int32_t)ws.desc_pitch;
   q.ts_desc_tiles = (int32_t)ws.desc_tiles;
+  q.ts_desc_chunks = ts_desc_chunks(q.L);
   int32_t* sched_out = ws.sched_bytes ? (int32_t*)(base + ws.bias_total()) : nullptr;
   q.sched = sched_out;
   q.items_max = ws.items_max;
@@ -4996,16 +5017,13 @@ int setup_workspace(const HstuAttnFwdArgs* args, const WorkspacePlan& ws, Params
   if ((ws.bias_total() || ws.sched_bytes) && (!(args->flags & HSTU_FWD_WORKSPACE_PREPARED) || (args->flags & HSTU_FWD_PREPARE_ONLY))) {
     static const TsKeys no_keys = {{0}, {0}, {0}};
     const TsKeys& keys = tab_out ? bucket_law(q.ts_bucket_size).keys : no_keys;
-    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)blocks), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out, sched_out, mrange_out, keys);
+    // (the descriptors: one more workgroup per tile slot and chunk of steps, behind the others)
+    const int n_chunks = ts_desc_chunks(q.L);
+    const long long desc_blocks = desc_out ? (long long)ws.desc_tiles * n_chunks : 0;
+    hipLaunchKernelGGL(hstu_prepare, dim3((unsigned)(blocks + desc_blocks)), dim3(256), 0, st, q, pos_out, tab_out, ok_out, rel_out, range_out,
+                       sched_out, mrange_out, desc_out, tquad_out, (int)blocks, n_chunks, keys);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "prepare kernel launch: %s", hipGetErrorString(e));
-    if (desc_out) {
-      const int n_chunks = ((q.L + BN - 1) / BN + TS_DESC_CHUNK - 1) / TS_DESC_CHUNK;
-      const long long slots = q.sched ? q.items_max : ws.desc_tiles;     // by work-list entry, else by tile slot
-      hipLaunchKernelGGL(hstu_prepare_ts_desc, dim3((unsigned)(slots * n_chunks)), dim3(256), 0, st, q, desc_out, tquad_out, n_chunks, keys);
-      e = hipGetLastError();
-      if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "descriptor kernel launch: %s", hipGetErrorString(e));
-    }
   }
   return HSTU_OK;
 }

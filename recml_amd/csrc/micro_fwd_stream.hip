@@ -9,7 +9,9 @@
 //
 // Build: hipcc -O3 -std=c++17 --offload-arch=gfx950 -Xclang -target-feature -Xclang -packed-fp32-ops
 //        -o micro_fwd_stream micro_fwd_stream.hip
-// Run:   ./micro_fwd_stream [rounds]        (one JSON line per variant)
+// Run:   ./micro_fwd_stream [rounds [zero_operands [probes]]]        (one JSON line per variant)
+//        zero_operands: bit 0 K, bit 1 V, bit 2 Q all zero (the same instructions on data that toggles no bits);
+//        probes 0: the blocks only, not the instruction-rate probes
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -352,6 +354,16 @@ __global__ __launch_bounds__(256, 2) void k_clock(int iters, float* out, long lo
   uintx4 lv[4] = {a, a, a, a};
   typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
   uintx2 lt[4] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};
+  // operands of modes 19 and 20: a hash of (lane, register, word) as two bf16 values each, exponents 126..127
+  uintx4 ra[4], rb[4];
+  for (int i = 0; i < 4; ++i)
+    for (int c = 0; c < 4; ++c) {
+      uint32_t h = (threadIdx.x * 16u + i * 4u + c) * 2654435761u;
+      h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+      const uint32_t g = h * 3266489917u ^ (h >> 16);
+      ra[i][c] = (h & 0x80ff80ffu) | 0x3f003f00u;
+      rb[i][c] = (g & 0x80ff80ffu) | 0x3f003f00u;
+    }
   const long long r0 = wall_clock64(), t0 = clock64();
   for (int it = 0; it < iters; ++it) {
     if (MODE == 0) {
@@ -469,6 +481,22 @@ __global__ __launch_bounds__(256, 2) void k_clock(int iters, float* out, long lo
 #pragma unroll
         for (int i = 0; i < 12; ++i) asm volatile("v_mul_f32 %0, %0, %1" : "+v"(x[i & 7]) : "v"(1.0001f));
       }
+    } else if (MODE == 19 || MODE == 20) {
+      // matrix instructions alone (19) or with the block's vector mix (20), on operands whose bits differ from lane
+      // to lane and from one instruction to the next (bf16 values of either sign between 0.5 and 2): the same
+      // instructions as modes 0 and 3, which multiply ones, with the data paths toggling as they do on real tiles
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[j & 3]) : "v"(ra[j & 3]), "v"(rb[(j >> 2) & 3]));
+        if (MODE == 20) {
+          asm volatile("v_exp_f32 %0, %0" : "+v"(x[0]));
+          asm volatile("v_mul_f32 %0, %0, %1" : "+v"(x[1]) : "v"(1.0001f));
+          asm volatile("v_mul_f32 %0, %0, %1" : "+v"(x[2]) : "v"(1.0001f));
+          asm volatile("v_exp_f32 %0, %0" : "+v"(x[3]));
+          asm volatile("v_mul_f32 %0, %0, %1" : "+v"(x[4]) : "v"(1.0001f));
+          asm volatile("v_mul_f32 %0, %0, %1" : "+v"(x[5]) : "v"(1.0001f));
+        }
+      }
     } else if (MODE == 10) {      // one chain of dependent matrix instructions
 #pragma unroll
       for (int j = 0; j < 16; ++j) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[0]) : "v"(a), "v"(b));
@@ -538,6 +566,11 @@ static float bf16_round(float x) {
 static uint16_t bf16_bits(float x) { float y = bf16_round(x); uint32_t b; memcpy(&b, &y, 4); return (uint16_t)(b >> 16); }
 static float frand(uint32_t& s) { s = s * 1664525u + 1013904223u; return ((s >> 8) & 0xffff) / 32768.0f - 1.0f; }
 
+// What the operands' values cost (second argument of the program): bit 0 makes K all zero, bit 1 V, bit 2 Q.
+// The instruction stream and its timing rules are the same; what changes is how many bits toggle in the matrix
+// cores' and the register file's data paths, i.e. the power the chip draws, and with it the clock it sustains.
+static int g_zero_data = 0;
+
 template <typename KernelT>
 static void run(const char* name, KernelT kern, bool pos, int rounds, int n_wg) {
   std::vector<float> q(BM * D), k(NSTAGE * BN * D), v(NSTAGE * BN * D), win(NSTAGE * WIN);
@@ -546,6 +579,9 @@ static void run(const char* name, KernelT kern, bool pos, int rounds, int n_wg) 
   for (auto& x : k) x = bf16_round(0.3f * frand(seed));
   for (auto& x : v) x = bf16_round(0.3f * frand(seed));
   for (auto& x : win) x = 0.05f * frand(seed) * LOG2E;
+  if (g_zero_data & 1) for (auto& x : k) x = 0.f;
+  if (g_zero_data & 2) for (auto& x : v) x = 0.f;
+  if (g_zero_data & 4) for (auto& x : q) x = 0.f;
   const float alpha2 = LOG2E;
   std::vector<uint16_t> qb(q.size()), kb(k.size()), vb(v.size());
   for (size_t i = 0; i < q.size(); ++i) qb[i] = bf16_bits(q[i]);
@@ -595,11 +631,11 @@ static void run(const char* name, KernelT kern, bool pos, int rounds, int n_wg) 
   for (auto c : cyc) { cyc_sum += (double)c; cyc_max = c > cyc_max ? c : cyc_max; }
   const double blocks = 4.0 * rounds;           // blocks per wave
   // two waves per SIMD when the grid holds two workgroups per CU: a SIMD's time per wave-block is half a wave's
-  printf("{\"variant\": \"%s\", \"pos_bias\": %s, \"workgroups\": %d, \"rounds\": %d, \"kernel_ms\": %.4f, "
+  printf("{\"variant\": \"%s\", \"zero_operands\": %d, \"pos_bias\": %s, \"workgroups\": %d, \"rounds\": %d, \"kernel_ms\": %.4f, "
          "\"wave_cycles_per_block_avg\": %.1f, \"wave_cycles_per_block_max\": %.1f, \"simd_cycles_per_wave_block\": %.1f, "
          "\"mfma_cycles_per_block\": 512, \"clock_mhz\": %.0f, \"tflops\": %.0f, \"max_abs_err_over_max_ref\": %.3e}\n",
-         name, pos ? "true" : "false", n_wg, rounds, ms, cyc_sum / cyc.size() / blocks, (double)cyc_max / blocks,
-         cyc_sum / cyc.size() / blocks / 2.0, mhz, 4.0 * n_wg * blocks * 16 * 32768 / (ms * 1e-3) * 1e-12, max_err / max_ref);
+         name, g_zero_data, pos ? "true" : "false", n_wg, rounds, ms, cyc_sum / cyc.size() / blocks, (double)cyc_max / blocks,
+         cyc_sum / cyc.size() / blocks / 2.0, mhz, 4.0 * n_wg * blocks * 16 * 32768 / (ms * 1e-3) * 1e-12, max_ref > 0 ? max_err / max_ref : max_err);
   fflush(stdout);
   CK(hipFree(dq)); CK(hipFree(dk)); CK(hipFree(dv)); CK(hipFree(dwin)); CK(hipFree(dout)); CK(hipFree(dcyc));
 }
@@ -613,6 +649,9 @@ static void run_dma(const char* name, KernelT kern, bool pos, int rounds, int re
   for (auto& x : k) x = bf16_round(0.3f * frand(seed));
   for (auto& x : v) x = bf16_round(0.3f * frand(seed));
   for (auto& x : ptab) x = 0.05f * frand(seed) * LOG2E;
+  if (g_zero_data & 1) for (auto& x : k) x = 0.f;
+  if (g_zero_data & 2) for (auto& x : v) x = 0.f;
+  if (g_zero_data & 4) for (auto& x : q) x = 0.f;
   const float alpha2 = LOG2E;
   std::vector<uint16_t> qb(q.size()), kb(k.size()), vb(v.size());
   for (size_t i = 0; i < q.size(); ++i) qb[i] = bf16_bits(q[i]);
@@ -660,17 +699,16 @@ static void run_dma(const char* name, KernelT kern, bool pos, int rounds, int re
   double cyc_sum = 0; long long cyc_max = 0;
   for (auto c : cyc) { cyc_sum += (double)c; cyc_max = c > cyc_max ? c : cyc_max; }
   const double blocks = (double)T * reps;
-  printf("{\"variant\": \"%s\", \"pos_bias\": %s, \"workgroups\": %d, \"steps_per_item\": %d, \"items\": %d, \"kernel_ms\": %.4f, "
+  printf("{\"variant\": \"%s\", \"zero_operands\": %d, \"pos_bias\": %s, \"workgroups\": %d, \"steps_per_item\": %d, \"items\": %d, \"kernel_ms\": %.4f, "
          "\"wave_cycles_per_block_avg\": %.1f, \"wave_cycles_per_block_max\": %.1f, \"simd_cycles_per_wave_block\": %.1f, "
          "\"mfma_cycles_per_block\": 512, \"clock_mhz\": %.0f, \"tflops\": %.0f, \"max_abs_err_over_max_ref\": %.3e}\n",
-         name, pos ? "true" : "false", n_wg, T, reps, ms, cyc_sum / cyc.size() / blocks, (double)cyc_max / blocks,
-         cyc_sum / cyc.size() / blocks / 2.0, mhz, 4.0 * n_wg * blocks * 16 * 32768 / (ms * 1e-3) * 1e-12, max_err / max_ref);
+         name, g_zero_data, pos ? "true" : "false", n_wg, T, reps, ms, cyc_sum / cyc.size() / blocks, (double)cyc_max / blocks,
+         cyc_sum / cyc.size() / blocks / 2.0, mhz, 4.0 * n_wg * blocks * 16 * 32768 / (ms * 1e-3) * 1e-12, max_ref > 0 ? max_err / max_ref : max_err);
   fflush(stdout);
   CK(hipFree(dq)); CK(hipFree(dk)); CK(hipFree(dv)); CK(hipFree(dtab)); CK(hipFree(dout)); CK(hipFree(dcyc));
 }
 
 #ifdef HSTU_STREAM_EXPERIMENTS
-static int g_zero_data = 0;     // bit 0: K all zero, bit 1: V, bit 2: Q (what the operands' values cost: second argument)
 // One variant of the sweep.  Compute-only variants go round the four ring stages (filled once) `rounds` times;
 // variants with loads stream 64 steps from global memory per item, `items` items.  ns per wave-block is the
 // kernel's time over the blocks a SIMD's two waves go through; 16 matrix instructions alone take 217 ns.
@@ -743,9 +781,7 @@ static void run_exp(const char* name, bool pos, bool wrong, int rounds, int n_wg
 
 int main(int argc, char** argv) {
   const int rounds = argc > 1 ? atoi(argv[1]) : 500;
-#ifdef HSTU_STREAM_EXPERIMENTS
   g_zero_data = argc > 2 ? atoi(argv[2]) : 0;
-#endif
   hipDeviceProp_t prop; CK(hipGetDeviceProperties(&prop, 0));
   const int n_wg = 2 * prop.multiProcessorCount;       // two workgroups per CU, eight waves: two per SIMD
 #if defined(HSTU_STREAM_EXPERIMENTS) && !defined(HSTU_PROBES_TOO)
@@ -758,12 +794,16 @@ int main(int argc, char** argv) {
   CK(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, 0));
   CK(hipDeviceGetAttribute(&clk_khz, hipDeviceAttributeClockRate, 0));
   printf("{\"device\": \"%s\", \"cus\": %d, \"wall_clock_khz\": %d, \"clock_khz\": %d}\n", prop.name, prop.multiProcessorCount, wall_khz, clk_khz);
+  const bool probes = !(argc > 3 && atoi(argv[3]) == 0);     // third argument 0: the blocks only, not the instruction-rate probes
+  if (probes) {
   run_clock<1>("exp2_only (64 per iter)", 10000, n_wg, 64);
   run_clock<1>("exp2_only (64 per iter)", 40000, n_wg, 64);
   run_clock<5>("mul_only (64 per iter)", 40000, n_wg, 64);
   run_clock<0>("mfma_only (16 per iter)", 10000, n_wg, 16);
   run_clock<0>("mfma_only (16 per iter)", 40000, n_wg, 16);
   run_clock<0>("mfma_only, one workgroup per CU", 40000, n_wg / 2, 16);
+  run_clock<19>("mfma_only, operands of random bits (16 per iter)", 40000, n_wg, 16);
+  run_clock<20>("mfma + 2 exp2 + 4 mul, operands of random bits (16 groups per iter)", 40000, n_wg, 16);
   run_clock<2>("mfma + 4 exp2 (16 groups per iter)", 40000, n_wg, 16);
   run_clock<3>("mfma + 2 exp2 + 4 mul (16 groups per iter)", 40000, n_wg, 16);
   run_clock<4>("2 exp2 + 4 mul (16 groups per iter)", 40000, n_wg, 16);
@@ -788,6 +828,7 @@ int main(int argc, char** argv) {
   run_clock<3>("mfma + 2 exp2 + 4 mul, one workgroup per CU", 40000, n_wg / 2, 16);
   run_clock<3>("mfma + 2 exp2 + 4 mul, one workgroup in all", 40000, 1, 16);
   run_clock<0>("mfma_only, one workgroup in all", 40000, 1, 16);
+  }
   run("cpp_block", k_cpp<false>, false, rounds, n_wg);
   run("cpp_block", k_cpp<true>, true, rounds, n_wg);
   run("hand_stream", k_stream<false>, false, rounds, n_wg);

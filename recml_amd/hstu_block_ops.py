@@ -131,11 +131,22 @@ def _wants_grad(*ts):
   return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in ts)
 
 
+NORM_GATE_BWD_MAX_WIDTH = 2048     # widest row hstu_norm_gate_bwd takes (the forward kernel: 8192)
+
+
+def _check_grad_width(W):
+  if W > NORM_GATE_BWD_MAX_WIDTH:
+    raise ValueError(f"the gradient of the layer norm is there for rows of up to {NORM_GATE_BWD_MAX_WIDTH} elements, got {W}: "
+                     "run the forward under torch.no_grad(), or use torch.nn.functional.layer_norm for this width")
+
+
 def norm_gate(attn, u, gamma, beta, eps: float = 1e-6):
   """u * layer_norm(attn) over the last axis.  attn, u: [..., W] bf16 whose last axis is contiguous
   and whose leading axes collapse to one row stride (a slice of a fused projection does);
-  gamma, beta: [W].  Differentiable in all four (W up to 2048 then)."""
+  gamma, beta: [W].  Differentiable in all four (W up to 2048 then: wider rows with a gradient wanted
+  raise here, not at backward time)."""
   if _wants_grad(attn, u, gamma, beta):
+    _check_grad_width(attn.shape[-1])
     return _NormGateFn.apply(attn, u, gamma, beta, eps)
   return _norm_gate_fwd(attn, u, gamma, beta, eps)
 
@@ -144,6 +155,7 @@ def layer_norm(x, gamma, beta, eps: float = 1e-6):
   """layer_norm(x) over the last axis (keras LayerNormalization as the block's input norm uses it,
   recml/layers/keras/hstu.py:442): the same kernels without the gate.  Differentiable in x, gamma, beta."""
   if _wants_grad(x, gamma, beta):
+    _check_grad_width(x.shape[-1])
     return _NormGateFn.apply(x, None, gamma, beta, eps)
   return _norm_gate_fwd(x, None, gamma, beta, eps)
 
@@ -170,8 +182,12 @@ def gemm_silu(x, w, bias=None, activation: bool = True, residual=None):
   if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[0]:
     raise ValueError(f"x [M, K] and w [K, N] expected, got {tuple(x.shape)} and {tuple(w.shape)}")
   # the library wants 16-byte aligned operands and a row stride that keeps rows so
-  if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
+  # (`contiguous()` returns a dense tensor as it is, misaligned or not: a view that starts off a 16-byte
+  # boundary needs a copy of its own)
+  if x.stride(1) != 1 or x.stride(0) % 8:
     x = x.contiguous()
+  if x.data_ptr() % 16:
+    x = x.clone(memory_format=torch.contiguous_format)
   w = w.contiguous()
   if w.data_ptr() % 16:
     w = w.clone()
@@ -201,8 +217,10 @@ def gemm_silu(x, w, bias=None, activation: bool = True, residual=None):
     _check("residual", residual)
     if tuple(residual.shape) != (M, N):
       raise ValueError(f"residual must be [{M}, {N}], got {tuple(residual.shape)}")
-    if residual.stride(1) != 1 or residual.stride(0) % 8 or residual.data_ptr() % 16:
+    if residual.stride(1) != 1 or residual.stride(0) % 8:
       residual = residual.contiguous()
+    if residual.data_ptr() % 16:
+      residual = residual.clone(memory_format=torch.contiguous_format)
     a.c, a.c_stride = residual.data_ptr(), residual.stride(0)
   with torch.cuda.device(x.device):
     rc = lib.hstu_gemm_silu_fwd(C.byref(a), C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream))

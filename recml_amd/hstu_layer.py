@@ -5,7 +5,8 @@ The harness for the end-to-end (config-4) shape: the attention is
 inference the projections' activation and the attention norm + U gate are the
 fused steps of `recml_amd.hstu_block_ops`; the rest is plain torch on the GPU
 (embedding gather, input layer norm, the output product with the residual as
-its C operand).  No dropout.
+its C operand).  No dropout: a block built with a rate refuses a training-mode
+forward (inference, where the reference applies none either, is unaffected).
 Parameters are created frozen; after `requires_grad_(True)` the attention goes
 through the HIP backward kernels; in bf16 on a GPU so do the layer norms and the
 U gate (one pass each way), the attention's and the gate's gradients landing in
@@ -136,7 +137,11 @@ class HSTUBlock(torch.nn.Module):
       raise NotImplementedError("softmax attention is outside this build; only the pointwise path is accelerated")
     if hidden_dim % num_heads:
       raise ValueError(f"hidden_dim {hidden_dim} is not a multiple of num_heads {num_heads}")
-    del dropout  # inference only
+    if not 0.0 <= dropout < 1.0:
+      raise ValueError(f"dropout must be in [0, 1), got {dropout}")
+    # The reference drops attention weights in training (recml/layers/keras/hstu.py:386-387); the kernels here have
+    # no dropout, so a block with a rate set refuses a training-mode forward rather than train without it.
+    self.dropout = float(dropout)
     self.num_heads = num_heads
     self.head_dim = hidden_dim // num_heads
     self.hidden_dim = hidden_dim
@@ -181,6 +186,11 @@ class HSTUBlock(torch.nn.Module):
     (recml/layers/keras/hstu.py:422-440).  `batch`: an `hstu_ops.AttentionBatch` shared with the
     other blocks that see the same lengths, timestamps and tables.
     """
+    if self.dropout > 0.0 and self.training:
+      raise NotImplementedError(
+          f"HSTUBlock(dropout={self.dropout}) in training mode: dropout on the attention weights "
+          "(recml/layers/keras/hstu.py:386-387) is not implemented by the attention kernels; "
+          "call .eval() for inference or build the block with dropout=0")
     B, L, D = inputs.shape
     H, hd = self.num_heads, self.head_dim
     fused = self._fused_inference(inputs, pos_bias, ts_bias, attention_bias)

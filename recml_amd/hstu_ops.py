@@ -86,7 +86,9 @@ class AttentionBatch:
   The preparation is reused when the call's shapes and options are the same and the tensors it was
   built from (`seq_lens` / `seq_offsets`, `timestamps`, `pos_bias`, `ts_bias`, a dense `mask`) are the same objects,
   unmodified since (torch's version counter); anything else prepares again.  q, k, v, `alpha` and `n`
-  may differ from call to call.  Not for concurrent use on several streams.
+  may differ from call to call.  Not for concurrent use on several streams.  Tensors created under
+  `torch.inference_mode()` have no version counter: a change made to one of them in place is not noticed, so
+  take a new AttentionBatch after such a change.
   """
 
   def __init__(self):
@@ -102,7 +104,9 @@ class AttentionBatch:
       return None
     if not isinstance(t, torch.Tensor):
       return False            # not a tensor: never reused
-    return (t.data_ptr(), t._version, tuple(t.shape), tuple(t.stride()), t.dtype)
+    # (tensors made under torch.inference_mode() carry no version counter, and reading it raises)
+    version = -1 if t.is_inference() else t._version
+    return (t.data_ptr(), version, tuple(t.shape), tuple(t.stride()), t.dtype)
 
   def _attach(self, args, keep, sig, tensors):
     ws = _lib.load().hstu_attn_fwd_workspace_bytes(C.byref(args))
@@ -537,44 +541,6 @@ def hstu_attention_autograd(q, k, v, *, pos_bias=None, ts_bias=None, bias=None, 
   and ts_bias, and a dense `bias` (its gradient is dS summed over the heads, and over the batch
   when the bias is shared by it)."""
   return _HstuAttentionFn.apply(q, k, v, pos_bias, ts_bias, bias, kwargs)
-
-
-def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=True, pos_bias=None,
-                          timestamps=None, ts_bias=None, ts_bucket_size=0.301, bias=None, mask=None,
-                          sliding_window_size=None):
-  """The op in plain torch on padded [B, L, H, d] tensors (recml/layers/keras/hstu.py:356-390 with the
-  bias tables expanded): materialises [B, H, L, L], differentiable through everything it reads, any
-  device.  A plain statement of the op for tests and comparisons: no code path of the package calls it
-  (the backward kernels return every gradient, the dense bias's included)."""
-  from recml_amd.hstu_bias import default_bucketization
-  B, L, H, d = q.shape
-  Lkv = k.shape[1]
-  n = L if n is None else n
-  s = alpha * torch.einsum("bihd,bjhd->bhij", q.float(), k.float())
-  i, j = torch.arange(L, device=q.device), torch.arange(Lkv, device=q.device)
-  if pos_bias is not None:
-    pt = pos_bias.float().reshape(-1, 2 * L - 1)
-    s = s + pt[:, (L - 1) + j[None, :] - i[:, None]][None]
-  if ts_bias is not None:
-    tt = ts_bias.float().reshape(-1, ts_bias.shape[-1])
-    ext = torch.cat([timestamps, timestamps[:, L - 1: L]], dim=1)
-    bucket = default_bucketization(ext[:, 1:, None] - ext[:, None, :-1], ts_bucket_size).clamp(0, tt.shape[1] - 1)
-    s = s + tt[:, bucket].transpose(0, 1)
-  if bias is not None:
-    bb = bias.float()
-    s = s + (bb if bb.dim() == 3 else bb[None])[:, None]
-  keep = torch.ones((1, L, Lkv), dtype=torch.bool, device=q.device)
-  if causal:
-    keep = keep & (j[None, None, :] <= i[None, :, None])
-  if sliding_window_size is not None:
-    keep = keep & ((i[None, :, None] - j[None, None, :]).abs() <= int(sliding_window_size))
-  if seq_lens is not None:
-    keep = keep & (i[None, :, None] < seq_lens[:, None, None]) & (j[None, None, :] < seq_lens[:, None, None])
-  if mask is not None:
-    mk = mask != 0
-    keep = keep & (mk if mk.dim() == 3 else mk[None])
-  p = torch.where(keep[:, None], torch.nn.functional.silu(s) / n, torch.zeros((), device=q.device))
-  return torch.einsum("bhij,bjhd->bihd", p, v.float()).to(v.dtype)
 
 
 def pointwise_splash_attention(

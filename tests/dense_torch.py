@@ -1,0 +1,41 @@
+"""The op in plain torch, for tests that compare the package's autograd path against torch's own."""
+
+import torch
+
+
+def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=True, pos_bias=None,
+                          timestamps=None, ts_bias=None, ts_bucket_size=0.301, bias=None, mask=None,
+                          sliding_window_size=None):
+  """The op in plain torch on padded [B, L, H, d] tensors (recml/layers/keras/hstu.py:356-390 with the
+  bias tables expanded): materialises [B, H, L, L], differentiable through everything it reads, any
+  device.  A plain statement of the op for the tests: the package has no such path (its kernels return every
+  gradient, the dense bias's included)."""
+  from recml_amd.hstu_bias import default_bucketization
+  B, L, H, d = q.shape
+  Lkv = k.shape[1]
+  n = L if n is None else n
+  s = alpha * torch.einsum("bihd,bjhd->bhij", q.float(), k.float())
+  i, j = torch.arange(L, device=q.device), torch.arange(Lkv, device=q.device)
+  if pos_bias is not None:
+    pt = pos_bias.float().reshape(-1, 2 * L - 1)
+    s = s + pt[:, (L - 1) + j[None, :] - i[:, None]][None]
+  if ts_bias is not None:
+    tt = ts_bias.float().reshape(-1, ts_bias.shape[-1])
+    ext = torch.cat([timestamps, timestamps[:, L - 1: L]], dim=1)
+    bucket = default_bucketization(ext[:, 1:, None] - ext[:, None, :-1], ts_bucket_size).clamp(0, tt.shape[1] - 1)
+    s = s + tt[:, bucket].transpose(0, 1)
+  if bias is not None:
+    bb = bias.float()
+    s = s + (bb if bb.dim() == 3 else bb[None])[:, None]
+  keep = torch.ones((1, L, Lkv), dtype=torch.bool, device=q.device)
+  if causal:
+    keep = keep & (j[None, None, :] <= i[None, :, None])
+  if sliding_window_size is not None:
+    keep = keep & ((i[None, :, None] - j[None, None, :]).abs() <= int(sliding_window_size))
+  if seq_lens is not None:
+    keep = keep & (i[None, :, None] < seq_lens[:, None, None]) & (j[None, None, :] < seq_lens[:, None, None])
+  if mask is not None:
+    mk = mask != 0
+    keep = keep & (mk if mk.dim() == 3 else mk[None])
+  p = torch.where(keep[:, None], torch.nn.functional.silu(s) / n, torch.zeros((), device=q.device))
+  return torch.einsum("bhij,bjhd->bihd", p, v.float()).to(v.dtype)

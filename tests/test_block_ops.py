@@ -262,6 +262,46 @@ def test_embed_norm_parity(gpu, shape, width, vocab, with_pos, scale):
 
 
 @pytest.mark.gpu
+def test_gemm_silu_takes_views_that_start_off_a_16_byte_boundary(gpu):
+  # dense tensors whose first element sits 2 bytes into an allocation: the wrapper copies them for the library
+  from recml_amd import hstu_block_ops as B
+  gen = torch.Generator().manual_seed(3)
+  dev, bf = "cuda:0", torch.bfloat16
+  M, K, N = 130, 256, 512
+  x = (torch.randn((M, K), generator=gen) * 0.5).to(dev).to(bf)
+  w = (torch.randn((K, N), generator=gen) * 0.05).to(dev).to(bf)
+  res = (torch.randn((M, N), generator=gen) * 0.5).to(dev).to(bf)
+
+  def shifted(t):
+    flat = torch.empty(t.numel() + 1, device=dev, dtype=bf)
+    view = flat[1:].view(t.shape)
+    view.copy_(t)
+    assert view.is_contiguous() and view.data_ptr() % 16 != 0
+    return view
+
+  ref = B.gemm_silu(x, w, None, True, residual=res)
+  assert torch.equal(B.gemm_silu(shifted(x), w, None, True, residual=res), ref)
+  assert torch.equal(B.gemm_silu(x, shifted(w), None, True, residual=res), ref)
+  assert torch.equal(B.gemm_silu(x, w, None, True, residual=shifted(res)), ref)
+
+
+@pytest.mark.gpu
+def test_layer_norm_gradient_width_is_checked_up_front(gpu):
+  from recml_amd import hstu_block_ops as B
+  dev, bf = "cuda:0", torch.bfloat16
+  W = 4096
+  x = torch.randn((3, W), device=dev).to(bf)
+  g, b = torch.ones(W, device=dev, dtype=bf), torch.zeros(W, device=dev, dtype=bf)
+  assert B.layer_norm(x, g, b).shape == (3, W)          # the forward alone takes this width
+  with pytest.raises(ValueError, match="gradient of the layer norm"):
+    B.layer_norm(x.requires_grad_(), g, b)
+  with pytest.raises(ValueError, match="gradient of the layer norm"):
+    B.norm_gate(x, x.detach(), g, b)
+  with torch.no_grad():
+    assert B.norm_gate(x, x, g, b).shape == (3, W)
+
+
+@pytest.mark.gpu
 def test_block_ops_argument_errors(gpu):
   from recml_amd import hstu_block_ops as B
   z = torch.zeros((4, 64), device="cuda:0", dtype=torch.bfloat16)

@@ -110,6 +110,25 @@ def test_model_prepares_once_for_its_blocks(gpu, monkeypatch):
       assert torch.equal(out, ref), jagged
 
 
+def test_model_forward_under_inference_mode(gpu):
+  """torch.inference_mode(): the tensors the model builds for its layers (lengths, offsets, packed timestamps)
+  are inference tensors; the shared preparation takes them, and the output is that of torch.no_grad()."""
+  torch.manual_seed(1)
+  B, L = 5, 256
+  model = recml_amd.HSTU(vocab_size=500, max_positions=L, model_dim=256, num_heads=2, num_layers=2,
+                         dtype=bf, device="cuda:0", add_head=False)
+  ids = torch.randint(0, 500, (B, L), device="cuda:0")
+  lens = torch.tensor([256, 200, 31, 128, 1], device="cuda:0", dtype=torch.int32)
+  pos = torch.randn(2, 2 * L - 1, device="cuda:0") * 0.1
+  for jagged in (False, True):
+    with torch.no_grad():
+      ref = model(ids, seq_lens=lens, pos_bias=pos, jagged=jagged)
+    with torch.inference_mode():
+      out = model(ids, seq_lens=lens, pos_bias=pos, jagged=jagged)
+      again = model(ids.clone(), seq_lens=lens.clone(), pos_bias=pos.clone(), jagged=jagged)    # inference tensors as inputs
+    assert torch.equal(out, ref) and torch.equal(again, ref), jagged
+
+
 def test_layers_share_the_scan_of_a_dense_mask(gpu):
   """The layer-side call with a [B, L, L] mask: the preparation reads the mask for each query tile's range of
   key steps; calls on the same batch reuse it, and a mask edited in place is read again."""

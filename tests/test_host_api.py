@@ -77,3 +77,17 @@ def test_library_bucket_thresholds_equal_the_oracle_law():
     if reach < 256:
       assert (got[reach:] == 2**31 - 1).all()
   assert lib.hstu_attn_bucket_thresholds(C.c_float(-1.0), None, 0) == -4
+
+
+def test_attention_batch_identity_of_inference_tensors():
+  # tensors made under torch.inference_mode() have no version counter: reading it raises
+  from recml_amd.hstu_ops import AttentionBatch
+  with torch.inference_mode():
+    t = torch.arange(5, dtype=torch.int32)
+    a = AttentionBatch._ident(t)
+    assert a == AttentionBatch._ident(t) and a[0] == t.data_ptr()
+  assert AttentionBatch._ident(t) == a                    # read outside the mode as well
+  u = torch.arange(5, dtype=torch.int32)
+  before = AttentionBatch._ident(u)
+  u.add_(1)
+  assert AttentionBatch._ident(u) != before               # ordinary tensors: in-place changes are noticed

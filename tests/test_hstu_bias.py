@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import hstu_oracle as O
+from dense_torch import dense_attention_torch
 from recml_amd import hstu_bias
 
 
@@ -80,7 +81,7 @@ def test_custom_bucketization_keeps_the_table_gradient(gpu):
   def grads(fused):
     saved = hstu_ops.hstu_attention_autograd
     if not fused:
-      hstu_ops.hstu_attention_autograd = lambda q, k, v, **kw: hstu_ops.dense_attention_torch(q, k, v, **kw)
+      hstu_ops.hstu_attention_autograd = lambda q, k, v, **kw: dense_attention_torch(q, k, v, **kw)
     try:
       for p in mod.parameters():
         p.grad = None
@@ -110,7 +111,7 @@ def test_dense_attention_in_plain_torch_equals_the_oracle():
   lens = np.array([L, 7])
   tsw, dense = torch.randn(17), torch.randn(B, L, L) * 0.1
   pos = mod._positional_bias.table(L).detach()
-  got = hstu_ops.dense_attention_torch(q, k, v, seq_lens=torch.from_numpy(lens), pos_bias=pos, timestamps=ts, ts_bias=tsw,
+  got = dense_attention_torch(q, k, v, seq_lens=torch.from_numpy(lens), pos_bias=pos, timestamps=ts, ts_bias=tsw,
                                        bias=dense).numpy()
   want = O.hstu_attention_ref(q.numpy(), k.numpy(), v.numpy(), seq_lens=lens, pos_tab=pos.numpy(), timestamps=ts.numpy(),
                               ts_tab=tsw.numpy(), bias=dense.numpy())

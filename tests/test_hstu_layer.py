@@ -7,6 +7,7 @@ import torch
 
 from oracle import hstu_block_oracle as BO
 from oracle import hstu_oracle as O
+from dense_torch import dense_attention_torch
 
 
 def test_layer_norm_definition_and_torch():
@@ -85,6 +86,48 @@ def _load_block(block, w, dtype):
   name_map = {"output_kernel": "output_kernel", "output_bias": "output_bias"}
   for k, val in w.items():
     getattr(block, name_map.get(k, k)).data = torch.from_numpy(np.asarray(val)).to(device="cuda:0", dtype=dtype)
+
+
+def test_block_with_dropout_refuses_training_mode_on_any_device():
+  # recml/layers/keras/hstu.py:386-387 drops attention weights when training; no kernel here does
+  from recml_amd.hstu_layer import HSTUBlock
+  blk = HSTUBlock(32, 2, dropout=0.1)
+  with pytest.raises(NotImplementedError, match="dropout"):
+    blk(torch.zeros(1, 4, 32), seq_lens=torch.tensor([4], dtype=torch.int32))
+  with pytest.raises(ValueError, match="dropout"):
+    HSTUBlock(32, 2, dropout=1.0)
+
+
+@pytest.mark.gpu
+def test_dropout_rate_refused_in_training_and_ignored_in_eval(gpu):
+  """A block (and a model) with a dropout rate: a training-mode forward raises before any kernel runs; in eval
+  mode, where the reference applies no dropout either, the output is that of a block without a rate."""
+  import recml_amd
+  from recml_amd.hstu_layer import HSTUBlock
+  bf, dev = torch.bfloat16, "cuda:0"
+  B, L, D = 2, 96, 128
+  g = lambda: torch.Generator(device="cpu").manual_seed(4)
+  blk = HSTUBlock(D, 2, dropout=0.2, dtype=bf, device=dev, generator=g())
+  plain = HSTUBlock(D, 2, dropout=0.0, dtype=bf, device=dev, generator=g())
+  x = torch.randn(B, L, D, device=dev).to(bf)
+  lens = torch.tensor([96, 40], device=dev, dtype=torch.int32)
+  assert blk.training
+  with pytest.raises(NotImplementedError, match="dropout"):
+    blk(x, seq_lens=lens)
+  blk.requires_grad_(True)
+  with pytest.raises(NotImplementedError, match="dropout"):
+    blk(x, seq_lens=lens)
+  blk.eval()
+  with torch.no_grad():
+    assert torch.equal(blk(x, seq_lens=lens), plain(x, seq_lens=lens))
+  model = recml_amd.HSTU(vocab_size=50, max_positions=L, model_dim=D, num_heads=2, num_layers=2, dropout=0.1,
+                         dtype=bf, device=dev, add_head=False)
+  ids = torch.randint(0, 50, (B, L), device=dev)
+  with pytest.raises(NotImplementedError, match="dropout"):
+    model(ids, seq_lens=lens)
+  model.eval()
+  with torch.no_grad():
+    assert model(ids, seq_lens=lens).shape == (B, L, D)
 
 
 @pytest.mark.gpu
@@ -354,7 +397,7 @@ def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol)
   def grads(fused):
     saved = hstu_ops.hstu_attention_autograd
     if not fused:
-      hstu_ops.hstu_attention_autograd = lambda q, k, v, **kw: hstu_ops.dense_attention_torch(q, k, v, **kw)
+      hstu_ops.hstu_attention_autograd = lambda q, k, v, **kw: dense_attention_torch(q, k, v, **kw)
     try:
       for t in [x, *blk.parameters()]:
         t.grad = None

@@ -74,12 +74,12 @@ def test_backward_variant_query():
   b.struct_size, b.version = C.sizeof(_lib.HstuAttnBwdArgs), _lib.ABI_VERSION
   b.fwd = _lib.new_args()
   f = b.fwd
-  f.B, f.L, f.Lkv, f.H, f.d_qk, f.d_v = 2, 256, 256, 4, 64, 64
+  f.B, f.L, f.Lkv, f.H, f.d_qk, f.d_v = 2, 1024, 1024, 4, 64, 64
   f.q = f.k = f.v = 0x10000
   f.q_stride_t = f.k_stride_t = f.v_stride_t = f.o_stride_t = 4 * 64
   f.q_stride_h = f.k_stride_h = f.v_stride_h = f.o_stride_h = 64
-  f.q_stride_b = f.k_stride_b = f.v_stride_b = f.o_stride_b = 256 * 4 * 64
-  f.alpha, f.inv_n, f.causal = 1.0, 1.0 / 256, 1
+  f.q_stride_b = f.k_stride_b = f.v_stride_b = f.o_stride_b = 1024 * 4 * 64
+  f.alpha, f.inv_n, f.causal = 1.0, 1.0 / 1024, 1
   f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_BF16
   b.dout = b.dq = b.dk = b.dv = 0x20000
   # bf16 at a matrix-core head dim, but no workspace: the general pair (bf16 products: rows on 16-byte boundaries)
@@ -101,6 +101,13 @@ def test_backward_variant_query():
   f.mask = 0x50000                                                    # an explicit mask does not (the forward would)
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16, bf16 products>"
   f.mask = None
+  # a batch small enough to go without a work list, and no bias table: no workspace to ask for, the matrix cores all the same
+  f.L = f.Lkv = 256
+  f.workspace, f.workspace_bytes = None, 0
+  f.out = 0x30000
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(f)) == 0
+  f.out = None
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
   f.qk_dtype = f.v_dtype = f.out_dtype = _lib.DTYPE_FP32
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<float>"
 
@@ -149,14 +156,22 @@ def test_variant_and_workspace_query():
   a.alpha, a.inv_n, a.causal = 1.0, 1.0 / 256, 1
   a.qk_dtype = a.v_dtype = a.out_dtype = _lib.DTYPE_BF16
   assert lib.hstu_attn_fwd_variant(C.byref(a)) == b"hstu_fwd_mfma_bf16"
-  # the matrix-core kernel always wants a workspace: a work list of one int4 per query tile
-  # (2 sequences x 2 tiles here) behind a 16-byte header and 16 counters behind that ...
+  # a batch this small (one workgroup per sequence, head and query tile fits the chip at once) goes without a work
+  # list: nothing to prepare unless a table comes with it ...
   up = lambda x: (x + 255) // 256 * 256
-  sched = up(16 + 16 * 2 * 2) + up(4 * 16)
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == 0
+  # ... with a position table, its scaled and padded copy
+  a.pos_tab, a.pos_heads = 0x20000, 4
+  assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == up(4 * (2 * 256 - 1 + 512) * 4)
+  a.pos_tab, a.pos_heads = None, 0
+  # a larger batch: a work list of one int4 per query tile (200 sequences x 2 tiles here) behind a 16-byte header
+  # and 16 counters behind that
+  a.B = 200
+  sched = up(16 + 16 * 200 * 2) + up(4 * 16)
   assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == sched
-  # ... plus, with a position table, its scaled and padded copy
   a.pos_tab, a.pos_heads = 0x20000, 4
   assert lib.hstu_attn_fwd_workspace_bytes(C.byref(a)) == up(4 * (2 * 256 - 1 + 512) * 4) + sched
+  a.B = 2
   # longer sequences can have query tiles whose key range is split over workgroups: room for the fp32
   # partial sums of up to 32 chunks per head, their arrival counters, and 32 more list entries
   a.pos_tab, a.pos_heads = None, 0

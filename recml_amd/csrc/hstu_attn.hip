@@ -1852,7 +1852,7 @@ __device__ __forceinline__ int64_t ts_range_slot0(const Params& p, int b, int64_
 // Timestamp descriptors.  The bucket of a pair depends on the sequence's timestamps alone: not on the head, not
 // on the layer.  With sorted timestamps the buckets of one row fall from key to key, and away from the diagonal
 // a step of 32 keys holds one bucket or two for a row.  This kernel works that out once per batch: for every
-// query row and every 32-key step at or below its diagonal one 16-bit word
+// query row and every 32-key step below its 128-row tile's first row one 16-bit word
 //   bits 0..6   bucket b of the step's last key the row keeps (the nearest in time)
 //   bits 7..12  c: the step's first c keys are one bucket further (b + 1), the others in b (0: one bucket)
 //   bit 15      neither holds (three buckets or more, timestamps out of order in the step, a key later than the
@@ -1916,7 +1916,9 @@ __device__ __forceinline__ void ts_desc_block(const Params& p, uint16_t* __restr
   const Seq s = seq_from(p, b, 0, o0, nraw);
   const int q0 = qt * BM;
   if (q0 >= s.rows) return;
-  const int n_steps_tile = (((q0 + BM < s.n_kv ? q0 + BM : s.n_kv) + BN - 1) / BN);   // steps a causal tile can touch
+  // The steps the stream can take: those whose 32 keys every row of the tile keeps (below the tile's first row and
+  // whole inside the sequence).  The tile's diagonal steps go through the block code, which does not read these words.
+  const int n_steps_tile = (q0 < s.n_kv ? q0 : s.n_kv) / BN;
   const int t0 = chunk * TS_DESC_CHUNK;
   if (t0 >= n_steps_tile) return;
   const int t1 = t0 + TS_DESC_CHUNK < n_steps_tile ? t0 + TS_DESC_CHUNK : n_steps_tile;
@@ -1967,44 +1969,47 @@ __device__ __forceinline__ void ts_desc_block(const Params& p, uint16_t* __restr
     return bk < p.ts_nb ? bk : p.ts_nb;
   };
   int my_general = 0x7fffffff;
-  for (int idx = tid; idx < BM * (t1 - t0); idx += 256) {
-    const int r = idx & (BM - 1), tl = idx >> 7, t = t0 + tl;
+  // A thread's four (row, step) pairs side by side and without branches: each is a chain of dependent LDS reads
+  // (two bucket lookups, five steps of bisection), and one after the other they cost the workgroup four times
+  // the chain's latency.  Indices of pairs that do not exist are clamped and their words are not written.
+  constexpr int NIT = BM * TS_DESC_CHUNK / 256;
+  const int n_idx = BM * (t1 - t0);
+#pragma unroll
+  for (int it = 0; it < NIT; ++it) {
+    const int idx = tid + 256 * it;
+    const bool on = idx < n_idx;
+    const int r = idx & (BM - 1), tl = on ? idx >> 7 : 0, t = t0 + tl;
     const int i = q0 + r;
-    uint32_t word = 0u;
     const int j0 = t * BN;
     int j1 = j0 + BN - 1;
     j1 = j1 < s.n_kv - 1 ? j1 : s.n_kv - 1;
     j1 = j1 < i ? j1 : i;                // (the causal mask: later keys are masked whatever their bucket)
-    if (i < s.n_q && j1 >= j0) {
-      const int l0 = tl * BN, l1 = j1 - t0 * BN;     // the step's first key and the row's last, as indices into k_l
-      const int64_t tq = tq_l[r];
-      const int64_t k_first = k_l[l0], k_last = k_l[l1];
-      bool general = sorted_to[tl] < l1 || tq < k_last;
-      if (!general) {
-        const int bn = bucket(tq - k_last), bf = bucket(tq - k_first);
-        if (bf == bn && bn < TS_KEYS) {
-          word = (uint32_t)bn;
-        } else if (bf == bn + 1 && bf < TS_KEYS) {
-          // keys in order: those with tq - ts >= thr, i.e. ts <= tq - thr, are the first c of the step
-          const int64_t cut = tq - (int64_t)thr_b[bf];
-          int lo = l0, hi = l1;        // k[lo] <= cut < k[hi]: the first and last key are on different sides
-          while (hi - lo > 1) {
-            const int mid = (lo + hi) >> 1;
-            if (k_l[mid] <= cut) lo = mid; else hi = mid;
-          }
-          word = (uint32_t)bn | ((uint32_t)(lo + 1 - l0) << 7);
-        } else {
-          general = true;
-        }
-      }
-      if (general) {
-        word = TS_DESC_GENERAL;
-        my_general = t < my_general ? t : my_general;
-      }
+    const bool pair = on && i < s.n_q && j1 >= j0;
+    const int l0 = tl * BN, l1 = pair ? j1 - t0 * BN : l0;     // the step's first key and the row's last, as indices into k_l
+    const int64_t tq = tq_l[r];
+    const int64_t k_first = k_l[l0], k_last = k_l[l1];
+    const bool in_order = sorted_to[tl] >= l1 && tq >= k_last;
+    const int bn = bucket(in_order ? tq - k_last : 0), bf = bucket(in_order ? tq - k_first : 0);
+    const bool one = in_order && bf == bn && bn < TS_KEYS, two = in_order && bf == bn + 1 && bf < TS_KEYS;
+    // keys in order: those with tq - ts >= thr, i.e. ts <= tq - thr, are the first c of the step
+    const int64_t cut = tq - (int64_t)thr_b[bf < TS_KEYS ? bf : TS_KEYS - 1];
+    int lo = l0, hi = l1;                // (when `two`) k[lo] <= cut < k[hi]: the first and last key are on different sides
+#pragma unroll
+    for (int step = 0; step < 5; ++step) {         // l1 - l0 <= 31
+      const int mid = (lo + hi) >> 1;
+      const bool more = hi - lo > 1, left = k_l[mid] <= cut;
+      lo = more && left ? mid : lo;
+      hi = more && !left ? mid : hi;
     }
+    uint32_t word = one ? (uint32_t)bn : ((uint32_t)bn | ((uint32_t)(lo + 1 - l0) << 7));
+    if (pair && !one && !two) {
+      word = TS_DESC_GENERAL;
+      my_general = t < my_general ? t : my_general;
+    }
+    word = pair ? word : 0u;
     // (a tile's last rows may lie past the sequence: those up to the next sequence's first row are this
     // workgroup's to clear, the rest are that sequence's own)
-    if (row0 + i < row_end) desc[(int64_t)t * p.ts_desc_pitch + row0 + i] = (uint16_t)word;
+    if (on && row0 + i < row_end) desc[(int64_t)t * p.ts_desc_pitch + row0 + i] = (uint16_t)word;
   }
   // the chunk's first flagged step, INT32_MAX when it has none: a slot of its own per (tile, chunk), written every time
   if (my_general != 0x7fffffff) atomicMin(&first_general, my_general);
@@ -2048,6 +2053,7 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     __shared__ int keys[SEG], firsts[SEG], order[SEG], tbase[SEG + 1];
     const bool sorted = p.B <= SEG;
     int4* items = (int4*)(sched_out + 4);
+    int walk_first = -1, walk_r = 0;      // memo of `walk` below: the first tile of the thread's run and its sequence
     // sum over the workgroup and exclusive prefix of this thread's value (all 256 threads take part)
     auto block_scan = [&](int v, int& total) {
       int inc = v;
@@ -2101,16 +2107,27 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
         firsts[i] = o0;
       }
       __syncthreads();
-      for (int i = tid; i < cnt; i += 256) {
+      // (the rank of a sequence: how many are longer, or as long and earlier.  A wave takes the lengths 64 at a
+      // time, one per lane, and every lane compares its own with each of them from the lanes' registers: one
+      // LDS read per 64 comparisons)
+      for (int i0 = 0; i0 < cnt; i0 += 256) {
+        const int i = i0 + tid;
         int rank = i;
         if (sorted) {
-          const int kb = keys[i];
+          const int kb = i < cnt ? keys[i] : 0;
           rank = 0;
-#pragma unroll 8
-          for (int c = 0; c < cnt; ++c) rank += (keys[c] > kb || (keys[c] == kb && c < i)) ? 1 : 0;
+          for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int mine = c0 + (tid & 63) < cnt ? keys[c0 + (tid & 63)] : (int)0x80000000;   // (past the end: shorter than any)
+#pragma unroll
+            for (int j = 0; j < 64; ++j) {
+              const int kc = __builtin_amdgcn_readlane(mine, j);
+              rank += (kc > kb || (kc == kb && c0 + j < i)) ? 1 : 0;
+            }
+          }
         }
-        order[rank] = i;
+        if (i < cnt) order[rank] = i;
       }
+      walk_first = -1;            // (the walks' memo of where a thread's run starts belongs to the segment before)
       __syncthreads();
       int c[SEG / 256], sum = 0;
 #pragma unroll
@@ -2146,12 +2163,18 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     // rest follow in order.  fn(i, qt, nq, nk): index of the sequence within the segment, query tile, dimensions.
     auto walk = [&](int cnt, int f_lo, int f_hi, auto&& fn) {
       if (f_lo >= f_hi) return;
-      int lo = 0, hi = cnt;       // the last r with tbase[r] <= f_lo (those before it with the same value have no tiles)
-      while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (tbase[mid] <= f_lo) lo = mid; else hi = mid;
+      // (a thread walks the same run several times over a segment: the bisection, a chain of dependent LDS reads,
+      // is done for the first walk only)
+      if (walk_first != f_lo) {
+        int lo = 0, hi = cnt;     // the last r with tbase[r] <= f_lo (those before it with the same value have no tiles)
+        while (hi - lo > 1) {
+          const int mid = (lo + hi) >> 1;
+          if (tbase[mid] <= f_lo) lo = mid; else hi = mid;
+        }
+        walk_first = f_lo;
+        walk_r = lo;
       }
-      int r = lo;
+      int r = walk_r;
       for (int f = f_lo; f < f_hi;) {
         while (f >= tbase[r + 1]) ++r;
         const int i = order[r], t0 = tbase[r], t1 = tbase[r + 1];

@@ -178,7 +178,7 @@ int hstu_attn_abi_version(void);
  * bf16 under the causal mask one 16-bit descriptor per (query row, step of 32
  * keys) -- the bucket of the step's nearest key and how many of its keys lie one
  * bucket further, or a flag that says the step needs the per-pair lookup --
- * written by a second small kernel (2 bytes x rows x ceil(L/32); left out, and
+ * written by extra workgroups of the same preparation launch, for the steps below each 128-row tile (2 bytes x rows x ceil(L/32); left out, and
  * the per-pair lookup used throughout, for L above 16384, above 256 MiB, or
  * when the buffer is too small for them), for a dense mask the range of key
  * steps in which it keeps anything per tile of 128 query rows (the mask is

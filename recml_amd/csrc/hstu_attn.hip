@@ -115,8 +115,9 @@ struct Params {
   int32_t persist;           // forward: resident workgroups that loop over the work list
   int32_t no_stream;         // forward: interior steps through the compiler-scheduled block code too (a comparison switch)
   // Timestamp descriptors (matrix-core forward at d = 128; null = none): one 16-bit word per (32-key step, query
-  // row), [step][row] with `ts_desc_pitch` rows per step, built by hstu_prepare_ts_desc for every head and layer of
-  // a batch; and per 128-row tile the number of leading quads of steps in which no row needs the per-pair lookup.
+  // row), [step][row] with `ts_desc_pitch` rows per step, built by hstu_prepare (ts_desc_block) for every head and layer of
+  // a batch; and per (128-row tile, chunk of TS_DESC_CHUNK steps) the first step in which some row needs the per-pair
+  // lookup (INT32_MAX: none).
   const uint16_t* ts_desc;
   const int32_t* ts_tquads;
   int32_t ts_desc_pitch;
@@ -2458,7 +2459,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  // TSD: the kernel can take timestamp descriptors (hstu_prepare_ts_desc).  The bias operands of a stage are then
+  // TSD: the kernel can take timestamp descriptors (ts_desc_block in hstu_prepare).  The bias operands of a stage are then
   // [4 x (window copy w | the 32 descriptors of wave w's rows)][key timestamps]: each wave's one bias load brings
   // its window copy and, in the four lanes behind it, its own rows' descriptors.
   constexpr bool TSD = fwd_takes_ts_desc(D, TS, F8, SEG, DENSE);
@@ -3123,7 +3124,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   };
   // ---- The interior steps as one hand-scheduled instruction stream (d = 128 in bf16, no segment ids or dense
   // operands; hstu_fwd_stream_d128.inc, written by gen_fwd_stream.py).  With timestamps it takes each (row, step)'s
-  // bias from the descriptors that hstu_prepare_ts_desc wrote (the bucket of the step's nearest key and how many of
+  // bias from the descriptors that hstu_prepare wrote (the bucket of the step's nearest key and how many of
   // its keys are one bucket further), and only the leading steps in which no row of the tile is flagged.  A step is interior when every key
   // of it is kept for every row of the tile: under the causal mask the steps below the tile's first row, without
   // it those that lie whole inside the sequence.  The stream takes them four at a time from the item's first step

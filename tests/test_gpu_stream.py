@@ -79,19 +79,22 @@ def test_stream_gives_the_bits_of_the_block_code(gpu, walk, name, lens, L, H, po
 
 
 TS_CASES = [
-    # name, lengths, L, H, position table
-    ("one long sequence, timestamps", [2048], 2048, 8, False),
-    ("one long sequence, table + timestamps", [2048], 2048, 8, True),
-    ("mixed lengths, table + timestamps", [2048, 1655, 1000, 777, 513, 512, 511, 385, 384, 256, 129, 128, 127, 16, 1], 2048, 8, True),
-    ("two long sequences (tiles split by keys), table + timestamps", [2048, 2048], 2048, 8, True),
-    ("three sequences, two heads", [2048, 1300, 700], 2048, 2, True),
+    # name, lengths, L, H, position table, jagged
+    ("one long sequence, timestamps", [2048], 2048, 8, False, True),
+    ("one long sequence, table + timestamps", [2048], 2048, 8, True, True),
+    ("mixed lengths, table + timestamps", [2048, 1655, 1000, 777, 513, 512, 511, 385, 384, 256, 129, 128, 127, 16, 1], 2048, 8, True, True),
+    ("two long sequences (tiles split by keys), table + timestamps", [2048, 2048], 2048, 8, True, True),
+    ("three sequences, two heads", [2048, 1300, 700], 2048, 2, True, True),
+    ("padded with lengths, [B, L] timestamps", [1024, 1000, 640, 641, 100], 1024, 4, True, False),
+    ("a small batch (no work list), padded", [512, 300], 512, 2, True, False),
+    ("a small batch (no work list), jagged", [512, 300, 129], 512, 2, False, True),
 ]
 
 
-@pytest.mark.parametrize("name,lens,L,H,pos", TS_CASES, ids=[c[0] for c in TS_CASES])
+@pytest.mark.parametrize("name,lens,L,H,pos,jagged", TS_CASES, ids=[c[0] for c in TS_CASES])
 @pytest.mark.parametrize("walk", ["one item per workgroup", "resident workgroups"])
-def test_stream_with_timestamps_gives_the_bits_of_the_block_code(gpu, walk, name, lens, L, H, pos):
-  q, k, v, kw = _inputs(lens, L, H, pos, True, True, timestamps=True)
+def test_stream_with_timestamps_gives_the_bits_of_the_block_code(gpu, walk, name, lens, L, H, pos, jagged):
+  q, k, v, kw = _inputs(lens, L, H, pos, True, jagged, timestamps=True)
   mode = _lib.FWD_ONE_ITEM_PER_WORKGROUP if walk == "one item per workgroup" else _lib.FWD_RESIDENT_WORKGROUPS
   for _ in range(2):      # (twice: a race between the workgroups that write the descriptors would not show every time)
     ref = _run(q, k, v, mode | _lib.FWD_COMPILER_SCHEDULED_BLOCKS, **kw)
@@ -138,6 +141,20 @@ def test_timestamps_out_of_order_and_wide_spans_with_descriptors(gpu):
   d = np.cumsum(rng.integers(1, 2**24, 640).astype(np.int64)) * 1000
   ts = np.concatenate([a, b, c, d])
   assert _ts_oracle_case(lens, 1024, 2, True, ts, seed=12) <= BF16_TOL
+
+
+def test_stream_with_timestamps_in_the_padded_layout_against_the_oracle(gpu):
+  # [B, L] timestamps (non-decreasing along the whole row, so the padding repeats nothing the rows read), lengths
+  lens, L, H = [1024, 700, 333], 1024, 2
+  q, k, v, kw = _inputs(lens, L, H, True, True, False, timestamps=True, seed=9)
+  got = _run(q, k, v, 0, **kw).float().cpu().numpy()
+  f = lambda t: t.float().cpu().numpy()
+  ref = O.hstu_attention_ref(f(q), f(k), f(v), seq_lens=np.asarray(lens), n=L, pos_tab=kw["pos_bias"].cpu().numpy(),
+                             timestamps=kw["timestamps"].cpu().numpy(), ts_tab=kw["ts_bias"].cpu().numpy())
+  err = np.abs(got - ref).max() / np.abs(ref).max()
+  assert err <= BF16_TOL, err
+  for b, n in enumerate(lens):
+    assert not got[b, n:].any()          # rows past a sequence's end: exactly 0
 
 
 @pytest.mark.parametrize("pos", [False, True])

@@ -570,7 +570,7 @@ def bench_backward(args, w, q, k, v, kw, dev):
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
       "dtype": "bf16" if (mfma or "bf16 products" in variant[-1]) else ("f32" if w.dtype == "fp32" else "bf16 storage, fp32 arithmetic"),
       "data": "synthetic",
-      "config": {"workload": w.name + " backward",
+      "config": {"workload": w.name + " backward" + (f" dropout={args.dropout}" if args.dropout > 0 else ""),
                  "kernel": "hstu_bwd_dq_mfma + hstu_bwd_dkv_mfma" if mfma else
                            ("hstu_bwd_dq_mm + hstu_bwd_dkv_mm" if w.d <= 128 else "hstu_bwd_dq + hstu_bwd_dkv")},
       "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
@@ -635,6 +635,9 @@ def main():
                   help="diagnostics: force resident workgroups that loop over the work list")
   ap.add_argument("--compiler-scheduled-blocks", action="store_true",
                   help="diagnostics: interior steps through the compiler-scheduled block code instead of the hand-scheduled stream")
+  ap.add_argument("--dropout", type=float, default=0.0,
+                  help="diagnostics: the training form with this dropout rate on the attention weights (not the contract's "
+                       "workload; the CPU leg is skipped, tests/test_gpu_dropout.py holds its parity)")
   ap.add_argument("--ramp-ms", type=float, default=300.0,
                   help="untimed calls for this long before anything is measured (clock ramp from idle)")
   ap.add_argument("--no-tuned-products", dest="tuned", action="store_false",
@@ -662,6 +665,9 @@ def main():
     return bench_dense(args, dev)
   w = make_workload(args.workload)
   q, k, v, kw = to_device(w, dev)
+  if args.dropout > 0:
+    kw.update(dropout_p=args.dropout, dropout_seed=1)
+    args.no_cpu = True
   if args.fp32:
     if w.dtype == "fp8":
       raise SystemExit("--fp32 goes with the bf16 workloads")
@@ -806,7 +812,8 @@ def main():
       "config": {"workload": f"{w.name}: B={w.B} max_len={w.L} H={w.H} d={w.d} {w.layout} "
                              f"lens mean {w.seq_lens.mean():.0f} max {w.seq_lens.max()}, causal, "
                              f"pos_bias={'yes' if w.pos_tab is not None else 'no'} "
-                             f"ts_bias={'yes' if w.ts_tab is not None else 'no'} N={w.n} alpha={w.alpha}",
+                             f"ts_bias={'yes' if w.ts_tab is not None else 'no'} N={w.n} alpha={w.alpha}"
+                             + (f" dropout={args.dropout}" if args.dropout > 0 else ""),
                  "kernel": variant},
       "seqs_per_s": w.B / (ms_per_step * 1e-3),
       "timed_call": "hstu_attn_fwd, self-contained: every call runs the preparation kernel and the main kernel (value, "

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HSTU_ATTN_ABI_VERSION 2
+#define HSTU_ATTN_ABI_VERSION 3
 
 /* Tensor layouts of q, k, v, out. */
 enum HstuLayout {
@@ -163,7 +163,25 @@ typedef struct HstuAttnFwdArgs {
 
   void* workspace;        /* device scratch of hstu_attn_fwd_workspace_bytes  */
   size_t workspace_bytes;
+
+  /* Dropout on the attention weights (the training-mode step of
+   * recml/layers/keras/hstu.py:386-387): each kept pair (b, h, i, j) is dropped
+   * with probability dropout_p and the others are scaled by 1 / (1 - dropout_p).
+   * Which pairs go is a function of (dropout_seed, b, h, i, j) alone -- a
+   * counter-based hash, hstu_attn_dropout_keep below -- so the backward, given
+   * the same two values, drops the same pairs, and a caller can reproduce the
+   * mask.  0 (the default) switches it off.  With dropout the matrix-core
+   * kernel runs every step through its compiler-scheduled block code. */
+  float dropout_p;        /* in [0, 1)                                        */
+  uint32_t reserved0;     /* 0                                                */
+  uint64_t dropout_seed;
 } HstuAttnFwdArgs;
+
+/* Whether dropout keeps pair (query i, key j) of sequence b and head h (of H
+ * heads): the rule every kernel follows, as a host function for callers and
+ * checkers.  i and j count from the start of the sequence.  Always 1 for
+ * dropout_p = 0. */
+int hstu_attn_dropout_keep(uint64_t dropout_seed, float dropout_p, int32_t b, int32_t h, int32_t H, int32_t i, int32_t j);
 
 /* ABI version of the loaded library (HSTU_ATTN_ABI_VERSION at build time). */
 int hstu_attn_abi_version(void);

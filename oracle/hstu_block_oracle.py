@@ -52,9 +52,10 @@ def layer_norm(x, gamma, beta, eps, axes=(-1,)):
 
 
 def hstu_block(x, w, *, num_heads, seq_lens, eps=1e-6, scaled_pointwise_attn=False,
-               pos_tab=None, timestamps=None, ts_tab=None):
+               pos_tab=None, timestamps=None, ts_tab=None, dropout_p=0.0, dropout_seed=0):
   """x [B, L, D]; w: dict with u/q/k/v_kernel [D,H,hd], output_kernel [H,hd,D],
-  input_ln_gamma/beta [D], attn_ln_gamma/beta [H,hd], optional *_bias."""
+  input_ln_gamma/beta [D], attn_ln_gamma/beta [H,hd], optional *_bias.  dropout_p > 0: the
+  block in training mode (dropout on the attention weights, hstu.py:386-387)."""
   x = np.asarray(x, dtype=np.float64)
   B, L, D = x.shape
   H = num_heads
@@ -74,7 +75,8 @@ def hstu_block(x, w, *, num_heads, seq_lens, eps=1e-6, scaled_pointwise_attn=Fal
     tb = O.time_bias(np.asarray(timestamps), np.asarray(ts_tab, np.float64).reshape(-1))
     bias = tb if bias is None else bias + tb
   attn = O.pointwise_attention_dense(proj["q"], proj["k"], proj["v"], mask, bias,
-                                     scaled=scaled_pointwise_attn)
+                                     scaled=scaled_pointwise_attn, dropout_p=dropout_p,
+                                     dropout_seed=dropout_seed)
   na = layer_norm(attn, f("attn_ln_gamma"), f("attn_ln_beta"), eps, axes=(-2, -1))
   out = np.einsum("btnh,nhd->btd", proj["u"] * na, f("output_kernel"))
   if "output_bias" in w:

@@ -19,6 +19,11 @@ reference checkout):
   splash_mask                   recml/core/ops/hstu_ops.py:926-945, 107-194
   hstu_attention_ref            the union of the above behind one signature
   hstu_attention_bwd_ref        its gradients; math of recml/core/ops/hstu_ops.py:461-517
+  dropout_keep_mask             which weights survive attention dropout
+                                (recml/layers/keras/hstu.py:386-387 applies keras'
+                                Dropout to the masked weights: survivors are
+                                scaled by 1/(1-rate)); the draw itself is this
+                                library's counter-based hash, not keras' generator
 
 How each function is pinned (tests/test_oracle.py):
 
@@ -39,6 +44,14 @@ How each function is pinned (tests/test_oracle.py):
   round_e4m3fn / encode_e4m3fn  torch's CPU float8_e4m3fn cast on every code
                                 point, every midpoint and random values (fp8
                                 is not in the reference at all).
+  dropout_keep_mask             the integer hash against known answers worked
+                                with Python's unbounded integers, rate 0 and the
+                                survivors' share; hstu_attention_ref with dropout
+                                by its mean over many seeds (the undropped
+                                output) and by brute force over the keep mask.
+                                The random stream itself is parity unpinned by
+                                nature: the reference draws from keras' seed
+                                generator and holds no dropout outputs.
   splash_mask with sliding_window_size  parity unpinned: the window rule
                                 (|i-j| <= w) comes from jax's splash-attention
                                 LocalMask, which is not vendored in the
@@ -279,8 +292,10 @@ def silu(x):
 
 
 def pointwise_attention_dense(q, k, v, attention_mask, attention_bias=None,
-                              scaled: bool = False, dtype=np.float64):
-  """recml/layers/keras/hstu.py:356-390 (inference: no dropout).
+                              scaled: bool = False, dtype=np.float64,
+                              dropout_p: float = 0.0, dropout_seed: int = 0):
+  """recml/layers/keras/hstu.py:356-390; dropout_p > 0 is its training form
+  (:386-387): the masked weights times dropout_keep_mask / (1 - dropout_p).
 
   q,k,v [B,L,H,d]; attention_mask [B,L,Lkv] (non-zero = keep);
   attention_bias [B or 1,L,Lkv] broadcast over heads.
@@ -298,6 +313,9 @@ def pointwise_attention_dense(q, k, v, attention_mask, attention_bias=None,
     p = p / q.shape[1]
   keep = np.asarray(attention_mask).astype(bool)[:, None]
   p = np.where(keep, p, np.zeros_like(p))
+  if dropout_p > 0:
+    B, H, L, Lkv = p.shape
+    p = p * _dropout_factor(dropout_p, dropout_seed, B, H, L, Lkv, 0, dtype)
   return np.einsum("bhts,bshd->bthd", p, v)
 
 
@@ -342,11 +360,78 @@ def _bias_term(L, Lkv, H, pos_tab, timestamps, ts_tab, ts_bucket_size, law):
   return bias
 
 
+# ---------------------------------------------------------------------------
+# Attention dropout: which (b, h, i, j) survive
+# ---------------------------------------------------------------------------
+
+_U32 = np.uint64(0xFFFFFFFF)
+DROP_CI = 0x85EBCA77
+DROP_CJ = 0xC2B2AE3D
+
+
+def _u32(x):
+  return np.asarray(x, dtype=np.uint64) & _U32
+
+
+def dropout_threshold(p: float) -> int:
+  """round(p * 2^32), 0 for p <= 0, capped at 2^32 - 1: a pair is dropped when its hash is below it."""
+  t = float(np.float32(p)) * 4294967296.0
+  if t <= 0.0:
+    return 0
+  return 0xFFFFFFFF if t >= 4294967295.0 else int(t + 0.5)
+
+
+def dropout_seed_key(seed: int) -> int:
+  """Folds a 64-bit seed into 32 bits (two rounds of xor-shift and multiply)."""
+  seed = int(seed) & 0xFFFFFFFFFFFFFFFF
+  z = (seed & 0xFFFFFFFF) ^ 0x9E3779B9
+  z = ((z ^ (z >> 16)) * 0x85EBCA6B) & 0xFFFFFFFF
+  z ^= seed >> 32
+  z = ((z ^ (z >> 13)) * 0xC2B2AE35) & 0xFFFFFFFF
+  return z ^ (z >> 16)
+
+
+def dropout_hash(seed: int, B: int, H: int, L: int, Lkv: int, b0: int = 0, rows=None, cols=None):
+  """uint32 [B, H, L, Lkv]: hash(b, h, i, j) = mix(bhkey(seedkey, (b0 + b) * H + h) + i * CI + j * CJ), all in
+  wrapping 32-bit arithmetic (bhkey: one multiply-add and one xor-shift-multiply round; mix: two rounds).
+  `rows` / `cols`: the query / key indices to evaluate instead of all of range(L) / range(Lkv)."""
+  key = np.uint64(dropout_seed_key(seed))
+  bh = _u32((np.arange(b0, b0 + B, dtype=np.uint64)[:, None] * np.uint64(H)
+             + np.arange(H, dtype=np.uint64)[None, :]))
+  z = _u32(key + _u32(bh * np.uint64(0x9E3779B1)))
+  z = _u32((z ^ (z >> np.uint64(15))) * np.uint64(0x2C1B3C6D))
+  kbh = z ^ (z >> np.uint64(13))                                             # [B, H]
+  i = _u32(np.asarray(range(L) if rows is None else rows, dtype=np.uint64) * np.uint64(DROP_CI))
+  j = _u32(np.asarray(range(Lkv) if cols is None else cols, dtype=np.uint64) * np.uint64(DROP_CJ))
+  ij = _u32(kbh[:, :, None, None] + i[None, None, :, None] + j[None, None, None, :])
+  z = _u32((ij ^ (ij >> np.uint64(15))) * np.uint64(0x2C1B3C6D))
+  z = _u32((z ^ (z >> np.uint64(12))) * np.uint64(0x297A2D39))
+  return (z ^ (z >> np.uint64(15))).astype(np.uint32)
+
+
+def dropout_keep_mask(seed: int, p: float, B: int, H: int, L: int, Lkv: int, b0: int = 0):
+  """bool [B, H, L, Lkv]: True where the weight of (sequence b0 + b, head h, query i, key j) survives:
+  dropout_hash >= dropout_threshold(p).  With p == 0 everything survives."""
+  thr = dropout_threshold(p)
+  if thr == 0:
+    return np.ones((B, H, L, Lkv), dtype=bool)
+  return dropout_hash(seed, B, H, L, Lkv, b0) >= np.uint32(thr)
+
+
+def _dropout_factor(p, seed, B, H, L, Lkv, b0, dtype):
+  """[B, H, L, Lkv] factor on the masked weights: 0 for a dropped pair, 1 / (1 - p) for a survivor (the
+  scale in fp32, as the library's host code forms it)."""
+  keep = dropout_keep_mask(seed, p, B, H, L, Lkv, b0)
+  scale = float(np.float32(1.0) / (np.float32(1.0) - np.float32(p)))
+  return np.where(keep, scale, 0.0).astype(dtype)
+
+
 def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
                        causal=True, pos_tab=None, timestamps=None,
                        ts_tab=None, ts_bucket_size=0.301, bucket_law=True,
                        q_segment_ids=None, kv_segment_ids=None,
                        sliding_window_size=None, mask=None, bias=None,
+                       dropout_p=0.0, dropout_seed=0, dropout_b0=0,
                        dtype=np.float64):
   """Dense restatement of the whole op on padded [B,L,H,d] inputs.
 
@@ -360,6 +445,9 @@ def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
   reproduce recml/core/ops/hstu_ops_test.py:44-58.
   `mask` is an explicit [L,Lkv] or [B,L,Lkv] keep-mask, `bias` a dense
   [B or 1,L,Lkv] additive term shared by all heads (hstu.py:373-374).
+  `dropout_p` > 0 is the training form (hstu.py:386-387): the masked weights
+  times dropout_keep_mask(dropout_seed, ...) / (1 - dropout_p); `dropout_b0` is
+  the index of the batch's first sequence in that mask.
   """
   q = np.asarray(q, dtype=dtype)
   k = np.asarray(k, dtype=dtype)
@@ -394,6 +482,8 @@ def hstu_attention_ref(q, k, v, *, seq_lens=None, n=None, alpha=1.0,
     vk = np.arange(Lkv)[None, :] < lens[:, None]
     m = m & (vq[:, :, None] & vk[:, None, :])
   p = np.where(m[:, None], p, np.zeros_like(p))
+  if dropout_p > 0:
+    p = p * _dropout_factor(dropout_p, dropout_seed, B, H, L, Lkv, dropout_b0, dtype)
   # Keys beyond the sequence never contribute, whatever the padding holds.
   return np.einsum("bhts,bshd->bthd", p, v)
 
@@ -403,7 +493,8 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
                            ts_tab=None, ts_bucket_size=0.301, bucket_law=True,
                            q_segment_ids=None, kv_segment_ids=None,
                            sliding_window_size=None, mask=None, bias=None,
-                           bias_grad=False, dtype=np.float64):
+                           bias_grad=False, dropout_p=0.0, dropout_seed=0,
+                           dropout_b0=0, dtype=np.float64):
   """Gradients of sum(out * dout) for hstu_attention_ref, dense, on padded inputs.
 
   The math of the reference's backward kernel (recml/core/ops/hstu_ops.py:461-517):
@@ -415,6 +506,7 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
   dts_tab (or None) with the shapes of the inputs; with bias_grad=True also the gradient
   of the dense `bias` (dS summed over the heads, and over the batch when the bias is
   shared by it: jax's derivative of recml/layers/keras/hstu.py:373-374), shaped like it.
+  With dropout the factor of the forward (0, or 1 / (1 - dropout_p)) multiplies P and dS alike.
   """
   q = np.asarray(q, dtype=dtype)
   k = np.asarray(k, dtype=dtype)
@@ -450,9 +542,14 @@ def hstu_attention_bwd_ref(q, k, v, dout, *, seq_lens=None, n=None, alpha=1.0,
   m = np.broadcast_to(m, (B, L, Lkv))[:, None]
   sg = 1.0 / (1.0 + np.exp(-s))
   p = np.where(m, s * sg / n, 0.0)
+  if dropout_p > 0:
+    fac = _dropout_factor(dropout_p, dropout_seed, B, H, L, Lkv, dropout_b0, dtype)
+    p = p * fac
   dv = np.einsum("bhts,bthd->bshd", p, dout)
   dp = np.einsum("bthd,bshd->bhts", dout, v)
   ds = np.where(m, dp * sg * (1.0 + s * (1.0 - sg)) / n, 0.0)
+  if dropout_p > 0:
+    ds = ds * fac
   dq = alpha * np.einsum("bhts,bshd->bthd", ds, k)
   dk = alpha * np.einsum("bhts,bthd->bshd", ds, q)
   dpos = dts = None
@@ -627,6 +724,7 @@ def hstu_attention_jagged_ref(q, k, v, seq_offsets, max_len, *, n=None,
                               alpha=1.0, causal=True, pos_tab=None,
                               timestamps=None, ts_tab=None,
                               ts_bucket_size=0.301, bucket_law=True,
+                              dropout_p=0.0, dropout_seed=0,
                               dtype=np.float64, sequences=None):
   """The op on jagged [T,H,d] inputs, one sequence at a time.
 
@@ -659,5 +757,6 @@ def hstu_attention_jagged_ref(q, k, v, seq_offsets, max_len, *, n=None,
         q[s:e][None], np.asarray(k)[s:e][None], np.asarray(v)[s:e][None],
         n=n, alpha=alpha, causal=causal, pos_tab=sub_pos, timestamps=ts,
         ts_tab=ts_tab, ts_bucket_size=ts_bucket_size, bucket_law=bucket_law,
+        dropout_p=dropout_p, dropout_seed=dropout_seed, dropout_b0=b,
         dtype=dtype)[0]
   return out

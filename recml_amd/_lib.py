@@ -9,7 +9,7 @@ import threading
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("RECML_AMD_LIB") or os.path.join(_HERE, "lib", "libhstu_attn.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 LAYOUT_PADDED, LAYOUT_JAGGED = 0, 1
 DTYPE_FP32, DTYPE_BF16, DTYPE_FP8_E4M3FN = 0, 1, 2
@@ -31,6 +31,7 @@ EXPORTS = (
     "hstu_attn_bwd",
     "hstu_attn_bwd_variant",
     "hstu_attn_bucket_thresholds",
+    "hstu_attn_dropout_keep",
 )
 
 
@@ -65,6 +66,7 @@ class HstuAttnFwdArgs(C.Structure):
       ("ts_num_buckets", C.c_int32), ("ts_bucket_size", C.c_float),
       ("q_scale", C.c_void_p), ("k_scale", C.c_void_p),
       ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+      ("dropout_p", C.c_float), ("reserved0", C.c_uint32), ("dropout_seed", C.c_uint64),
   ]
 
 
@@ -117,6 +119,8 @@ def load():
     lib.hstu_attn_bwd_variant.argtypes = [C.POINTER(HstuAttnBwdArgs)]
     lib.hstu_attn_bucket_thresholds.restype = C.c_int
     lib.hstu_attn_bucket_thresholds.argtypes = [C.c_float, C.POINTER(C.c_int32), C.c_int]
+    lib.hstu_attn_dropout_keep.restype = C.c_int
+    lib.hstu_attn_dropout_keep.argtypes = [C.c_uint64, C.c_float, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_int32]
     ver = lib.hstu_attn_abi_version()
     if ver != ABI_VERSION:
       raise RuntimeError(f"libhstu_attn.so has ABI {ver}, expected {ABI_VERSION}")

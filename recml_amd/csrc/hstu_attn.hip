@@ -114,6 +114,9 @@ struct Params {
   const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
   int32_t no_stream;         // forward: interior steps through the compiler-scheduled block code too (a comparison switch)
+  // Dropout on the attention weights: pair (b, h, i, j) is kept when drop_hash(...) >= drop_thr (0: no dropout).
+  // The survivors' scale 1 / (1 - p) is folded into inv_n by the host.
+  uint32_t drop_thr, drop_key;
   // Timestamp descriptors (matrix-core forward at d = 128; null = none): one 16-bit word per (32-key step, query
   // row), [step][row] with `ts_desc_pitch` rows per step, built by hstu_prepare (ts_desc_block) for every head and layer of
   // a batch; and per (128-row tile, chunk of TS_DESC_CHUNK steps) the first step in which some row needs the per-pair
@@ -395,6 +398,58 @@ __device__ __forceinline__ void general_dense_col(const Params& p, int b, int i0
     v[r] = col[(int64_t)(i < p.L - 1 ? i : p.L - 1) * p.Lkv];
   }
 }
+// Dropout's keep rule: a counter-based hash of (seed, b, h, i, j), the same on the host, in every kernel and in
+// the CPU oracle.  drop_seed_key folds the 64-bit seed (host, once per call), drop_bh_key the sequence and the
+// head (once per work item), drop_keep the pair: two multiply-add steps on the indices, of which a kernel hoists
+// the one that is fixed for its lane, and two rounds of xor-shift and multiply.
+__host__ __device__ inline uint32_t drop_seed_key(uint64_t seed) {
+  uint32_t z = (uint32_t)seed ^ 0x9E3779B9u;
+  z = (z ^ (z >> 16)) * 0x85EBCA6Bu;
+  z ^= (uint32_t)(seed >> 32);
+  z = (z ^ (z >> 13)) * 0xC2B2AE35u;
+  return z ^ (z >> 16);
+}
+__host__ __device__ inline uint32_t drop_bh_key(uint32_t key, uint32_t bh) {
+  uint32_t z = key + bh * 0x9E3779B1u;
+  z = (z ^ (z >> 15)) * 0x2C1B3C6Du;
+  return z ^ (z >> 13);
+}
+constexpr uint32_t DROP_CI = 0x85EBCA77u, DROP_CJ = 0xC2B2AE3Du;
+// ij = kbh + i * DROP_CI + j * DROP_CJ (wrapping)
+__host__ __device__ inline bool drop_keep_mixed(uint32_t ij, uint32_t thr) {
+  uint32_t z = (ij ^ (ij >> 15)) * 0x2C1B3C6Du;
+  z = (z ^ (z >> 12)) * 0x297A2D39u;
+  return (z ^ (z >> 15)) >= thr;
+}
+__host__ __device__ inline bool drop_keep(uint32_t kbh, uint32_t i, uint32_t j, uint32_t thr) {
+  return drop_keep_mixed(kbh + i * DROP_CI + j * DROP_CJ, thr);
+}
+// The 16 values a lane holds in a 32 x 32 block sit at offsets c(r) = 8 (r / 4) + r % 4 along the axis that is not the
+// lane's own: ij0 carries everything else, `step` is that axis's multiplier.  One value after the other on purpose (the
+// scheduling barrier): sixteen hashes in flight at once would cost the kernels around this forty registers on a path
+// that inference and most training never take.
+__device__ __forceinline__ void drop_apply16(float (&x)[16], uint32_t ij0, uint32_t step, uint32_t thr) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    x[r] = drop_keep_mixed(ij0 + (uint32_t)(8 * (r >> 2) + (r & 3)) * step, thr) ? x[r] : 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+__device__ __forceinline__ void drop_apply16(float (&x)[16], float (&y)[16], uint32_t ij0, uint32_t step, uint32_t thr) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const bool keep = drop_keep_mixed(ij0 + (uint32_t)(8 * (r >> 2) + (r & 3)) * step, thr);
+    x[r] = keep ? x[r] : 0.f;
+    y[r] = keep ? y[r] : 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+// p in [0, 1) -> the threshold on the 32-bit hash: a pair is dropped with probability thr / 2^32
+__host__ inline uint32_t drop_threshold(float p) {
+  const double t = (double)p * 4294967296.0;
+  return t <= 0.0 ? 0u : (t >= 4294967295.0 ? 0xffffffffu : (uint32_t)(t + 0.5));
+}
+
 // pair (i, j) under the segment ids alone (SEGMENT mode)
 __device__ __forceinline__ bool general_same_segment(const Params& p, int b, int i, int j) {
   return p.q_seg[(int64_t)b * p.L + i] == p.kv_seg[(int64_t)b * p.Lkv + j];
@@ -696,11 +751,14 @@ __global__ __launch_bounds__(256, DMAX <= 128 ? 2 : 1) void hstu_fwd_general(con
       if (qi >= s.n_q) hi = -1;
       const bool by_seg = p.mask_mode == HSTU_MASK_SEGMENT;
       const bool tabled = TAB && (p.pos_tab != nullptr || p.ts_tab != nullptr);
+      // (dropout: the part of the pair's hash that this lane's row fixes)
+      const uint32_t drop_row = drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h) + (uint32_t)qi * DROP_CI;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
         bool keep = j >= lo && j <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
         if (by_seg) keep = keep && general_same_segment(p, b, qi, j);
+        if (p.drop_thr) keep = keep && drop_keep_mixed(drop_row + (uint32_t)j * DROP_CJ, p.drop_thr);
         float x = p.alpha * sacc[r];
         if (tabled && keep) x += general_table_bias(p, s, b, h, qi, j);
         if constexpr (DENSE_AHEAD) {
@@ -754,6 +812,7 @@ __device__ __forceinline__ float bwd_pair(const Params& p, const Seq& s, int b, 
                                           float qk, float dp, float* pout, int* bucket) {
   *pout = 0.f;
   if (!general_keep(p, s, b, i, j)) return 0.f;
+  if (p.drop_thr && !drop_keep(drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h), (uint32_t)i, (uint32_t)j, p.drop_thr)) return 0.f;
   const float x = p.alpha * qk + general_bias(p, s, b, h, i, j, bucket);
   const float sg = 1.0f / (1.0f + expf(-x));
   *pout = x * sg * p.inv_n;
@@ -1346,6 +1405,7 @@ __global__ __launch_bounds__(256, (BP && !TAB) ? 2 : 1) void hstu_bwd_dq_mm(cons
         const int j = kv0 + 8 * (r >> 2) + 4 * hh + (r & 3);
         bool keep = j >= lo && j <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
         if (by_seg) keep = keep && general_same_segment(p, b, qi, j);
+        if (p.drop_thr) keep = keep && drop_keep(drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h), (uint32_t)qi, (uint32_t)j, p.drop_thr);
         float x = p.alpha * sacc[r];
         int bk = 0;
         if (tabled && keep) x += general_table_bias(p, s, b, h, qi, j, &bk);
@@ -1533,6 +1593,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_mm(const Params p) {
         const int i = i0 + 8 * (r >> 2) + 4 * hh + (r & 3);
         bool keep = i >= lo && i <= hi && ((mw[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0u;
         if (by_seg) keep = keep && general_same_segment(p, b, i, kj);
+        if (p.drop_thr) keep = keep && drop_keep(drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h), (uint32_t)i, (uint32_t)kj, p.drop_thr);
         float x = p.alpha * sacc[r];
         if (tabled && keep) x += general_table_bias(p, s, b, h, i, kj);
         if (p.dense_bias) x += db[r];
@@ -2697,6 +2758,7 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
   struct { int n_q, n_kv, rows, n_ts; } s;       // of the item's sequence
   int h = 0, q0 = 0, r0 = 0, qrow = 0, wave_last = -1, nt = 0, t_lo = 0, n_chunks = 1, chunk = 0, pslot = 0, ts32 = 0;
   int has_desc = 0, desc_first = 0x7fffffff;   // descriptors at hand; per lane, a chunk's first step with a flagged row
+  uint32_t drop_thr = 0u, drop_kbh = 0u;       // dropout: the threshold (0: off) and the item's (sequence, head) key
   float alpha2 = 0.f;
   const int64_t* tsg = nullptr;
   bf16_t* og = nullptr;
@@ -2727,6 +2789,8 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
         desc_first = pf.ts_tquads[(ts_desc_tile0(pf.jagged, pf.n_qtiles, k.b, k.s.tok0) + k.qt) * pf.ts_desc_chunks + lane];
     }
     og = (bf16_t*)pf.out + k.s.bo;
+    drop_thr = pf.drop_thr;
+    drop_kbh = drop_thr ? drop_bh_key(pf.drop_key, (uint32_t)k.b * (uint32_t)pf.H + (uint32_t)k.h) : 0u;
   };
   // the head's bucket table: three direct loads of up to 1 KB, one each by waves 0 to 2 (the last wave repeats the first)
   auto load_ts_table = [&](int head) {
@@ -2950,6 +3014,10 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
     if (DENSE & 2) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) u[r] = ((mbits[r >> 2] >> (8 * (r & 3))) & 0xffu) ? u[r] : 0.f;
+    }
+    if (drop_thr) {
+      // dropout: a dropped pair is one more masked logit (the survivors' scale is in the output scale)
+      drop_apply16(u, drop_kbh + (uint32_t)qrow * DROP_CI + (uint32_t)(kbs + 4 * hh) * DROP_CJ, DROP_CJ, drop_thr);
     }
     // SiLU and P V in two halves of 8 keys, each in four phases of 8 independent operations with the order
     // fixed by scheduling barriers: left to itself under register pressure, the compiler has run the 16
@@ -3907,6 +3975,11 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         ds[4 * g + 3] = ks4.w == qseg ? ds[4 * g + 3] : 0.f;
       }
     }
+    if (p.drop_thr) {
+      // dropout: the pairs the forward dropped carry no gradient
+      drop_apply16(ds, drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h) + (uint32_t)qrow * DROP_CI +
+                           (uint32_t)(kbs + 4 * hh) * DROP_CJ, DROP_CJ, p.drop_thr);
+    }
     if (want_dpos) {
       // Pair (row m, key offset c = 8g + 4hh + tt) lies on diagonal c - m.  Lane j takes, for each of
       // its 16 offsets, the value of row (j + c) mod 32 of its half: all 16 are then on diagonal -j or,
@@ -4415,6 +4488,11 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
         pv[4 * g + 3] = k3 ? pv[4 * g + 3] : 0.f;  ds[4 * g + 3] = k3 ? ds[4 * g + 3] : 0.f;
       }
     }
+    if (p.drop_thr) {
+      // dropout: register r holds row qbs + 4hh + c(r) of this lane's key
+      drop_apply16(pv, ds, drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h) + (uint32_t)kcol * DROP_CJ +
+                               (uint32_t)(qbs + 4 * hh) * DROP_CI, DROP_CI, p.drop_thr);
+    }
 #pragma unroll
     for (int cc = 0; cc < 2; ++cc) {
       uint4 pk, dk4;
@@ -4584,6 +4662,8 @@ int validate(const HstuAttnFwdArgs* a) {
   constexpr uint32_t known_flags = HSTU_FWD_WORKSPACE_PREPARED | HSTU_FWD_PREPARE_ONLY | HSTU_FWD_ONE_ITEM_PER_WORKGROUP |
                                    HSTU_FWD_RESIDENT_WORKGROUPS | HSTU_FWD_COMPILER_SCHEDULED_BLOCKS;
   if ((uint32_t)a->flags & ~known_flags) return fail(HSTU_ERR_SHAPE, "unknown bits in flags: 0x%x", (unsigned)a->flags);
+  if (!(a->dropout_p >= 0.0f && a->dropout_p < 1.0f)) return fail(HSTU_ERR_SHAPE, "dropout_p must be in [0, 1), got %g", (double)a->dropout_p);
+  if (a->reserved0 != 0u) return fail(HSTU_ERR_SHAPE, "reserved0 must be 0");
   const bool empty = a->B == 0 || (a->layout == HSTU_LAYOUT_JAGGED && a->total_tokens == 0);
   if (!empty && (!a->q || !a->k || !a->v || !a->out))
     return fail(HSTU_ERR_NULL, "q, k, v and out must be non-null");
@@ -4747,6 +4827,9 @@ Params make_params(const HstuAttnFwdArgs* a) {
   p.ts_nb = a->ts_num_buckets;
   p.ts_bucket_size = a->ts_bucket_size;
   p.alpha = a->alpha; p.inv_n = a->inv_n;
+  p.drop_thr = drop_threshold(a->dropout_p);
+  p.drop_key = drop_seed_key(a->dropout_seed);
+  if (p.drop_thr) p.inv_n = a->inv_n / (1.0f - a->dropout_p);     // the survivors' scale rides on 1 / N
   p.q_scale = a->q_scale; p.k_scale = a->k_scale;
   p.n_qtiles = (a->L + BM - 1) / BM;
   return p;
@@ -5155,6 +5238,13 @@ extern "C" {
 
 int hstu_attn_abi_version(void) { return HSTU_ATTN_ABI_VERSION; }
 
+int hstu_attn_dropout_keep(uint64_t dropout_seed, float dropout_p, int32_t b, int32_t h, int32_t H, int32_t i, int32_t j) {
+  const uint32_t thr = drop_threshold(dropout_p);
+  if (!thr) return 1;
+  const uint32_t kbh = drop_bh_key(drop_seed_key(dropout_seed), (uint32_t)b * (uint32_t)H + (uint32_t)h);
+  return drop_keep(kbh, (uint32_t)i, (uint32_t)j, thr) ? 1 : 0;
+}
+
 const char* hstu_attn_last_error(void) { return g_err; }
 
 size_t hstu_attn_fwd_workspace_bytes(const HstuAttnFwdArgs* args) {
@@ -5268,7 +5358,7 @@ int hstu_attn_fwd(const HstuAttnFwdArgs* args, void* stream) {
       const bool count_known = q.jagged || !q.seq_lens;
       const long long tiles = q.jagged ? args->total_tokens / BM + args->B : (long long)args->B * q.n_qtiles;
       const long long jobs_per_xcd = q.H >= 8 ? tiles * (q.H >> 3) : tiles / (8 / q.H);
-      q.no_stream = (args->flags & HSTU_FWD_COMPILER_SCHEDULED_BLOCKS) ? 1 : 0;
+      q.no_stream = ((args->flags & HSTU_FWD_COMPILER_SCHEDULED_BLOCKS) || q.drop_thr) ? 1 : 0;   // (the stream has no dropout)
       // (with timestamp descriptors the interior steps run as the hand-scheduled stream, which the resident instances
       // with timestamps do not have: one workgroup per item there)
       q.persist = can_stay && !(args->flags & HSTU_FWD_ONE_ITEM_PER_WORKGROUP) &&

@@ -5,8 +5,10 @@ The harness for the end-to-end (config-4) shape: the attention is
 inference the projections' activation and the attention norm + U gate are the
 fused steps of `recml_amd.hstu_block_ops`; the rest is plain torch on the GPU
 (embedding gather, input layer norm, the output product with the residual as
-its C operand).  No dropout: a block built with a rate refuses a training-mode
-forward (inference, where the reference applies none either, is unaffected).
+its C operand).  A block built with a dropout rate drops attention weights in
+training mode inside the attention kernels (forward and backward regenerate the
+same keep pattern from a seed drawn per call), and the model drops embedding
+entries with torch's dropout; in eval mode neither does anything.
 Parameters are created frozen; after `requires_grad_(True)` the attention goes
 through the HIP backward kernels; in bf16 on a GPU so do the layer norms and the
 U gate (one pass each way), the attention's and the gate's gradients landing in
@@ -139,8 +141,8 @@ class HSTUBlock(torch.nn.Module):
       raise ValueError(f"hidden_dim {hidden_dim} is not a multiple of num_heads {num_heads}")
     if not 0.0 <= dropout < 1.0:
       raise ValueError(f"dropout must be in [0, 1), got {dropout}")
-    # The reference drops attention weights in training (recml/layers/keras/hstu.py:386-387); the kernels here have
-    # no dropout, so a block with a rate set refuses a training-mode forward rather than train without it.
+    # The reference drops attention weights in training (recml/layers/keras/hstu.py:386-387): here the attention
+    # kernels do it, from a seed this block draws per forward.
     self.dropout = float(dropout)
     self.num_heads = num_heads
     self.head_dim = hidden_dim // num_heads
@@ -175,8 +177,18 @@ class HSTUBlock(torch.nn.Module):
       rf *= s
     return shape[-2] * rf, shape[-1] * rf
 
+  def _dropout_kw(self, dropout_seed=None) -> dict:
+    """The attention's dropout arguments for this call: none in eval mode or at rate 0; in training mode the
+    block's rate and a seed from torch's CPU generator (so torch.manual_seed makes a run repeatable, and no GPU
+    work waits on it) unless the caller brings one."""
+    if not (self.training and self.dropout > 0.0):
+      return {}
+    if dropout_seed is None:
+      dropout_seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+    return dict(dropout_p=self.dropout, dropout_seed=int(dropout_seed))
+
   def forward(self, inputs, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None,
-              attention_mask=None, attention_bias=None, batch=None):
+              attention_mask=None, attention_bias=None, batch=None, dropout_seed=None):
     """inputs [B, L, D] -> [B, L, D].
 
     Give `seq_lens` [B] (keys and rows at or past the length are masked, as
@@ -184,20 +196,17 @@ class HSTUBlock(torch.nn.Module):
     or, for the reference's calling convention, a dense `attention_mask`
     [B, L, L] and optional `attention_bias` [B, L, L]
     (recml/layers/keras/hstu.py:422-440).  `batch`: an `hstu_ops.AttentionBatch` shared with the
-    other blocks that see the same lengths, timestamps and tables.
+    other blocks that see the same lengths, timestamps and tables.  `dropout_seed`: in training mode
+    with a dropout rate, the seed of this call's keep pattern (default: drawn from torch's generator).
     """
-    if self.dropout > 0.0 and self.training:
-      raise NotImplementedError(
-          f"HSTUBlock(dropout={self.dropout}) in training mode: dropout on the attention weights "
-          "(recml/layers/keras/hstu.py:386-387) is not implemented by the attention kernels; "
-          "call .eval() for inference or build the block with dropout=0")
+    drop = self._dropout_kw(dropout_seed)
     B, L, D = inputs.shape
     H, hd = self.num_heads, self.head_dim
     fused = self._fused_inference(inputs, pos_bias, ts_bias, attention_bias)
     if attention_mask is None and attention_bias is None and self._fused_training(inputs, pos_bias, ts_bias):
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       return self._train_steps(inputs.reshape(B * L, D), (B, L), pos_bias, ts_bias, batch,
-                               dict(seq_lens=seq_lens, n=n, alpha=alpha, timestamps=timestamps)).reshape(B, L, D)
+                               dict(seq_lens=seq_lens, n=n, alpha=alpha, timestamps=timestamps, **drop)).reshape(B, L, D)
     x = self._input_norm(inputs, fused)
     w, b = self._uqkv_weights()
     if fused:
@@ -213,14 +222,15 @@ class HSTUBlock(torch.nn.Module):
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       if _wants_grad(q, k, v, attention_bias):
         # training: forward and backward kernels, the gradient of a dense bias included
-        attn = hstu_ops.hstu_attention_autograd(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask, bias=attention_bias)
+        attn = hstu_ops.hstu_attention_autograd(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask,
+                                                bias=attention_bias, **drop)
       else:
         attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
-                                            scaled_pointwise_attn=self.scaled_pointwise_attn, batch=batch)
+                                            scaled_pointwise_attn=self.scaled_pointwise_attn, batch=batch, **drop)
     else:
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
-                        timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias, batch=batch)
+                        timestamps=timestamps, ts_bias=ts_bias, bias=attention_bias, batch=batch, **drop)
     if fused:
       gated = hstu_block_ops.norm_gate(attn.reshape(B * L, H * hd), u.reshape(B * L, H * hd), self.attn_ln_gamma.reshape(-1),
                                        self.attn_ln_beta.reshape(-1), self.eps)
@@ -276,20 +286,22 @@ class HSTUBlock(torch.nn.Module):
     b = torch.cat([self.u_bias, self.q_bias, self.k_bias, self.v_bias], dim=0).reshape(-1) if self.use_bias else None
     return w, b
 
-  def forward_jagged(self, tokens, seq_offsets, max_len, *, pos_bias=None, timestamps=None, ts_bias=None, batch=None):
+  def forward_jagged(self, tokens, seq_offsets, max_len, *, pos_bias=None, timestamps=None, ts_bias=None, batch=None,
+                     dropout_seed=None):
     """The block on packed tokens [T, D] (sequence b = rows seq_offsets[b]..seq_offsets[b+1]):
     no work at all for padding, in the projections either.  `timestamps` is jagged [T].
 
     Inference in bf16 takes the fused steps: the projections' SiLU in the epilogue of their one
     matrix product, the attention norm and the U gate in one pass (recml_amd.hstu_block_ops), the
     residual as the C operand of the output product."""
+    drop = self._dropout_kw(dropout_seed)
     T, D = tokens.shape
     H, hd = self.num_heads, self.head_dim
     fused = self._fused_inference(tokens, pos_bias, ts_bias)
     if self._fused_training(tokens, pos_bias, ts_bias):
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
       return self._train_steps(tokens, (T,), pos_bias, ts_bias, batch,
-                               dict(seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha, timestamps=timestamps))
+                               dict(seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha, timestamps=timestamps, **drop))
     x = self._input_norm(tokens, fused)
     w, b = self._uqkv_weights()
     if fused:
@@ -302,7 +314,7 @@ class HSTUBlock(torch.nn.Module):
     u, q, k, v = uqkv.unbind(dim=1)
     alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(max_len))
     attn = _attention(q, k, v, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
-                      pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, batch=batch)
+                      pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, batch=batch, **drop)
     if fused:
       gated = hstu_block_ops.norm_gate(attn.reshape(T, H * hd), u.reshape(T, H * hd), self.attn_ln_gamma.reshape(-1),
                                        self.attn_ln_beta.reshape(-1), self.eps)
@@ -339,6 +351,7 @@ class HSTU(torch.nn.Module):
     self.model_dim = model_dim
     self.eps = norm_eps
     self.scale_by_sqrt_dim = scale_by_sqrt_dim
+    self.dropout = float(dropout)      # on the embeddings here (hstu.py:541-543, 602), on the attention weights in the blocks
 
   def count_params(self) -> int:
     return sum(p.numel() for p in self.parameters())
@@ -391,6 +404,7 @@ class HSTU(torch.nn.Module):
       if self.position_embedding is not None:
         x = x + self.position_embedding[: x.shape[1]]
       x = self._final_norm(x)
+    x = F.dropout(x, self.dropout, self.training)
     # every block sees the same lengths, timestamps and tables: the attention prepares them once
     batch = hstu_ops.AttentionBatch()
     for block in self.decoder_blocks:
@@ -420,6 +434,7 @@ class HSTU(torch.nn.Module):
       if pos_idx is not None:
         x = x + self.position_embedding[pos_idx]
       x = self._final_norm(x)
+    x = F.dropout(x, self.dropout, self.training)
     ts = None if timestamps is None else timestamps.reshape(-1)[where]
     batch = hstu_ops.AttentionBatch()
     for block in self.decoder_blocks:

@@ -158,7 +158,7 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
                timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                q_segment_ids=None, kv_segment_ids=None,
                sliding_window_size=None, mask=None, bias=None,
-               q_scale=None, k_scale=None, batch=None):
+               q_scale=None, k_scale=None, batch=None, dropout_p=0.0, dropout_seed=0):
   """Validates the call and fills an HstuAttnFwdArgs.  Returns (args, keepalive)."""
   given = (seq_lens, seq_offsets, timestamps, pos_bias, ts_bias, mask)
   for name, t in (("q", q), ("k", k), ("v", v)):
@@ -277,6 +277,10 @@ def build_args(q, k, v, out, *, seq_lens=None, seq_offsets=None, max_len=None,
     if int(sliding_window_size) < 0:
       raise ValueError("sliding_window_size must be >= 0")
     a.window = min(int(sliding_window_size), 2 ** 31 - 1)   # beyond the sequence it restricts nothing
+  if not 0.0 <= float(dropout_p) < 1.0:
+    raise ValueError(f"dropout_p must be in [0, 1), got {dropout_p}")
+  a.dropout_p = float(dropout_p)
+  a.dropout_seed = int(dropout_seed) & 0xFFFFFFFFFFFFFFFF
 
   if mask is not None:
     if isinstance(mask, np.ndarray):
@@ -354,7 +358,7 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
                    timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                    q_segment_ids=None, kv_segment_ids=None,
                    sliding_window_size=None, mask=None, bias=None, out=None,
-                   q_scale=None, k_scale=None, batch=None):
+                   q_scale=None, k_scale=None, batch=None, dropout_p=0.0, dropout_seed=0):
   """out = (silu(alpha * q k^T + bias) / n, masked) v.
 
   Args:
@@ -383,6 +387,11 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
     bias: dense additive logit bias [L, Lkv] or [B, L, Lkv] shared by heads
       (hstu.py:373-374).
     out: optional preallocated output.
+    dropout_p, dropout_seed: training-time dropout on the masked attention weights
+      (hstu.py:386-387): each weight is dropped with probability dropout_p, the others are
+      scaled by 1 / (1 - dropout_p).  Which pairs survive is a fixed function of
+      (dropout_seed, sequence, head, i, j) -- `dropout_keep` gives it on the host -- so
+      hstu_attention_bwd with the same two values differentiates exactly this output.
     batch: optional AttentionBatch shared by the calls on one batch (a model's layers): the first
       call prepares the work list, timestamps and tables, the later ones reuse them.
 
@@ -400,7 +409,7 @@ def hstu_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None,
       timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
       q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids,
       sliding_window_size=sliding_window_size, mask=mask, bias=bias,
-      q_scale=q_scale, k_scale=k_scale, batch=batch)
+      q_scale=q_scale, k_scale=k_scale, batch=batch, dropout_p=dropout_p, dropout_seed=dropout_seed)
   with torch.cuda.device(q.device):
     _run(args, keep)
   if batch is not None:
@@ -412,7 +421,7 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
                        n=None, alpha=1.0, causal=True, pos_bias=None,
                        timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                        q_segment_ids=None, kv_segment_ids=None,
-                       sliding_window_size=None, mask=None, bias=None,
+                       sliding_window_size=None, mask=None, bias=None, dropout_p=0.0, dropout_seed=0,
                        table_grads=True, bias_grad=False, grads_out=None, _variant_out=None):
   """Gradients of sum(hstu_attention(q, k, v, ...) * dout).
 
@@ -440,7 +449,7 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
       q, k, v, dout, seq_lens=seq_lens, seq_offsets=seq_offsets, max_len=max_len, n=n, alpha=alpha,
       causal=causal, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, ts_bucket_size=ts_bucket_size,
       q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids, sliding_window_size=sliding_window_size,
-      mask=mask, bias=bias)
+      mask=mask, bias=bias, dropout_p=dropout_p, dropout_seed=dropout_seed)
   # build_args may have made q, k, v contiguous in d: the gradients take the layout it passed on
   qi, ki, vi = _passed_inputs(keep)
   if grads_out is None:
@@ -488,6 +497,12 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   if bias_grad:
     return dq, dk, dv, dpos, dts, dbias.reshape(bias.shape)
   return dq, dk, dv, dpos, dts
+
+
+def dropout_keep(seed, p, b, h, H, i, j) -> bool:
+  """Whether the weight of (sequence b, head h of H, query i, key j) survives dropout with this seed and
+  rate: the library's own rule, evaluated on the host (no GPU needed)."""
+  return bool(_lib.load().hstu_attn_dropout_keep(int(seed) & 0xFFFFFFFFFFFFFFFF, float(p), b, h, H, i, j))
 
 
 def _grad_buffers(q, k, v):
@@ -589,8 +604,10 @@ def pointwise_splash_attention(
 
 
 def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
-                        scaled_pointwise_attn=False, seq_lens=None, batch=None):
-  """Layer-side call, recml/layers/keras/hstu.py:356-390 (inference).
+                        scaled_pointwise_attn=False, seq_lens=None, batch=None,
+                        dropout_p=0.0, dropout_seed=0):
+  """Layer-side call, recml/layers/keras/hstu.py:356-390 (with dropout_p > 0 its training
+  form: dropout on the masked weights, hstu.py:386-387).
 
   `attention_mask` is the [B, L, L] 0/1 mask the layer builds with
   make_causal_mask; `attention_bias` an optional [B or 1, L, L] additive bias
@@ -608,6 +625,8 @@ def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
     if seq_lens is None:
       raise ValueError("pass attention_mask or seq_lens")
     return hstu_attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha,
-                          causal=True, bias=attention_bias, batch=batch)
+                          causal=True, bias=attention_bias, batch=batch,
+                          dropout_p=dropout_p, dropout_seed=dropout_seed)
   return hstu_attention(q, k, v, n=n, alpha=alpha, causal=False,
-                        mask=attention_mask, bias=attention_bias, batch=batch)
+                        mask=attention_mask, bias=attention_bias, batch=batch,
+                        dropout_p=dropout_p, dropout_seed=dropout_seed)

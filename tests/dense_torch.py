@@ -5,11 +5,12 @@ import torch
 
 def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=True, pos_bias=None,
                           timestamps=None, ts_bias=None, ts_bucket_size=0.301, bias=None, mask=None,
-                          sliding_window_size=None):
+                          sliding_window_size=None, dropout_p=0.0, dropout_seed=0):
   """The op in plain torch on padded [B, L, H, d] tensors (recml/layers/keras/hstu.py:356-390 with the
   bias tables expanded): materialises [B, H, L, L], differentiable through everything it reads, any
   device.  A plain statement of the op for the tests: the package has no such path (its kernels return every
-  gradient, the dense bias's included)."""
+  gradient, the dense bias's included).  With dropout_p > 0 the weights are multiplied by the oracle's keep
+  pattern for that seed over 1 - dropout_p (hstu.py:386-387)."""
   from recml_amd.hstu_bias import default_bucketization
   B, L, H, d = q.shape
   Lkv = k.shape[1]
@@ -38,4 +39,8 @@ def dense_attention_torch(q, k, v, *, seq_lens=None, n=None, alpha=1.0, causal=T
     mk = mask != 0
     keep = keep & (mk if mk.dim() == 3 else mk[None])
   p = torch.where(keep[:, None], torch.nn.functional.silu(s) / n, torch.zeros((), device=q.device))
+  if dropout_p > 0:
+    from oracle import hstu_oracle as O
+    kept = torch.from_numpy(O.dropout_keep_mask(dropout_seed, dropout_p, B, H, L, Lkv)).to(q.device)
+    p = p * kept / (1.0 - dropout_p)
   return torch.einsum("bhij,bjhd->bihd", p, v.float()).to(v.dtype)

@@ -88,46 +88,80 @@ def _load_block(block, w, dtype):
     getattr(block, name_map.get(k, k)).data = torch.from_numpy(np.asarray(val)).to(device="cuda:0", dtype=dtype)
 
 
-def test_block_with_dropout_refuses_training_mode_on_any_device():
-  # recml/layers/keras/hstu.py:386-387 drops attention weights when training; no kernel here does
+def test_block_dropout_arguments_follow_the_mode():
+  # recml/layers/keras/hstu.py:386-387 drops attention weights when training and only then
   from recml_amd.hstu_layer import HSTUBlock
-  blk = HSTUBlock(32, 2, dropout=0.1)
-  with pytest.raises(NotImplementedError, match="dropout"):
-    blk(torch.zeros(1, 4, 32), seq_lens=torch.tensor([4], dtype=torch.int32))
   with pytest.raises(ValueError, match="dropout"):
     HSTUBlock(32, 2, dropout=1.0)
+  blk = HSTUBlock(32, 2, dropout=0.1)
+  assert blk.training
+  assert blk._dropout_kw(5) == dict(dropout_p=0.1, dropout_seed=5)
+  torch.manual_seed(3)
+  a, b = blk._dropout_kw(), blk._dropout_kw()
+  torch.manual_seed(3)
+  assert blk._dropout_kw() == a and a != b and a["dropout_p"] == 0.1 and 0 <= a["dropout_seed"] < 2 ** 62
+  blk.eval()
+  assert blk._dropout_kw() == {} and blk._dropout_kw(5) == {}
+  assert HSTUBlock(32, 2)._dropout_kw(5) == {}
 
 
 @pytest.mark.gpu
-def test_dropout_rate_refused_in_training_and_ignored_in_eval(gpu):
-  """A block (and a model) with a dropout rate: a training-mode forward raises before any kernel runs; in eval
-  mode, where the reference applies no dropout either, the output is that of a block without a rate."""
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_block_in_training_mode_drops_attention_weights(gpu, dtype, tol):
+  """A block with a dropout rate: in training mode its output is the oracle's block with the same rate and seed
+  (padded and packed); the seed it draws follows torch's generator; in eval mode, where the reference applies no
+  dropout either, the output is that of a block without a rate.  The model adds dropout on the embeddings."""
   import recml_amd
   from recml_amd.hstu_layer import HSTUBlock
-  bf, dev = torch.bfloat16, "cuda:0"
-  B, L, D = 2, 96, 128
-  g = lambda: torch.Generator(device="cpu").manual_seed(4)
-  blk = HSTUBlock(D, 2, dropout=0.2, dtype=bf, device=dev, generator=g())
-  plain = HSTUBlock(D, 2, dropout=0.0, dtype=bf, device=dev, generator=g())
-  x = torch.randn(B, L, D, device=dev).to(bf)
-  lens = torch.tensor([96, 40], device=dev, dtype=torch.int32)
+  dev = "cuda:0"
+  rng = np.random.default_rng(12)
+  B, L, D, H = 3, 150, 128, 2
+  lens = np.array([150, 40, 97], dtype=np.int32)
+  w = _rand_block(rng, D, H)
+  blk = HSTUBlock(D, H, dropout=0.3, dtype=dtype, device=dev)
+  plain = HSTUBlock(D, H, dtype=dtype, device=dev)
+  _load_block(blk, w, dtype)
+  _load_block(plain, w, dtype)
+  rd = lambda a: torch.from_numpy(np.asarray(a)).to(device=dev, dtype=dtype).double().cpu().numpy()
+  wq = {k: rd(v) for k, v in w.items()}
+  xq = rd(rng.standard_normal((B, L, D)))
+  pos = 0.1 * rng.standard_normal(2 * L - 1)
+  x, lt, pt = torch.from_numpy(xq).to(device=dev, dtype=dtype), torch.from_numpy(lens).to(dev), torch.from_numpy(pos).float().to(dev)
   assert blk.training
-  with pytest.raises(NotImplementedError, match="dropout"):
-    blk(x, seq_lens=lens)
-  blk.requires_grad_(True)
-  with pytest.raises(NotImplementedError, match="dropout"):
-    blk(x, seq_lens=lens)
+  ref = BO.hstu_block(xq, wq, num_heads=H, seq_lens=lens, pos_tab=pos, dropout_p=0.3, dropout_seed=77)
+  base = BO.hstu_block(xq, wq, num_heads=H, seq_lens=lens, pos_tab=pos)
+  assert np.abs(ref - base).max() > 0.05 * np.abs(base).max()          # the case tells the two apart
+  out = blk(x, seq_lens=lt, pos_bias=pt, dropout_seed=77).double().cpu().numpy()
+  for b in range(B):
+    assert np.abs(out[b, :lens[b]] - ref[b, :lens[b]]).max() <= tol * np.abs(ref).max(), b
+  # packed tokens: the same pattern (it is a function of the sequence's index and the positions within it)
+  off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+  xj = torch.cat([x[b, :lens[b]] for b in range(B)])
+  outj = blk.forward_jagged(xj, torch.from_numpy(off).to(dev), L, pos_bias=pt, dropout_seed=77).double().cpu().numpy()
+  for b in range(B):
+    assert np.abs(outj[off[b]:off[b + 1]] - ref[b, :lens[b]]).max() <= tol * np.abs(ref).max(), b
+  # seeds drawn from torch's generator: repeatable under manual_seed, different from call to call
+  torch.manual_seed(5)
+  o1, o2 = blk(x, seq_lens=lt, pos_bias=pt), blk(x, seq_lens=lt, pos_bias=pt)
+  torch.manual_seed(5)
+  assert torch.equal(blk(x, seq_lens=lt, pos_bias=pt), o1) and not torch.equal(o1, o2)
   blk.eval()
-  with torch.no_grad():
-    assert torch.equal(blk(x, seq_lens=lens), plain(x, seq_lens=lens))
-  model = recml_amd.HSTU(vocab_size=50, max_positions=L, model_dim=D, num_heads=2, num_layers=2, dropout=0.1,
-                         dtype=bf, device=dev, add_head=False)
-  ids = torch.randint(0, 50, (B, L), device=dev)
-  with pytest.raises(NotImplementedError, match="dropout"):
-    model(ids, seq_lens=lens)
-  model.eval()
-  with torch.no_grad():
-    assert model(ids, seq_lens=lens).shape == (B, L, D)
+  assert torch.equal(blk(x, seq_lens=lt, pos_bias=pt), plain(x, seq_lens=lt, pos_bias=pt))
+  assert torch.equal(blk(x, seq_lens=lt, pos_bias=pt, dropout_seed=77), plain(x, seq_lens=lt, pos_bias=pt))
+  if dtype == torch.bfloat16:
+    model = recml_amd.HSTU(vocab_size=50, max_positions=L, model_dim=D, num_heads=H, num_layers=2, dropout=0.2,
+                           dtype=dtype, device=dev, add_head=False)
+    ids = torch.randint(0, 50, (B, L), device=dev)
+    torch.manual_seed(1)                # (seeds torch's CPU generator, where the blocks draw, and the GPU's, where F.dropout does)
+    t1 = model(ids, seq_lens=lt)
+    t2 = model(ids, seq_lens=lt)
+    torch.manual_seed(1)
+    t3 = model(ids, seq_lens=lt)
+    assert t1.shape == (B, L, D) and torch.equal(t1, t3) and not torch.equal(t1, t2) and bool(torch.isfinite(t1.float()).all())
+    model.eval()
+    with torch.no_grad():
+      e1, e2 = model(ids, seq_lens=lt), model(ids, seq_lens=lt)
+    assert torch.equal(e1, e2) and not torch.equal(e1, t1)
 
 
 @pytest.mark.gpu
@@ -255,8 +289,10 @@ def test_model_config4_full_size_bf16(gpu):
       assert err <= 3e-2, (name, b, n, err)
 
 
-def _dense_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None, n=None, alpha=1.0, pos_bias=None, **_):
-  """Differentiable dense torch form of the op (padded layout, causal, lengths, position table)."""
+def _dense_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None, n=None, alpha=1.0, pos_bias=None,
+                     dropout_p=0.0, dropout_seed=0, **_):
+  """Differentiable dense torch form of the op (padded layout, causal, lengths, position table, dropout by the
+  oracle's keep pattern)."""
   B, L, H, d = q.shape
   s = alpha * torch.einsum("bihd,bjhd->bhij", q.float(), k.float())
   i = torch.arange(L, device=q.device)
@@ -264,21 +300,25 @@ def _dense_attention(q, k, v, *, seq_lens=None, seq_offsets=None, max_len=None, 
     s = s + pos_bias.float()[:, (L - 1) + i[None, :] - i[:, None]][None]
   keep = (i[None, :] <= i[:, None])[None] & (i[None, None, :] < seq_lens[:, None, None]) & (i[None, :, None] < seq_lens[:, None, None])
   p = torch.nn.functional.silu(s) / n * keep[:, None]
+  if dropout_p > 0:
+    p = p * torch.from_numpy(O.dropout_keep_mask(dropout_seed, dropout_p, B, H, L, L)).to(q.device) / (1.0 - dropout_p)
   return torch.einsum("bhij,bjhd->bihd", p, v.float()).to(q.dtype)
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("drop", [0.0, 0.25])
 @pytest.mark.parametrize("dtype,hd,tol", [(torch.float32, 16, 2e-4), (torch.bfloat16, 64, 6e-2)])
-def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
+def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol, drop):
   """A trainable block: gradients with the HIP attention (forward and backward kernels, q / k / v being
-  strided slices of the fused projection) against the same block with a dense torch attention."""
+  strided slices of the fused projection) against the same block with a dense torch attention; with a
+  dropout rate too (training mode, the seed given: the backward kernels regenerate the forward's pattern)."""
   from recml_amd import hstu_layer
   from recml_amd.hstu_layer import HSTUBlock
   dev = torch.device("cuda:0")
   B, L, H = 3, 160, 2
   D = H * hd
   gen = torch.Generator().manual_seed(5)
-  blk = HSTUBlock(D, H, dtype=dtype, device=dev, generator=gen)
+  blk = HSTUBlock(D, H, dropout=drop, dtype=dtype, device=dev, generator=gen)
   blk.requires_grad_(True)
   x = (torch.randn((B, L, D), generator=gen) * 0.5).to(dev).to(dtype).requires_grad_(True)
   lens = torch.tensor([160, 77, 1], dtype=torch.int32, device=dev)
@@ -293,7 +333,7 @@ def test_block_gradients_through_the_hip_backward(gpu, dtype, hd, tol):
     try:
       for t in [x, pos, *blk.parameters()]:
         t.grad = None
-      out = blk(x, seq_lens=lens, pos_bias=pos)
+      out = blk(x, seq_lens=lens, pos_bias=pos, dropout_seed=4242)
       (out.float() * dout.float()).sum().backward()
       return {"x": x.grad.float().clone(), "pos": pos.grad.float().clone(),
               **{n: p.grad.float().clone() for n, p in blk.named_parameters() if p.grad is not None}}
@@ -374,8 +414,9 @@ def test_packed_block_trains_through_the_fused_steps(gpu, use_bias):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("drop", [0.0, 0.2])
 @pytest.mark.parametrize("dtype,hd,tol", [(torch.float32, 16, 2e-4), (torch.bfloat16, 64, 6e-2)])
-def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol):
+def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol, drop):
   """Training a block the way the reference calls it -- a dense [B, L, L] mask and a constant dense bias:
   the attention's forward and backward kernels take the mask and the bias as they are (no gradient is asked
   for the bias); against the same block with the attention in plain torch."""
@@ -385,7 +426,7 @@ def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol)
   B, L, H = 2, 144, 2
   D = H * hd
   gen = torch.Generator().manual_seed(6)
-  blk = HSTUBlock(D, H, dtype=dtype, device=dev, generator=gen)
+  blk = HSTUBlock(D, H, dropout=drop, dtype=dtype, device=dev, generator=gen)
   blk.requires_grad_(True)
   x = (torch.randn((B, L, D), generator=gen) * 0.5).to(dev).to(dtype).requires_grad_(True)
   lens = torch.tensor([144, 50], device=dev)
@@ -401,7 +442,7 @@ def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol)
     try:
       for t in [x, *blk.parameters()]:
         t.grad = None
-      out = blk(x, attention_mask=mask, attention_bias=bias)
+      out = blk(x, attention_mask=mask, attention_bias=bias, dropout_seed=9)
       (out.float() * dout.float()).sum().backward()
       return {"x": x.grad.float().clone(), **{n: p.grad.float().clone() for n, p in blk.named_parameters() if p.grad is not None}}
     finally:

@@ -171,7 +171,9 @@ typedef struct HstuAttnFwdArgs {
    * counter-based hash, hstu_attn_dropout_keep below -- so the backward, given
    * the same two values, drops the same pairs, and a caller can reproduce the
    * mask.  0 (the default) switches it off.  With dropout the matrix-core
-   * kernel runs every step through its compiler-scheduled block code. */
+   * kernel runs every step through its compiler-scheduled block code.
+   * Both values travel as kernel arguments: a HIP graph that recorded a call
+   * replays that call's pattern until its kernel nodes are given new ones. */
   float dropout_p;        /* in [0, 1)                                        */
   uint32_t reserved0;     /* 0                                                */
   uint64_t dropout_seed;

@@ -34,12 +34,13 @@ def _variant(q, k, v, **kw):
   return hstu_ops.kernel_variant(args)
 
 
-def _one_hot_rows(B, L, H, d, base=1.0):
-  """x[b, t, h, t % d] = base * 2^(t // d), 0 elsewhere: a product with it files every position under its own
-  column, the positions that share a column under different binary digits."""
+def _one_hot_rows(B, L, H, d, base=1.0, lo=0, n=None):
+  """x[b, t, h, (t - lo) % d] = base * 2^((t - lo) // d) for the positions t in [lo, lo + n), 0 elsewhere: a product
+  with it files every such position under its own column, the positions that share a column under different binary
+  digits."""
   x = np.zeros((B, L, H, d), np.float32)
-  t = np.arange(L)
-  x[:, t, :, t % d] = (base * 2.0 ** (t // d))[:, None, None]
+  t = np.arange(lo, L if n is None else min(L, lo + n))
+  x[:, t, :, (t - lo) % d] = (base * 2.0 ** ((t - lo) // d))[:, None, None]
   return x
 
 
@@ -88,6 +89,11 @@ FWD_PATTERN_CASES = [
     ("d128 fp8", 128, 2, 2, 512, [512, 129], ("fp8",), False, "hstu_fwd_mfma_fp8"),
     ("d64 ts", 64, 2, 4, 256, [256, 100], ("ts",), False, "hstu_fwd_mfma_bf16"),
     ("d32 pos", 32, 2, 2, 128, [128, 33], ("pos",), True, "hstu_fwd_mfma_bf16"),
+    # one long sequence among short ones: its tiles' key ranges are split between workgroups; read back through the
+    # first and through the last 512 keys
+    ("d128 split tiles, first keys", 128, 3, 2, 2048, [2048, 64, 64], ("pos", "ts", "lo=0"), True, "hstu_fwd_mfma_bf16"),
+    ("d128 split tiles, last keys", 128, 3, 2, 2048, [2048, 64, 64], ("lo=1536",), True, "hstu_fwd_mfma_bf16"),
+    ("d128 not causal", 128, 2, 2, 384, [384, 130], ("full",), False, "hstu_fwd_mfma_bf16"),
     ("fp32 general", 48, 2, 3, 192, [192, 50], ("pos", "fp32"), False, "hstu_fwd_general<float>"),
     ("bf16 general d48", 48, 2, 2, 192, [192, 101], ("pos",), False, "hstu_fwd_general<bf16>"),
 ]
@@ -103,15 +109,17 @@ def test_forward_drops_exactly_the_oracles_pairs(gpu, name, d, B, H, L, lens, ex
   ln = np.array(lens, np.int32) if lens is not None else rng.integers(1, L + 1, B).astype(np.int32)
   ln[0] = L
   dt = torch.float32 if "fp32" in extras else BF
+  lo = next((int(e[3:]) for e in extras if e.startswith("lo=")), 0)
+  causal = "full" not in extras
   q = np.full((B, L, H, d), 0.125, np.float32)
-  v = _one_hot_rows(B, L, H, d)
-  kw = dict(n=1.0, alpha=8.0 / d, dropout_p=p, dropout_seed=seed)
+  v = _one_hot_rows(B, L, H, d, lo=lo, n=4 * d)
+  kw = dict(n=1.0, alpha=8.0 / d, dropout_p=p, dropout_seed=seed, causal=causal)
   if "pos" in extras:
     kw["pos_bias"] = _dev(np.zeros((H, 2 * L - 1), np.float32))
   if "ts" in extras:
     kw["ts_bias"] = _dev(np.zeros((H, 65), np.float32))
     stamps = 1_600_000_000 + np.cumsum(rng.integers(1, 100_000, (B, L)), axis=1).astype(np.int64)
-  valid = _valid(ln, L)
+  valid = _valid(ln, L, causal)
   if "seg" in extras:
     seg = np.ones((B, L), np.int32)
     seg[1, 200:] = 2
@@ -140,7 +148,8 @@ def test_forward_drops_exactly_the_oracles_pairs(gpu, name, d, B, H, L, lens, ex
   if jagged:
     out = O.jagged_to_padded(out, off, L)
   keep = O.dropout_keep_mask(seed, p, B, H, L, L) & valid[:, None]            # [B, H, L, L]
-  want = _digits(keep.astype(np.float64), L, d, axis=3).transpose(0, 2, 1, 3)   # [B, L, H, d]
+  seen = keep[..., lo:lo + 4 * d].astype(np.float64)                           # the keys V files
+  want = _digits(seen, seen.shape[3], d, axis=3).transpose(0, 2, 1, 3)         # [B, L, H, d]
   _check_pattern(out.astype(np.float64), want, name)
   # and about the rate's share of the valid pairs was dropped
   share = keep.sum() / (valid.sum() * H)
@@ -376,3 +385,21 @@ def test_autograd_function_with_dropout(gpu):
   want = O.hstu_attention_bwd_ref(n(q), n(k), n(v), n(dout), **kw)
   for name, g, w in zip(("dq", "dk", "dv", "dpos"), (q.grad, k.grad, v.grad, pos.grad), want):
     assert _rel(n(g), w) <= 2e-5, name
+
+
+def test_matrix_core_forward_with_keys_and_queries_of_different_lengths(gpu):
+  """Lq != Lkv (padded, not causal): i counts queries and j keys in the keep rule, also where the two axes differ."""
+  rng = np.random.default_rng(44)
+  B, Lq, Lk, H, d = 2, 200, 330, 2, 128
+  q, k, v, _ = _random_case(rng, B, Lq, Lk, H, d, d, bf16=True)
+  qt, kt, vt = (_dev(x, BF) for x in (q, k, v))
+  kw = dict(causal=False, n=50.0, dropout_p=0.5, dropout_seed=99)
+  assert _variant(qt, kt, vt, **kw) == "hstu_fwd_mfma_bf16"
+  out = recml_amd.hstu_attention(qt, kt, vt, **kw).float().cpu().numpy()
+  want = O.hstu_attention_ref(q, k, v, **kw)
+  assert _rel(out, want) <= 2e-2
+  # with i and j swapped in the rule the result is another one altogether
+  keep_t = O.dropout_keep_mask(99, 0.5, B, H, Lk, Lq).transpose(0, 1, 3, 2)
+  s = np.einsum("bthd,bshd->bhts", q.astype(np.float64), k.astype(np.float64))
+  wrong = np.einsum("bhts,bshd->bthd", O.silu(s) / 50.0 * keep_t * 2.0, v.astype(np.float64))
+  assert _rel(wrong, want) > 0.2

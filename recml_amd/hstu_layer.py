@@ -218,15 +218,10 @@ class HSTUBlock(torch.nn.Module):
       uqkv = F.silu(uqkv).reshape(B, L, 4, H, hd)
     u, q, k, v = uqkv.unbind(dim=2)
     if attention_mask is not None:
-      # the reference's calling convention: a dense [B, L, L] mask and bias
-      alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
-      if _wants_grad(q, k, v, attention_bias):
-        # training: forward and backward kernels, the gradient of a dense bias included
-        attn = hstu_ops.hstu_attention_autograd(q, k, v, n=n, alpha=alpha, causal=False, mask=attention_mask,
-                                                bias=attention_bias, **drop)
-      else:
-        attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
-                                            scaled_pointwise_attn=self.scaled_pointwise_attn, batch=batch, **drop)
+      # the reference's calling convention: a dense [B, L, L] mask and bias (training: forward and backward kernels,
+      # the gradient of a dense bias included)
+      attn = hstu_ops.pointwise_attention(q, k, v, attention_mask, attention_bias,
+                                          scaled_pointwise_attn=self.scaled_pointwise_attn, batch=batch, **drop)
     else:
       alpha, n = (1.0 / math.sqrt(hd), 1.0) if self.scaled_pointwise_attn else (1.0, float(L))
       attn = _attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha, pos_bias=pos_bias,
@@ -378,17 +373,22 @@ class HSTU(torch.nn.Module):
                                      self.eps, scale=scale, positions=None if positions is None else positions.to(torch.int64),
                                      pos_table=self.position_embedding)
 
-  def forward(self, inputs, padding_mask=None, *, seq_lens=None, pos_bias=None, timestamps=None, ts_bias=None,
-              jagged=False):
-    """inputs: item ids [B, L]; `padding_mask` [B, L] (1 = real item, end-padded) or `seq_lens` [B].
+  def forward(self, inputs, padding_mask=None, attention_mask=None, *, seq_lens=None, pos_bias=None, timestamps=None,
+              ts_bias=None, jagged=False):
+    """inputs: item ids [B, L]; `padding_mask` [B, L] (1 = real item, end-padded) or `seq_lens` [B]; or, as
+    the reference's call also allows (hstu.py:585-615), a dense `attention_mask` [B, L, L] that every block
+    then takes as it is (any mask, at the price of reading it in every layer).
 
     jagged=True packs the valid tokens once and runs every block on [T, D]: nothing is computed
     for padding.  Rows past a sequence's length are then returned as zeros, whereas the padded
     form (like the reference) carries the padded positions' own embeddings through the blocks.
     """
-    if seq_lens is None:
+    if attention_mask is not None:
+      if jagged or pos_bias is not None or ts_bias is not None or seq_lens is not None:
+        raise ValueError("`attention_mask` goes with the padded form and without `seq_lens` and bias tables")
+    elif seq_lens is None:
       if padding_mask is None:
-        raise ValueError("Either `padding_mask` or `seq_lens` must be set.")
+        raise ValueError("Either `attention_mask`, `padding_mask` or `seq_lens` must be set.")
       seq_lens = masks.lengths_from_padding_mask(padding_mask)
     if jagged:
       return self._forward_jagged(inputs, seq_lens, pos_bias, timestamps, ts_bias)
@@ -408,7 +408,10 @@ class HSTU(torch.nn.Module):
     # every block sees the same lengths, timestamps and tables: the attention prepares them once
     batch = hstu_ops.AttentionBatch()
     for block in self.decoder_blocks:
-      x = block(x, seq_lens=seq_lens, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, batch=batch)
+      if attention_mask is not None:
+        x = block(x, attention_mask=attention_mask, batch=batch)
+      else:
+        x = block(x, seq_lens=seq_lens, pos_bias=pos_bias, timestamps=timestamps, ts_bias=ts_bias, batch=batch)
     x = self._final_norm(x)
     if self.reverse_embedding is None:
       return x

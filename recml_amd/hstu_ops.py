@@ -551,6 +551,10 @@ class _HstuAttentionFn(torch.autograd.Function):
             cast(got[5], bias) if want_bias else None, None)
 
 
+def _wants_grad(*tensors) -> bool:
+  return torch.is_grad_enabled() and any(isinstance(t, torch.Tensor) and t.requires_grad for t in tensors)
+
+
 def hstu_attention_autograd(q, k, v, *, pos_bias=None, ts_bias=None, bias=None, **kwargs):
   """hstu_attention as a differentiable torch op: gradients for q, k, v, the bias tables pos_bias
   and ts_bias, and a dense `bias` (its gradient is dS summed over the heads, and over the batch
@@ -571,7 +575,9 @@ def pointwise_splash_attention(
   1/sqrt(head_dim) (hstu_ops.py:909, 238).  `mask_type` is MaskType.CAUSAL,
   MaskType.FULL or an explicit boolean [q_len, kv_len] array.  The tile-size,
   sharding and interpret arguments belong to the TPU kernel and are accepted
-  and ignored.
+  and ignored.  Differentiable like the reference's op (its custom_vjp,
+  hstu_ops.py:417-548): when q, k or v asks for a gradient the call goes
+  through the autograd function and the HIP backward kernels.
   """
   del qkv_axis_names, segment_id_axis_names, block_q, block_kv
   del block_kv_compute, block_q_dkv, block_kv_dkv, block_kv_dkv_compute
@@ -597,7 +603,8 @@ def pointwise_splash_attention(
   else:
     raise ValueError(f"Unsupported mask type: '{mask_type}'.")
   scale = scale if scale is not None else 1.0 / (head_dim**0.5)
-  return hstu_attention(
+  op = hstu_attention_autograd if _wants_grad(q, k, v) else hstu_attention
+  return op(
       q, k, v, n=q_len, alpha=scale, causal=causal, mask=explicit,
       q_segment_ids=q_segment_ids, kv_segment_ids=kv_segment_ids,
       sliding_window_size=sliding_window_size)
@@ -616,17 +623,18 @@ def pointwise_attention(q, k, v, attention_mask, attention_bias=None, *,
   causal can pass `seq_lens` with attention_mask=None: same result without
   ever building the [B, L, L] mask.  `batch`: an AttentionBatch shared by the
   calls that bring the same mask (the layers of a model): the mask is then
-  scanned for its key-step ranges once, by the first of them.
+  scanned for its key-step ranges once, by the first of them (inference only).
+  When q, k, v or the bias asks for a gradient the call goes through the
+  autograd function (gradients by the HIP backward kernels, the bias's included).
   """
   d = q.shape[-1]
   alpha = 1.0 / math.sqrt(d) if scaled_pointwise_attn else 1.0
   n = 1.0 if scaled_pointwise_attn else q.shape[1]
-  if attention_mask is None:
-    if seq_lens is None:
-      raise ValueError("pass attention_mask or seq_lens")
-    return hstu_attention(q, k, v, seq_lens=seq_lens, n=n, alpha=alpha,
-                          causal=True, bias=attention_bias, batch=batch,
-                          dropout_p=dropout_p, dropout_seed=dropout_seed)
-  return hstu_attention(q, k, v, n=n, alpha=alpha, causal=False,
-                        mask=attention_mask, bias=attention_bias, batch=batch,
-                        dropout_p=dropout_p, dropout_seed=dropout_seed)
+  if attention_mask is None and seq_lens is None:
+    raise ValueError("pass attention_mask or seq_lens")
+  how = dict(seq_lens=seq_lens, causal=True) if attention_mask is None else dict(mask=attention_mask, causal=False)
+  if _wants_grad(q, k, v, attention_bias):
+    return hstu_attention_autograd(q, k, v, n=n, alpha=alpha, bias=attention_bias, dropout_p=dropout_p,
+                                   dropout_seed=dropout_seed, **how)
+  return hstu_attention(q, k, v, n=n, alpha=alpha, bias=attention_bias, batch=batch,
+                        dropout_p=dropout_p, dropout_seed=dropout_seed, **how)

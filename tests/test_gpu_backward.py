@@ -655,3 +655,44 @@ def test_general_backward_in_bf16_storage(gpu, d, dv, view, products, layout):
     assert np.isfinite(g).all() and _rel(g, w) <= 2e-2, (nm, _rel(g, w))
   for nm, g, w in (("dpos", got[3], want[3]), ("dts", got[4], want[4])):
     assert _rel(g.cpu().numpy().reshape(w.shape), w) <= 2e-2, nm
+
+
+def test_reference_named_entry_points_are_differentiable(gpu):
+  """The reference's own test of the op (recml/core/ops/hstu_ops_test.py:25-96): value_and_grad of
+  sum((attn - targets)^2) through pointwise_splash_attention with segment ids, against the dense form.  Here through
+  torch autograd, against the oracle's pw_attn_ref and its backward; the layer-side call the same way."""
+  rng = np.random.default_rng(50)
+  B, L, H, d = 2, 64, 2, 32
+  q, k, v, targets = (rng.standard_normal((B, L, H, d)).astype(np.float32) for _ in range(4))
+  seg = np.zeros((B, L), np.int32)
+  seg[0, :40] = 1
+  seg[1, :13] = 1
+  qt, kt, vt = (_dev(x).requires_grad_(True) for x in (q, k, v))
+  attn = recml_amd.pointwise_splash_attention(recml_amd.MaskType.CAUSAL, qt, kt, vt, q_segment_ids=_dev(seg),
+                                              kv_segment_ids=_dev(seg))
+  ((attn - _dev(targets)) ** 2).sum().backward()
+  ref = O.pw_attn_ref(q, k, v, seg)
+  got = attn.detach().cpu().numpy()
+  np.testing.assert_allclose(got, ref, atol=1e-5, rtol=1e-5)           # the reference accepts 5e-3
+  dq, dk, dv, _, _ = O.hstu_attention_bwd_ref(q, k, v, 2.0 * (ref - targets), alpha=1 / np.sqrt(d), n=L,
+                                              q_segment_ids=seg, kv_segment_ids=seg)
+  for nm, g, w in (("dq", qt.grad, dq), ("dk", kt.grad, dk), ("dv", vt.grad, dv)):
+    assert _rel(g.cpu().numpy(), w) <= 2e-5, nm
+  # without a gradient asked for, the same values from the forward alone
+  with torch.no_grad():
+    again = recml_amd.pointwise_splash_attention(recml_amd.MaskType.CAUSAL, qt, kt, vt, q_segment_ids=_dev(seg),
+                                                 kv_segment_ids=_dev(seg))
+  assert torch.equal(again, attn.detach())
+  # the layer-side call with a dense mask and a bias that is trained
+  mask = O.make_causal_mask((np.arange(L)[None] < np.array([[40], [13]])).astype(np.float32))
+  bias = (rng.standard_normal((B, L, L)) * 0.3).astype(np.float32)
+  for t in (qt, kt, vt):
+    t.grad = None
+  bt = _dev(bias).requires_grad_(True)
+  out = recml_amd.pointwise_attention(qt, kt, vt, _dev(mask), bt)
+  ((out - _dev(targets)) ** 2).sum().backward()
+  ref = O.pointwise_attention_dense(q, k, v, mask, bias)
+  np.testing.assert_allclose(out.detach().cpu().numpy(), ref, atol=1e-5, rtol=1e-5)
+  want = O.hstu_attention_bwd_ref(q, k, v, 2.0 * (ref - targets), causal=False, mask=mask, bias=bias, bias_grad=True)
+  for nm, g, w in (("dq", qt.grad, want[0]), ("dk", kt.grad, want[1]), ("dv", vt.grad, want[2]), ("dbias", bt.grad, want[5])):
+    assert _rel(g.cpu().numpy(), w) <= 2e-5, nm

@@ -210,6 +210,12 @@ def test_model_on_gpu_against_oracle(gpu):
   outj = m(ids, pm, jagged=True).double().cpu().numpy()
   assert np.abs(outj[0] - ref[0]).max() / np.abs(ref).max() <= 2e-5
   assert np.abs(outj[1, :2] - ref[1, :2]).max() / np.abs(ref).max() <= 2e-5 and (outj[1, 2] == 0).all()
+  # the reference's other way in (hstu.py:604-615): the dense mask itself, here the one it would build
+  import recml_amd
+  outm = m(ids, attention_mask=recml_amd.make_causal_mask(pm.float())).double().cpu().numpy()
+  assert np.abs(outm - ref).max() / np.abs(ref).max() <= 2e-5
+  with pytest.raises(ValueError, match="attention_mask"):
+    m(ids, attention_mask=recml_amd.make_causal_mask(pm.float()), seq_lens=torch.tensor([3, 2], device="cuda:0"))
 
 
 @pytest.mark.gpu

@@ -393,7 +393,8 @@ def dropout_seed_key(seed: int) -> int:
 
 def dropout_hash(seed: int, B: int, H: int, L: int, Lkv: int, b0: int = 0, rows=None, cols=None):
   """uint32 [B, H, L, Lkv]: hash(b, h, i, j) = mix(bhkey(seedkey, (b0 + b) * H + h) + i * CI + j * CJ), all in
-  wrapping 32-bit arithmetic (bhkey: one multiply-add and one xor-shift-multiply round; mix: two rounds).
+  wrapping 32-bit arithmetic (bhkey: one multiply-add and one xor-shift-multiply round; mix(x): y = x * M1, then
+  (y ^ (y >> 16)) * M2).
   `rows` / `cols`: the query / key indices to evaluate instead of all of range(L) / range(Lkv)."""
   key = np.uint64(dropout_seed_key(seed))
   bh = _u32((np.arange(b0, b0 + B, dtype=np.uint64)[:, None] * np.uint64(H)
@@ -404,9 +405,9 @@ def dropout_hash(seed: int, B: int, H: int, L: int, Lkv: int, b0: int = 0, rows=
   i = _u32(np.asarray(range(L) if rows is None else rows, dtype=np.uint64) * np.uint64(DROP_CI))
   j = _u32(np.asarray(range(Lkv) if cols is None else cols, dtype=np.uint64) * np.uint64(DROP_CJ))
   ij = _u32(kbh[:, :, None, None] + i[None, None, :, None] + j[None, None, None, :])
-  z = _u32((ij ^ (ij >> np.uint64(15))) * np.uint64(0x2C1B3C6D))
-  z = _u32((z ^ (z >> np.uint64(12))) * np.uint64(0x297A2D39))
-  return (z ^ (z >> np.uint64(15))).astype(np.uint32)
+  z = _u32(ij * np.uint64(0x2C1B3C6D))
+  z = _u32((z ^ (z >> np.uint64(16))) * np.uint64(0x297A2D39))
+  return z.astype(np.uint32)
 
 
 def dropout_keep_mask(seed: int, p: float, B: int, H: int, L: int, Lkv: int, b0: int = 0):

@@ -401,7 +401,7 @@ __device__ __forceinline__ void general_dense_col(const Params& p, int b, int i0
 // Dropout's keep rule: a counter-based hash of (seed, b, h, i, j), the same on the host, in every kernel and in
 // the CPU oracle.  drop_seed_key folds the 64-bit seed (host, once per call), drop_bh_key the sequence and the
 // head (once per work item), drop_keep the pair: two multiply-add steps on the indices, of which a kernel hoists
-// the one that is fixed for its lane, and two rounds of xor-shift and multiply.
+// the one that is fixed for its lane, then drop_keep_mixed.
 __host__ __device__ inline uint32_t drop_seed_key(uint64_t seed) {
   uint32_t z = (uint32_t)seed ^ 0x9E3779B9u;
   z = (z ^ (z >> 16)) * 0x85EBCA6Bu;
@@ -416,10 +416,12 @@ __host__ __device__ inline uint32_t drop_bh_key(uint32_t key, uint32_t bh) {
 }
 constexpr uint32_t DROP_CI = 0x85EBCA77u, DROP_CJ = 0xC2B2AE3Du;
 // ij = kbh + i * DROP_CI + j * DROP_CJ (wrapping)
+// (two multiplications with one fold of the high half onto the low half between them: the comparison reads the product
+// from its top bits down, which depend on every bit of ij; seven instructions per pair with the index step and the select)
 __host__ __device__ inline bool drop_keep_mixed(uint32_t ij, uint32_t thr) {
-  uint32_t z = (ij ^ (ij >> 15)) * 0x2C1B3C6Du;
-  z = (z ^ (z >> 12)) * 0x297A2D39u;
-  return (z ^ (z >> 15)) >= thr;
+  uint32_t z = ij * 0x2C1B3C6Du;
+  z = (z ^ (z >> 16)) * 0x297A2D39u;
+  return z >= thr;
 }
 __host__ __device__ inline bool drop_keep(uint32_t kbh, uint32_t i, uint32_t j, uint32_t thr) {
   return drop_keep_mixed(kbh + i * DROP_CI + j * DROP_CJ, thr);

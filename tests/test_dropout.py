@@ -29,18 +29,17 @@ def _scalar_hash(seed, b, h, H, i, j):
   z = ((z ^ (z >> 15)) * 0x2C1B3C6D) & M
   kbh = z ^ (z >> 13)
   ij = (kbh + i * 0x85EBCA77 + j * 0xC2B2AE3D) & M
-  z = ((ij ^ (ij >> 15)) * 0x2C1B3C6D) & M
-  z = ((z ^ (z >> 12)) * 0x297A2D39) & M
-  return z ^ (z >> 15)
+  z = (ij * 0x2C1B3C6D) & M
+  return ((z ^ (z >> 16)) * 0x297A2D39) & M
 
 
 # (seed, b, h, H, i, j) -> seed key, hash: worked once and kept as literals
 KNOWN = [
-    ((0, 0, 0, 1, 0, 0), 0x92CA2F0E, 0x849B9C0B),
-    ((1, 0, 0, 1, 0, 0), 0x36DEB503, 0xCA0192A1),
-    ((0x123456789ABCDEF0, 3, 5, 8, 2047, 1023), 0x6546363E, 0xF4EA7194),
-    ((42, 1, 1, 2, 7, 3), 0xE5D9EED0, 0xAF49A80C),
-    ((2 ** 64 - 1, 63, 7, 8, 8191, 8190), 0x786EF1A2, 0xA8A2B570),
+    ((0, 0, 0, 1, 0, 0), 0x92CA2F0E, 0xE5E1963A),
+    ((1, 0, 0, 1, 0, 0), 0x36DEB503, 0x87169A29),
+    ((0x123456789ABCDEF0, 3, 5, 8, 2047, 1023), 0x6546363E, 0xA8933E67),
+    ((42, 1, 1, 2, 7, 3), 0xE5D9EED0, 0xA3B70A2A),
+    ((2 ** 64 - 1, 63, 7, 8, 8191, 8190), 0x786EF1A2, 0xB3570E92),
 ]
 
 
@@ -114,6 +113,27 @@ def test_keep_share_and_independence(p):
   assert abs(corr(x, other - other.mean())) < lim            # neighbouring seeds
   # the same pair under a smaller rate survives whenever it survives under a larger one (one hash, two thresholds)
   assert (O.dropout_keep_mask(1234, p / 2, B, H, L, L) | ~keep).all()
+
+
+@pytest.mark.parametrize("p", [0.1, 0.5, 0.9])
+def test_keep_pattern_has_no_structure_along_the_index_lattice(p):
+  """The pair's part of the hash sees a lattice (a constant step per row and per key): lag correlations along rows,
+  keys and both diagonals up to 128 apart, and the variance of the survivors' count in square patches, rows and
+  columns, against what independent draws give."""
+  L = 512
+  keep = O.dropout_keep_mask(77, p, 2, 2, L, L).astype(np.float64)
+  x = keep - (1 - p)
+  var = p * (1 - p)
+  worst = 0.0
+  for lag in (1, 2, 3, 4, 7, 8, 16, 31, 32, 33, 64, 127, 128):
+    for a, b in ((x[..., lag:], x[..., :-lag]), (x[..., lag:, :], x[..., :-lag, :]),
+                 (x[..., lag:, lag:], x[..., :-lag, :-lag]), (x[..., lag:, :-lag], x[..., :-lag, lag:])):
+      worst = max(worst, abs(float((a * b).mean()) / var * a.size ** 0.5))
+  assert worst < 5.0                                    # 52 z-scores of about a million products each
+  for ps in (2, 4, 8, 32):
+    counts = keep.reshape(2, 2, L // ps, ps, L // ps, ps).sum(axis=(3, 5))
+    assert 0.9 < counts.var() / (ps * ps * var) < 1.1, ps
+  assert 0.8 < keep.sum(axis=3).var() / (L * var) < 1.2 and 0.8 < keep.sum(axis=2).var() / (L * var) < 1.2
 
 
 def _tiny(rng, B=2, L=7, H=2, d=4, dv=3):

@@ -576,7 +576,57 @@ def full_variant(pos: bool, base: int, **kw) -> Gen:
   return g
 
 
+def loads_only_variant(pos: bool, ts: bool) -> Gen:
+  """What a wave without query rows (all 32 past the sequence's end) runs in place of full_variant: its share of the
+  direct loads, the waits for them and every barrier of the workgroup, in the same order and number, and nothing else.
+  A pair's loads go to ring stages whose last readers finished before the barrier that starts the pair, so they may
+  all go out right behind it."""
+  g = Gen(pos, dma=True, base=152 if ts else 160, ts=ts, **PRODUCT)     # (the register window goes unused)
+  g.loads_only = True
+  S = g.S = Stream()
+  S.emit("s_mov_b64 s[90:91], %[kp]")
+  S.emit("s_mov_b64 s[92:93], %[vp]")
+  if pos or ts: S.emit("s_mov_b64 s[94:95], %[bp]")
+  S.emit("s_barrier")                      # (full_variant: behind the first block's logits)
+  def quad(first: bool):
+    for pair in range(2):
+      vst = 2 * pair
+      lines = g.dma_pair(vst)
+      if first and pair == 0: lines = g.dma_k_side(2) + lines
+      for l in lines: S.emit(l)
+      if first and pair == 0:
+        own = (3 if (pos or ts) else 2) * 2 + 2 * 2
+        S.emit(f"s_waitcnt vmcnt({own})")
+        S.emit("s_barrier")
+      S.emit("s_waitcnt vmcnt(0)")
+      S.emit("s_barrier")
+  quad(True)
+  S.emit("s_sub_u32 %[n], %[n], 1")
+  S.emit("s_cmp_eq_u32 %[n], 0")
+  S.emit("s_cbranch_scc1 2f")
+  S.emit("1:")
+  quad(False)
+  S.emit("s_sub_u32 %[n], %[n], 1")
+  S.emit("s_cmp_lg_u32 %[n], 0")
+  S.emit("s_cbranch_scc1 1b")
+  S.emit("2:")
+  return g
+
+
 def asm_statement(g: Gen) -> str:
+  if getattr(g, "loads_only", False):
+    ins = ['[kdst] "s"(hs_kdst)', '[vdst] "s"(hs_vdst)', '[kstep] "s"(hs_kstep)', '[vstep] "s"(hs_vstep)']
+    ins += [f'[koff{r}] "v"(hs_koff[{r}])' for r in range(2)] + [f'[voff{r}] "v"(hs_voff[{r}])' for r in range(2)]
+    ins += ['[kp] "s"(hs_kp)', '[vp] "s"(hs_vp)']
+    outs = ['[n] "+s"(hs_n)']
+    if g.ts:
+      ins += ['[bdst] "s"(hs_bdst)', '[binc] "v"(hs_binc)', '[bexec] "s"(hs_bexec)', '[bp] "s"(hs_bp)']
+      outs.append('[boff] "+v"(hs_boff)')
+    elif g.pos:
+      ins += ['[bdst] "s"(hs_bdst)', '[boff] "v"(hs_boff)', '[bexec] "s"(hs_bexec)', '[bp] "s"(hs_bp)']
+    clob = ['"memory"', '"scc"', '"m0"'] + [f'"s{i}"' for i in range(90, 96)]
+    return (f"  asm volatile(\n{g.S.text()}"
+            f"      : {', '.join(outs)}\n      : {', '.join(ins)}\n      : {', '.join(clob)});\n")
   ins = ['[alpha] "s"(hs_alpha)']
   ins += [f'[q{ks}] "v"(hs_q[{ks}])' for ks in range(8)]
   ins += [f'[ka{ks}] "v"(hs_ka[{ks}])' for ks in range(8)]
@@ -653,13 +703,19 @@ def main():
   a = ap.parse_args()
   parts = ["// Generated by gen_fwd_stream.py: do not edit.  The hand-scheduled stream of the forward kernel's interior blocks.\n",
            "#define HSTU_STREAM_COMPUTE_ONLY 1\n#define HSTU_STREAM_COMPUTE_ONLY_POS 2\n#define HSTU_STREAM_FULL 3\n#define HSTU_STREAM_FULL_POS 4\n"
-           "#define HSTU_STREAM_FULL_TS 5\n#define HSTU_STREAM_FULL_POS_TS 6\n"]
+           "#define HSTU_STREAM_FULL_TS 5\n#define HSTU_STREAM_FULL_POS_TS 6\n"
+           "#define HSTU_STREAM_LOADS_ONLY 7\n#define HSTU_STREAM_LOADS_ONLY_POS 8\n#define HSTU_STREAM_LOADS_ONLY_TS 9\n"
+           "#define HSTU_STREAM_LOADS_ONLY_POS_TS 10\n"]
   parts.append(statement(compute_only_variant(False, a.base, **PRODUCT), "HSTU_STREAM_COMPUTE_ONLY"))
   parts.append(statement(compute_only_variant(True, a.base, **PRODUCT), "HSTU_STREAM_COMPUTE_ONLY_POS"))
   parts.append(statement(full_variant(False, a.base, **PRODUCT), "HSTU_STREAM_FULL"))
   parts.append(statement(full_variant(True, a.base, **PRODUCT), "HSTU_STREAM_FULL_POS"))
   parts.append(statement(full_variant(False, a.base - 8, ts=True, **PRODUCT), "HSTU_STREAM_FULL_TS"))
   parts.append(statement(full_variant(True, a.base - 8, ts=True, **PRODUCT), "HSTU_STREAM_FULL_POS_TS"))
+  parts.append(statement(loads_only_variant(False, False), "HSTU_STREAM_LOADS_ONLY"))
+  parts.append(statement(loads_only_variant(True, False), "HSTU_STREAM_LOADS_ONLY_POS"))
+  parts.append(statement(loads_only_variant(False, True), "HSTU_STREAM_LOADS_ONLY_TS"))
+  parts.append(statement(loads_only_variant(True, True), "HSTU_STREAM_LOADS_ONLY_POS_TS"))    # (another pitch of the bias stages)
   with open(a.out, "w") as f:
     f.write("".join(parts))
   print("wrote", a.out)

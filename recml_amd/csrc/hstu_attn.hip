@@ -3286,7 +3286,26 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Para
       const float hs_alpha = alpha2;
       int hs_n = n_quads;
       floatx16 (&hs_o)[DVB] = o;
-      if constexpr (POS && TS) {
+      if (wave_last < 0) {
+        // a wave whose 32 rows lie past the sequence's end: its share of the loads and every barrier, nothing else
+        if constexpr (POS && TS) {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_LOADS_ONLY_POS_TS
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+        } else if constexpr (TS) {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_LOADS_ONLY_TS
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+        } else if constexpr (POS) {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_LOADS_ONLY_POS
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+        } else {
+#define HSTU_STREAM_VARIANT HSTU_STREAM_LOADS_ONLY
+#include "hstu_fwd_stream_d128.inc"
+#undef HSTU_STREAM_VARIANT
+        }
+      } else if constexpr (POS && TS) {
 #define HSTU_STREAM_VARIANT HSTU_STREAM_FULL_POS_TS
 #include "hstu_fwd_stream_d128.inc"
 #undef HSTU_STREAM_VARIANT

@@ -32,6 +32,9 @@ Wait states written out by hand (gfx950; the assembler does not add them inside 
   exp2 / rcp result -> other vector instruction                    1
   write of m0 -> direct load                                       1
 
+A wave without query rows (all 32 past the sequence's end) takes loads_only_variant instead: the loads,
+waits and barriers of full_variant in the same order and number, and none of its arithmetic.
+
 Usage:  python gen_fwd_stream.py [--out hstu_fwd_stream_d128.inc] [--experiments FILE]
 The output is C++ source: `asm volatile(...)` statements for the kernel to #include, one per
 variant (HSTU_STREAM_VARIANT selects which the including code expands).

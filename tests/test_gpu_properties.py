@@ -8,7 +8,9 @@ The oracle is too slow for whole batches of configuration 3; what does not depen
   * heads are independent and see only their own rows of the bias tables;
   * the jagged and the padded layout give the same rows;
   * backward: sum(q dq) = sum(k dk) (the logits are bilinear in q and k and the biases depend on
-    neither), sum(v dv) = sum(out dout) (out is linear in v), gradients are linear in dout.
+    neither), sum(v dv) = sum(out dout) (out is linear in v), gradients are linear in dout;
+  * with dropout: all of the above for a fixed seed, the second backward identity tying the two
+    directions' keep patterns together.
 
 bf16 storage throughout: exact statements are asserted bit for bit, the others to the tolerance of
 the parity tests (2e-2 of the largest value).
@@ -208,3 +210,58 @@ def test_backward_at_full_size_against_the_oracle(c3):
       assert err <= 2e-2, (b, n, name, err)
     checked += 1
   assert checked >= 40
+
+
+def test_dropout_at_full_size(c3):
+  """The training form at configuration 3's size: the pattern is a function of (sequence, head, i, j), so the
+  padded layout drops the same pairs bit for bit; out stays linear in V; the backward's identities hold with the
+  forward's output on one side -- which they only do when both directions drop the same pairs; and the sequences
+  the oracle can afford agree with it."""
+  w = c3.w
+  B, L, H, d = w.B, w.L, w.H, w.d
+  drop = dict(dropout_p=0.3, dropout_seed=0x5EED0123456789)
+  base = c3.run(**drop)
+  assert not torch.equal(_bits(base), _bits(c3.run()))
+  qp, kp, vp = (torch.zeros((B, L, H, d), dtype=torch.bfloat16, device="cuda:0") for _ in range(3))
+  tsp = torch.zeros((B, L), dtype=torch.int64, device="cuda:0")
+  for b in range(B):
+    s, n = int(w.seq_offsets[b]), int(w.seq_lens[b])
+    qp[b, :n], kp[b, :n], vp[b, :n] = c3.q[s:s + n], c3.k[s:s + n], c3.v[s:s + n]
+    tsp[b, :n] = c3.ts[s:s + n]
+    tsp[b, n:] = c3.ts[s + n - 1]
+  out = recml_amd.hstu_attention(qp, kp, vp, seq_lens=_dev(w.seq_lens), n=w.n, alpha=w.alpha,
+                                 pos_bias=c3.pos, timestamps=tsp, ts_bias=c3.tst, **drop)
+  torch.cuda.synchronize()
+  for b in range(B):
+    s, n = int(w.seq_offsets[b]), int(w.seq_lens[b])
+    assert torch.equal(_bits(out[b, :n]), _bits(base[s:s + n])), f"sequence {b}"
+  # linear in V with the pattern fixed
+  g = torch.Generator(device="cuda:0").manual_seed(3)
+  v2 = (torch.randn(c3.v.shape, device="cuda:0", generator=g) * 0.1).to(torch.bfloat16)
+  mix = (0.5 * c3.v.float() + 2.0 * v2.float()).to(torch.bfloat16)
+  want = 0.5 * base.float() + 2.0 * c3.run(v=v2, **drop).float()
+  assert (c3.run(v=mix, **drop).float() - want).abs().max().item() <= TOL * want.abs().max().item()
+  # the backward with the same rate and seed
+  dout = (torch.randn(c3.v.shape, device="cuda:0", generator=g) * 0.1).to(torch.bfloat16)
+  kw = c3.kwargs(**drop)
+  dq, dk, dv, _, _ = recml_amd.hstu_attention_bwd(c3.q, c3.k, c3.v, dout, **kw)
+  torch.cuda.synchronize()
+  dot = lambda a, b: (a.double() * b.double()).sum().item()
+  qdq, kdk = dot(c3.q, dq), dot(c3.k, dk)
+  assert abs(qdq) > 1e-3 and abs(qdq - kdk) <= 5e-3 * abs(qdq), (qdq, kdk)
+  vdv, odo = dot(c3.v, dv), dot(base, dout)
+  assert abs(odo) > 1e-3 and abs(vdv - odo) <= 5e-3 * abs(odo), (vdv, odo)
+  # ... and with another seed on the backward's side the second identity is gone
+  dv_other = recml_amd.hstu_attention_bwd(c3.q, c3.k, c3.v, dout, **c3.kwargs(dropout_p=0.3, dropout_seed=1))[2]
+  assert abs(dot(c3.v, dv_other) - odo) > 5e-2 * abs(odo)
+  # the oracle on every sequence of up to 200 tokens
+  short = [b for b in range(B) if int(w.seq_lens[b]) <= 200]
+  assert len(short) >= 8
+  f = lambda t: t.float().cpu().numpy()
+  ref = O.hstu_attention_jagged_ref(f(c3.q), f(c3.k), f(c3.v), w.seq_offsets, L, n=w.n, alpha=w.alpha, pos_tab=w.pos_tab,
+                                    timestamps=w.timestamps, ts_tab=w.ts_tab, sequences=short, **drop)
+  got = f(base)
+  scale = max(np.abs(ref[int(w.seq_offsets[b]):int(w.seq_offsets[b + 1])]).max() for b in short)
+  for b in short:
+    s, e = int(w.seq_offsets[b]), int(w.seq_offsets[b + 1])
+    assert np.abs(got[s:e] - ref[s:e]).max() <= TOL * scale, b

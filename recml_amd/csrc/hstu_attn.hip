@@ -3676,7 +3676,10 @@ __device__ __forceinline__ void lds_atomic_add(float* lds_location, float v) {
 // the same bucket are summed across the wave and one lane adds the sum to the workgroup's
 // histogram (an LDS atomic, but of one lane); only blocks with more buckets per lane use one
 // atomic per lane and run of equal buckets.
-template <int D, bool POS, bool TS, bool TG, bool SEG = false>
+// MSK: a dense keep-mask [L, Lkv] or [B, L, Lkv] (the layer-side calling convention, without the dense bias): each
+// step's tile of it -- this workgroup's 128 rows x 32 keys, 4 KB -- rides in the ring like the segment ids, every
+// wave fetching its own 32 rows, and the steps outside the range the preparation found for the tile are left out.
+template <int D, bool POS, bool TS, bool TG, bool SEG = false, bool MSK = false>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
@@ -3684,18 +3687,20 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;            // 1 KB pieces of a tile; small tiles: several waves repeat a piece
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
+  static_assert(!MSK || (!POS && !TS && !TG && !SEG), "a dense mask comes without the table biases and the segment ids");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG);
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG) + (MSK ? SM::DM_BYTES : 0);
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
+  auto Mk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS, SEG); };   // MSK: [128 rows][32 bytes]
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   float* TgBase = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
   const bool want_dpos = TG && POS && p.dpos != nullptr, want_dts = TG && TS && p.dts != nullptr;
@@ -3728,10 +3733,17 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
   const int r0 = q0 + 32 * w;
   const int qrow = r0 + m;
   const bool wave_live = r0 < s.n_q;
-  const int nt = tile_steps(p, s, q0);
+  int nt = tile_steps(p, s, q0);
   // a sliding window drops the steps before the tile's first key, and for each wave the blocks outside its band
   const int win = p.window;
-  const int t_lo = (win >= 0 && q0 - win > 0) ? (q0 - win) / BN : 0;
+  int t_lo = (win >= 0 && q0 - win > 0) ? (q0 - win) / BN : 0;
+  if (MSK) {
+    // the steps in which the keep-mask keeps a pair of this tile at all (found by the preparation kernel)
+    const int2 mr = ((const int2*)p.mask_range)[(p.mask_batched ? b : 0) * p.n_qtiles + qt];
+    t_lo = t_lo > mr.x ? t_lo : mr.x;
+    nt = nt < mr.y ? nt : mr.y;
+    nt = nt > t_lo ? nt : t_lo;
+  }
   int wave_last = p.causal ? r0 + 31 : (win >= 0 ? r0 + 31 + win : s.n_kv - 1);
   wave_last = wave_last < s.n_kv - 1 ? wave_last : s.n_kv - 1;
   if (!wave_live) wave_last = -1;
@@ -3788,6 +3800,16 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         g4 = g4 < p.Lkv - 4 ? g4 : p.Lkv - 4;
         lds_dma16_at(p.kv_seg + (int64_t)b * p.Lkv, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
       }
+    }
+    if (MSK) {
+      // the wave's own 32 rows of the step's mask tile, two lanes per row; rows past L and the second half of a last
+      // step of 16 keys re-read bytes inside the matrix (those pairs are masked by their index)
+      const uint8_t* mg = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      int gr = r0 + (lane >> 1);
+      gr = gr < p.L - 1 ? gr : p.L - 1;
+      int col = kv0 + 16 * (lane & 1);
+      col = col < p.Lkv - 16 ? col : p.Lkv - 16;
+      lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Mk(st) + w * 1024);
     }
   };
 
@@ -3996,6 +4018,18 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
         ds[4 * g + 3] = ks4.w == qseg ? ds[4 * g + 3] : 0.f;
       }
     }
+    if (MSK) {
+      // the lane's row of the mask tile: bytes of keys 8g + 4hh .. + 3
+      const unsigned char* mrow = Mk(st) + (32 * w + m) * 32 + 4 * hh;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint32_t mb = *(const uint32_t*)(mrow + 8 * g);
+        ds[4 * g + 0] = (mb & 0xffu) ? ds[4 * g + 0] : 0.f;
+        ds[4 * g + 1] = (mb & 0xff00u) ? ds[4 * g + 1] : 0.f;
+        ds[4 * g + 2] = (mb & 0xff0000u) ? ds[4 * g + 2] : 0.f;
+        ds[4 * g + 3] = (mb & 0xff000000u) ? ds[4 * g + 3] : 0.f;
+      }
+    }
     if (p.drop_thr) {
       // dropout: the pairs the forward dropped carry no gradient
       drop_apply16(ds, drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h) + (uint32_t)qrow * DROP_CI +
@@ -4180,7 +4214,10 @@ struct DkvShape {
   static constexpr int DW = D / DSPLIT;                  // channels of dK / dV per wave
 };
 
-template <int D, bool POS, bool TS, bool SEG = false>
+// MSK: the dense keep-mask as in the other backward kernel; here a step's tile is 32 query rows x this workgroup's
+// 128 keys (wave w fetches rows 8w .. 8w + 7 of it, 128 bytes each), a lane reads the 16 bytes of its key's column,
+// and the workgroup finds the query steps in which the mask keeps one of its keys by one pass over its columns.
+template <int D, bool POS, bool TS, bool SEG = false, bool MSK = false>
 __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
   using SH = DkvShape<D>;
   constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
@@ -4192,8 +4229,9 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;
   constexpr int LD = NPIECE >= NW ? NPIECE / NW : 1;
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0);
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
+  static_assert(!MSK || (!POS && !TS && !SEG && SH::DSPLIT == 1), "a dense mask comes without the table biases and the segment ids");
   // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
   // (min, max) of timestamp tiles t and t + 1
   constexpr int TQ_LANES = BN / 4 + 2;
@@ -4205,8 +4243,9 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   auto Qs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Os = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0) + (SEG ? SM::SEG_BYTES : 0);
+  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0) + (SEG ? SM::SEG_BYTES : 0) + (MSK ? SM::DM_BYTES : 0);
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0)); };
+  auto Mk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE; };      // MSK (alone in the stage): [32 rows][128 bytes]
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
@@ -4253,7 +4292,15 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   const int win = p.window;
   int nt = (s.n_q + BN - 1) / BN;
   if (win >= 0 && (kv0 + BM - 1 + win) / BN + 1 < nt) nt = (kv0 + BM - 1 + win) / BN + 1;
-  const int t_lo = p.causal ? kv0 / BN : ((win >= 0 && kv0 - win > 0) ? (kv0 - win) / BN : 0);
+  int t_lo = p.causal ? kv0 / BN : ((win >= 0 && kv0 - win > 0) ? (kv0 - win) / BN : 0);
+  if (MSK) {
+    // the query steps in which the mask keeps one of this tile's keys (a mask that carries the causal rule is
+    // empty above the diagonal: without this every key tile would walk all the rows)
+    int lo = t_lo < nt ? t_lo : nt, hi = nt;
+    general_mask_live_steps<false>(p, b, kv0, tid, lo, hi);
+    t_lo = lo;
+    nt = hi > lo ? hi : lo;
+  }
   const int t_wave = p.causal ? r0 / BN : ((win >= 0 && r0 - win > 0) ? (r0 - win) / BN : 0);   // first step with a row that sees a key of this wave
   const int t_wave_end = win >= 0 ? (r0 + 31 + win) / BN : 0x7fffffff / BN;                     // last such step
 
@@ -4312,6 +4359,16 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
         g4 = g4 < p.L - 4 ? g4 : p.L - 4;
         lds_dma16_at(p.q_seg + (int64_t)b * p.L, (uint32_t)g4 * 4u, smem_lds + (uint32_t)((const unsigned char*)Sg(st) - smem));
       }
+    }
+    if (MSK) {
+      // rows 8w .. 8w + 7 of the step's mask tile, eight lanes per row (16 bytes each = this tile's 128 keys); rows past
+      // L and pieces past Lkv re-read bytes inside the matrix (those pairs are masked by their index)
+      const uint8_t* mg = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      int gr = qbs + 8 * w + (lane >> 3);
+      gr = gr < p.L - 1 ? gr : p.L - 1;
+      int col = kv0 + 16 * (lane & 7);
+      col = col < p.Lkv - 16 ? col : p.Lkv - 16;
+      lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Mk(st) + w * 1024);
     }
   };
 
@@ -4507,6 +4564,16 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
         pv[4 * g + 1] = k1 ? pv[4 * g + 1] : 0.f;  ds[4 * g + 1] = k1 ? ds[4 * g + 1] : 0.f;
         pv[4 * g + 2] = k2 ? pv[4 * g + 2] : 0.f;  ds[4 * g + 2] = k2 ? ds[4 * g + 2] : 0.f;
         pv[4 * g + 3] = k3 ? pv[4 * g + 3] : 0.f;  ds[4 * g + 3] = k3 ? ds[4 * g + 3] : 0.f;
+      }
+    }
+    if (MSK) {
+      // the lane's column of the mask tile: byte of row 8g + 4hh + tt at key 32w + m
+      const unsigned char* mcol = Mk(st) + 32 * w + m + (4 * hh) * 128;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const bool keep = mcol[(8 * (r >> 2) + (r & 3)) * 128] != 0;
+        pv[r] = keep ? pv[r] : 0.f;
+        ds[r] = keep ? ds[r] : 0.f;
       }
     }
     if (p.drop_thr) {
@@ -5167,7 +5234,9 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
   if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
-  if (f.mask || f.dense_bias || f.L != f.Lkv) return false;   // dense operands, keys and queries of different lengths: the general pair
+  // a dense bias (or its gradient), keys and queries of different lengths: the general pair.  A dense keep-mask alone
+  // is taken (mfma_eligible has checked its rows: a multiple of 16 bytes, aligned, no table bias, no segment ids).
+  if (f.dense_bias || b->ddense_bias || f.L != f.Lkv) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
@@ -5176,20 +5245,20 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
 }
 
-template <int D, bool POS, bool TS, bool TG, bool SEG = false>
+template <int D, bool POS, bool TS, bool TG, bool SEG = false, bool MSK = false>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG);
+  const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG) + (MSK ? NSTAGE * MfmaSmem<D, 2>::DM_BYTES : 0);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
   const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
   static int granted_q[64], granted_kv[64];
-  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG>, smem_q, granted_q)) return rc;
-  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG>, smem_kv, granted_kv)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK>, smem_q, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK>, smem_kv, granted_kv)) return rc;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG, SEG>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS, SEG>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
@@ -5207,6 +5276,7 @@ int launch_bwd_mfma_ds(const Params& q, hipStream_t st) {
 
 template <int D>
 int launch_bwd_mfma_d(const Params& q, hipStream_t st) {
+  if (q.mask) return launch_bwd_mfma_inst<D, false, false, false, false, true>(q, st);
   return q.mask_mode == HSTU_MASK_SEGMENT ? launch_bwd_mfma_ds<D, true>(q, st) : launch_bwd_mfma_ds<D, false>(q, st);
 }
 

@@ -98,9 +98,18 @@ def test_backward_variant_query():
   f.window = 8                                                        # a sliding window stays on the matrix cores
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
   f.window = -1
-  f.mask = 0x50000                                                    # an explicit mask does not (the forward would)
+  f.mask = 0x50000                                                    # a dense keep-mask rides along tile by tile ...
+  f.out = 0x30000
+  plain_bytes = f.workspace_bytes
+  f.workspace_bytes = lib.hstu_attn_fwd_workspace_bytes(C.byref(f))   # (its workspace also holds the tiles' step ranges)
+  f.out = None
+  assert f.workspace_bytes > 0
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
+  f.dense_bias = 0x60000                                              # ... a dense bias does not (the forward would)
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16, bf16 products>"
+  f.dense_bias = None
   f.mask = None
+  f.workspace_bytes = plain_bytes
   # a batch small enough to go without a work list, and no bias table: no workspace to ask for, the matrix cores all the same
   f.L = f.Lkv = 256
   f.workspace, f.workspace_bytes = None, 0

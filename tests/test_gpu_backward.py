@@ -696,3 +696,60 @@ def test_reference_named_entry_points_are_differentiable(gpu):
   want = O.hstu_attention_bwd_ref(q, k, v, 2.0 * (ref - targets), causal=False, mask=mask, bias=bias, bias_grad=True)
   for nm, g, w in (("dq", qt.grad, want[0]), ("dk", kt.grad, want[1]), ("dv", vt.grad, want[2]), ("dbias", bt.grad, want[5])):
     assert _rel(g.cpu().numpy(), w) <= 2e-5, nm
+
+
+MASK_CASES = [
+    # name, d, B, L, H, mask kind, batched, causal flag, dropout
+    ("d128 causal + lengths as a mask", 128, 2, 300 - 300 % 16, 2, "causal_lens", True, False, 0.0),
+    ("d128 random mask, shared", 128, 2, 272, 2, "random", False, False, 0.0),
+    ("d128 random mask with the causal flag", 128, 3, 400, 1, "random", True, True, 0.0),
+    ("d128 band", 128, 2, 512, 2, "band", False, False, 0.0),
+    ("d128 causal + lengths, dropout", 128, 2, 256, 2, "causal_lens", True, False, 0.3),
+    ("d64 causal + lengths as a mask", 64, 3, 208, 4, "causal_lens", True, False, 0.0),
+    ("d64 random mask", 64, 2, 160, 2, "random", True, False, 0.0),
+    ("d32 random mask, shared", 32, 2, 144, 2, "random", False, False, 0.0),
+    ("d128 empty rows and columns", 128, 2, 256, 2, "holes", True, False, 0.0),
+]
+
+
+@pytest.mark.parametrize("name,d,B,L,H,kind,batched,causal,drop", MASK_CASES, ids=[c[0] for c in MASK_CASES])
+def test_backward_with_a_dense_mask_on_the_matrix_cores(gpu, name, d, B, L, H, kind, batched, causal, drop):
+  """The layer-side calling convention without a dense bias (recml/layers/keras/hstu.py:380-384 with
+  make_causal_mask's [B, L, L] mask): bf16, d in {32, 64, 128} take the matrix-core pair, the mask tile by tile."""
+  rng = np.random.default_rng(60)
+  bf = torch.bfloat16
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  i = np.arange(L)
+  if kind == "causal_lens":
+    lens = np.array([L, L // 2 + 5, 1][:B])
+    m = (i[None, None, :] <= i[None, :, None]) & (i[None, :, None] < lens[:, None, None]) & (i[None, None, :] < lens[:, None, None])
+  elif kind == "random":
+    m = rng.random((B if batched else 1, L, L)) > 0.4
+  elif kind == "band":
+    m = (np.abs(i[None, :, None] - i[None, None, :]) <= 70) & (i[None, None, :] <= i[None, :, None] + 3)
+  else:
+    # whole 128-row tiles, whole 32-key steps and whole 128-key tiles without a kept pair, and single kept pairs
+    m = np.zeros((B, L, L), bool)
+    m[0, 130:140, 0:20] = True
+    m[0, 255, 255] = True
+    m[1, 0, 0] = True
+    m[1, 200:256, 64:96] = rng.random((56, 32)) > 0.5
+  if not batched:
+    m = m[0] if m.ndim == 3 else m
+  kw = dict(causal=causal, mask=m, n=float(L) / 3, dropout_p=drop, dropout_seed=77)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), _variant_out=variant,
+                                     **{**kw, "mask": _dev(m)})
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    g = g.float().cpu().numpy()
+    assert np.abs(w).max() > 0, nm
+    assert _rel(g, w) <= 2e-2, nm
+    assert ((w == 0) <= (g == 0)).all(), nm          # rows and keys that keep nothing: exactly 0
+  assert got[3] is None and got[4] is None
+  # with the gradient of a dense bias asked for, or keys and queries of different lengths: the general pair
+  variant = []
+  recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), _variant_out=variant, causal=causal,
+                               mask=_dev(m), bias=torch.zeros((L, L), device="cuda:0"), bias_grad=True)
+  assert variant[0].startswith("hstu_bwd_general")

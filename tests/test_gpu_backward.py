@@ -753,3 +753,23 @@ def test_backward_with_a_dense_mask_on_the_matrix_cores(gpu, name, d, B, L, H, k
   recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), _variant_out=variant, causal=causal,
                                mask=_dev(m), bias=torch.zeros((L, L), device="cuda:0"), bias_grad=True)
   assert variant[0].startswith("hstu_bwd_general")
+
+
+def test_backward_with_a_dense_mask_and_lengths_on_the_matrix_cores(gpu):
+  """The mask as one more factor next to the lengths and the causal flag (the C ABI's meaning of `mask`)."""
+  rng = np.random.default_rng(61)
+  B, L, H, d = 3, 336, 2, 128
+  bf = torch.bfloat16
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  lens = np.array([336, 129, 40], np.int32)
+  m = rng.random((L, L)) > 0.5
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, seq_lens=lens, mask=m, alpha=0.5)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), seq_lens=_dev(lens), mask=_dev(m),
+                                     alpha=0.5, _variant_out=variant)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    g = g.float().cpu().numpy()
+    assert _rel(g, w) <= 2e-2, nm
+    for b in range(B):
+      assert (g[b, lens[b]:] == 0).all(), nm

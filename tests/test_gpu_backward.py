@@ -773,3 +773,34 @@ def test_backward_with_a_dense_mask_and_lengths_on_the_matrix_cores(gpu):
     assert _rel(g, w) <= 2e-2, nm
     for b in range(B):
       assert (g[b, lens[b]:] == 0).all(), nm
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_backward_with_a_dense_mask_random_shapes(gpu, seed):
+  rng = np.random.default_rng(700 + seed)
+  bf = torch.bfloat16
+  d = int(rng.choice([32, 64, 128]))
+  B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+  L = 16 * int(rng.integers(1, 30))
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  batched = bool(rng.integers(0, 2))
+  density = float(rng.choice([0.02, 0.3, 0.9]))
+  m = rng.random((B, L, L) if batched else (L, L)) < density
+  kw = dict(causal=bool(rng.integers(0, 2)), mask=m, n=float(rng.integers(1, L + 1)), alpha=float(rng.uniform(0.2, 1.0)))
+  if rng.integers(0, 2):
+    kw["seq_lens"] = rng.integers(0, L + 1, B).astype(np.int32)
+  if rng.integers(0, 2):
+    kw.update(dropout_p=0.25, dropout_seed=int(rng.integers(0, 2 ** 40)))
+  case = dict(seed=seed, d=d, B=B, H=H, L=L, batched=batched, density=density, keys=sorted(kw))
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, **kw)
+  gk = {**kw, "mask": _dev(m)}
+  if "seq_lens" in kw:
+    gk["seq_lens"] = _dev(kw["seq_lens"])
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), _variant_out=variant, **gk)
+  assert variant == ["hstu_bwd_mfma_bf16"], case
+  scale = max(np.abs(w).max() for w in want[:3])
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    g = g.float().cpu().numpy()
+    assert np.abs(g - w).max() <= 2e-2 * max(np.abs(w).max(), 0.05 * scale), (nm, case)
+    assert ((w == 0) <= (g == 0)).all(), (nm, case)

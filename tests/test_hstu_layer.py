@@ -459,3 +459,45 @@ def test_block_gradients_with_the_reference_mask_convention(gpu, dtype, hd, tol,
   for name in want:
     err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
     assert err <= tol, (name, err)
+
+
+@pytest.mark.gpu
+def test_model_trains_the_same_from_a_dense_mask_and_from_lengths(gpu):
+  """The reference's model hands every block make_causal_mask's dense [B, L, L] mask (hstu.py:604-615); here the
+  same model trains from the lengths.  Both ways in, bf16, gradients of every parameter: the same up to the
+  rounding of two different kernel paths (the dense mask goes through the matrix-core kernels tile by tile)."""
+  import recml_amd
+  from recml_amd import hstu_ops
+  dev, bf = "cuda:0", torch.bfloat16
+  B, L, D, H = 3, 160, 128, 2
+  model = recml_amd.HSTU(vocab_size=60, max_positions=L, model_dim=D, num_heads=H, num_layers=2, dtype=bf, device=dev,
+                         add_head=False, seed=2)
+  model.requires_grad_(True)
+  ids = torch.randint(1, 60, (B, L), device=dev)
+  pm = (torch.arange(L, device=dev)[None, :] < torch.tensor([160, 77, 9], device=dev)[:, None]).float()
+  dout = torch.randn((B, L, D), device=dev).to(bf)
+  seen = []
+  real = hstu_ops.hstu_attention_bwd
+
+  def spy(*a, **k):
+    k["_variant_out"] = seen
+    return real(*a, **k)
+
+  def grads(**kw):
+    for prm in model.parameters():
+      prm.grad = None
+    out = model(ids, **kw)
+    (out.float() * dout.float() * pm[:, :, None]).sum().backward()      # (padded rows carry their embeddings: not compared)
+    return {n: prm.grad.float().clone() for n, prm in model.named_parameters() if prm.grad is not None}
+
+  hstu_ops.hstu_attention_bwd = spy
+  try:
+    got = grads(attention_mask=recml_amd.make_causal_mask(pm))
+  finally:
+    hstu_ops.hstu_attention_bwd = real
+  assert seen == ["hstu_bwd_mfma_bf16"] * 2
+  want = grads(padding_mask=pm)
+  assert set(got) == set(want) and "item_embedding" in got
+  for name in want:
+    err = float((got[name] - want[name]).abs().max() / want[name].abs().max().clamp_min(1e-30))
+    assert err <= 6e-2, (name, err)

@@ -509,9 +509,9 @@ def bench_dense_backward(args, q, k, v, mask, bias):
   variant = []
   steps, warm = max(1, args.steps // 10), max(1, args.warmup // 10)
 
-  def timed(bias_grad):
-    run = lambda: recml_amd.hstu_attention_bwd(q, k, v, dout, n=L, alpha=1.0, causal=False, mask=mask, bias=bias,
-                                               bias_grad=bias_grad, _variant_out=variant)
+  def timed(bias_grad, with_bias=True):
+    run = lambda: recml_amd.hstu_attention_bwd(q, k, v, dout, n=L, alpha=1.0, causal=False, mask=mask,
+                                               bias=bias if with_bias else None, bias_grad=bias_grad, _variant_out=variant)
     for _ in range(warm):
       run()
     torch.cuda.synchronize()
@@ -521,6 +521,9 @@ def bench_dense_backward(args, q, k, v, mask, bias):
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
 
+  # the mask alone (what the reference's model hands its blocks): the matrix-core pair for bf16
+  ms_mask = timed(False, with_bias=False)
+  variant_mask = variant[-1]
   ms, ms_bias = timed(False), timed(True)
   flops = 8.0 * d * H * B * L * (L + 1) / 2
   fp32 = q.dtype == torch.float32
@@ -530,6 +533,8 @@ def bench_dense_backward(args, q, k, v, mask, bias):
       "metric": "HSTU attn bwd TFLOP/s (kept pairs), dense mask + bias, L=%d %s" % (L, "fp32" if fp32 else "bf16"),
       "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": ms,
       "ms_per_step_with_bias_gradient": ms_bias,
+      "ms_per_step_mask_only": ms_mask, "kernel_mask_only": variant_mask,
+      "value_mask_only": flops / (ms_mask * 1e-3) / 1e12,
       "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
       "dtype": "f32" if fp32 else ("bf16" if bf16_products else "bf16 storage, fp32 arithmetic"), "data": "synthetic",
       "config": {"workload": f"A1-dense backward: B={B} L={L} H={H} d={d} padded, [B,L,L] causal byte mask + fp32 bias, N={L}",

@@ -527,7 +527,8 @@ def bench_dense_backward(args, q, k, v, mask, bias):
   ms, ms_bias = timed(False), timed(True)
   flops = 8.0 * d * H * B * L * (L + 1) / 2
   fp32 = q.dtype == torch.float32
-  bf16_products = "bf16 products" in variant[-1]
+  mfma = variant[-1] == "hstu_bwd_mfma_bf16"
+  bf16_products = mfma or "bf16 products" in variant[-1]
   peak = PEAK_BF16_TFLOPS if bf16_products else PEAK_FP32_TFLOPS
   print(json.dumps({
       "metric": "HSTU attn bwd TFLOP/s (kept pairs), dense mask + bias, L=%d %s" % (L, "fp32" if fp32 else "bf16"),
@@ -541,8 +542,8 @@ def bench_dense_backward(args, q, k, v, mask, bias):
                  "kernel": variant[-1]},
       "roofline": {"bound": "mfma", "achieved": flops / (ms * 1e-3) / 1e12, "peak": peak, "unit": "TFLOP/s",
                    "frac": flops / (ms * 1e-3) / 1e12 / peak, "traffic": None,
-                   "note": "general kernels, products on the %s matrix cores; time covers both kernels, the memsets and the host call"
-                           % ("bf16" if bf16_products else "fp32")},
+                   "note": ("bf16 matrix-core kernels" if mfma else "general kernels, products on the %s matrix cores"
+                            % ("bf16" if bf16_products else "fp32")) + "; time covers both kernels, the preparation, the memsets and the host call"},
   }))
 
 

@@ -3679,28 +3679,33 @@ __device__ __forceinline__ void lds_atomic_add(float* lds_location, float v) {
 // MSK: a dense keep-mask [L, Lkv] or [B, L, Lkv] (the layer-side calling convention, without the dense bias): each
 // step's tile of it -- this workgroup's 128 rows x 32 keys, 4 KB -- rides in the ring like the segment ids, every
 // wave fetching its own 32 rows, and the steps outside the range the preparation found for the tile are left out.
-template <int D, bool POS, bool TS, bool TG, bool SEG = false, bool MSK = false>
-__global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params p) {
+// DB: the dense additive bias of that calling convention ([L, Lkv] or [B, L, Lkv] fp32, shared by the heads), the
+// same way: a step's tile of 128 rows x 32 keys (16 KB) in the ring, each wave fetching its own 32 rows, 16-byte
+// chunks XOR-swizzled by the row as in the forward.  Its gradient (p.dbias, when asked for) is dS: the wave writes
+// its block of dS over its rows of the tile, which it has just read, and adds it to the matrix in memory by rows.
+template <int D, bool POS, bool TS, bool TG, bool SEG = false, bool MSK = false, bool DB = false>
+__global__ __launch_bounds__(MFMA_THREADS, DB ? 1 : 2) void hstu_bwd_dq_mfma(const Params p) {
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
   constexpr int QCH = D / 16;
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;            // 1 KB pieces of a tile; small tiles: several waves repeat a piece
   constexpr int LD = NPIECE >= NWAVES ? NPIECE / NWAVES : 1;
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0);
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0) + (DB ? 4 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
-  static_assert(!MSK || (!POS && !TS && !TG && !SEG), "a dense mask comes without the table biases and the segment ids");
+  static_assert(!(MSK || DB) || (!POS && !TS && !TG && !SEG), "dense operands come without the table biases and the segment ids");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const uint32_t smem_lds = __builtin_amdgcn_groupstaticsize();   // LDS byte address of smem
   auto Ks = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Vs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG) + (MSK ? SM::DM_BYTES : 0);
+  constexpr int BIAS_STAGE = SM::bias_stage(POS, TS, SEG) + (MSK ? SM::DM_BYTES : 0) + (DB ? SM::DB_BYTES : 0);
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tk = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS)); };
   auto Mk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS, SEG); };   // MSK: [128 rows][32 bytes]
+  auto Bk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE + SM::bias_stage(POS, TS, SEG) + (MSK ? SM::DM_BYTES : 0); };   // DB: [128 rows][128 bytes]
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
   float* TgBase = (float*)(smem + BIAS_OFF + NSTAGE * BIAS_STAGE + (TS ? SM::TAB_BYTES : 0));   // TG only
   const bool want_dpos = TG && POS && p.dpos != nullptr, want_dts = TG && TS && p.dts != nullptr;
@@ -3810,6 +3815,21 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       int col = kv0 + 16 * (lane & 1);
       col = col < p.Lkv - 16 ? col : p.Lkv - 16;
       lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Mk(st) + w * 1024);
+    }
+    if (DB) {
+      // the wave's own 32 rows of the step's bias tile in four pieces of 8 rows: row r at byte 128 r, lane l of a piece
+      // lands at row l / 8, physical chunk l % 8, and fetches the logical chunk the swizzle maps there.  Rows past L
+      // and keys past Lkv re-read the last row / the last four keys (those pairs are masked by their index).
+      const float* bg = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = 32 * w + 8 * r + (lane >> 3), pc = lane & 7;
+        int gr = q0 + row;
+        gr = gr < p.L - 1 ? gr : p.L - 1;
+        int col = kv0 + 4 * (pc ^ (row & 7));
+        col = col < p.Lkv - 4 ? col : p.Lkv - 4;
+        lds_dma16(bg, ((uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col) * 4u, Bk(st) + (4 * w + r) * 1024);
+      }
     }
   };
 
@@ -3923,6 +3943,19 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
 #pragma unroll
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
     }
+    if (DB) {
+      // the lane's row of the bias tile: keys 8g + 4hh .. + 3 are logical chunk 2g + hh
+      const int row = 32 * w + m;
+      const unsigned char* brow = Bk(st) + row * 128;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const float4 bv = *(const float4*)(brow + (((2 * g + hh) ^ (row & 7)) * 16));
+        u[4 * g + 0] = __builtin_fmaf(bv.x, LOG2E, u[4 * g + 0]);
+        u[4 * g + 1] = __builtin_fmaf(bv.y, LOG2E, u[4 * g + 1]);
+        u[4 * g + 2] = __builtin_fmaf(bv.z, LOG2E, u[4 * g + 2]);
+        u[4 * g + 3] = __builtin_fmaf(bv.w, LOG2E, u[4 * g + 3]);
+      }
+    }
     if (TS) {
       if (ts32) {
         const int32_t* tk = Tk(st);
@@ -4034,6 +4067,27 @@ __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_bwd_dq_mfma(const Params
       // dropout: the pairs the forward dropped carry no gradient
       drop_apply16(ds, drop_bh_key(p.drop_key, (uint32_t)b * (uint32_t)p.H + (uint32_t)h) + (uint32_t)qrow * DROP_CI +
                            (uint32_t)(kbs + 4 * hh) * DROP_CJ, DROP_CJ, p.drop_thr);
+    }
+    if (DB && p.dbias != nullptr) {
+      // Dense-bias gradient: the heads' workgroups, and the sequences' for a shared bias, add dS / N into one matrix.
+      // A lane's 16 pairs lie in one row of it; written over the wave's rows of the bias tile (read above; the wave's
+      // LDS operations run in order, and nobody else touches these rows before the next barrier but one) and read
+      // back by rows, an instruction adds two whole rows of the block: two cache lines instead of 32.  Masked pairs
+      // and pairs outside the matrix are 0 and are skipped.
+      const int row = 32 * w + m;
+      unsigned char* brow = Bk(st) + row * 128;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *(float4*)(brow + (((2 * g + hh) ^ (row & 7)) * 16)) =
+            float4{ds[4 * g + 0] * p.inv_n, ds[4 * g + 1] * p.inv_n, ds[4 * g + 2] * p.inv_n, ds[4 * g + 3] * p.inv_n};
+      float* dbp = p.dbias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0) + (int64_t)r0 * p.Lkv + kbs;
+      const int col = lane & 31;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int rr = 2 * i + (lane >> 5), rw = 32 * w + rr;
+        const float val = *(const float*)(Bk(st) + rw * 128 + (((col >> 2) ^ (rw & 7)) * 16) + (col & 3) * 4);
+        if (val != 0.f) atomicAdd(dbp + (int64_t)rr * p.Lkv + col, val);
+      }
     }
     if (want_dpos) {
       // Pair (row m, key offset c = 8g + 4hh + tt) lies on diagonal c - m.  Lane j takes, for each of
@@ -4217,8 +4271,11 @@ struct DkvShape {
 // MSK: the dense keep-mask as in the other backward kernel; here a step's tile is 32 query rows x this workgroup's
 // 128 keys (wave w fetches rows 8w .. 8w + 7 of it, 128 bytes each), a lane reads the 16 bytes of its key's column,
 // and the workgroup finds the query steps in which the mask keeps one of its keys by one pass over its columns.
-template <int D, bool POS, bool TS, bool SEG = false, bool MSK = false>
-__global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
+// DB: the dense bias likewise, a step's tile of 32 rows x 128 keys (16 KB): wave w fetches rows 8w .. 8w + 7, a lane
+// reads the 16 values of its key's column (consecutive lanes, consecutive words: no swizzle needed).  The bias's
+// gradient is the other kernel's business.
+template <int D, bool POS, bool TS, bool SEG = false, bool MSK = false, bool DB = false>
+__global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) void hstu_bwd_dkv_mfma(const Params p) {
   using SH = DkvShape<D>;
   constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
   constexpr bool ACC_ASM = SH::ACC_ASM;
@@ -4229,9 +4286,9 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   constexpr int DVB = D / 32;
   constexpr int NPIECE = SM::V_BYTES / 1024;
   constexpr int LD = NPIECE >= NW ? NPIECE / NW : 1;
-  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0);
+  constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0) + (DB ? 4 : 0);
   static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
-  static_assert(!MSK || (!POS && !TS && !SEG && SH::DSPLIT == 1), "a dense mask comes without the table biases and the segment ids");
+  static_assert(!(MSK || DB) || (!POS && !TS && !SEG && SH::DSPLIT == 1), "dense operands come without the table biases and the segment ids");
   // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
   // (min, max) of timestamp tiles t and t + 1
   constexpr int TQ_LANES = BN / 4 + 2;
@@ -4243,9 +4300,11 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
   auto Qs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Os = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
   constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
-  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0) + (SEG ? SM::SEG_BYTES : 0) + (MSK ? SM::DM_BYTES : 0);
+  constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0) + (SEG ? SM::SEG_BYTES : 0) + (MSK ? SM::DM_BYTES : 0) +
+                             (DB ? SM::DB_BYTES : 0);
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0)); };
-  auto Mk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE; };      // MSK (alone in the stage): [32 rows][128 bytes]
+  auto Mk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE; };      // MSK (first in the stage): [32 rows][128 bytes]
+  auto Bk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE + (MSK ? SM::DM_BYTES : 0); };   // DB: [32 rows][128 floats]
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
   const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
@@ -4370,6 +4429,19 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
       col = col < p.Lkv - 16 ? col : p.Lkv - 16;
       lds_dma16(mg, (uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col, Mk(st) + w * 1024);
     }
+    if (DB) {
+      // rows 8w .. 8w + 7 of the step's bias tile in four pieces of two rows (512 bytes a row = this tile's 128 keys);
+      // rows past L and pieces past Lkv re-read values inside the matrix (those pairs are masked by their index)
+      const float* bg = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int gr = qbs + 8 * w + 2 * r + (lane >> 5);
+        gr = gr < p.L - 1 ? gr : p.L - 1;
+        int col = kv0 + 4 * (lane & 31);
+        col = col < p.Lkv - 4 ? col : p.Lkv - 4;
+        lds_dma16(bg, ((uint32_t)gr * (uint32_t)p.Lkv + (uint32_t)col) * 4u, Bk(st) + (4 * w + r) * 1024);
+      }
+    }
   };
 
   if (TS) {
@@ -4478,6 +4550,12 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, D == 128 ? 1 : 2) void hstu_b
     } else {
 #pragma unroll
       for (int r = 0; r < 16; ++r) u[r] = sacc[r] * alpha2;
+    }
+    if (DB) {
+      // the lane's column of the bias tile: row 8g + 4hh + tt at key 32w + m
+      const float* bcol = (const float*)Bk(st) + 32 * w + m + (4 * hh) * 128;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) u[r] = __builtin_fmaf(bcol[(8 * (r >> 2) + (r & 3)) * 128], LOG2E, u[r]);
     }
     if (TS) {
       const int32_t* tqs = Tq(st);
@@ -5234,9 +5312,9 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   HstuAttnFwdArgs f = b->fwd;
   f.out = (void*)b->dout;
   if (f.qk_dtype != HSTU_DTYPE_BF16 || !mfma_eligible(&f)) return false;
-  // a dense bias (or its gradient), keys and queries of different lengths: the general pair.  A dense keep-mask alone
-  // is taken (mfma_eligible has checked its rows: a multiple of 16 bytes, aligned, no table bias, no segment ids).
-  if (f.dense_bias || b->ddense_bias || f.L != f.Lkv) return false;
+  // keys and queries of different lengths: the general pair.  A dense keep-mask and a dense bias are taken
+  // (mfma_eligible has checked their rows: whole 16-byte pieces, aligned, no table bias, no segment ids).
+  if (f.L != f.Lkv) return false;
   if (!aligned16(b->dq) || !aligned16(b->dk) || !aligned16(b->dv)) return false;
   // q rows are addressed with 32-bit byte offsets here, like k and v rows in the forward
   if ((int64_t)f.L * f.q_stride_t * 2 >= (1LL << 31) || (int64_t)f.L * f.o_stride_t * 2 >= (1LL << 31) ||
@@ -5245,20 +5323,21 @@ bool bwd_mfma_eligible(const HstuAttnBwdArgs* b) {
   return ws.total() == 0 || (f.workspace && f.workspace_bytes >= ws.total() && ((uintptr_t)f.workspace & 255u) == 0);
 }
 
-template <int D, bool POS, bool TS, bool TG, bool SEG = false, bool MSK = false>
+template <int D, bool POS, bool TS, bool TG, bool SEG = false, bool MSK = false, bool DB = false>
 int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
-  const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG) + (MSK ? NSTAGE * MfmaSmem<D, 2>::DM_BYTES : 0);
+  const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG) + (MSK ? NSTAGE * MfmaSmem<D, 2>::DM_BYTES : 0) +
+                   (DB ? NSTAGE * MfmaSmem<D, 2>::DB_BYTES : 0);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
   const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
   static int granted_q[64], granted_kv[64];
-  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK>, smem_q, granted_q)) return rc;
-  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK>, smem_kv, granted_kv)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK, DB>, smem_q, granted_q)) return rc;
+  if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK, DB>, smem_kv, granted_kv)) return rc;
   const long long blocks = mfma_grid(p);
   if (blocks > 0x7fffffffLL) return fail(HSTU_ERR_SHAPE, "grid too large");
-  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK, DB>), dim3((unsigned)blocks), dim3(MFMA_THREADS), smem_q, st, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dq kernel launch: %s", hipGetErrorString(e));
-  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
+  hipLaunchKernelGGL((hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK, DB>), dim3((unsigned)blocks), dim3(DkvShape<D>::THREADS), smem_kv, st, p);
   e = hipGetLastError();
   if (e != hipSuccess) return fail(HSTU_ERR_LAUNCH, "backward dk/dv kernel launch: %s", hipGetErrorString(e));
   return HSTU_OK;
@@ -5276,6 +5355,8 @@ int launch_bwd_mfma_ds(const Params& q, hipStream_t st) {
 
 template <int D>
 int launch_bwd_mfma_d(const Params& q, hipStream_t st) {
+  if (q.mask && q.dense_bias) return launch_bwd_mfma_inst<D, false, false, false, false, true, true>(q, st);
+  if (q.dense_bias) return launch_bwd_mfma_inst<D, false, false, false, false, false, true>(q, st);
   if (q.mask) return launch_bwd_mfma_inst<D, false, false, false, false, true>(q, st);
   return q.mask_mode == HSTU_MASK_SEGMENT ? launch_bwd_mfma_ds<D, true>(q, st) : launch_bwd_mfma_ds<D, false>(q, st);
 }

@@ -105,8 +105,14 @@ def test_backward_variant_query():
   f.out = None
   assert f.workspace_bytes > 0
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
-  f.dense_bias = 0x60000                                              # ... a dense bias does not (the forward would)
+  f.dense_bias = 0x60000                                              # ... and so does a dense bias, with its gradient
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
+  b.ddense_bias = 0x70000
+  assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_mfma_bf16"
+  f.Lkv = f.L + 16                                                    # keys and queries of different lengths do not
   assert lib.hstu_attn_bwd_variant(C.byref(b)) == b"hstu_bwd_general<bf16, bf16 products>"
+  f.Lkv = f.L
+  b.ddense_bias = None
   f.dense_bias = None
   f.mask = None
   f.workspace_bytes = plain_bytes

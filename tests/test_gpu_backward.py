@@ -748,10 +748,11 @@ def test_backward_with_a_dense_mask_on_the_matrix_cores(gpu, name, d, B, L, H, k
     assert _rel(g, w) <= 2e-2, nm
     assert ((w == 0) <= (g == 0)).all(), nm          # rows and keys that keep nothing: exactly 0
   assert got[3] is None and got[4] is None
-  # with the gradient of a dense bias asked for, or keys and queries of different lengths: the general pair
+  # keys and queries of different lengths: the general pair
   variant = []
-  recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), _variant_out=variant, causal=causal,
-                               mask=_dev(m), bias=torch.zeros((L, L), device="cuda:0"), bias_grad=True)
+  m2 = np.ones((L, L + 16), bool)
+  recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(np.concatenate([k, k[:, :16]], 1), bf), _dev(np.concatenate([v, v[:, :16]], 1), bf),
+                               _dev(dout, bf), _variant_out=variant, causal=False, mask=_dev(m2))
   assert variant[0].startswith("hstu_bwd_general")
 
 
@@ -804,3 +805,52 @@ def test_backward_with_a_dense_mask_random_shapes(gpu, seed):
     g = g.float().cpu().numpy()
     assert np.abs(g - w).max() <= 2e-2 * max(np.abs(w).max(), 0.05 * scale), (nm, case)
     assert ((w == 0) <= (g == 0)).all(), (nm, case)
+
+
+BIAS_CASES = [
+    # name, d, B, L, H, bias batched, with a mask, the bias gradient, dropout
+    ("d128 bias per sequence + mask, gradient", 128, 2, 272, 2, True, True, True, 0.0),
+    ("d128 shared bias, lengths, gradient", 128, 3, 400, 2, False, False, True, 0.0),
+    ("d128 bias + mask, no gradient", 128, 2, 256, 1, True, True, False, 0.0),
+    ("d128 shared bias + shared mask, gradient, dropout", 128, 2, 208, 2, False, True, True, 0.3),
+    ("d64 bias per sequence + mask, gradient", 64, 3, 176, 4, True, True, True, 0.0),
+    ("d32 shared bias, gradient", 32, 2, 144, 2, False, False, True, 0.0),
+]
+
+
+@pytest.mark.parametrize("name,d,B,L,H,batched,with_mask,grad,drop", BIAS_CASES, ids=[c[0] for c in BIAS_CASES])
+def test_backward_with_a_dense_bias_on_the_matrix_cores(gpu, name, d, B, L, H, batched, with_mask, grad, drop):
+  """The layer-side calling convention in full (recml/layers/keras/hstu.py:371-384: a dense bias shared by the heads,
+  a dense mask): the matrix-core pair takes both operands tile by tile and returns the bias's gradient (dS summed
+  over the heads, and over the sequences for a shared bias)."""
+  rng = np.random.default_rng(62)
+  bf = torch.bfloat16
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  bias = (rng.standard_normal((B if batched else 1, L, L)) * 0.5).astype(np.float32)
+  lens = np.array([L, L // 2 + 5, 1][:B], np.int32)
+  kw = dict(n=float(L) / 3, bias=bias, dropout_p=drop, dropout_seed=5)
+  gk = dict(n=float(L) / 3, bias=_dev(bias), dropout_p=drop, dropout_seed=5)
+  if with_mask:
+    i = np.arange(L)
+    m = (rng.random((B, L, L) if batched else (L, L)) > 0.3) & (i[None, :] <= i[:, None] + 2)
+    kw.update(causal=False, mask=m)
+    gk.update(causal=False, mask=_dev(m))
+  else:
+    kw.update(seq_lens=lens)
+    gk.update(seq_lens=_dev(lens))
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, bias_grad=grad, **kw)
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(q, bf), _dev(k, bf), _dev(v, bf), _dev(dout, bf), bias_grad=grad,
+                                     _variant_out=variant, **gk)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    g = g.float().cpu().numpy()
+    assert np.abs(w).max() > 0 and _rel(g, w) <= 2e-2, nm
+    assert ((w == 0) <= (g == 0)).all(), nm
+  if grad:
+    g, w = got[5].cpu().numpy(), want[5]
+    assert g.shape == w.shape == bias.shape
+    assert np.abs(w).max() > 0 and _rel(g, w) <= 2e-2
+    assert ((w == 0) <= (g == 0)).all()                # pairs nobody keeps get no gradient
+  else:
+    assert len(got) == 5

@@ -114,6 +114,7 @@ struct Params {
   const int32_t* mask_range; // workspace: per (mask batch, query tile) the first 32-key step with a kept pair and one past the last
   int32_t persist;           // forward: resident workgroups that loop over the work list
   int32_t no_stream;         // forward: interior steps through the compiler-scheduled block code too (a comparison switch)
+  int32_t mask_pres;         // the preparation also fills the dense mask's presence table (the backward asks for it)
   // Dropout on the attention weights: pair (b, h, i, j) is kept when drop_hash(...) >= drop_thr (0: no dropout).
   // The survivors' scale 1 / (1 - p) is folded into inv_n by the host.
   uint32_t drop_thr, drop_key;
@@ -1792,6 +1793,14 @@ __device__ __forceinline__ uint2 lds_read_tr(const bf16_t* p) {
 constexpr int MAX_CHUNKS = 4;
 constexpr int CTR_RESERVED = 16;     // counters in front of the arrival counters
 
+// The dense keep-mask's presence table, behind the ranges in the workspace: for mask batch mb, query tile qt and key
+// tile kt (128 keys) one byte whose bit i says that rows 32 i .. 32 i + 31 of the query tile keep a pair among the
+// key tile's keys.  Written by hstu_prepare with the ranges; read by the dK/dV kernel, which walks query steps.
+constexpr int MASK_PRES_MAX_KT = 256;      // key tiles the preparation's LDS has room for (beyond: the kernel looks itself)
+__device__ __forceinline__ const uint8_t* mask_presence(const Params& p) {
+  return (const uint8_t*)(p.mask_range + 2 * (int64_t)(p.mask_batched ? p.B : 1) * p.n_qtiles);
+}
+
 // Steps of a tile: keys [0, kv_end) in 32-key steps
 __device__ __forceinline__ int tile_steps(const Params& p, const Seq& s, int q0) {
   int kv_end = s.n_kv;
@@ -2349,8 +2358,12 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
     // main kernel then leaves the other steps out altogether, loads included).  One workgroup per tile, 16
     // bytes per lane and load, eight loads in flight; rows are whole 16-byte pieces (Lkv is a multiple of 16).
     __shared__ int mr_lo[4], mr_hi[4];
+    __shared__ unsigned int kbits[MASK_PRES_MAX_KT];      // per key tile: which of the tile's four 32-row steps keep a pair there
     const int nb = p.mask_batched ? p.B : 1;
     const int ppr = p.Lkv / 16;
+    const int n_kt = (p.Lkv + BM - 1) / BM;
+    const bool pres_on = p.mask_pres && n_kt <= MASK_PRES_MAX_KT;
+    uint8_t* pres = (uint8_t*)(mrange_out + 2 * (int64_t)nb * p.n_qtiles);
     for (int tile = blockIdx.x; tile < nb * p.n_qtiles; tile += n_prep) {
       const int b = tile / p.n_qtiles, qt = tile - b * p.n_qtiles;
       const int r0 = qt * BM;
@@ -2358,6 +2371,10 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
       const uint4* mg = (const uint4*)(p.mask + ((int64_t)b * p.L + r0) * p.Lkv);
       const int n = rows * ppr;
       int lo = 0x7fffffff, hi = 0;
+      if (pres_on) {
+        for (int i = tid; i < n_kt; i += 256) kbits[i] = 0u;      // (a thread clears what it wrote out for the tile before)
+        __syncthreads();
+      }
       for (int i0 = 0; i0 < n; i0 += 8 * 256) {
         uint4 v[8];
 #pragma unroll
@@ -2369,9 +2386,16 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
         for (int k = 0; k < 8; ++k) {
           if ((v[k].x | v[k].y | v[k].z | v[k].w) != 0u) {
             const int i = i0 + 256 * k + tid;
-            const int step = (i % ppr) >> 1;
+            const int row = i / ppr, piece = i - row * ppr;
+            const int step = piece >> 1;
             lo = step < lo ? step : lo;
             hi = step + 1 > hi ? step + 1 : hi;
+            if (pres_on) {
+              // (looked at before it is set: once the tile's bits are up, which is soon for a mask with any density,
+              // the atomics stop)
+              const unsigned int bit = 1u << (row >> 5);
+              if (!(kbits[piece >> 3] & bit)) atomicOr(&kbits[piece >> 3], bit);
+            }
           }
         }
       }
@@ -2393,6 +2417,9 @@ __global__ __launch_bounds__(256) void hstu_prepare(const Params p, float* __res
         mrange_out[2 * tile] = hi > 0 ? lo : 0;
         mrange_out[2 * tile + 1] = hi;
       }
+      // (every thread's atomics on kbits lie before the barriers above)
+      if (pres_on)
+        for (int i = tid; i < n_kt; i += 256) pres[(int64_t)tile * n_kt + i] = (uint8_t)kbits[i];
     }
   }
   if (!ok_out) return;
@@ -4356,7 +4383,38 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
     // the query steps in which the mask keeps one of this tile's keys (a mask that carries the causal rule is
     // empty above the diagonal: without this every key tile would walk all the rows)
     int lo = t_lo < nt ? t_lo : nt, hi = nt;
-    general_mask_live_steps<false>(p, b, kv0, tid, lo, hi);
+    const int n_kt = (p.Lkv + BM - 1) / BM;
+    if (p.mask_pres && n_kt <= MASK_PRES_MAX_KT) {
+      // from the preparation's presence table: the first and the last 32-row step with a kept pair among this tile's
+      // keys (every wave works the same two numbers out for itself)
+      const uint8_t* pres = mask_presence(p) + (int64_t)(p.mask_batched ? b : 0) * p.n_qtiles * n_kt + kt;
+      int first = 0x7fffffff, last = 0;
+      for (int qt_ = lane; qt_ < p.n_qtiles; qt_ += 64) {
+        const uint32_t by = pres[(int64_t)qt_ * n_kt];
+        if (by) {
+          const int a = 4 * qt_ + __builtin_ctz(by), c = 4 * qt_ + 32 - __builtin_clz(by);
+          first = a < first ? a : first;
+          last = c > last ? c : last;
+        }
+      }
+#pragma unroll
+      for (int dl = 32; dl >= 1; dl >>= 1) {
+        const int a = __shfl_xor(first, dl, 64), c = __shfl_xor(last, dl, 64);
+        first = a < first ? a : first;
+        last = c > last ? c : last;
+      }
+      first = __builtin_amdgcn_readfirstlane(first);
+      last = __builtin_amdgcn_readfirstlane(last);
+      if (last == 0) {
+        hi = lo;                      // nothing kept among these keys
+      } else {
+        lo = first > lo ? first : lo;
+        hi = last < hi ? last : hi;
+        hi = hi > lo ? hi : lo;
+      }
+    } else {
+      general_mask_live_steps<false>(p, b, kv0, tid, lo, hi);
+    }
     t_lo = lo;
     nt = hi > lo ? hi : lo;
   }
@@ -4933,7 +4991,8 @@ WorkspacePlan plan_workspace(const HstuAttnFwdArgs* a, bool allow_split = true, 
     w.rel_bytes = up(n_ts * sizeof(int32_t) + 160);
     w.range_bytes = up(tiles * 2 * sizeof(int32_t) + 16);
   }
-  if (a->mask) w.mrange_bytes = up((size_t)(a->mask_batched ? a->B : 1) * (size_t)n_qtiles * 2 * sizeof(int32_t));
+  // (behind the ranges: per (mask batch, query tile, key tile of 128) one byte, see mask_presence)
+  if (a->mask) w.mrange_bytes = up((size_t)(a->mask_batched ? a->B : 1) * (size_t)n_qtiles * (2 * sizeof(int32_t) + (size_t)((a->Lkv + BM - 1) / BM)));
   // Timestamp descriptors: the forward at d = 128 in bf16 under the causal mask with lengths (what the descriptor
   // kernel's LDS holds; tables small enough to be worth their memory), when the caller's workspace has the room.
   if (want_desc && a->ts_tab && var == V_MFMA_BF16 && a->d_qk == 128 && a->causal && effective_window(a) < 0 && a->L == a->Lkv &&
@@ -5367,6 +5426,7 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
   f.flags &= ~HSTU_FWD_WORKSPACE_PREPARED;   // the backward lays the work list out without key-range splits
   const WorkspacePlan ws = plan_workspace(&f, false, ~(size_t)0, false);
   Params q = p;
+  q.mask_pres = 1;
   if (int rc = setup_workspace(&f, ws, q, st)) return rc;
   if (q.d_qk == 128) return launch_bwd_mfma_d<128>(q, st);
 #ifndef HSTU_ONLY_D128

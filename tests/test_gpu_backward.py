@@ -854,3 +854,29 @@ def test_backward_with_a_dense_bias_on_the_matrix_cores(gpu, name, d, B, L, H, b
     assert ((w == 0) <= (g == 0)).all()                # pairs nobody keeps get no gradient
   else:
     assert len(got) == 5
+
+
+@pytest.mark.parametrize("batched", [False, True])
+def test_backward_with_dense_operands_in_the_jagged_layout(gpu, batched):
+  """Packed tokens with a dense mask and bias ([L, L]-shaped per sequence position): forward and backward on the matrix
+  cores, the bias gradient included."""
+  rng = np.random.default_rng(63)
+  B, L, H, d = 3, 272, 2, 128
+  lens = np.array([272, 100, 33], np.int32)
+  bf = torch.bfloat16
+  q, k, v, dout = (O.round_bf16(rng.standard_normal((B, L, H, d)).astype(np.float32) * 0.5) for _ in range(4))
+  m = rng.random((B, L, L) if batched else (L, L)) > 0.4
+  bias = (rng.standard_normal((B if batched else 1, L, L)) * 0.5).astype(np.float32)
+  want = O.hstu_attention_bwd_ref(q, k, v, dout, seq_lens=lens, mask=m, bias=bias, bias_grad=True)
+  want_out = O.hstu_attention_ref(q, k, v, seq_lens=lens, mask=m, bias=bias)
+  pack = lambda x: O.padded_to_jagged(x, lens)
+  (qj, off), (kj, _), (vj, _), (dj, _) = pack(q), pack(k), pack(v), pack(dout)
+  kw = dict(seq_offsets=_dev(off.astype(np.int32)), max_len=L, mask=_dev(m), bias=_dev(bias))
+  out = recml_amd.hstu_attention(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), **kw)
+  assert _rel(O.jagged_to_padded(out.float().cpu().numpy(), off, L), want_out) <= 2e-2
+  variant = []
+  got = recml_amd.hstu_attention_bwd(_dev(qj, bf), _dev(kj, bf), _dev(vj, bf), _dev(dj, bf), bias_grad=True, _variant_out=variant, **kw)
+  assert variant == ["hstu_bwd_mfma_bf16"]
+  for nm, g, w in zip(("dq", "dk", "dv"), got[:3], want[:3]):
+    assert _rel(O.jagged_to_padded(g.float().cpu().numpy(), off, L), w) <= 2e-2, nm
+  assert _rel(got[5].cpu().numpy(), want[5]) <= 2e-2

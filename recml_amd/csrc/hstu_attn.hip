@@ -1740,9 +1740,11 @@ __device__ __forceinline__ void lds_dma16(const void* gbase_uniform, uint32_t by
   // the low half of a flat pointer into LDS is the LDS address (no address-space cast: its null check
   // trips the compiler in some instantiations)
   const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_dst_wave_uniform);
+  // (the base pointer through scalar_ptr: a pointer the compiler does not see to be uniform would be handed over in
+  // vector registers, which the instruction does not take)
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(base), "v"(byte_off), "s"(gbase_uniform)
+               : "s"(base), "v"(byte_off), "s"(scalar_ptr(gbase_uniform))
                : "memory", "m0");
 }
 // The same with the destination given as an LDS byte address: the dynamic LDS array of a kernel
@@ -1751,7 +1753,7 @@ __device__ __forceinline__ void lds_dma16_at(const void* gbase_uniform, uint32_t
   const uint32_t base = __builtin_amdgcn_readfirstlane(lds_addr_wave_uniform);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(base), "v"(byte_off), "s"(gbase_uniform)
+               : "s"(base), "v"(byte_off), "s"(scalar_ptr(gbase_uniform))
                : "memory", "m0");
 }
 __device__ __forceinline__ void lds_dma4(const void* gbase_uniform, uint32_t byte_off, const void* lds_dst_wave_uniform) {
@@ -2517,6 +2519,7 @@ constexpr int FWD_XCH_BYTES = 16;     // behind everything else in the forward k
 constexpr bool fwd_takes_ts_desc(int d, bool ts, bool f8, bool seg, int dense) { return ts && d == 128 && !f8 && !seg && dense == 0; }
 
 #include "hstu_fwd_stream_d128.inc"   // (the variants' names; the statements are expanded inside the kernel)
+#include "hstu_bwd_stream_d128.inc"
 
 template <int D, bool POS, bool TS, bool F8, bool SEG = false, int DENSE = 0, bool PERSIST = false>
 __global__ __launch_bounds__(MFMA_THREADS, 2) void hstu_fwd_mfma_bf16(const Params p) {
@@ -4275,16 +4278,27 @@ __global__ __launch_bounds__(MFMA_THREADS, DB ? 1 : 2) void hstu_bwd_dq_mfma(con
 // this way every definition of them is an accumulation register, so they stay there.  They are
 // only ever read as the C operand of the same instruction (chained by the hardware without wait
 // states) and by the final stores, which wait out the last product first.
+// VREG: the accumulator in ordinary vector registers instead (the instances whose interior blocks run as the
+// hand-scheduled stream, which keeps them there: as the C / D operand of this instruction an accumulation
+// register costs about 140 cycles an instruction against 32, measured; every statement that names an
+// accumulator must use the same kind, or the compiler copies all of them across).
+template <bool VREG>
 __device__ __forceinline__ void mfma_acc_zero(floatx16& acc) {
   const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-  asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=a"(acc) : "v"(z));
+  if constexpr (VREG) asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=v"(acc) : "v"(z));
+  else asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %1, 0" : "=a"(acc) : "v"(z));
 }
+template <bool VREG>
 __device__ __forceinline__ void mfma_acc(floatx16& acc, bf16x8 a, bf16x8 b) {
   // The wait states cover an operand written by the vector ALU just before: the compiler pads such a
   // pair to two wait states for its own matrix instructions but does not look into this statement
   // (without them results were wrong); four leave a margin.
-  asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+  if constexpr (VREG) asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+  else asm volatile("s_nop 3\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
 }
+
+// Ring depth of the dK/dV kernel (see there).
+constexpr int dkv_stages(int d, bool dense_bias) { return (d == 128 && !dense_bias) ? 6 : NSTAGE; }
 
 template <int D>
 struct DkvShape {
@@ -4306,6 +4320,9 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
   using SH = DkvShape<D>;
   constexpr int NW = SH::NW, THREADS = SH::THREADS, DW = SH::DW;
   constexpr bool ACC_ASM = SH::ACC_ASM;
+  // A pair of blocks that needs no mask runs as one hand-scheduled instruction stream (hstu_bwd_stream_d128.inc,
+  // written by gen_bwd_stream.py): the vector part of one block behind the matrix instructions of the other.
+  constexpr bool STREAM = D == 128 && !POS && !TS && !SEG && !MSK && !DB && SH::DSPLIT == 1;
   constexpr int DVBW = DW / 32;          // 32-channel blocks of dK / dV per wave
   using SM = MfmaSmem<D, 2>;
   constexpr int CPR = SM::CPR;
@@ -4314,7 +4331,12 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
   constexpr int NPIECE = SM::V_BYTES / 1024;
   constexpr int LD = NPIECE >= NW ? NPIECE / NW : 1;
   constexpr int NDMA = 2 * LD + ((POS || TS) ? 1 : 0) + (SEG ? 1 : 0) + (MSK ? 1 : 0) + (DB ? 4 : 0);
-  static_assert((NSTAGE - 1) * NDMA <= 63, "vmcnt range");
+  // Ring depth: 4 stages (two pairs of steps: one at work, one on its way), or 6 where the workgroup has the CU's
+  // LDS to itself anyway (d = 128) and the stages are small enough: the loads of a pair then have the time of two
+  // pairs to arrive, which the hand-scheduled pairs need (one pair's time is less than a trip to memory).
+  constexpr int NST = dkv_stages(D, DB);
+  constexpr int AHEAD = NST - 2;           // steps between a load and its use
+  static_assert((NST - 1) * NDMA <= 63, "vmcnt range");
   static_assert(!(MSK || DB) || (!POS && !TS && !SEG && SH::DSPLIT == 1), "dense operands come without the table biases and the segment ids");
   // timestamp operands of a step: 36 int32 query-side timestamps (rows qbs .. qbs + 35), then the
   // (min, max) of timestamp tiles t and t + 1
@@ -4326,7 +4348,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
   // ring stage: [Q tile | dO tile], 32 rows each
   auto Qs = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE); };
   auto Os = [&](int st) { return (bf16_t*)(smem + st * SM::STAGE + SM::K_BYTES); };
-  constexpr int BIAS_OFF = NSTAGE * SM::STAGE;
+  constexpr int BIAS_OFF = NST * SM::STAGE;
   constexpr int BIAS_STAGE = (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0) + (SEG ? SM::SEG_BYTES : 0) + (MSK ? SM::DM_BYTES : 0) +
                              (DB ? SM::DB_BYTES : 0);
   auto Sg = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0) + (TS ? TQ_BYTES : 0)); };
@@ -4334,7 +4356,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
   auto Bk = [&](int st) { return smem + BIAS_OFF + st * BIAS_STAGE + (MSK ? SM::DM_BYTES : 0); };   // DB: [32 rows][128 floats]
   auto Wc = [&](int st) { return (float*)(smem + BIAS_OFF + st * BIAS_STAGE); };
   auto Tq = [&](int st) { return (int32_t*)(smem + BIAS_OFF + st * BIAS_STAGE + (POS ? SM::POS_BYTES : 0)); };
-  const unsigned char* TsKey = smem + BIAS_OFF + NSTAGE * BIAS_STAGE;   // the keyed bucket table of this head
+  const unsigned char* TsKey = smem + BIAS_OFF + NST * BIAS_STAGE;   // the keyed bucket table of this head
 
   Work wk;
   if (!work_of_block(p, blockIdx.x, wk)) return;
@@ -4354,8 +4376,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
   const int w = w8 % NWAVES;            // which 32 keys of the tile
   const int dh = w8 / NWAVES;           // which part of the channels
   const int m = lane & 31, hh = lane >> 5;
-  const char* __restrict__ qg = (const char*)p.q + s.bq * 2;
-  const char* __restrict__ dog = (const char*)p.dout + s.bo * 2;
+  const char* __restrict__ qg = (const char*)scalar_ptr((const char*)p.q + s.bq * 2);
+  const char* __restrict__ dog = (const char*)scalar_ptr((const char*)p.dout + s.bo * 2);
   bf16_t* __restrict__ dkg = (bf16_t*)p.dk + s.bk;
   bf16_t* __restrict__ dvg = (bf16_t*)p.dv + s.bv;
 
@@ -4431,8 +4453,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
   const uint32_t rel_off = TS ? (uint32_t)((const char*)trel - wsb) : 0u;
   const uint32_t rng_off = TS ? (uint32_t)((const char*)(p.ts_range + 2 * ts_range_slot0(p, b, s.tok0)) - wsb) : 0u;
 
-  auto dma_step = [&](int t) {
-    const int st = t % NSTAGE;
+  auto dma_step = [&](int t) __attribute__((always_inline)) {
+    const int st = (t - t_lo) % NST;      // (a pair of steps starts at an even stage)
     const int qbs = t * BN;
     const int last = s.n_q - 1;
 #pragma unroll
@@ -4480,7 +4502,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
     if (MSK) {
       // rows 8w .. 8w + 7 of the step's mask tile, eight lanes per row (16 bytes each = this tile's 128 keys); rows past
       // L and pieces past Lkv re-read bytes inside the matrix (those pairs are masked by their index)
-      const uint8_t* mg = p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      const uint8_t* mg = (const uint8_t*)scalar_ptr(p.mask + (p.mask_batched ? (int64_t)b * p.L * p.Lkv : 0));
       int gr = qbs + 8 * w + (lane >> 3);
       gr = gr < p.L - 1 ? gr : p.L - 1;
       int col = kv0 + 16 * (lane & 7);
@@ -4490,7 +4512,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
     if (DB) {
       // rows 8w .. 8w + 7 of the step's bias tile in four pieces of two rows (512 bytes a row = this tile's 128 keys);
       // rows past L and pieces past Lkv re-read values inside the matrix (those pairs are masked by their index)
-      const float* bg = p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0);
+      const float* bg = (const float*)scalar_ptr(p.dense_bias + (p.dense_bias_batched ? (int64_t)b * p.L * p.Lkv : 0));
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         int gr = qbs + 8 * w + 2 * r + (lane >> 5);
@@ -4508,13 +4530,16 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
     if (1024 * c + 16 * lane < TS_LDS_BYTES)
       lds_dma16((const unsigned char*)p.ts_keyed + (int64_t)(p.ts_heads > 1 ? h : 0) * (3 * 1024) + 1024 * c, (uint32_t)lane * 16u, TsKey + 1024 * c);
   }
-  // the first pair of steps in flight (the step loop runs in pairs, see there)
-  if (t_lo < nt) dma_step(t_lo);
-  if (t_lo + 1 < nt) dma_step(t_lo + 1);
+  // the first pairs of steps in flight (the step loop runs in pairs, see there)
+#pragma unroll
+  for (int i = 0; i < AHEAD; ++i)
+    if (t_lo + i < nt) dma_step(t_lo + i);
 
   // K and V fragments of this lane's key (B operands)
-  uint4 kfr[QCH], vfr[QCH];
+  typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+  uintx4 hs_k[QCH], hs_v[QCH];
   {
+    uint4 kfr[QCH], vfr[QCH];
     const char* kp = (const char*)p.k + (s.bk + (int64_t)kcol * p.k_st) * 2 + 16 * hh;
     const char* vp = (const char*)p.v + (s.bv + (int64_t)kcol * p.v_st) * 2 + 16 * hh;
 #pragma unroll
@@ -4528,6 +4553,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
     for (int ks = 0; ks < QCH; ++ks) {
       asm volatile("" ::"v"(kfr[ks].x), "v"(kfr[ks].y), "v"(kfr[ks].z), "v"(kfr[ks].w));
       asm volatile("" ::"v"(vfr[ks].x), "v"(vfr[ks].y), "v"(vfr[ks].z), "v"(vfr[ks].w));
+      hs_k[ks] = uintx4{kfr[ks].x, kfr[ks].y, kfr[ks].z, kfr[ks].w};
+      hs_v[ks] = uintx4{vfr[ks].x, vfr[ks].y, vfr[ks].z, vfr[ks].w};
     }
   }
   int32_t kseg = 0;
@@ -4549,8 +4576,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
 #pragma unroll
   for (int i = 0; i < DVBW; ++i) {
     if (ACC_ASM) {
-      mfma_acc_zero(dka[i]);
-      mfma_acc_zero(dva[i]);
+      mfma_acc_zero<STREAM>(dka[i]);
+      mfma_acc_zero<STREAM>(dva[i]);
     } else {
 #pragma unroll
       for (int r = 0; r < 16; ++r) { dka[i][r] = 0.f; dva[i][r] = 0.f; }
@@ -4565,8 +4592,8 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
 
   // One block: 32 query rows against this wave's 32 keys.  Lane (key m, half hh) holds
   // S[q = qbs + 8g + 4hh + tt][kcol], r = 4g + tt.
-  auto block = [&](int t) {
-    const int st = t % NSTAGE;
+  auto block = [&](int t) __attribute__((always_inline)) {
+    const int st = (t - t_lo) % NST;      // (a pair of steps starts at an even stage)
     const int qbs = t * BN;
     const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     floatx16 sacc, dpacc;
@@ -4577,7 +4604,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
       for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
 #pragma unroll
       for (int ks = 0; ks < QCH; ++ks)
-        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, kfr[ks]),
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, hs_k[ks]),
                                                        ks == 0 ? zero : sacc, 0, 0, 0);
     }
     {
@@ -4587,7 +4614,7 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
       for (int ks = 0; ks < QCH; ++ks) af[ks] = *(const uint4*)(ar + (((2 * ks + hh) ^ gk) * 16));
 #pragma unroll
       for (int ks = 0; ks < QCH; ++ks)
-        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, vfr[ks]),
+        dpacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[ks]), __builtin_bit_cast(bf16x8, hs_v[ks]),
                                                         ks == 0 ? zero : dpacc, 0, 0, 0);
     }
     float u[16];
@@ -4732,28 +4759,76 @@ __global__ __launch_bounds__(DkvShape<D>::THREADS, (D == 128 || DB) ? 1 : 2) voi
 #pragma unroll
       for (int dvb = 0; dvb < DVBW; ++dvb) {
         if (ACC_ASM) {
-          mfma_acc(dva[dvb], __builtin_bit_cast(bf16x8, otf[cc][dvb]), pb);
-          mfma_acc(dka[dvb], __builtin_bit_cast(bf16x8, qtf[cc][dvb]), db);
+          mfma_acc<STREAM>(dva[dvb], __builtin_bit_cast(bf16x8, otf[cc][dvb]), pb);
+          mfma_acc<STREAM>(dka[dvb], __builtin_bit_cast(bf16x8, qtf[cc][dvb]), db);
         } else {
           dva[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, otf[cc][dvb]), pb, dva[dvb], 0, 0, 0);
           dka[dvb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, qtf[cc][dvb]), db, dka[dvb], 0, 0, 0);
         }
       }
     }
+    // The compiler does not know of the matrix instructions above: whatever it puts behind them (a copy of an
+    // accumulator at a join of two paths, say) must find the last product's result in place.
+    if (ACC_ASM) asm volatile("s_nop 15");
   };
 
-  // steps in pairs, one barrier per pair (see the other backward kernel)
-  static_assert(NSTAGE == 4, "two pairs of stages");
-  HSTU_WAIT_VMCNT(0);
-  __syncthreads();
-  for (int t = t_lo; t < nt; t += 2) {
-    if (t + 2 < nt) dma_step(t + 2);
-    if (t + 3 < nt) dma_step(t + 3);
+  // (the stream's operands)
+  const bool stream_on = STREAM && !p.no_stream && !p.drop_thr && win < 0 && wave_live && r0 + 32 <= s.n_kv;
+  const uint32_t hs_a0 = (uint32_t)(m * (D * 2) + ((hh ^ gk) * 16));
+  const uint32_t hs_t0 = (uint32_t)(vrow * (D * 2) + 8 * (gi & 1) + 64 * swz_rt_group<D>(gi) + 16 * c_lo);
+  const float hs_alpha = alpha2;
+
+  // steps in pairs, one barrier per pair (see the other backward kernel).  Three loops, so that the stream's loop
+  // holds nothing of the block code: pairs ahead of the stream's (the diagonal), the stream's, the rest (the
+  // sequence's end).  Every wave passes one barrier per pair whichever loop the pair falls into.
+  static_assert(NST % 2 == 0 && NST >= 4, "pairs of stages");
+  int t_s0 = nt, t_s1 = nt;           // the stream's pairs: [t_s0, t_s1), in steps of 2 from t_lo
+  if constexpr (STREAM) {
+    if (stream_on) {
+      // both blocks whole: every row at or past the wave's last key (causal), inside the sequence
+      int first = p.causal ? (r0 + 31 + BN - 1) / BN : 0;
+      first = first > t_lo ? first : t_lo;
+      first += (first - t_lo) & 1;
+      int end = s.n_q / BN;                              // steps [first, end) are whole
+      end = end < nt ? end : nt;
+      end -= (end - t_lo) & 1;
+      if (end > first) { t_s0 = first; t_s1 = end; }
+    }
+  }
+  // a pair's loads go out AHEAD steps before it; at its end the next pair's must have landed, the ones just sent need not
+  auto send_ahead = [&](int t) __attribute__((always_inline)) {
+    int n = 0;
+    if (t + AHEAD < nt) { dma_step(t + AHEAD); ++n; }
+    if (t + AHEAD + 1 < nt) { dma_step(t + AHEAD + 1); ++n; }
+    return n;
+  };
+  auto end_of_pair = [&](int n_sent) __attribute__((always_inline)) {
+    if (AHEAD == 2 || n_sent == 0) HSTU_WAIT_VMCNT(0);
+    else if (n_sent == 1) HSTU_WAIT_VMCNT(NDMA);
+    else HSTU_WAIT_VMCNT(2 * NDMA);
+    __syncthreads();
+  };
+  auto block_pair = [&](int t) __attribute__((always_inline)) {
+    const int n_sent = send_ahead(t);
     if (wave_live && t >= t_wave && t <= t_wave_end) block(t);
     if (t + 1 < nt && wave_live && t + 1 >= t_wave && t + 1 <= t_wave_end) block(t + 1);
-    HSTU_WAIT_VMCNT(0);
-    __syncthreads();
+    end_of_pair(n_sent);
+  };
+  HSTU_WAIT_VMCNT(0);
+  __syncthreads();
+  int t = t_lo;
+  for (; t < nt && t < t_s0; t += 2) block_pair(t);
+  if constexpr (STREAM) {
+    for (; t < t_s1; t += 2) {
+      const int n_sent = send_ahead(t);
+      const uint32_t hs_sb = __builtin_amdgcn_readfirstlane(smem_lds + (uint32_t)(((t - t_lo) % NST) * SM::STAGE));
+#define HSTU_BWD_STREAM_VARIANT HSTU_BWD_STREAM_PAIR
+#include "hstu_bwd_stream_d128.inc"
+#undef HSTU_BWD_STREAM_VARIANT
+      end_of_pair(n_sent);
+    }
   }
+  for (; t < nt; t += 2) block_pair(t);
 
   if (ACC_ASM) asm volatile("s_nop 15\n\ts_nop 15");   // the last product has left the pipeline before its result is read
   unsigned char* ot = smem + w8 * (32 * DW * 2);
@@ -5387,7 +5462,10 @@ int launch_bwd_mfma_inst(const Params& p, hipStream_t st) {
   const int smem = MfmaSmem<D, 2>::total(POS, TS, SEG) + (MSK ? NSTAGE * MfmaSmem<D, 2>::DM_BYTES : 0) +
                    (DB ? NSTAGE * MfmaSmem<D, 2>::DB_BYTES : 0);
   const int smem_q = smem + (TG ? BWD_TG_BYTES : 0);
-  const int smem_kv = smem + (TS ? NSTAGE * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
+  constexpr int nst_kv = dkv_stages(D, DB);
+  const int smem_kv = MfmaSmem<D, 2>::total(POS, TS, SEG, 0, nst_kv) + (MSK ? nst_kv * MfmaSmem<D, 2>::DM_BYTES : 0) +
+                      (DB ? nst_kv * MfmaSmem<D, 2>::DB_BYTES : 0) +
+                      (TS ? nst_kv * 16 : 0);     // one more 16-byte piece of timestamp operands per stage
   static int granted_q[64], granted_kv[64];
   if (int rc = allow_lds((const void*)hstu_bwd_dq_mfma<D, POS, TS, TG, SEG, MSK, DB>, smem_q, granted_q)) return rc;
   if (int rc = allow_lds((const void*)hstu_bwd_dkv_mfma<D, POS, TS, SEG, MSK, DB>, smem_kv, granted_kv)) return rc;
@@ -5427,6 +5505,7 @@ int launch_bwd_mfma(const HstuAttnBwdArgs* b, const Params& p, hipStream_t st) {
   const WorkspacePlan ws = plan_workspace(&f, false, ~(size_t)0, false);
   Params q = p;
   q.mask_pres = 1;
+  q.no_stream = (b->fwd.flags & HSTU_FWD_COMPILER_SCHEDULED_BLOCKS) ? 1 : 0;
   if (int rc = setup_workspace(&f, ws, q, st)) return rc;
   if (q.d_qk == 128) return launch_bwd_mfma_d<128>(q, st);
 #ifndef HSTU_ONLY_D128

@@ -422,7 +422,7 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
                        timestamps=None, ts_bias=None, ts_bucket_size=0.301,
                        q_segment_ids=None, kv_segment_ids=None,
                        sliding_window_size=None, mask=None, bias=None, dropout_p=0.0, dropout_seed=0,
-                       table_grads=True, bias_grad=False, grads_out=None, _variant_out=None):
+                       table_grads=True, bias_grad=False, grads_out=None, _variant_out=None, _flags=0):
   """Gradients of sum(hstu_attention(q, k, v, ...) * dout).
 
   Same arguments as hstu_attention (fp32 or bf16; not fp8).  Returns
@@ -463,6 +463,7 @@ def hstu_attention_bwd(q, k, v, dout, *, seq_lens=None, seq_offsets=None, max_le
   ba = _lib.HstuAttnBwdArgs()
   ba.struct_size = C.sizeof(_lib.HstuAttnBwdArgs)
   ba.version = _lib.ABI_VERSION
+  fa.flags |= int(_flags)       # (comparison switches of the tests)
   ba.fwd = fa
   ba.dout, ba.dq, ba.dk, ba.dv = dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
   dpos = dts = None

@@ -172,3 +172,43 @@ def test_stream_against_the_oracle(gpu, pos):
   ref = O.hstu_attention_jagged_ref(f(q), f(k), f(v), off, L, n=L, **okw)
   err = np.abs(got - ref).max() / np.abs(ref).max()
   assert err <= BF16_TOL, err
+
+
+# ---- the backward's dK/dV kernel: pairs of unmasked blocks as one hand-scheduled stream (d = 128, no bias)
+
+BWD_CASES = [
+    # name, lengths, L, H, causal, jagged
+    ("one long sequence", [2048], 2048, 2, True, True),
+    ("mixed lengths around every tile edge", [2048, 1655, 1000, 777, 513, 512, 511, 385, 384, 256, 129, 128, 127, 16, 1], 2048, 2, True, True),
+    ("no causal mask, jagged", [1024, 1000, 515, 300], 1024, 2, False, True),
+    ("padded with lengths", [2048, 1655, 1000, 640, 641, 639, 100], 2048, 2, True, False),
+    ("a first step that is odd", [1952, 700], 2048, 3, True, True),
+]
+
+
+@pytest.mark.parametrize("name,lens,L,H,causal,jagged", BWD_CASES, ids=[c[0] for c in BWD_CASES])
+def test_backward_stream_gives_the_bits_of_the_block_code(gpu, name, lens, L, H, causal, jagged):
+  q, k, v, kw = _inputs(lens, L, H, False, causal, jagged, seed=3)
+  dout = torch.randn(v.shape, device="cuda:0", generator=torch.Generator(device="cuda:0").manual_seed(4)).mul_(0.5).to(torch.bfloat16)
+  var = []
+  ref = hstu_ops.hstu_attention_bwd(q, k, v, dout, _flags=_lib.FWD_COMPILER_SCHEDULED_BLOCKS, _variant_out=var, alpha=0.2, **kw)
+  assert var[0] == "hstu_bwd_mfma_bf16"
+  for _ in range(2):
+    got = hstu_ops.hstu_attention_bwd(q, k, v, dout, alpha=0.2, **kw)
+    torch.cuda.synchronize()
+    for name_, a, b in zip(("dq", "dk", "dv"), ref[:3], got[:3]):
+      assert not torch.isnan(b.float()).any(), name_
+      assert torch.equal(a.view(torch.int16), b.view(torch.int16)), name_
+
+
+def test_backward_stream_against_the_fp32_kernels(gpu):
+  # every accumulator register of dK and dV: the general kernels in fp32 on the same inputs
+  q, k, v, kw = _inputs([2048, 700], 2048, 2, False, True, True, seed=5)
+  dout = torch.randn(v.shape, device="cuda:0", generator=torch.Generator(device="cuda:0").manual_seed(6)).mul_(0.5).to(torch.bfloat16)
+  ref = hstu_ops.hstu_attention_bwd(q.float(), k.float(), v.float(), dout.float(), alpha=0.2, **kw)
+  for flags in (0, _lib.FWD_COMPILER_SCHEDULED_BLOCKS):
+    got = hstu_ops.hstu_attention_bwd(q, k, v, dout, alpha=0.2, _flags=flags, **kw)
+    for name_, a, b in zip(("dq", "dk", "dv"), ref[:3], got[:3]):
+      # per channel: a register that is read too early shows in one channel of every key
+      err = (b.float() - a).abs().amax(dim=(0, 1)) / a.abs().amax()
+      assert float(err.max()) <= 1e-2, (name_, flags, int(err.argmax()), float(err.max()))

@@ -183,16 +183,8 @@ class PairGen:
   # ---- the 64 matrix instructions of the pair and the LDS reads that feed them
   def slot_info(self, i):
     """(kind, block, index within its group)"""
-    # the two chains of a block alternate: a matrix instruction that adds to the one before it cannot follow it
-    # at full rate when the wave is alone on its SIMD
-    if i < 32:
-      if "alt" in self.ablate: return ("s" if i % 2 == 0 else "dp", i // 16, (i % 16) // 2)
-      return ("s" if (i % 16) < 8 else "dp", i // 16, i % 8)
+    if i < 32: return ("s" if (i % 16) < 8 else "dp", i // 16, i % 8)
     j = i - 32
-    if "chain" in self.ablate:
-      # accumulator by accumulator: the four products into one accumulator (two blocks, two halves) in a row
-      acc, k = j // 4, j % 4
-      return ("dvk", k // 2, 8 * (k % 2) + acc)          # acc = 2 dvb + which
     blk, j = j // 16, j % 16
     return ("dvk", blk, j)           # j = 8 cc + 2 dvb + (0: dV, 1: dK)
 
@@ -275,12 +267,8 @@ class PairGen:
       for k, o in enumerate(ops):
         slot = first + (k * (last - first + 1)) // n
         plan.setdefault(slot, []).append(o)
-    if "alt" in self.ablate:
-      spread(va, 16, 35)
-      spread(vb, 36, 55)
-    else:
-      spread(va, 8, 31)
-      spread(vb, 32, 55)
+    spread(va, 8, 31)
+    spread(vb, 32, 55)
     for i in range(64):
       self.matrix(i)
       for o in plan.get(i, ()): o()
@@ -311,7 +299,7 @@ def main():
   ap = argparse.ArgumentParser()
   ap.add_argument("--out", default=os.path.join(os.path.dirname(os.path.abspath(__file__)), "hstu_bwd_stream_d128.inc"))
   ap.add_argument("--base", type=int, default=136)
-  ap.add_argument("--ablate", default="", help="measurements only: comma-separated of novalu, nolds (wrong results)")
+  ap.add_argument("--ablate", default="", help="measurements only, wrong results: comma-separated of novalu, nolds, nomfma, nosdp (no S / dP products), nodvk (no dV / dK products)")
   a = ap.parse_args()
   parts = ["// Generated by gen_bwd_stream.py: do not edit.  The hand-scheduled stream of the dK/dV kernel's interior blocks, a pair at a time.\n",
            "#define HSTU_BWD_STREAM_PAIR 1\n"]

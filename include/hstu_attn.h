@@ -82,7 +82,9 @@ enum HstuFwdFlags {
    * as one hand-scheduled instruction stream (software-pipelined across steps).
    * This bit sends those steps through the compiler-scheduled code that handles
    * every other step instead: a comparison switch; same arithmetic in the same
-   * order, the same bits out. */
+   * order, the same bits out.  In the `fwd` member of hstu_attn_bwd's arguments
+   * it does the same to the backward's dK/dV kernel, which runs its unmasked
+   * blocks without bias as such a stream at d = 128. */
   HSTU_FWD_COMPILER_SCHEDULED_BLOCKS = 16
 };
 
